@@ -1,0 +1,141 @@
+/*
+ * torch_col_hip.h -- flat C ABI of libtorch_col_hip.so, part 1: the device side
+ * of the colocated training step on MI355X (gfx950).
+ *
+ * The reference (SiriusInfTra/Sirius) has no arithmetic of its own on this
+ * path: train/resnet152.py:22-29,84-91 (and train/swin_b.py:38-45,83-95) build
+ * a torchvision model, nn.CrossEntropyLoss and torch.optim.SGD, and every
+ * kernel launch of that model travels through the xsched launch queue
+ * (third_party/xsched/shim/cuda/shim.cpp:162-203).  The entry points below are
+ * what a binding for that path calls instead: NHWC operators that ENQUEUE
+ * hand-written HIP kernels on a context (stream + optional preemptible launch
+ * queue + optional recording), and the queue controls the reference exposes
+ * through common/xsched_ctrl.h:12-40.
+ *
+ * Conventions
+ *   - plain pointers are DEVICE pointers unless a name says host;
+ *   - dtype: 0 = fp32, 1 = bf16 (activations and filter shadows); parameters,
+ *     gradients, statistics and the loss are always fp32;
+ *   - activations are NHWC, filters are [K][R][S][C] (output channel major);
+ *   - channel counts must be multiples of one 16-byte chunk (4 fp32 / 8 bf16);
+ *   - return value 0 = enqueued, negative = -errno style failure with a
+ *     message in tch_last_error() (thread local).  Nothing aborts the process.
+ */
+#ifndef TORCH_COL_HIP_H_
+#define TORCH_COL_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct tch_context tch_context;
+typedef struct tch_program tch_program;
+
+const char* tch_last_error(void);
+/* 1 when the library was built with device code for gfx950 (always, for this build). */
+int tch_has_device_code(void);
+
+/* ---- context: where launches go ------------------------------------------------ */
+/* hip_stream: a hipStream_t (0 = the null stream).  If the stream is registered
+ * (tch_RegisterStream) launches pass through its launch queue. */
+int tch_context_create(void* hip_stream, tch_context** out);
+void tch_context_destroy(tch_context* ctx);
+/* launches skipped since the last call because the reject flag was up */
+uint64_t tch_context_take_rejected(tch_context* ctx);
+
+/* ---- programs: record once, replay every step ---------------------------------- */
+int tch_program_create(tch_program** out);
+void tch_program_destroy(tch_program* prog);
+int64_t tch_program_size(const tch_program* prog);
+/* Between begin and end every operator call on ctx appends to prog instead of launching. */
+int tch_program_begin_record(tch_context* ctx, tch_program* prog);
+int tch_program_end_record(tch_context* ctx);
+/* Replay launches [first, last) (last < 0: to the end).  The reject flag is a
+ * checkpoint between launches: returns 1 if any launch was skipped because of it. */
+int tch_program_run(tch_context* ctx, const tch_program* prog, int64_t first, int64_t last);
+
+/* ---- preemptible launch queues (replaces common/xsched_ctrl.h:12-40) ------------ */
+uint64_t tch_RegisterStream(uint64_t hip_stream);   /* xsched_ctrl.cc:27-46; 0 on failure */
+int tch_UnRegisterStream(uint64_t hip_stream);      /* xsched_ctrl.cc:70-78 */
+void tch_UnRegisterAllStreams(void);                /* xsched_ctrl.cc:80-86 */
+size_t tch_GetXQueueSize(uint64_t hip_stream);      /* xsched_ctrl.cc:158-166 */
+size_t tch_GetXQueueSizeAllStreams(void);           /* xsched_ctrl.cc:168-178 */
+size_t tch_GetTotalXQueueSize(void);                /* xsched_ctrl.cc:180-190 */
+size_t tch_AbortStream(uint64_t hip_stream);        /* xsched_ctrl.cc:110-115 */
+size_t tch_AbortAllStreams(void);                   /* xsched_ctrl.cc:117-138 */
+int tch_SyncStream(uint64_t hip_stream);            /* xsched_ctrl.cc:140-147 */
+int tch_SyncAllStreams(void);                       /* xsched_ctrl.cc:149-156 */
+int tch_QueryRejectCudaCalls(void);                 /* xsched_ctrl.cc:192-194 */
+void tch_SetRejectCudaCalls(int reject);            /* xsched_ctrl.cc:196-198 */
+/* queue length / sync interval used by later tch_RegisterStream calls (reference: 16, 8) */
+void tch_SetXQueueShape(int queue_length, int sync_interval);
+size_t tch_GetXQueueInFlight(uint64_t hip_stream);
+
+/* ---- convolution (implicit GEMM on MFMA) ---------------------------------------- */
+/* y[N,Ho,Wo,K] = conv(x[N,H,W,C], w[K,R,S,C]) (+ bias[K]) (+ add, optionally gated by mask > 0).
+ * out_f32 != 0 stores y as fp32 whatever dtype is.  tile_cfg: -1 auto, 0 = 128x128, 1 = 128x64, 2 = 64x64. */
+int tch_conv2d_fwd(tch_context* ctx, int dtype, const void* x, const void* w, void* y, const void* add,
+                   const void* mask, const float* bias, int out_f32, int N, int H, int W, int C, int K, int R, int S,
+                   int stride, int pad, int tile_cfg);
+/* dx[N,H,W,C] = conv_transpose(dy[N,Ho,Wo,K], w) (+ add, optionally gated by mask > 0) */
+int tch_conv2d_dgrad(tch_context* ctx, int dtype, const void* dy, const void* w, void* dx, const void* add,
+                     const void* mask, int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
+                     int tile_cfg);
+/* dw[K,R,S,C] (fp32) (+)= sum over pixels of dy x x.  splits > 1 needs a workspace of
+ * tch_conv2d_wgrad_workspace_bytes(); splits <= 0 lets the library choose (query with _pick_splits). */
+int tch_conv2d_wgrad_pick_splits(int dtype, int N, int H, int W, int C, int K, int R, int S, int stride, int pad);
+int64_t tch_conv2d_wgrad_workspace_bytes(int dtype, int K, int R, int S, int C, int splits);
+int tch_conv2d_wgrad(tch_context* ctx, int dtype, const void* x, const void* dy, float* dw, float* workspace,
+                     int splits, int accumulate, int N, int H, int W, int C, int K, int R, int S, int stride,
+                     int pad, int tile_cfg);
+
+/* ---- BatchNorm (training mode) with fused ReLU / residual ---------------------- */
+int64_t tch_bn_workspace_bytes(int dtype, int64_t rows, int C);
+/* y = relu?(bn(x) + residual?) over x viewed as [rows, C]; updates running stats (may be NULL),
+ * writes save_mean / save_invstd for the backward pass. */
+int tch_bn_fwd_train(tch_context* ctx, int dtype, const void* x, void* y, const void* residual, int relu,
+                     int64_t rows, int C, const float* gamma, const float* beta, float* running_mean,
+                     float* running_var, float* save_mean, float* save_invstd, float momentum, float eps,
+                     float* workspace);
+/* g = dy * (relu_mask > 0) (relu_mask may be NULL); dgamma/dbeta (+)=; dx = bn'(g) */
+int tch_bn_bwd(tch_context* ctx, int dtype, const void* dy, const void* relu_mask, const void* x, void* dx,
+               int64_t rows, int C, const float* gamma, const float* save_mean, const float* save_invstd,
+               float* dgamma, float* dbeta, int accumulate, float* workspace);
+
+/* ---- pooling -------------------------------------------------------------------- */
+/* index[N,Ho,Wo,C] (int32) = h*W + w of the FIRST maximum in row-major window order (NaN wins). */
+int tch_maxpool_fwd(tch_context* ctx, int dtype, const void* x, void* y, int32_t* index, int N, int H, int W, int C,
+                    int ksize, int stride, int pad);
+int tch_maxpool_bwd(tch_context* ctx, int dtype, const void* dy, const int32_t* index, void* dx, int N, int H, int W,
+                    int C, int ksize, int stride, int pad);
+int tch_avgpool_fwd(tch_context* ctx, int dtype, const void* x, void* y, int N, int HW, int C);
+int tch_avgpool_bwd(tch_context* ctx, int dtype, const void* dy, void* dx, int N, int HW, int C);
+
+/* ---- loss, optimizer, accumulation ---------------------------------------------- */
+/* loss_rows[i] = logsumexp(logits[i]) - logits[i, label]; loss_mean = mean; dlogits (dtype, leading
+ * dimension ld_dlogits) = (softmax - onehot) * grad_scale, grad_scale = loss_scale / rows. */
+int tch_softmax_ce_fwd_bwd(tch_context* ctx, int dtype, const float* logits, const int64_t* labels, float* loss_rows,
+                           float* loss_mean, void* dlogits, int rows, int classes, int ld_dlogits, float grad_scale);
+/* g += wd*p; buf = momentum*buf + g; p -= lr*buf; shadow_bf16 (may be NULL) = bf16(p) */
+int tch_sgd_momentum_step(tch_context* ctx, float* param, const float* grad, float* momentum_buf, void* shadow_bf16,
+                          int64_t n, float lr, float momentum, float weight_decay);
+/* global += grad; grad = 0   (pytorch/torch_col/accumulate.py:20-24) */
+int tch_grad_accumulate(tch_context* ctx, float* global, float* grad, int64_t n);
+int tch_fill_zero(tch_context* ctx, void* ptr, int64_t bytes);
+int tch_bias_grad(tch_context* ctx, int dtype, const void* dy, float* dbias, int rows, int cols, int ld,
+                  int accumulate);
+
+/* ---- layout / precision ---------------------------------------------------------- */
+int tch_nchw_to_nhwc_pad(tch_context* ctx, int dtype, const float* x_nchw, void* y_nhwc, int N, int C, int H, int W,
+                         int Cpad);
+int tch_cast_from_f32(tch_context* ctx, int dtype, const float* src, void* dst, int64_t n);
+int tch_cast_to_f32(tch_context* ctx, int dtype, const void* src, float* dst, int64_t n);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* TORCH_COL_HIP_H_ */

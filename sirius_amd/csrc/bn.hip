@@ -1,0 +1,347 @@
+// Training-mode BatchNorm over NHWC activations viewed as [rows, C], with the
+// ReLU and the residual add of a bottleneck block fused into the apply pass.
+// HBM-bound: every pass moves 16-byte chunks per lane, channel = fastest dim.
+//
+// Arithmetic restated from torch.nn.BatchNorm2d as used by torchvision's
+// ResNet (reference call site train/resnet152.py:22): batch statistics with
+// biased variance for normalisation, unbiased variance into running_var,
+// momentum update running = (1-m)*running + m*batch.
+//
+//   forward : partial (sum, sum of squares) per row block  -> finalize (fp64)
+//             -> y = relu(x*scale + shift [+ residual])
+//   backward: g = dy * (mask > 0); partial (sum g, sum g*xhat) -> finalize
+//             -> dx = gamma*invstd*(g - mean(g) - xhat*mean(g*xhat))
+#include "kernels.h"
+#include "ops.h"
+
+namespace tch {
+namespace {
+
+struct ColReduceArgs {
+  const void* a;     // stats: x        bwd: dy
+  const void* mask;  // bwd: tensor whose sign gates dy (may be null)
+  const void* x;     // bwd: x
+  const float* mean;
+  const float* invstd;
+  float* partial;  // [row_blocks][C][2]
+  int64_t rows;
+  int C, cc, ccb, rowlanes;
+  int64_t rows_per_block;
+};
+
+template <typename T, int BWD>
+__global__ __launch_bounds__(256) void col_reduce_kernel(ColReduceArgs p) {
+  constexpr int E = Elem<T>::kPerChunk;
+  __shared__ float red[256 * 2 * E];
+  const int tid = threadIdx.x;
+  const int tx = tid % p.ccb, ty = tid / p.ccb;
+  const int col = blockIdx.x * p.ccb + tx;  // chunk column
+  const bool col_ok = col < p.cc;
+  float s1[E], s2[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) s1[e] = s2[e] = 0.f;
+  float mu[E], is[E];
+  if (BWD && col_ok) {
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      mu[e] = p.mean[col * E + e];
+      is[e] = p.invstd[col * E + e];
+    }
+  }
+  const int64_t r0 = static_cast<int64_t>(blockIdx.y) * p.rows_per_block;
+  int64_t r1 = r0 + p.rows_per_block;
+  if (r1 > p.rows) r1 = p.rows;
+  if (col_ok) {
+    for (int64_t r = r0 + ty; r < r1; r += p.rowlanes) {
+      const int64_t ci = r * p.cc + col;
+      Chunk ca;
+      ca.u = static_cast<const uint4*>(p.a)[ci];
+      float va[E];
+      chunk_to_float<T>(ca, va);
+      if (BWD) {
+        Chunk cx;
+        cx.u = static_cast<const uint4*>(p.x)[ci];
+        float vx[E];
+        chunk_to_float<T>(cx, vx);
+        if (p.mask) {
+          Chunk cm;
+          cm.u = static_cast<const uint4*>(p.mask)[ci];
+          float vm[E];
+          chunk_to_float<T>(cm, vm);
+#pragma unroll
+          for (int e = 0; e < E; ++e)
+            if (!(vm[e] > 0.f)) va[e] = 0.f;
+        }
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          s1[e] += va[e];
+          s2[e] += va[e] * ((vx[e] - mu[e]) * is[e]);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          s1[e] += va[e];
+          s2[e] += va[e] * va[e];
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    red[(tid * 2 * E) + e] = s1[e];
+    red[(tid * 2 * E) + E + e] = s2[e];
+  }
+  __syncthreads();
+  if (ty == 0 && col_ok) {
+    for (int y = 1; y < p.rowlanes; ++y) {
+      const float* o = red + ((y * p.ccb + tx) * 2 * E);
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        s1[e] += o[e];
+        s2[e] += o[E + e];
+      }
+    }
+    float* dst = p.partial + (static_cast<int64_t>(blockIdx.y) * p.C + col * E) * 2;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      dst[2 * e] = s1[e];
+      dst[2 * e + 1] = s2[e];
+    }
+  }
+}
+
+struct FwdFinalizeArgs {
+  const float* partial;
+  int row_blocks, C;
+  int64_t rows;
+  const float* gamma;
+  const float* beta;
+  float* running_mean;
+  float* running_var;
+  float* save_mean;
+  float* save_invstd;
+  float* scale;
+  float* shift;
+  float momentum, eps;
+};
+
+__global__ __launch_bounds__(64) void bn_fwd_finalize_kernel(FwdFinalizeArgs p) {
+  const int c = blockIdx.x * 64 + threadIdx.x;
+  if (c >= p.C) return;
+  double s = 0.0, q = 0.0;
+  for (int b = 0; b < p.row_blocks; ++b) {
+    const float* src = p.partial + (static_cast<int64_t>(b) * p.C + c) * 2;
+    s += src[0];
+    q += src[1];
+  }
+  const double n = static_cast<double>(p.rows);
+  const double mean = s / n;
+  double var = q / n - mean * mean;
+  if (var < 0.0) var = 0.0;
+  const float invstd = 1.0f / sqrtf(static_cast<float>(var) + p.eps);
+  p.save_mean[c] = static_cast<float>(mean);
+  p.save_invstd[c] = invstd;
+  if (p.running_mean) {
+    const double unbiased = p.rows > 1 ? var * n / (n - 1.0) : var;
+    p.running_mean[c] = (1.f - p.momentum) * p.running_mean[c] + p.momentum * static_cast<float>(mean);
+    p.running_var[c] = (1.f - p.momentum) * p.running_var[c] + p.momentum * static_cast<float>(unbiased);
+  }
+  const float sc = p.gamma[c] * invstd;
+  p.scale[c] = sc;
+  p.shift[c] = p.beta[c] - static_cast<float>(mean) * sc;
+}
+
+struct BwdFinalizeArgs {
+  const float* partial;
+  int row_blocks, C;
+  int64_t rows;
+  const float* gamma;
+  const float* mean;
+  const float* invstd;
+  float* dgamma;
+  float* dbeta;
+  float* coef;  // [3][C]: dx = coef0*g + coef1*x + coef2
+  int accumulate;
+};
+
+__global__ __launch_bounds__(64) void bn_bwd_finalize_kernel(BwdFinalizeArgs p) {
+  const int c = blockIdx.x * 64 + threadIdx.x;
+  if (c >= p.C) return;
+  double s1 = 0.0, s2 = 0.0;
+  for (int b = 0; b < p.row_blocks; ++b) {
+    const float* src = p.partial + (static_cast<int64_t>(b) * p.C + c) * 2;
+    s1 += src[0];
+    s2 += src[1];
+  }
+  const float db = static_cast<float>(s1), dg = static_cast<float>(s2);
+  p.dbeta[c] = p.accumulate ? p.dbeta[c] + db : db;
+  p.dgamma[c] = p.accumulate ? p.dgamma[c] + dg : dg;
+  const double n = static_cast<double>(p.rows);
+  const double scale = static_cast<double>(p.gamma[c]) * p.invstd[c];
+  const double cb = -scale * p.invstd[c] * (s2 / n);
+  const double c0 = -scale * (s1 / n) - cb * p.mean[c];
+  p.coef[c] = static_cast<float>(scale);
+  p.coef[p.C + c] = static_cast<float>(cb);
+  p.coef[2 * p.C + c] = static_cast<float>(c0);
+}
+
+struct ApplyArgs {
+  const void* a;     // fwd: x         bwd: dy
+  const void* b;     // fwd: residual  bwd: relu mask   (may be null)
+  const void* x;     // bwd: x
+  void* out;         // fwd: y         bwd: dx
+  const float* c0;   // fwd: scale     bwd: coef0
+  const float* c1;   // fwd: shift     bwd: coef1
+  const float* c2;   //                bwd: coef2
+  int64_t chunks;
+  FastDiv div_cc;
+  int relu;
+};
+
+template <typename T, int BWD>
+__global__ __launch_bounds__(256) void bn_apply_kernel(ApplyArgs p) {
+  constexpr int E = Elem<T>::kPerChunk;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < p.chunks; i += stride) {
+    // chunk column: i % cc, evaluated on the low 31 bits when i is large
+    uint32_t colq, col;
+    if (i < 0x7fffffffll) {
+      p.div_cc.divmod(static_cast<uint32_t>(i), colq, col);
+    } else {
+      col = static_cast<uint32_t>(i % p.div_cc.d);
+    }
+    const int ch = col * E;
+    Chunk ca;
+    ca.u = static_cast<const uint4*>(p.a)[i];
+    float va[E], vo[E];
+    chunk_to_float<T>(ca, va);
+    if (BWD) {
+      Chunk cx;
+      cx.u = static_cast<const uint4*>(p.x)[i];
+      float vx[E];
+      chunk_to_float<T>(cx, vx);
+      if (p.b) {
+        Chunk cm;
+        cm.u = static_cast<const uint4*>(p.b)[i];
+        float vm[E];
+        chunk_to_float<T>(cm, vm);
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+          if (!(vm[e] > 0.f)) va[e] = 0.f;
+      }
+#pragma unroll
+      for (int e = 0; e < E; ++e) vo[e] = p.c0[ch + e] * va[e] + p.c1[ch + e] * vx[e] + p.c2[ch + e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < E; ++e) vo[e] = va[e] * p.c0[ch + e] + p.c1[ch + e];
+      if (p.b) {
+        Chunk cr;
+        cr.u = static_cast<const uint4*>(p.b)[i];
+        float vr[E];
+        chunk_to_float<T>(cr, vr);
+#pragma unroll
+        for (int e = 0; e < E; ++e) vo[e] += vr[e];
+      }
+      if (p.relu) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) vo[e] = vo[e] > 0.f ? vo[e] : 0.f;
+      }
+    }
+    static_cast<uint4*>(p.out)[i] = float_to_chunk<T>(vo).u;
+  }
+}
+
+struct Geometry {
+  int cc, ccb, col_blocks, rowlanes, row_blocks;
+  int64_t rows_per_block;
+};
+
+Geometry geometry(int64_t rows, int C, int dtype) {
+  const int E = dtype == kBF16 ? 8 : 4;
+  Geometry g;
+  g.cc = C / E;
+  int ccb = 1;
+  while (ccb < g.cc && ccb < 32) ccb <<= 1;
+  g.ccb = ccb;
+  g.col_blocks = (g.cc + ccb - 1) / ccb;
+  g.rowlanes = 256 / ccb;
+  int64_t rb = rows / (static_cast<int64_t>(g.rowlanes) * 8);
+  int64_t cap = 2048 / g.col_blocks;
+  if (cap < 1) cap = 1;
+  if (rb > cap) rb = cap;
+  if (rb < 1) rb = 1;
+  g.rows_per_block = (rows + rb - 1) / rb;
+  g.row_blocks = static_cast<int>((rows + g.rows_per_block - 1) / g.rows_per_block);
+  return g;
+}
+
+unsigned apply_blocks(int64_t chunks) {
+  int64_t b = (chunks + 255) / 256;
+  if (b > 8192) b = 8192;
+  if (b < 1) b = 1;
+  return static_cast<unsigned>(b);
+}
+
+int check_common(int64_t rows, int C, int dtype) {
+  TCH_CHECK_ARG(dtype == kBF16 || dtype == kF32, "bn: dtype must be f32(0) or bf16(1)");
+  const int E = dtype == kBF16 ? 8 : 4;
+  TCH_CHECK_ARG(rows > 0 && C > 0 && C % E == 0, "bn: C must be a positive multiple of a 16-byte chunk");
+  return 0;
+}
+
+}  // namespace
+
+int bn_partial_rows(int64_t rows, int C, int dtype) { return geometry(rows, C, dtype).row_blocks; }
+
+int64_t bn_workspace_bytes(int64_t rows, int C, int dtype) {
+  Geometry g = geometry(rows, C, dtype);
+  return (static_cast<int64_t>(g.row_blocks) * C * 2 + 3ll * C) * 4;
+}
+
+int bn_fwd_train(Context* ctx, int dtype, const void* x, void* y, const void* residual, int relu, int64_t rows, int C,
+                 const float* gamma, const float* beta, float* running_mean, float* running_var, float* save_mean,
+                 float* save_invstd, float momentum, float eps, float* workspace) {
+  if (int rc = check_common(rows, C, dtype)) return rc;
+  TCH_CHECK_ARG(x && y && gamma && beta && save_mean && save_invstd && workspace, "bn_fwd_train: null tensor");
+  TCH_CHECK_ARG((running_mean == nullptr) == (running_var == nullptr), "bn_fwd_train: running stats come in pairs");
+  Geometry g = geometry(rows, C, dtype);
+  float* partial = workspace;
+  float* scale = workspace + static_cast<int64_t>(g.row_blocks) * C * 2;
+  float* shift = scale + C;
+  ColReduceArgs r{x, nullptr, nullptr, nullptr, nullptr, partial, rows, C, g.cc, g.ccb, g.rowlanes, g.rows_per_block};
+  dim3 grid(g.col_blocks, g.row_blocks);
+  int rc = dtype == kBF16 ? launch(ctx, col_reduce_kernel<bf16, 0>, grid, dim3(256), r)
+                          : launch(ctx, col_reduce_kernel<float, 0>, grid, dim3(256), r);
+  if (rc) return rc;
+  FwdFinalizeArgs f{partial, g.row_blocks, C, rows, gamma, beta, running_mean, running_var, save_mean, save_invstd,
+                    scale,   shift,        momentum, eps};
+  rc = launch(ctx, bn_fwd_finalize_kernel, dim3((C + 63) / 64), dim3(64), f);
+  if (rc) return rc;
+  ApplyArgs a{x, residual, nullptr, y, scale, shift, nullptr, rows * g.cc, FastDiv(g.cc), relu};
+  return dtype == kBF16 ? launch(ctx, bn_apply_kernel<bf16, 0>, dim3(apply_blocks(a.chunks)), dim3(256), a)
+                        : launch(ctx, bn_apply_kernel<float, 0>, dim3(apply_blocks(a.chunks)), dim3(256), a);
+}
+
+int bn_bwd(Context* ctx, int dtype, const void* dy, const void* relu_mask, const void* x, void* dx, int64_t rows,
+           int C, const float* gamma, const float* save_mean, const float* save_invstd, float* dgamma, float* dbeta,
+           int accumulate, float* workspace) {
+  if (int rc = check_common(rows, C, dtype)) return rc;
+  TCH_CHECK_ARG(dy && x && dx && gamma && save_mean && save_invstd && dgamma && dbeta && workspace,
+                "bn_bwd: null tensor");
+  Geometry g = geometry(rows, C, dtype);
+  float* partial = workspace;
+  float* coef = workspace + static_cast<int64_t>(g.row_blocks) * C * 2;
+  ColReduceArgs r{dy, relu_mask, x, save_mean, save_invstd, partial, rows, C, g.cc, g.ccb, g.rowlanes, g.rows_per_block};
+  dim3 grid(g.col_blocks, g.row_blocks);
+  int rc = dtype == kBF16 ? launch(ctx, col_reduce_kernel<bf16, 1>, grid, dim3(256), r)
+                          : launch(ctx, col_reduce_kernel<float, 1>, grid, dim3(256), r);
+  if (rc) return rc;
+  BwdFinalizeArgs f{partial, g.row_blocks, C, rows, gamma, save_mean, save_invstd, dgamma, dbeta, coef, accumulate};
+  rc = launch(ctx, bn_bwd_finalize_kernel, dim3((C + 63) / 64), dim3(64), f);
+  if (rc) return rc;
+  ApplyArgs a{dy, relu_mask, x, dx, coef, coef + C, coef + 2 * C, rows * g.cc, FastDiv(g.cc), 0};
+  return dtype == kBF16 ? launch(ctx, bn_apply_kernel<bf16, 1>, dim3(apply_blocks(a.chunks)), dim3(256), a)
+                        : launch(ctx, bn_apply_kernel<float, 1>, dim3(apply_blocks(a.chunks)), dim3(256), a);
+}
+
+}  // namespace tch

@@ -1,0 +1,222 @@
+// Flat C ABI over the device operators, contexts, programs and launch queues.
+#include "../../include/torch_col_hip.h"
+
+#include "context.h"
+#include "ops.h"
+
+using namespace tch;
+
+struct tch_context {
+  Context ctx;
+  explicit tch_context(hipStream_t s) : ctx(s) {}
+};
+struct tch_program {
+  Program prog;
+};
+
+namespace {
+inline Context* C(tch_context* c) { return c ? &c->ctx : nullptr; }
+inline ConvShape shape(int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad) {
+  ConvShape s{N, H, W, Cc, K, R, S, stride, pad};
+  return s;
+}
+}  // namespace
+
+extern "C" {
+
+const char* tch_last_error(void) { return last_error(); }
+int tch_has_device_code(void) { return 1; }
+
+int tch_context_create(void* hip_stream, tch_context** out) {
+  if (!out) {
+    set_error("tch_context_create: null output");
+    return -22;
+  }
+  auto* c = new tch_context(static_cast<hipStream_t>(hip_stream));
+  c->ctx.queue = queue_for_stream(reinterpret_cast<uint64_t>(hip_stream));
+  *out = c;
+  return 0;
+}
+
+void tch_context_destroy(tch_context* ctx) { delete ctx; }
+
+uint64_t tch_context_take_rejected(tch_context* ctx) { return ctx ? ctx->ctx.rejected.exchange(0) : 0; }
+
+int tch_program_create(tch_program** out) {
+  if (!out) {
+    set_error("tch_program_create: null output");
+    return -22;
+  }
+  *out = new tch_program();
+  return 0;
+}
+
+void tch_program_destroy(tch_program* prog) { delete prog; }
+
+int64_t tch_program_size(const tch_program* prog) { return prog ? static_cast<int64_t>(prog->prog.launches.size()) : 0; }
+
+int tch_program_begin_record(tch_context* ctx, tch_program* prog) {
+  if (!ctx || !prog) {
+    set_error("tch_program_begin_record: null argument");
+    return -22;
+  }
+  if (ctx->ctx.recording) {
+    set_error("tch_program_begin_record: context is already recording");
+    return -16;
+  }
+  ctx->ctx.recording = &prog->prog;
+  return 0;
+}
+
+int tch_program_end_record(tch_context* ctx) {
+  if (!ctx || !ctx->ctx.recording) {
+    set_error("tch_program_end_record: context is not recording");
+    return -22;
+  }
+  ctx->ctx.recording = nullptr;
+  return 0;
+}
+
+int tch_program_run(tch_context* ctx, const tch_program* prog, int64_t first, int64_t last) {
+  if (!ctx || !prog) {
+    set_error("tch_program_run: null argument");
+    return -22;
+  }
+  if (ctx->ctx.recording) {
+    set_error("tch_program_run: context is recording");
+    return -16;
+  }
+  const int64_t n = static_cast<int64_t>(prog->prog.launches.size());
+  if (last < 0 || last > n) last = n;
+  if (first < 0 || first > last) {
+    set_error("tch_program_run: bad range");
+    return -22;
+  }
+  // the stream may have been registered after the context was made
+  ctx->ctx.queue = queue_for_stream(reinterpret_cast<uint64_t>(ctx->ctx.stream));
+  const uint64_t before = ctx->ctx.rejected.load();
+  for (int64_t i = first; i < last; ++i) {
+    int rc = ctx->ctx.dispatch(prog->prog.launches[static_cast<size_t>(i)]);
+    if (rc) return rc;
+  }
+  return ctx->ctx.rejected.load() != before ? 1 : 0;
+}
+
+uint64_t tch_RegisterStream(uint64_t hip_stream) { return register_stream(hip_stream); }
+int tch_UnRegisterStream(uint64_t hip_stream) { return unregister_stream(hip_stream); }
+void tch_UnRegisterAllStreams(void) { unregister_all_streams(); }
+size_t tch_GetXQueueSize(uint64_t hip_stream) { return queue_size(hip_stream); }
+size_t tch_GetXQueueSizeAllStreams(void) { return queue_size_all_streams(); }
+size_t tch_GetTotalXQueueSize(void) { return queue_size_all_streams(); }
+size_t tch_AbortStream(uint64_t hip_stream) { return abort_stream(hip_stream); }
+size_t tch_AbortAllStreams(void) { return abort_all_streams(); }
+int tch_SyncStream(uint64_t hip_stream) { return sync_stream(hip_stream); }
+int tch_SyncAllStreams(void) { return sync_all_streams(); }
+int tch_QueryRejectCudaCalls(void) { return query_reject_calls() ? 1 : 0; }
+void tch_SetRejectCudaCalls(int reject) { set_reject_calls(reject != 0); }
+void tch_SetXQueueShape(int queue_length, int sync_interval) { set_queue_shape(queue_length, sync_interval); }
+size_t tch_GetXQueueInFlight(uint64_t hip_stream) {
+  auto q = queue_for_stream(hip_stream);
+  return q ? q->in_flight() : 0;
+}
+
+int tch_conv2d_fwd(tch_context* ctx, int dtype, const void* x, const void* w, void* y, const void* add,
+                   const void* mask, const float* bias, int out_f32, int N, int H, int W, int Cc, int K, int R, int S,
+                   int stride, int pad, int tile_cfg) {
+  return conv2d_fwd(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad), x, w, y, add, mask, bias, out_f32,
+                    tile_cfg);
+}
+
+int tch_conv2d_dgrad(tch_context* ctx, int dtype, const void* dy, const void* w, void* dx, const void* add,
+                     const void* mask, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad,
+                     int tile_cfg) {
+  return conv2d_dgrad(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad), dy, w, dx, add, mask, tile_cfg);
+}
+
+int tch_conv2d_wgrad_pick_splits(int dtype, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad) {
+  return conv2d_wgrad_pick_splits(shape(N, H, W, Cc, K, R, S, stride, pad), dtype);
+}
+
+int64_t tch_conv2d_wgrad_workspace_bytes(int dtype, int K, int R, int S, int Cc, int splits) {
+  return conv2d_wgrad_workspace_bytes(shape(1, 1, 1, Cc, K, R, S, 1, 0), dtype, splits);
+}
+
+int tch_conv2d_wgrad(tch_context* ctx, int dtype, const void* x, const void* dy, float* dw, float* workspace,
+                     int splits, int accumulate, int N, int H, int W, int Cc, int K, int R, int S, int stride,
+                     int pad, int tile_cfg) {
+  ConvShape s = shape(N, H, W, Cc, K, R, S, stride, pad);
+  if (splits <= 0) splits = workspace ? conv2d_wgrad_pick_splits(s, dtype) : 1;
+  return conv2d_wgrad(C(ctx), dtype, s, x, dy, dw, workspace, splits, accumulate, tile_cfg);
+}
+
+int64_t tch_bn_workspace_bytes(int dtype, int64_t rows, int Cc) { return bn_workspace_bytes(rows, Cc, dtype); }
+
+int tch_bn_fwd_train(tch_context* ctx, int dtype, const void* x, void* y, const void* residual, int relu,
+                     int64_t rows, int Cc, const float* gamma, const float* beta, float* running_mean,
+                     float* running_var, float* save_mean, float* save_invstd, float momentum, float eps,
+                     float* workspace) {
+  return bn_fwd_train(C(ctx), dtype, x, y, residual, relu, rows, Cc, gamma, beta, running_mean, running_var,
+                      save_mean, save_invstd, momentum, eps, workspace);
+}
+
+int tch_bn_bwd(tch_context* ctx, int dtype, const void* dy, const void* relu_mask, const void* x, void* dx,
+               int64_t rows, int Cc, const float* gamma, const float* save_mean, const float* save_invstd,
+               float* dgamma, float* dbeta, int accumulate, float* workspace) {
+  return bn_bwd(C(ctx), dtype, dy, relu_mask, x, dx, rows, Cc, gamma, save_mean, save_invstd, dgamma, dbeta,
+                accumulate, workspace);
+}
+
+int tch_maxpool_fwd(tch_context* ctx, int dtype, const void* x, void* y, int32_t* index, int N, int H, int W, int Cc,
+                    int ksize, int stride, int pad) {
+  return maxpool_fwd(C(ctx), dtype, x, y, index, N, H, W, Cc, ksize, stride, pad);
+}
+
+int tch_maxpool_bwd(tch_context* ctx, int dtype, const void* dy, const int32_t* index, void* dx, int N, int H, int W,
+                    int Cc, int ksize, int stride, int pad) {
+  return maxpool_bwd(C(ctx), dtype, dy, index, dx, N, H, W, Cc, ksize, stride, pad);
+}
+
+int tch_avgpool_fwd(tch_context* ctx, int dtype, const void* x, void* y, int N, int HW, int Cc) {
+  return avgpool_fwd(C(ctx), dtype, x, y, N, HW, Cc);
+}
+
+int tch_avgpool_bwd(tch_context* ctx, int dtype, const void* dy, void* dx, int N, int HW, int Cc) {
+  return avgpool_bwd(C(ctx), dtype, dy, dx, N, HW, Cc);
+}
+
+int tch_softmax_ce_fwd_bwd(tch_context* ctx, int dtype, const float* logits, const int64_t* labels, float* loss_rows,
+                           float* loss_mean, void* dlogits, int rows, int classes, int ld_dlogits, float grad_scale) {
+  return softmax_ce_fwd_bwd(C(ctx), dtype, logits, labels, loss_rows, loss_mean, dlogits, rows, classes, ld_dlogits,
+                            grad_scale);
+}
+
+int tch_sgd_momentum_step(tch_context* ctx, float* param, const float* grad, float* momentum_buf, void* shadow_bf16,
+                          int64_t n, float lr, float momentum, float weight_decay) {
+  return sgd_momentum_step(C(ctx), param, grad, momentum_buf, shadow_bf16, n, lr, momentum, weight_decay);
+}
+
+int tch_grad_accumulate(tch_context* ctx, float* global, float* grad, int64_t n) {
+  return grad_accumulate(C(ctx), global, grad, n);
+}
+
+int tch_fill_zero(tch_context* ctx, void* ptr, int64_t bytes) { return fill_zero(C(ctx), ptr, bytes); }
+
+int tch_bias_grad(tch_context* ctx, int dtype, const void* dy, float* dbias, int rows, int cols, int ld,
+                  int accumulate) {
+  return bias_grad(C(ctx), dtype, dy, dbias, rows, cols, ld, accumulate);
+}
+
+int tch_nchw_to_nhwc_pad(tch_context* ctx, int dtype, const float* x_nchw, void* y_nhwc, int N, int Cc, int H, int W,
+                         int Cpad) {
+  return nchw_to_nhwc_pad(C(ctx), dtype, x_nchw, y_nhwc, N, Cc, H, W, Cpad);
+}
+
+int tch_cast_from_f32(tch_context* ctx, int dtype, const float* src, void* dst, int64_t n) {
+  return cast_f32(C(ctx), dtype, src, dst, n);
+}
+
+int tch_cast_to_f32(tch_context* ctx, int dtype, const void* src, float* dst, int64_t n) {
+  return cast_to_f32(C(ctx), dtype, src, dst, n);
+}
+
+}  // extern "C"

@@ -1,0 +1,340 @@
+#include "context.h"
+
+#include <string.h>
+
+#include <map>
+
+namespace tch {
+
+namespace {
+thread_local std::string g_error;
+std::atomic<bool> g_reject{false};
+std::mutex g_stream_mu;
+std::map<uint64_t, std::shared_ptr<LaunchQueue>> g_streams;
+int g_queue_length = 16;
+int g_sync_interval = 8;
+
+int launch_now(hipStream_t stream, const LaunchRecord& rec) {
+  void* args[1] = {const_cast<unsigned char*>(rec.args)};
+  hipError_t e = hipLaunchKernel(rec.fn, rec.grid, rec.block, args, 0, stream);
+  if (e != hipSuccess) {
+    set_error(std::string("hipLaunchKernel failed: ") + hipGetErrorString(e));
+    return -5;
+  }
+  return 0;
+}
+}  // namespace
+
+void set_error(const std::string& msg) { g_error = msg; }
+const char* last_error() { return g_error.c_str(); }
+
+// ---------------------------------------------------------------------------
+// LaunchQueue
+// ---------------------------------------------------------------------------
+
+LaunchQueue::LaunchQueue(hipStream_t stream, int queue_length, int sync_interval)
+    : stream_(stream),
+      queue_length_(queue_length < 1 ? 1 : static_cast<size_t>(queue_length)),
+      sync_interval_(sync_interval < 1 ? 1 : static_cast<uint64_t>(sync_interval)) {
+  if (hipGetDevice(&device_) != hipSuccess) device_ = 0;
+  worker_ = std::thread([this] { worker_loop(); });
+}
+
+LaunchQueue::~LaunchQueue() {
+  {
+    std::lock_guard<std::mutex> lock(mu_);
+    stop_ = true;
+  }
+  cv_work_.notify_all();
+  if (worker_.joinable()) worker_.join();
+  for (auto& l : log_)
+    if (l.event) (void)hipEventDestroy(l.event);
+  for (auto e : free_events_) (void)hipEventDestroy(e);
+}
+
+void LaunchQueue::submit(const LaunchRecord& rec) {
+  {
+    std::lock_guard<std::mutex> lock(mu_);
+    wait_.emplace_back();
+    wait_.back().rec = rec;
+  }
+  cv_work_.notify_one();
+}
+
+size_t LaunchQueue::clear() {
+  std::lock_guard<std::mutex> lock(mu_);
+  size_t removed = 0;
+  for (auto it = wait_.begin(); it != wait_.end();) {
+    if (!it->is_sync) {
+      it = wait_.erase(it);
+      ++removed;
+    } else {
+      ++it;
+    }
+  }
+  return removed;
+}
+
+int LaunchQueue::synchronize() {
+  std::unique_lock<std::mutex> lock(mu_);
+  if (stop_) return 0;
+  const uint64_t ticket = next_ticket_++;
+  wait_.emplace_back();
+  wait_.back().is_sync = true;
+  wait_.back().sync_ticket = ticket;
+  cv_work_.notify_one();
+  cv_done_.wait(lock, [&] { return done_ticket_ >= ticket; });
+  return error_.load();
+}
+
+size_t LaunchQueue::size() {
+  std::lock_guard<std::mutex> lock(mu_);
+  size_t n = 0;
+  for (auto& it : wait_)
+    if (!it.is_sync) ++n;
+  return n;
+}
+
+size_t LaunchQueue::in_flight() { return in_flight_.load(); }
+
+hipEvent_t LaunchQueue::take_event() {
+  if (!free_events_.empty()) {
+    hipEvent_t e = free_events_.back();
+    free_events_.pop_back();
+    return e;
+  }
+  hipEvent_t e = nullptr;
+  if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess) return nullptr;
+  return e;
+}
+
+// Wait on the oldest sync point so that at most `keep` commands stay logged.
+void LaunchQueue::drain_log_until(size_t keep) {
+  while (log_.size() > keep) {
+    size_t pos = 0;
+    bool found = false;
+    for (; pos < log_.size(); ++pos) {
+      if (log_[pos].event) {
+        found = true;
+        break;
+      }
+    }
+    if (found) {
+      hipError_t e = hipEventSynchronize(log_[pos].event);
+      if (e != hipSuccess) error_.store(static_cast<int>(e));
+      for (size_t i = 0; i <= pos; ++i) {
+        if (log_.front().event) free_events_.push_back(log_.front().event);
+        log_.pop_front();
+      }
+    } else {
+      hipError_t e = hipStreamSynchronize(stream_);
+      if (e != hipSuccess) error_.store(static_cast<int>(e));
+      log_.clear();
+    }
+  }
+  in_flight_.store(log_.size());
+}
+
+void LaunchQueue::launch_one(const LaunchRecord& rec) {
+  if (log_.size() >= queue_length_) drain_log_until(queue_length_ - 1);
+  void* args[1] = {const_cast<unsigned char*>(rec.args)};
+  hipError_t e = hipLaunchKernel(rec.fn, rec.grid, rec.block, args, 0, stream_);
+  if (e != hipSuccess) {
+    error_.store(static_cast<int>(e));
+    return;
+  }
+  const uint64_t idx = ++next_idx_;
+  hipEvent_t ev = nullptr;
+  if (idx - last_sync_idx_ >= sync_interval_) {
+    ev = take_event();
+    if (ev && hipEventRecord(ev, stream_) == hipSuccess) {
+      last_sync_idx_ = idx;
+    } else if (ev) {
+      free_events_.push_back(ev);
+      ev = nullptr;
+    }
+  }
+  log_.push_back(Logged{idx, ev});
+  in_flight_.store(log_.size());
+  submitted_total_.fetch_add(1);
+}
+
+void LaunchQueue::worker_loop() {
+  (void)hipSetDevice(device_);
+  for (;;) {
+    Item item;
+    {
+      std::unique_lock<std::mutex> lock(mu_);
+      cv_work_.wait(lock, [&] { return stop_ || !wait_.empty(); });
+      if (wait_.empty()) {
+        if (stop_) break;
+        continue;
+      }
+      item = wait_.front();
+      wait_.pop_front();
+    }
+    if (item.is_sync) {
+      hipError_t e = hipStreamSynchronize(stream_);
+      if (e != hipSuccess) error_.store(static_cast<int>(e));
+      for (auto& l : log_)
+        if (l.event) free_events_.push_back(l.event);
+      log_.clear();
+      in_flight_.store(0);
+      {
+        std::lock_guard<std::mutex> lock(mu_);
+        done_ticket_ = item.sync_ticket;
+      }
+      cv_done_.notify_all();
+    } else {
+      launch_one(item.rec);
+    }
+  }
+  // release waiters that raced with shutdown
+  {
+    std::lock_guard<std::mutex> lock(mu_);
+    done_ticket_ = next_ticket_;
+  }
+  cv_done_.notify_all();
+}
+
+// ---------------------------------------------------------------------------
+// Context
+// ---------------------------------------------------------------------------
+
+int Context::dispatch(const LaunchRecord& rec) {
+  if (g_reject.load(std::memory_order_acquire)) {
+    rejected.fetch_add(1);
+    return 0;
+  }
+  if (queue) {
+    queue->submit(rec);
+    return 0;
+  }
+  return launch_now(stream, rec);
+}
+
+int submit(Context* ctx, const void* fn, dim3 grid, dim3 block, const void* args, size_t arg_bytes) {
+  if (!ctx) {
+    set_error("null context");
+    return -22;
+  }
+  if (grid.x == 0 || grid.y == 0 || grid.z == 0 || block.x == 0 || block.x * block.y * block.z > 1024) {
+    set_error("launch with an empty grid or an oversized block");
+    return -22;
+  }
+  LaunchRecord rec;
+  rec.fn = fn;
+  rec.grid = grid;
+  rec.block = block;
+  rec.arg_bytes = static_cast<uint32_t>(arg_bytes);
+  memcpy(rec.args, args, arg_bytes);
+  if (ctx->recording) {
+    ctx->recording->launches.push_back(rec);
+    return 0;
+  }
+  return ctx->dispatch(rec);
+}
+
+// ---------------------------------------------------------------------------
+// stream registry
+// ---------------------------------------------------------------------------
+
+void set_queue_shape(int queue_length, int sync_interval) {
+  std::lock_guard<std::mutex> lock(g_stream_mu);
+  g_queue_length = queue_length < 1 ? 1 : queue_length;
+  g_sync_interval = sync_interval < 1 ? 1 : sync_interval;
+}
+
+uint64_t register_stream(uint64_t stream) {
+  std::lock_guard<std::mutex> lock(g_stream_mu);
+  if (g_streams.count(stream)) {
+    set_error("stream already registered");
+    return 0;
+  }
+  auto q = std::make_shared<LaunchQueue>(reinterpret_cast<hipStream_t>(stream), g_queue_length, g_sync_interval);
+  g_streams[stream] = q;
+  return reinterpret_cast<uint64_t>(q.get());
+}
+
+int unregister_stream(uint64_t stream) {
+  std::shared_ptr<LaunchQueue> q;
+  {
+    std::lock_guard<std::mutex> lock(g_stream_mu);
+    auto it = g_streams.find(stream);
+    if (it == g_streams.end()) {
+      set_error("stream not registered");
+      return -2;
+    }
+    q = it->second;
+    g_streams.erase(it);
+  }
+  q->synchronize();
+  return 0;
+}
+
+void unregister_all_streams() {
+  std::map<uint64_t, std::shared_ptr<LaunchQueue>> taken;
+  {
+    std::lock_guard<std::mutex> lock(g_stream_mu);
+    taken.swap(g_streams);
+  }
+  for (auto& kv : taken) kv.second->synchronize();
+}
+
+std::shared_ptr<LaunchQueue> queue_for_stream(uint64_t stream) {
+  std::lock_guard<std::mutex> lock(g_stream_mu);
+  auto it = g_streams.find(stream);
+  return it == g_streams.end() ? nullptr : it->second;
+}
+
+size_t abort_stream(uint64_t stream) {
+  auto q = queue_for_stream(stream);
+  return q ? q->clear() : 0;
+}
+
+size_t abort_all_streams() {
+  std::lock_guard<std::mutex> lock(g_stream_mu);
+  size_t total = 0;
+  for (auto& kv : g_streams) total += kv.second->clear();
+  return total;
+}
+
+int sync_stream(uint64_t stream) {
+  auto q = queue_for_stream(stream);
+  if (!q) {
+    set_error("stream not registered");
+    return -2;
+  }
+  return q->synchronize();
+}
+
+int sync_all_streams() {
+  std::vector<std::shared_ptr<LaunchQueue>> qs;
+  {
+    std::lock_guard<std::mutex> lock(g_stream_mu);
+    for (auto& kv : g_streams) qs.push_back(kv.second);
+  }
+  int rc = 0;
+  for (auto& q : qs) {
+    int r = q->synchronize();
+    if (r) rc = r;
+  }
+  return rc;
+}
+
+size_t queue_size(uint64_t stream) {
+  auto q = queue_for_stream(stream);
+  return q ? q->size() : 0;
+}
+
+size_t queue_size_all_streams() {
+  std::lock_guard<std::mutex> lock(g_stream_mu);
+  size_t total = 0;
+  for (auto& kv : g_streams) total += kv.second->size();
+  return total;
+}
+
+void set_reject_calls(bool reject) { g_reject.store(reject, std::memory_order_release); }
+bool query_reject_calls() { return g_reject.load(std::memory_order_acquire); }
+
+}  // namespace tch

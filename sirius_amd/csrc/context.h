@@ -1,0 +1,124 @@
+// Execution context of the device operators: which HIP stream launches go to,
+// whether they pass through a preemptible launch queue, and whether they are
+// being recorded into a replayable program instead of being launched.
+//
+// The launch queue restates, for HIP and without interposing on the driver,
+// what the reference gets from xsched in STOP_SUBMISSION mode
+// (common/xsched_ctrl.cc:27-46 creates the queue with length 16 and sync
+// interval 8; third_party/xsched/preempt/xqueue/worker.cpp:155-260 bounds the
+// commands in flight; xqueue.cpp:150-152 / wait_queue.cpp:135-148 erase the
+// not-yet-submitted ones on abort; shim/cuda/intercept.cpp:20-22 turns every
+// call into a successful no-op while the reject flag is set).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <condition_variable>
+#include <deque>
+#include <memory>
+#include <mutex>
+#include <thread>
+#include <vector>
+
+#include "kernels.h"
+
+namespace tch {
+
+class LaunchQueue {
+ public:
+  LaunchQueue(hipStream_t stream, int queue_length, int sync_interval);
+  ~LaunchQueue();
+  LaunchQueue(const LaunchQueue&) = delete;
+  LaunchQueue& operator=(const LaunchQueue&) = delete;
+
+  void submit(const LaunchRecord& rec);
+  // Erase every launch that has not been handed to the hardware queue yet.
+  size_t clear();
+  // Wait until everything submitted before this call has finished on the GPU.
+  // Returns 0 on success, a HIP error code otherwise.
+  int synchronize();
+  // Launches still waiting in the software queue.
+  size_t size();
+  // Launches handed to the stream and not yet known to be complete.
+  size_t in_flight();
+  hipStream_t stream() const { return stream_; }
+  int sticky_error() const { return error_.load(); }
+  uint64_t submitted_total() const { return submitted_total_.load(); }
+
+ private:
+  struct Item {
+    bool is_sync = false;
+    uint64_t sync_ticket = 0;
+    LaunchRecord rec;
+  };
+  struct Logged {
+    uint64_t idx;
+    hipEvent_t event;  // nullptr unless this command carries a sync point
+  };
+  void worker_loop();
+  void launch_one(const LaunchRecord& rec);
+  void drain_log_until(size_t keep);
+  hipEvent_t take_event();
+
+  hipStream_t stream_;
+  const size_t queue_length_;
+  const uint64_t sync_interval_;
+  int device_ = 0;
+
+  std::mutex mu_;
+  std::condition_variable cv_work_;
+  std::condition_variable cv_done_;
+  std::deque<Item> wait_;
+  bool stop_ = false;
+  uint64_t next_ticket_ = 1;
+  uint64_t done_ticket_ = 0;
+
+  // worker-private
+  std::deque<Logged> log_;
+  std::vector<hipEvent_t> free_events_;
+  uint64_t next_idx_ = 0;
+  uint64_t last_sync_idx_ = 0;
+
+  std::atomic<size_t> in_flight_{0};
+  std::atomic<int> error_{0};
+  std::atomic<uint64_t> submitted_total_{0};
+  std::thread worker_;
+};
+
+// A recorded sequence of launches, replayed through a context.
+struct Program {
+  std::vector<LaunchRecord> launches;
+};
+
+class Context {
+ public:
+  explicit Context(hipStream_t s) : stream(s) {}
+  hipStream_t stream;
+  // set while the stream is registered for preemption; owned by the registry
+  std::shared_ptr<LaunchQueue> queue;
+  Program* recording = nullptr;
+  // launches skipped because the reject flag was up since the last reset
+  std::atomic<uint64_t> rejected{0};
+
+  int dispatch(const LaunchRecord& rec);
+};
+
+// ---- process-wide registry of preemptible streams (xsched_ctrl equivalent) ----
+uint64_t register_stream(uint64_t stream);  // returns a handle, 0 on failure
+int unregister_stream(uint64_t stream);
+void unregister_all_streams();
+std::shared_ptr<LaunchQueue> queue_for_stream(uint64_t stream);
+size_t abort_stream(uint64_t stream);
+size_t abort_all_streams();
+int sync_stream(uint64_t stream);
+int sync_all_streams();
+size_t queue_size(uint64_t stream);
+size_t queue_size_all_streams();
+void set_reject_calls(bool reject);
+bool query_reject_calls();
+void set_queue_shape(int queue_length, int sync_interval);
+
+const char* last_error();
+
+}  // namespace tch

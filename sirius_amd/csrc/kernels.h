@@ -1,0 +1,202 @@
+// Shared device-side helpers and the host-side launch plumbing for the HIP
+// kernels of the colocated training step (gfx950 / CDNA4 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+#include <type_traits>
+
+namespace tch {
+
+// ---------------------------------------------------------------------------
+// element types
+// ---------------------------------------------------------------------------
+
+// bf16 is kept as raw bits in memory; arithmetic is always done in fp32.
+struct bf16 {
+  uint16_t v;
+};
+
+enum DType : int { kF32 = 0, kBF16 = 1 };
+
+__host__ __device__ inline float bf16_bits_to_float(uint16_t b) {
+  union {
+    uint32_t u;
+    float f;
+  } c;
+  c.u = static_cast<uint32_t>(b) << 16;
+  return c.f;
+}
+
+// round-to-nearest-even, NaN stays NaN (quiet bit forced)
+__host__ __device__ inline uint16_t float_to_bf16_bits(float f) {
+  union {
+    uint32_t u;
+    float f;
+  } c;
+  c.f = f;
+  uint32_t u = c.u;
+  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return static_cast<uint16_t>(u >> 16);
+}
+
+template <typename T>
+struct Elem;
+template <>
+struct Elem<float> {
+  static constexpr int kPerChunk = 4;  // elements in one 16-byte chunk
+  __device__ static inline float load(const float* p) { return *p; }
+  __device__ static inline void store(float* p, float v) { *p = v; }
+};
+template <>
+struct Elem<bf16> {
+  static constexpr int kPerChunk = 8;
+  __device__ static inline float load(const bf16* p) { return bf16_bits_to_float(p->v); }
+  __device__ static inline void store(bf16* p, float v) { p->v = float_to_bf16_bits(v); }
+};
+
+// A 16-byte chunk as it travels global -> register -> LDS -> MFMA operand.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+
+union Chunk {
+  uint4 u;
+  uint32_t w[4];
+  float f[4];
+  bf16x8_t h;
+};
+
+__device__ inline Chunk zero_chunk() {
+  Chunk c;
+  c.u = make_uint4(0u, 0u, 0u, 0u);
+  return c;
+}
+
+// unpack a chunk into fp32 lanes (E = 4 or 8)
+template <typename T>
+__device__ inline void chunk_to_float(const Chunk& c, float* out);
+template <>
+__device__ inline void chunk_to_float<float>(const Chunk& c, float* out) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) out[i] = c.f[i];
+}
+template <>
+__device__ inline void chunk_to_float<bf16>(const Chunk& c, float* out) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    out[2 * i] = __uint_as_float(c.w[i] << 16);
+    out[2 * i + 1] = __uint_as_float(c.w[i] & 0xffff0000u);
+  }
+}
+template <typename T>
+__device__ inline Chunk float_to_chunk(const float* in);
+template <>
+__device__ inline Chunk float_to_chunk<float>(const float* in) {
+  Chunk c;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) c.f[i] = in[i];
+  return c;
+}
+template <>
+__device__ inline Chunk float_to_chunk<bf16>(const float* in) {
+  Chunk c;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    c.w[i] = static_cast<uint32_t>(float_to_bf16_bits(in[2 * i])) |
+             (static_cast<uint32_t>(float_to_bf16_bits(in[2 * i + 1])) << 16);
+  return c;
+}
+
+// ---------------------------------------------------------------------------
+// division by a run-time constant without the integer divider
+// valid for dividends in [0, 2^31)
+// ---------------------------------------------------------------------------
+struct FastDiv {
+  uint32_t mul;
+  uint32_t shr;
+  uint32_t d;
+  __host__ __device__ FastDiv() : mul(0), shr(0), d(1) {}
+  __host__ explicit FastDiv(uint32_t denom) : mul(0), shr(0), d(denom) {
+    if (denom > 1) {
+      uint32_t lg = 0;
+      while ((1u << lg) < denom) ++lg;  // ceil(log2(denom))
+      // p = 31 + ceil(log2(d)); m = ceil(2^p / d); fits 32 bits for d >= 2
+      unsigned p = 31 + lg;  // <= 62, so 2^p fits 64 bits
+      uint64_t m = ((1ull << p) + denom - 1) / denom;
+      mul = static_cast<uint32_t>(m);
+      shr = p - 32;
+    }
+  }
+  __device__ inline uint32_t div(uint32_t n) const { return d == 1 ? n : (__umulhi(n, mul) >> shr); }
+  __device__ inline void divmod(uint32_t n, uint32_t& q, uint32_t& r) const {
+    q = div(n);
+    r = n - q * d;
+  }
+};
+
+// ---------------------------------------------------------------------------
+// wavefront reductions (64 lanes)
+// ---------------------------------------------------------------------------
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+__device__ inline float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+// Workgroups are dealt round-robin to the 8 XCDs (each with a private L2).
+// Remap the hardware workgroup id so that CONSECUTIVE logical ids land on the
+// same XCD: neighbouring tiles then share operand rows through one L2.
+__device__ inline uint32_t xcd_remap(uint32_t wg, uint32_t nwg) {
+  constexpr uint32_t kXcd = 8;
+  uint32_t xcd = wg % kXcd;
+  uint32_t local = wg / kXcd;
+  uint32_t q = nwg / kXcd, rem = nwg % kXcd;
+  uint32_t start = xcd * q + (xcd < rem ? xcd : rem);
+  return start + local;
+}
+
+// ---------------------------------------------------------------------------
+// host side: launch sink
+// ---------------------------------------------------------------------------
+
+// Every kernel in this library takes exactly ONE trivially copyable argument
+// struct by value, so a launch is (function, grid, block, bytes-of-args) and
+// can be queued, recorded and replayed without knowing the kernel.
+struct LaunchRecord {
+  const void* fn;
+  dim3 grid;
+  dim3 block;
+  uint32_t arg_bytes;
+  alignas(16) unsigned char args[360];
+};
+
+class Context;  // defined in context.h
+
+int submit(Context* ctx, const void* fn, dim3 grid, dim3 block, const void* args, size_t arg_bytes);
+
+template <typename Args>
+inline int launch(Context* ctx, void (*kernel)(Args), dim3 grid, dim3 block, const Args& args) {
+  static_assert(sizeof(Args) <= sizeof(LaunchRecord::args), "kernel argument struct too large");
+  static_assert(std::is_trivially_copyable<Args>::value, "kernel arguments must be POD");
+  return submit(ctx, reinterpret_cast<const void*>(kernel), grid, block, &args, sizeof(Args));
+}
+
+void set_error(const std::string& msg);
+
+#define TCH_CHECK_ARG(cond, msg)                       \
+  do {                                                 \
+    if (!(cond)) {                                     \
+      ::tch::set_error(std::string("invalid argument: ") + (msg)); \
+      return -22;                                      \
+    }                                                  \
+  } while (0)
+
+}  // namespace tch

@@ -1,0 +1,212 @@
+// Fused softmax-cross-entropy (forward + gradient in one pass over the
+// logits), fused SGD-momentum over a flat fp32 parameter buffer with a bf16
+// shadow copy, the micro-batch gradient accumulator, and small helpers.
+// All HBM-bound.
+//
+// Restated arithmetic and its reference call sites:
+//   nn.CrossEntropyLoss (mean)              train/swin_b.py:42, train/resnet152.py:26
+//   loss /= global_batch / batch            pytorch/torch_col/dynamic_batch.py:112-120
+//   torch.optim.SGD(momentum, weight_decay) train/resnet152.py:27-28,
+//     with momentum buffers pre-zeroed      pytorch/torch_col/util.py:182-191
+//   GradAccumulator.accumulate              pytorch/torch_col/accumulate.py:20-24
+#include "kernels.h"
+#include "ops.h"
+
+namespace tch {
+namespace {
+
+struct CeArgs {
+  const float* logits;
+  const int64_t* labels;
+  float* loss_rows;
+  void* dlogits;
+  int rows, classes, ld;
+  float grad_scale;  // d(loss_mean * loss_scale)/d(loss_row) = loss_scale / rows
+};
+
+// one wavefront per row
+template <typename T>
+__global__ __launch_bounds__(64) void softmax_ce_kernel(CeArgs p) {
+  const int row = blockIdx.x;
+  const int lane = threadIdx.x;
+  const float* z = p.logits + static_cast<int64_t>(row) * p.classes;
+  float mx = -INFINITY;
+  for (int c = lane; c < p.classes; c += 64) mx = fmaxf(mx, z[c]);
+  mx = wave_max(mx);
+  float sum = 0.f;
+  for (int c = lane; c < p.classes; c += 64) sum += expf(z[c] - mx);
+  sum = wave_sum(sum);
+  const float lse = mx + logf(sum);
+  const int label = static_cast<int>(p.labels[row]);
+  if (lane == 0) p.loss_rows[row] = lse - z[label];
+  T* g = static_cast<T*>(p.dlogits) + static_cast<int64_t>(row) * p.ld;
+  const float inv = 1.f / sum;
+  for (int c = lane; c < p.classes; c += 64) {
+    float sm = expf(z[c] - mx) * inv;
+    Elem<T>::store(g + c, (sm - (c == label ? 1.f : 0.f)) * p.grad_scale);
+  }
+}
+
+struct MeanArgs {
+  const float* in;
+  float* out;
+  int n;
+};
+
+__global__ __launch_bounds__(64) void mean_kernel(MeanArgs p) {
+  float s = 0.f;
+  for (int i = threadIdx.x; i < p.n; i += 64) s += p.in[i];
+  s = wave_sum(s);
+  if (threadIdx.x == 0) *p.out = s / static_cast<float>(p.n);
+}
+
+struct SgdArgs {
+  float* param;
+  const float* grad;
+  float* buf;
+  uint16_t* shadow;
+  int64_t n;
+  float lr, momentum, wd;
+};
+
+__global__ __launch_bounds__(256) void sgd_kernel(SgdArgs p) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * 256 * 4;
+  for (int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4; i < p.n; i += stride) {
+    if (i + 4 <= p.n) {
+      float4 w = *reinterpret_cast<float4*>(p.param + i);
+      float4 g = *reinterpret_cast<const float4*>(p.grad + i);
+      float4 b = *reinterpret_cast<float4*>(p.buf + i);
+      b.x = p.momentum * b.x + (g.x + p.wd * w.x);
+      b.y = p.momentum * b.y + (g.y + p.wd * w.y);
+      b.z = p.momentum * b.z + (g.z + p.wd * w.z);
+      b.w = p.momentum * b.w + (g.w + p.wd * w.w);
+      w.x -= p.lr * b.x;
+      w.y -= p.lr * b.y;
+      w.z -= p.lr * b.z;
+      w.w -= p.lr * b.w;
+      *reinterpret_cast<float4*>(p.param + i) = w;
+      *reinterpret_cast<float4*>(p.buf + i) = b;
+      if (p.shadow) {
+        uint2 s;
+        s.x = float_to_bf16_bits(w.x) | (static_cast<uint32_t>(float_to_bf16_bits(w.y)) << 16);
+        s.y = float_to_bf16_bits(w.z) | (static_cast<uint32_t>(float_to_bf16_bits(w.w)) << 16);
+        *reinterpret_cast<uint2*>(p.shadow + i) = s;
+      }
+    } else {
+      for (int64_t j = i; j < p.n; ++j) {
+        float w = p.param[j];
+        float b = p.momentum * p.buf[j] + (p.grad[j] + p.wd * w);
+        w -= p.lr * b;
+        p.param[j] = w;
+        p.buf[j] = b;
+        if (p.shadow) p.shadow[j] = float_to_bf16_bits(w);
+      }
+    }
+  }
+}
+
+struct AccumArgs {
+  float* global;
+  float* grad;
+  int64_t n;
+};
+
+// global += grad; grad = 0
+__global__ __launch_bounds__(256) void accumulate_kernel(AccumArgs p) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * 256 * 4;
+  for (int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4; i < p.n; i += stride) {
+    if (i + 4 <= p.n) {
+      float4 a = *reinterpret_cast<float4*>(p.global + i);
+      float4 g = *reinterpret_cast<float4*>(p.grad + i);
+      a.x += g.x;
+      a.y += g.y;
+      a.z += g.z;
+      a.w += g.w;
+      *reinterpret_cast<float4*>(p.global + i) = a;
+      *reinterpret_cast<float4*>(p.grad + i) = make_float4(0.f, 0.f, 0.f, 0.f);
+    } else {
+      for (int64_t j = i; j < p.n; ++j) {
+        p.global[j] += p.grad[j];
+        p.grad[j] = 0.f;
+      }
+    }
+  }
+}
+
+struct FillArgs {
+  uint32_t* ptr;
+  int64_t words;
+};
+
+__global__ __launch_bounds__(256) void fill_zero_kernel(FillArgs p) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < p.words; i += stride) p.ptr[i] = 0u;
+}
+
+struct BiasGradArgs {
+  const void* dy;
+  float* dbias;
+  int rows, cols, ld, accumulate;
+};
+
+// one lane per column; rows are few (the batch)
+template <typename T>
+__global__ __launch_bounds__(256) void bias_grad_kernel(BiasGradArgs p) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= p.cols) return;
+  float s = 0.f;
+  const T* src = static_cast<const T*>(p.dy) + c;
+  for (int r = 0; r < p.rows; ++r) s += Elem<T>::load(src + static_cast<int64_t>(r) * p.ld);
+  p.dbias[c] = p.accumulate ? p.dbias[c] + s : s;
+}
+
+unsigned flat_blocks(int64_t n_vec) {
+  int64_t b = (n_vec + 255) / 256;
+  if (b > 4096) b = 4096;
+  if (b < 1) b = 1;
+  return static_cast<unsigned>(b);
+}
+
+}  // namespace
+
+int softmax_ce_fwd_bwd(Context* ctx, int dtype, const float* logits, const int64_t* labels, float* loss_rows,
+                       float* loss_mean, void* dlogits, int rows, int classes, int ld_dlogits, float grad_scale) {
+  TCH_CHECK_ARG(dtype == kBF16 || dtype == kF32, "softmax_ce: dtype must be f32(0) or bf16(1)");
+  TCH_CHECK_ARG(logits && labels && loss_rows && loss_mean && dlogits, "softmax_ce: null tensor");
+  TCH_CHECK_ARG(rows > 0 && classes > 0 && ld_dlogits >= classes, "softmax_ce: bad shape");
+  CeArgs a{logits, labels, loss_rows, dlogits, rows, classes, ld_dlogits, grad_scale};
+  int rc = dtype == kBF16 ? launch(ctx, softmax_ce_kernel<bf16>, dim3(rows), dim3(64), a)
+                          : launch(ctx, softmax_ce_kernel<float>, dim3(rows), dim3(64), a);
+  if (rc) return rc;
+  MeanArgs m{loss_rows, loss_mean, rows};
+  return launch(ctx, mean_kernel, dim3(1), dim3(64), m);
+}
+
+int sgd_momentum_step(Context* ctx, float* param, const float* grad, float* momentum_buf, void* shadow_bf16,
+                      int64_t n, float lr, float momentum, float weight_decay) {
+  TCH_CHECK_ARG(param && grad && momentum_buf && n > 0, "sgd_momentum_step: null tensor or empty");
+  SgdArgs a{param, grad, momentum_buf, static_cast<uint16_t*>(shadow_bf16), n, lr, momentum, weight_decay};
+  return launch(ctx, sgd_kernel, dim3(flat_blocks((n + 3) / 4)), dim3(256), a);
+}
+
+int grad_accumulate(Context* ctx, float* global, float* grad, int64_t n) {
+  TCH_CHECK_ARG(global && grad && n > 0, "grad_accumulate: null tensor or empty");
+  AccumArgs a{global, grad, n};
+  return launch(ctx, accumulate_kernel, dim3(flat_blocks((n + 3) / 4)), dim3(256), a);
+}
+
+int fill_zero(Context* ctx, void* ptr, int64_t bytes) {
+  TCH_CHECK_ARG(ptr && bytes > 0 && bytes % 4 == 0, "fill_zero: size must be a positive multiple of 4 bytes");
+  FillArgs a{static_cast<uint32_t*>(ptr), bytes / 4};
+  return launch(ctx, fill_zero_kernel, dim3(flat_blocks(a.words)), dim3(256), a);
+}
+
+int bias_grad(Context* ctx, int dtype, const void* dy, float* dbias, int rows, int cols, int ld, int accumulate) {
+  TCH_CHECK_ARG(dtype == kBF16 || dtype == kF32, "bias_grad: dtype must be f32(0) or bf16(1)");
+  TCH_CHECK_ARG(dy && dbias && rows > 0 && cols > 0 && ld >= cols, "bias_grad: bad arguments");
+  BiasGradArgs a{dy, dbias, rows, cols, ld, accumulate};
+  return dtype == kBF16 ? launch(ctx, bias_grad_kernel<bf16>, dim3((cols + 255) / 256), dim3(256), a)
+                        : launch(ctx, bias_grad_kernel<float>, dim3((cols + 255) / 256), dim3(256), a);
+}
+
+}  // namespace tch

@@ -1,0 +1,64 @@
+// Host-side entry points of the device operators (C++ level; the flat C ABI
+// in capi.cc forwards to these).  All tensors are NHWC, dtype 0 = fp32,
+// 1 = bf16; every function only ENQUEUES work on the context and returns 0 or
+// a negative errno-style code with a message retrievable via last_error().
+#pragma once
+
+#include <stdint.h>
+
+namespace tch {
+
+class Context;
+
+struct ConvShape {
+  int N, H, W, C;  // input batch / height / width / channels
+  int K;           // output channels
+  int R, S;        // filter height / width
+  int stride, pad;
+};
+
+void conv_output_hw(const ConvShape& s, int* Ho, int* Wo);
+
+// conv_igemm.hip
+int conv2d_fwd(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* w, void* y, const void* add,
+               const void* mask, const float* bias, int out_f32, int tile_cfg);
+int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, const void* w, void* dx,
+                 const void* add, const void* mask, int tile_cfg);
+int conv2d_wgrad_pick_splits(const ConvShape& s, int dtype);
+int64_t conv2d_wgrad_workspace_bytes(const ConvShape& s, int dtype, int splits);
+int conv2d_wgrad(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* dy, float* dw,
+                 float* workspace, int splits, int accumulate, int tile_cfg);
+
+// bn.hip -- training-mode BatchNorm over [rows, C] with fused ReLU / residual
+int bn_partial_rows(int64_t rows, int C, int dtype);  // number of row blocks the reductions use
+int64_t bn_workspace_bytes(int64_t rows, int C, int dtype);
+int bn_fwd_train(Context* ctx, int dtype, const void* x, void* y, const void* residual, int relu, int64_t rows, int C,
+                 const float* gamma, const float* beta, float* running_mean, float* running_var, float* save_mean,
+                 float* save_invstd, float momentum, float eps, float* workspace);
+int bn_bwd(Context* ctx, int dtype, const void* dy, const void* relu_mask, const void* x, void* dx, int64_t rows,
+           int C, const float* gamma, const float* save_mean, const float* save_invstd, float* dgamma, float* dbeta,
+           int accumulate, float* workspace);
+
+// pool.hip
+int maxpool_fwd(Context* ctx, int dtype, const void* x, void* y, int32_t* index, int N, int H, int W, int C, int ksize,
+                int stride, int pad);
+int maxpool_bwd(Context* ctx, int dtype, const void* dy, const int32_t* index, void* dx, int N, int H, int W, int C,
+                int ksize, int stride, int pad);
+int avgpool_fwd(Context* ctx, int dtype, const void* x, void* y, int N, int HW, int C);
+int avgpool_bwd(Context* ctx, int dtype, const void* dy, void* dx, int N, int HW, int C);
+
+// loss_optim.hip
+int softmax_ce_fwd_bwd(Context* ctx, int dtype, const float* logits, const int64_t* labels, float* loss_rows,
+                       float* loss_mean, void* dlogits, int rows, int classes, int ld_dlogits, float grad_scale);
+int sgd_momentum_step(Context* ctx, float* param, const float* grad, float* momentum_buf, void* shadow_bf16,
+                      int64_t n, float lr, float momentum, float weight_decay);
+int grad_accumulate(Context* ctx, float* global, float* grad, int64_t n);
+int fill_zero(Context* ctx, void* ptr, int64_t bytes);
+int bias_grad(Context* ctx, int dtype, const void* dy, float* dbias, int rows, int cols, int ld, int accumulate);
+
+// layout.hip
+int nchw_to_nhwc_pad(Context* ctx, int dtype, const float* x_nchw, void* y_nhwc, int N, int C, int H, int W, int Cpad);
+int cast_f32(Context* ctx, int dtype, const float* src, void* dst, int64_t n);
+int cast_to_f32(Context* ctx, int dtype, const void* src, float* dst, int64_t n);
+
+}  // namespace tch

@@ -1,0 +1,276 @@
+"""Tensor-level wrappers over the C ABI (include/torch_col_hip.h).
+
+torch is used for device memory and streams only: every function takes tensors
+that already live on the GPU, passes their raw pointers to the shared library,
+and the library enqueues hand-written HIP kernels.  Layout is NHWC throughout;
+filters are [K, R, S, C].
+"""
+import ctypes
+
+import torch
+
+from ._lib import check, lib
+
+F32, BF16 = 0, 1
+
+
+def dtype_code(t):
+    if t.dtype == torch.float32:
+        return F32
+    if t.dtype == torch.bfloat16:
+        return BF16
+    raise TypeError(f"unsupported dtype {t.dtype}")
+
+
+def chunk_elems(dtype):
+    return 8 if dtype in (BF16, torch.bfloat16) else 4
+
+
+def _p(t):
+    if t is None:
+        return None
+    if not t.is_cuda:
+        raise ValueError("device operators need GPU tensors")
+    if not t.is_contiguous():
+        raise ValueError("device operators need contiguous tensors")
+    return ctypes.c_void_p(t.data_ptr())
+
+
+class Program:
+    """A recorded sequence of launches (replayed without touching Python per launch)."""
+
+    def __init__(self):
+        h = ctypes.c_void_p()
+        check(lib().tch_program_create(ctypes.byref(h)), "tch_program_create")
+        self.handle = h
+        self.keepalive = []  # tensors whose addresses are baked into the launches
+
+    def __len__(self):
+        return int(lib().tch_program_size(self.handle))
+
+    def __del__(self):
+        try:
+            if self.handle:
+                lib().tch_program_destroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+
+class Context:
+    """Launch target: a HIP stream, optionally behind a preemptible launch queue."""
+
+    def __init__(self, stream=None):
+        if stream is None:
+            stream = torch.cuda.current_stream()
+        self.stream = stream
+        h = ctypes.c_void_p()
+        check(lib().tch_context_create(ctypes.c_void_p(stream.cuda_stream), ctypes.byref(h)), "tch_context_create")
+        self.handle = h
+        self._recording = None
+
+    def __del__(self):
+        try:
+            if self.handle:
+                lib().tch_context_destroy(self.handle)
+                self.handle = None
+        except Exception:
+            pass
+
+    def begin_record(self, program):
+        check(lib().tch_program_begin_record(self.handle, program.handle), "tch_program_begin_record")
+        self._recording = program
+
+    def end_record(self):
+        check(lib().tch_program_end_record(self.handle), "tch_program_end_record")
+        self._recording = None
+
+    def run(self, program, first=0, last=-1):
+        """Replay; returns True when the reject flag made the library skip launches."""
+        return check(lib().tch_program_run(self.handle, program.handle, first, last), "tch_program_run") == 1
+
+    def take_rejected(self):
+        return int(lib().tch_context_take_rejected(self.handle))
+
+
+# ---------------------------------------------------------------------------
+# convolution
+# ---------------------------------------------------------------------------
+
+def conv_out_hw(H, W, R, S, stride, pad):
+    return (H + 2 * pad - R) // stride + 1, (W + 2 * pad - S) // stride + 1
+
+
+def conv2d_fwd(ctx, x, w, y, stride, pad, add=None, mask=None, bias=None, tile_cfg=-1):
+    N, H, W, C = x.shape
+    K, R, S, C2 = w.shape
+    assert C == C2, "filter / input channel mismatch"
+    Ho, Wo = conv_out_hw(H, W, R, S, stride, pad)
+    assert tuple(y.shape) == (N, Ho, Wo, K), f"output shape {tuple(y.shape)} != {(N, Ho, Wo, K)}"
+    assert w.dtype == x.dtype
+    out_f32 = int(y.dtype == torch.float32 and x.dtype != torch.float32)
+    for t in (add, mask):
+        assert t is None or (t.shape == y.shape and t.dtype == x.dtype)
+    assert bias is None or (bias.dtype == torch.float32 and bias.numel() == K)
+    check(lib().tch_conv2d_fwd(ctx.handle, dtype_code(x), _p(x), _p(w), _p(y), _p(add), _p(mask), _p(bias), out_f32,
+                               N, H, W, C, K, R, S, stride, pad, tile_cfg), "tch_conv2d_fwd")
+
+
+def conv2d_dgrad(ctx, dy, w, dx, stride, pad, add=None, mask=None, tile_cfg=-1):
+    N, H, W, C = dx.shape
+    K, R, S, C2 = w.shape
+    assert C == C2
+    Ho, Wo = conv_out_hw(H, W, R, S, stride, pad)
+    assert tuple(dy.shape) == (N, Ho, Wo, K)
+    assert dy.dtype == w.dtype == dx.dtype
+    for t in (add, mask):
+        assert t is None or (t.shape == dx.shape and t.dtype == dx.dtype)
+    check(lib().tch_conv2d_dgrad(ctx.handle, dtype_code(dy), _p(dy), _p(w), _p(dx), _p(add), _p(mask),
+                                 N, H, W, C, K, R, S, stride, pad, tile_cfg), "tch_conv2d_dgrad")
+
+
+def conv2d_wgrad_splits(x, K, R, S, stride, pad):
+    N, H, W, C = x.shape
+    return int(lib().tch_conv2d_wgrad_pick_splits(dtype_code(x), N, H, W, C, K, R, S, stride, pad))
+
+
+def conv2d_wgrad_workspace_bytes(dtype, K, R, S, C, splits):
+    return int(lib().tch_conv2d_wgrad_workspace_bytes(dtype, K, R, S, C, splits))
+
+
+def conv2d_wgrad(ctx, x, dy, dw, stride, pad, workspace=None, splits=0, accumulate=False, tile_cfg=-1):
+    N, H, W, C = x.shape
+    K, R, S, C2 = dw.shape
+    assert C == C2 and dw.dtype == torch.float32
+    Ho, Wo = conv_out_hw(H, W, R, S, stride, pad)
+    assert tuple(dy.shape) == (N, Ho, Wo, K) and dy.dtype == x.dtype
+    if workspace is not None:
+        if splits <= 0:
+            splits = conv2d_wgrad_splits(x, K, R, S, stride, pad)
+        need = conv2d_wgrad_workspace_bytes(dtype_code(x), K, R, S, C, splits)
+        assert workspace.numel() * workspace.element_size() >= need, "wgrad workspace too small"
+    check(lib().tch_conv2d_wgrad(ctx.handle, dtype_code(x), _p(x), _p(dy), _p(dw), _p(workspace), splits,
+                                 int(accumulate), N, H, W, C, K, R, S, stride, pad, tile_cfg), "tch_conv2d_wgrad")
+
+
+# ---------------------------------------------------------------------------
+# BatchNorm
+# ---------------------------------------------------------------------------
+
+def bn_workspace_bytes(dtype, rows, C):
+    return int(lib().tch_bn_workspace_bytes(dtype, rows, C))
+
+
+def bn_fwd_train(ctx, x, y, gamma, beta, running_mean, running_var, save_mean, save_invstd, workspace,
+                 residual=None, relu=False, momentum=0.1, eps=1e-5):
+    C = x.shape[-1]
+    rows = x.numel() // C
+    assert y.shape == x.shape and y.dtype == x.dtype
+    assert residual is None or (residual.shape == x.shape and residual.dtype == x.dtype)
+    for t in (gamma, beta, save_mean, save_invstd):
+        assert t.dtype == torch.float32 and t.numel() == C
+    assert workspace.numel() * workspace.element_size() >= bn_workspace_bytes(dtype_code(x), rows, C)
+    check(lib().tch_bn_fwd_train(ctx.handle, dtype_code(x), _p(x), _p(y), _p(residual), int(relu), rows, C,
+                                 _p(gamma), _p(beta), _p(running_mean), _p(running_var), _p(save_mean),
+                                 _p(save_invstd), momentum, eps, _p(workspace)), "tch_bn_fwd_train")
+
+
+def bn_bwd(ctx, dy, x, dx, gamma, save_mean, save_invstd, dgamma, dbeta, workspace, relu_mask=None,
+           accumulate=False):
+    C = x.shape[-1]
+    rows = x.numel() // C
+    assert dy.shape == x.shape == dx.shape and dy.dtype == x.dtype == dx.dtype
+    assert relu_mask is None or (relu_mask.shape == x.shape and relu_mask.dtype == x.dtype)
+    assert workspace.numel() * workspace.element_size() >= bn_workspace_bytes(dtype_code(x), rows, C)
+    check(lib().tch_bn_bwd(ctx.handle, dtype_code(x), _p(dy), _p(relu_mask), _p(x), _p(dx), rows, C, _p(gamma),
+                           _p(save_mean), _p(save_invstd), _p(dgamma), _p(dbeta), int(accumulate), _p(workspace)),
+          "tch_bn_bwd")
+
+
+# ---------------------------------------------------------------------------
+# pooling
+# ---------------------------------------------------------------------------
+
+def maxpool_fwd(ctx, x, y, index, ksize, stride, pad):
+    N, H, W, C = x.shape
+    Ho, Wo = conv_out_hw(H, W, ksize, ksize, stride, pad)
+    assert tuple(y.shape) == (N, Ho, Wo, C) and tuple(index.shape) == (N, Ho, Wo, C)
+    assert index.dtype == torch.int32 and y.dtype == x.dtype
+    check(lib().tch_maxpool_fwd(ctx.handle, dtype_code(x), _p(x), _p(y), _p(index), N, H, W, C, ksize, stride, pad),
+          "tch_maxpool_fwd")
+
+
+def maxpool_bwd(ctx, dy, index, dx, ksize, stride, pad):
+    N, H, W, C = dx.shape
+    Ho, Wo = conv_out_hw(H, W, ksize, ksize, stride, pad)
+    assert tuple(dy.shape) == (N, Ho, Wo, C) and tuple(index.shape) == (N, Ho, Wo, C)
+    assert index.dtype == torch.int32 and dy.dtype == dx.dtype
+    check(lib().tch_maxpool_bwd(ctx.handle, dtype_code(dy), _p(dy), _p(index), _p(dx), N, H, W, C, ksize, stride,
+                                pad), "tch_maxpool_bwd")
+
+
+def avgpool_fwd(ctx, x, y):
+    N, H, W, C = x.shape
+    assert tuple(y.shape) == (N, C) and y.dtype == x.dtype
+    check(lib().tch_avgpool_fwd(ctx.handle, dtype_code(x), _p(x), _p(y), N, H * W, C), "tch_avgpool_fwd")
+
+
+def avgpool_bwd(ctx, dy, dx):
+    N, H, W, C = dx.shape
+    assert tuple(dy.shape) == (N, C) and dy.dtype == dx.dtype
+    check(lib().tch_avgpool_bwd(ctx.handle, dtype_code(dy), _p(dy), _p(dx), N, H * W, C), "tch_avgpool_bwd")
+
+
+# ---------------------------------------------------------------------------
+# loss / optimizer / helpers
+# ---------------------------------------------------------------------------
+
+def softmax_ce_fwd_bwd(ctx, logits, labels, loss_rows, loss_mean, dlogits, loss_scale=1.0):
+    rows, classes = logits.shape
+    assert logits.dtype == torch.float32 and labels.dtype == torch.int64 and labels.numel() == rows
+    assert loss_rows.dtype == torch.float32 and loss_rows.numel() >= rows and loss_mean.dtype == torch.float32
+    assert dlogits.shape[0] == rows and dlogits.shape[1] >= classes and dlogits.stride(0) == dlogits.shape[1]
+    check(lib().tch_softmax_ce_fwd_bwd(ctx.handle, dtype_code(dlogits), _p(logits), _p(labels), _p(loss_rows),
+                                       _p(loss_mean), _p(dlogits), rows, classes, dlogits.shape[1],
+                                       float(loss_scale) / rows), "tch_softmax_ce_fwd_bwd")
+
+
+def sgd_momentum_step(ctx, param, grad, buf, lr, momentum, weight_decay, shadow=None):
+    n = param.numel()
+    assert param.dtype == grad.dtype == buf.dtype == torch.float32 and grad.numel() == n and buf.numel() == n
+    assert shadow is None or (shadow.dtype == torch.bfloat16 and shadow.numel() == n)
+    check(lib().tch_sgd_momentum_step(ctx.handle, _p(param), _p(grad), _p(buf), _p(shadow), n, lr, momentum,
+                                      weight_decay), "tch_sgd_momentum_step")
+
+
+def grad_accumulate(ctx, global_grad, grad):
+    assert global_grad.dtype == grad.dtype == torch.float32 and global_grad.numel() == grad.numel()
+    check(lib().tch_grad_accumulate(ctx.handle, _p(global_grad), _p(grad), grad.numel()), "tch_grad_accumulate")
+
+
+def fill_zero(ctx, t):
+    check(lib().tch_fill_zero(ctx.handle, _p(t), t.numel() * t.element_size()), "tch_fill_zero")
+
+
+def bias_grad(ctx, dy, dbias, cols=None, accumulate=False):
+    rows, ld = dy.shape
+    cols = ld if cols is None else cols
+    check(lib().tch_bias_grad(ctx.handle, dtype_code(dy), _p(dy), _p(dbias), rows, cols, ld, int(accumulate)),
+          "tch_bias_grad")
+
+
+def nchw_to_nhwc_pad(ctx, x_nchw, y_nhwc):
+    N, C, H, W = x_nchw.shape
+    assert x_nchw.dtype == torch.float32 and tuple(y_nhwc.shape[:3]) == (N, H, W)
+    check(lib().tch_nchw_to_nhwc_pad(ctx.handle, dtype_code(y_nhwc), _p(x_nchw), _p(y_nhwc), N, C, H, W,
+                                     y_nhwc.shape[3]), "tch_nchw_to_nhwc_pad")
+
+
+def cast_from_f32(ctx, src, dst):
+    assert src.dtype == torch.float32 and src.numel() == dst.numel()
+    check(lib().tch_cast_from_f32(ctx.handle, dtype_code(dst), _p(src), _p(dst), src.numel()), "tch_cast_from_f32")
+
+
+def cast_to_f32(ctx, src, dst):
+    assert dst.dtype == torch.float32 and src.numel() == dst.numel()
+    check(lib().tch_cast_to_f32(ctx.handle, dtype_code(src), _p(src), _p(dst), src.numel()), "tch_cast_to_f32")

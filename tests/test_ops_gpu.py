@@ -1,0 +1,330 @@
+"""Operator parity on the GPU: every HIP kernel, called through the C ABI, against the
+CPU oracle (oracle/nn_ops.py) on the same seeded inputs.
+
+Tolerances (stated per the path's contract): fp32 rtol 1e-3; bf16 rtol 2e-2, both
+measured against the largest magnitude of the oracle tensor (norm-wise), which is
+the meaningful bound for sums of thousands of products.  Integer results (argmax
+indices) must be bit-exact.
+"""
+import pytest
+import torch
+
+from oracle import nn_ops as O
+
+pytestmark = pytest.mark.gpu
+
+RTOL = {torch.float32: 1e-3, torch.bfloat16: 2e-2}
+
+
+def _gen(seed):
+    g = torch.Generator()
+    g.manual_seed(seed)
+    return g
+
+
+def rnd(shape, dtype, g, scale=1.0):
+    """Seeded N(0,1) values, rounded to `dtype` so that oracle and kernel see identical inputs."""
+    t = torch.randn(shape, generator=g) * scale
+    return t.to(dtype)
+
+
+def close(got, ref, dtype, what, rtol=None):
+    rtol = RTOL[dtype] if rtol is None else rtol
+    got = got.detach().float().cpu()
+    ref = ref.detach().float()
+    assert got.shape == ref.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(ref.shape)}"
+    assert torch.isfinite(got).all(), f"{what}: non-finite values"
+    scale = ref.abs().max().item() + 1e-12
+    err = (got - ref).abs().max().item()
+    assert err <= rtol * scale, f"{what}: max err {err:.3e} > {rtol:g} * {scale:.3e}"
+
+
+CONV_CASES = [
+    # N, H, W, C, K, R, S, stride, pad
+    (2, 14, 14, 64, 64, 3, 3, 1, 1),      # the dominant ResNet shape family
+    (2, 14, 14, 256, 64, 1, 1, 1, 0),     # pointwise reduce
+    (2, 14, 14, 64, 256, 1, 1, 1, 0),     # pointwise expand
+    (2, 16, 16, 64, 128, 3, 3, 2, 1),     # strided 3x3
+    (2, 16, 16, 64, 128, 1, 1, 2, 0),     # strided 1x1 (downsample)
+    (2, 32, 32, 8, 64, 7, 7, 2, 3),       # stem with the channel dim padded to one chunk
+    (3, 7, 7, 32, 40, 3, 3, 1, 1),        # ragged: rows, cols and reduction all off-tile
+    (5, 1, 1, 64, 1000, 1, 1, 1, 0),      # fully connected as a 1x1 convolution
+    (1, 9, 11, 16, 24, 3, 3, 1, 1),       # non-square
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", CONV_CASES)
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2])
+def test_conv_fwd(ctx, dtype, case, tile_cfg):
+    from sirius_amd import ops
+    N, H, W, C, K, R, S, st, pad = case
+    print("case", case, dtype, tile_cfg, flush=True)
+    g = _gen(1)
+    x = rnd((N, H, W, C), dtype, g)
+    w = rnd((K, R, S, C), dtype, g, (R * S * C) ** -0.5)
+    ref = O.conv2d_fwd(x, w, st, pad)
+    y = torch.empty(ref.shape, dtype=dtype, device="cuda")
+    ops.conv2d_fwd(ctx, x.cuda(), w.cuda(), y, st, pad, tile_cfg=tile_cfg)
+    torch.cuda.synchronize()
+    close(y, ref, dtype, "conv fwd")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_conv_fwd_epilogue(ctx, dtype):
+    """bias, fp32 output, gated addend"""
+    from sirius_amd import ops
+    N, H, W, C, K, R, S, st, pad = 2, 8, 8, 32, 48, 3, 3, 1, 1
+    g = _gen(2)
+    x, w = rnd((N, H, W, C), dtype, g), rnd((K, R, S, C), dtype, g, 0.06)
+    bias = torch.randn(K, generator=g)
+    add = rnd((N, H, W, K), dtype, g)
+    mask = rnd((N, H, W, K), dtype, g)
+    ref = O.conv2d_fwd(x, w, st, pad, bias) + add.float() * (mask.float() > 0)
+    y = torch.empty(ref.shape, dtype=torch.float32, device="cuda")
+    ops.conv2d_fwd(ctx, x.cuda(), w.cuda(), y, st, pad, add=add.cuda(), mask=mask.cuda(), bias=bias.cuda())
+    torch.cuda.synchronize()
+    close(y, ref, dtype, "conv fwd epilogue", rtol=1e-3 if dtype == torch.float32 else 5e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", CONV_CASES)
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 2])
+def test_conv_dgrad(ctx, dtype, case, tile_cfg):
+    from sirius_amd import ops
+    N, H, W, C, K, R, S, st, pad = case
+    print("case", case, dtype, tile_cfg, flush=True)
+    g = _gen(3)
+    Ho, Wo = ops.conv_out_hw(H, W, R, S, st, pad)
+    dy = rnd((N, Ho, Wo, K), dtype, g)
+    w = rnd((K, R, S, C), dtype, g, (R * S * K) ** -0.5)
+    ref = O.conv2d_dgrad(dy, w, (N, H, W, C), st, pad)
+    dx = torch.empty((N, H, W, C), dtype=dtype, device="cuda")
+    ops.conv2d_dgrad(ctx, dy.cuda(), w.cuda(), dx, st, pad, tile_cfg=tile_cfg)
+    torch.cuda.synchronize()
+    close(dx, ref, dtype, "conv dgrad")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_conv_dgrad_residual(ctx, dtype):
+    """dx = dgrad + addend gated by a ReLU mask (the identity branch of a bottleneck)"""
+    from sirius_amd import ops
+    N, H, W, C, K, R, S, st, pad = 2, 8, 8, 64, 32, 1, 1, 1, 0
+    g = _gen(4)
+    dy, w = rnd((N, H, W, K), dtype, g), rnd((K, R, S, C), dtype, g, 0.2)
+    add, mask = rnd((N, H, W, C), dtype, g), rnd((N, H, W, C), dtype, g)
+    ref = O.conv2d_dgrad(dy, w, (N, H, W, C), st, pad) + add.float() * (mask.float() > 0)
+    dx = torch.empty((N, H, W, C), dtype=dtype, device="cuda")
+    ops.conv2d_dgrad(ctx, dy.cuda(), w.cuda(), dx, st, pad, add=add.cuda(), mask=mask.cuda())
+    torch.cuda.synchronize()
+    close(dx, ref, dtype, "conv dgrad + residual")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", CONV_CASES)
+@pytest.mark.parametrize("splits", [1, 0, 3])
+def test_conv_wgrad(ctx, dtype, case, splits):
+    from sirius_amd import ops
+    N, H, W, C, K, R, S, st, pad = case
+    print("case", case, dtype, splits, flush=True)
+    g = _gen(5)
+    Ho, Wo = ops.conv_out_hw(H, W, R, S, st, pad)
+    x = rnd((N, H, W, C), dtype, g)
+    dy = rnd((N, Ho, Wo, K), dtype, g, (N * Ho * Wo) ** -0.5)
+    ref = O.conv2d_wgrad(x, dy, (K, R, S, C), st, pad)
+    dw = torch.full((K, R, S, C), 7.0, dtype=torch.float32, device="cuda")
+    ws = None
+    if splits != 1:
+        n_split = splits if splits > 0 else ops.conv2d_wgrad_splits(x, K, R, S, st, pad)
+        nbytes = max(4, ops.conv2d_wgrad_workspace_bytes(ops.dtype_code(x), K, R, S, C, n_split))
+        ws = torch.empty(nbytes // 4, dtype=torch.float32, device="cuda")
+    ops.conv2d_wgrad(ctx, x.cuda(), dy.cuda(), dw, st, pad, workspace=ws, splits=splits)
+    torch.cuda.synchronize()
+    close(dw, ref, dtype, "conv wgrad", rtol=1e-3 if dtype == torch.float32 else 5e-3)
+    # accumulate: a second pass adds the same gradient on top
+    ops.conv2d_wgrad(ctx, x.cuda(), dy.cuda(), dw, st, pad, workspace=ws, splits=splits, accumulate=True)
+    torch.cuda.synchronize()
+    close(dw, 2 * ref, dtype, "conv wgrad accumulate", rtol=1e-3 if dtype == torch.float32 else 5e-3)
+
+
+BN_CASES = [(2 * 14 * 14, 64), (4 * 28 * 28, 128), (3 * 7 * 7, 2048), (37, 8), (100000, 64)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,C", BN_CASES)
+@pytest.mark.parametrize("fuse", ["plain", "relu", "residual_relu"])
+def test_bn_fwd(ctx, dtype, rows, C, fuse):
+    from sirius_amd import ops
+    g = _gen(6)
+    x = rnd((1, 1, rows, C), dtype, g) * 1.7 + 0.3
+    x = x.to(dtype)
+    gamma, beta = torch.rand(C, generator=g) + 0.5, torch.randn(C, generator=g) * 0.1
+    rm, rv = torch.randn(C, generator=g) * 0.1, torch.rand(C, generator=g) + 0.5
+    res = rnd(x.shape, dtype, g) if fuse == "residual_relu" else None
+    relu = fuse != "plain"
+    rm_ref, rv_ref = rm.clone(), rv.clone()
+    y_ref, mean_ref, invstd_ref = O.bn_fwd_train(x, gamma, beta, rm_ref, rv_ref, residual=res, relu=relu)
+    d = lambda t: t.cuda() if t is not None else None
+    y = torch.empty(x.shape, dtype=dtype, device="cuda")
+    rm_d, rv_d = rm.cuda(), rv.cuda()
+    sm, si = torch.empty(C, device="cuda"), torch.empty(C, device="cuda")
+    ws = torch.empty(ops.bn_workspace_bytes(ops.dtype_code(x), rows, C) // 4, dtype=torch.float32, device="cuda")
+    ops.bn_fwd_train(ctx, x.cuda(), y, gamma.cuda(), beta.cuda(), rm_d, rv_d, sm, si, ws, residual=d(res), relu=relu)
+    torch.cuda.synchronize()
+    close(sm, mean_ref, torch.float32, "bn mean", rtol=1e-4)
+    close(si, invstd_ref, torch.float32, "bn invstd", rtol=1e-4)
+    close(rm_d, rm_ref, torch.float32, "bn running_mean", rtol=1e-4)
+    close(rv_d, rv_ref, torch.float32, "bn running_var", rtol=1e-4)
+    close(y, y_ref, dtype, "bn y", rtol=1e-4 if dtype == torch.float32 else 1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,C", BN_CASES)
+@pytest.mark.parametrize("masked", [False, True])
+def test_bn_bwd(ctx, dtype, rows, C, masked):
+    from sirius_amd import ops
+    g = _gen(7)
+    x = (rnd((1, 1, rows, C), dtype, g) * 1.3 - 0.2).to(dtype)
+    dy = rnd(x.shape, dtype, g)
+    mask = rnd(x.shape, dtype, g) if masked else None
+    gamma = torch.rand(C, generator=g) + 0.5
+    dx_ref, dg_ref, db_ref = O.bn_bwd(dy, x, gamma, relu_mask=mask)
+    x2 = x.float().reshape(-1, C)
+    mean, invstd = x2.mean(0), 1.0 / torch.sqrt(x2.var(0, unbiased=False) + 1e-5)
+    dx = torch.empty(x.shape, dtype=dtype, device="cuda")
+    dg, db = torch.zeros(C, device="cuda"), torch.zeros(C, device="cuda")
+    ws = torch.empty(ops.bn_workspace_bytes(ops.dtype_code(x), rows, C) // 4, dtype=torch.float32, device="cuda")
+    ops.bn_bwd(ctx, dy.cuda(), x.cuda(), dx, gamma.cuda(), mean.cuda(), invstd.cuda(), dg, db, ws,
+               relu_mask=mask.cuda() if masked else None)
+    torch.cuda.synchronize()
+    close(dg, dg_ref, torch.float32, "bn dgamma", rtol=1e-3)
+    close(db, db_ref, torch.float32, "bn dbeta", rtol=1e-3)
+    close(dx, dx_ref, dtype, "bn dx", rtol=1e-3 if dtype == torch.float32 else 1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(2, 16, 16, 64), (1, 7, 9, 8), (3, 112, 112, 16)])
+def test_maxpool(ctx, dtype, shape):
+    from sirius_amd import ops
+    g = _gen(8)
+    x = torch.relu(rnd(shape, dtype, g))  # post-ReLU: zeros tie constantly
+    y_ref, idx_ref = O.maxpool_fwd(x, 3, 2, 1)
+    N, Ho, Wo, C = y_ref.shape
+    y = torch.empty(y_ref.shape, dtype=dtype, device="cuda")
+    idx = torch.empty(y_ref.shape, dtype=torch.int32, device="cuda")
+    ops.maxpool_fwd(ctx, x.cuda(), y, idx, 3, 2, 1)
+    torch.cuda.synchronize()
+    assert torch.equal(y.float().cpu(), y_ref), "maxpool values must be exact"
+    assert torch.equal(idx.cpu().long(), idx_ref), "maxpool argmax indices must be bit-exact (first maximum wins)"
+    dy = rnd(y_ref.shape, dtype, g)
+    dx_ref = O.maxpool_bwd(dy, x, 3, 2, 1)
+    dx = torch.empty(shape, dtype=dtype, device="cuda")
+    ops.maxpool_bwd(ctx, dy.cuda(), idx, dx, 3, 2, 1)
+    torch.cuda.synchronize()
+    close(dx, dx_ref, dtype, "maxpool bwd", rtol=1e-6 if dtype == torch.float32 else 1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_avgpool(ctx, dtype):
+    from sirius_amd import ops
+    g = _gen(9)
+    x = rnd((3, 7, 7, 64), dtype, g)
+    y = torch.empty((3, 64), dtype=dtype, device="cuda")
+    ops.avgpool_fwd(ctx, x.cuda(), y)
+    dy = rnd((3, 64), dtype, g)
+    dx = torch.empty(x.shape, dtype=dtype, device="cuda")
+    ops.avgpool_bwd(ctx, dy.cuda(), dx)
+    torch.cuda.synchronize()
+    close(y, O.avgpool_fwd(x), dtype, "avgpool fwd", rtol=1e-5 if dtype == torch.float32 else 1e-2)
+    close(dx, O.avgpool_bwd(dy, x.shape), dtype, "avgpool bwd", rtol=1e-5 if dtype == torch.float32 else 1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,classes,scale", [(4, 1000, 1.0), (64, 1000, 0.25), (3, 10, 1.0)])
+def test_softmax_ce(ctx, dtype, rows, classes, scale):
+    from sirius_amd import ops
+    g = _gen(10)
+    z = torch.randn(rows, classes, generator=g) * 3
+    labels = torch.randint(0, classes, (rows,), generator=g)
+    rows_ref, mean_ref, g_ref = O.softmax_ce(z, labels, scale)
+    loss_rows, loss_mean = torch.empty(rows, device="cuda"), torch.empty(1, device="cuda")
+    ld = (classes + 7) // 8 * 8
+    dz = torch.zeros(rows, ld, dtype=dtype, device="cuda")
+    ops.softmax_ce_fwd_bwd(ctx, z.cuda(), labels.cuda(), loss_rows, loss_mean, dz, loss_scale=scale)
+    torch.cuda.synchronize()
+    close(loss_rows, rows_ref, torch.float32, "ce rows", rtol=1e-5)
+    close(loss_mean, mean_ref.reshape(1), torch.float32, "ce mean", rtol=1e-5)
+    close(dz[:, :classes], g_ref, dtype, "ce grad", rtol=1e-4 if dtype == torch.float32 else 1e-2)
+    assert (dz[:, classes:] == 0).all()
+
+
+@pytest.mark.parametrize("n", [1024, 1000003])
+def test_sgd_and_accumulate(ctx, n):
+    from sirius_amd import ops
+    g = _gen(11)
+    p, gr, buf = torch.randn(n, generator=g), torch.randn(n, generator=g), torch.zeros(n)
+    p_ref, buf_ref = O.sgd_momentum(p, gr, buf, 0.1, 0.9, 1e-4, steps=2)
+    p_d, g_d, b_d = p.cuda(), gr.cuda(), buf.cuda()
+    shadow = torch.empty(n, dtype=torch.bfloat16, device="cuda")
+    for _ in range(2):
+        ops.sgd_momentum_step(ctx, p_d, g_d, b_d, 0.1, 0.9, 1e-4, shadow=shadow)
+    torch.cuda.synchronize()
+    close(p_d, p_ref, torch.float32, "sgd param", rtol=1e-6)
+    close(b_d, buf_ref, torch.float32, "sgd momentum", rtol=1e-6)
+    assert torch.equal(shadow.cpu(), p_d.cpu().to(torch.bfloat16)), "bf16 shadow must be the RNE rounding of the master"
+    acc = torch.randn(n, generator=g)
+    acc_d = acc.cuda()
+    ops.grad_accumulate(ctx, acc_d, g_d)
+    torch.cuda.synchronize()
+    assert torch.equal(acc_d.cpu(), acc + gr) and (g_d == 0).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_layout_and_cast(ctx, dtype):
+    from sirius_amd import ops
+    g = _gen(12)
+    x = torch.randn(2, 3, 10, 12, generator=g)
+    y = torch.empty(2, 10, 12, 8, dtype=dtype, device="cuda")
+    ops.nchw_to_nhwc_pad(ctx, x.cuda(), y)
+    torch.cuda.synchronize()
+    ref = torch.zeros(2, 10, 12, 8)
+    ref[..., :3] = x.permute(0, 2, 3, 1)
+    assert torch.equal(y.cpu(), ref.to(dtype)), "layout conversion must round exactly like torch"
+    src = torch.randn(1001, generator=g)
+    dst = torch.empty(1001, dtype=dtype, device="cuda")
+    back = torch.empty(1001, device="cuda")
+    ops.cast_from_f32(ctx, src.cuda(), dst)
+    ops.cast_to_f32(ctx, dst, back)
+    torch.cuda.synchronize()
+    assert torch.equal(dst.cpu(), src.to(dtype)) and torch.equal(back.cpu(), src.to(dtype).float())
+
+
+def test_bias_grad(ctx):
+    from sirius_amd import ops
+    g = _gen(13)
+    dy = rnd((16, 1000), torch.bfloat16, g)
+    db = torch.zeros(1000, device="cuda")
+    ops.bias_grad(ctx, dy.cuda(), db)
+    torch.cuda.synchronize()
+    close(db, dy.float().sum(0), torch.float32, "bias grad", rtol=1e-5)
+
+
+def test_program_record_replay(ctx):
+    """A recorded program replays the same launches: results equal the eager ones."""
+    from sirius_amd import ops
+    g = _gen(14)
+    x, w = rnd((2, 8, 8, 32), torch.bfloat16, g).cuda(), rnd((64, 3, 3, 32), torch.bfloat16, g, 0.06).cuda()
+    y_eager = torch.empty((2, 8, 8, 64), dtype=torch.bfloat16, device="cuda")
+    ops.conv2d_fwd(ctx, x, w, y_eager, 1, 1)
+    prog = ops.Program()
+    y_prog = torch.zeros_like(y_eager)
+    ctx.begin_record(prog)
+    ops.conv2d_fwd(ctx, x, w, y_prog, 1, 1)
+    ctx.end_record()
+    torch.cuda.synchronize()
+    assert len(prog) == 1 and (y_prog == 0).all(), "recording must not launch"
+    for _ in range(3):
+        y_prog.zero_()
+        assert ctx.run(prog) is False
+        torch.cuda.synchronize()
+        assert torch.equal(y_prog, y_eager)
