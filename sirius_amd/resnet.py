@@ -1,0 +1,455 @@
+"""ResNet (Bottleneck) training-step engine over the HIP operators.
+
+What the reference does with ``torchvision.models.resnet152`` + autograd +
+``torch.optim.SGD`` (train/resnet152.py:22-29,84-91), this engine does with one
+recorded program of hand-written kernels per batch size:
+
+* parameters, gradients and momentum live in three flat fp32 buffers (filters in
+  [K,R,S,C] order, the stem's 3 input channels zero-padded to one 16-byte chunk);
+  bf16 mode keeps a flat bf16 shadow the kernels read, rewritten by the optimizer;
+* activations are NHWC in the compute dtype; per batch size a static plan owns
+  them, so a step is a replay of pre-bound launches (no Python per kernel);
+* backward is written out by hand (no autograd): BatchNorm backward takes the
+  ReLU mask of the block output, the identity branch is added in the epilogue of
+  the first convolution's data gradient;
+* the reject flag of the launch queues is a checkpoint between any two launches:
+  a replay that was cut short reports it, the caller frees the plan
+  (``release_activations``) and the memory returns to the pool.
+
+torch supplies device memory and streams only.
+"""
+import math
+
+import torch
+
+from . import ops
+
+STEM_CIN_PAD = 8
+
+
+class _Conv:
+    def __init__(self, name, cin, cout, k, stride, pad):
+        self.name, self.cin, self.cout, self.k, self.stride, self.pad = name, cin, cout, k, stride, pad
+        self.cin_store = max(cin, STEM_CIN_PAD) if cin < STEM_CIN_PAD else cin
+
+
+class _Param:
+    __slots__ = ("name", "kind", "shape", "store_shape", "offset", "numel")
+
+    def __init__(self, name, kind, shape, store_shape, offset):
+        self.name, self.kind, self.shape, self.store_shape, self.offset = name, kind, shape, store_shape, offset
+        self.numel = int(math.prod(store_shape))
+
+
+class _Block:
+    pass
+
+
+class ResNetEngine:
+    def __init__(self, depths=(3, 8, 36, 3), num_classes=1000, width=64, dtype=torch.bfloat16, image_size=224,
+                 lr=0.1, momentum=0.9, weight_decay=1e-4, bn_momentum=0.1, bn_eps=1e-5, stream=None):
+        if not torch.cuda.is_available():
+            raise RuntimeError("ResNetEngine runs on the GPU only; there is no CPU path")
+        assert dtype in (torch.bfloat16, torch.float32)
+        assert num_classes % 8 == 0, "class count must be a multiple of one 16-byte chunk"
+        self.dtype, self.image_size, self.num_classes = dtype, image_size, num_classes
+        self.lr, self.momentum, self.weight_decay = lr, momentum, weight_decay
+        self.bn_momentum, self.bn_eps = bn_momentum, bn_eps
+        self.dev = torch.device("cuda", torch.cuda.current_device())
+        self.ctx = ops.Context(stream if stream is not None else torch.cuda.current_stream())
+        self.depths, self.width = tuple(depths), width
+
+        # ---- architecture + parameter table (torchvision naming and order) ----
+        self._specs, self._bn_names = [], []
+        self._off = 0
+        self.stem = _Conv("conv1", 3, width, 7, 2, 3)
+        self._add_conv(self.stem)
+        self._add_bn("bn1", width)
+        self.blocks = []
+        inplanes = width
+        for i, depth in enumerate(self.depths):
+            planes = width * (2 ** i)
+            for b in range(depth):
+                s = (1 if i == 0 else 2) if b == 0 else 1
+                blk = _Block()
+                pre = f"layer{i + 1}.{b}"
+                blk.c1 = _Conv(pre + ".conv1", inplanes, planes, 1, 1, 0)
+                blk.c2 = _Conv(pre + ".conv2", planes, planes, 3, s, 1)
+                blk.c3 = _Conv(pre + ".conv3", planes, planes * 4, 1, 1, 0)
+                for j, c in enumerate((blk.c1, blk.c2, blk.c3)):
+                    self._add_conv(c)
+                    self._add_bn(f"{pre}.bn{j + 1}", c.cout)
+                blk.cd = None
+                if b == 0 and (s != 1 or inplanes != planes * 4):
+                    blk.cd = _Conv(pre + ".downsample.0", inplanes, planes * 4, 1, s, 0)
+                    self._add_conv(blk.cd)
+                    self._add_bn(pre + ".downsample.1", planes * 4)
+                blk.stride, blk.cin, blk.planes, blk.prefix = s, inplanes, planes, pre
+                self.blocks.append(blk)
+                inplanes = planes * 4
+        self.feat = inplanes
+        self._add_param("fc.weight", "fc_w", (num_classes, inplanes), (num_classes, 1, 1, inplanes))
+        self._add_param("fc.bias", "fc_b", (num_classes,), (num_classes,))
+        self.n_store = self._off
+        self.spec = {p.name: p for p in self._specs}
+
+        f32 = dict(dtype=torch.float32, device=self.dev)
+        self.params = torch.zeros(self.n_store, **f32)
+        self.grads = torch.zeros(self.n_store, **f32)
+        self.momentum_buf = torch.zeros(self.n_store, **f32)
+        self.global_grads = None
+        self.shadow = torch.zeros(self.n_store, dtype=torch.bfloat16, device=self.dev) if dtype == torch.bfloat16 else None
+        nbn = sum(c for _, c in self._bn_names)
+        self.running_mean = torch.zeros(nbn, **f32)
+        self.running_var = torch.ones(nbn, **f32)
+        self._bn_off, o = {}, 0
+        for name, c in self._bn_names:
+            self._bn_off[name] = (o, c)
+            o += c
+        self._plans = {}
+        self._opt_prog = None
+        self._acc_prog = None
+        self._opt_global_prog = None
+
+    # ------------------------------------------------------------------ parameter table
+    def _add_param(self, name, kind, shape, store_shape):
+        p = _Param(name, kind, shape, store_shape, self._off)
+        self._specs.append(p)
+        self._off += (p.numel + 3) // 4 * 4
+        return p
+
+    def _add_conv(self, c):
+        self._add_param(c.name + ".weight", "conv", (c.cout, c.cin, c.k, c.k), (c.cout, c.k, c.k, c.cin_store))
+
+    def _add_bn(self, name, c):
+        self._add_param(name + ".weight", "bn_w", (c,), (c,))
+        self._add_param(name + ".bias", "bn_b", (c,), (c,))
+        self._bn_names.append((name, c))
+
+    def num_parameters(self):
+        return sum(int(math.prod(p.shape)) for p in self._specs)
+
+    def _view(self, flat, name):
+        p = self.spec[name]
+        return flat[p.offset:p.offset + p.numel].view(p.store_shape)
+
+    def _w(self, name):
+        """The tensor the kernels read for a filter: bf16 shadow or the fp32 master."""
+        return self._view(self.shadow if self.shadow is not None else self.params, name)
+
+    def _to_store(self, p, t):
+        t = t.detach().to(torch.float32)
+        if p.kind == "conv":
+            t = t.permute(0, 2, 3, 1)  # OIHW -> KRSC
+            if p.store_shape[3] != t.shape[3]:
+                t = torch.nn.functional.pad(t, (0, p.store_shape[3] - t.shape[3]))
+        return t.reshape(p.store_shape).contiguous()
+
+    def _from_store(self, p, flat):
+        t = flat[p.offset:p.offset + p.numel].view(p.store_shape)
+        if p.kind == "conv":
+            t = t[..., :p.shape[1]].permute(0, 3, 1, 2)  # KRSC -> OIHW, padding stripped
+        return t.reshape(p.shape).contiguous().cpu()
+
+    def load_state_dict(self, sd):
+        """Take weights and BN statistics from a torchvision-style state dict (CPU, OIHW)."""
+        host = torch.zeros(self.n_store, dtype=torch.float32)
+        for p in self._specs:
+            host[p.offset:p.offset + p.numel] = self._to_store(p, sd[p.name]).reshape(-1)
+        self.params.copy_(host)
+        for name, (o, c) in self._bn_off.items():
+            self.running_mean[o:o + c].copy_(sd[name + ".running_mean"])
+            self.running_var[o:o + c].copy_(sd[name + ".running_var"])
+        self.momentum_buf.zero_()
+        self.grads.zero_()
+        self.refresh_shadow()
+        torch.cuda.synchronize()
+
+    def refresh_shadow(self):
+        if self.shadow is not None:
+            ops.cast_from_f32(self.ctx, self.params, self.shadow)
+
+    def state_dict(self):
+        torch.cuda.synchronize()
+        sd = {p.name: self._from_store(p, self.params) for p in self._specs}
+        for name, (o, c) in self._bn_off.items():
+            sd[name + ".running_mean"] = self.running_mean[o:o + c].cpu()
+            sd[name + ".running_var"] = self.running_var[o:o + c].cpu()
+        return sd
+
+    def grads_dict(self, use_global=False):
+        torch.cuda.synchronize()
+        flat = self.global_grads if use_global else self.grads
+        return {p.name: self._from_store(p, flat) for p in self._specs}
+
+    # ------------------------------------------------------------------ the plan for one batch size
+    def _build_plan(self, B, loss_scale):
+        T, dev, ctx = self.dtype, self.dev, self.ctx
+        S = self.image_size
+        plan = _Block()
+        plan.batch, plan.loss_scale = B, loss_scale
+        keep = []
+
+        def act(*shape, dtype=T):
+            t = torch.empty(shape, dtype=dtype, device=dev)
+            keep.append(t)
+            return t
+
+        # gradient buffers are recycled through a size-keyed free list: the program is
+        # one in-order stream of launches, so program order is the only hazard
+        free = {}
+
+        def galloc(shape):
+            n = int(math.prod(shape))
+            lst = free.get(n)
+            if lst:
+                return lst.pop().view(shape)
+            t = torch.empty(n, dtype=T, device=dev)
+            keep.append(t)
+            return t.view(shape)
+
+        def gfree(t):
+            free.setdefault(t.numel(), []).append(t.reshape(-1))
+
+        code = ops.dtype_code(torch.empty(0, dtype=T))
+        plan.x_in = act(B, 3, S, S, dtype=torch.float32)
+        plan.labels = torch.zeros(B, dtype=torch.int64, device=dev)
+        plan.loss_rows = act(B, dtype=torch.float32)
+        plan.loss = act(1, dtype=torch.float32)
+        bn_save = act(2 * self.running_mean.numel(), dtype=torch.float32)
+        nbn = self.running_mean.numel()
+
+        # workspaces sized over every layer of the plan
+        bn_ws_bytes, wg_ws_bytes = [0], [4]
+        geo = []  # (conv, x_shape) for the workspace pass
+
+        def conv_shape(c, H, W):
+            Ho, Wo = ops.conv_out_hw(H, W, c.k, c.k, c.stride, c.pad)
+            return Ho, Wo
+
+        # ---- shapes ----
+        H0, W0 = conv_shape(self.stem, S, S)
+        Hp, Wp = ops.conv_out_hw(H0, W0, 3, 3, 2, 1)
+        shapes = []
+        H, W = Hp, Wp
+        for blk in self.blocks:
+            Ho, Wo = conv_shape(blk.c2, H, W)
+            shapes.append((H, W, Ho, Wo))
+            H, W = Ho, Wo
+        Hl, Wl = H, W
+
+        def wg_need(c, N, H, W):
+            x_like = torch.empty((N, H, W, c.cin_store), dtype=T, device="meta")
+            sp = int(ops.lib().tch_conv2d_wgrad_pick_splits(code, N, H, W, c.cin_store, c.cout, c.k, c.k, c.stride, c.pad))
+            wg_ws_bytes[0] = max(wg_ws_bytes[0], ops.conv2d_wgrad_workspace_bytes(code, c.cout, c.k, c.k, c.cin_store, sp))
+            del x_like
+
+        def bn_need(rows, C):
+            bn_ws_bytes[0] = max(bn_ws_bytes[0], ops.bn_workspace_bytes(code, rows, C))
+
+        wg_need(self.stem, B, S, S)
+        bn_need(B * H0 * W0, self.width)
+        for blk, (H, W, Ho, Wo) in zip(self.blocks, shapes):
+            wg_need(blk.c1, B, H, W)
+            wg_need(blk.c2, B, H, W)
+            wg_need(blk.c3, B, Ho, Wo)
+            bn_need(B * H * W, blk.planes)
+            bn_need(B * Ho * Wo, blk.planes * 4)
+            if blk.cd is not None:
+                wg_need(blk.cd, B, H, W)
+        fc = _Conv("fc", self.feat, self.num_classes, 1, 1, 0)
+        wg_need(fc, B, 1, 1)
+        bn_ws = act(bn_ws_bytes[0] // 4, dtype=torch.float32)
+        wg_ws = act(wg_ws_bytes[0] // 4, dtype=torch.float32)
+
+        def bn_fwd(name, x, y, residual=None, relu=True):
+            o, c = self._bn_off[name]
+            ops.bn_fwd_train(ctx, x, y, self._view(self.params, name + ".weight"), self._view(self.params, name + ".bias"),
+                             self.running_mean[o:o + c], self.running_var[o:o + c], bn_save[o:o + c],
+                             bn_save[nbn + o:nbn + o + c], bn_ws, residual=residual, relu=relu,
+                             momentum=self.bn_momentum, eps=self.bn_eps)
+
+        def bn_bwd(name, dy, x, dx, mask):
+            o, c = self._bn_off[name]
+            ops.bn_bwd(ctx, dy, x, dx, self._view(self.params, name + ".weight"), bn_save[o:o + c],
+                       bn_save[nbn + o:nbn + o + c], self._view(self.grads, name + ".weight"),
+                       self._view(self.grads, name + ".bias"), bn_ws, relu_mask=mask)
+
+        def conv_fwd(c, x, y, **kw):
+            ops.conv2d_fwd(ctx, x, self._w(c.name + ".weight"), y, c.stride, c.pad, **kw)
+
+        def conv_wgrad(c, x, dy):
+            ops.conv2d_wgrad(ctx, x, dy, self._view(self.grads, c.name + ".weight"), c.stride, c.pad, workspace=wg_ws)
+
+        def conv_dgrad(c, dy, dx, **kw):
+            ops.conv2d_dgrad(ctx, dy, self._w(c.name + ".weight"), dx, c.stride, c.pad, **kw)
+
+        prog = ops.Program()
+        ctx.begin_record(prog)
+        try:
+            # ================= forward =================
+            x0 = act(B, S, S, STEM_CIN_PAD)
+            ops.nchw_to_nhwc_pad(ctx, plan.x_in, x0)
+            z0, a0 = act(B, H0, W0, self.width), act(B, H0, W0, self.width)
+            conv_fwd(self.stem, x0, z0)
+            bn_fwd("bn1", z0, a0)
+            p0 = act(B, Hp, Wp, self.width)
+            p0_idx = act(B, Hp, Wp, self.width, dtype=torch.int32)
+            ops.maxpool_fwd(ctx, a0, p0, p0_idx, 3, 2, 1)
+            x = p0
+            saved = []
+            for blk, (H, W, Ho, Wo) in zip(self.blocks, shapes):
+                P, pre = blk.planes, blk.prefix
+                z1, a1 = act(B, H, W, P), act(B, H, W, P)
+                conv_fwd(blk.c1, x, z1)
+                bn_fwd(pre + ".bn1", z1, a1)
+                z2, a2 = act(B, Ho, Wo, P), act(B, Ho, Wo, P)
+                conv_fwd(blk.c2, a1, z2)
+                bn_fwd(pre + ".bn2", z2, a2)
+                z3, out = act(B, Ho, Wo, 4 * P), act(B, Ho, Wo, 4 * P)
+                conv_fwd(blk.c3, a2, z3)
+                zd = None
+                if blk.cd is not None:
+                    zd, idn = act(B, Ho, Wo, 4 * P), act(B, Ho, Wo, 4 * P)
+                    conv_fwd(blk.cd, x, zd)
+                    bn_fwd(pre + ".downsample.1", zd, idn, relu=False)
+                else:
+                    idn = x
+                bn_fwd(pre + ".bn3", z3, out, residual=idn, relu=True)
+                saved.append((x, z1, a1, z2, a2, z3, zd, out))
+                x = out
+            pooled = act(B, self.feat)
+            ops.avgpool_fwd(ctx, x, pooled)
+            logits = act(B, self.num_classes, dtype=torch.float32)
+            ops.conv2d_fwd(ctx, pooled.view(B, 1, 1, self.feat), self._w("fc.weight"),
+                           logits.view(B, 1, 1, self.num_classes), 1, 0, bias=self._view(self.params, "fc.bias"))
+            dlogits = act(B, self.num_classes)
+            ops.softmax_ce_fwd_bwd(ctx, logits, plan.labels, plan.loss_rows, plan.loss, dlogits, loss_scale=loss_scale)
+            plan.n_forward = len(prog)
+
+            # ================= backward =================
+            ops.conv2d_wgrad(ctx, pooled.view(B, 1, 1, self.feat), dlogits.view(B, 1, 1, self.num_classes),
+                             self._view(self.grads, "fc.weight"), 1, 0, workspace=wg_ws)
+            ops.bias_grad(ctx, dlogits, self._view(self.grads, "fc.bias"))
+            g_pooled = galloc((B, self.feat))
+            ops.conv2d_dgrad(ctx, dlogits.view(B, 1, 1, self.num_classes), self._w("fc.weight"),
+                             g_pooled.view(B, 1, 1, self.feat), 1, 0)
+            g_out = galloc((B, Hl, Wl, self.feat))
+            ops.avgpool_bwd(ctx, g_pooled, g_out)
+            gfree(g_pooled)
+            for blk, (H, W, Ho, Wo), sv in zip(reversed(self.blocks), reversed(shapes), reversed(saved)):
+                xin, z1, a1, z2, a2, z3, zd, out = sv
+                P, pre = blk.planes, blk.prefix
+                dz3 = galloc(z3.shape)
+                bn_bwd(pre + ".bn3", g_out, z3, dz3, out)
+                conv_wgrad(blk.c3, a2, dz3)
+                g_a2 = galloc(a2.shape)
+                conv_dgrad(blk.c3, dz3, g_a2)
+                gfree(dz3)
+                dz2 = galloc(z2.shape)
+                bn_bwd(pre + ".bn2", g_a2, z2, dz2, a2)
+                gfree(g_a2)
+                conv_wgrad(blk.c2, a1, dz2)
+                g_a1 = galloc(a1.shape)
+                conv_dgrad(blk.c2, dz2, g_a1)
+                gfree(dz2)
+                dz1 = galloc(z1.shape)
+                bn_bwd(pre + ".bn1", g_a1, z1, dz1, a1)
+                gfree(g_a1)
+                conv_wgrad(blk.c1, xin, dz1)
+                gx = galloc(xin.shape)
+                if blk.cd is not None:
+                    dzd = galloc(zd.shape)
+                    bn_bwd(pre + ".downsample.1", g_out, zd, dzd, out)
+                    conv_wgrad(blk.cd, xin, dzd)
+                    gx_id = galloc(xin.shape)
+                    conv_dgrad(blk.cd, dzd, gx_id)
+                    gfree(dzd)
+                    conv_dgrad(blk.c1, dz1, gx, add=gx_id)
+                    gfree(gx_id)
+                else:
+                    conv_dgrad(blk.c1, dz1, gx, add=g_out, mask=out)
+                gfree(dz1)
+                gfree(g_out)
+                g_out = gx
+            g_a0 = galloc(a0.shape)
+            ops.maxpool_bwd(ctx, g_out, p0_idx, g_a0, 3, 2, 1)
+            gfree(g_out)
+            dz0 = galloc(z0.shape)
+            bn_bwd("bn1", g_a0, z0, dz0, a0)
+            gfree(g_a0)
+            conv_wgrad(self.stem, x0, dz0)
+            gfree(dz0)
+        finally:
+            ctx.end_record()
+        plan.prog = prog
+        plan.keep = keep
+        plan.logits = logits
+        plan.bytes = sum(t.numel() * t.element_size() for t in keep)
+        return plan
+
+    def plan(self, batch, loss_scale=1.0):
+        key = (int(batch), float(loss_scale))
+        p = self._plans.get(key)
+        if p is None:
+            # plans of other batch sizes own activation memory: drop them first
+            for k in [k for k in self._plans if k[0] != key[0]]:
+                del self._plans[k]
+            p = self._plans[key] = self._build_plan(*key)
+        return p
+
+    def release_activations(self):
+        """Drop every plan (and with it all activation / gradient-scratch memory)."""
+        n = sum(p.bytes for p in self._plans.values())
+        self._plans.clear()
+        return n
+
+    # ------------------------------------------------------------------ the step
+    def forward_backward(self, x, y, loss_scale=1.0):
+        """x [B,3,S,S] fp32 and y [B] int64 on the GPU.  Returns (plan, cut_short)."""
+        p = self.plan(x.shape[0], loss_scale)
+        p.x_in.copy_(x, non_blocking=True)
+        p.labels.copy_(y, non_blocking=True)
+        cut = self.ctx.run(p.prog)
+        return p, cut
+
+    def forward_backward_resident(self, batch, loss_scale=1.0):
+        """Replay on whatever already sits in the plan's input buffers."""
+        p = self.plan(batch, loss_scale)
+        return p, self.ctx.run(p.prog)
+
+    def _flat_prog(self, fn):
+        prog = ops.Program()
+        self.ctx.begin_record(prog)
+        try:
+            fn()
+        finally:
+            self.ctx.end_record()
+        return prog
+
+    def accumulate(self):
+        """global += grads; grads = 0   (GradAccumulator.accumulate)"""
+        if self.global_grads is None:
+            self.global_grads = torch.zeros_like(self.grads)
+        if self._acc_prog is None:
+            self._acc_prog = self._flat_prog(lambda: ops.grad_accumulate(self.ctx, self.global_grads, self.grads))
+        return self.ctx.run(self._acc_prog)
+
+    def optimizer_step(self, use_global=False):
+        """SGD-momentum over the flat buffers; with use_global the accumulated gradients are
+        consumed and zeroed (GradAccumulator.step)."""
+        if use_global:
+            if self.global_grads is None:
+                raise RuntimeError("optimizer_step(use_global=True) before any accumulate()")
+            if self._opt_global_prog is None:
+                def rec():
+                    ops.sgd_momentum_step(self.ctx, self.params, self.global_grads, self.momentum_buf, self.lr,
+                                          self.momentum, self.weight_decay, shadow=self.shadow)
+                    ops.fill_zero(self.ctx, self.global_grads)
+                self._opt_global_prog = self._flat_prog(rec)
+            return self.ctx.run(self._opt_global_prog)
+        if self._opt_prog is None:
+            self._opt_prog = self._flat_prog(lambda: ops.sgd_momentum_step(
+                self.ctx, self.params, self.grads, self.momentum_buf, self.lr, self.momentum, self.weight_decay,
+                shadow=self.shadow))
+        return self.ctx.run(self._opt_prog)
