@@ -1,0 +1,151 @@
+#!/usr/bin/env python3
+"""bench.py -- ResNet-152 bf16 batch-64 training step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps 20] [--warmup 5]
+
+A step is one pass of the hot path over one synthetic batch that already sits in HBM:
+NCHW->NHWC conversion, forward, softmax-CE, hand-written backward, SGD-momentum with the
+bf16 shadow refresh.  Prints ONE JSON line.  After the timed region the same programs
+are replayed with a HIP event between any two launches to attribute time to kernels
+(`roofline`, `conv_mfma_util`), and the CPU oracle step is timed on the host cores
+(`cpu_baseline`).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_FLOPS = 2.5e15   # MI355X dense bf16 MFMA
+PEAK_HBM_BYTES = 8.0e12    # MI355X HBM3E
+METRIC = "ResNet-152 bf16 bs64 train images/sec on 1 GPU; conv MFMA util %"
+
+
+def cpu_baseline(batch, timed_steps):
+    """The CPU oracle step (oracle/resnet.py: plain torch.nn ResNet-152, fp32, SGD) on the
+    host cores of this box: 1 warm-up step + `timed_steps` timed steps at the bench batch."""
+    import torch
+    from oracle import resnet as R
+    cores = torch.get_num_threads()
+    model = R.make_model((3, 8, 36, 3), 1000, 64, seed=0)
+    x, y = R.make_batch(batch, 224, 1000, seed=0)
+    R.train_steps(model, x, y, 1)
+    t0 = time.perf_counter()
+    R.train_steps(model, x, y, timed_steps)
+    dt = time.perf_counter() - t0
+    return {"value": batch * timed_steps / dt, "unit": "images/s", "cores": cores, "kind": "port",
+            "sample": f"ResNet-152 fp32 batch {batch} @224, torch CPU oracle step, 1 warm-up + {timed_steps} timed steps"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--profile-reps", type=int, default=2)
+    ap.add_argument("--cpu-steps", type=int, default=2, help="timed CPU oracle steps (0 = skip the CPU baseline)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from sirius_amd.resnet import ResNetEngine
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU; there is no CPU fallback"
+    torch.cuda.set_device(0)
+    B = args.batch
+    eng = ResNetEngine((3, 8, 36, 3), 1000, 64, dtype=torch.bfloat16, image_size=224, lr=0.1, momentum=0.9,
+                       weight_decay=1e-4)
+    eng.init_kaiming(seed=0)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(1)
+    x = torch.randn(B, 3, 224, 224, device="cuda", generator=g)
+    y = torch.randint(0, 1000, (B,), device="cuda", generator=g)
+    torch.cuda.synchronize()
+
+    def step():
+        eng.forward_backward(x, y)
+        eng.optimizer_step()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms = dt / args.steps * 1e3
+    plan = eng.plan(B)
+    loss = plan.loss.item()
+
+    # ---- per-kernel attribution (HIP events on the stream the kernels run on) ----
+    reps = max(1, args.profile_reps)
+    rows = eng.ctx.profile(plan.prog, reps) + eng.ctx.profile(eng._opt_prog, reps)
+    rows.sort(key=lambda r: -r["total_ms"])
+    total_ms = sum(r["total_ms"] for r in rows) / reps
+    conv = [r for r in rows if r["name"].startswith("igemm_kernel")]
+    conv_ms = sum(r["total_ms"] for r in conv) / reps
+    conv_flops = sum(r["work"] for r in conv) / reps
+    top = rows[0]
+    peak = PEAK_HBM_BYTES if top["work_is_bytes"] else PEAK_BF16_FLOPS
+    per_launch_work = top["work"] / top["launches"]
+    per_launch_s = top["total_ms"] / top["launches"] * 1e-3
+    achieved = per_launch_work / per_launch_s
+    roofline = {
+        "kernel": top["name"],
+        "bound": "hbm" if top["work_is_bytes"] else "mfma",
+        "achieved": achieved / (1e9 if top["work_is_bytes"] else 1e12),
+        "peak": peak / (1e9 if top["work_is_bytes"] else 1e12),
+        "unit": "GB/s" if top["work_is_bytes"] else "TFLOP/s",
+        "frac": achieved / peak,
+        "traffic": None,
+        "avg_launch_us": per_launch_s * 1e6,
+        "launches_per_step": top["launches"] // reps,
+        "share_of_step_kernel_time": top["total_ms"] / reps / total_ms,
+    }
+    breakdown = [{"kernel": r["name"], "ms_per_step": round(r["total_ms"] / reps, 4), "launches": r["launches"] // reps,
+                  ("GB/s" if r["work_is_bytes"] else "TFLOP/s"):
+                      round(r["work"] / (r["total_ms"] * 1e-3) / (1e9 if r["work_is_bytes"] else 1e12), 2)
+                  if r["total_ms"] > 0 else None}
+                 for r in rows[:12]]
+
+    out = {
+        "metric": METRIC,
+        "value": B * args.steps / dt,
+        "unit": "images/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"ResNet-152 training step, bf16 compute with fp32 master weights, batch {B} @ 3x224x224 "
+                               "N(0,1), labels uniform [0,1000), SGD-momentum(0.9, lr 0.1, wd 1e-4), Kaiming-normal init "
+                               "(BASELINE configs[1])",
+                   "global_batch": B, "launches_per_step": len(plan.prog) + len(eng._opt_prog)},
+        "loss_after_run": loss,
+        "roofline": roofline,
+        "conv_mfma_util": conv_flops / (conv_ms * 1e-3) / PEAK_BF16_FLOPS if conv_ms > 0 else None,
+        "conv_ms_per_step": conv_ms,
+        "conv_tflop_per_step": conv_flops / 1e12,
+        "kernel_ms_per_step": total_ms,
+        "breakdown": breakdown,
+    }
+    if args.cpu_steps > 0:
+        out["cpu_baseline"] = cpu_baseline(B, args.cpu_steps)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

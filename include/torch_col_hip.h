@@ -57,6 +57,19 @@ int tch_program_end_record(tch_context* ctx);
  * checkpoint between launches: returns 1 if any launch was skipped because of it. */
 int tch_program_run(tch_context* ctx, const tch_program* prog, int64_t first, int64_t last);
 
+/* ---- per-kernel timing of a program ---------------------------------------------- */
+typedef struct tch_kernel_stat {
+  char name[96];      /* kernel name, e.g. "igemm_kernel<bf16,fwd,128x128>" */
+  double total_ms;    /* summed HIP-event time of its launches over all repetitions */
+  double work;        /* summed ALGORITHMIC work of those launches: flops or bytes */
+  int64_t launches;
+  int work_is_bytes;  /* 1: work counts bytes (HBM-bound kernel), 0: flops (MFMA-bound) */
+} tch_kernel_stat;
+/* Replays prog `reps` times directly on the context's stream (not through a launch queue)
+ * with a HIP event between any two launches; one row per kernel name. */
+int tch_program_profile(tch_context* ctx, const tch_program* prog, int reps, tch_kernel_stat* out, int max_out,
+                        int* n_out);
+
 /* ---- preemptible launch queues (replaces common/xsched_ctrl.h:12-40) ------------ */
 uint64_t tch_RegisterStream(uint64_t hip_stream);   /* xsched_ctrl.cc:27-46; 0 on failure */
 int tch_UnRegisterStream(uint64_t hip_stream);      /* xsched_ctrl.cc:70-78 */
@@ -76,21 +89,24 @@ size_t tch_GetXQueueInFlight(uint64_t hip_stream);
 
 /* ---- convolution (implicit GEMM on MFMA) ---------------------------------------- */
 /* y[N,Ho,Wo,K] = conv(x[N,H,W,C], w[K,R,S,C]) (+ bias[K]) (+ add, optionally gated by mask > 0).
- * out_f32 != 0 stores y as fp32 whatever dtype is.  tile_cfg: -1 auto, 0 = 128x128, 1 = 128x64, 2 = 64x64. */
+ * out_f32 != 0 stores y as fp32 whatever dtype is.  tile_cfg: -1 auto, 0 = 128x128, 1 = 128x64, 2 = 64x64.
+ * c_logical: input channels that carry data when C is zero-padded to a chunk (0 = C); it only enters the
+ * algorithmic-work figure the profiler reports, never the arithmetic. */
 int tch_conv2d_fwd(tch_context* ctx, int dtype, const void* x, const void* w, void* y, const void* add,
                    const void* mask, const float* bias, int out_f32, int N, int H, int W, int C, int K, int R, int S,
-                   int stride, int pad, int tile_cfg);
-/* dx[N,H,W,C] = conv_transpose(dy[N,Ho,Wo,K], w) (+ add, optionally gated by mask > 0) */
-int tch_conv2d_dgrad(tch_context* ctx, int dtype, const void* dy, const void* w, void* dx, const void* add,
+                   int stride, int pad, int tile_cfg, int c_logical);
+/* dx[N,H,W,C] = conv_transpose(dy[N,Ho,Wo,K], w) (+ add, optionally gated by mask > 0).
+ * wt is the filter TRANSPOSED to [C][R][S][K] (tch_filter_transpose_batched). */
+int tch_conv2d_dgrad(tch_context* ctx, int dtype, const void* dy, const void* wt, void* dx, const void* add,
                      const void* mask, int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
-                     int tile_cfg);
+                     int tile_cfg, int c_logical);
 /* dw[K,R,S,C] (fp32) (+)= sum over pixels of dy x x.  splits > 1 needs a workspace of
  * tch_conv2d_wgrad_workspace_bytes(); splits <= 0 lets the library choose (query with _pick_splits). */
 int tch_conv2d_wgrad_pick_splits(int dtype, int N, int H, int W, int C, int K, int R, int S, int stride, int pad);
 int64_t tch_conv2d_wgrad_workspace_bytes(int dtype, int K, int R, int S, int C, int splits);
 int tch_conv2d_wgrad(tch_context* ctx, int dtype, const void* x, const void* dy, float* dw, float* workspace,
                      int splits, int accumulate, int N, int H, int W, int C, int K, int R, int S, int stride,
-                     int pad, int tile_cfg);
+                     int pad, int tile_cfg, int c_logical);
 
 /* ---- BatchNorm (training mode) with fused ReLU / residual ---------------------- */
 int64_t tch_bn_workspace_bytes(int dtype, int64_t rows, int C);
@@ -131,6 +147,12 @@ int tch_bias_grad(tch_context* ctx, int dtype, const void* dy, float* dbias, int
 /* ---- layout / precision ---------------------------------------------------------- */
 int tch_nchw_to_nhwc_pad(tch_context* ctx, int dtype, const float* x_nchw, void* y_nhwc, int N, int C, int H, int W,
                          int Cpad);
+/* dst[C][R*S][K] = src[K][R*S][C] for n_filters filters that live at the same element offsets inside
+ * two flat buffers, in ONE launch.  table_dev: device int64[n_filters][5] = {first tile, element offset,
+ * K, R*S, C}; a filter owns R*S * ceil(K/32) * ceil(C/32) tiles; total_tiles is their sum.
+ * tch_conv2d_dgrad reads filters in this transposed layout. */
+int tch_filter_transpose_batched(tch_context* ctx, int dtype, const void* src, void* dst, const int64_t* table_dev,
+                                 int n_filters, int64_t total_tiles, int64_t total_elems);
 int tch_cast_from_f32(tch_context* ctx, int dtype, const float* src, void* dst, int64_t n);
 int tch_cast_to_f32(tch_context* ctx, int dtype, const void* src, float* dst, int64_t n);
 

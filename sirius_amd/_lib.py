@@ -17,6 +17,12 @@ class TorchColHipError(RuntimeError):
     pass
 
 
+class KernelStat(ctypes.Structure):
+    """Mirror of tch_kernel_stat (include/torch_col_hip.h)."""
+    _fields_ = [("name", ctypes.c_char * 96), ("total_ms", ctypes.c_double), ("work", ctypes.c_double),
+                ("launches", c_int64), ("work_is_bytes", c_int)]
+
+
 def _declare(lib):
     vp, i, i64, f = c_void_p, c_int, c_int64, c_float
     sig = {
@@ -45,11 +51,12 @@ def _declare(lib):
         "tch_SetRejectCudaCalls": (None, [i]),
         "tch_SetXQueueShape": (None, [i, i]),
         "tch_GetXQueueInFlight": (c_size_t, [c_uint64]),
-        "tch_conv2d_fwd": (i, [vp, i, vp, vp, vp, vp, vp, vp, i] + [i] * 10),
-        "tch_conv2d_dgrad": (i, [vp, i, vp, vp, vp, vp, vp] + [i] * 10),
+        "tch_program_profile": (i, [vp, vp, i, vp, i, POINTER(c_int)]),
+        "tch_conv2d_fwd": (i, [vp, i, vp, vp, vp, vp, vp, vp, i] + [i] * 11),
+        "tch_conv2d_dgrad": (i, [vp, i, vp, vp, vp, vp, vp] + [i] * 11),
         "tch_conv2d_wgrad_pick_splits": (i, [i] * 10),
         "tch_conv2d_wgrad_workspace_bytes": (i64, [i] * 6),
-        "tch_conv2d_wgrad": (i, [vp, i, vp, vp, vp, vp, i, i] + [i] * 10),
+        "tch_conv2d_wgrad": (i, [vp, i, vp, vp, vp, vp, i, i] + [i] * 11),
         "tch_bn_workspace_bytes": (i64, [i, i64, i]),
         "tch_bn_fwd_train": (i, [vp, i, vp, vp, vp, i, i64, i, vp, vp, vp, vp, vp, vp, f, f, vp]),
         "tch_bn_bwd": (i, [vp, i, vp, vp, vp, vp, i64, i, vp, vp, vp, vp, vp, i, vp]),
@@ -63,6 +70,7 @@ def _declare(lib):
         "tch_fill_zero": (i, [vp, vp, i64]),
         "tch_bias_grad": (i, [vp, i, vp, vp, i, i, i, i]),
         "tch_nchw_to_nhwc_pad": (i, [vp, i, vp, vp, i, i, i, i, i]),
+        "tch_filter_transpose_batched": (i, [vp, i, vp, vp, vp, i, i64, i64]),
         "tch_cast_from_f32": (i, [vp, i, vp, vp, i64]),
         "tch_cast_to_f32": (i, [vp, i, vp, vp, i64]),
     }

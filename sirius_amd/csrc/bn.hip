@@ -125,15 +125,39 @@ struct FwdFinalizeArgs {
   float momentum, eps;
 };
 
-__global__ __launch_bounds__(64) void bn_fwd_finalize_kernel(FwdFinalizeArgs p) {
-  const int c = blockIdx.x * 64 + threadIdx.x;
-  if (c >= p.C) return;
+// Sum the per-row-block partials of one channel: 8 channels x 32 lanes per workgroup, each
+// lane strides over the row blocks in fp64, then a tree over the 32 lanes through LDS.
+__device__ inline bool finalize_sums(const float* partial, int row_blocks, int C, int c, int lane, double* s_out,
+                                     double* q_out) {
+  __shared__ double red[32][8][2];
   double s = 0.0, q = 0.0;
-  for (int b = 0; b < p.row_blocks; ++b) {
-    const float* src = p.partial + (static_cast<int64_t>(b) * p.C + c) * 2;
-    s += src[0];
-    q += src[1];
+  if (c < C) {
+    for (int b = lane; b < row_blocks; b += 32) {
+      const float2 v = *reinterpret_cast<const float2*>(partial + (static_cast<int64_t>(b) * C + c) * 2);
+      s += v.x;
+      q += v.y;
+    }
   }
+  const int cl = threadIdx.x & 7;
+  red[lane][cl][0] = s;
+  red[lane][cl][1] = q;
+  __syncthreads();
+  for (int off = 16; off > 0; off >>= 1) {
+    if (lane < off) {
+      red[lane][cl][0] += red[lane + off][cl][0];
+      red[lane][cl][1] += red[lane + off][cl][1];
+    }
+    __syncthreads();
+  }
+  *s_out = red[0][cl][0];
+  *q_out = red[0][cl][1];
+  return lane == 0 && c < C;
+}
+
+__global__ __launch_bounds__(256) void bn_fwd_finalize_kernel(FwdFinalizeArgs p) {
+  const int c = blockIdx.x * 8 + (threadIdx.x & 7);
+  double s, q;
+  if (!finalize_sums(p.partial, p.row_blocks, p.C, c, threadIdx.x >> 3, &s, &q)) return;
   const double n = static_cast<double>(p.rows);
   const double mean = s / n;
   double var = q / n - mean * mean;
@@ -164,15 +188,10 @@ struct BwdFinalizeArgs {
   int accumulate;
 };
 
-__global__ __launch_bounds__(64) void bn_bwd_finalize_kernel(BwdFinalizeArgs p) {
-  const int c = blockIdx.x * 64 + threadIdx.x;
-  if (c >= p.C) return;
-  double s1 = 0.0, s2 = 0.0;
-  for (int b = 0; b < p.row_blocks; ++b) {
-    const float* src = p.partial + (static_cast<int64_t>(b) * p.C + c) * 2;
-    s1 += src[0];
-    s2 += src[1];
-  }
+__global__ __launch_bounds__(256) void bn_bwd_finalize_kernel(BwdFinalizeArgs p) {
+  const int c = blockIdx.x * 8 + (threadIdx.x & 7);
+  double s1, s2;
+  if (!finalize_sums(p.partial, p.row_blocks, p.C, c, threadIdx.x >> 3, &s1, &s2)) return;
   const float db = static_cast<float>(s1), dg = static_cast<float>(s2);
   p.dbeta[c] = p.accumulate ? p.dbeta[c] + db : db;
   p.dgamma[c] = p.accumulate ? p.dgamma[c] + dg : dg;
@@ -266,7 +285,7 @@ Geometry geometry(int64_t rows, int C, int dtype) {
   g.col_blocks = (g.cc + ccb - 1) / ccb;
   g.rowlanes = 256 / ccb;
   int64_t rb = rows / (static_cast<int64_t>(g.rowlanes) * 8);
-  int64_t cap = 2048 / g.col_blocks;
+  int64_t cap = 1024 / g.col_blocks;
   if (cap < 1) cap = 1;
   if (rb > cap) rb = cap;
   if (rb < 1) rb = 1;
@@ -310,16 +329,22 @@ int bn_fwd_train(Context* ctx, int dtype, const void* x, void* y, const void* re
   float* shift = scale + C;
   ColReduceArgs r{x, nullptr, nullptr, nullptr, nullptr, partial, rows, C, g.cc, g.ccb, g.rowlanes, g.rows_per_block};
   dim3 grid(g.col_blocks, g.row_blocks);
-  int rc = dtype == kBF16 ? launch(ctx, col_reduce_kernel<bf16, 0>, grid, dim3(256), r)
-                          : launch(ctx, col_reduce_kernel<float, 0>, grid, dim3(256), r);
+  const double eb = dtype == kBF16 ? 2.0 : 4.0;
+  const double tensor_bytes = static_cast<double>(rows) * C * eb;
+  int rc = dtype == kBF16 ? launch(ctx, col_reduce_kernel<bf16, 0>, grid, dim3(256), r, "bn_stats_kernel<bf16>", tensor_bytes, 1)
+                          : launch(ctx, col_reduce_kernel<float, 0>, grid, dim3(256), r, "bn_stats_kernel<f32>", tensor_bytes, 1);
   if (rc) return rc;
   FwdFinalizeArgs f{partial, g.row_blocks, C, rows, gamma, beta, running_mean, running_var, save_mean, save_invstd,
                     scale,   shift,        momentum, eps};
-  rc = launch(ctx, bn_fwd_finalize_kernel, dim3((C + 63) / 64), dim3(64), f);
+  rc = launch(ctx, bn_fwd_finalize_kernel, dim3((C + 7) / 8), dim3(256), f, "bn_fwd_finalize_kernel",
+              8.0 * g.row_blocks * C, 1);
   if (rc) return rc;
   ApplyArgs a{x, residual, nullptr, y, scale, shift, nullptr, rows * g.cc, FastDiv(g.cc), relu};
-  return dtype == kBF16 ? launch(ctx, bn_apply_kernel<bf16, 0>, dim3(apply_blocks(a.chunks)), dim3(256), a)
-                        : launch(ctx, bn_apply_kernel<float, 0>, dim3(apply_blocks(a.chunks)), dim3(256), a);
+  const double apply_bytes = tensor_bytes * (residual ? 3.0 : 2.0);
+  return dtype == kBF16 ? launch(ctx, bn_apply_kernel<bf16, 0>, dim3(apply_blocks(a.chunks)), dim3(256), a,
+                                 "bn_apply_kernel<bf16,fwd>", apply_bytes, 1)
+                        : launch(ctx, bn_apply_kernel<float, 0>, dim3(apply_blocks(a.chunks)), dim3(256), a,
+                                 "bn_apply_kernel<f32,fwd>", apply_bytes, 1);
 }
 
 int bn_bwd(Context* ctx, int dtype, const void* dy, const void* relu_mask, const void* x, void* dx, int64_t rows,
@@ -333,15 +358,23 @@ int bn_bwd(Context* ctx, int dtype, const void* dy, const void* relu_mask, const
   float* coef = workspace + static_cast<int64_t>(g.row_blocks) * C * 2;
   ColReduceArgs r{dy, relu_mask, x, save_mean, save_invstd, partial, rows, C, g.cc, g.ccb, g.rowlanes, g.rows_per_block};
   dim3 grid(g.col_blocks, g.row_blocks);
-  int rc = dtype == kBF16 ? launch(ctx, col_reduce_kernel<bf16, 1>, grid, dim3(256), r)
-                          : launch(ctx, col_reduce_kernel<float, 1>, grid, dim3(256), r);
+  const double eb = dtype == kBF16 ? 2.0 : 4.0;
+  const double tensor_bytes = static_cast<double>(rows) * C * eb;
+  const double in_tensors = relu_mask ? 3.0 : 2.0;
+  int rc = dtype == kBF16 ? launch(ctx, col_reduce_kernel<bf16, 1>, grid, dim3(256), r, "bn_bwd_reduce_kernel<bf16>",
+                                   tensor_bytes * in_tensors, 1)
+                          : launch(ctx, col_reduce_kernel<float, 1>, grid, dim3(256), r, "bn_bwd_reduce_kernel<f32>",
+                                   tensor_bytes * in_tensors, 1);
   if (rc) return rc;
   BwdFinalizeArgs f{partial, g.row_blocks, C, rows, gamma, save_mean, save_invstd, dgamma, dbeta, coef, accumulate};
-  rc = launch(ctx, bn_bwd_finalize_kernel, dim3((C + 63) / 64), dim3(64), f);
+  rc = launch(ctx, bn_bwd_finalize_kernel, dim3((C + 7) / 8), dim3(256), f, "bn_bwd_finalize_kernel",
+              8.0 * g.row_blocks * C, 1);
   if (rc) return rc;
   ApplyArgs a{dy, relu_mask, x, dx, coef, coef + C, coef + 2 * C, rows * g.cc, FastDiv(g.cc), 0};
-  return dtype == kBF16 ? launch(ctx, bn_apply_kernel<bf16, 1>, dim3(apply_blocks(a.chunks)), dim3(256), a)
-                        : launch(ctx, bn_apply_kernel<float, 1>, dim3(apply_blocks(a.chunks)), dim3(256), a);
+  return dtype == kBF16 ? launch(ctx, bn_apply_kernel<bf16, 1>, dim3(apply_blocks(a.chunks)), dim3(256), a,
+                                 "bn_apply_kernel<bf16,bwd>", tensor_bytes * (in_tensors + 1.0), 1)
+                        : launch(ctx, bn_apply_kernel<float, 1>, dim3(apply_blocks(a.chunks)), dim3(256), a,
+                                 "bn_apply_kernel<f32,bwd>", tensor_bytes * (in_tensors + 1.0), 1);
 }
 
 }  // namespace tch

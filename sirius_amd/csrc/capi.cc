@@ -4,6 +4,8 @@
 #include "context.h"
 #include "ops.h"
 
+#include <stdio.h>
+
 using namespace tch;
 
 struct tch_context {
@@ -16,8 +18,8 @@ struct tch_program {
 
 namespace {
 inline Context* C(tch_context* c) { return c ? &c->ctx : nullptr; }
-inline ConvShape shape(int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad) {
-  ConvShape s{N, H, W, Cc, K, R, S, stride, pad};
+inline ConvShape shape(int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad, int c_logical = 0) {
+  ConvShape s{N, H, W, Cc, K, R, S, stride, pad, c_logical};
   return s;
 }
 }  // namespace
@@ -122,15 +124,15 @@ size_t tch_GetXQueueInFlight(uint64_t hip_stream) {
 
 int tch_conv2d_fwd(tch_context* ctx, int dtype, const void* x, const void* w, void* y, const void* add,
                    const void* mask, const float* bias, int out_f32, int N, int H, int W, int Cc, int K, int R, int S,
-                   int stride, int pad, int tile_cfg) {
-  return conv2d_fwd(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad), x, w, y, add, mask, bias, out_f32,
+                   int stride, int pad, int tile_cfg, int c_logical) {
+  return conv2d_fwd(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad, c_logical), x, w, y, add, mask, bias, out_f32,
                     tile_cfg);
 }
 
 int tch_conv2d_dgrad(tch_context* ctx, int dtype, const void* dy, const void* w, void* dx, const void* add,
                      const void* mask, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad,
-                     int tile_cfg) {
-  return conv2d_dgrad(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad), dy, w, dx, add, mask, tile_cfg);
+                     int tile_cfg, int c_logical) {
+  return conv2d_dgrad(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad, c_logical), dy, w, dx, add, mask, tile_cfg);
 }
 
 int tch_conv2d_wgrad_pick_splits(int dtype, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad) {
@@ -143,8 +145,8 @@ int64_t tch_conv2d_wgrad_workspace_bytes(int dtype, int K, int R, int S, int Cc,
 
 int tch_conv2d_wgrad(tch_context* ctx, int dtype, const void* x, const void* dy, float* dw, float* workspace,
                      int splits, int accumulate, int N, int H, int W, int Cc, int K, int R, int S, int stride,
-                     int pad, int tile_cfg) {
-  ConvShape s = shape(N, H, W, Cc, K, R, S, stride, pad);
+                     int pad, int tile_cfg, int c_logical) {
+  ConvShape s = shape(N, H, W, Cc, K, R, S, stride, pad, c_logical);
   if (splits <= 0) splits = workspace ? conv2d_wgrad_pick_splits(s, dtype) : 1;
   return conv2d_wgrad(C(ctx), dtype, s, x, dy, dw, workspace, splits, accumulate, tile_cfg);
 }
@@ -211,6 +213,11 @@ int tch_nchw_to_nhwc_pad(tch_context* ctx, int dtype, const float* x_nchw, void*
   return nchw_to_nhwc_pad(C(ctx), dtype, x_nchw, y_nhwc, N, Cc, H, W, Cpad);
 }
 
+int tch_filter_transpose_batched(tch_context* ctx, int dtype, const void* src, void* dst, const int64_t* table_dev,
+                                 int n_filters, int64_t total_tiles, int64_t total_elems) {
+  return filter_transpose_batched(C(ctx), dtype, src, dst, table_dev, n_filters, total_tiles, total_elems);
+}
+
 int tch_cast_from_f32(tch_context* ctx, int dtype, const float* src, void* dst, int64_t n) {
   return cast_f32(C(ctx), dtype, src, dst, n);
 }
@@ -220,3 +227,27 @@ int tch_cast_to_f32(tch_context* ctx, int dtype, const void* src, float* dst, in
 }
 
 }  // extern "C"
+
+// ---- built-in per-kernel profiler -------------------------------------------------
+extern "C" int tch_program_profile(tch_context* ctx, const tch_program* prog, int reps, tch_kernel_stat* out,
+                                   int max_out, int* n_out) {
+  if (!ctx || !prog || !out || !n_out || max_out < 1) {
+    set_error("tch_program_profile: bad arguments");
+    return -22;
+  }
+  std::vector<KernelStat> stats;
+  int rc = profile_program(&ctx->ctx, prog->prog, reps, &stats);
+  if (rc) return rc;
+  int n = 0;
+  for (auto& s : stats) {
+    if (n >= max_out) break;
+    tch_kernel_stat& o = out[n++];
+    snprintf(o.name, sizeof(o.name), "%s", s.name.c_str());
+    o.total_ms = s.total_ms;
+    o.work = s.work;
+    o.launches = s.launches;
+    o.work_is_bytes = s.work_is_bytes;
+  }
+  *n_out = n;
+  return 0;
+}

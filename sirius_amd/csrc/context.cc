@@ -213,7 +213,8 @@ int Context::dispatch(const LaunchRecord& rec) {
   return launch_now(stream, rec);
 }
 
-int submit(Context* ctx, const void* fn, dim3 grid, dim3 block, const void* args, size_t arg_bytes) {
+int submit(Context* ctx, const void* fn, dim3 grid, dim3 block, const void* args, size_t arg_bytes,
+           const char* name, double work, int work_is_bytes) {
   if (!ctx) {
     set_error("null context");
     return -22;
@@ -227,12 +228,62 @@ int submit(Context* ctx, const void* fn, dim3 grid, dim3 block, const void* args
   rec.grid = grid;
   rec.block = block;
   rec.arg_bytes = static_cast<uint32_t>(arg_bytes);
+  rec.name = name;
+  rec.work = work;
+  rec.work_is_bytes = work_is_bytes;
   memcpy(rec.args, args, arg_bytes);
   if (ctx->recording) {
     ctx->recording->launches.push_back(rec);
     return 0;
   }
   return ctx->dispatch(rec);
+}
+
+// ---------------------------------------------------------------------------
+// per-kernel timing of a recorded program
+// ---------------------------------------------------------------------------
+
+int profile_program(Context* ctx, const Program& prog, int reps, std::vector<KernelStat>* out) {
+  const size_t n = prog.launches.size();
+  if (n == 0 || reps < 1) return 0;
+  std::vector<hipEvent_t> ev(n + 1, nullptr);
+  for (auto& e : ev) {
+    if (hipEventCreate(&e) != hipSuccess) {
+      set_error("profile_program: hipEventCreate failed");
+      for (auto x : ev)
+        if (x) (void)hipEventDestroy(x);
+      return -12;
+    }
+  }
+  std::map<std::string, KernelStat> agg;
+  int rc = 0;
+  for (int r = 0; r < reps && rc == 0; ++r) {
+    // one event between any two launches: launch i runs between ev[i] and ev[i+1]
+    (void)hipEventRecord(ev[0], ctx->stream);
+    for (size_t i = 0; i < n && rc == 0; ++i) {
+      rc = launch_now(ctx->stream, prog.launches[i]);
+      (void)hipEventRecord(ev[i + 1], ctx->stream);
+    }
+    if (hipStreamSynchronize(ctx->stream) != hipSuccess) {
+      set_error("profile_program: stream synchronize failed");
+      rc = -5;
+    }
+    for (size_t i = 0; i < n && rc == 0; ++i) {
+      float ms = 0.f;
+      (void)hipEventElapsedTime(&ms, ev[i], ev[i + 1]);
+      const LaunchRecord& l = prog.launches[i];
+      KernelStat& k = agg[l.name ? l.name : "kernel"];
+      k.name = l.name ? l.name : "kernel";
+      k.total_ms += ms;
+      k.work += l.work;
+      k.launches += 1;
+      k.work_is_bytes = l.work_is_bytes;
+    }
+  }
+  for (auto e : ev) (void)hipEventDestroy(e);
+  if (rc == 0)
+    for (auto& kv : agg) out->push_back(kv.second);
+  return rc;
 }
 
 // ---------------------------------------------------------------------------

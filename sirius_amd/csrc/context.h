@@ -18,6 +18,7 @@
 #include <deque>
 #include <memory>
 #include <mutex>
+#include <string>
 #include <thread>
 #include <vector>
 
@@ -103,6 +104,18 @@ class Context {
 
   int dispatch(const LaunchRecord& rec);
 };
+
+struct KernelStat {
+  std::string name;
+  double total_ms = 0.0;
+  double work = 0.0;  // sum of the algorithmic work of the launches
+  int64_t launches = 0;
+  int work_is_bytes = 1;
+};
+
+// Replays prog `reps` times directly on the context's stream with a HIP event between any
+// two launches and sums the elapsed time per kernel name.
+int profile_program(Context* ctx, const Program& prog, int reps, std::vector<KernelStat>* out);
 
 // ---- process-wide registry of preemptible streams (xsched_ctrl equivalent) ----
 uint64_t register_stream(uint64_t stream);  // returns a handle, 0 on failure

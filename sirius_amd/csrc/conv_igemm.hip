@@ -22,6 +22,8 @@
 #include "kernels.h"
 #include "ops.h"
 
+#include <string>
+
 namespace tch {
 namespace {
 
@@ -190,12 +192,6 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm_kernel(IgemmArgs p) {
       }
     }
   }
-  if constexpr (MODE == kDgrad) {
-    t_act_b = tid < B_BLOCKS;
-    t_kc_b = tid & 3;
-    t_row0_b = n0 + (tid >> 2) * E;
-    b_walk.init(k_begin + t_kc_b * E, p.K);
-  }
   if constexpr (MODE == kWgrad) {
     t_act_a = tid < A_BLOCKS;
     t_kc_a = tid & 3;
@@ -212,7 +208,7 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm_kernel(IgemmArgs p) {
   }
 
   Chunk ra[(MODE == kWgrad) ? E : A_PT];
-  Chunk rb[(MODE == kFwd) ? B_PT : E];
+  Chunk rb[(MODE == kWgrad) ? E : B_PT];
 
   auto load_tiles = [&](int kt) {
     const int k0 = k_begin + kt * BK;
@@ -252,7 +248,8 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm_kernel(IgemmArgs p) {
       }
     }
     // ---- operand B ----
-    if constexpr (MODE == kFwd) {
+    if constexpr (MODE == kFwd || MODE == kDgrad) {
+      // dense filter rows: FWD reads w[K][R*S*C], DGRAD reads the transposed filter wt[C][R*S*K]
 #pragma unroll
       for (int i = 0; i < B_PT; ++i) {
         int q = tid + i * NT;
@@ -261,15 +258,6 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm_kernel(IgemmArgs p) {
         bool ok = (q < BN * 4) && row < p.gemm_n && k < k_end;
         rb[i] = load_chunk(p.b_src, static_cast<int64_t>(row) * p.gemm_k + k, EB, ok);
       }
-    } else if constexpr (MODE == kDgrad) {
-      // rows = input channels (contiguous in w), reduction = (tap, out channel)
-      const bool ok = t_act_b && t_row0_b < p.gemm_n && b_walk.tap < RS && (k0 + t_kc_b * E) < k_end;
-#pragma unroll
-      for (int j = 0; j < E; ++j) {
-        int64_t off = (static_cast<int64_t>(b_walk.ch + j) * RS + b_walk.tap) * p.C + t_row0_b;
-        rb[j] = load_chunk(p.b_src, off, EB, ok);
-      }
-      b_walk.advance(BK, p.K);
     } else {
       // WGRAD B: rows = (tap, in channel) fixed per thread, reduction = pixels
       const int pix0 = k0 + t_kc_b * E;
@@ -324,7 +312,7 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm_kernel(IgemmArgs p) {
         for (int e = 0; e < E; ++e) lds_a[buf][(row + e) * kLdsStride + t_kc_a] = t[e].u;
       }
     }
-    if constexpr (MODE == kFwd) {
+    if constexpr (MODE == kFwd || MODE == kDgrad) {
 #pragma unroll
       for (int i = 0; i < B_PT; ++i) {
         int q = tid + i * NT;
@@ -457,7 +445,15 @@ int ilog2_exact(int v) {
 }
 
 template <typename T, int MODE, int WM, int WN, int TM, int TN>
-int launch_cfg(Context* ctx, IgemmArgs& a) {
+const char* igemm_name() {
+  static const std::string name = std::string("igemm_kernel<") + (sizeof(T) == 2 ? "bf16" : "f32") + "," +
+                                  (MODE == kFwd ? "fwd" : MODE == kDgrad ? "dgrad" : "wgrad") + "," +
+                                  std::to_string(WM * TM * 32) + "x" + std::to_string(WN * TN * 32) + ">";
+  return name.c_str();
+}
+
+template <typename T, int MODE, int WM, int WN, int TM, int TN>
+int launch_cfg(Context* ctx, IgemmArgs& a, double flops) {
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
   a.tiles_m = (a.gemm_m + BM - 1) / BM;
   a.tiles_n = (a.gemm_n + BN - 1) / BN;
@@ -466,19 +462,27 @@ int launch_cfg(Context* ctx, IgemmArgs& a) {
     set_error("igemm: grid out of range");
     return -22;
   }
-  return launch(ctx, igemm_kernel<T, MODE, WM, WN, TM, TN>, dim3(static_cast<unsigned>(wgs)), dim3(WM * WN * 64), a);
+  return launch(ctx, igemm_kernel<T, MODE, WM, WN, TM, TN>, dim3(static_cast<unsigned>(wgs)), dim3(WM * WN * 64), a,
+                igemm_name<T, MODE, WM, WN, TM, TN>(), flops, 0);
 }
 
 template <typename T, int MODE>
-int launch_mode(Context* ctx, IgemmArgs& a, int tile_cfg) {
+int launch_mode(Context* ctx, IgemmArgs& a, int tile_cfg, double flops) {
   switch (tile_cfg) {
     case 0:
-      return launch_cfg<T, MODE, 2, 2, 2, 2>(ctx, a);  // 128 x 128
+      return launch_cfg<T, MODE, 2, 2, 2, 2>(ctx, a, flops);  // 128 x 128
     case 1:
-      return launch_cfg<T, MODE, 2, 2, 2, 1>(ctx, a);  // 128 x 64
+      return launch_cfg<T, MODE, 2, 2, 2, 1>(ctx, a, flops);  // 128 x 64
     default:
-      return launch_cfg<T, MODE, 2, 2, 1, 1>(ctx, a);  // 64 x 64
+      return launch_cfg<T, MODE, 2, 2, 1, 1>(ctx, a, flops);  // 64 x 64
   }
+}
+
+// 2 * N*Ho*Wo * K * R*S*C: the same for forward, data gradient and weight gradient;
+// zero-padded input channels do no algorithmic work
+double conv_flops(const ConvShape& s, int Ho, int Wo) {
+  const int c = (s.c_logical > 0 && s.c_logical < s.C) ? s.c_logical : s.C;
+  return 2.0 * s.N * Ho * Wo * static_cast<double>(s.K) * s.R * s.S * c;
 }
 
 int64_t tiles_for(int m, int n, int bm, int bn) {
@@ -555,7 +559,8 @@ int conv2d_fwd(Context* ctx, int dtype, const ConvShape& s, const void* x, const
   a.div_plane = FastDiv(a.Ho * a.Wo);
   a.div_width = FastDiv(a.Wo);
   if (tile_cfg < 0) tile_cfg = pick_tile(a.gemm_m, a.gemm_n, 1);
-  return dtype == kBF16 ? launch_mode<bf16, kFwd>(ctx, a, tile_cfg) : launch_mode<float, kFwd>(ctx, a, tile_cfg);
+  return dtype == kBF16 ? launch_mode<bf16, kFwd>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo))
+                        : launch_mode<float, kFwd>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo));
 }
 
 int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, const void* w, void* dx, const void* add,
@@ -575,7 +580,8 @@ int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, co
   a.div_plane = FastDiv(s.H * s.W);
   a.div_width = FastDiv(s.W);
   if (tile_cfg < 0) tile_cfg = pick_tile(a.gemm_m, a.gemm_n, 1);
-  return dtype == kBF16 ? launch_mode<bf16, kDgrad>(ctx, a, tile_cfg) : launch_mode<float, kDgrad>(ctx, a, tile_cfg);
+  return dtype == kBF16 ? launch_mode<bf16, kDgrad>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo))
+                        : launch_mode<float, kDgrad>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo));
 }
 
 int64_t conv2d_wgrad_workspace_bytes(const ConvShape& s, int dtype, int splits) {
@@ -626,13 +632,15 @@ int conv2d_wgrad(Context* ctx, int dtype, const ConvShape& s, const void* x, con
   if (tile_cfg < 0) {
     tile_cfg = (a.gemm_m >= 128 && a.gemm_n >= 128 && tiles_for(a.gemm_m, a.gemm_n, 128, 128) * splits >= 256) ? 0 : 2;
   }
-  int rc = dtype == kBF16 ? launch_mode<bf16, kWgrad>(ctx, a, tile_cfg) : launch_mode<float, kWgrad>(ctx, a, tile_cfg);
+  int rc = dtype == kBF16 ? launch_mode<bf16, kWgrad>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo))
+                          : launch_mode<float, kWgrad>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo));
   if (rc) return rc;
   if (splits > 1) {
     ReduceArgs r{workspace, dw, static_cast<int64_t>(a.gemm_m) * a.gemm_n, splits, accumulate};
     TCH_CHECK_ARG(r.n % 4 == 0, "conv2d_wgrad: filter size must be a multiple of 4");
     unsigned blocks = static_cast<unsigned>((r.n / 4 + 255) / 256);
-    return launch(ctx, splitk_reduce_kernel, dim3(blocks), dim3(256), r);
+    return launch(ctx, splitk_reduce_kernel, dim3(blocks), dim3(256), r, "splitk_reduce_kernel",
+                  4.0 * r.n * (splits + 1 + (accumulate ? 1 : 0)), 1);
   }
   return 0;
 }

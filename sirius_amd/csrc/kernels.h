@@ -175,18 +175,27 @@ struct LaunchRecord {
   dim3 grid;
   dim3 block;
   uint32_t arg_bytes;
+  // annotation for the built-in profiler: a static name and the ALGORITHMIC work of
+  // this launch (flops for MFMA-bound kernels, bytes for HBM-bound ones)
+  const char* name;
+  double work;
+  int work_is_bytes;
   alignas(16) unsigned char args[360];
 };
 
 class Context;  // defined in context.h
 
-int submit(Context* ctx, const void* fn, dim3 grid, dim3 block, const void* args, size_t arg_bytes);
+int submit(Context* ctx, const void* fn, dim3 grid, dim3 block, const void* args, size_t arg_bytes,
+           const char* name, double work, int work_is_bytes);
 
+// name must have static storage duration
 template <typename Args>
-inline int launch(Context* ctx, void (*kernel)(Args), dim3 grid, dim3 block, const Args& args) {
+inline int launch(Context* ctx, void (*kernel)(Args), dim3 grid, dim3 block, const Args& args,
+                  const char* name = "kernel", double work = 0.0, int work_is_bytes = 1) {
   static_assert(sizeof(Args) <= sizeof(LaunchRecord::args), "kernel argument struct too large");
   static_assert(std::is_trivially_copyable<Args>::value, "kernel arguments must be POD");
-  return submit(ctx, reinterpret_cast<const void*>(kernel), grid, block, &args, sizeof(Args));
+  return submit(ctx, reinterpret_cast<const void*>(kernel), grid, block, &args, sizeof(Args), name, work,
+                work_is_bytes);
 }
 
 void set_error(const std::string& msg);

@@ -175,38 +175,43 @@ int softmax_ce_fwd_bwd(Context* ctx, int dtype, const float* logits, const int64
   TCH_CHECK_ARG(logits && labels && loss_rows && loss_mean && dlogits, "softmax_ce: null tensor");
   TCH_CHECK_ARG(rows > 0 && classes > 0 && ld_dlogits >= classes, "softmax_ce: bad shape");
   CeArgs a{logits, labels, loss_rows, dlogits, rows, classes, ld_dlogits, grad_scale};
-  int rc = dtype == kBF16 ? launch(ctx, softmax_ce_kernel<bf16>, dim3(rows), dim3(64), a)
-                          : launch(ctx, softmax_ce_kernel<float>, dim3(rows), dim3(64), a);
+  const double bytes = static_cast<double>(rows) * classes * (4.0 + (dtype == kBF16 ? 2.0 : 4.0));
+  int rc = dtype == kBF16 ? launch(ctx, softmax_ce_kernel<bf16>, dim3(rows), dim3(64), a, "softmax_ce_kernel<bf16>", bytes, 1)
+                          : launch(ctx, softmax_ce_kernel<float>, dim3(rows), dim3(64), a, "softmax_ce_kernel<f32>", bytes, 1);
   if (rc) return rc;
   MeanArgs m{loss_rows, loss_mean, rows};
-  return launch(ctx, mean_kernel, dim3(1), dim3(64), m);
+  return launch(ctx, mean_kernel, dim3(1), dim3(64), m, "mean_kernel", 4.0 * rows, 1);
 }
 
 int sgd_momentum_step(Context* ctx, float* param, const float* grad, float* momentum_buf, void* shadow_bf16,
                       int64_t n, float lr, float momentum, float weight_decay) {
   TCH_CHECK_ARG(param && grad && momentum_buf && n > 0, "sgd_momentum_step: null tensor or empty");
   SgdArgs a{param, grad, momentum_buf, static_cast<uint16_t*>(shadow_bf16), n, lr, momentum, weight_decay};
-  return launch(ctx, sgd_kernel, dim3(flat_blocks((n + 3) / 4)), dim3(256), a);
+  return launch(ctx, sgd_kernel, dim3(flat_blocks((n + 3) / 4)), dim3(256), a, "sgd_kernel",
+                static_cast<double>(n) * (shadow_bf16 ? 22.0 : 20.0), 1);
 }
 
 int grad_accumulate(Context* ctx, float* global, float* grad, int64_t n) {
   TCH_CHECK_ARG(global && grad && n > 0, "grad_accumulate: null tensor or empty");
   AccumArgs a{global, grad, n};
-  return launch(ctx, accumulate_kernel, dim3(flat_blocks((n + 3) / 4)), dim3(256), a);
+  return launch(ctx, accumulate_kernel, dim3(flat_blocks((n + 3) / 4)), dim3(256), a, "accumulate_kernel",
+                static_cast<double>(n) * 16.0, 1);
 }
 
 int fill_zero(Context* ctx, void* ptr, int64_t bytes) {
   TCH_CHECK_ARG(ptr && bytes > 0 && bytes % 4 == 0, "fill_zero: size must be a positive multiple of 4 bytes");
   FillArgs a{static_cast<uint32_t*>(ptr), bytes / 4};
-  return launch(ctx, fill_zero_kernel, dim3(flat_blocks(a.words)), dim3(256), a);
+  return launch(ctx, fill_zero_kernel, dim3(flat_blocks(a.words)), dim3(256), a, "fill_zero_kernel",
+                static_cast<double>(bytes), 1);
 }
 
 int bias_grad(Context* ctx, int dtype, const void* dy, float* dbias, int rows, int cols, int ld, int accumulate) {
   TCH_CHECK_ARG(dtype == kBF16 || dtype == kF32, "bias_grad: dtype must be f32(0) or bf16(1)");
   TCH_CHECK_ARG(dy && dbias && rows > 0 && cols > 0 && ld >= cols, "bias_grad: bad arguments");
   BiasGradArgs a{dy, dbias, rows, cols, ld, accumulate};
-  return dtype == kBF16 ? launch(ctx, bias_grad_kernel<bf16>, dim3((cols + 255) / 256), dim3(256), a)
-                        : launch(ctx, bias_grad_kernel<float>, dim3((cols + 255) / 256), dim3(256), a);
+  const double bytes = static_cast<double>(rows) * cols * (dtype == kBF16 ? 2.0 : 4.0);
+  return dtype == kBF16 ? launch(ctx, bias_grad_kernel<bf16>, dim3((cols + 255) / 256), dim3(256), a, "bias_grad_kernel<bf16>", bytes, 1)
+                        : launch(ctx, bias_grad_kernel<float>, dim3((cols + 255) / 256), dim3(256), a, "bias_grad_kernel<f32>", bytes, 1);
 }
 
 }  // namespace tch

@@ -15,6 +15,7 @@ struct ConvShape {
   int K;           // output channels
   int R, S;        // filter height / width
   int stride, pad;
+  int c_logical;  // input channels that carry data (<= C; the rest is zero padding); 0 = C
 };
 
 void conv_output_hw(const ConvShape& s, int* Ho, int* Wo);
@@ -58,6 +59,8 @@ int bias_grad(Context* ctx, int dtype, const void* dy, float* dbias, int rows, i
 
 // layout.hip
 int nchw_to_nhwc_pad(Context* ctx, int dtype, const float* x_nchw, void* y_nhwc, int N, int C, int H, int W, int Cpad);
+int filter_transpose_batched(Context* ctx, int dtype, const void* src, void* dst, const int64_t* table_dev,
+                             int n_filters, int64_t total_tiles, int64_t total_elems);
 int cast_f32(Context* ctx, int dtype, const float* src, void* dst, int64_t n);
 int cast_to_f32(Context* ctx, int dtype, const void* src, float* dst, int64_t n);
 

@@ -180,8 +180,10 @@ int maxpool_fwd(Context* ctx, int dtype, const void* x, void* y, int32_t* index,
   TCH_CHECK_ARG(a.Ho > 0 && a.Wo > 0, "maxpool_fwd: empty output");
   a.total = static_cast<int64_t>(N) * a.Ho * a.Wo * a.cc;
   dim3 grid(static_cast<unsigned>((a.total + 255) / 256));
-  return dtype == kBF16 ? launch(ctx, maxpool_fwd_kernel<bf16>, grid, dim3(256), a)
-                        : launch(ctx, maxpool_fwd_kernel<float>, grid, dim3(256), a);
+  const double eb = dtype == kBF16 ? 2.0 : 4.0;
+  const double bytes = static_cast<double>(N) * C * (H * W * eb + a.Ho * a.Wo * (eb + 4.0));
+  return dtype == kBF16 ? launch(ctx, maxpool_fwd_kernel<bf16>, grid, dim3(256), a, "maxpool_fwd_kernel<bf16>", bytes, 1)
+                        : launch(ctx, maxpool_fwd_kernel<float>, grid, dim3(256), a, "maxpool_fwd_kernel<f32>", bytes, 1);
 }
 
 int maxpool_bwd(Context* ctx, int dtype, const void* dy, const int32_t* index, void* dx, int N, int H, int W, int C,
@@ -193,8 +195,10 @@ int maxpool_bwd(Context* ctx, int dtype, const void* dy, const int32_t* index, v
                 (W + 2 * pad - ksize) / stride + 1, C / E, ksize, stride, pad, 0};
   a.total = static_cast<int64_t>(N) * H * W * a.cc;
   dim3 grid(static_cast<unsigned>((a.total + 255) / 256));
-  return dtype == kBF16 ? launch(ctx, maxpool_bwd_kernel<bf16>, grid, dim3(256), a)
-                        : launch(ctx, maxpool_bwd_kernel<float>, grid, dim3(256), a);
+  const double eb = dtype == kBF16 ? 2.0 : 4.0;
+  const double bytes = static_cast<double>(N) * C * (H * W * eb + a.Ho * a.Wo * (eb + 4.0));
+  return dtype == kBF16 ? launch(ctx, maxpool_bwd_kernel<bf16>, grid, dim3(256), a, "maxpool_bwd_kernel<bf16>", bytes, 1)
+                        : launch(ctx, maxpool_bwd_kernel<float>, grid, dim3(256), a, "maxpool_bwd_kernel<f32>", bytes, 1);
 }
 
 int avgpool_fwd(Context* ctx, int dtype, const void* x, void* y, int N, int HW, int C) {
@@ -203,8 +207,9 @@ int avgpool_fwd(Context* ctx, int dtype, const void* x, void* y, int N, int HW, 
   const int E = dtype == kBF16 ? 8 : 4;
   AvgPoolArgs a{x, y, N, HW, C / E, 1.0f / static_cast<float>(HW), static_cast<int64_t>(N) * (C / E)};
   dim3 grid(static_cast<unsigned>((a.total + 255) / 256));
-  return dtype == kBF16 ? launch(ctx, avgpool_fwd_kernel<bf16>, grid, dim3(256), a)
-                        : launch(ctx, avgpool_fwd_kernel<float>, grid, dim3(256), a);
+  const double bytes = static_cast<double>(N) * C * (HW + 1) * (dtype == kBF16 ? 2.0 : 4.0);
+  return dtype == kBF16 ? launch(ctx, avgpool_fwd_kernel<bf16>, grid, dim3(256), a, "avgpool_fwd_kernel<bf16>", bytes, 1)
+                        : launch(ctx, avgpool_fwd_kernel<float>, grid, dim3(256), a, "avgpool_fwd_kernel<f32>", bytes, 1);
 }
 
 int avgpool_bwd(Context* ctx, int dtype, const void* dy, void* dx, int N, int HW, int C) {
@@ -213,8 +218,9 @@ int avgpool_bwd(Context* ctx, int dtype, const void* dy, void* dx, int N, int HW
   const int E = dtype == kBF16 ? 8 : 4;
   AvgPoolArgs a{dy, dx, N, HW, C / E, 1.0f / static_cast<float>(HW), static_cast<int64_t>(N) * HW * (C / E)};
   dim3 grid(static_cast<unsigned>((a.total + 255) / 256));
-  return dtype == kBF16 ? launch(ctx, avgpool_bwd_kernel<bf16>, grid, dim3(256), a)
-                        : launch(ctx, avgpool_bwd_kernel<float>, grid, dim3(256), a);
+  const double bytes = static_cast<double>(N) * C * (HW + 1) * (dtype == kBF16 ? 2.0 : 4.0);
+  return dtype == kBF16 ? launch(ctx, avgpool_bwd_kernel<bf16>, grid, dim3(256), a, "avgpool_bwd_kernel<bf16>", bytes, 1)
+                        : launch(ctx, avgpool_bwd_kernel<float>, grid, dim3(256), a, "avgpool_bwd_kernel<f32>", bytes, 1);
 }
 
 }  // namespace tch

@@ -92,6 +92,18 @@ class Context:
     def take_rejected(self):
         return int(lib().tch_context_take_rejected(self.handle))
 
+    def profile(self, program, reps=1):
+        """Per-kernel HIP-event timing of `reps` replays: list of dicts with name, total_ms,
+        launches, work (algorithmic flops or bytes, summed) and work_is_bytes."""
+        from ._lib import KernelStat
+        cap = 256
+        buf = (KernelStat * cap)()
+        n = ctypes.c_int(0)
+        check(lib().tch_program_profile(self.handle, program.handle, reps, buf, cap, ctypes.byref(n)),
+              "tch_program_profile")
+        return [dict(name=buf[i].name.decode(), total_ms=buf[i].total_ms, launches=int(buf[i].launches),
+                     work=buf[i].work, work_is_bytes=bool(buf[i].work_is_bytes)) for i in range(n.value)]
+
 
 # ---------------------------------------------------------------------------
 # convolution
@@ -101,7 +113,7 @@ def conv_out_hw(H, W, R, S, stride, pad):
     return (H + 2 * pad - R) // stride + 1, (W + 2 * pad - S) // stride + 1
 
 
-def conv2d_fwd(ctx, x, w, y, stride, pad, add=None, mask=None, bias=None, tile_cfg=-1):
+def conv2d_fwd(ctx, x, w, y, stride, pad, add=None, mask=None, bias=None, tile_cfg=-1, c_logical=0):
     N, H, W, C = x.shape
     K, R, S, C2 = w.shape
     assert C == C2, "filter / input channel mismatch"
@@ -113,12 +125,14 @@ def conv2d_fwd(ctx, x, w, y, stride, pad, add=None, mask=None, bias=None, tile_c
         assert t is None or (t.shape == y.shape and t.dtype == x.dtype)
     assert bias is None or (bias.dtype == torch.float32 and bias.numel() == K)
     check(lib().tch_conv2d_fwd(ctx.handle, dtype_code(x), _p(x), _p(w), _p(y), _p(add), _p(mask), _p(bias), out_f32,
-                               N, H, W, C, K, R, S, stride, pad, tile_cfg), "tch_conv2d_fwd")
+                               N, H, W, C, K, R, S, stride, pad, tile_cfg, c_logical), "tch_conv2d_fwd")
 
 
-def conv2d_dgrad(ctx, dy, w, dx, stride, pad, add=None, mask=None, tile_cfg=-1):
+def conv2d_dgrad(ctx, dy, wt, dx, stride, pad, add=None, mask=None, tile_cfg=-1, c_logical=0):
+    """wt is the filter transposed to [C,R,S,K] (filter_transpose)."""
+    w = wt
     N, H, W, C = dx.shape
-    K, R, S, C2 = w.shape
+    C2, R, S, K = wt.shape
     assert C == C2
     Ho, Wo = conv_out_hw(H, W, R, S, stride, pad)
     assert tuple(dy.shape) == (N, Ho, Wo, K)
@@ -126,7 +140,7 @@ def conv2d_dgrad(ctx, dy, w, dx, stride, pad, add=None, mask=None, tile_cfg=-1):
     for t in (add, mask):
         assert t is None or (t.shape == dx.shape and t.dtype == dx.dtype)
     check(lib().tch_conv2d_dgrad(ctx.handle, dtype_code(dy), _p(dy), _p(w), _p(dx), _p(add), _p(mask),
-                                 N, H, W, C, K, R, S, stride, pad, tile_cfg), "tch_conv2d_dgrad")
+                                 N, H, W, C, K, R, S, stride, pad, tile_cfg, c_logical), "tch_conv2d_dgrad")
 
 
 def conv2d_wgrad_splits(x, K, R, S, stride, pad):
@@ -138,7 +152,7 @@ def conv2d_wgrad_workspace_bytes(dtype, K, R, S, C, splits):
     return int(lib().tch_conv2d_wgrad_workspace_bytes(dtype, K, R, S, C, splits))
 
 
-def conv2d_wgrad(ctx, x, dy, dw, stride, pad, workspace=None, splits=0, accumulate=False, tile_cfg=-1):
+def conv2d_wgrad(ctx, x, dy, dw, stride, pad, workspace=None, splits=0, accumulate=False, tile_cfg=-1, c_logical=0):
     N, H, W, C = x.shape
     K, R, S, C2 = dw.shape
     assert C == C2 and dw.dtype == torch.float32
@@ -150,7 +164,8 @@ def conv2d_wgrad(ctx, x, dy, dw, stride, pad, workspace=None, splits=0, accumula
         need = conv2d_wgrad_workspace_bytes(dtype_code(x), K, R, S, C, splits)
         assert workspace.numel() * workspace.element_size() >= need, "wgrad workspace too small"
     check(lib().tch_conv2d_wgrad(ctx.handle, dtype_code(x), _p(x), _p(dy), _p(dw), _p(workspace), splits,
-                                 int(accumulate), N, H, W, C, K, R, S, stride, pad, tile_cfg), "tch_conv2d_wgrad")
+                                 int(accumulate), N, H, W, C, K, R, S, stride, pad, tile_cfg, c_logical),
+          "tch_conv2d_wgrad")
 
 
 # ---------------------------------------------------------------------------
@@ -264,6 +279,37 @@ def nchw_to_nhwc_pad(ctx, x_nchw, y_nhwc):
     assert x_nchw.dtype == torch.float32 and tuple(y_nhwc.shape[:3]) == (N, H, W)
     check(lib().tch_nchw_to_nhwc_pad(ctx.handle, dtype_code(y_nhwc), _p(x_nchw), _p(y_nhwc), N, C, H, W,
                                      y_nhwc.shape[3]), "tch_nchw_to_nhwc_pad")
+
+
+class FilterTransposeTable:
+    """Device table for tch_filter_transpose_batched: filters [(element offset, K, RS, C), ...]
+    that sit at the same offsets inside a flat source and a flat destination buffer."""
+
+    def __init__(self, filters, device):
+        rows, tile = [], 0
+        self.total_elems = 0
+        for off, K, RS, C in filters:
+            rows.append([tile, off, K, RS, C])
+            tile += RS * ((K + 31) // 32) * ((C + 31) // 32)
+            self.total_elems += K * RS * C
+        self.total_tiles = tile
+        self.n = len(rows)
+        self.table = torch.tensor(rows, dtype=torch.int64).to(device)
+
+
+def filter_transpose_batched(ctx, src, dst, table):
+    """dst[C][RS][K] = src[K][RS][C] for every filter of the table (one launch)."""
+    assert src.dtype == dst.dtype and src.numel() == dst.numel()
+    check(lib().tch_filter_transpose_batched(ctx.handle, dtype_code(src), _p(src), _p(dst), _p(table.table), table.n,
+                                             table.total_tiles, table.total_elems), "tch_filter_transpose_batched")
+
+
+def filter_transpose(ctx, w):
+    """[K,R,S,C] -> [C,R,S,K] (the layout conv2d_dgrad reads)."""
+    K, R, S, C = w.shape
+    out = torch.empty((C, R, S, K), dtype=w.dtype, device=w.device)
+    filter_transpose_batched(ctx, w, out, FilterTransposeTable([(0, K, R * S, C)], w.device))
+    return out
 
 
 def cast_from_f32(ctx, src, dst):

@@ -99,6 +99,12 @@ class ResNetEngine:
         self.momentum_buf = torch.zeros(self.n_store, **f32)
         self.global_grads = None
         self.shadow = torch.zeros(self.n_store, dtype=torch.bfloat16, device=self.dev) if dtype == torch.bfloat16 else None
+        # filters transposed to [C,R,S,K] for the data-gradient GEMM, same offsets, rewritten
+        # in one launch whenever the weights change
+        self.wt = torch.zeros(self.n_store, dtype=dtype, device=self.dev)
+        self._tt = ops.FilterTransposeTable(
+            [(p.offset, p.store_shape[0], p.store_shape[1] * p.store_shape[2], p.store_shape[3])
+             for p in self._specs if p.kind in ("conv", "fc_w")], self.dev)
         nbn = sum(c for _, c in self._bn_names)
         self.running_mean = torch.zeros(nbn, **f32)
         self.running_var = torch.ones(nbn, **f32)
@@ -165,9 +171,46 @@ class ResNetEngine:
         self.refresh_shadow()
         torch.cuda.synchronize()
 
+    def init_kaiming(self, seed=0):
+        """Random initial weights generated on the GPU: convolutions N(0, 2/fan_out) (Kaiming
+        normal, fan_out, relu), BatchNorm gamma 1 / beta 0, fc U(-1/sqrt(fan_in), 1/sqrt(fan_in)).
+        Same distribution as the oracle's init, different stream of random numbers."""
+        g = torch.Generator(device=self.dev)
+        g.manual_seed(seed)
+        for p in self._specs:
+            v = self._view(self.params, p.name)
+            if p.kind == "conv":
+                K, R, S, C = p.store_shape
+                v.normal_(0.0, math.sqrt(2.0 / (K * R * S)), generator=g)
+                if p.shape[1] != C:
+                    v[..., p.shape[1]:] = 0
+            elif p.kind == "bn_w":
+                v.fill_(1.0)
+            elif p.kind == "bn_b":
+                v.zero_()
+            else:
+                bound = 1.0 / math.sqrt(self.feat)
+                v.uniform_(-bound, bound, generator=g)
+        self.running_mean.zero_()
+        self.running_var.fill_(1.0)
+        self.momentum_buf.zero_()
+        self.grads.zero_()
+        self.refresh_shadow()
+        torch.cuda.synchronize()
+
     def refresh_shadow(self):
         if self.shadow is not None:
             ops.cast_from_f32(self.ctx, self.params, self.shadow)
+        self._refresh_transposed()
+
+    def _refresh_transposed(self):
+        ops.filter_transpose_batched(self.ctx, self.shadow if self.shadow is not None else self.params, self.wt,
+                                     self._tt)
+
+    def _wt(self, name):
+        p = self.spec[name]
+        K, R, S, C = p.store_shape
+        return self.wt[p.offset:p.offset + p.numel].view(C, R, S, K)
 
     def state_dict(self):
         torch.cuda.synchronize()
@@ -276,13 +319,14 @@ class ResNetEngine:
                        self._view(self.grads, name + ".bias"), bn_ws, relu_mask=mask)
 
         def conv_fwd(c, x, y, **kw):
-            ops.conv2d_fwd(ctx, x, self._w(c.name + ".weight"), y, c.stride, c.pad, **kw)
+            ops.conv2d_fwd(ctx, x, self._w(c.name + ".weight"), y, c.stride, c.pad, c_logical=c.cin, **kw)
 
         def conv_wgrad(c, x, dy):
-            ops.conv2d_wgrad(ctx, x, dy, self._view(self.grads, c.name + ".weight"), c.stride, c.pad, workspace=wg_ws)
+            ops.conv2d_wgrad(ctx, x, dy, self._view(self.grads, c.name + ".weight"), c.stride, c.pad, workspace=wg_ws,
+                             c_logical=c.cin)
 
         def conv_dgrad(c, dy, dx, **kw):
-            ops.conv2d_dgrad(ctx, dy, self._w(c.name + ".weight"), dx, c.stride, c.pad, **kw)
+            ops.conv2d_dgrad(ctx, dy, self._wt(c.name + ".weight"), dx, c.stride, c.pad, c_logical=c.cin, **kw)
 
         prog = ops.Program()
         ctx.begin_record(prog)
@@ -332,7 +376,7 @@ class ResNetEngine:
                              self._view(self.grads, "fc.weight"), 1, 0, workspace=wg_ws)
             ops.bias_grad(ctx, dlogits, self._view(self.grads, "fc.bias"))
             g_pooled = galloc((B, self.feat))
-            ops.conv2d_dgrad(ctx, dlogits.view(B, 1, 1, self.num_classes), self._w("fc.weight"),
+            ops.conv2d_dgrad(ctx, dlogits.view(B, 1, 1, self.num_classes), self._wt("fc.weight"),
                              g_pooled.view(B, 1, 1, self.feat), 1, 0)
             g_out = galloc((B, Hl, Wl, self.feat))
             ops.avgpool_bwd(ctx, g_pooled, g_out)
@@ -445,11 +489,14 @@ class ResNetEngine:
                 def rec():
                     ops.sgd_momentum_step(self.ctx, self.params, self.global_grads, self.momentum_buf, self.lr,
                                           self.momentum, self.weight_decay, shadow=self.shadow)
+                    self._refresh_transposed()
                     ops.fill_zero(self.ctx, self.global_grads)
                 self._opt_global_prog = self._flat_prog(rec)
             return self.ctx.run(self._opt_global_prog)
         if self._opt_prog is None:
-            self._opt_prog = self._flat_prog(lambda: ops.sgd_momentum_step(
-                self.ctx, self.params, self.grads, self.momentum_buf, self.lr, self.momentum, self.weight_decay,
-                shadow=self.shadow))
+            def rec():
+                ops.sgd_momentum_step(self.ctx, self.params, self.grads, self.momentum_buf, self.lr, self.momentum,
+                                      self.weight_decay, shadow=self.shadow)
+                self._refresh_transposed()
+            self._opt_prog = self._flat_prog(rec)
         return self.ctx.run(self._opt_prog)

@@ -100,7 +100,7 @@ def test_conv_dgrad(ctx, dtype, case, tile_cfg):
     w = rnd((K, R, S, C), dtype, g, (R * S * K) ** -0.5)
     ref = O.conv2d_dgrad(dy, w, (N, H, W, C), st, pad)
     dx = torch.empty((N, H, W, C), dtype=dtype, device="cuda")
-    ops.conv2d_dgrad(ctx, dy.cuda(), w.cuda(), dx, st, pad, tile_cfg=tile_cfg)
+    ops.conv2d_dgrad(ctx, dy.cuda(), ops.filter_transpose(ctx, w.cuda()), dx, st, pad, tile_cfg=tile_cfg)
     torch.cuda.synchronize()
     close(dx, ref, dtype, "conv dgrad")
 
@@ -115,7 +115,7 @@ def test_conv_dgrad_residual(ctx, dtype):
     add, mask = rnd((N, H, W, C), dtype, g), rnd((N, H, W, C), dtype, g)
     ref = O.conv2d_dgrad(dy, w, (N, H, W, C), st, pad) + add.float() * (mask.float() > 0)
     dx = torch.empty((N, H, W, C), dtype=dtype, device="cuda")
-    ops.conv2d_dgrad(ctx, dy.cuda(), w.cuda(), dx, st, pad, add=add.cuda(), mask=mask.cuda())
+    ops.conv2d_dgrad(ctx, dy.cuda(), ops.filter_transpose(ctx, w.cuda()), dx, st, pad, add=add.cuda(), mask=mask.cuda())
     torch.cuda.synchronize()
     close(dx, ref, dtype, "conv dgrad + residual")
 
