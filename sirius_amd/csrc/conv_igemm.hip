@@ -7,18 +7,29 @@
 // torchvision's ResNet (train/resnet152.py:22) and the arithmetic is
 // F.conv2d / its autograd formulas.  These kernels restate that arithmetic:
 //   FWD    y[n,ho,wo,k]  = sum_{r,s,c} x[n, ho*st-p+r, wo*st-p+s, c] * w[k,r,s,c]
-//   DGRAD  dx[n,h,w,c]   = sum_{r,s,k} dy[n,(h+p-r)/st,(w+p-s)/st,k] * w[k,r,s,c]
+//   DGRAD  dx[n,h,w,c]   = sum_{r,s,k} dy[n,(h+p-r)/st,(w+p-s)/st,k] * wt[c,r,s,k]
 //   WGRAD  dw[k,r,s,c]   = sum_{n,ho,wo} dy[n,ho,wo,k] * x[n, ho*st-p+r, wo*st-p+s, c]
 //
 // GEMM view (rows x cols, reduction):
 //   FWD    (N*Ho*Wo) x K,        over R*S*C
-//   DGRAD  (N*H*W)   x C,        over R*S*K
+//   DGRAD  (N*H*W)   x C,        over R*S*K     (filter pre-transposed to [C][R][S][K])
 //   WGRAD  K         x (R*S*C),  over N*Ho*Wo, split across workgroups
 //
-// A tile row in LDS holds one GEMM row (or column) and BK reduction elements
-// = 4 chunks of 16 bytes (+1 chunk of padding).  A lane's MFMA operand is one
-// chunk: lanes 0-31 take chunk 2j, lanes 32-63 chunk 2j+1 of their row, so the
-// two operands always agree on which reduction elements a lane group holds.
+// FWD / DGRAD: a tile row in LDS holds one GEMM row (or column) and BK reduction
+// elements = 4 chunks of 16 bytes (+1 chunk of padding); a lane's MFMA operand is
+// one chunk (lanes 0-31 chunk 2j, lanes 32-63 chunk 2j+1 of their row).
+//
+// WGRAD: both operands are contiguous along the GEMM row/column (channels) and
+// strided along the reduction (pixels), the opposite of what an MFMA operand
+// wants.  The tiles are kept as they come, [pixel][channel], and the operand is
+// formed by the LDS transpose read of gfx950 (ds_read_b64_tr_b16): a group of 16
+// lanes reads a 4-pixel x 16-channel block and every lane receives the 4 pixels
+// of ONE channel.
+//
+// The MFMA is issued with the filter-side fragment as the first operand, so a
+// lane's 16 accumulators belong to ONE output row and to groups of 4 consecutive
+// output columns: the epilogue moves them through LDS as 16-byte vectors and
+// writes (and reads the residual / mask) as full 16-byte chunks per lane.
 #include "kernels.h"
 #include "ops.h"
 
@@ -27,13 +38,15 @@
 namespace tch {
 namespace {
 
-constexpr int kLdsStride = 5;  // chunks per LDS tile row: 4 data + 1 pad
+constexpr int kLdsStride = 5;  // FWD/DGRAD: chunks per LDS tile row: 4 data + 1 pad
+constexpr int kRowPad = 4;     // WGRAD: chunks of padding per [pixel] row (64 bytes)
+constexpr int kStagePad = 4;   // epilogue staging: floats of padding per row
 
 enum Mode : int { kFwd = 0, kDgrad = 1, kWgrad = 2 };
 
 struct IgemmArgs {
   const void* a_src;  // FWD: x        DGRAD: dy       WGRAD: dy
-  const void* b_src;  // FWD: w        DGRAD: w        WGRAD: x
+  const void* b_src;  // FWD: w        DGRAD: wt       WGRAD: x
   void* out;          // FWD: y        DGRAD: dx       WGRAD: dw (fp32) or split partials
   const void* add;    // optional addend, laid out like out (FWD/DGRAD)
   const void* mask;   // optional: addend counts only where mask > 0
@@ -51,16 +64,25 @@ struct IgemmArgs {
   FastDiv div_width;  // row width on the gather side
 };
 
+typedef short short4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) short4_t* lds_short4_ptr;
+union TrPart {
+  short4_t s;
+  uint32_t w[2];
+};
+
+// first operand = filter-side fragment (its rows become accumulator registers),
+// second operand = activation-side fragment (its rows become accumulator lanes)
 template <typename T>
-__device__ inline void mma(const Chunk& a, const Chunk& b, f32x16_t& acc);
+__device__ inline void mma(const Chunk& first, const Chunk& second, f32x16_t& acc);
 template <>
-__device__ inline void mma<bf16>(const Chunk& a, const Chunk& b, f32x16_t& acc) {
-  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.h, b.h, acc, 0, 0, 0);
+__device__ inline void mma<bf16>(const Chunk& first, const Chunk& second, f32x16_t& acc) {
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(first.h, second.h, acc, 0, 0, 0);
 }
 template <>
-__device__ inline void mma<float>(const Chunk& a, const Chunk& b, f32x16_t& acc) {
+__device__ inline void mma<float>(const Chunk& first, const Chunk& second, f32x16_t& acc) {
 #pragma unroll
-  for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.f[e], b.f[e], acc, 0, 0, 0);
+  for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(first.f[e], second.f[e], acc, 0, 0, 0);
 }
 
 __device__ inline Chunk load_chunk(const void* base, int64_t elem_off, int elem_bytes, bool valid) {
@@ -69,47 +91,84 @@ __device__ inline Chunk load_chunk(const void* base, int64_t elem_off, int elem_
   return c;
 }
 
-// v[j] holds E consecutive elements of memory row j; produce out[e] = the e-th
-// element of every row, i.e. the ExE transpose.
-template <typename T>
-__device__ inline void transpose_block(const Chunk* v, Chunk* out);
-template <>
-__device__ inline void transpose_block<float>(const Chunk* v, Chunk* out) {
-#pragma unroll
-  for (int e = 0; e < 4; ++e)
-#pragma unroll
-    for (int q = 0; q < 4; ++q) out[e].w[q] = v[q].w[e];
-}
-template <>
-__device__ inline void transpose_block<bf16>(const Chunk* v, Chunk* out) {
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const int src = e >> 1;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      uint32_t lo = v[2 * q].w[src], hi = v[2 * q + 1].w[src];
-      out[e].w[q] = (e & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
-    }
-  }
-}
-
-// Walks the reduction index of a filter-tap-major operand: (tap, channel) with
-// `channels` per tap, advancing by BK per step.
+// Walks the reduction index of a filter-tap-major operand: (r, s, channel) with
+// `channels` per tap, advancing by a fixed step; no division after init.
 struct TapWalker {
-  int tap, ch;
-  __device__ inline void init(int k, int channels) {
-    tap = k / channels;
+  int r, s, ch;
+  __device__ inline void init(int k, int channels, int S) {
+    int tap = k / channels;
     ch = k - tap * channels;
+    r = tap / S;
+    s = tap - r * S;
   }
-  __device__ inline void advance(int step, int channels) {
+  __device__ inline void advance(int step, int channels, int S) {
     ch += step;
     while (ch >= channels) {
       ch -= channels;
-      ++tap;
+      if (++s == S) {
+        s = 0;
+        ++r;
+      }
     }
   }
 };
 
+// The accumulators of one workgroup tile, one 32-row band (index tm) at a time:
+// lanes write float4 groups into the staging tile [WM*32][BN + pad], then every
+// thread takes E consecutive columns of one row and hands them to `fin`.
+template <typename T, int WM, int WN, int TM, int TN, typename Fin>
+__device__ inline void staged_epilogue(f32x16_t (&acc)[TM][TN], float* stage, int tid, Fin fin) {
+  constexpr int E = Elem<T>::kPerChunk;
+  constexpr int BN = WN * TN * 32;
+  constexpr int NT = WM * WN * 64;
+  constexpr int LD = BN + kStagePad;
+  constexpr int CH = BN / E;
+  constexpr int ITERS = (WM * 32 * CH) / NT;
+  static_assert((WM * 32 * CH) % NT == 0, "epilogue mapping");
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm) {
+    __syncthreads();
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int r = wm * 32 + (lane & 31);
+        const int c = (wn * TN + tn) * 32 + 8 * j + 4 * (lane >> 5);
+        float4 v = make_float4(acc[tm][tn][4 * j], acc[tm][tn][4 * j + 1], acc[tm][tn][4 * j + 2],
+                               acc[tm][tn][4 * j + 3]);
+        *reinterpret_cast<float4*>(stage + r * LD + c) = v;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int q = tid + it * NT;
+      const int r = q / CH, cc = q - r * CH;
+      float v[E];
+#pragma unroll
+      for (int e = 0; e < E; e += 4) {
+        float4 t = *reinterpret_cast<const float4*>(stage + r * LD + cc * E + e);
+        v[e] = t.x;
+        v[e + 1] = t.y;
+        v[e + 2] = t.z;
+        v[e + 3] = t.w;
+      }
+      fin(((r >> 5) * TM + tm) * 32 + (r & 31), cc * E, v);
+    }
+  }
+}
+
+template <int E>
+__device__ inline void store_floats(float* dst, const float* v) {
+#pragma unroll
+  for (int e = 0; e < E; e += 4) *reinterpret_cast<float4*>(dst + e) = make_float4(v[e], v[e + 1], v[e + 2], v[e + 3]);
+}
+
+// ---------------------------------------------------------------------------
+// forward / data gradient
+// ---------------------------------------------------------------------------
 template <typename T, int MODE, int WM, int WN, int TM, int TN>
 __global__ __launch_bounds__(WM* WN * 64) void igemm_kernel(IgemmArgs p) {
   constexpr int E = Elem<T>::kPerChunk;
@@ -118,70 +177,51 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm_kernel(IgemmArgs p) {
   constexpr int BN = WN * TN * 32;
   constexpr int NT = WM * WN * 64;
   constexpr int EB = sizeof(T);
-  // direct loaders: one chunk per (row, chunk-in-row)
-  constexpr int A_PT = (BM * 4 + NT - 1) / NT;
-  constexpr int B_PT = (BN * 4 + NT - 1) / NT;
-  static_assert((BM * 4) % NT == 0 || BM * 4 < NT, "tile/loader mismatch");
-  static_assert((BN * 4) % NT == 0 || BN * 4 < NT, "tile/loader mismatch");
-  // transposing loaders: one ExE block per active thread
-  constexpr int A_BLOCKS = (BM / E) * 4;
-  constexpr int B_BLOCKS = (BN / E) * 4;
-  static_assert(A_BLOCKS <= NT && B_BLOCKS <= NT, "transposing loader needs one block per thread");
+  constexpr int A_PT = (BM * 4) / NT;
+  constexpr int B_PT = (BN * 4) / NT;
+  static_assert((BM * 4) % NT == 0 && (BN * 4) % NT == 0, "tile/loader mismatch");
+  constexpr int OPER_BYTES = (BM + BN) * kLdsStride * 16 * 2;
+  constexpr int STAGE_BYTES = WM * 32 * (BN + kStagePad) * 4;
+  constexpr int LDS_BYTES = OPER_BYTES > STAGE_BYTES ? OPER_BYTES : STAGE_BYTES;
 
-  __shared__ uint4 lds_a[2][BM * kLdsStride];
-  __shared__ uint4 lds_b[2][BN * kLdsStride];
+  __shared__ uint4 lds[LDS_BYTES / 16];
+  uint4* lds_a = lds;                            // [2][BM * kLdsStride]
+  uint4* lds_b = lds + 2 * BM * kLdsStride;      // [2][BN * kLdsStride]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
 
-  const uint32_t nwg = gridDim.x;
-  uint32_t id = xcd_remap(blockIdx.x, nwg);
-  const int tiles_mn = p.tiles_m * p.tiles_n;
-  const int split = id / tiles_mn;
-  id -= split * tiles_mn;
+  uint32_t id = xcd_remap(blockIdx.x, gridDim.x);
   const int tile_m = id / p.tiles_n;
   const int tile_n = id - tile_m * p.tiles_n;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int k_end = p.gemm_k;
+  const int nk = (k_end + BK - 1) / BK;
 
-  const int k_begin = split * p.k_per_split;
-  int k_end = k_begin + p.k_per_split;
-  if (k_end > p.gemm_k) k_end = p.gemm_k;
-  const int nk = (k_end - k_begin + BK - 1) / BK;
-
-  const int RS = p.R * p.S;
-
-  // ---------------- per-thread loader state ----------------
-  // FWD / DGRAD operand A: gather of activation rows
+  // ---- operand A: gather of activation rows; the chunk column is the same for every i ----
+  const int in_h = (MODE == kFwd) ? p.H : p.Ho;
+  const int in_w = (MODE == kFwd) ? p.W : p.Wo;
+  const int in_c = (MODE == kFwd) ? p.C : p.K;
+  const int chunk_col = tid & 3;
   int a_base[A_PT], a_h0[A_PT], a_w0[A_PT];
   bool a_row_ok[A_PT];
-  TapWalker a_walk;  // same chunk column for every i, so one walker
-  int in_h = 0, in_w = 0, in_c = 0;
-  // FWD operand B: dense filter rows
-  // DGRAD operand B / WGRAD operands: transposing loaders
-  int t_row0_a = 0, t_kc_a = 0;
-  int t_row0_b = 0, t_kc_b = 0;
-  bool t_act_a = false, t_act_b = false;
-  TapWalker b_walk;
-  int wb_r = 0, wb_s = 0, wb_c = 0;  // WGRAD B: this thread's filter tap / channel
-
-  if constexpr (MODE == kFwd || MODE == kDgrad) {
-    in_h = (MODE == kFwd) ? p.H : p.Ho;
-    in_w = (MODE == kFwd) ? p.W : p.Wo;
-    in_c = (MODE == kFwd) ? p.C : p.K;
-    const int chunk_col = tid & 3;
-    a_walk.init(k_begin + chunk_col * E, in_c);
+  TapWalker walk;
+  walk.init(chunk_col * E, in_c, p.S);
 #pragma unroll
-    for (int i = 0; i < A_PT; ++i) {
-      int q = tid + i * NT;
-      int row = m0 + (q >> 2);
-      a_row_ok[i] = (q < BM * 4) && row < p.gemm_m;
-      uint32_t img = 0, pix = 0, oh = 0, ow = 0;
-      if (a_row_ok[i]) {
-        p.div_plane.divmod(static_cast<uint32_t>(row), img, pix);
-        p.div_width.divmod(pix, oh, ow);
-      }
+  for (int i = 0; i < A_PT; ++i) {
+    const int row = m0 + ((tid + i * NT) >> 2);
+    a_row_ok[i] = row < p.gemm_m;
+    uint32_t img = 0, pix = 0, oh = 0, ow = 0;
+    if (a_row_ok[i]) {
+      p.div_plane.divmod(static_cast<uint32_t>(row), img, pix);
+      p.div_width.divmod(pix, oh, ow);
+    }
+    if (p.pointwise) {
+      a_base[i] = row * in_c;  // dense [gemm_m][in_c]
+      a_h0[i] = a_w0[i] = 0;
+    } else {
       a_base[i] = static_cast<int>(img) * in_h * in_w * in_c;
       if (MODE == kFwd) {
         a_h0[i] = static_cast<int>(oh) * p.stride - p.pad;
@@ -192,140 +232,59 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm_kernel(IgemmArgs p) {
       }
     }
   }
-  if constexpr (MODE == kWgrad) {
-    t_act_a = tid < A_BLOCKS;
-    t_kc_a = tid & 3;
-    t_row0_a = m0 + (tid >> 2) * E;
-    t_act_b = tid < B_BLOCKS;
-    t_kc_b = tid & 3;
-    t_row0_b = n0 + (tid >> 2) * E;
-    if (t_act_b && t_row0_b < p.gemm_n) {
-      int tap = t_row0_b / p.C;
-      wb_c = t_row0_b - tap * p.C;
-      wb_r = tap / p.S;
-      wb_s = tap - wb_r * p.S;
-    }
-  }
 
-  Chunk ra[(MODE == kWgrad) ? E : A_PT];
-  Chunk rb[(MODE == kWgrad) ? E : B_PT];
+  Chunk ra[A_PT], rb[B_PT];
 
   auto load_tiles = [&](int kt) {
-    const int k0 = k_begin + kt * BK;
-    // ---- operand A ----
-    if constexpr (MODE == kFwd || MODE == kDgrad) {
-      const int r = a_walk.tap / p.S, s = a_walk.tap - r * p.S;
-      const bool tap_ok = a_walk.tap < RS && (k0 + (tid & 3) * E) < k_end;
+    const int k0 = kt * BK;
+    const int kk = k0 + chunk_col * E;
+    if (p.pointwise) {
+      const bool k_ok = kk < k_end;
+#pragma unroll
+      for (int i = 0; i < A_PT; ++i)
+        ra[i] = load_chunk(p.a_src, static_cast<int64_t>(a_base[i]) + kk, EB, a_row_ok[i] && k_ok);
+    } else {
+      const bool tap_ok = walk.r < p.R && kk < k_end;
 #pragma unroll
       for (int i = 0; i < A_PT; ++i) {
         int hi, wi;
         bool ok = a_row_ok[i] && tap_ok;
         if (MODE == kFwd) {
-          hi = a_h0[i] + r;
-          wi = a_w0[i] + s;
+          hi = a_h0[i] + walk.r;
+          wi = a_w0[i] + walk.s;
         } else {
-          int th = a_h0[i] - r, tw = a_w0[i] - s;
-          int sm = p.stride - 1;
+          const int th = a_h0[i] - walk.r, tw = a_w0[i] - walk.s;
+          const int sm = p.stride - 1;
           ok = ok && th >= 0 && tw >= 0 && ((th & sm) == 0) && ((tw & sm) == 0);
           hi = th >> p.stride_log2;
           wi = tw >> p.stride_log2;
         }
         ok = ok && static_cast<unsigned>(hi) < static_cast<unsigned>(in_h) &&
              static_cast<unsigned>(wi) < static_cast<unsigned>(in_w);
-        int64_t off = static_cast<int64_t>(a_base[i]) + (hi * in_w + wi) * in_c + a_walk.ch;
+        const int64_t off = static_cast<int64_t>(a_base[i]) + (hi * in_w + wi) * in_c + walk.ch;
         ra[i] = load_chunk(p.a_src, off, EB, ok);
       }
-      a_walk.advance(BK, in_c);
-    } else {
-      // WGRAD A: rows = output channels (contiguous in dy), reduction = pixels
-      const int pix0 = k0 + t_kc_a * E;
-      const bool ok_rows = t_act_a && t_row0_a < p.gemm_m;
-#pragma unroll
-      for (int j = 0; j < E; ++j) {
-        int pix = pix0 + j;
-        bool ok = ok_rows && pix < k_end;
-        ra[j] = load_chunk(p.a_src, static_cast<int64_t>(pix) * p.K + t_row0_a, EB, ok);
-      }
+      walk.advance(BK, in_c, p.S);
     }
-    // ---- operand B ----
-    if constexpr (MODE == kFwd || MODE == kDgrad) {
-      // dense filter rows: FWD reads w[K][R*S*C], DGRAD reads the transposed filter wt[C][R*S*K]
+    // operand B: dense filter rows: FWD reads w[K][R*S*C], DGRAD reads wt[C][R*S*K]
 #pragma unroll
-      for (int i = 0; i < B_PT; ++i) {
-        int q = tid + i * NT;
-        int row = n0 + (q >> 2);
-        int k = k0 + (q & 3) * E;
-        bool ok = (q < BN * 4) && row < p.gemm_n && k < k_end;
-        rb[i] = load_chunk(p.b_src, static_cast<int64_t>(row) * p.gemm_k + k, EB, ok);
-      }
-    } else {
-      // WGRAD B: rows = (tap, in channel) fixed per thread, reduction = pixels
-      const int pix0 = k0 + t_kc_b * E;
-      const bool ok_rows = t_act_b && t_row0_b < p.gemm_n;
-      if (p.pointwise) {
-#pragma unroll
-        for (int j = 0; j < E; ++j) {
-          int pix = pix0 + j;
-          bool ok = ok_rows && pix < k_end;
-          rb[j] = load_chunk(p.b_src, static_cast<int64_t>(pix) * p.C + wb_c, EB, ok);
-        }
-      } else {
-        uint32_t img = 0, rem = 0, oh = 0, ow = 0;
-        if (pix0 < k_end) {
-          p.div_plane.divmod(static_cast<uint32_t>(pix0), img, rem);
-          p.div_width.divmod(rem, oh, ow);
-        }
-        int n = img, ho = oh, wo = ow;
-#pragma unroll
-        for (int j = 0; j < E; ++j) {
-          int hi = ho * p.stride - p.pad + wb_r;
-          int wi = wo * p.stride - p.pad + wb_s;
-          bool ok = ok_rows && (pix0 + j) < k_end && static_cast<unsigned>(hi) < static_cast<unsigned>(p.H) &&
-                    static_cast<unsigned>(wi) < static_cast<unsigned>(p.W);
-          int64_t off = (static_cast<int64_t>(n) * p.H * p.W + hi * p.W + wi) * p.C + wb_c;
-          rb[j] = load_chunk(p.b_src, off, EB, ok);
-          if (++wo == p.Wo) {
-            wo = 0;
-            if (++ho == p.Ho) {
-              ho = 0;
-              ++n;
-            }
-          }
-        }
-      }
+    for (int i = 0; i < B_PT; ++i) {
+      const int row = n0 + ((tid + i * NT) >> 2);
+      const bool ok = row < p.gemm_n && kk < k_end;
+      rb[i] = load_chunk(p.b_src, static_cast<int64_t>(row) * p.gemm_k + kk, EB, ok);
     }
   };
 
   auto store_tiles = [&](int buf) {
-    if constexpr (MODE == kFwd || MODE == kDgrad) {
 #pragma unroll
-      for (int i = 0; i < A_PT; ++i) {
-        int q = tid + i * NT;
-        if (q < BM * 4) lds_a[buf][(q >> 2) * kLdsStride + (q & 3)] = ra[i].u;
-      }
-    } else {
-      if (t_act_a) {
-        Chunk t[E];
-        transpose_block<T>(ra, t);
-        int row = (tid >> 2) * E;
-#pragma unroll
-        for (int e = 0; e < E; ++e) lds_a[buf][(row + e) * kLdsStride + t_kc_a] = t[e].u;
-      }
+    for (int i = 0; i < A_PT; ++i) {
+      const int q = tid + i * NT;
+      lds_a[buf * BM * kLdsStride + (q >> 2) * kLdsStride + (q & 3)] = ra[i].u;
     }
-    if constexpr (MODE == kFwd || MODE == kDgrad) {
 #pragma unroll
-      for (int i = 0; i < B_PT; ++i) {
-        int q = tid + i * NT;
-        if (q < BN * 4) lds_b[buf][(q >> 2) * kLdsStride + (q & 3)] = rb[i].u;
-      }
-    } else {
-      if (t_act_b) {
-        Chunk t[E];
-        transpose_block<T>(rb, t);
-        int row = (tid >> 2) * E;
-#pragma unroll
-        for (int e = 0; e < E; ++e) lds_b[buf][(row + e) * kLdsStride + t_kc_b] = t[e].u;
-      }
+    for (int i = 0; i < B_PT; ++i) {
+      const int q = tid + i * NT;
+      lds_b[buf * BN * kLdsStride + (q >> 2) * kLdsStride + (q & 3)] = rb[i].u;
     }
   };
 
@@ -349,63 +308,246 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm_kernel(IgemmArgs p) {
     const int buf = kt & 1;
     const bool more = (kt + 1) < nk;
     if (more) load_tiles(kt + 1);
+    const uint4* la = lds_a + buf * BM * kLdsStride;
+    const uint4* lb = lds_b + buf * BN * kLdsStride;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       Chunk fa[TM], fb[TN];
 #pragma unroll
-      for (int tm = 0; tm < TM; ++tm)
-        fa[tm].u = lds_a[buf][((wm * TM + tm) * 32 + frag_row) * kLdsStride + 2 * j + frag_half];
+      for (int tm = 0; tm < TM; ++tm) fa[tm].u = la[((wm * TM + tm) * 32 + frag_row) * kLdsStride + 2 * j + frag_half];
 #pragma unroll
-      for (int tn = 0; tn < TN; ++tn)
-        fb[tn].u = lds_b[buf][((wn * TN + tn) * 32 + frag_row) * kLdsStride + 2 * j + frag_half];
+      for (int tn = 0; tn < TN; ++tn) fb[tn].u = lb[((wn * TN + tn) * 32 + frag_row) * kLdsStride + 2 * j + frag_half];
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
-        for (int tn = 0; tn < TN; ++tn) mma<T>(fa[tm], fb[tn], acc[tm][tn]);
+        for (int tn = 0; tn < TN; ++tn) mma<T>(fb[tn], fa[tm], acc[tm][tn]);
     }
     if (more) store_tiles(buf ^ 1);
     __syncthreads();
   }
 
-  // ---------------- epilogue ----------------
-  // 32x32 accumulator: lane owns column (lane % 32); element i sits in row
-  // 8*(i/4) + 4*(lane/32) + i%4.
+  // ---- epilogue: bias, gated residual, rounding; 16-byte accesses per lane ----
+  staged_epilogue<T, WM, WN, TM, TN>(acc, reinterpret_cast<float*>(lds), tid, [&](int tr, int tc, float* v) {
+    const int row = m0 + tr, col = n0 + tc;
+    if (row >= p.gemm_m || col >= p.gemm_n) return;
+    const int64_t idx = static_cast<int64_t>(row) * p.gemm_n + col;
+    if (MODE == kFwd && p.bias) {
 #pragma unroll
-  for (int tm = 0; tm < TM; ++tm) {
+      for (int e = 0; e < E; ++e) v[e] += p.bias[col + e];
+    }
+    if (p.add) {
+      Chunk ca;
+      ca.u = *reinterpret_cast<const uint4*>(static_cast<const T*>(p.add) + idx);
+      float a[E];
+      chunk_to_float<T>(ca, a);
+      if (p.mask) {
+        Chunk cm;
+        cm.u = *reinterpret_cast<const uint4*>(static_cast<const T*>(p.mask) + idx);
+        float m[E];
+        chunk_to_float<T>(cm, m);
 #pragma unroll
-    for (int tn = 0; tn < TN; ++tn) {
-      const int col = n0 + (wn * TN + tn) * 32 + frag_row;
-      if (col >= p.gemm_n) continue;
-      float bias = 0.f;
-      if (MODE == kFwd && p.bias) bias = p.bias[col];
+        for (int e = 0; e < E; ++e)
+          if (!(m[e] > 0.f)) a[e] = 0.f;
+      }
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int row = m0 + (wm * TM + tm) * 32 + 8 * (i >> 2) + 4 * frag_half + (i & 3);
-        if (row >= p.gemm_m) continue;
-        const int64_t idx = static_cast<int64_t>(row) * p.gemm_n + col;
-        float v = acc[tm][tn][i];
-        if constexpr (MODE == kWgrad) {
-          float* o = static_cast<float*>(p.out);
-          if (p.splits > 1) {
-            o[static_cast<int64_t>(split) * p.gemm_m * p.gemm_n + idx] = v;
-          } else {
-            o[idx] = p.accumulate ? o[idx] + v : v;
-          }
-        } else {
-          v += bias;
-          if (p.add) {
-            float a = Elem<T>::load(static_cast<const T*>(p.add) + idx);
-            if (p.mask && !(Elem<T>::load(static_cast<const T*>(p.mask) + idx) > 0.f)) a = 0.f;
-            v += a;
-          }
-          if (p.out_f32)
-            static_cast<float*>(p.out)[idx] = v;
-          else
-            Elem<T>::store(static_cast<T*>(p.out) + idx, v);
+      for (int e = 0; e < E; ++e) v[e] += a[e];
+    }
+    if (p.out_f32)
+      store_floats<E>(static_cast<float*>(p.out) + idx, v);
+    else
+      *reinterpret_cast<uint4*>(static_cast<T*>(p.out) + idx) = float_to_chunk<T>(v).u;
+  });
+}
+
+// ---------------------------------------------------------------------------
+// weight gradient
+// ---------------------------------------------------------------------------
+template <typename T, int WM, int WN, int TM, int TN>
+__global__ __launch_bounds__(WM* WN * 64) void wgrad_kernel(IgemmArgs p) {
+  constexpr int E = Elem<T>::kPerChunk;
+  constexpr int BKP = 4 * E;  // pixels per reduction step
+  constexpr int BM = WM * TM * 32;
+  constexpr int BN = WN * TN * 32;
+  constexpr int NT = WM * WN * 64;
+  constexpr int EB = sizeof(T);
+  constexpr int CA = BM / E, CB = BN / E;        // data chunks per [pixel] row
+  constexpr int LDA = CA + kRowPad, LDB = CB + kRowPad;  // row stride in chunks
+  constexpr int A_PT = (BKP * CA) / NT;
+  constexpr int B_PT = (BKP * CB) / NT;
+  static_assert((BKP * CA) % NT == 0 && (BKP * CB) % NT == 0, "tile/loader mismatch");
+  static_assert(NT % CA == 0 && NT % CB == 0, "a thread keeps one chunk column");
+  constexpr int OPER_BYTES = 2 * BKP * (LDA + LDB) * 16;
+  constexpr int STAGE_BYTES = WM * 32 * (BN + kStagePad) * 4;
+  constexpr int LDS_BYTES = OPER_BYTES > STAGE_BYTES ? OPER_BYTES : STAGE_BYTES;
+
+  __shared__ uint4 lds[LDS_BYTES / 16];
+  uint4* lds_a = lds;                      // [2][BKP][LDA]
+  uint4* lds_b = lds + 2 * BKP * LDA;      // [2][BKP][LDB]
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+
+  uint32_t id = xcd_remap(blockIdx.x, gridDim.x);
+  const int tiles_mn = p.tiles_m * p.tiles_n;
+  const int split = id / tiles_mn;
+  id -= split * tiles_mn;
+  const int tile_m = id / p.tiles_n;
+  const int tile_n = id - tile_m * p.tiles_n;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int k_begin = split * p.k_per_split;
+  int k_end = k_begin + p.k_per_split;
+  if (k_end > p.gemm_k) k_end = p.gemm_k;
+  const int nk = (k_end - k_begin + BKP - 1) / BKP;
+
+  // operand A = dy[pixel][K]: this thread's channel chunk and first pixel row
+  const int a_cc = tid % CA, a_prow = tid / CA;
+  const int a_ch = m0 + a_cc * E;
+  const bool a_ch_ok = a_ch < p.gemm_m;
+  // operand B = x gathered: column n = (tap, channel) is fixed per thread
+  const int b_cc = tid % CB, b_prow = tid / CB;
+  const int b_n = n0 + b_cc * E;
+  const bool b_n_ok = b_n < p.gemm_n;
+  int b_r = 0, b_s = 0, b_c = 0;
+  if (b_n_ok) {
+    const int tap = b_n / p.C;
+    b_c = b_n - tap * p.C;
+    b_r = tap / p.S;
+    b_s = tap - b_r * p.S;
+  }
+
+  Chunk ra[A_PT], rb[B_PT];
+
+  auto load_tiles = [&](int kt) {
+    const int k0 = k_begin + kt * BKP;
+#pragma unroll
+    for (int i = 0; i < A_PT; ++i) {
+      const int pix = k0 + a_prow + i * (NT / CA);
+      ra[i] = load_chunk(p.a_src, static_cast<int64_t>(pix) * p.K + a_ch, EB, a_ch_ok && pix < k_end);
+    }
+#pragma unroll
+    for (int i = 0; i < B_PT; ++i) {
+      const int pix = k0 + b_prow + i * (NT / CB);
+      bool ok = b_n_ok && pix < k_end;
+      int64_t off;
+      if (p.pointwise) {
+        off = static_cast<int64_t>(pix) * p.C + b_c;
+      } else {
+        uint32_t img = 0, rem = 0, oh = 0, ow = 0;
+        if (ok) {
+          p.div_plane.divmod(static_cast<uint32_t>(pix), img, rem);
+          p.div_width.divmod(rem, oh, ow);
         }
+        const int hi = static_cast<int>(oh) * p.stride - p.pad + b_r;
+        const int wi = static_cast<int>(ow) * p.stride - p.pad + b_s;
+        ok = ok && static_cast<unsigned>(hi) < static_cast<unsigned>(p.H) &&
+             static_cast<unsigned>(wi) < static_cast<unsigned>(p.W);
+        off = (static_cast<int64_t>(img) * p.H * p.W + hi * p.W + wi) * p.C + b_c;
+      }
+      rb[i] = load_chunk(p.b_src, off, EB, ok);
+    }
+  };
+
+  auto store_tiles = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < A_PT; ++i) lds_a[(buf * BKP + a_prow + i * (NT / CA)) * LDA + a_cc] = ra[i].u;
+#pragma unroll
+    for (int i = 0; i < B_PT; ++i) lds_b[(buf * BKP + b_prow + i * (NT / CB)) * LDB + b_cc] = rb[i].u;
+  };
+
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  if (nk > 0) {
+    load_tiles(0);
+    store_tiles(0);
+  }
+  __syncthreads();
+
+  // transpose-read geometry (bf16): lane = 16*G + q; the 16 lanes of a group read
+  // pixels {base + q/4 ...} x channels {16*(G%2) + 4*(q%4) ...}; after the transpose
+  // lane q owns channel 16*(G%2) + q of the band and 4 pixels.
+  const int grp = lane >> 4, q16 = lane & 15;
+  const int tr_pix = 8 * (grp >> 1) + (q16 >> 2);
+  const int tr_ch = 16 * (grp & 1) + 4 * (q16 & 3);
+
+  for (int kt = 0; kt < nk; ++kt) {
+    const int buf = kt & 1;
+    const bool more = (kt + 1) < nk;
+    if (more) load_tiles(kt + 1);
+    if constexpr (sizeof(T) == 2) {
+      const uint16_t* la = reinterpret_cast<const uint16_t*>(lds_a + buf * BKP * LDA);
+      const uint16_t* lb = reinterpret_cast<const uint16_t*>(lds_b + buf * BKP * LDB);
+#pragma unroll
+      for (int ks = 0; ks < BKP / 16; ++ks) {
+        Chunk fa[TM], fb[TN];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          const int prow = ks * 16 + tr_pix + 4 * t;
+#pragma unroll
+          for (int tm = 0; tm < TM; ++tm) {
+            const uint16_t* ptr = la + prow * (LDA * 8) + (wm * TM + tm) * 32 + tr_ch;
+            TrPart v;
+            v.s = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)(ptr));
+            fa[tm].w[2 * t] = v.w[0];
+            fa[tm].w[2 * t + 1] = v.w[1];
+          }
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn) {
+            const uint16_t* ptr = lb + prow * (LDB * 8) + (wn * TN + tn) * 32 + tr_ch;
+            TrPart v;
+            v.s = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)(ptr));
+            fb[tn].w[2 * t] = v.w[0];
+            fb[tn].w[2 * t + 1] = v.w[1];
+          }
+        }
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn) mma<T>(fb[tn], fa[tm], acc[tm][tn]);
+      }
+    } else {
+      // fp32: one reduction element per lane and MFMA, no transposition needed
+      const float* la = reinterpret_cast<const float*>(lds_a + buf * BKP * LDA);
+      const float* lb = reinterpret_cast<const float*>(lds_b + buf * BKP * LDB);
+#pragma unroll
+      for (int ks = 0; ks < BKP / 2; ++ks) {
+        const int prow = ks * 2 + (lane >> 5);
+        float fa[TM], fb[TN];
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) fa[tm] = la[prow * (LDA * 4) + (wm * TM + tm) * 32 + (lane & 31)];
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn) fb[tn] = lb[prow * (LDB * 4) + (wn * TN + tn) * 32 + (lane & 31)];
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+          for (int tn = 0; tn < TN; ++tn)
+            acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[tn], fa[tm], acc[tm][tn], 0, 0, 0);
       }
     }
+    if (more) store_tiles(buf ^ 1);
+    __syncthreads();
   }
+
+  float* out = static_cast<float*>(p.out);
+  if (p.splits > 1) out += static_cast<int64_t>(split) * p.gemm_m * p.gemm_n;
+  const bool accumulate = p.splits == 1 && p.accumulate;
+  staged_epilogue<T, WM, WN, TM, TN>(acc, reinterpret_cast<float*>(lds), tid, [&](int tr, int tc, float* v) {
+    const int row = m0 + tr, col = n0 + tc;
+    if (row >= p.gemm_m || col >= p.gemm_n) return;
+    float* dst = out + static_cast<int64_t>(row) * p.gemm_n + col;
+    if (accumulate) {
+#pragma unroll
+      for (int e = 0; e < E; ++e) v[e] += dst[e];
+    }
+    store_floats<E>(dst, v);
+  });
 }
 
 struct ReduceArgs {
@@ -446,8 +588,9 @@ int ilog2_exact(int v) {
 
 template <typename T, int MODE, int WM, int WN, int TM, int TN>
 const char* igemm_name() {
-  static const std::string name = std::string("igemm_kernel<") + (sizeof(T) == 2 ? "bf16" : "f32") + "," +
-                                  (MODE == kFwd ? "fwd" : MODE == kDgrad ? "dgrad" : "wgrad") + "," +
+  static const std::string name = std::string(MODE == kWgrad ? "wgrad_kernel<" : "igemm_kernel<") +
+                                  (sizeof(T) == 2 ? "bf16" : "f32") + "," +
+                                  (MODE == kFwd ? "fwd," : MODE == kDgrad ? "dgrad," : "") +
                                   std::to_string(WM * TM * 32) + "x" + std::to_string(WN * TN * 32) + ">";
   return name.c_str();
 }
@@ -462,8 +605,12 @@ int launch_cfg(Context* ctx, IgemmArgs& a, double flops) {
     set_error("igemm: grid out of range");
     return -22;
   }
-  return launch(ctx, igemm_kernel<T, MODE, WM, WN, TM, TN>, dim3(static_cast<unsigned>(wgs)), dim3(WM * WN * 64), a,
-                igemm_name<T, MODE, WM, WN, TM, TN>(), flops, 0);
+  const dim3 grid(static_cast<unsigned>(wgs)), block(WM * WN * 64);
+  if constexpr (MODE == kWgrad)
+    return launch(ctx, wgrad_kernel<T, WM, WN, TM, TN>, grid, block, a, igemm_name<T, MODE, WM, WN, TM, TN>(), flops, 0);
+  else
+    return launch(ctx, igemm_kernel<T, MODE, WM, WN, TM, TN>, grid, block, a, igemm_name<T, MODE, WM, WN, TM, TN>(),
+                  flops, 0);
 }
 
 template <typename T, int MODE>
@@ -563,13 +710,13 @@ int conv2d_fwd(Context* ctx, int dtype, const ConvShape& s, const void* x, const
                         : launch_mode<float, kFwd>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo));
 }
 
-int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, const void* w, void* dx, const void* add,
-                 const void* mask, int tile_cfg) {
+int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, const void* wt, void* dx,
+                 const void* add, const void* mask, int tile_cfg) {
   IgemmArgs a{};
   if (int rc = fill_common(a, s, dtype)) return rc;
-  TCH_CHECK_ARG(dy && w && dx, "conv2d_dgrad: null tensor");
+  TCH_CHECK_ARG(dy && wt && dx, "conv2d_dgrad: null tensor");
   a.a_src = dy;
-  a.b_src = w;
+  a.b_src = wt;
   a.out = dx;
   a.add = add;
   a.mask = mask;
@@ -577,6 +724,7 @@ int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, co
   a.gemm_n = s.C;
   a.gemm_k = s.R * s.S * s.K;
   a.k_per_split = (a.gemm_k + 31) / 32 * 32;
+  // 1x1 stride 1: dy is a dense [pixels][K] matrix in the same pixel order as dx
   a.div_plane = FastDiv(s.H * s.W);
   a.div_width = FastDiv(s.W);
   if (tile_cfg < 0) tile_cfg = pick_tile(a.gemm_m, a.gemm_n, 1);
