@@ -60,6 +60,7 @@ struct IgemmArgs {
   int out_f32;      // FWD/DGRAD: store fp32 instead of T
   int accumulate;   // WGRAD with splits == 1: out += result
   int pointwise;    // 1x1, stride 1, pad 0
+  uint32_t a_bytes, b_bytes;  // extents of a_src / b_src for the bounds-checked buffer loads
   FastDiv div_plane;  // pixels per image on the gather side
   FastDiv div_width;  // row width on the gather side
 };
@@ -85,9 +86,23 @@ __device__ inline void mma<float>(const Chunk& first, const Chunk& second, f32x1
   for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(first.f[e], second.f[e], acc, 0, 0, 0);
 }
 
-__device__ inline Chunk load_chunk(const void* base, int64_t elem_off, int elem_bytes, bool valid) {
-  Chunk c = zero_chunk();
-  if (valid) c.u = *reinterpret_cast<const uint4*>(static_cast<const char*>(base) + elem_off * elem_bytes);
+// Operand loads go through buffer instructions: an offset outside the declared extent
+// returns zeros, so padding, ragged edges and the tail of the reduction need neither a
+// branch nor a select, and the loads stay in flight across the multiply of earlier tiles.
+typedef unsigned int uint4_t __attribute__((ext_vector_type(4)));
+constexpr uint32_t kOutOfRange = 0x80000000u;
+
+__device__ inline __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
+}
+
+__device__ inline Chunk load_chunk(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_off, bool valid) {
+  uint4_t v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, static_cast<int>(valid ? byte_off : kOutOfRange), 0, 0);
+  Chunk c;
+  c.w[0] = v[0];
+  c.w[1] = v[1];
+  c.w[2] = v[2];
+  c.w[3] = v[3];
   return c;
 }
 
@@ -101,14 +116,17 @@ struct TapWalker {
     r = tap / S;
     s = tap - r * S;
   }
+  // branch-free; a step covers at most 4 taps (channels >= one chunk, step = 4 chunks)
   __device__ inline void advance(int step, int channels, int S) {
     ch += step;
-    while (ch >= channels) {
-      ch -= channels;
-      if (++s == S) {
-        s = 0;
-        ++r;
-      }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool wrap = ch >= channels;
+      ch -= wrap ? channels : 0;
+      s += wrap ? 1 : 0;
+      const bool wrap_s = s >= S;
+      s = wrap_s ? 0 : s;
+      r += wrap_s ? 1 : 0;
     }
   }
 };
@@ -233,16 +251,19 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm_kernel(IgemmArgs p) {
     }
   }
 
-  Chunk ra[A_PT], rb[B_PT];
+  // two register sets: the tiles kt+1 and kt+2 are in flight while tile kt is multiplied
+  Chunk ra0[A_PT], rb0[B_PT], ra1[A_PT], rb1[B_PT];
+  const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(p.a_src, p.a_bytes);
+  const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(p.b_src, p.b_bytes);
 
-  auto load_tiles = [&](int kt) {
+  auto load_tiles = [&](int kt, Chunk* ra, Chunk* rb) {
     const int k0 = kt * BK;
     const int kk = k0 + chunk_col * E;
     if (p.pointwise) {
       const bool k_ok = kk < k_end;
 #pragma unroll
       for (int i = 0; i < A_PT; ++i)
-        ra[i] = load_chunk(p.a_src, static_cast<int64_t>(a_base[i]) + kk, EB, a_row_ok[i] && k_ok);
+        ra[i] = load_chunk(rsrc_a, static_cast<uint32_t>(a_base[i] + kk) * EB, a_row_ok[i] && k_ok);
     } else {
       const bool tap_ok = walk.r < p.R && kk < k_end;
 #pragma unroll
@@ -261,8 +282,8 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm_kernel(IgemmArgs p) {
         }
         ok = ok && static_cast<unsigned>(hi) < static_cast<unsigned>(in_h) &&
              static_cast<unsigned>(wi) < static_cast<unsigned>(in_w);
-        const int64_t off = static_cast<int64_t>(a_base[i]) + (hi * in_w + wi) * in_c + walk.ch;
-        ra[i] = load_chunk(p.a_src, off, EB, ok);
+        const uint32_t off = static_cast<uint32_t>(a_base[i] + (hi * in_w + wi) * in_c + walk.ch) * EB;
+        ra[i] = load_chunk(rsrc_a, off, ok);
       }
       walk.advance(BK, in_c, p.S);
     }
@@ -271,11 +292,11 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm_kernel(IgemmArgs p) {
     for (int i = 0; i < B_PT; ++i) {
       const int row = n0 + ((tid + i * NT) >> 2);
       const bool ok = row < p.gemm_n && kk < k_end;
-      rb[i] = load_chunk(p.b_src, static_cast<int64_t>(row) * p.gemm_k + kk, EB, ok);
+      rb[i] = load_chunk(rsrc_b, static_cast<uint32_t>(row * p.gemm_k + kk) * EB, ok);
     }
   };
 
-  auto store_tiles = [&](int buf) {
+  auto store_tiles = [&](int buf, const Chunk* ra, const Chunk* rb) {
 #pragma unroll
     for (int i = 0; i < A_PT; ++i) {
       const int q = tid + i * NT;
@@ -296,18 +317,9 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm_kernel(IgemmArgs p) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  if (nk > 0) {
-    load_tiles(0);
-    store_tiles(0);
-  }
-  __syncthreads();
-
   const int frag_row = lane & 31;
   const int frag_half = lane >> 5;
-  for (int kt = 0; kt < nk; ++kt) {
-    const int buf = kt & 1;
-    const bool more = (kt + 1) < nk;
-    if (more) load_tiles(kt + 1);
+  auto compute = [&](int buf) {
     const uint4* la = lds_a + buf * BM * kLdsStride;
     const uint4* lb = lds_b + buf * BN * kLdsStride;
 #pragma unroll
@@ -322,8 +334,25 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm_kernel(IgemmArgs p) {
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn) mma<T>(fb[tn], fa[tm], acc[tm][tn]);
     }
-    if (more) store_tiles(buf ^ 1);
+  };
+
+  // Register set 0 carries the even tiles, set 1 the odd ones.  The loop has no
+  // conditionals: tiles past the end of the reduction load as zeros (out-of-range
+  // buffer offsets) and multiply to nothing, so an odd tile count costs one empty step.
+  load_tiles(0, ra0, rb0);
+  load_tiles(1, ra1, rb1);
+  store_tiles(0, ra0, rb0);
+  __syncthreads();
+  load_tiles(2, ra0, rb0);
+  for (int kt = 0; kt < nk; kt += 2) {
+    compute(0);  // tile kt
+    store_tiles(1, ra1, rb1);
     __syncthreads();
+    load_tiles(kt + 3, ra1, rb1);
+    compute(1);  // tile kt + 1
+    store_tiles(0, ra0, rb0);
+    __syncthreads();
+    load_tiles(kt + 4, ra0, rb0);
   }
 
   // ---- epilogue: bias, gated residual, rounding; 16-byte accesses per lane ----
@@ -417,39 +446,39 @@ __global__ __launch_bounds__(WM* WN * 64) void wgrad_kernel(IgemmArgs p) {
     b_s = tap - b_r * p.S;
   }
 
-  Chunk ra[A_PT], rb[B_PT];
+  Chunk ra0[A_PT], rb0[B_PT], ra1[A_PT], rb1[B_PT];
+  const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(p.a_src, p.a_bytes);
+  const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(p.b_src, p.b_bytes);
 
-  auto load_tiles = [&](int kt) {
+  auto load_tiles = [&](int kt, Chunk* ra, Chunk* rb) {
     const int k0 = k_begin + kt * BKP;
 #pragma unroll
     for (int i = 0; i < A_PT; ++i) {
       const int pix = k0 + a_prow + i * (NT / CA);
-      ra[i] = load_chunk(p.a_src, static_cast<int64_t>(pix) * p.K + a_ch, EB, a_ch_ok && pix < k_end);
+      ra[i] = load_chunk(rsrc_a, static_cast<uint32_t>(pix * p.K + a_ch) * EB, a_ch_ok && pix < k_end);
     }
 #pragma unroll
     for (int i = 0; i < B_PT; ++i) {
       const int pix = k0 + b_prow + i * (NT / CB);
       bool ok = b_n_ok && pix < k_end;
-      int64_t off;
+      uint32_t off;
       if (p.pointwise) {
-        off = static_cast<int64_t>(pix) * p.C + b_c;
+        off = static_cast<uint32_t>(pix * p.C + b_c) * EB;
       } else {
-        uint32_t img = 0, rem = 0, oh = 0, ow = 0;
-        if (ok) {
-          p.div_plane.divmod(static_cast<uint32_t>(pix), img, rem);
-          p.div_width.divmod(rem, oh, ow);
-        }
+        uint32_t img, rem, oh, ow;
+        p.div_plane.divmod(static_cast<uint32_t>(pix), img, rem);
+        p.div_width.divmod(rem, oh, ow);
         const int hi = static_cast<int>(oh) * p.stride - p.pad + b_r;
         const int wi = static_cast<int>(ow) * p.stride - p.pad + b_s;
         ok = ok && static_cast<unsigned>(hi) < static_cast<unsigned>(p.H) &&
              static_cast<unsigned>(wi) < static_cast<unsigned>(p.W);
-        off = (static_cast<int64_t>(img) * p.H * p.W + hi * p.W + wi) * p.C + b_c;
+        off = static_cast<uint32_t>((static_cast<int>(img) * p.H * p.W + hi * p.W + wi) * p.C + b_c) * EB;
       }
-      rb[i] = load_chunk(p.b_src, off, EB, ok);
+      rb[i] = load_chunk(rsrc_b, off, ok);
     }
   };
 
-  auto store_tiles = [&](int buf) {
+  auto store_tiles = [&](int buf, const Chunk* ra, const Chunk* rb) {
 #pragma unroll
     for (int i = 0; i < A_PT; ++i) lds_a[(buf * BKP + a_prow + i * (NT / CA)) * LDA + a_cc] = ra[i].u;
 #pragma unroll
@@ -464,11 +493,6 @@ __global__ __launch_bounds__(WM* WN * 64) void wgrad_kernel(IgemmArgs p) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  if (nk > 0) {
-    load_tiles(0);
-    store_tiles(0);
-  }
-  __syncthreads();
 
   // transpose-read geometry (bf16): lane = 16*G + q; the 16 lanes of a group read
   // pixels {base + q/4 ...} x channels {16*(G%2) + 4*(q%4) ...}; after the transpose
@@ -477,10 +501,7 @@ __global__ __launch_bounds__(WM* WN * 64) void wgrad_kernel(IgemmArgs p) {
   const int tr_pix = 8 * (grp >> 1) + (q16 >> 2);
   const int tr_ch = 16 * (grp & 1) + 4 * (q16 & 3);
 
-  for (int kt = 0; kt < nk; ++kt) {
-    const int buf = kt & 1;
-    const bool more = (kt + 1) < nk;
-    if (more) load_tiles(kt + 1);
+  auto compute = [&](int buf) {
     if constexpr (sizeof(T) == 2) {
       const uint16_t* la = reinterpret_cast<const uint16_t*>(lds_a + buf * BKP * LDA);
       const uint16_t* lb = reinterpret_cast<const uint16_t*>(lds_b + buf * BKP * LDB);
@@ -531,9 +552,27 @@ __global__ __launch_bounds__(WM* WN * 64) void wgrad_kernel(IgemmArgs p) {
             acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(fb[tn], fa[tm], acc[tm][tn], 0, 0, 0);
       }
     }
-    if (more) store_tiles(buf ^ 1);
+  };
+
+  // Register set 0 carries the even tiles, set 1 the odd ones.  The loop has no
+  // conditionals: tiles past the end of the reduction load as zeros (out-of-range
+  // buffer offsets) and multiply to nothing, so an odd tile count costs one empty step.
+  load_tiles(0, ra0, rb0);
+  load_tiles(1, ra1, rb1);
+  store_tiles(0, ra0, rb0);
+  __syncthreads();
+  load_tiles(2, ra0, rb0);
+  for (int kt = 0; kt < nk; kt += 2) {
+    compute(0);  // tile kt
+    store_tiles(1, ra1, rb1);
     __syncthreads();
+    load_tiles(kt + 3, ra1, rb1);
+    compute(1);  // tile kt + 1
+    store_tiles(0, ra0, rb0);
+    __syncthreads();
+    load_tiles(kt + 4, ra0, rb0);
   }
+
 
   float* out = static_cast<float*>(p.out);
   if (p.splits > 1) out += static_cast<int64_t>(split) * p.gemm_m * p.gemm_n;
@@ -657,6 +696,8 @@ int fill_common(IgemmArgs& a, const ConvShape& s, int dtype) {
   const int64_t in_elems = static_cast<int64_t>(s.N) * s.H * s.W * s.C;
   const int64_t out_elems = static_cast<int64_t>(s.N) * Ho * Wo * s.K;
   TCH_CHECK_ARG(in_elems < (1ll << 31) && out_elems < (1ll << 31), "conv: tensor exceeds 2^31 elements");
+  TCH_CHECK_ARG(in_elems * (16 / E) < (1ll << 31) && out_elems * (16 / E) < (1ll << 31),
+                "conv: tensor exceeds the 2 GiB reach of a buffer offset");
   TCH_CHECK_ARG(static_cast<int64_t>(s.K) * s.R * s.S * s.C < (1ll << 31), "conv: filter exceeds 2^31 elements");
   a.N = s.N;
   a.H = s.H;
@@ -692,8 +733,11 @@ int conv2d_fwd(Context* ctx, int dtype, const ConvShape& s, const void* x, const
   IgemmArgs a{};
   if (int rc = fill_common(a, s, dtype)) return rc;
   TCH_CHECK_ARG(x && w && y, "conv2d_fwd: null tensor");
+  const int eb = dtype == kBF16 ? 2 : 4;
   a.a_src = x;
   a.b_src = w;
+  a.a_bytes = static_cast<uint32_t>(static_cast<int64_t>(s.N) * s.H * s.W * s.C * eb);
+  a.b_bytes = static_cast<uint32_t>(static_cast<int64_t>(s.K) * s.R * s.S * s.C * eb);
   a.out = y;
   a.add = add;
   a.mask = mask;
@@ -715,8 +759,11 @@ int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, co
   IgemmArgs a{};
   if (int rc = fill_common(a, s, dtype)) return rc;
   TCH_CHECK_ARG(dy && wt && dx, "conv2d_dgrad: null tensor");
+  const int eb = dtype == kBF16 ? 2 : 4;
   a.a_src = dy;
   a.b_src = wt;
+  a.a_bytes = static_cast<uint32_t>(static_cast<int64_t>(s.N) * a.Ho * a.Wo * s.K * eb);
+  a.b_bytes = static_cast<uint32_t>(static_cast<int64_t>(s.K) * s.R * s.S * s.C * eb);
   a.out = dx;
   a.add = add;
   a.mask = mask;
@@ -760,11 +807,14 @@ int conv2d_wgrad(Context* ctx, int dtype, const ConvShape& s, const void* x, con
   IgemmArgs a{};
   if (int rc = fill_common(a, s, dtype)) return rc;
   TCH_CHECK_ARG(x && dy && dw, "conv2d_wgrad: null tensor");
+  const int eb = dtype == kBF16 ? 2 : 4;
   TCH_CHECK_ARG(splits >= 1, "conv2d_wgrad: splits must be >= 1");
   TCH_CHECK_ARG(splits == 1 || workspace, "conv2d_wgrad: split reduction needs a workspace");
   const int BK = dtype == kBF16 ? 32 : 16;
   a.a_src = dy;
   a.b_src = x;
+  a.a_bytes = static_cast<uint32_t>(static_cast<int64_t>(s.N) * a.Ho * a.Wo * s.K * eb);
+  a.b_bytes = static_cast<uint32_t>(static_cast<int64_t>(s.N) * s.H * s.W * s.C * eb);
   a.gemm_m = s.K;
   a.gemm_n = s.R * s.S * s.C;
   a.gemm_k = s.N * a.Ho * a.Wo;
