@@ -1,14 +1,16 @@
-"""ctypes binding of libtorch_col_hip.so (the C ABI declared in include/*.h).
+"""ctypes binding of libtorch_col_hip.so, generated from the C ABI headers in include/.
 
-There is no fallback: if the shared library has not been built, importing the
-handle raises, so no caller can silently run anything but the HIP path.
+There is no fallback: if the shared library has not been built, asking for the handle
+raises, so no caller can silently run anything but the HIP path.
 """
 import ctypes
 import os
-from ctypes import POINTER, c_char_p, c_float, c_int, c_int32, c_int64, c_size_t, c_uint64, c_void_p
+import re
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libtorch_col_hip.so")
+INCLUDE_DIR = os.path.join(os.path.dirname(_HERE), "include")
+HEADERS = ("torch_col_hip.h", "torch_col_host.h")
 
 _lib = None
 
@@ -20,82 +22,77 @@ class TorchColHipError(RuntimeError):
 class KernelStat(ctypes.Structure):
     """Mirror of tch_kernel_stat (include/torch_col_hip.h)."""
     _fields_ = [("name", ctypes.c_char * 96), ("total_ms", ctypes.c_double), ("work", ctypes.c_double),
-                ("launches", c_int64), ("work_is_bytes", c_int)]
+                ("launches", ctypes.c_int64), ("work_is_bytes", ctypes.c_int)]
 
 
-def _declare(lib):
-    vp, i, i64, f = c_void_p, c_int, c_int64, c_float
-    sig = {
-        "tch_last_error": (c_char_p, []),
-        "tch_has_device_code": (i, []),
-        "tch_context_create": (i, [vp, POINTER(vp)]),
-        "tch_context_destroy": (None, [vp]),
-        "tch_context_take_rejected": (c_uint64, [vp]),
-        "tch_program_create": (i, [POINTER(vp)]),
-        "tch_program_destroy": (None, [vp]),
-        "tch_program_size": (i64, [vp]),
-        "tch_program_begin_record": (i, [vp, vp]),
-        "tch_program_end_record": (i, [vp]),
-        "tch_program_run": (i, [vp, vp, i64, i64]),
-        "tch_RegisterStream": (c_uint64, [c_uint64]),
-        "tch_UnRegisterStream": (i, [c_uint64]),
-        "tch_UnRegisterAllStreams": (None, []),
-        "tch_GetXQueueSize": (c_size_t, [c_uint64]),
-        "tch_GetXQueueSizeAllStreams": (c_size_t, []),
-        "tch_GetTotalXQueueSize": (c_size_t, []),
-        "tch_AbortStream": (c_size_t, [c_uint64]),
-        "tch_AbortAllStreams": (c_size_t, []),
-        "tch_SyncStream": (i, [c_uint64]),
-        "tch_SyncAllStreams": (i, []),
-        "tch_QueryRejectCudaCalls": (i, []),
-        "tch_SetRejectCudaCalls": (None, [i]),
-        "tch_SetXQueueShape": (None, [i, i]),
-        "tch_GetXQueueInFlight": (c_size_t, [c_uint64]),
-        "tch_program_profile": (i, [vp, vp, i, vp, i, POINTER(c_int)]),
-        "tch_conv2d_fwd": (i, [vp, i, vp, vp, vp, vp, vp, vp, i] + [i] * 11),
-        "tch_conv2d_dgrad": (i, [vp, i, vp, vp, vp, vp, vp] + [i] * 11),
-        "tch_conv2d_wgrad_pick_splits": (i, [i] * 10),
-        "tch_conv2d_wgrad_workspace_bytes": (i64, [i] * 6),
-        "tch_conv2d_wgrad": (i, [vp, i, vp, vp, vp, vp, i, i] + [i] * 11),
-        "tch_bn_workspace_bytes": (i64, [i, i64, i]),
-        "tch_bn_fwd_train": (i, [vp, i, vp, vp, vp, i, i64, i, vp, vp, vp, vp, vp, vp, f, f, vp]),
-        "tch_bn_bwd": (i, [vp, i, vp, vp, vp, vp, i64, i, vp, vp, vp, vp, vp, i, vp]),
-        "tch_maxpool_fwd": (i, [vp, i, vp, vp, vp] + [i] * 7),
-        "tch_maxpool_bwd": (i, [vp, i, vp, vp, vp] + [i] * 7),
-        "tch_avgpool_fwd": (i, [vp, i, vp, vp, i, i, i]),
-        "tch_avgpool_bwd": (i, [vp, i, vp, vp, i, i, i]),
-        "tch_softmax_ce_fwd_bwd": (i, [vp, i, vp, vp, vp, vp, vp, i, i, i, f]),
-        "tch_sgd_momentum_step": (i, [vp, vp, vp, vp, vp, i64, f, f, f]),
-        "tch_grad_accumulate": (i, [vp, vp, vp, i64]),
-        "tch_fill_zero": (i, [vp, vp, i64]),
-        "tch_bias_grad": (i, [vp, i, vp, vp, i, i, i, i]),
-        "tch_nchw_to_nhwc_pad": (i, [vp, i, vp, vp, i, i, i, i, i]),
-        "tch_filter_transpose_batched": (i, [vp, i, vp, vp, vp, i, i64, i64]),
-        "tch_cast_from_f32": (i, [vp, i, vp, vp, i64]),
-        "tch_cast_to_f32": (i, [vp, i, vp, vp, i64]),
-    }
-    for name, (res, args) in sig.items():
-        fn = getattr(lib, name)
-        fn.restype = res
-        fn.argtypes = args
+class CtrlMsg(ctypes.Structure):
+    """Mirror of tch_ctrl_msg (include/torch_col_host.h)."""
+    _fields_ = [("id", ctypes.c_uint64), ("event", ctypes.c_int), ("value", ctypes.c_int)]
+
+
+_SCALARS = {
+    "int": ctypes.c_int, "unsigned": ctypes.c_uint, "float": ctypes.c_float, "double": ctypes.c_double,
+    "int32_t": ctypes.c_int32, "uint32_t": ctypes.c_uint32, "int64_t": ctypes.c_int64, "uint64_t": ctypes.c_uint64,
+    "size_t": ctypes.c_size_t, "ptrdiff_t": ctypes.c_ssize_t,
+}
+
+
+def _ctype(decl, is_return):
+    d = decl.replace("const", " ").strip()
+    if "*" in d:
+        base = d.replace("*", " ").split()[0]
+        if base == "char":
+            return ctypes.c_char_p if (is_return or "const" in decl) else ctypes.c_void_p
+        return ctypes.c_void_p
+    base = d.split()[0]
+    if base == "void":
+        return None
+    return _SCALARS[base]
+
+
+def parse_header(path):
+    """{function name: (restype, [argtypes])} for every prototype in a C ABI header."""
+    text = open(path).read()
+    text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", " ", text)
+    text = re.sub(r"^\s*#.*$", " ", text, flags=re.M)
+    text = re.sub(r"typedef\s+struct\s+\w+\s*\{.*?\}\s*\w+\s*;", " ", text, flags=re.S)
+    text = re.sub(r"typedef[^;]*;", " ", text)
+    text = text.replace('extern "C" {', " ").replace("}", " ")
+    out = {}
+    for m in re.finditer(r"([\w\s\*]+?)\b(tch_\w+)\s*\(([^;{]*?)\)\s*;", text):
+        ret, name, args = m.group(1).strip(), m.group(2), m.group(3).strip()
+        argtypes = []
+        if args and args != "void":
+            for a in args.split(","):
+                a = a.strip()
+                # drop the parameter name (last identifier not part of the type)
+                a = re.sub(r"\b\w+$", "", a).strip() if re.search(r"[\*\s]\w+$", a) else a
+                argtypes.append(_ctype(a, False))
+        out[name] = (_ctype(ret, True), argtypes)
+    return out
+
+
+def declared_symbols():
+    sig = {}
+    for h in HEADERS:
+        sig.update(parse_header(os.path.join(INCLUDE_DIR, h)))
     return sig
-
-
-DEVICE_SYMBOLS = None
 
 
 def lib():
     """The loaded shared library; raises if it was never built."""
-    global _lib, DEVICE_SYMBOLS
+    global _lib
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise TorchColHipError(
                 f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
                 "or `make -C sirius_amd/csrc`. There is no CPU fallback for this path.")
         handle = ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
-        DEVICE_SYMBOLS = _declare(handle)
-        from . import _lib_host  # noqa: F401  (declares the host-runtime half of the ABI)
-        _lib_host.declare(handle)
+        for name, (res, args) in declared_symbols().items():
+            fn = getattr(handle, name)  # AttributeError here = header and library disagree
+            fn.restype = res
+            fn.argtypes = args
         _lib = handle
     return _lib
 
@@ -103,5 +100,12 @@ def lib():
 def check(rc, what=""):
     if rc < 0:
         msg = lib().tch_last_error()
+        raise TorchColHipError(f"{what} failed ({rc}): {msg.decode() if msg else ''}")
+    return rc
+
+
+def check_host(rc, what=""):
+    if rc < 0:
+        msg = lib().tch_host_last_error()
         raise TorchColHipError(f"{what} failed ({rc}): {msg.decode() if msg else ''}")
     return rc

@@ -6,6 +6,7 @@ and the library enqueues hand-written HIP kernels.  Layout is NHWC throughout;
 filters are [K, R, S, C].
 """
 import ctypes
+import time
 
 import torch
 
@@ -91,6 +92,19 @@ class Context:
 
     def take_rejected(self):
         return int(lib().tch_context_take_rejected(self.handle))
+
+    def flush(self):
+        """Wait until every queued launch has been handed to the HIP stream.  Work torch puts on
+        the stream itself (copies, fills, read-backs) does not pass through the launch queue, so
+        stream order only covers it once the queue is empty.  No-op for an unregistered stream."""
+        s = self.stream.cuda_stream
+        while lib().tch_GetXQueueSize(s):
+            time.sleep(0)
+
+    def synchronize(self):
+        """Everything submitted so far, queued or not, has finished on the GPU."""
+        self.flush()
+        self.stream.synchronize()
 
     def profile(self, program, reps=1):
         """Per-kernel HIP-event timing of `reps` replays: list of dicts with name, total_ms,

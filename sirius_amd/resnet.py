@@ -47,7 +47,7 @@ class _Block:
 
 class ResNetEngine:
     def __init__(self, depths=(3, 8, 36, 3), num_classes=1000, width=64, dtype=torch.bfloat16, image_size=224,
-                 lr=0.1, momentum=0.9, weight_decay=1e-4, bn_momentum=0.1, bn_eps=1e-5, stream=None):
+                 lr=0.1, momentum=0.9, weight_decay=1e-4, bn_momentum=0.1, bn_eps=1e-5, stream=None, allocator=None):
         if not torch.cuda.is_available():
             raise RuntimeError("ResNetEngine runs on the GPU only; there is no CPU path")
         assert dtype in (torch.bfloat16, torch.float32)
@@ -58,6 +58,11 @@ class ResNetEngine:
         self.dev = torch.device("cuda", torch.cuda.current_device())
         self.ctx = ops.Context(stream if stream is not None else torch.cuda.current_stream())
         self.depths, self.width = tuple(depths), width
+        # allocator(shape, dtype) -> uninitialised device tensor; the shared HBM pool plugs in here
+        # (torch_col.pool_empty), torch's own allocator is the default
+        self._alloc = allocator if allocator is not None else (
+            lambda shape, dtype: torch.empty(shape, dtype=dtype, device=self.dev))
+        self._hook = None
 
         # ---- architecture + parameter table (torchvision naming and order) ----
         self._specs, self._bn_names = [], []
@@ -93,21 +98,22 @@ class ResNetEngine:
         self.n_store = self._off
         self.spec = {p.name: p for p in self._specs}
 
-        f32 = dict(dtype=torch.float32, device=self.dev)
-        self.params = torch.zeros(self.n_store, **f32)
-        self.grads = torch.zeros(self.n_store, **f32)
-        self.momentum_buf = torch.zeros(self.n_store, **f32)
+        def zeros(n, dt=torch.float32):
+            return self._alloc((n,), dt).zero_()
+        self.params = zeros(self.n_store)
+        self.grads = zeros(self.n_store)
+        self.momentum_buf = zeros(self.n_store)
         self.global_grads = None
-        self.shadow = torch.zeros(self.n_store, dtype=torch.bfloat16, device=self.dev) if dtype == torch.bfloat16 else None
+        self.shadow = zeros(self.n_store, torch.bfloat16) if dtype == torch.bfloat16 else None
         # filters transposed to [C,R,S,K] for the data-gradient GEMM, same offsets, rewritten
         # in one launch whenever the weights change
-        self.wt = torch.zeros(self.n_store, dtype=dtype, device=self.dev)
+        self.wt = zeros(self.n_store, dtype)
         self._tt = ops.FilterTransposeTable(
             [(p.offset, p.store_shape[0], p.store_shape[1] * p.store_shape[2], p.store_shape[3])
              for p in self._specs if p.kind in ("conv", "fc_w")], self.dev)
         nbn = sum(c for _, c in self._bn_names)
-        self.running_mean = torch.zeros(nbn, **f32)
-        self.running_var = torch.ones(nbn, **f32)
+        self.running_mean = zeros(nbn)
+        self.running_var = zeros(nbn).fill_(1.0)
         self._bn_off, o = {}, 0
         for name, c in self._bn_names:
             self._bn_off[name] = (o, c)
@@ -234,7 +240,7 @@ class ResNetEngine:
         keep = []
 
         def act(*shape, dtype=T):
-            t = torch.empty(shape, dtype=dtype, device=dev)
+            t = self._alloc(tuple(shape), dtype)
             keep.append(t)
             return t
 
@@ -247,7 +253,7 @@ class ResNetEngine:
             lst = free.get(n)
             if lst:
                 return lst.pop().view(shape)
-            t = torch.empty(n, dtype=T, device=dev)
+            t = self._alloc((n,), T)
             keep.append(t)
             return t.view(shape)
 
@@ -256,7 +262,7 @@ class ResNetEngine:
 
         code = ops.dtype_code(torch.empty(0, dtype=T))
         plan.x_in = act(B, 3, S, S, dtype=torch.float32)
-        plan.labels = torch.zeros(B, dtype=torch.int64, device=dev)
+        plan.labels = act(B, dtype=torch.int64).zero_()
         plan.loss_rows = act(B, dtype=torch.float32)
         plan.loss = act(1, dtype=torch.float32)
         bn_save = act(2 * self.running_mean.numel(), dtype=torch.float32)
@@ -329,6 +335,11 @@ class ResNetEngine:
             ops.conv2d_dgrad(ctx, dy, self._wt(c.name + ".weight"), dx, c.stride, c.pad, c_logical=c.cin, **kw)
 
         prog = ops.Program()
+        marks = []  # (launch index one past the layer, 'fwd' | 'bwd', layer name): checkpoint positions
+
+        def mark(phase, name):
+            marks.append((len(prog), phase, name))
+
         ctx.begin_record(prog)
         try:
             # ================= forward =================
@@ -337,6 +348,7 @@ class ResNetEngine:
             z0, a0 = act(B, H0, W0, self.width), act(B, H0, W0, self.width)
             conv_fwd(self.stem, x0, z0)
             bn_fwd("bn1", z0, a0)
+            mark("fwd", "bn1")
             p0 = act(B, Hp, Wp, self.width)
             p0_idx = act(B, Hp, Wp, self.width, dtype=torch.int32)
             ops.maxpool_fwd(ctx, a0, p0, p0_idx, 3, 2, 1)
@@ -347,9 +359,11 @@ class ResNetEngine:
                 z1, a1 = act(B, H, W, P), act(B, H, W, P)
                 conv_fwd(blk.c1, x, z1)
                 bn_fwd(pre + ".bn1", z1, a1)
+                mark("fwd", pre + ".bn1")
                 z2, a2 = act(B, Ho, Wo, P), act(B, Ho, Wo, P)
                 conv_fwd(blk.c2, a1, z2)
                 bn_fwd(pre + ".bn2", z2, a2)
+                mark("fwd", pre + ".bn2")
                 z3, out = act(B, Ho, Wo, 4 * P), act(B, Ho, Wo, 4 * P)
                 conv_fwd(blk.c3, a2, z3)
                 zd = None
@@ -360,6 +374,7 @@ class ResNetEngine:
                 else:
                     idn = x
                 bn_fwd(pre + ".bn3", z3, out, residual=idn, relu=True)
+                mark("fwd", pre + ".bn3")
                 saved.append((x, z1, a1, z2, a2, z3, zd, out))
                 x = out
             pooled = act(B, self.feat)
@@ -370,6 +385,7 @@ class ResNetEngine:
             dlogits = act(B, self.num_classes)
             ops.softmax_ce_fwd_bwd(ctx, logits, plan.labels, plan.loss_rows, plan.loss, dlogits, loss_scale=loss_scale)
             plan.n_forward = len(prog)
+            mark("fwd", "loss")
 
             # ================= backward =================
             ops.conv2d_wgrad(ctx, pooled.view(B, 1, 1, self.feat), dlogits.view(B, 1, 1, self.num_classes),
@@ -389,6 +405,7 @@ class ResNetEngine:
                 conv_wgrad(blk.c3, a2, dz3)
                 g_a2 = galloc(a2.shape)
                 conv_dgrad(blk.c3, dz3, g_a2)
+                mark("bwd", pre + ".conv3")
                 gfree(dz3)
                 dz2 = galloc(z2.shape)
                 bn_bwd(pre + ".bn2", g_a2, z2, dz2, a2)
@@ -396,6 +413,7 @@ class ResNetEngine:
                 conv_wgrad(blk.c2, a1, dz2)
                 g_a1 = galloc(a1.shape)
                 conv_dgrad(blk.c2, dz2, g_a1)
+                mark("bwd", pre + ".conv2")
                 gfree(dz2)
                 dz1 = galloc(z1.shape)
                 bn_bwd(pre + ".bn1", g_a1, z1, dz1, a1)
@@ -413,6 +431,7 @@ class ResNetEngine:
                     gfree(gx_id)
                 else:
                     conv_dgrad(blk.c1, dz1, gx, add=g_out, mask=out)
+                mark("bwd", pre + ".conv1")
                 gfree(dz1)
                 gfree(g_out)
                 g_out = gx
@@ -427,6 +446,7 @@ class ResNetEngine:
         finally:
             ctx.end_record()
         plan.prog = prog
+        plan.marks = marks
         plan.keep = keep
         plan.logits = logits
         plan.bytes = sum(t.numel() * t.element_size() for t in keep)
@@ -448,19 +468,37 @@ class ResNetEngine:
         self._plans.clear()
         return n
 
+    def set_checkpoint_hook(self, fn):
+        """fn(phase, layer name) runs between the launch segments of forward_backward, once per
+        layer and direction: the place of the forward / backward module hooks of the reference
+        (torch_col/colocate_ctrl.py:360-402).  An exception raised by fn ends the step there."""
+        self._hook = fn
+
+    def _run_plan(self, p):
+        if self._hook is None:
+            return self.ctx.run(p.prog)
+        first, cut = 0, False
+        for idx, phase, name in p.marks:
+            cut = self.ctx.run(p.prog, first, idx) or cut
+            first = idx
+            self._hook(phase, name)
+        if first < len(p.prog):
+            cut = self.ctx.run(p.prog, first, len(p.prog)) or cut
+        return cut
+
     # ------------------------------------------------------------------ the step
     def forward_backward(self, x, y, loss_scale=1.0):
         """x [B,3,S,S] fp32 and y [B] int64 on the GPU.  Returns (plan, cut_short)."""
         p = self.plan(x.shape[0], loss_scale)
+        self.ctx.flush()
         p.x_in.copy_(x, non_blocking=True)
         p.labels.copy_(y, non_blocking=True)
-        cut = self.ctx.run(p.prog)
-        return p, cut
+        return p, self._run_plan(p)
 
     def forward_backward_resident(self, batch, loss_scale=1.0):
         """Replay on whatever already sits in the plan's input buffers."""
         p = self.plan(batch, loss_scale)
-        return p, self.ctx.run(p.prog)
+        return p, self._run_plan(p)
 
     def _flat_prog(self, fn):
         prog = ops.Program()
@@ -471,15 +509,33 @@ class ResNetEngine:
             self.ctx.end_record()
         return prog
 
+    def ensure_global_grads(self):
+        if self.global_grads is None:
+            self.global_grads = self._alloc((self.n_store,), torch.float32).zero_()
+
+    def zero_global_grads(self):
+        if self.global_grads is not None:
+            ops.fill_zero(self.ctx, self.global_grads)
+
+    def synchronize(self):
+        self.ctx.synchronize()
+
+    def zero_grad(self):
+        ops.fill_zero(self.ctx, self.grads)
+
+    def discard_partial_grads(self):
+        """After a killed micro-batch: its gradients are partial.  Every backward overwrites the
+        whole gradient buffer, so zeroing is only for the reader of grads_dict()."""
+        ops.fill_zero(self.ctx, self.grads)
+
     def accumulate(self):
         """global += grads; grads = 0   (GradAccumulator.accumulate)"""
-        if self.global_grads is None:
-            self.global_grads = torch.zeros_like(self.grads)
+        self.ensure_global_grads()
         if self._acc_prog is None:
             self._acc_prog = self._flat_prog(lambda: ops.grad_accumulate(self.ctx, self.global_grads, self.grads))
         return self.ctx.run(self._acc_prog)
 
-    def optimizer_step(self, use_global=False):
+    def optimizer_step(self, use_global=False, zero_global=True):
         """SGD-momentum over the flat buffers; with use_global the accumulated gradients are
         consumed and zeroed (GradAccumulator.step)."""
         if use_global:
@@ -490,9 +546,11 @@ class ResNetEngine:
                     ops.sgd_momentum_step(self.ctx, self.params, self.global_grads, self.momentum_buf, self.lr,
                                           self.momentum, self.weight_decay, shadow=self.shadow)
                     self._refresh_transposed()
-                    ops.fill_zero(self.ctx, self.global_grads)
                 self._opt_global_prog = self._flat_prog(rec)
-            return self.ctx.run(self._opt_global_prog)
+            cut = self.ctx.run(self._opt_global_prog)
+            if zero_global:
+                ops.fill_zero(self.ctx, self.global_grads)
+            return cut
         if self._opt_prog is None:
             def rec():
                 ops.sgd_momentum_step(self.ctx, self.params, self.grads, self.momentum_buf, self.lr, self.momentum,
