@@ -56,6 +56,9 @@ const char* tch_TorchColConfig_GetTrainProfileLogPath(void);
 int tch_pool_init(int device, uint64_t pool_bytes, int use_gpu);
 void tch_pool_shutdown(int device);
 int tch_pool_is_enabled(int device);
+/* number of pools this device has had so far: a holder of a pool pointer compares it with the value
+ * at allocation time before freeing, so that a pointer into a pool that was shut down is dropped */
+uint64_t tch_pool_generation(int device);
 uint64_t tch_cuda_memory_pool_infer_usage(int device);
 uint64_t tch_cuda_memory_pool_train_usage(int device);
 uint64_t tch_cuda_memory_pool_train_peak_usage(int device);

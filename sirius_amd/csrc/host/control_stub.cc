@@ -10,7 +10,20 @@ namespace host {
 namespace {
 std::mutex g_prof_mu;
 std::vector<int64_t> g_adjust_request, g_adjust_done;
+// stubs whose control thread is running: the thread blocks on the shared segment, so it has to
+// be stopped before the segment goes away
+std::mutex g_live_mu;
+std::vector<StubBase*> g_live;
 }  // namespace
+
+void StubBase::stop_all() {
+  std::vector<StubBase*> live;
+  {
+    std::lock_guard<std::mutex> l(g_live_mu);
+    live = g_live;
+  }
+  for (StubBase* s : live) s->stop();
+}
 
 void StubProfiler::record_adjust_request() {
   std::lock_guard<std::mutex> l(g_prof_mu);
@@ -44,6 +57,10 @@ int StubBase::config_rank() { return config().train_rank; }
 void StubBase::start() {
   if (!config().has_colocated_infer_server || !communicator() || thread_) return;
   running_.store(true);
+  {
+    std::lock_guard<std::mutex> l(g_live_mu);
+    g_live.push_back(this);
+  }
   thread_.reset(new std::thread([this] {
     while (running_.load()) {
       CtrlMsgEntry msg;
@@ -53,10 +70,17 @@ void StubBase::start() {
 }
 
 void StubBase::stop() {
+  std::lock_guard<std::mutex> stop_lock(stop_mutex_);
   if (thread_) {
     running_.store(false);
     thread_->join();
     thread_.reset();
+    std::lock_guard<std::mutex> l(g_live_mu);
+    for (size_t i = 0; i < g_live.size(); ++i)
+      if (g_live[i] == this) {
+        g_live.erase(g_live.begin() + i);
+        break;
+      }
   }
 }
 

@@ -29,6 +29,7 @@ class StubBase {
   virtual ~StubBase();
   void start();  // spawns the control thread when an inference server is colocated
   void stop();
+  static void stop_all();  // every running control thread; call before the shared segments are unmapped
   int cmd() const { return cmd_.load(std::memory_order_acquire); }
   void set_cmd(int c);
   void train_start();
@@ -58,6 +59,7 @@ class StubBase {
   std::atomic<bool> running_{false};
   std::unique_ptr<std::thread> thread_;
   std::mutex mutex_;
+  std::mutex stop_mutex_;
   std::string error_;
 };
 

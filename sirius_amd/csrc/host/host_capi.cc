@@ -70,6 +70,8 @@ int tch_TorchColInit(int train_rank, int train_world_size, int use_gpu) {
 }
 
 void tch_TorchColShutdown(void) {
+  StubBase::stop_all();
+  StubProfiler::clear();
   DynamicBatchDistributor::shutdown();
   DistTrainSync::shutdown();
   communicator_shutdown();
@@ -107,6 +109,7 @@ int tch_pool_init(int device, uint64_t pool_bytes, int use_gpu) {
 }
 void tch_pool_shutdown(int device) { pool_shutdown(device); }
 int tch_pool_is_enabled(int device) { return pool(device) != nullptr; }
+uint64_t tch_pool_generation(int device) { return pool_generation(device); }
 uint64_t tch_cuda_memory_pool_infer_usage(int d) { return pool(d) ? pool(d)->stats().infer_usage : 0; }
 uint64_t tch_cuda_memory_pool_train_usage(int d) { return pool(d) ? pool(d)->stats().train_usage : 0; }
 uint64_t tch_cuda_memory_pool_train_peak_usage(int d) { return pool(d) ? pool(d)->stats().train_peak_usage : 0; }
@@ -169,7 +172,10 @@ int tch_InfTraCommunicator_Init(int is_server, int cleanup, int world) {
   if (!communicator_init(is_server != 0, cleanup != 0, world, &err)) return fail(err);
   return 0;
 }
-void tch_InfTraCommunicator_Shutdown(void) { communicator_shutdown(); }
+void tch_InfTraCommunicator_Shutdown(void) {
+  StubBase::stop_all();
+  communicator_shutdown();
+}
 int tch_InfTraCommunicator_IsInitialized(void) { return communicator() != nullptr; }
 
 #define NEED_COMM() \

@@ -10,6 +10,7 @@ namespace host {
 namespace {
 std::unique_ptr<HbmPool> g_pools[kMaxDeviceNum];
 std::mutex g_pools_mu;
+uint64_t g_generation[kMaxDeviceNum] = {};  // bumped per pool_init: tells a stale pointer from a live one
 
 inline size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 }  // namespace
@@ -234,6 +235,7 @@ size_t HbmPool::process_events() {
 
 size_t HbmPool::empty_cache_locked() {
   size_t bytes = 0;
+  bool quiesced = false;
   for (Segment* s : {&small_, &large_}) {
     for (auto& kv : s->blocks) {
       if (kv.second.allocated) continue;
@@ -244,6 +246,12 @@ size_t HbmPool::empty_cache_locked() {
         const int page = slot_page_[slot];
         if (page < 0) continue;
         std::string err;
+        if (!quiesced) {
+          // a freed block may still be read by launches in flight on its own stream (frees are
+          // stream ordered): nothing may be running when its pages lose their mapping
+          backend_->quiesce();
+          quiesced = true;
+        }
         if (!backend_->unmap(base_ + a, page, &err)) continue;
         slot_page_[slot] = -1;
         owner_[page] = kOwnerFree;
@@ -377,7 +385,13 @@ bool pool_init(int device, size_t pool_bytes, bool use_gpu, std::string* err) {
   }
   PoolBackend* be = use_gpu ? make_hip_vmm_backend(device) : new NullBackend();
   g_pools[device].reset(HbmPool::create(device, pool_bytes, be, err));
+  if (g_pools[device]) ++g_generation[device];
   return g_pools[device] != nullptr;
+}
+
+uint64_t pool_generation(int device) {
+  std::lock_guard<std::mutex> lock(g_pools_mu);
+  return device >= 0 && device < kMaxDeviceNum ? g_generation[device] : 0;
 }
 
 void pool_shutdown(int device) {

@@ -52,6 +52,7 @@ class PoolBackend {
   virtual bool create_pages(int n, std::string* err) = 0;
   virtual bool map(uint64_t va, int page, std::string* err) = 0;
   virtual bool unmap(uint64_t va, int page, std::string* err) = 0;
+  virtual void quiesce() {}  // wait until the device is idle (called once before a round of unmaps)
   // event support for frees that must wait for other streams
   virtual uint64_t record_event(uint64_t stream) = 0;
   virtual bool event_done(uint64_t event) = 0;  // also destroys a finished event
@@ -162,6 +163,7 @@ class HbmPool {
 HbmPool* pool(int device);
 bool pool_init(int device, size_t pool_bytes, bool use_gpu, std::string* err);
 void pool_shutdown(int device);
+uint64_t pool_generation(int device);  // how many pools this device has had
 
 }  // namespace host
 }  // namespace tch

@@ -78,6 +78,11 @@ class HipVmmBackend : public PoolBackend {
     return true;
   }
 
+  void quiesce() override {
+    (void)hipSetDevice(device_);
+    (void)hipDeviceSynchronize();
+  }
+
   uint64_t record_event(uint64_t stream) override {
     hipEvent_t e = nullptr;
     if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess) return 0;

@@ -63,6 +63,7 @@ class ResNetEngine:
         self._alloc = allocator if allocator is not None else (
             lambda shape, dtype: torch.empty(shape, dtype=dtype, device=self.dev))
         self._hook = None
+        self._cut_exception = None
 
         # ---- architecture + parameter table (torchvision naming and order) ----
         self._specs, self._bn_names = [], []
@@ -474,16 +475,27 @@ class ResNetEngine:
         (torch_col/colocate_ctrl.py:360-402).  An exception raised by fn ends the step there."""
         self._hook = fn
 
+    def set_cut_exception(self, exc_type):
+        """Raise exc_type from forward_backward when the reject flag cut the replay short (the
+        control thread killed the batch on receipt of a request): what the reference's autograd
+        engine hook does with EngineColocateAdjustL1Exception (csrc/mem_tagging.cc:54-58)."""
+        self._cut_exception = exc_type
+
     def _run_plan(self, p):
         if self._hook is None:
-            return self.ctx.run(p.prog)
-        first, cut = 0, False
-        for idx, phase, name in p.marks:
-            cut = self.ctx.run(p.prog, first, idx) or cut
-            first = idx
-            self._hook(phase, name)
-        if first < len(p.prog):
-            cut = self.ctx.run(p.prog, first, len(p.prog)) or cut
+            cut = self.ctx.run(p.prog)
+        else:
+            first, cut = 0, False
+            for idx, phase, name in p.marks:
+                cut = self.ctx.run(p.prog, first, idx) or cut
+                first = idx
+                self._hook(phase, name)
+                if cut and self._cut_exception is not None:
+                    break
+            if first < len(p.prog) and not (cut and self._cut_exception is not None):
+                cut = self.ctx.run(p.prog, first, len(p.prog)) or cut
+        if cut and self._cut_exception is not None:
+            raise self._cut_exception("launches rejected: batch killed on request")
         return cut
 
     # ------------------------------------------------------------------ the step

@@ -214,6 +214,7 @@ class _PoolBlock:
 
     def __init__(self, device, nbytes, stream):
         self.device, self.nbytes = device, nbytes
+        self.generation = lib().tch_pool_generation(device)
         self.ptr = lib().tch_pool_malloc(nbytes, device, stream)
         if not self.ptr:
             raise TorchColHipError(f"pool allocation of {nbytes} bytes failed: "
@@ -224,7 +225,9 @@ class _PoolBlock:
     def __del__(self):
         try:
             if self.ptr:
-                lib().tch_pool_free(self.ptr, self.nbytes, self.device, None)
+                # a block of a pool that has been shut down meanwhile went away with that pool
+                if lib().tch_pool_generation(self.device) == self.generation:
+                    lib().tch_pool_free(self.ptr, self.nbytes, self.device, None)
                 self.ptr = None
         except Exception:
             pass
@@ -255,10 +258,30 @@ def install_pluggable_allocator():
     CUDAColAllocator before the first allocation, csrc/torch_allocator_plugin.cc:31-58).
     Must run before torch allocates on the device."""
     import torch
-    from .._lib import LIB_PATH
-    alloc = torch.cuda.memory.CUDAPluggableAllocator(LIB_PATH, "tch_pool_malloc", "tch_pool_free")
+    alloc = pluggable_allocator()
     torch.cuda.memory.change_current_allocator(alloc)
     return alloc
+
+
+_pluggable = None
+
+
+def pluggable_allocator():
+    """torch's view of the pool's allocator hook (tch_pool_malloc / tch_pool_free)."""
+    global _pluggable
+    if _pluggable is None:
+        import torch
+        from .._lib import LIB_PATH
+        _pluggable = torch.cuda.memory.CUDAPluggableAllocator(LIB_PATH, "tch_pool_malloc", "tch_pool_free")
+    return _pluggable
+
+
+def torch_mem_pool():
+    """A torch.cuda.MemPool on the pool's allocator: inside `with torch.cuda.use_mem_pool(p):`
+    every torch allocation of this thread is a pool block, without replacing torch's allocator
+    for the whole process."""
+    import torch
+    return torch.cuda.MemPool(pluggable_allocator().allocator())
 
 
 # memory that is not model state and is dropped on a handover: engines register a callable that

@@ -274,10 +274,16 @@ class ColocateCtrl(CtrlBase):
                     _C.SyncAllStreams()
                     if self._adjust_l1_pending():
                         raise ColocateAdjustL1Exception('[Adjust SYNC BWD]')
+        elif self.hook_mode == ColocateCtrlHookMode.XSCHED_SYNC2:
+            # the control thread kills on receipt; the engine notices the rejected launches
+            print("SetUpTorchColEngine")
+            self._stub.EnableTorchColEngine()
+            for module in module_list:
+                if hasattr(module, "set_cut_exception"):
+                    module.set_cut_exception(EngineColocateAdjustL1Exception)
+                    _C.register_interm_memory_owner(module.release_activations)
+            return
         elif self.hook_mode.use_xsched():
-            if self.hook_mode == ColocateCtrlHookMode.XSCHED_SYNC2:
-                self._stub.EnableTorchColEngine()
-
             # one event per layer would swamp the log at 310 segments a step: the checks are silent
             def fwd_hook(module, input, output):
                 if self._adjust_l1_pending():

@@ -1,0 +1,206 @@
+"""Colocation path on the GPU: the HBM page pool on HIP virtual memory, the engine on pool
+memory, checkpoint hooks, and the 64 -> 16 -> 64 handover with an in-process peer.
+
+Bars: offsets and integer bookkeeping bit-exact against the CPU model of the pool; the engine on
+pool memory bit-exact against the engine on torch memory (same kernels, same inputs); handover
+request -> AdjustL1Done under 50 ms (BASELINE's bound for the path)."""
+import ctypes
+import os
+import random
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from sirius_amd._lib import lib
+
+pytestmark = pytest.mark.gpu
+MB = 1 << 20
+SMALL = dict(depths=(1, 1, 1, 1), width=16, num_classes=16, image_size=64)
+
+
+def _trace(L, seed, n=300):
+    rng = random.Random(seed)
+    live, offs = [], []
+    for _ in range(n):
+        r = rng.random()
+        if r < 0.55 or not live:
+            size = rng.choice([512, 4096, 100_000, MB, 3 * MB, 20 * MB, 40 * MB])
+            p = L.tch_pool_malloc(size, 0, None)
+            if p:
+                live.append(p)
+                offs.append(L.tch_pool_offset_of(0, p))
+            else:
+                offs.append(-1)
+        elif r < 0.95:
+            L.tch_pool_free(live.pop(rng.randrange(len(live))), 0, 0, None)
+        else:
+            offs.append(("ec", L.tch_cuda_memory_pool_free_train_local(0)))
+    for p in live:
+        L.tch_pool_free(p, 0, 0, None)
+    return offs
+
+
+@pytest.fixture()
+def clean_runtime(monkeypatch):
+    port = 50000 + os.getpid() % 10000
+    monkeypatch.setenv("SIRIUS_PORT", str(port))
+    for k in list(os.environ):
+        if k.startswith("COLTRAIN_"):
+            monkeypatch.delenv(k)
+    import sirius_amd.torch_col as tc
+    tc.torch_col_shutdown()
+    tc.reset_for_tests()
+    yield tc
+    tc.UnRegisterAllStreams()
+    tc.SetRejectCudaCalls(False)
+    tc.reset_for_tests()
+    tc.torch_col_shutdown()
+    for f in os.listdir("/dev/shm"):
+        if f.startswith(f"colserve_shm_{os.getuid()}_p{port}"):
+            os.unlink(os.path.join("/dev/shm", f))
+
+
+def test_pool_on_hip_vmm_matches_cpu_model(clean_runtime):
+    L = lib()
+    torch.cuda.init()
+    print("pool trace seed 11, 1 GB", flush=True)
+    assert L.tch_pool_init(0, 1024 * MB, 0) == 0
+    cpu = _trace(L, 11)
+    L.tch_pool_shutdown(0)
+    assert L.tch_pool_init(0, 1024 * MB, 1) == 0, L.tch_host_last_error()
+    try:
+        gpu = _trace(L, 11)
+        assert gpu == cpu
+        # memory is real: write through one mapping, keep it across an unmap of its neighbours
+        tc = clean_runtime
+        a = tc.pool_empty((8 * MB,), torch.uint8, device=0)
+        b = tc.pool_empty((40 * MB // 4,), torch.float32, device=0)
+        c = tc.pool_empty((3, 5, 7), torch.bfloat16, device=0)
+        a.fill_(7)
+        b.copy_(torch.arange(b.numel(), device="cuda", dtype=torch.float32))
+        c.fill_(1.5)
+        torch.cuda.synchronize()
+        used = L.tch_cuda_memory_pool_train_all_usage(0)
+        del b
+        freed = L.tch_cuda_memory_pool_free_train_local(0)
+        assert freed >= 32 * MB and L.tch_cuda_memory_pool_train_all_usage(0) == used - freed
+        assert int(a.sum().item()) == 7 * 8 * MB and float(c.float().sum()) == 1.5 * 105
+        b2 = tc.pool_empty((40 * MB // 4,), torch.float32, device=0)   # pages are mapped again
+        b2.fill_(2.0)
+        assert float(b2[-1].item()) == 2.0
+        del a, b2, c
+        assert L.tch_cuda_memory_pool_train_usage(0) == 0
+    finally:
+        torch.cuda.synchronize()
+        L.tch_pool_shutdown(0)
+
+
+def _one_step(engine, x, y):
+    plan, cut = engine.forward_backward(x, y)
+    assert not cut
+    engine.synchronize()
+    return float(plan.loss.item()), engine.grads.clone()
+
+
+def test_engine_on_pool_memory_is_bit_identical(clean_runtime):
+    from sirius_amd.resnet import ResNetEngine
+    tc = clean_runtime
+    L = lib()
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(8, 3, 64, 64, generator=g).cuda()
+    y = torch.randint(0, 16, (8,), generator=g).cuda()
+    ref = ResNetEngine(dtype=torch.bfloat16, **SMALL)
+    ref.init_kaiming(5)
+    loss0, g0 = _one_step(ref, x, y)
+    assert L.tch_pool_init(0, 1024 * MB, 1) == 0, L.tch_host_last_error()
+    try:
+        eng = ResNetEngine(dtype=torch.bfloat16, allocator=lambda s, d: tc.pool_empty(s, d, device=0), **SMALL)
+        eng.init_kaiming(5)
+        assert L.tch_cuda_memory_pool_train_usage(0) > 0
+        # a no-op checkpoint hook cuts the program into segments without changing it
+        seen = []
+        eng.set_checkpoint_hook(lambda phase, name: seen.append((phase, name)))
+        loss1, g1 = _one_step(eng, x, y)
+        assert loss1 == loss0 and torch.equal(g0, g1)
+        assert seen[0] == ("fwd", "bn1") and seen[-1][0] == "bwd" and ("fwd", "loss") in seen
+        before = L.tch_cuda_memory_pool_train_usage(0)
+        released = eng.release_activations()
+        assert released > 0 and L.tch_cuda_memory_pool_train_usage(0) <= before - released
+        del eng, g1
+    finally:
+        torch.cuda.synchronize()
+        L.tch_pool_shutdown(0)
+
+
+def _handover(tc, monkeypatch, tmp_path, hook_mode):
+    from sirius_amd.train import resnet152 as script
+    env = {"COLTRAIN_MODE": "colocate-l1", "COLTRAIN_HOOK_MODE": hook_mode, "COLTRAIN_USE_XSCHED": "1",
+           "COLTRAIN_HAS_INFER_SERVER": "1", "COLTRAIN_USE_SHARED_TENSOR": "1",
+           "COLTRAIN_SHARED_TENSOR_POOL_GB": "2", "COLTRAIN_PROFILE_LOG_PATH": str(tmp_path / "train-profile.csv")}
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    peer = script.PeerScript({3: ("l1", 16), 12: ("exit", 64)}, delay_ms=2.0)
+    sizes = []
+    orig = tc.Trainer.train_one_epoch
+    try:
+        out = script.train(1, 64, global_batch_size=None, dataset_size=64 * 8, dtype=torch.bfloat16,
+                           peer=peer, num_distinct_samples=64, **SMALL)
+    finally:
+        peer.stop()
+    return out, peer
+
+
+@pytest.mark.parametrize("hook_mode", ["xsched-sync", "xsched-sync2"])
+def test_handover_64_16_64_on_gpu(clean_runtime, monkeypatch, tmp_path, hook_mode, capsys):
+    tc = clean_runtime
+    print(f"handover {hook_mode}", flush=True)
+    out, peer = _handover(tc, monkeypatch, tmp_path, hook_mode)
+    trainer, model, ctrl = out["trainer"], out["model"], out["ctrl"]
+    stat = trainer.get_last_epoch_stat()
+    assert stat.finished_sample == 64 * 8                      # every sample trained exactly once
+    assert [k for _, k, _ in peer.sent] == ["l1", "exit"]
+    req, fin = tc.get_adjust_request_time_stamp(), tc.get_adjust_done_time_stamp()
+    assert len(req) == 1 and len(fin) == 1
+    latency_ms = (fin[0] - req[0]) / 1e3
+    print(f"adjust latency {latency_ms:.2f} ms, {ctrl.last_adjust}", flush=True)
+    assert 0 <= latency_ms < 50.0
+    assert ctrl.last_adjust["released_bytes"] > 0
+    import csv
+    rows = list(csv.DictReader(open(out["profile"])))
+    batches = [r["name"] for r in rows if r["name"].startswith("batch_0")]
+    sizes = [int(n.split("_")[-1]) for n in batches]
+    assert sizes[0] == 64 and 16 in sizes and sizes[-1] == 64  # 64 -> 16 -> 64
+    assert sum(s for r, s in zip([r for r in rows if r["name"].startswith("batch_0")], sizes)
+               if r["tag"] == "finish") == 64 * 8
+    sd = model.state_dict()
+    assert all(torch.isfinite(v).all() for v in sd.values())
+    assert tc.GetXQueueSizeAllStreams() == 0
+
+
+def test_torch_allocations_through_the_pool_hook(clean_runtime):
+    """torch's own allocations land in the pool through the allocator hook
+    (tch_pool_malloc / tch_pool_free in the shape torch's pluggable allocator binds; the
+    reference installs CUDAColAllocator for the same purpose, csrc/torch_allocator_plugin.cc:31-58).
+    Scoped with a torch MemPool so that the rest of the process keeps torch's allocator."""
+    tc = clean_runtime
+    L = lib()
+    if not hasattr(torch.cuda, "MemPool") or not hasattr(torch.cuda, "use_mem_pool"):
+        pytest.skip("this torch has no MemPool / use_mem_pool")
+    assert L.tch_pool_init(0, 512 * MB, 1) == 0, L.tch_host_last_error()
+    try:
+        pool = tc.torch_mem_pool()
+        with torch.cuda.use_mem_pool(pool):
+            a = torch.empty(1 << 20, device="cuda")
+            used = L.tch_cuda_memory_pool_train_usage(0)
+            assert used >= 4 * MB
+            assert L.tch_pool_offset_of(0, ctypes.c_void_p(a.data_ptr())) >= 0
+            a.fill_(3.0)
+            assert (a * 2).sum().item() == 6.0 * (1 << 20)
+        del a
+        torch.cuda.synchronize()
+        del pool
+    finally:
+        torch.cuda.synchronize()
+        L.tch_pool_shutdown(0)
