@@ -40,8 +40,58 @@ def cpu_baseline(batch, timed_steps):
             "sample": f"ResNet-152 fp32 batch {batch} @224, torch CPU oracle step, 1 warm-up + {timed_steps} timed steps"}
 
 
+def handover(batch):
+    """BASELINE configs[2]: ResNet-152 bf16 under the colocation protocol, global batch fixed at
+    `batch`; a stand-in inference peer asks for memory (target batch 16) during the 4th micro-batch
+    and leaves later (target back to `batch`).  Reports request -> AdjustL1Done as the server sees
+    it, split into wait (request received -> release starts) and release, and the bytes returned."""
+    import contextlib
+    import csv
+    import tempfile
+
+    import torch
+    from sirius_amd import torch_col
+    from sirius_amd.train import resnet152 as script
+
+    tmp = tempfile.mkdtemp(prefix="tch_bench_")
+    env = {"COLTRAIN_MODE": "colocate-l1", "COLTRAIN_HOOK_MODE": "xsched-sync", "COLTRAIN_USE_XSCHED": "1",
+           "COLTRAIN_HAS_INFER_SERVER": "1", "COLTRAIN_USE_SHARED_TENSOR": "1",
+           "COLTRAIN_SHARED_TENSOR_POOL_GB": "48", "COLTRAIN_PROFILE_LOG_PATH": os.path.join(tmp, "train-profile.csv"),
+           "SIRIUS_PORT": str(18000 + os.getpid() % 1000)}
+    os.environ.update(env)
+    peer = script.PeerScript({3: ("l1", 16), 14: ("exit", batch)}, delay_ms=8.0)
+    try:
+        with contextlib.redirect_stdout(sys.stderr):
+            out = script.train(1, batch, dataset_size=batch * 10, dtype=torch.bfloat16, peer=peer,
+                               num_distinct_samples=batch)
+    finally:
+        peer.stop()
+    req, fin = torch_col.get_adjust_request_time_stamp(), torch_col.get_adjust_done_time_stamp()
+    rows = list(csv.DictReader(open(out["profile"])))
+    adj = [r for r in rows if r["name"] == "adjust_l1"]
+    sizes = [int(r["name"].split("_")[-1]) for r in rows if r["name"].startswith("batch_0")]
+    stat = out["trainer"].get_last_epoch_stat()
+    res = {
+        "request_to_done_ms": (fin[0] - req[0]) / 1e3 if req and fin else None,
+        "wait_ms": float(adj[0]["timestamp"]) - req[0] / 1e3 if adj and req else None,
+        "release_ms": float(adj[0]["duration"]) if adj else None,
+        "stages_ms": {k: round(v, 3) for k, v in out["ctrl"].last_adjust.items() if k.endswith("_ms")},
+        "activation_bytes_released": out["ctrl"].last_adjust.get("released_bytes"),
+        "pool_bytes_returned": out["ctrl"].last_adjust.get("pool_bytes_returned"),
+        "micro_batch_sizes": sizes,
+        "killed_batches": stat.killed_batch,
+        "finished_samples": stat.finished_sample,
+        "bound_ms": 50.0,
+    }
+    del out
+    torch_col.reset_for_tests()
+    torch_col.torch_col_shutdown()
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--no-handover", action="store_true", help="skip the 64 -> 16 -> 64 handover measurement")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
@@ -144,6 +194,13 @@ def main():
         out["cpu_baseline"] = cpu_baseline(B, args.cpu_steps)
     else:
         out["cpu_baseline"] = None
+    if not args.no_handover:
+        del eng, plan, x, y
+        torch.cuda.empty_cache()
+        try:
+            out["handover"] = handover(B)
+        except Exception as e:  # the headline figure stands on its own; say what went wrong
+            out["handover"] = {"error": repr(e)}
     print(json.dumps(out), flush=True)
 
 

@@ -75,8 +75,13 @@ void tch_pool_free(void* ptr, ptrdiff_t nbytes, int device, void* hip_stream);
 void tch_pool_record_stream(void* ptr, int device, void* hip_stream); /* :200-229 */
 uint64_t tch_pool_process_events(int device);                          /* :383-412 */
 int64_t tch_pool_offset_of(int device, const void* ptr);
-/* counters: allocs, frees, maps, unmaps (4 x u64) */
-void tch_pool_counters(int device, uint64_t* out4);
+/* counters (6 x u64): allocs, frees, driver maps, driver unmaps, slots that got their page back
+ * without a driver call, stale mappings currently in place */
+void tch_pool_counters(int device, uint64_t* out6);
+/* FreeTrainLocals relabels pages and leaves their mappings in place (unmapping costs the driver
+ * ~0.24 ms per 32 MB page, which would dominate a handover); this removes up to max_pages of
+ * those stale mappings and returns how many it removed.  Never needed for correctness. */
+uint64_t tch_pool_trim(int device, uint64_t max_pages);
 /* the inference side as a fake peer needs it: label n FREE pages inference-owned / give back */
 int tch_pool_infer_claim_pages(int device, int n);
 int tch_pool_infer_release_pages(int device, int n);

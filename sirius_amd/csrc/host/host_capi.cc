@@ -145,15 +145,18 @@ void tch_pool_record_stream(void* ptr, int device, void* hip_stream) {
 }
 uint64_t tch_pool_process_events(int device) { return pool(device) ? pool(device)->process_events() : 0; }
 int64_t tch_pool_offset_of(int device, const void* ptr) { return pool(device) ? pool(device)->offset_of(ptr) : -1; }
-void tch_pool_counters(int device, uint64_t* out4) {
-  if (!out4) return;
+void tch_pool_counters(int device, uint64_t* out6) {
+  if (!out6) return;
   PoolStats s{};
   if (pool(device)) s = pool(device)->stats();
-  out4[0] = s.num_allocs;
-  out4[1] = s.num_frees;
-  out4[2] = s.num_maps;
-  out4[3] = s.num_unmaps;
+  out6[0] = s.num_allocs;
+  out6[1] = s.num_frees;
+  out6[2] = s.num_maps;
+  out6[3] = s.num_unmaps;
+  out6[4] = s.num_revives;
+  out6[5] = s.stale_pages;
 }
+uint64_t tch_pool_trim(int device, uint64_t max_pages) { return pool(device) ? pool(device)->trim(max_pages) : 0; }
 int tch_pool_infer_claim_pages(int d, int n) { return pool(d) ? pool(d)->infer_claim_pages(n) : 0; }
 int tch_pool_infer_release_pages(int d, int n) { return pool(d) ? pool(d)->infer_release_pages(n) : 0; }
 void tch_tag_model_start(int d) { if (pool(d)) pool(d)->tag_model_start(); }

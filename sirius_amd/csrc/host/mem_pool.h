@@ -15,9 +15,11 @@
 //     rest); inside a segment: best fit (smallest free block that fits, lowest offset on
 //     ties), split when the remainder is at least one alignment unit, coalesce on free,
 //     otherwise grow the segment at its end;
-//   * a freed block keeps its pages ("train-local free"); empty_cache() unmaps every page
-//     that lies wholly inside free blocks and hands it back as FREE;
-//   * physical pages are taken lowest index first.
+//   * a freed block keeps its pages ("train-local free"); empty_cache() hands every page that
+//     lies wholly inside free blocks back as FREE.  That is bookkeeping: the mapping stays in
+//     place (stale) and is reused if the page is still FREE when the range grows again;
+//   * physical pages are taken lowest index first, pages without a stale mapping before pages
+//     with one.
 // Offsets are therefore a pure function of the alloc / free / empty_cache sequence, and the
 // CPU model (NullBackend) and the GPU pool (HipVmmBackend) produce the same ones.
 #pragma once
@@ -84,6 +86,8 @@ struct PoolStats {
   size_t infer_usage;       // pages labelled inference x page size
   size_t free_pages;
   size_t num_allocs, num_frees, num_maps, num_unmaps;
+  size_t num_revives;   // slots that got their page back without a driver call
+  size_t stale_pages;   // mappings left in place over pages training no longer owns
 };
 
 class HbmPool {
@@ -97,6 +101,7 @@ class HbmPool {
   void record_stream(void* ptr, uint64_t stream);
   size_t process_events();  // reap deferred frees; returns how many blocks were released
   size_t empty_cache();     // FreeTrainLocals; returns bytes handed back as FREE pages
+  size_t trim(size_t max_pages);  // remove up to max_pages stale mappings; returns how many
   PoolStats stats();
   uint64_t base() const { return base_; }
   PoolBackend* backend() { return backend_.get(); }
@@ -139,7 +144,7 @@ class HbmPool {
   bool ensure_mapped(uint64_t off, size_t n, std::string* err);
   void free_block(Segment& s, uint64_t off);
   size_t empty_cache_locked();
-  int take_free_page();
+  int take_free_page(std::string* err);
 
   int device_ = 0;
   std::unique_ptr<PoolBackend> backend_;
@@ -147,7 +152,10 @@ class HbmPool {
   size_t pool_bytes_ = 0, va_bytes_ = 0;
   int num_pages_ = 0;
   std::vector<uint8_t> owner_;     // per physical page
-  std::vector<int> slot_page_;     // per VA slot: physical page or -1
+  std::vector<int> slot_page_;     // per VA slot: physical page mapped there, or -1
+  std::vector<uint8_t> slot_live_; // per VA slot: 1 while training owns the mapped page, 0 = stale mapping
+  std::vector<int64_t> page_slot_; // per physical page: the slot it is mapped at (live or stale), or -1
+  size_t n_revive_ = 0;
   Segment small_, large_;
   std::mutex mu_;
   size_t train_usage_ = 0, train_peak_ = 0;

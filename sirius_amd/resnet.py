@@ -466,8 +466,26 @@ class ResNetEngine:
     def release_activations(self):
         """Drop every plan (and with it all activation / gradient-scratch memory)."""
         n = sum(p.bytes for p in self._plans.values())
+        # an exception in flight may still hold a plan through its traceback: with an allocator
+        # that can release a block under a live tensor, give the memory back now
+        release = getattr(self._alloc, "release", None)
+        if release is not None:
+            self.ctx.synchronize()
+            for p in self._plans.values():
+                for t in p.keep:
+                    release(t)
+                p.keep = []
         self._plans.clear()
+        self._last_plan = None
         return n
+
+    def last_loss(self):
+        """Mean loss of the most recent micro-batch (nan once its plan has been released)."""
+        p = getattr(self, "_last_plan", None)
+        if p is None or not p.keep:
+            return float("nan")
+        self.ctx.synchronize()
+        return float(p.loss.item())
 
     def set_checkpoint_hook(self, fn):
         """fn(phase, layer name) runs between the launch segments of forward_backward, once per
@@ -501,7 +519,7 @@ class ResNetEngine:
     # ------------------------------------------------------------------ the step
     def forward_backward(self, x, y, loss_scale=1.0):
         """x [B,3,S,S] fp32 and y [B] int64 on the GPU.  Returns (plan, cut_short)."""
-        p = self.plan(x.shape[0], loss_scale)
+        p = self._last_plan = self.plan(x.shape[0], loss_scale)
         self.ctx.flush()
         p.x_in.copy_(x, non_blocking=True)
         p.labels.copy_(y, non_blocking=True)

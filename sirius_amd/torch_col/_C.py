@@ -222,15 +222,36 @@ class _PoolBlock:
         self.__cuda_array_interface__ = {"shape": (nbytes,), "typestr": "|u1", "data": (self.ptr, False),
                                          "version": 2, "strides": None}
 
+        _live_blocks[self.ptr] = weakref.ref(self)
+
+    def release(self):
+        """Give the block back now, whoever still holds a tensor over it (the holder must not
+        touch it again): ReleaseUnderlyingStorage of the reference (csrc/util.cc)."""
+        if self.ptr:
+            _live_blocks.pop(self.ptr, None)
+            # a block of a pool that has been shut down meanwhile went away with that pool
+            if lib().tch_pool_generation(self.device) == self.generation:
+                lib().tch_pool_free(self.ptr, self.nbytes, self.device, None)
+            self.ptr = None
+            return self.nbytes
+        return 0
+
     def __del__(self):
         try:
-            if self.ptr:
-                # a block of a pool that has been shut down meanwhile went away with that pool
-                if lib().tch_pool_generation(self.device) == self.generation:
-                    lib().tch_pool_free(self.ptr, self.nbytes, self.device, None)
-                self.ptr = None
+            self.release()
         except Exception:
             pass
+
+
+_live_blocks = {}
+
+
+def pool_release(tensor):
+    """Free the pool block under `tensor` at once (no-op for a tensor that is not the start of a
+    live pool block).  Returns the bytes released."""
+    ref = _live_blocks.get(tensor.data_ptr())
+    blk = ref() if ref is not None else None
+    return blk.release() if blk is not None else 0
 
 
 def pool_empty(shape, dtype, device=None):
@@ -251,6 +272,9 @@ def pool_empty(shape, dtype, device=None):
     blk = _PoolBlock(device, n * itemsize, stream)
     flat = torch.as_tensor(blk, device=f"cuda:{device}")
     return flat.view(dtype).view(shape)
+
+
+pool_empty.release = pool_release  # allocator protocol of the engines: allocator(shape, dtype), allocator.release(t)
 
 
 def install_pluggable_allocator():

@@ -97,7 +97,6 @@ def train(num_epoch: int, batch_size: int, global_batch_size: Optional[int] = No
           f'cached {MemoryPool.get_memory_usage()}', flush=True, file=sys.stderr)
 
     counter = {"n": 0}
-    losses = []
 
     def iter_train_fn(batch: dynamic_batch.Batch):
         if peer is not None:
@@ -107,14 +106,14 @@ def train(num_epoch: int, batch_size: int, global_batch_size: Optional[int] = No
         # loss /= global_batch_size / batch_size is folded into the loss kernel
         plan, _ = model.forward_backward(images, targets, loss_scale=batch_manager.loss_scale(batch))
         batch_manager.optimizer_step(batch, model, grad_accumulator=grad_accumulator)
-        losses.append(plan.loss)
+        # the loss stays on the GPU (no read-back per micro-batch): the epoch line reads the last one
         return 0.0
 
     trainer = torch_col.Trainer(model, iter_train_fn)
     for epoch in range(num_epoch):
         trainer.train_one_epoch(epoch)
         model.synchronize()
-        running_loss = float(losses[-1].item()) if losses else float('nan')
+        running_loss = model.last_loss()
         epoch_stat = trainer.get_last_epoch_stat()
         epoch_duration = trainer.get_last_epoch_duration()
         mem_info = f'mem {MemoryPool.get_memory_usage():.2f}Gb'

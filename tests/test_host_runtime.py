@@ -688,6 +688,46 @@ def test_pool_no_overlap_and_best_fit(fresh):
         L.tch_pool_shutdown(0)
 
 
+def _counters(L):
+    c = (ctypes.c_uint64 * 6)()
+    L.tch_pool_counters(0, c)
+    return dict(zip(("allocs", "frees", "maps", "unmaps", "revives", "stale"), (int(v) for v in c)))
+
+
+def test_pool_hands_pages_back_without_unmapping(fresh):
+    """Returning pages is bookkeeping: no driver unmap on the handover path; the mapping is reused
+    when the page is still free at regrowth, and replaced when inference has taken the page."""
+    L = fresh
+    assert L.tch_pool_init(0, 128 * MB, 0) == 0            # 4 pages
+    try:
+        a = L.tch_pool_malloc(64 * MB, 0, None)
+        assert _counters(L)["maps"] == 2
+        L.tch_pool_free(a, 0, 0, None)
+        assert L.tch_cuda_memory_pool_free_train_local(0) == 64 * MB
+        c = _counters(L)
+        assert c["unmaps"] == 0 and c["stale"] == 2
+        assert L.tch_cuda_memory_pool_num_free_pages(0) == 4 and L.tch_cuda_memory_pool_train_all_usage(0) == 0
+        # 64 -> 16 -> 64: the same range grows back over pages that are still free
+        a2 = L.tch_pool_malloc(64 * MB, 0, None)
+        assert a2 == a
+        c = _counters(L)
+        assert c["maps"] == 2 and c["unmaps"] == 0 and c["revives"] == 2 and c["stale"] == 0
+        L.tch_pool_free(a2, 0, 0, None)
+        L.tch_cuda_memory_pool_free_train_local(0)
+        # inference takes three of the four pages, among them the two with stale mappings
+        assert L.tch_pool_infer_claim_pages(0, 3) == 3
+        b = L.tch_pool_malloc(32 * MB, 0, None)            # slot 0 again: its old page is gone
+        assert b == a
+        c = _counters(L)
+        assert c["unmaps"] == 1 and c["maps"] == 3 and c["stale"] == 1
+        assert L.tch_pool_malloc(64 * MB, 0, None) is None  # nothing left
+        assert L.tch_pool_trim(0, 100) == 1 and _counters(L)["stale"] == 0
+        L.tch_pool_free(b, 0, 0, None)
+        assert L.tch_pool_infer_release_pages(0, 3) == 3
+    finally:
+        L.tch_pool_shutdown(0)
+
+
 def test_pool_cross_stream_free_is_deferred(fresh):
     """A block used on another stream is only reusable once that stream's event has finished
     (csrc/torch_allocator_plugin.cc:141-178,383-412); recording the block's own stream is
