@@ -92,6 +92,9 @@ def handover(batch):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--no-handover", action="store_true", help="skip the 64 -> 16 -> 64 handover measurement")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also launch accumulate_kernel once over two 512 MiB buffers (reads 1 GiB, writes 1 GiB): "
+                         "the known-size dispatch that scales FETCH_SIZE / WRITE_SIZE counter readings")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
@@ -121,6 +124,14 @@ def main():
     def step():
         eng.forward_backward(x, y)
         eng.optimizer_step()
+
+    if args.calibrate:
+        from sirius_amd import ops
+        a = torch.zeros(128 << 20, device="cuda")
+        b = torch.ones(128 << 20, device="cuda")
+        ops.grad_accumulate(eng.ctx, a, b)
+        torch.cuda.synchronize()
+        del a, b
 
     for _ in range(args.warmup):
         step()

@@ -36,6 +36,25 @@ class DebugServer:
     def infer_exit(self, batch_size: int):
         return self._send(CtrlEvent.kInferExit, batch_size)
 
+    # -- requests in megabytes, through the server's own arithmetic (server/train_adjuster.cc)
+    def require_memory_mb(self, required_mem_mb: float, adjuster=None):
+        """Inference needs required_mem_mb more: shrink training by ceil(MB / slope) samples."""
+        from .train_adjuster import TrainAdjuster
+        adjuster = adjuster or TrainAdjuster()
+        target = adjuster.infer_require_mem_adjust_plan(required_mem_mb)
+        if target is None:
+            return None
+        self.colocate_l1(target)
+        return target
+
+    def release_memory_mb(self, avail_mem_mb: float, adjuster=None):
+        """Inference left avail_mem_mb to training: grow to what fits (at most the initial size)."""
+        from .train_adjuster import TrainAdjuster
+        adjuster = adjuster or TrainAdjuster()
+        target = adjuster.infer_release_mem_adjust_plan(avail_mem_mb)
+        self.infer_exit(target)
+        return target
+
     def _recv_from_train(self):
         while self._running:
             msg = self._inf_tra_comm.timed_get_tra2inf(10, 0)

@@ -278,43 +278,41 @@ def test_distributor_truncates_last_global_batch(fresh):
     assert L.tch_distributor_get_num_proced_global_batch() == 2
 
 
-class _Model:
-    """Independent statement of the single-rank rules: an ordered set of unprocessed ranges,
-    GetBatch takes from the lowest index and slices the last range it touches; abort puts the
-    ranges back as they are (the reference never merges neighbours: csrc/dynamic_batch.cc:533-563);
-    the batch that empties the unprocessed set is the stepping one."""
+from oracle.host import DistributorModel as _Model  # noqa: E402  (the independent restatement)
+from oracle.host import PerfModelOracle, split_global_batch  # noqa: E402
 
-    def __init__(self, lo, hi):
-        self.unproc = [(lo, hi)] if hi > lo else []
-        self.procing, self.proced = [], []
 
-    def get(self, bs):
-        out, need = [], bs
-        while need > 0 and self.unproc:
-            a, b = self.unproc[0]
-            take = min(need, b - a)
-            out.append((a, a + take))
-            need -= take
-            if a + take == b:
-                self.unproc.pop(0)
-            else:
-                self.unproc[0] = (a + take, b)
-        self.procing += out
-        return out, not self.unproc
+def test_perf_model_against_restatement(fresh):
+    L = fresh
+    assert L.tch_TorchColInit(0, 1, 0) == 0
+    L.tch_perf_model_clear()
+    rng, ref = random.Random(9), PerfModelOracle()
+    for _ in range(40):
+        bs, ms = rng.choice([4, 8, 16, 24, 64]), rng.uniform(5, 200)
+        L.tch_perf_model_record_thpt(bs, ms)
+        ref.record(bs, ms)
+    for bs in range(-2, 100):
+        assert L.tch_perf_model_get_thpt(bs) == pytest.approx(ref.get(bs), rel=1e-12, abs=1e-15)
 
-    @staticmethod
-    def _merge(rs):
-        return sorted(rs)
 
-    def finish(self, r):
-        for x in r:
-            self.procing.remove(x)
-        self.proced = self._merge(self.proced + r)
-
-    def abort(self, r):
-        for x in r:
-            self.procing.remove(x)
-        self.unproc = self._merge(self.unproc + r)
+def test_adjust_arithmetic_of_the_peer():
+    """server/train_adjuster.cc:69-145,521-538 by hand: ResNet-152, (base, slope) = (1150, 85)."""
+    from oracle import host
+    base, slope = host.MODEL_MEM_PARAM_SHARED["resnet152"]
+    assert host.predict_train_mem_usage_mb(base, slope, 64) == 1150 + 85 * 64
+    assert host.predict_train_mem_usage_mb(base, slope, 0) == 1150
+    assert host.delta_batch_size(slope, 4080) == 48          # 4080 / 85 = 48 exactly
+    assert host.delta_batch_size(slope, 4081) == 49          # ceil
+    assert host.predict_target_batch_size(base, slope, 1150 + 85 * 16 + 84, 64) == 16   # floor
+    assert host.predict_target_batch_size(base, slope, 100, 64) == 0
+    assert host.predict_target_batch_size(base, slope, 1e6, 64) == 64
+    assert host.infer_require_mem_target(64, 4080, slope) == 16
+    assert host.infer_require_mem_target(0, 4080, slope) is None
+    assert host.infer_require_mem_target(64, 0, slope) is None
+    assert host.infer_require_mem_target(8, 4080, slope, min_train_bs=1, num_gpus=2) == 1
+    assert split_global_batch(21, 2) == [11, 10]
+    assert split_global_batch(21, 2, "by_performance", [1.0, 1.0]) == [11, 10]
+    assert sum(split_global_batch(64, 3, "by_performance", [3.0, 1.0, 0.01])) == 64
 
 
 @pytest.mark.parametrize("seed", range(6))

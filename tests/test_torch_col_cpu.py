@@ -148,7 +148,8 @@ def test_handover_64_16_64(colocate_env, capsys):
             # global batch 2 (third call), in the middle of backward: inference asks for memory
             if state["n"] == 3 and phase == "bwd" and i == 5 and not state.get("sent"):
                 state["sent"] = True
-                server.colocate_l1(16)
+                # 4080 MB at 85 MB per sample (server/train_adjuster.cc:535-538,658) = 48 samples less
+                assert server.require_memory_mb(4080) == 16
                 for _ in range(2000):
                     if ctrl._stub.cmd == tc.CtrlEvent.kColocateAdjustL1:
                         break
@@ -159,7 +160,7 @@ def test_handover_64_16_64(colocate_env, capsys):
         def iter_train_fn(batch):
             state["n"] += 1
             if state["n"] == 9:                        # later: inference leaves
-                server.infer_exit(64)
+                assert server.release_memory_mb(1150 + 85 * 64 + 10) == 64
             sizes.append(len(batch))
             scales.append(mgr.loss_scale(batch))
             loss = engine.forward_backward(len(batch))
