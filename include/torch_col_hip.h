@@ -45,6 +45,15 @@ int tch_context_create(void* hip_stream, tch_context** out);
 void tch_context_destroy(tch_context* ctx);
 /* launches skipped since the last call because the reject flag was up */
 uint64_t tch_context_take_rejected(tch_context* ctx);
+/* While recording: launches are stamped with `lane` (0 = the context's stream, 1 = may run beside
+ * lane 0 on a second stream of the same priority); with wait_main the next lane-1 launch first
+ * waits for everything lane 0 was given before it.  tch_context_join records the point where
+ * lane 0 waits for lane 1.  A program stays a valid serial order: behind a registered
+ * (preemptible) stream and under tch_program_profile it runs on one stream, in order.
+ * No counterpart in the reference (its backward runs on one stream). */
+int tch_context_set_lane(tch_context* ctx, int lane, int wait_main);
+int tch_context_join(tch_context* ctx);
+int tch_context_synchronize(tch_context* ctx); /* both streams of the context */
 
 /* ---- programs: record once, replay every step ---------------------------------- */
 int tch_program_create(tch_program** out);

@@ -44,6 +44,32 @@ void tch_context_destroy(tch_context* ctx) { delete ctx; }
 
 uint64_t tch_context_take_rejected(tch_context* ctx) { return ctx ? ctx->ctx.rejected.exchange(0) : 0; }
 
+int tch_context_set_lane(tch_context* ctx, int lane, int wait_main) {
+  if (!ctx || (lane != 0 && lane != 1)) {
+    set_error("tch_context_set_lane: lane must be 0 or 1");
+    return -22;
+  }
+  ctx->ctx.lane = lane;
+  ctx->ctx.wait_main = lane == 1 && wait_main != 0;
+  return 0;
+}
+
+int tch_context_join(tch_context* ctx) {
+  if (!ctx) {
+    set_error("tch_context_join: null context");
+    return -22;
+  }
+  return ctx->ctx.record_join();
+}
+
+int tch_context_synchronize(tch_context* ctx) {
+  if (!ctx) {
+    set_error("tch_context_synchronize: null context");
+    return -22;
+  }
+  return ctx->ctx.synchronize();
+}
+
 int tch_program_create(tch_program** out) {
   if (!out) {
     set_error("tch_program_create: null output");
@@ -76,6 +102,8 @@ int tch_program_end_record(tch_context* ctx) {
     return -22;
   }
   ctx->ctx.recording = nullptr;
+  ctx->ctx.lane = 0;
+  ctx->ctx.wait_main = false;
   return 0;
 }
 

@@ -201,14 +201,83 @@ void LaunchQueue::worker_loop() {
 // Context
 // ---------------------------------------------------------------------------
 
+Context::~Context() {
+  if (side) {
+    (void)hipStreamSynchronize(side);
+    (void)hipStreamDestroy(side);
+  }
+  for (hipEvent_t e : events_) (void)hipEventDestroy(e);
+}
+
+hipEvent_t Context::next_event() {
+  constexpr size_t kRing = 64;
+  if (events_.size() < kRing) {
+    hipEvent_t e = nullptr;
+    if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess) return nullptr;
+    events_.push_back(e);
+    return e;
+  }
+  return events_[event_next_++ % kRing];
+}
+
+int Context::record_join() {
+  if (!recording) return 0;
+  LaunchRecord rec{};
+  rec.fn = nullptr;
+  rec.name = "join";
+  rec.op = kOpJoin;
+  recording->launches.push_back(rec);
+  return 0;
+}
+
+int Context::synchronize() {
+  if (side && hipStreamSynchronize(side) != hipSuccess) {
+    set_error("side stream synchronize failed");
+    return -5;
+  }
+  if (hipStreamSynchronize(stream) != hipSuccess) {
+    set_error("stream synchronize failed");
+    return -5;
+  }
+  side_dirty = false;
+  return 0;
+}
+
 int Context::dispatch(const LaunchRecord& rec) {
   if (g_reject.load(std::memory_order_acquire)) {
-    rejected.fetch_add(1);
+    if (rec.fn) rejected.fetch_add(1);
     return 0;
   }
   if (queue) {
-    queue->submit(rec);
+    // behind the preemptible queue everything runs in program order on the one registered stream
+    if (rec.fn) queue->submit(rec);
     return 0;
+  }
+  if (rec.op == kOpJoin) {
+    if (side_dirty) {
+      hipEvent_t e = next_event();
+      if (!e || hipEventRecord(e, side) != hipSuccess || hipStreamWaitEvent(stream, e, 0) != hipSuccess) {
+        set_error("join of the side stream failed");
+        return -5;
+      }
+      side_dirty = false;
+    }
+    return 0;
+  }
+  if (rec.lane == 1) {
+    if (!side && hipStreamCreateWithFlags(&side, hipStreamNonBlocking) != hipSuccess) {
+      set_error("hipStreamCreateWithFlags failed");
+      return -5;
+    }
+    if (rec.op == kOpLaunchAfter) {
+      hipEvent_t e = next_event();
+      if (!e || hipEventRecord(e, stream) != hipSuccess || hipStreamWaitEvent(side, e, 0) != hipSuccess) {
+        set_error("fork to the side stream failed");
+        return -5;
+      }
+    }
+    side_dirty = true;
+    return launch_now(side, rec);
   }
   return launch_now(stream, rec);
 }
@@ -232,6 +301,15 @@ int submit(Context* ctx, const void* fn, dim3 grid, dim3 block, const void* args
   rec.work = work;
   rec.work_is_bytes = work_is_bytes;
   memcpy(rec.args, args, arg_bytes);
+  rec.lane = 0;
+  rec.op = kOpLaunch;
+  if (ctx->recording && ctx->lane == 1) {
+    rec.lane = 1;
+    if (ctx->wait_main) {
+      rec.op = kOpLaunchAfter;
+      ctx->wait_main = false;
+    }
+  }
   if (ctx->recording) {
     ctx->recording->launches.push_back(rec);
     return 0;
@@ -261,7 +339,8 @@ int profile_program(Context* ctx, const Program& prog, int reps, std::vector<Ker
     // one event between any two launches: launch i runs between ev[i] and ev[i+1]
     (void)hipEventRecord(ev[0], ctx->stream);
     for (size_t i = 0; i < n && rc == 0; ++i) {
-      rc = launch_now(ctx->stream, prog.launches[i]);
+      // everything on the one stream, in program order: lanes only matter for a plain replay
+      if (prog.launches[i].fn) rc = launch_now(ctx->stream, prog.launches[i]);
       (void)hipEventRecord(ev[i + 1], ctx->stream);
     }
     if (hipStreamSynchronize(ctx->stream) != hipSuccess) {
@@ -272,6 +351,7 @@ int profile_program(Context* ctx, const Program& prog, int reps, std::vector<Ker
       float ms = 0.f;
       (void)hipEventElapsedTime(&ms, ev[i], ev[i + 1]);
       const LaunchRecord& l = prog.launches[i];
+      if (!l.fn) continue;
       KernelStat& k = agg[l.name ? l.name : "kernel"];
       k.name = l.name ? l.name : "kernel";
       k.total_ms += ms;

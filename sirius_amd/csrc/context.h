@@ -95,7 +95,17 @@ struct Program {
 class Context {
  public:
   explicit Context(hipStream_t s) : stream(s) {}
+  ~Context();
   hipStream_t stream;
+  // second stream (default priority) for lane-1 launches of a replayed program; made on first use
+  hipStream_t side = nullptr;
+  bool side_dirty = false;  // lane 1 was given work since the last join
+  // recording state: the lane new launches are stamped with, and whether the next lane-1 launch
+  // has to wait for lane 0
+  int lane = 0;
+  bool wait_main = false;
+  int record_join();
+  int synchronize();  // both streams
   // set while the stream is registered for preemption; owned by the registry
   std::shared_ptr<LaunchQueue> queue;
   Program* recording = nullptr;
@@ -103,6 +113,11 @@ class Context {
   std::atomic<uint64_t> rejected{0};
 
   int dispatch(const LaunchRecord& rec);
+
+ private:
+  hipEvent_t next_event();
+  std::vector<hipEvent_t> events_;
+  size_t event_next_ = 0;
 };
 
 struct KernelStat {

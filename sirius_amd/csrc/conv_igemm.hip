@@ -589,6 +589,257 @@ __global__ __launch_bounds__(WM* WN * 64) void wgrad_kernel(IgemmArgs p) {
   });
 }
 
+// ---------------------------------------------------------------------------
+// forward / data gradient, bf16, channel counts that are multiples of 64
+// ---------------------------------------------------------------------------
+// Same GEMM view as igemm_kernel, restructured around what gfx950 offers:
+//   * operand tiles go from global memory straight into LDS (buffer_load ... lds, 16 bytes
+//     per lane, out-of-range offsets land as zeros): no staging registers, no LDS stores;
+//   * one reduction step is 64 elements = one 128-byte LDS row per GEMM row, unpadded, with
+//     the 16-byte slot index XOR-ed by (row >> 1) & 7 so that a 16-lane group of an MFMA
+//     operand read touches every bank once;
+//   * a step never straddles a filter tap (channels % 64 == 0), so the tap walk is scalar:
+//     a lane keeps one byte offset and one validity bit per tap for each row it loads;
+//   * NBUF tiles in flight, one barrier per step.
+constexpr int kStep2 = 64;                  // reduction elements per step
+constexpr int kRowBytes2 = kStep2 * 2;      // 128
+
+typedef __attribute__((address_space(3))) void* lds_void_ptr;
+
+// 16 bytes per lane from `rsrc` at byte offset voff (+ the wave-uniform soff) to dst + lane*16 in
+// LDS; an offset outside the resource stores zeros.  (Kept in a device function: named directly
+// in a kernel body, the builtin makes the host pass drop the kernel's launch stub.)
+__device__ inline void load_to_lds(__amdgpu_buffer_rsrc_t rsrc, unsigned char* dst, int voff, int soff) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)dst, 16, voff, soff, 0, 0);
+}
+
+template <int MODE, int WM, int WN, int TM, int TN, int NBUF>
+__global__ __launch_bounds__(WM* WN * 64) void igemm2_kernel(IgemmArgs p) {
+  using T = bf16;
+  constexpr int E = 8;
+  constexpr int BM = WM * TM * 32;
+  constexpr int BN = WN * TN * 32;
+  constexpr int NW = WM * WN;
+  constexpr int A_LD = BM / 8 / NW;  // direct loads per wave and step for the activation tile (8 rows each)
+  constexpr int B_LD = BN / 8 / NW;
+  static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile/loader mismatch");
+  constexpr int A_BYTES = BM * kRowBytes2, B_BYTES = BN * kRowBytes2;
+  constexpr int BUF_BYTES = A_BYTES + B_BYTES;
+  constexpr int STAGE_BYTES = WM * 32 * (BN + kStagePad) * 4;
+  constexpr int LDS_BYTES = NBUF * BUF_BYTES > STAGE_BYTES ? NBUF * BUF_BYTES : STAGE_BYTES;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[LDS_BYTES];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+
+  uint32_t id = xcd_remap(blockIdx.x, gridDim.x);
+  const int tile_m = id / p.tiles_n;
+  const int tile_n = id - tile_m * p.tiles_n;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  const int in_h = (MODE == kFwd) ? p.H : p.Ho;
+  const int in_w = (MODE == kFwd) ? p.W : p.Wo;
+  const int in_c = (MODE == kFwd) ? p.C : p.K;
+  const int cblocks = in_c / kStep2;
+  const int nk = p.R * p.S * cblocks;
+  const int sl = p.stride_log2, sm = p.stride - 1;
+
+  // ---- per lane: the rows it feeds, their byte offset at tap (0,0) and which taps exist ----
+  const int sub_row = lane >> 3, slot = lane & 7;
+  int a_off[A_LD];
+  uint32_t a_taps[A_LD];
+#pragma unroll
+  for (int j = 0; j < A_LD; ++j) {
+    const int trow = (wave * A_LD + j) * 8 + sub_row;
+    const int chunk = slot ^ ((trow >> 1) & 7);
+    const int row = m0 + trow;
+    uint32_t img = 0, pix = 0, oh = 0, ow = 0, taps = 0;
+    int base = 0;
+    if (row < p.gemm_m) {
+      p.div_plane.divmod(static_cast<uint32_t>(row), img, pix);
+      p.div_width.divmod(pix, oh, ow);
+      if (MODE == kFwd) {
+        const int h0 = static_cast<int>(oh) * p.stride - p.pad, w0 = static_cast<int>(ow) * p.stride - p.pad;
+        base = ((static_cast<int>(img) * in_h + h0) * in_w + w0) * in_c;
+        for (int r = 0; r < p.R; ++r)
+          for (int s = 0; s < p.S; ++s)
+            if (static_cast<unsigned>(h0 + r) < static_cast<unsigned>(in_h) &&
+                static_cast<unsigned>(w0 + s) < static_cast<unsigned>(in_w))
+              taps |= 1u << (r * p.S + s);
+      } else {
+        const int hp = static_cast<int>(oh) + p.pad, wp = static_cast<int>(ow) + p.pad;
+        base = ((static_cast<int>(img) * in_h + (hp >> sl)) * in_w + (wp >> sl)) * in_c;
+        for (int r = 0; r < p.R; ++r)
+          for (int s = 0; s < p.S; ++s) {
+            const int th = hp - r, tw = wp - s;
+            if (th >= 0 && tw >= 0 && (th & sm) == 0 && (tw & sm) == 0 && (th >> sl) < in_h && (tw >> sl) < in_w)
+              taps |= 1u << (r * p.S + s);
+          }
+      }
+    }
+    a_off[j] = (base + chunk * E) * 2;
+    a_taps[j] = taps;
+  }
+  int b_off[B_LD];
+#pragma unroll
+  for (int j = 0; j < B_LD; ++j) {
+    const int trow = (wave * B_LD + j) * 8 + sub_row;
+    const int chunk = slot ^ ((trow >> 1) & 7);
+    const int row = n0 + trow;
+    b_off[j] = row < p.gemm_n ? (row * p.gemm_k + chunk * E) * 2 : static_cast<int>(kOutOfRange);
+  }
+
+  const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(p.a_src, p.a_bytes);
+  const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(p.b_src, p.b_bytes);
+
+  // scalar walk over (tap, channel block)
+  int ld_r = 0, ld_s = 0, ld_cb = 0, ld_t = 0, ld_kt = 0;
+  auto issue_loads = [&](int buf) {
+    // element offset of this tap relative to tap (0,0), then bytes
+    const int tap_elems = (MODE == kFwd) ? (ld_r * in_w + ld_s) * in_c : -((ld_r >> sl) * in_w + (ld_s >> sl)) * in_c;
+    const int a_step = (tap_elems + ld_cb * kStep2) * 2;
+    const int b_step = ld_kt * kRowBytes2;
+    unsigned char* dst_a = lds + buf * BUF_BYTES + wave * A_LD * 1024;
+    unsigned char* dst_b = lds + buf * BUF_BYTES + A_BYTES + wave * B_LD * 1024;
+#pragma unroll
+    for (int j = 0; j < A_LD; ++j) {
+      const bool ok = (a_taps[j] >> ld_t) & 1u;
+      const int off = ok ? a_off[j] + a_step : static_cast<int>(kOutOfRange);
+      load_to_lds(rsrc_a, dst_a + j * 1024, off, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < B_LD; ++j)
+      load_to_lds(rsrc_b, dst_b + j * 1024, b_off[j], b_step);
+    ++ld_kt;
+    if (++ld_cb == cblocks) {
+      ld_cb = 0;
+      ++ld_t;
+      if (++ld_s == p.S) {
+        ld_s = 0;
+        ++ld_r;
+      }
+    }
+  };
+
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  // operand reads: row = tile row of the lane, slot = chunk ^ ((row >> 1) & 7); the tile bases are
+  // multiples of 32 rows, so the swizzle term depends on the lane only
+  const int frag_row = lane & 31, frag_half = lane >> 5;
+  const int swz = (frag_row >> 1) & 7;
+  const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
+  const uint32_t a_rd = lds_base + (wm * TM * 32 + frag_row) * kRowBytes2 + swz * 16;
+  const uint32_t b_rd = lds_base + A_BYTES + (wn * TN * 32 + frag_row) * kRowBytes2 + swz * 16;
+  // The operand reads are written as asm: the compiler orders every LDS read it can see behind
+  // ALL outstanding direct-to-LDS loads (vmcnt(0)), which would serialise the prefetch of the
+  // next tiles with the multiply of this one.  Which loads must have landed is known here (the
+  // counted wait + barrier at the top of a step), so the reads carry their own lgkmcnt waits.
+  auto read_frags = [&](int buf, int kk, uint4_t* fa, uint4_t* fb) {
+    const uint32_t cx = (2 * kk + frag_half) * 16;
+    const uint32_t pa = (a_rd ^ cx) + buf * BUF_BYTES, pb = (b_rd ^ cx) + buf * BUF_BYTES;
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fa[tm]) : "v"(pa), "n"(tm * 32 * kRowBytes2));
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn)
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fb[tn]) : "v"(pb), "n"(tn * 32 * kRowBytes2));
+  };
+  auto multiply = [&](uint4_t* fa, uint4_t* fb) {
+    // ties the registers to the wait that precedes this call in program order
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) asm volatile("" : "+v"(fa[tm]));
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) asm volatile("" : "+v"(fb[tn]));
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+        acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fb[tn]),
+                                                              __builtin_bit_cast(bf16x8_t, fa[tm]), acc[tm][tn], 0, 0, 0);
+  };
+  auto compute = [&](int buf) {
+    uint4_t fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+    read_frags(buf, 0, fa0, fb0);
+    read_frags(buf, 1, fa1, fb1);
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(TM + TN));
+    multiply(fa0, fb0);
+    read_frags(buf, 2, fa0, fb0);
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(TM + TN));
+    multiply(fa1, fb1);
+    read_frags(buf, 3, fa1, fb1);
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(TM + TN));
+    multiply(fa0, fb0);
+    asm volatile("s_waitcnt lgkmcnt(0)");
+    multiply(fa1, fb1);
+  };
+
+  // vmcnt(n): at most n of this wave's loads still in flight (gfx9 encoding, nothing else waited for)
+  constexpr int LOADS = A_LD + B_LD;
+  constexpr int AHEAD = (NBUF - 2) * LOADS;
+  constexpr int WAIT_IMM = (AHEAD & 0xF) | ((AHEAD >> 4) << 14) | (0x7 << 4) | (0xF << 8);
+  static_assert(AHEAD < 64, "vmcnt range");
+
+#pragma unroll
+  for (int s = 0; s < NBUF - 1; ++s)
+    if (s < nk) issue_loads(s);
+  for (int kt0 = 0; kt0 < nk; kt0 += NBUF) {
+#pragma unroll
+    for (int u = 0; u < NBUF; ++u) {
+      const int kt = kt0 + u;
+      if (kt < nk) {
+        // tile kt has landed for this wave once only the newer tiles' loads are outstanding; near the
+        // end fewer newer tiles exist, so wait for everything
+        if (kt + NBUF - 1 <= nk)
+          __builtin_amdgcn_s_waitcnt(WAIT_IMM);
+        else
+          __builtin_amdgcn_s_waitcnt((0x7 << 4) | (0xF << 8));
+        __syncthreads();  // every wave's part of tile kt is in LDS, and every wave is done with tile kt-1
+        if (kt + NBUF - 1 < nk) issue_loads((u + NBUF - 1) % NBUF);
+        compute(u);
+      }
+    }
+  }
+
+  staged_epilogue<T, WM, WN, TM, TN>(acc, reinterpret_cast<float*>(lds), tid, [&](int tr, int tc, float* v) {
+    const int row = m0 + tr, col = n0 + tc;
+    if (row >= p.gemm_m || col >= p.gemm_n) return;
+    const int64_t idx = static_cast<int64_t>(row) * p.gemm_n + col;
+    if (MODE == kFwd && p.bias) {
+#pragma unroll
+      for (int e = 0; e < E; ++e) v[e] += p.bias[col + e];
+    }
+    if (p.add) {
+      Chunk ca;
+      ca.u = *reinterpret_cast<const uint4*>(static_cast<const T*>(p.add) + idx);
+      float a[E];
+      chunk_to_float<T>(ca, a);
+      if (p.mask) {
+        Chunk cm;
+        cm.u = *reinterpret_cast<const uint4*>(static_cast<const T*>(p.mask) + idx);
+        float m[E];
+        chunk_to_float<T>(cm, m);
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+          if (!(m[e] > 0.f)) a[e] = 0.f;
+      }
+#pragma unroll
+      for (int e = 0; e < E; ++e) v[e] += a[e];
+    }
+    if (p.out_f32)
+      store_floats<E>(static_cast<float*>(p.out) + idx, v);
+    else
+      *reinterpret_cast<uint4*>(static_cast<T*>(p.out) + idx) = float_to_chunk<T>(v).u;
+  });
+}
+
 struct ReduceArgs {
   const float* partial;
   float* out;
@@ -652,8 +903,43 @@ int launch_cfg(Context* ctx, IgemmArgs& a, double flops) {
                   flops, 0);
 }
 
+template <int MODE, int WM, int WN, int TM, int TN, int NBUF>
+int launch_cfg2(Context* ctx, IgemmArgs& a, double flops) {
+  constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+  static const std::string name = std::string("igemm2_kernel<bf16,") + (MODE == kFwd ? "fwd," : "dgrad,") +
+                                  std::to_string(BM) + "x" + std::to_string(BN) + "," + std::to_string(NBUF) + "buf>";
+  a.tiles_m = (a.gemm_m + BM - 1) / BM;
+  a.tiles_n = (a.gemm_n + BN - 1) / BN;
+  int64_t wgs = static_cast<int64_t>(a.tiles_m) * a.tiles_n;
+  if (wgs <= 0 || wgs > 0x7fffffff) {
+    set_error("igemm: grid out of range");
+    return -22;
+  }
+  return launch(ctx, igemm2_kernel<MODE, WM, WN, TM, TN, NBUF>, dim3(static_cast<unsigned>(wgs)), dim3(WM * WN * 64), a,
+                name.c_str(), flops, 0);
+}
+
+// TCH_IGEMM2 = 0 keeps every convolution on igemm_kernel; 2 or 3 picks the number of LDS tiles
+// in flight of igemm2_kernel (default: 2 for 128x128, 3 for 128x64)
+int igemm2_setting() {
+  static const int v = [] {
+    const char* e = getenv("TCH_IGEMM2");
+    return e ? atoi(e) : -1;
+  }();
+  return v;
+}
+
 template <typename T, int MODE>
 int launch_mode(Context* ctx, IgemmArgs& a, int tile_cfg, double flops) {
+  if constexpr (sizeof(T) == 2 && (MODE == kFwd || MODE == kDgrad)) {
+    const int in_c = MODE == kFwd ? a.C : a.K;
+    const int setting = igemm2_setting();
+    if (setting != 0 && in_c % kStep2 == 0 && a.R * a.S <= 32 && (tile_cfg == 0 || tile_cfg == 1)) {
+      if (tile_cfg == 0)
+        return setting == 3 ? launch_cfg2<MODE, 2, 2, 2, 2, 3>(ctx, a, flops) : launch_cfg2<MODE, 2, 2, 2, 2, 2>(ctx, a, flops);
+      return setting == 2 ? launch_cfg2<MODE, 2, 2, 2, 1, 2>(ctx, a, flops) : launch_cfg2<MODE, 2, 2, 2, 1, 3>(ctx, a, flops);
+    }
+  }
   switch (tile_cfg) {
     case 0:
       return launch_cfg<T, MODE, 2, 2, 2, 2>(ctx, a, flops);  // 128 x 128
@@ -793,7 +1079,11 @@ int conv2d_wgrad_pick_splits(const ConvShape& s, int dtype) {
   const int gemm_m = s.K, gemm_n = s.R * s.S * s.C;
   int64_t tiles = tiles_for(gemm_m, gemm_n, 128, 128);
   if (tiles < 8) tiles = tiles_for(gemm_m, gemm_n, 64, 64);
-  int64_t want = (768 + tiles - 1) / tiles;
+  static const int target_wgs = [] {
+    const char* e = getenv("TCH_WGRAD_WGS");
+    return e && atoi(e) > 0 ? atoi(e) : 384;
+  }();
+  int64_t want = (target_wgs + tiles - 1) / tiles;
   int64_t max_by_k = pixels / (4 * BK);  // at least four reduction steps per split
   if (max_by_k < 1) max_by_k = 1;
   if (want > max_by_k) want = max_by_k;

@@ -180,8 +180,16 @@ struct LaunchRecord {
   const char* name;
   double work;
   int work_is_bytes;
+  // A recorded program is a valid serial order of launches.  `lane` 1 marks launches that may
+  // run beside the lane-0 ones on a second stream; `op` says how the lanes meet:
+  //   kOpLaunch       plain launch on its lane
+  //   kOpLaunchAfter  lane-1 launch that must see everything lane 0 was given before it
+  //   kOpJoin         no kernel: lane 0 waits for everything lane 1 was given so far
+  int lane;
+  int op;
   alignas(16) unsigned char args[360];
 };
+enum LaunchOp : int { kOpLaunch = 0, kOpLaunchAfter = 1, kOpJoin = 2 };
 
 class Context;  // defined in context.h
 

@@ -5,6 +5,7 @@ that already live on the GPU, passes their raw pointers to the shared library,
 and the library enqueues hand-written HIP kernels.  Layout is NHWC throughout;
 filters are [K, R, S, C].
 """
+import contextlib
 import ctypes
 import time
 
@@ -102,9 +103,23 @@ class Context:
             time.sleep(0)
 
     def synchronize(self):
-        """Everything submitted so far, queued or not, has finished on the GPU."""
+        """Everything submitted so far, queued or not, on either lane, has finished on the GPU."""
         self.flush()
-        self.stream.synchronize()
+        check(lib().tch_context_synchronize(self.handle), "tch_context_synchronize")
+
+    @contextlib.contextmanager
+    def side_lane(self, wait_main=True):
+        """While recording: the launches inside may run beside the main ones on a second stream;
+        the first of them waits for everything recorded before it.  `join()` is where the main
+        lane waits for them."""
+        check(lib().tch_context_set_lane(self.handle, 1, int(wait_main)), "tch_context_set_lane")
+        try:
+            yield
+        finally:
+            check(lib().tch_context_set_lane(self.handle, 0, 0), "tch_context_set_lane")
+
+    def join(self):
+        check(lib().tch_context_join(self.handle), "tch_context_join")
 
     def profile(self, program, reps=1):
         """Per-kernel HIP-event timing of `reps` replays: list of dicts with name, total_ms,

@@ -47,7 +47,8 @@ class _Block:
 
 class ResNetEngine:
     def __init__(self, depths=(3, 8, 36, 3), num_classes=1000, width=64, dtype=torch.bfloat16, image_size=224,
-                 lr=0.1, momentum=0.9, weight_decay=1e-4, bn_momentum=0.1, bn_eps=1e-5, stream=None, allocator=None):
+                 lr=0.1, momentum=0.9, weight_decay=1e-4, bn_momentum=0.1, bn_eps=1e-5, stream=None, allocator=None,
+                 overlap_wgrad=True):
         if not torch.cuda.is_available():
             raise RuntimeError("ResNetEngine runs on the GPU only; there is no CPU path")
         assert dtype in (torch.bfloat16, torch.float32)
@@ -64,6 +65,10 @@ class ResNetEngine:
             lambda shape, dtype: torch.empty(shape, dtype=dtype, device=self.dev))
         self._hook = None
         self._cut_exception = None
+        # weight gradients depend only on dy and the saved input: recorded on a second lane so that
+        # they run beside the data-gradient chain (each kernel alone leaves CUs idle at batch 64);
+        # costs the recycling of the dy buffers (they stay alive until the lanes join)
+        self.overlap_wgrad = overlap_wgrad
 
         # ---- architecture + parameter table (torchvision naming and order) ----
         self._specs, self._bn_names = [], []
@@ -258,7 +263,10 @@ class ResNetEngine:
             keep.append(t)
             return t.view(shape)
 
-        def gfree(t):
+        def gfree(t, read_by_wgrad=False):
+            # a buffer the side lane still reads must not be handed out again before the join
+            if read_by_wgrad and self.overlap_wgrad:
+                return
             free.setdefault(t.numel(), []).append(t.reshape(-1))
 
         code = ops.dtype_code(torch.empty(0, dtype=T))
@@ -329,8 +337,13 @@ class ResNetEngine:
             ops.conv2d_fwd(ctx, x, self._w(c.name + ".weight"), y, c.stride, c.pad, c_logical=c.cin, **kw)
 
         def conv_wgrad(c, x, dy):
-            ops.conv2d_wgrad(ctx, x, dy, self._view(self.grads, c.name + ".weight"), c.stride, c.pad, workspace=wg_ws,
-                             c_logical=c.cin)
+            if self.overlap_wgrad:
+                with ctx.side_lane(wait_main=True):
+                    ops.conv2d_wgrad(ctx, x, dy, self._view(self.grads, c.name + ".weight"), c.stride, c.pad,
+                                     workspace=wg_ws, c_logical=c.cin)
+            else:
+                ops.conv2d_wgrad(ctx, x, dy, self._view(self.grads, c.name + ".weight"), c.stride, c.pad,
+                                 workspace=wg_ws, c_logical=c.cin)
 
         def conv_dgrad(c, dy, dx, **kw):
             ops.conv2d_dgrad(ctx, dy, self._wt(c.name + ".weight"), dx, c.stride, c.pad, c_logical=c.cin, **kw)
@@ -389,8 +402,8 @@ class ResNetEngine:
             mark("fwd", "loss")
 
             # ================= backward =================
-            ops.conv2d_wgrad(ctx, pooled.view(B, 1, 1, self.feat), dlogits.view(B, 1, 1, self.num_classes),
-                             self._view(self.grads, "fc.weight"), 1, 0, workspace=wg_ws)
+            fc_conv = _Conv("fc", self.feat, self.num_classes, 1, 1, 0)
+            conv_wgrad(fc_conv, pooled.view(B, 1, 1, self.feat), dlogits.view(B, 1, 1, self.num_classes))
             ops.bias_grad(ctx, dlogits, self._view(self.grads, "fc.bias"))
             g_pooled = galloc((B, self.feat))
             ops.conv2d_dgrad(ctx, dlogits.view(B, 1, 1, self.num_classes), self._wt("fc.weight"),
@@ -407,7 +420,7 @@ class ResNetEngine:
                 g_a2 = galloc(a2.shape)
                 conv_dgrad(blk.c3, dz3, g_a2)
                 mark("bwd", pre + ".conv3")
-                gfree(dz3)
+                gfree(dz3, True)
                 dz2 = galloc(z2.shape)
                 bn_bwd(pre + ".bn2", g_a2, z2, dz2, a2)
                 gfree(g_a2)
@@ -415,7 +428,7 @@ class ResNetEngine:
                 g_a1 = galloc(a1.shape)
                 conv_dgrad(blk.c2, dz2, g_a1)
                 mark("bwd", pre + ".conv2")
-                gfree(dz2)
+                gfree(dz2, True)
                 dz1 = galloc(z1.shape)
                 bn_bwd(pre + ".bn1", g_a1, z1, dz1, a1)
                 gfree(g_a1)
@@ -427,13 +440,13 @@ class ResNetEngine:
                     conv_wgrad(blk.cd, xin, dzd)
                     gx_id = galloc(xin.shape)
                     conv_dgrad(blk.cd, dzd, gx_id)
-                    gfree(dzd)
+                    gfree(dzd, True)
                     conv_dgrad(blk.c1, dz1, gx, add=gx_id)
                     gfree(gx_id)
                 else:
                     conv_dgrad(blk.c1, dz1, gx, add=g_out, mask=out)
                 mark("bwd", pre + ".conv1")
-                gfree(dz1)
+                gfree(dz1, True)
                 gfree(g_out)
                 g_out = gx
             g_a0 = galloc(a0.shape)
@@ -443,7 +456,8 @@ class ResNetEngine:
             bn_bwd("bn1", g_a0, z0, dz0, a0)
             gfree(g_a0)
             conv_wgrad(self.stem, x0, dz0)
-            gfree(dz0)
+            gfree(dz0, True)
+            ctx.join()
         finally:
             ctx.end_record()
         plan.prog = prog
