@@ -104,6 +104,15 @@ size_t tch_GetXQueueInFlight(uint64_t hip_stream);
 int tch_conv2d_fwd(tch_context* ctx, int dtype, const void* x, const void* w, void* y, const void* add,
                    const void* mask, const float* bias, int out_f32, int N, int H, int W, int C, int K, int R, int S,
                    int stride, int pad, int tile_cfg, int c_logical);
+/* The convolution that feeds a BatchNorm (torchvision's conv -> bn pairs, train/resnet152.py:22): y as
+ * above (no bias / addend), and per (row tile, output channel) the sum and the sum of squares of y as
+ * stored: bn_partial[(tile * K + k) * 2 + {0,1}], tch_conv2d_fwd_stat_rows(...) row tiles.  Saves the
+ * statistics pass over y; feed the partials to tch_bn_fwd_train_partials. */
+int tch_conv2d_fwd_bnstats(tch_context* ctx, int dtype, const void* x, const void* w, void* y, int N, int H, int W,
+                           int C, int K, int R, int S, int stride, int pad, int tile_cfg, int c_logical,
+                           float* bn_partial);
+int tch_conv2d_fwd_stat_rows(int dtype, int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
+                             int tile_cfg);
 /* dx[N,H,W,C] = conv_transpose(dy[N,Ho,Wo,K], w) (+ add, optionally gated by mask > 0).
  * wt is the filter TRANSPOSED to [C][R][S][K] (tch_filter_transpose_batched). */
 int tch_conv2d_dgrad(tch_context* ctx, int dtype, const void* dy, const void* wt, void* dx, const void* add,
@@ -125,6 +134,12 @@ int tch_bn_fwd_train(tch_context* ctx, int dtype, const void* x, void* y, const 
                      int64_t rows, int C, const float* gamma, const float* beta, float* running_mean,
                      float* running_var, float* save_mean, float* save_invstd, float momentum, float eps,
                      float* workspace);
+/* The same, with the batch statistics already summed per row block (tch_conv2d_fwd_bnstats):
+ * partial[(b * C + c) * 2 + {0,1}] for b < row_blocks; scratch holds 2 C floats. */
+int tch_bn_fwd_train_partials(tch_context* ctx, int dtype, const void* x, void* y, const void* residual, int relu,
+                              int64_t rows, int C, const float* gamma, const float* beta, float* running_mean,
+                              float* running_var, float* save_mean, float* save_invstd, float momentum, float eps,
+                              const float* partial, int row_blocks, float* scratch);
 /* g = dy * (relu_mask > 0) (relu_mask may be NULL); dgamma/dbeta (+)=; dx = bn'(g) */
 int tch_bn_bwd(tch_context* ctx, int dtype, const void* dy, const void* relu_mask, const void* x, void* dx,
                int64_t rows, int C, const float* gamma, const float* save_mean, const float* save_invstd,

@@ -347,6 +347,33 @@ int bn_fwd_train(Context* ctx, int dtype, const void* x, void* y, const void* re
                                  "bn_apply_kernel<f32,fwd>", apply_bytes, 1);
 }
 
+int bn_fwd_train_partials(Context* ctx, int dtype, const void* x, void* y, const void* residual, int relu,
+                          int64_t rows, int C, const float* gamma, const float* beta, float* running_mean,
+                          float* running_var, float* save_mean, float* save_invstd, float momentum, float eps,
+                          const float* partial, int row_blocks, float* scratch) {
+  if (int rc = check_common(rows, C, dtype)) return rc;
+  TCH_CHECK_ARG(x && y && gamma && beta && save_mean && save_invstd && partial && scratch,
+                "bn_fwd_train_partials: null tensor");
+  TCH_CHECK_ARG(row_blocks >= 1, "bn_fwd_train_partials: no partial statistics");
+  TCH_CHECK_ARG((running_mean == nullptr) == (running_var == nullptr), "bn_fwd_train: running stats come in pairs");
+  Geometry g = geometry(rows, C, dtype);
+  float* scale = scratch;
+  float* shift = scratch + C;
+  FwdFinalizeArgs f{partial, row_blocks, C, rows, gamma, beta, running_mean, running_var, save_mean, save_invstd,
+                    scale,   shift,      momentum, eps};
+  int rc = launch(ctx, bn_fwd_finalize_kernel, dim3((C + 7) / 8), dim3(256), f, "bn_fwd_finalize_kernel",
+                  8.0 * row_blocks * C, 1);
+  if (rc) return rc;
+  const double eb = dtype == kBF16 ? 2.0 : 4.0;
+  const double tensor_bytes = static_cast<double>(rows) * C * eb;
+  ApplyArgs a{x, residual, nullptr, y, scale, shift, nullptr, rows * g.cc, FastDiv(g.cc), relu};
+  const double apply_bytes = tensor_bytes * (residual ? 3.0 : 2.0);
+  return dtype == kBF16 ? launch(ctx, bn_apply_kernel<bf16, 0>, dim3(apply_blocks(a.chunks)), dim3(256), a,
+                                 "bn_apply_kernel<bf16,fwd>", apply_bytes, 1)
+                        : launch(ctx, bn_apply_kernel<float, 0>, dim3(apply_blocks(a.chunks)), dim3(256), a,
+                                 "bn_apply_kernel<f32,fwd>", apply_bytes, 1);
+}
+
 int bn_bwd(Context* ctx, int dtype, const void* dy, const void* relu_mask, const void* x, void* dx, int64_t rows,
            int C, const float* gamma, const float* save_mean, const float* save_invstd, float* dgamma, float* dbeta,
            int accumulate, float* workspace) {

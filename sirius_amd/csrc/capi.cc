@@ -157,6 +157,30 @@ int tch_conv2d_fwd(tch_context* ctx, int dtype, const void* x, const void* w, vo
                     tile_cfg);
 }
 
+int tch_conv2d_fwd_bnstats(tch_context* ctx, int dtype, const void* x, const void* w, void* y, int N, int H, int W,
+                           int Cc, int K, int R, int S, int stride, int pad, int tile_cfg, int c_logical,
+                           float* bn_partial) {
+  if (!bn_partial) {
+    set_error("tch_conv2d_fwd_bnstats: null statistics buffer");
+    return -22;
+  }
+  return conv2d_fwd(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad, c_logical), x, w, y, nullptr, nullptr, nullptr,
+                    0, tile_cfg, bn_partial);
+}
+
+int tch_conv2d_fwd_stat_rows(int dtype, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad,
+                             int tile_cfg) {
+  return conv2d_fwd_stat_rows(shape(N, H, W, Cc, K, R, S, stride, pad), dtype, tile_cfg);
+}
+
+int tch_bn_fwd_train_partials(tch_context* ctx, int dtype, const void* x, void* y, const void* residual, int relu,
+                              int64_t rows, int Cc, const float* gamma, const float* beta, float* running_mean,
+                              float* running_var, float* save_mean, float* save_invstd, float momentum, float eps,
+                              const float* partial, int row_blocks, float* scratch) {
+  return bn_fwd_train_partials(C(ctx), dtype, x, y, residual, relu, rows, Cc, gamma, beta, running_mean, running_var,
+                               save_mean, save_invstd, momentum, eps, partial, row_blocks, scratch);
+}
+
 int tch_conv2d_dgrad(tch_context* ctx, int dtype, const void* dy, const void* w, void* dx, const void* add,
                      const void* mask, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad,
                      int tile_cfg, int c_logical) {

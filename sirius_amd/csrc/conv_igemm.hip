@@ -51,6 +51,7 @@ struct IgemmArgs {
   const void* add;    // optional addend, laid out like out (FWD/DGRAD)
   const void* mask;   // optional: addend counts only where mask > 0
   const float* bias;  // optional per-column bias (FWD)
+  float* stats;       // optional (FWD): per (row tile, column) sum and sum of squares of the stored output
   int N, H, W, C;     // x side
   int Ho, Wo, K;      // y side
   int R, S, stride, stride_log2, pad;
@@ -182,6 +183,94 @@ template <int E>
 __device__ inline void store_floats(float* dst, const float* v) {
 #pragma unroll
   for (int e = 0; e < E; e += 4) *reinterpret_cast<float4*>(dst + e) = make_float4(v[e], v[e + 1], v[e + 2], v[e + 3]);
+}
+
+// ---------------------------------------------------------------------------
+// epilogue of forward / data gradient: bias, gated residual, rounding, 16-byte accesses per
+// lane; optionally the BatchNorm batch statistics of the tile (forward): per output column the
+// sum and the sum of squares of the values AS STORED (after rounding to T), one pair per
+// (row tile, column) at stats[(tile_m * gemm_n + col) * 2], summed in a fixed order.
+// ---------------------------------------------------------------------------
+template <typename T, int MODE, int WM, int WN, int TM, int TN>
+__device__ inline void finish_tile(const IgemmArgs& p, f32x16_t (&acc)[TM][TN], float* stage, int tid, int m0, int n0,
+                                   int tile_m) {
+  constexpr int E = Elem<T>::kPerChunk;
+  constexpr int BN = WN * TN * 32;
+  constexpr int NT = WM * WN * 64;
+  constexpr int CH = BN / E;   // column chunks of the tile; a thread always gets chunk tid % CH
+  constexpr int ROWS = NT / CH;
+  static_assert(NT % CH == 0, "stats mapping");
+  const bool want_stats = MODE == kFwd && p.stats != nullptr;
+  float st_sum[E], st_sq[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) st_sum[e] = st_sq[e] = 0.f;
+
+  staged_epilogue<T, WM, WN, TM, TN>(acc, stage, tid, [&](int tr, int tc, float* v) {
+    const int row = m0 + tr, col = n0 + tc;
+    if (row >= p.gemm_m || col >= p.gemm_n) return;
+    const int64_t idx = static_cast<int64_t>(row) * p.gemm_n + col;
+    if (MODE == kFwd && p.bias) {
+#pragma unroll
+      for (int e = 0; e < E; ++e) v[e] += p.bias[col + e];
+    }
+    if (p.add) {
+      Chunk ca;
+      ca.u = *reinterpret_cast<const uint4*>(static_cast<const T*>(p.add) + idx);
+      float a[E];
+      chunk_to_float<T>(ca, a);
+      if (p.mask) {
+        Chunk cm;
+        cm.u = *reinterpret_cast<const uint4*>(static_cast<const T*>(p.mask) + idx);
+        float m[E];
+        chunk_to_float<T>(cm, m);
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+          if (!(m[e] > 0.f)) a[e] = 0.f;
+      }
+#pragma unroll
+      for (int e = 0; e < E; ++e) v[e] += a[e];
+    }
+    if (p.out_f32) {
+      store_floats<E>(static_cast<float*>(p.out) + idx, v);
+    } else {
+      const Chunk c = float_to_chunk<T>(v);
+      *reinterpret_cast<uint4*>(static_cast<T*>(p.out) + idx) = c.u;
+      if (want_stats) chunk_to_float<T>(c, v);  // the statistics are those of the stored values
+    }
+    if (want_stats) {
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        st_sum[e] += v[e];
+        st_sq[e] += v[e] * v[e];
+      }
+    }
+  });
+
+  if (want_stats) {
+    // threads tid, tid + CH, tid + 2 CH, ... hold partial sums of the same E columns
+    __syncthreads();
+    float* red = stage;  // [ROWS][CH][2E]
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      red[(tid * 2 * E) + e] = st_sum[e];
+      red[(tid * 2 * E) + E + e] = st_sq[e];
+    }
+    __syncthreads();
+    if (tid < BN) {
+      const int cc = tid / E, e = tid - cc * E;
+      float a = 0.f, b = 0.f;
+#pragma unroll 4
+      for (int r = 0; r < ROWS; ++r) {
+        a += red[((r * CH + cc) * 2 * E) + e];
+        b += red[((r * CH + cc) * 2 * E) + E + e];
+      }
+      const int col = n0 + tid;
+      if (col < p.gemm_n) {
+        float2* dst = reinterpret_cast<float2*>(p.stats + (static_cast<int64_t>(tile_m) * p.gemm_n + col) * 2);
+        *dst = make_float2(a, b);
+      }
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -355,37 +444,7 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm_kernel(IgemmArgs p) {
     load_tiles(kt + 4, ra0, rb0);
   }
 
-  // ---- epilogue: bias, gated residual, rounding; 16-byte accesses per lane ----
-  staged_epilogue<T, WM, WN, TM, TN>(acc, reinterpret_cast<float*>(lds), tid, [&](int tr, int tc, float* v) {
-    const int row = m0 + tr, col = n0 + tc;
-    if (row >= p.gemm_m || col >= p.gemm_n) return;
-    const int64_t idx = static_cast<int64_t>(row) * p.gemm_n + col;
-    if (MODE == kFwd && p.bias) {
-#pragma unroll
-      for (int e = 0; e < E; ++e) v[e] += p.bias[col + e];
-    }
-    if (p.add) {
-      Chunk ca;
-      ca.u = *reinterpret_cast<const uint4*>(static_cast<const T*>(p.add) + idx);
-      float a[E];
-      chunk_to_float<T>(ca, a);
-      if (p.mask) {
-        Chunk cm;
-        cm.u = *reinterpret_cast<const uint4*>(static_cast<const T*>(p.mask) + idx);
-        float m[E];
-        chunk_to_float<T>(cm, m);
-#pragma unroll
-        for (int e = 0; e < E; ++e)
-          if (!(m[e] > 0.f)) a[e] = 0.f;
-      }
-#pragma unroll
-      for (int e = 0; e < E; ++e) v[e] += a[e];
-    }
-    if (p.out_f32)
-      store_floats<E>(static_cast<float*>(p.out) + idx, v);
-    else
-      *reinterpret_cast<uint4*>(static_cast<T*>(p.out) + idx) = float_to_chunk<T>(v).u;
-  });
+  finish_tile<T, MODE, WM, WN, TM, TN>(p, acc, reinterpret_cast<float*>(lds), tid, m0, n0, tile_m);
 }
 
 // ---------------------------------------------------------------------------
@@ -808,36 +867,7 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm2_kernel(IgemmArgs p) {
     }
   }
 
-  staged_epilogue<T, WM, WN, TM, TN>(acc, reinterpret_cast<float*>(lds), tid, [&](int tr, int tc, float* v) {
-    const int row = m0 + tr, col = n0 + tc;
-    if (row >= p.gemm_m || col >= p.gemm_n) return;
-    const int64_t idx = static_cast<int64_t>(row) * p.gemm_n + col;
-    if (MODE == kFwd && p.bias) {
-#pragma unroll
-      for (int e = 0; e < E; ++e) v[e] += p.bias[col + e];
-    }
-    if (p.add) {
-      Chunk ca;
-      ca.u = *reinterpret_cast<const uint4*>(static_cast<const T*>(p.add) + idx);
-      float a[E];
-      chunk_to_float<T>(ca, a);
-      if (p.mask) {
-        Chunk cm;
-        cm.u = *reinterpret_cast<const uint4*>(static_cast<const T*>(p.mask) + idx);
-        float m[E];
-        chunk_to_float<T>(cm, m);
-#pragma unroll
-        for (int e = 0; e < E; ++e)
-          if (!(m[e] > 0.f)) a[e] = 0.f;
-      }
-#pragma unroll
-      for (int e = 0; e < E; ++e) v[e] += a[e];
-    }
-    if (p.out_f32)
-      store_floats<E>(static_cast<float*>(p.out) + idx, v);
-    else
-      *reinterpret_cast<uint4*>(static_cast<T*>(p.out) + idx) = float_to_chunk<T>(v).u;
-  });
+  finish_tile<T, MODE, WM, WN, TM, TN>(p, acc, reinterpret_cast<float*>(lds), tid, m0, n0, tile_m);
 }
 
 struct ReduceArgs {
@@ -1015,10 +1045,12 @@ void conv_output_hw(const ConvShape& s, int* Ho, int* Wo) {
 }
 
 int conv2d_fwd(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* w, void* y, const void* add,
-               const void* mask, const float* bias, int out_f32, int tile_cfg) {
+               const void* mask, const float* bias, int out_f32, int tile_cfg, float* bn_partial) {
   IgemmArgs a{};
   if (int rc = fill_common(a, s, dtype)) return rc;
   TCH_CHECK_ARG(x && w && y, "conv2d_fwd: null tensor");
+  TCH_CHECK_ARG(!(bn_partial && out_f32), "conv2d_fwd: statistics are taken of outputs stored in the compute type");
+  a.stats = bn_partial;
   const int eb = dtype == kBF16 ? 2 : 4;
   a.a_src = x;
   a.b_src = w;
@@ -1038,6 +1070,16 @@ int conv2d_fwd(Context* ctx, int dtype, const ConvShape& s, const void* x, const
   if (tile_cfg < 0) tile_cfg = pick_tile(a.gemm_m, a.gemm_n, 1);
   return dtype == kBF16 ? launch_mode<bf16, kFwd>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo))
                         : launch_mode<float, kFwd>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo));
+}
+
+int conv2d_fwd_stat_rows(const ConvShape& s, int dtype, int tile_cfg) {
+  (void)dtype;
+  int Ho, Wo;
+  conv_output_hw(s, &Ho, &Wo);
+  const int gemm_m = s.N * Ho * Wo;
+  if (tile_cfg < 0) tile_cfg = pick_tile(gemm_m, s.K, 1);
+  const int bm = tile_cfg == 2 ? 64 : 128;
+  return (gemm_m + bm - 1) / bm;
 }
 
 int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, const void* wt, void* dx,

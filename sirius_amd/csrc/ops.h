@@ -22,7 +22,9 @@ void conv_output_hw(const ConvShape& s, int* Ho, int* Wo);
 
 // conv_igemm.hip
 int conv2d_fwd(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* w, void* y, const void* add,
-               const void* mask, const float* bias, int out_f32, int tile_cfg);
+               const void* mask, const float* bias, int out_f32, int tile_cfg, float* bn_partial = nullptr);
+// rows of partial statistics conv2d_fwd writes for this shape and tiling (one per row tile)
+int conv2d_fwd_stat_rows(const ConvShape& s, int dtype, int tile_cfg);
 int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, const void* w, void* dx,
                  const void* add, const void* mask, int tile_cfg);
 int conv2d_wgrad_pick_splits(const ConvShape& s, int dtype);
@@ -36,6 +38,12 @@ int64_t bn_workspace_bytes(int64_t rows, int C, int dtype);
 int bn_fwd_train(Context* ctx, int dtype, const void* x, void* y, const void* residual, int relu, int64_t rows, int C,
                  const float* gamma, const float* beta, float* running_mean, float* running_var, float* save_mean,
                  float* save_invstd, float momentum, float eps, float* workspace);
+// the same with the batch statistics already summed per row block by the producer of x:
+// partial[(b * C + c) * 2 + {0, 1}] = sum, sum of squares over the rows of block b; scratch holds 2 C floats
+int bn_fwd_train_partials(Context* ctx, int dtype, const void* x, void* y, const void* residual, int relu,
+                          int64_t rows, int C, const float* gamma, const float* beta, float* running_mean,
+                          float* running_var, float* save_mean, float* save_invstd, float momentum, float eps,
+                          const float* partial, int row_blocks, float* scratch);
 int bn_bwd(Context* ctx, int dtype, const void* dy, const void* relu_mask, const void* x, void* dx, int64_t rows,
            int C, const float* gamma, const float* save_mean, const float* save_invstd, float* dgamma, float* dbeta,
            int accumulate, float* workspace);

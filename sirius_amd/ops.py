@@ -157,6 +157,26 @@ def conv2d_fwd(ctx, x, w, y, stride, pad, add=None, mask=None, bias=None, tile_c
                                N, H, W, C, K, R, S, stride, pad, tile_cfg, c_logical), "tch_conv2d_fwd")
 
 
+def conv2d_fwd_stat_rows(x, K, R, S, stride, pad, tile_cfg=-1):
+    N, H, W, C = x.shape
+    return int(lib().tch_conv2d_fwd_stat_rows(dtype_code(x), N, H, W, C, K, R, S, stride, pad, tile_cfg))
+
+
+def conv2d_fwd_bnstats(ctx, x, w, y, stride, pad, partial, tile_cfg=-1, c_logical=0):
+    """conv2d_fwd that also leaves the per-row-tile BatchNorm sums of y in `partial`
+    ([row tiles, K, 2] fp32); returns the number of row tiles."""
+    N, H, W, C = x.shape
+    K, R, S, C2 = w.shape
+    assert C == C2 and w.dtype == x.dtype == y.dtype
+    Ho, Wo = conv_out_hw(H, W, R, S, stride, pad)
+    assert tuple(y.shape) == (N, Ho, Wo, K)
+    rb = conv2d_fwd_stat_rows(x, K, R, S, stride, pad, tile_cfg)
+    assert partial.dtype == torch.float32 and partial.numel() >= rb * K * 2
+    check(lib().tch_conv2d_fwd_bnstats(ctx.handle, dtype_code(x), _p(x), _p(w), _p(y), N, H, W, C, K, R, S, stride, pad,
+                                       tile_cfg, c_logical, _p(partial)), "tch_conv2d_fwd_bnstats")
+    return rb
+
+
 def conv2d_dgrad(ctx, dy, wt, dx, stride, pad, add=None, mask=None, tile_cfg=-1, c_logical=0):
     """wt is the filter transposed to [C,R,S,K] (filter_transpose)."""
     w = wt
@@ -217,6 +237,23 @@ def bn_fwd_train(ctx, x, y, gamma, beta, running_mean, running_var, save_mean, s
     check(lib().tch_bn_fwd_train(ctx.handle, dtype_code(x), _p(x), _p(y), _p(residual), int(relu), rows, C,
                                  _p(gamma), _p(beta), _p(running_mean), _p(running_var), _p(save_mean),
                                  _p(save_invstd), momentum, eps, _p(workspace)), "tch_bn_fwd_train")
+
+
+def bn_fwd_train_partials(ctx, x, y, gamma, beta, running_mean, running_var, save_mean, save_invstd, partial,
+                          row_blocks, scratch, residual=None, relu=False, momentum=0.1, eps=1e-5):
+    """bn_fwd_train on statistics the producer of x has already summed per row block."""
+    C = x.shape[-1]
+    rows = x.numel() // C
+    assert y.shape == x.shape and y.dtype == x.dtype
+    assert residual is None or (residual.shape == x.shape and residual.dtype == x.dtype)
+    for t in (gamma, beta, save_mean, save_invstd):
+        assert t.dtype == torch.float32 and t.numel() == C
+    assert partial.dtype == torch.float32 and partial.numel() >= row_blocks * C * 2
+    assert scratch.dtype == torch.float32 and scratch.numel() >= 2 * C
+    check(lib().tch_bn_fwd_train_partials(ctx.handle, dtype_code(x), _p(x), _p(y), _p(residual), int(relu), rows, C,
+                                          _p(gamma), _p(beta), _p(running_mean), _p(running_var), _p(save_mean),
+                                          _p(save_invstd), momentum, eps, _p(partial), int(row_blocks), _p(scratch)),
+          "tch_bn_fwd_train_partials")
 
 
 def bn_bwd(ctx, dy, x, dx, gamma, save_mean, save_invstd, dgamma, dbeta, workspace, relu_mask=None,

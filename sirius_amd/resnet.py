@@ -48,7 +48,7 @@ class _Block:
 class ResNetEngine:
     def __init__(self, depths=(3, 8, 36, 3), num_classes=1000, width=64, dtype=torch.bfloat16, image_size=224,
                  lr=0.1, momentum=0.9, weight_decay=1e-4, bn_momentum=0.1, bn_eps=1e-5, stream=None, allocator=None,
-                 overlap_wgrad=True):
+                 overlap_wgrad=True, fuse_bn_stats=True):
         if not torch.cuda.is_available():
             raise RuntimeError("ResNetEngine runs on the GPU only; there is no CPU path")
         assert dtype in (torch.bfloat16, torch.float32)
@@ -69,6 +69,7 @@ class ResNetEngine:
         # they run beside the data-gradient chain (each kernel alone leaves CUs idle at batch 64);
         # costs the recycling of the dy buffers (they stay alive until the lanes join)
         self.overlap_wgrad = overlap_wgrad
+        self.fuse_bn_stats = fuse_bn_stats
 
         # ---- architecture + parameter table (torchvision naming and order) ----
         self._specs, self._bn_names = [], []
@@ -305,9 +306,13 @@ class ResNetEngine:
         def bn_need(rows, C):
             bn_ws_bytes[0] = max(bn_ws_bytes[0], ops.bn_workspace_bytes(code, rows, C))
 
+        conv_inputs = [(self.stem, (B, S, S))]
         wg_need(self.stem, B, S, S)
         bn_need(B * H0 * W0, self.width)
         for blk, (H, W, Ho, Wo) in zip(self.blocks, shapes):
+            conv_inputs += [(blk.c1, (B, H, W)), (blk.c2, (B, H, W)), (blk.c3, (B, Ho, Wo))]
+            if blk.cd is not None:
+                conv_inputs.append((blk.cd, (B, H, W)))
             wg_need(blk.c1, B, H, W)
             wg_need(blk.c2, B, H, W)
             wg_need(blk.c3, B, Ho, Wo)
@@ -336,6 +341,29 @@ class ResNetEngine:
         def conv_fwd(c, x, y, **kw):
             ops.conv2d_fwd(ctx, x, self._w(c.name + ".weight"), y, c.stride, c.pad, c_logical=c.cin, **kw)
 
+        # convolution -> BatchNorm pairs: the convolution's epilogue leaves the per-tile batch sums,
+        # the BatchNorm starts at its finalize (no statistics pass over the convolution's output)
+        stat_elems = [0]
+        for c_, (n_, h_, w_) in conv_inputs:
+            xm = torch.empty((n_, h_, w_, c_.cin_store), dtype=T, device="meta")
+            stat_elems[0] = max(stat_elems[0],
+                                ops.conv2d_fwd_stat_rows(xm, c_.cout, c_.k, c_.k, c_.stride, c_.pad) * c_.cout * 2)
+        stat_partial = act(max(stat_elems[0], 2), dtype=torch.float32)
+        bn_scratch = act(2 * max(c_.cout for c_, _ in conv_inputs), dtype=torch.float32)
+
+        def conv_bn_fwd(c, name, x, z, y, residual=None, relu=True):
+            if not self.fuse_bn_stats:
+                conv_fwd(c, x, z)
+                return bn_fwd(name, z, y, residual=residual, relu=relu)
+            rb = ops.conv2d_fwd_bnstats(ctx, x, self._w(c.name + ".weight"), z, c.stride, c.pad, stat_partial,
+                                        c_logical=c.cin)
+            o, ch = self._bn_off[name]
+            ops.bn_fwd_train_partials(ctx, z, y, self._view(self.params, name + ".weight"),
+                                      self._view(self.params, name + ".bias"), self.running_mean[o:o + ch],
+                                      self.running_var[o:o + ch], bn_save[o:o + ch], bn_save[nbn + o:nbn + o + ch],
+                                      stat_partial, rb, bn_scratch, residual=residual, relu=relu,
+                                      momentum=self.bn_momentum, eps=self.bn_eps)
+
         def conv_wgrad(c, x, dy):
             if self.overlap_wgrad:
                 with ctx.side_lane(wait_main=True):
@@ -360,8 +388,7 @@ class ResNetEngine:
             x0 = act(B, S, S, STEM_CIN_PAD)
             ops.nchw_to_nhwc_pad(ctx, plan.x_in, x0)
             z0, a0 = act(B, H0, W0, self.width), act(B, H0, W0, self.width)
-            conv_fwd(self.stem, x0, z0)
-            bn_fwd("bn1", z0, a0)
+            conv_bn_fwd(self.stem, "bn1", x0, z0, a0)
             mark("fwd", "bn1")
             p0 = act(B, Hp, Wp, self.width)
             p0_idx = act(B, Hp, Wp, self.width, dtype=torch.int32)
@@ -371,23 +398,19 @@ class ResNetEngine:
             for blk, (H, W, Ho, Wo) in zip(self.blocks, shapes):
                 P, pre = blk.planes, blk.prefix
                 z1, a1 = act(B, H, W, P), act(B, H, W, P)
-                conv_fwd(blk.c1, x, z1)
-                bn_fwd(pre + ".bn1", z1, a1)
+                conv_bn_fwd(blk.c1, pre + ".bn1", x, z1, a1)
                 mark("fwd", pre + ".bn1")
                 z2, a2 = act(B, Ho, Wo, P), act(B, Ho, Wo, P)
-                conv_fwd(blk.c2, a1, z2)
-                bn_fwd(pre + ".bn2", z2, a2)
+                conv_bn_fwd(blk.c2, pre + ".bn2", a1, z2, a2)
                 mark("fwd", pre + ".bn2")
                 z3, out = act(B, Ho, Wo, 4 * P), act(B, Ho, Wo, 4 * P)
-                conv_fwd(blk.c3, a2, z3)
                 zd = None
                 if blk.cd is not None:
                     zd, idn = act(B, Ho, Wo, 4 * P), act(B, Ho, Wo, 4 * P)
-                    conv_fwd(blk.cd, x, zd)
-                    bn_fwd(pre + ".downsample.1", zd, idn, relu=False)
+                    conv_bn_fwd(blk.cd, pre + ".downsample.1", x, zd, idn, relu=False)
                 else:
                     idn = x
-                bn_fwd(pre + ".bn3", z3, out, residual=idn, relu=True)
+                conv_bn_fwd(blk.c3, pre + ".bn3", a2, z3, out, residual=idn, relu=True)
                 mark("fwd", pre + ".bn3")
                 saved.append((x, z1, a1, z2, a2, z3, zd, out))
                 x = out

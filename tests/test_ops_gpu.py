@@ -179,6 +179,46 @@ def test_bn_fwd(ctx, dtype, rows, C, fuse):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", [CONV_CASES[0], CONV_CASES[2], CONV_CASES[3], CONV_CASES[5], CONV_CASES[6]])
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2])
+def test_conv_with_bn_statistics(ctx, dtype, case, tile_cfg):
+    """The convolution leaves per-tile sums of its stored output; BatchNorm starts from them.
+    Checked against the oracle's conv -> BatchNorm(train) on the same inputs; the statistics must be
+    those of the ROUNDED convolution output (what the unfused pair would see)."""
+    from sirius_amd import ops
+    N, H, W, C, K, R, S, st, pad = case
+    print("case", case, dtype, tile_cfg, flush=True)
+    g = _gen(21)
+    x = rnd((N, H, W, C), dtype, g)
+    w = rnd((K, R, S, C), dtype, g, (R * S * C) ** -0.5)
+    gamma, beta = torch.rand(K, generator=g) + 0.5, torch.randn(K, generator=g) * 0.1
+    z_ref = O.conv2d_fwd(x, w, st, pad).to(dtype)
+    rm_ref, rv_ref = torch.zeros(K), torch.ones(K)
+    y_ref, mean_ref, invstd_ref = O.bn_fwd_train(z_ref, gamma, beta, rm_ref, rv_ref, relu=True)
+    xd, wd = x.cuda(), w.cuda()
+    z = torch.empty(z_ref.shape, dtype=dtype, device="cuda")
+    rb = ops.conv2d_fwd_stat_rows(xd, K, R, S, st, pad, tile_cfg)
+    partial = torch.full((rb * K * 2,), float("nan"), device="cuda")
+    assert ops.conv2d_fwd_bnstats(ctx, xd, wd, z, st, pad, partial, tile_cfg=tile_cfg) == rb
+    y = torch.empty_like(z)
+    rm, rv = torch.zeros(K, device="cuda"), torch.ones(K, device="cuda")
+    sm, si = torch.empty(K, device="cuda"), torch.empty(K, device="cuda")
+    scratch = torch.empty(2 * K, device="cuda")
+    ops.bn_fwd_train_partials(ctx, z, y, gamma.cuda(), beta.cuda(), rm, rv, sm, si, partial, rb, scratch, relu=True)
+    torch.cuda.synchronize()
+    close(z, z_ref, dtype, "conv out")
+    # statistics of what was stored, exactly: compare with sums over the kernel's own z
+    z32 = z.float().cpu().reshape(-1, K)
+    sums = partial.cpu().reshape(rb, K, 2).double().sum(0)
+    close(sums[:, 0].float(), z32.double().sum(0).float(), torch.float32, "sum", rtol=1e-5)
+    close(sums[:, 1].float(), (z32.double() ** 2).sum(0).float(), torch.float32, "sum of squares", rtol=1e-5)
+    tol = 1e-3 if dtype == torch.float32 else 2e-2
+    close(sm, mean_ref, torch.float32, "bn mean", rtol=tol)
+    close(si, invstd_ref, torch.float32, "bn invstd", rtol=tol)
+    close(y, y_ref, dtype, "bn y", rtol=tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("rows,C", BN_CASES)
 @pytest.mark.parametrize("masked", [False, True])
 def test_bn_bwd(ctx, dtype, rows, C, masked):
