@@ -92,6 +92,7 @@ def handover(batch):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--no-handover", action="store_true", help="skip the 64 -> 16 -> 64 handover measurement")
+    ap.add_argument("--no-autotune", action="store_true", help="keep the library's tiling heuristic")
     ap.add_argument("--no-overlap", action="store_true", help="record weight gradients on the main lane (one stream)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch accumulate_kernel once over two 512 MiB buffers (reads 1 GiB, writes 1 GiB): "
@@ -114,7 +115,7 @@ def main():
     torch.cuda.set_device(0)
     B = args.batch
     eng = ResNetEngine((3, 8, 36, 3), 1000, 64, dtype=torch.bfloat16, image_size=224, lr=0.1, momentum=0.9,
-                       weight_decay=1e-4, overlap_wgrad=not args.no_overlap)
+                       weight_decay=1e-4, overlap_wgrad=not args.no_overlap, autotune=not args.no_autotune)
     eng.init_kaiming(seed=0)
     g = torch.Generator(device="cuda")
     g.manual_seed(1)

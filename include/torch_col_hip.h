@@ -98,7 +98,8 @@ size_t tch_GetXQueueInFlight(uint64_t hip_stream);
 
 /* ---- convolution (implicit GEMM on MFMA) ---------------------------------------- */
 /* y[N,Ho,Wo,K] = conv(x[N,H,W,C], w[K,R,S,C]) (+ bias[K]) (+ add, optionally gated by mask > 0).
- * out_f32 != 0 stores y as fp32 whatever dtype is.  tile_cfg: -1 auto, 0 = 128x128, 1 = 128x64, 2 = 64x64.
+ * out_f32 != 0 stores y as fp32 whatever dtype is.  tile_cfg: -1 auto, 0 = 128x128, 1 = 128x64, 2 = 64x64,
+ * 3 = 64x64 on the register-staged kernel even where the direct-to-LDS kernel applies.
  * c_logical: input channels that carry data when C is zero-padded to a chunk (0 = C); it only enters the
  * algorithmic-work figure the profiler reports, never the arithmetic. */
 int tch_conv2d_fwd(tch_context* ctx, int dtype, const void* x, const void* w, void* y, const void* add,

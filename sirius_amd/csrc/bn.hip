@@ -132,10 +132,21 @@ __device__ inline bool finalize_sums(const float* partial, int row_blocks, int C
   __shared__ double red[32][8][2];
   double s = 0.0, q = 0.0;
   if (c < C) {
-    for (int b = lane; b < row_blocks; b += 32) {
-      const float2 v = *reinterpret_cast<const float2*>(partial + (static_cast<int64_t>(b) * C + c) * 2);
-      s += v.x;
-      q += v.y;
+    // eight loads in flight per lane: what this loop costs is its count of dependent round trips
+    constexpr int U = 8;
+    for (int b = lane; b < row_blocks; b += U * 32) {
+      float2 v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int bb = b + u * 32;
+        v[u] = bb < row_blocks ? *reinterpret_cast<const float2*>(partial + (static_cast<int64_t>(bb) * C + c) * 2)
+                               : make_float2(0.f, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        s += v[u].x;
+        q += v[u].y;
+      }
     }
   }
   const int cl = threadIdx.x & 7;

@@ -964,10 +964,12 @@ int launch_mode(Context* ctx, IgemmArgs& a, int tile_cfg, double flops) {
   if constexpr (sizeof(T) == 2 && (MODE == kFwd || MODE == kDgrad)) {
     const int in_c = MODE == kFwd ? a.C : a.K;
     const int setting = igemm2_setting();
-    if (setting != 0 && in_c % kStep2 == 0 && a.R * a.S <= 32 && (tile_cfg == 0 || tile_cfg == 1)) {
+    if (setting != 0 && in_c % kStep2 == 0 && a.R * a.S <= 32 && tile_cfg >= 0 && tile_cfg <= 2) {
       if (tile_cfg == 0)
         return setting == 3 ? launch_cfg2<MODE, 2, 2, 2, 2, 3>(ctx, a, flops) : launch_cfg2<MODE, 2, 2, 2, 2, 2>(ctx, a, flops);
-      return setting == 2 ? launch_cfg2<MODE, 2, 2, 2, 1, 2>(ctx, a, flops) : launch_cfg2<MODE, 2, 2, 2, 1, 3>(ctx, a, flops);
+      if (tile_cfg == 1)
+        return setting == 2 ? launch_cfg2<MODE, 2, 2, 2, 1, 2>(ctx, a, flops) : launch_cfg2<MODE, 2, 2, 2, 1, 3>(ctx, a, flops);
+      return setting == 2 ? launch_cfg2<MODE, 2, 2, 1, 1, 2>(ctx, a, flops) : launch_cfg2<MODE, 2, 2, 1, 1, 3>(ctx, a, flops);
     }
   }
   switch (tile_cfg) {
@@ -976,7 +978,7 @@ int launch_mode(Context* ctx, IgemmArgs& a, int tile_cfg, double flops) {
     case 1:
       return launch_cfg<T, MODE, 2, 2, 2, 1>(ctx, a, flops);  // 128 x 64
     default:
-      return launch_cfg<T, MODE, 2, 2, 1, 1>(ctx, a, flops);  // 64 x 64
+      return launch_cfg<T, MODE, 2, 2, 1, 1>(ctx, a, flops);  // 64 x 64 (2, and 3 = never the direct-to-LDS kernel)
   }
 }
 
@@ -1078,7 +1080,7 @@ int conv2d_fwd_stat_rows(const ConvShape& s, int dtype, int tile_cfg) {
   conv_output_hw(s, &Ho, &Wo);
   const int gemm_m = s.N * Ho * Wo;
   if (tile_cfg < 0) tile_cfg = pick_tile(gemm_m, s.K, 1);
-  const int bm = tile_cfg == 2 ? 64 : 128;
+  const int bm = tile_cfg >= 2 ? 64 : 128;
   return (gemm_m + bm - 1) / bm;
 }
 

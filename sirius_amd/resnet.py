@@ -48,7 +48,7 @@ class _Block:
 class ResNetEngine:
     def __init__(self, depths=(3, 8, 36, 3), num_classes=1000, width=64, dtype=torch.bfloat16, image_size=224,
                  lr=0.1, momentum=0.9, weight_decay=1e-4, bn_momentum=0.1, bn_eps=1e-5, stream=None, allocator=None,
-                 overlap_wgrad=True, fuse_bn_stats=True):
+                 overlap_wgrad=True, fuse_bn_stats=True, autotune=False):
         if not torch.cuda.is_available():
             raise RuntimeError("ResNetEngine runs on the GPU only; there is no CPU path")
         assert dtype in (torch.bfloat16, torch.float32)
@@ -70,6 +70,11 @@ class ResNetEngine:
         # costs the recycling of the dy buffers (they stay alive until the lanes join)
         self.overlap_wgrad = overlap_wgrad
         self.fuse_bn_stats = fuse_bn_stats
+        # autotune: when a plan is built, time each distinct convolution shape with every tiling and
+        # keep the fastest (forward and data gradient separately); off = the library's heuristic
+        self.autotune = autotune
+        self._tile_cache = {}
+        self.tile_timings = {}   # what the tuner measured: {shape key: {"fwd_ms": {cfg: ms}, "dgrad_ms": {cfg: ms}}}
 
         # ---- architecture + parameter table (torchvision naming and order) ----
         self._specs, self._bn_names = [], []
@@ -238,6 +243,56 @@ class ResNetEngine:
         flat = self.global_grads if use_global else self.grads
         return {p.name: self._from_store(p, flat) for p in self._specs}
 
+    # ------------------------------------------------------------------ tiling choice
+    def _time_program(self, fn, reps=3):
+        prog = self._flat_prog(fn)
+        self.ctx.run(prog)
+        best = float("inf")
+        for _ in range(reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(self.ctx.stream)
+            self.ctx.run(prog)
+            e1.record(self.ctx.stream)
+            e1.synchronize()
+            best = min(best, e0.elapsed_time(e1))
+        return best
+
+    def _tune_conv(self, c, n, h, w):
+        """(forward tiling, data-gradient tiling) for one convolution at one input shape."""
+        key = (c.cin_store, c.cout, c.k, c.stride, c.pad, n, h, w)
+        hit = self._tile_cache.get(key)
+        if hit is not None:
+            return hit
+        T, ctx = self.dtype, self.ctx
+        ho, wo = ops.conv_out_hw(h, w, c.k, c.k, c.stride, c.pad)
+        x = torch.zeros((n, h, w, c.cin_store), dtype=T, device=self.dev)
+        z = torch.zeros((n, ho, wo, c.cout), dtype=T, device=self.dev)
+        wgt, wt = self._w(c.name + ".weight"), self._wt(c.name + ".weight")
+        part = torch.empty(ops.conv2d_fwd_stat_rows(x, c.cout, c.k, c.k, c.stride, c.pad, 2) * c.cout * 2,
+                           dtype=torch.float32, device=self.dev)
+        reps = 4
+
+        def fwd(cfg):
+            def rec():
+                for _ in range(reps):
+                    ops.conv2d_fwd_bnstats(ctx, x, wgt, z, c.stride, c.pad, part, tile_cfg=cfg, c_logical=c.cin)
+            return rec
+
+        def dgrad(cfg):
+            def rec():
+                for _ in range(reps):
+                    ops.conv2d_dgrad(ctx, z, wt, x, c.stride, c.pad, tile_cfg=cfg, c_logical=c.cin)
+            return rec
+        cfgs = (0, 1, 2, 3) if c.cout > 64 else (1, 2, 3)
+        t_f = {cfg: self._time_program(fwd(cfg)) / reps for cfg in cfgs}
+        tf = min(t_f, key=t_f.get)
+        cfgs_d = (0, 1, 2, 3) if c.cin_store > 64 else (1, 2, 3)
+        t_d = {cfg: self._time_program(dgrad(cfg)) / reps for cfg in cfgs_d} if c.cin_store >= 64 else {-1: 0.0}
+        td = min(t_d, key=t_d.get)
+        self._tile_cache[key] = (tf, td)
+        self.tile_timings[key] = {"fwd_ms": t_f, "dgrad_ms": t_d}
+        return tf, td
+
     # ------------------------------------------------------------------ the plan for one batch size
     def _build_plan(self, B, loss_scale):
         T, dev, ctx = self.dtype, self.dev, self.ctx
@@ -344,10 +399,13 @@ class ResNetEngine:
         # convolution -> BatchNorm pairs: the convolution's epilogue leaves the per-tile batch sums,
         # the BatchNorm starts at its finalize (no statistics pass over the convolution's output)
         stat_elems = [0]
+        tiles = {}
         for c_, (n_, h_, w_) in conv_inputs:
             xm = torch.empty((n_, h_, w_, c_.cin_store), dtype=T, device="meta")
+            # sized for the smallest row tile, whichever tiling is picked
             stat_elems[0] = max(stat_elems[0],
-                                ops.conv2d_fwd_stat_rows(xm, c_.cout, c_.k, c_.k, c_.stride, c_.pad) * c_.cout * 2)
+                                ops.conv2d_fwd_stat_rows(xm, c_.cout, c_.k, c_.k, c_.stride, c_.pad, 2) * c_.cout * 2)
+            tiles[c_.name] = self._tune_conv(c_, n_, h_, w_) if self.autotune else (-1, -1)
         stat_partial = act(max(stat_elems[0], 2), dtype=torch.float32)
         bn_scratch = act(2 * max(c_.cout for c_, _ in conv_inputs), dtype=torch.float32)
 
@@ -356,7 +414,7 @@ class ResNetEngine:
                 conv_fwd(c, x, z)
                 return bn_fwd(name, z, y, residual=residual, relu=relu)
             rb = ops.conv2d_fwd_bnstats(ctx, x, self._w(c.name + ".weight"), z, c.stride, c.pad, stat_partial,
-                                        c_logical=c.cin)
+                                        tile_cfg=tiles[c.name][0], c_logical=c.cin)
             o, ch = self._bn_off[name]
             ops.bn_fwd_train_partials(ctx, z, y, self._view(self.params, name + ".weight"),
                                       self._view(self.params, name + ".bias"), self.running_mean[o:o + ch],
@@ -374,7 +432,8 @@ class ResNetEngine:
                                  workspace=wg_ws, c_logical=c.cin)
 
         def conv_dgrad(c, dy, dx, **kw):
-            ops.conv2d_dgrad(ctx, dy, self._wt(c.name + ".weight"), dx, c.stride, c.pad, c_logical=c.cin, **kw)
+            ops.conv2d_dgrad(ctx, dy, self._wt(c.name + ".weight"), dx, c.stride, c.pad, c_logical=c.cin,
+                             tile_cfg=tiles.get(c.name, (-1, -1))[1], **kw)
 
         prog = ops.Program()
         marks = []  # (launch index one past the layer, 'fwd' | 'bwd', layer name): checkpoint positions

@@ -55,7 +55,7 @@ CONV_CASES = [
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", CONV_CASES)
-@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2])
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3])
 def test_conv_fwd(ctx, dtype, case, tile_cfg):
     from sirius_amd import ops
     N, H, W, C, K, R, S, st, pad = case
@@ -89,7 +89,7 @@ def test_conv_fwd_epilogue(ctx, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", CONV_CASES)
-@pytest.mark.parametrize("tile_cfg", [-1, 0, 2])
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3])
 def test_conv_dgrad(ctx, dtype, case, tile_cfg):
     from sirius_amd import ops
     N, H, W, C, K, R, S, st, pad = case
@@ -180,7 +180,7 @@ def test_bn_fwd(ctx, dtype, rows, C, fuse):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", [CONV_CASES[0], CONV_CASES[2], CONV_CASES[3], CONV_CASES[5], CONV_CASES[6]])
-@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2])
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3])
 def test_conv_with_bn_statistics(ctx, dtype, case, tile_cfg):
     """The convolution leaves per-tile sums of its stored output; BatchNorm starts from them.
     Checked against the oracle's conv -> BatchNorm(train) on the same inputs; the statistics must be
