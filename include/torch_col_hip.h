@@ -119,6 +119,17 @@ int tch_conv2d_fwd_stat_rows(int dtype, int N, int H, int W, int C, int K, int R
 int tch_conv2d_dgrad(tch_context* ctx, int dtype, const void* dy, const void* wt, void* dx, const void* add,
                      const void* mask, int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
                      int tile_cfg, int c_logical);
+/* The same where dx is the gradient behind a BatchNorm (+ReLU) whose input is bn_x (laid out like dx) and
+ * whose ReLU output is bn_mask (may be NULL: no ReLU): dx is zeroed where bn_mask <= 0 before it is stored
+ * and the epilogue leaves, per row tile and channel, sum(dx) and sum(dx * (bn_x - mean) * invstd) at
+ * bn_partial[(tile * C + c) * 2 + {0,1}], tile < tch_conv2d_dgrad_stat_rows(): the two reductions of that
+ * BatchNorm's backward, with no pass over dx; feed them to tch_bn_bwd_partials. */
+int tch_conv2d_dgrad_bnsums(tch_context* ctx, int dtype, const void* dy, const void* wt, void* dx, const void* add,
+                            const void* mask, int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
+                            int tile_cfg, int c_logical, const void* bn_mask, const void* bn_x, const float* bn_mean,
+                            const float* bn_invstd, float* bn_partial);
+int tch_conv2d_dgrad_stat_rows(int dtype, int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
+                               int tile_cfg);
 /* dw[K,R,S,C] (fp32) (+)= sum over pixels of dy x x.  splits > 1 needs a workspace of
  * tch_conv2d_wgrad_workspace_bytes(); splits <= 0 lets the library choose (query with _pick_splits). */
 int tch_conv2d_wgrad_pick_splits(int dtype, int N, int H, int W, int C, int K, int R, int S, int stride, int pad);
@@ -145,6 +156,10 @@ int tch_bn_fwd_train_partials(tch_context* ctx, int dtype, const void* x, void* 
 int tch_bn_bwd(tch_context* ctx, int dtype, const void* dy, const void* relu_mask, const void* x, void* dx,
                int64_t rows, int C, const float* gamma, const float* save_mean, const float* save_invstd,
                float* dgamma, float* dbeta, int accumulate, float* workspace);
+/* The same from the sums tch_conv2d_dgrad_bnsums left; g is already gated by the ReLU; scratch holds 3 C floats. */
+int tch_bn_bwd_partials(tch_context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int C,
+                        const float* gamma, const float* save_mean, const float* save_invstd, float* dgamma,
+                        float* dbeta, int accumulate, const float* partial, int row_blocks, float* scratch);
 
 /* ---- pooling -------------------------------------------------------------------- */
 /* index[N,Ho,Wo,C] (int32) = h*W + w of the FIRST maximum in row-major window order (NaN wins). */

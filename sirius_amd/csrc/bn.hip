@@ -415,4 +415,26 @@ int bn_bwd(Context* ctx, int dtype, const void* dy, const void* relu_mask, const
                                  "bn_apply_kernel<f32,bwd>", tensor_bytes * (in_tensors + 1.0), 1);
 }
 
+int bn_bwd_partials(Context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int C,
+                    const float* gamma, const float* save_mean, const float* save_invstd, float* dgamma,
+                    float* dbeta, int accumulate, const float* partial, int row_blocks, float* scratch) {
+  if (int rc = check_common(rows, C, dtype)) return rc;
+  TCH_CHECK_ARG(g && x && dx && gamma && save_mean && save_invstd && dgamma && dbeta && partial && scratch,
+                "bn_bwd_partials: null tensor");
+  TCH_CHECK_ARG(row_blocks >= 1, "bn_bwd_partials: no partial sums");
+  Geometry geo = geometry(rows, C, dtype);
+  float* coef = scratch;
+  BwdFinalizeArgs f{partial, row_blocks, C, rows, gamma, save_mean, save_invstd, dgamma, dbeta, coef, accumulate};
+  int rc = launch(ctx, bn_bwd_finalize_kernel, dim3((C + 7) / 8), dim3(256), f, "bn_bwd_finalize_kernel",
+                  8.0 * row_blocks * C, 1);
+  if (rc) return rc;
+  const double eb = dtype == kBF16 ? 2.0 : 4.0;
+  const double tensor_bytes = static_cast<double>(rows) * C * eb;
+  ApplyArgs a{g, nullptr, x, dx, coef, coef + C, coef + 2 * C, rows * geo.cc, FastDiv(geo.cc), 0};
+  return dtype == kBF16 ? launch(ctx, bn_apply_kernel<bf16, 1>, dim3(apply_blocks(a.chunks)), dim3(256), a,
+                                 "bn_apply_kernel<bf16,bwd>", tensor_bytes * 3.0, 1)
+                        : launch(ctx, bn_apply_kernel<float, 1>, dim3(apply_blocks(a.chunks)), dim3(256), a,
+                                 "bn_apply_kernel<f32,bwd>", tensor_bytes * 3.0, 1);
+}
+
 }  // namespace tch

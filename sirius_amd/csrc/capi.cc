@@ -187,6 +187,27 @@ int tch_conv2d_dgrad(tch_context* ctx, int dtype, const void* dy, const void* w,
   return conv2d_dgrad(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad, c_logical), dy, w, dx, add, mask, tile_cfg);
 }
 
+int tch_conv2d_dgrad_bnsums(tch_context* ctx, int dtype, const void* dy, const void* w, void* dx, const void* add,
+                            const void* mask, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad,
+                            int tile_cfg, int c_logical, const void* bn_mask, const void* bn_x, const float* bn_mean,
+                            const float* bn_invstd, float* bn_partial) {
+  BnBwdSums bn{bn_mask, bn_x, bn_mean, bn_invstd, bn_partial};
+  return conv2d_dgrad(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad, c_logical), dy, w, dx, add, mask, tile_cfg,
+                      &bn);
+}
+
+int tch_conv2d_dgrad_stat_rows(int dtype, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad,
+                               int tile_cfg) {
+  return conv2d_dgrad_stat_rows(shape(N, H, W, Cc, K, R, S, stride, pad), dtype, tile_cfg);
+}
+
+int tch_bn_bwd_partials(tch_context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int Cc,
+                        const float* gamma, const float* save_mean, const float* save_invstd, float* dgamma,
+                        float* dbeta, int accumulate, const float* partial, int row_blocks, float* scratch) {
+  return bn_bwd_partials(C(ctx), dtype, g, x, dx, rows, Cc, gamma, save_mean, save_invstd, dgamma, dbeta, accumulate,
+                         partial, row_blocks, scratch);
+}
+
 int tch_conv2d_wgrad_pick_splits(int dtype, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad) {
   return conv2d_wgrad_pick_splits(shape(N, H, W, Cc, K, R, S, stride, pad), dtype);
 }

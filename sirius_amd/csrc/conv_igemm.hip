@@ -51,7 +51,11 @@ struct IgemmArgs {
   const void* add;    // optional addend, laid out like out (FWD/DGRAD)
   const void* mask;   // optional: addend counts only where mask > 0
   const float* bias;  // optional per-column bias (FWD)
-  float* stats;       // optional (FWD): per (row tile, column) sum and sum of squares of the stored output
+  float* stats;       // optional: per (row tile, column) pair of sums over the stored output (see finish_tile)
+  const void* bn_mask;      // DGRAD with stats, optional: the stored output is zeroed where bn_mask <= 0
+  const void* bn_x;         // DGRAD with stats: input of the BatchNorm this gradient flows into, laid out like out
+  const float* bn_mean;     // DGRAD with stats: that BatchNorm's saved batch mean / inverse std per column
+  const float* bn_invstd;
   int N, H, W, C;     // x side
   int Ho, Wo, K;      // y side
   int R, S, stride, stride_log2, pad;
@@ -134,7 +138,8 @@ struct TapWalker {
 
 // The accumulators of one workgroup tile, one 32-row band (index tm) at a time:
 // lanes write float4 groups into the staging tile [WM*32][BN + pad], then every
-// thread takes E consecutive columns of one row and hands them to `fin`.
+// thread takes E consecutive columns of one row and hands them to `fin` together with the
+// number of the visit (tm * ITERS + it, a compile-time constant after unrolling).
 template <typename T, int WM, int WN, int TM, int TN, typename Fin>
 __device__ inline void staged_epilogue(f32x16_t (&acc)[TM][TN], float* stage, int tid, Fin fin) {
   constexpr int E = Elem<T>::kPerChunk;
@@ -174,7 +179,7 @@ __device__ inline void staged_epilogue(f32x16_t (&acc)[TM][TN], float* stage, in
         v[e + 2] = t.z;
         v[e + 3] = t.w;
       }
-      fin(((r >> 5) * TM + tm) * 32 + (r & 31), cc * E, v);
+      fin(tm * ITERS + it, ((r >> 5) * TM + tm) * 32 + (r & 31), cc * E, v);
     }
   }
 }
@@ -187,9 +192,14 @@ __device__ inline void store_floats(float* dst, const float* v) {
 
 // ---------------------------------------------------------------------------
 // epilogue of forward / data gradient: bias, gated residual, rounding, 16-byte accesses per
-// lane; optionally the BatchNorm batch statistics of the tile (forward): per output column the
-// sum and the sum of squares of the values AS STORED (after rounding to T), one pair per
-// (row tile, column) at stats[(tile_m * gemm_n + col) * 2], summed in a fixed order.
+// lane; optionally the sums a BatchNorm next to the convolution needs, one pair per (row tile,
+// column) at stats[(tile_m * gemm_n + col) * 2], summed in a fixed order:
+//   forward:       sum and sum of squares of the values AS STORED (after rounding to T): the
+//                  batch statistics of the BatchNorm that follows;
+//   data gradient: the output g is the gradient behind a BatchNorm(+ReLU): it is rounded to T,
+//                  zeroed where bn_mask <= 0 (the ReLU), stored, and the pair is sum(g) and
+//                  sum(g * xhat), xhat = (bn_x - mean) * invstd: the two reductions of the
+//                  BatchNorm backward.
 // ---------------------------------------------------------------------------
 template <typename T, int MODE, int WM, int WN, int TM, int TN>
 __device__ inline void finish_tile(const IgemmArgs& p, f32x16_t (&acc)[TM][TN], float* stage, int tid, int m0, int n0,
@@ -200,12 +210,39 @@ __device__ inline void finish_tile(const IgemmArgs& p, f32x16_t (&acc)[TM][TN], 
   constexpr int CH = BN / E;   // column chunks of the tile; a thread always gets chunk tid % CH
   constexpr int ROWS = NT / CH;
   static_assert(NT % CH == 0, "stats mapping");
-  const bool want_stats = MODE == kFwd && p.stats != nullptr;
+  const bool want_stats = p.stats != nullptr;
   float st_sum[E], st_sq[E];
 #pragma unroll
   for (int e = 0; e < E; ++e) st_sum[e] = st_sq[e] = 0.f;
+  // data gradient with BatchNorm sums: the chunks of bn_x and bn_mask this thread will meet are
+  // requested up front, so that their latency overlaps the staging of the accumulators
+  constexpr int ITERS = (WM * 32 * CH) / NT;
+  constexpr int VISITS = TM * ITERS;
+  float bn_mu[E], bn_is[E];
+  uint4 pre_x[VISITS], pre_m[VISITS];
+  if (MODE == kDgrad && want_stats) {
+    const int col = n0 + (tid % CH) * E;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      bn_mu[e] = col < p.gemm_n ? p.bn_mean[col + e] : 0.f;
+      bn_is[e] = col < p.gemm_n ? p.bn_invstd[col + e] : 0.f;
+    }
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const int q = tid + it * NT;
+        const int r = q / CH;
+        const int row = m0 + ((r >> 5) * TM + tm) * 32 + (r & 31);
+        const bool ok = row < p.gemm_m && col < p.gemm_n;
+        const int64_t idx = static_cast<int64_t>(row) * p.gemm_n + col;
+        pre_x[tm * ITERS + it] = ok ? *reinterpret_cast<const uint4*>(static_cast<const T*>(p.bn_x) + idx) : make_uint4(0, 0, 0, 0);
+        pre_m[tm * ITERS + it] = (ok && p.bn_mask) ? *reinterpret_cast<const uint4*>(static_cast<const T*>(p.bn_mask) + idx)
+                                                   : make_uint4(0, 0, 0, 0);
+      }
+  }
 
-  staged_epilogue<T, WM, WN, TM, TN>(acc, stage, tid, [&](int tr, int tc, float* v) {
+  staged_epilogue<T, WM, WN, TM, TN>(acc, stage, tid, [&](int visit, int tr, int tc, float* v) {
     const int row = m0 + tr, col = n0 + tc;
     if (row >= p.gemm_m || col >= p.gemm_n) return;
     const int64_t idx = static_cast<int64_t>(row) * p.gemm_n + col;
@@ -232,16 +269,39 @@ __device__ inline void finish_tile(const IgemmArgs& p, f32x16_t (&acc)[TM][TN], 
     }
     if (p.out_f32) {
       store_floats<E>(static_cast<float*>(p.out) + idx, v);
-    } else {
-      const Chunk c = float_to_chunk<T>(v);
+    } else if (MODE == kDgrad && want_stats) {
+      Chunk c = float_to_chunk<T>(v);
+      chunk_to_float<T>(c, v);
+      Chunk cx;
+      cx.u = pre_x[visit];
+      if (p.bn_mask) {
+        Chunk cm;
+        cm.u = pre_m[visit];
+        float m[E];
+        chunk_to_float<T>(cm, m);
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+          if (!(m[e] > 0.f)) v[e] = 0.f;
+        c = float_to_chunk<T>(v);  // exact: every v[e] is a value of T
+      }
       *reinterpret_cast<uint4*>(static_cast<T*>(p.out) + idx) = c.u;
-      if (want_stats) chunk_to_float<T>(c, v);  // the statistics are those of the stored values
-    }
-    if (want_stats) {
+      float x[E];
+      chunk_to_float<T>(cx, x);
 #pragma unroll
       for (int e = 0; e < E; ++e) {
         st_sum[e] += v[e];
-        st_sq[e] += v[e] * v[e];
+        st_sq[e] += v[e] * ((x[e] - bn_mu[e]) * bn_is[e]);
+      }
+    } else {
+      const Chunk c = float_to_chunk<T>(v);
+      *reinterpret_cast<uint4*>(static_cast<T*>(p.out) + idx) = c.u;
+      if (want_stats) {
+        chunk_to_float<T>(c, v);  // the statistics are those of the stored values
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          st_sum[e] += v[e];
+          st_sq[e] += v[e] * v[e];
+        }
       }
     }
   });
@@ -636,7 +696,7 @@ __global__ __launch_bounds__(WM* WN * 64) void wgrad_kernel(IgemmArgs p) {
   float* out = static_cast<float*>(p.out);
   if (p.splits > 1) out += static_cast<int64_t>(split) * p.gemm_m * p.gemm_n;
   const bool accumulate = p.splits == 1 && p.accumulate;
-  staged_epilogue<T, WM, WN, TM, TN>(acc, reinterpret_cast<float*>(lds), tid, [&](int tr, int tc, float* v) {
+  staged_epilogue<T, WM, WN, TM, TN>(acc, reinterpret_cast<float*>(lds), tid, [&](int, int tr, int tc, float* v) {
     const int row = m0 + tr, col = n0 + tc;
     if (row >= p.gemm_m || col >= p.gemm_n) return;
     float* dst = out + static_cast<int64_t>(row) * p.gemm_n + col;
@@ -1084,11 +1144,27 @@ int conv2d_fwd_stat_rows(const ConvShape& s, int dtype, int tile_cfg) {
   return (gemm_m + bm - 1) / bm;
 }
 
+int conv2d_dgrad_stat_rows(const ConvShape& s, int dtype, int tile_cfg) {
+  (void)dtype;
+  const int gemm_m = s.N * s.H * s.W;
+  if (tile_cfg < 0) tile_cfg = pick_tile(gemm_m, s.C, 1);
+  const int bm = tile_cfg >= 2 ? 64 : 128;
+  return (gemm_m + bm - 1) / bm;
+}
+
 int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, const void* wt, void* dx,
-                 const void* add, const void* mask, int tile_cfg) {
+                 const void* add, const void* mask, int tile_cfg, const BnBwdSums* bn) {
   IgemmArgs a{};
   if (int rc = fill_common(a, s, dtype)) return rc;
   TCH_CHECK_ARG(dy && wt && dx, "conv2d_dgrad: null tensor");
+  if (bn) {
+    TCH_CHECK_ARG(bn->x && bn->mean && bn->invstd && bn->partial, "conv2d_dgrad: incomplete BatchNorm operands");
+    a.stats = bn->partial;
+    a.bn_mask = bn->mask;
+    a.bn_x = bn->x;
+    a.bn_mean = bn->mean;
+    a.bn_invstd = bn->invstd;
+  }
   const int eb = dtype == kBF16 ? 2 : 4;
   a.a_src = dy;
   a.b_src = wt;

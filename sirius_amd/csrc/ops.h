@@ -25,8 +25,18 @@ int conv2d_fwd(Context* ctx, int dtype, const ConvShape& s, const void* x, const
                const void* mask, const float* bias, int out_f32, int tile_cfg, float* bn_partial = nullptr);
 // rows of partial statistics conv2d_fwd writes for this shape and tiling (one per row tile)
 int conv2d_fwd_stat_rows(const ConvShape& s, int dtype, int tile_cfg);
+// The two reductions of a BatchNorm backward, taken in the epilogue of the data-gradient
+// convolution that produces the gradient behind that BatchNorm (+ReLU): see finish_tile.
+struct BnBwdSums {
+  const void* mask;     // optional ReLU output: the gradient is zeroed where mask <= 0 before it is stored
+  const void* x;        // the BatchNorm's input, laid out like dx
+  const float* mean;    // saved batch statistics, one per channel of dx
+  const float* invstd;
+  float* partial;       // [conv2d_dgrad_stat_rows][C][2]
+};
 int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, const void* w, void* dx,
-                 const void* add, const void* mask, int tile_cfg);
+                 const void* add, const void* mask, int tile_cfg, const BnBwdSums* bn = nullptr);
+int conv2d_dgrad_stat_rows(const ConvShape& s, int dtype, int tile_cfg);
 int conv2d_wgrad_pick_splits(const ConvShape& s, int dtype);
 int64_t conv2d_wgrad_workspace_bytes(const ConvShape& s, int dtype, int splits);
 int conv2d_wgrad(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* dy, float* dw,
@@ -47,6 +57,11 @@ int bn_fwd_train_partials(Context* ctx, int dtype, const void* x, void* y, const
 int bn_bwd(Context* ctx, int dtype, const void* dy, const void* relu_mask, const void* x, void* dx, int64_t rows,
            int C, const float* gamma, const float* save_mean, const float* save_invstd, float* dgamma, float* dbeta,
            int accumulate, float* workspace);
+// the same from the sums a convolution epilogue left ([row_blocks][C][2]); g is already gated by the
+// ReLU; scratch: 3*C floats
+int bn_bwd_partials(Context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int C,
+                    const float* gamma, const float* save_mean, const float* save_invstd, float* dgamma,
+                    float* dbeta, int accumulate, const float* partial, int row_blocks, float* scratch);
 
 // pool.hip
 int maxpool_fwd(Context* ctx, int dtype, const void* x, void* y, int32_t* index, int N, int H, int W, int C, int ksize,

@@ -192,6 +192,34 @@ def conv2d_dgrad(ctx, dy, wt, dx, stride, pad, add=None, mask=None, tile_cfg=-1,
                                  N, H, W, C, K, R, S, stride, pad, tile_cfg, c_logical), "tch_conv2d_dgrad")
 
 
+def conv2d_dgrad_stat_rows(dx, K, R, S, stride, pad, tile_cfg=-1):
+    N, H, W, C = dx.shape
+    return int(lib().tch_conv2d_dgrad_stat_rows(dtype_code(dx), N, H, W, C, K, R, S, stride, pad, tile_cfg))
+
+
+def conv2d_dgrad_bnsums(ctx, dy, wt, dx, stride, pad, bn_x, bn_mean, bn_invstd, partial, bn_mask=None, add=None,
+                        mask=None, tile_cfg=-1, c_logical=0):
+    """conv2d_dgrad whose output is the gradient behind a BatchNorm(+ReLU) with input bn_x and ReLU output
+    bn_mask: dx is stored already gated by the ReLU, and `partial` ([row tiles, C, 2] fp32) receives the two
+    reductions of that BatchNorm's backward.  Returns the number of row tiles."""
+    N, H, W, C = dx.shape
+    C2, R, S, K = wt.shape
+    assert C == C2
+    Ho, Wo = conv_out_hw(H, W, R, S, stride, pad)
+    assert tuple(dy.shape) == (N, Ho, Wo, K)
+    assert dy.dtype == wt.dtype == dx.dtype
+    for t in (add, mask, bn_mask, bn_x):
+        assert t is None or (t.shape == dx.shape and t.dtype == dx.dtype)
+    assert bn_x is not None and bn_mean.numel() == C and bn_invstd.numel() == C
+    assert bn_mean.dtype == bn_invstd.dtype == torch.float32
+    rb = conv2d_dgrad_stat_rows(dx, K, R, S, stride, pad, tile_cfg)
+    assert partial.dtype == torch.float32 and partial.numel() >= rb * C * 2
+    check(lib().tch_conv2d_dgrad_bnsums(ctx.handle, dtype_code(dy), _p(dy), _p(wt), _p(dx), _p(add), _p(mask),
+                                        N, H, W, C, K, R, S, stride, pad, tile_cfg, c_logical, _p(bn_mask), _p(bn_x),
+                                        _p(bn_mean), _p(bn_invstd), _p(partial)), "tch_conv2d_dgrad_bnsums")
+    return rb
+
+
 def conv2d_wgrad_splits(x, K, R, S, stride, pad):
     N, H, W, C = x.shape
     return int(lib().tch_conv2d_wgrad_pick_splits(dtype_code(x), N, H, W, C, K, R, S, stride, pad))
@@ -266,6 +294,18 @@ def bn_bwd(ctx, dy, x, dx, gamma, save_mean, save_invstd, dgamma, dbeta, workspa
     check(lib().tch_bn_bwd(ctx.handle, dtype_code(x), _p(dy), _p(relu_mask), _p(x), _p(dx), rows, C, _p(gamma),
                            _p(save_mean), _p(save_invstd), _p(dgamma), _p(dbeta), int(accumulate), _p(workspace)),
           "tch_bn_bwd")
+
+
+def bn_bwd_partials(ctx, g, x, dx, gamma, save_mean, save_invstd, dgamma, dbeta, partial, row_blocks, scratch,
+                    accumulate=False):
+    """bn_bwd from the sums conv2d_dgrad_bnsums left in `partial`; g is already gated by the ReLU."""
+    C = x.shape[-1]
+    rows = x.numel() // C
+    assert g.shape == x.shape == dx.shape and g.dtype == x.dtype == dx.dtype
+    assert partial.numel() >= row_blocks * C * 2 and scratch.numel() >= 3 * C
+    check(lib().tch_bn_bwd_partials(ctx.handle, dtype_code(x), _p(g), _p(x), _p(dx), rows, C, _p(gamma), _p(save_mean),
+                                    _p(save_invstd), _p(dgamma), _p(dbeta), int(accumulate), _p(partial),
+                                    int(row_blocks), _p(scratch)), "tch_bn_bwd_partials")
 
 
 # ---------------------------------------------------------------------------

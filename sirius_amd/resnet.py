@@ -48,7 +48,7 @@ class _Block:
 class ResNetEngine:
     def __init__(self, depths=(3, 8, 36, 3), num_classes=1000, width=64, dtype=torch.bfloat16, image_size=224,
                  lr=0.1, momentum=0.9, weight_decay=1e-4, bn_momentum=0.1, bn_eps=1e-5, stream=None, allocator=None,
-                 overlap_wgrad=True, fuse_bn_stats=True, autotune=False):
+                 overlap_wgrad=True, fuse_bn_stats=True, fuse_bn_bwd=True, autotune=False):
         if not torch.cuda.is_available():
             raise RuntimeError("ResNetEngine runs on the GPU only; there is no CPU path")
         assert dtype in (torch.bfloat16, torch.float32)
@@ -70,6 +70,9 @@ class ResNetEngine:
         # costs the recycling of the dy buffers (they stay alive until the lanes join)
         self.overlap_wgrad = overlap_wgrad
         self.fuse_bn_stats = fuse_bn_stats
+        # fuse_bn_bwd: a data-gradient convolution whose output flows into a BatchNorm(+ReLU) backward applies
+        # the ReLU gate and takes that BatchNorm's two reductions in its epilogue (no reduction pass)
+        self.fuse_bn_bwd = fuse_bn_bwd
         # autotune: when a plan is built, time each distinct convolution shape with every tiling and
         # keep the fastest (forward and data gradient separately); off = the library's heuristic
         self.autotune = autotune
@@ -278,10 +281,19 @@ class ResNetEngine:
                     ops.conv2d_fwd_bnstats(ctx, x, wgt, z, c.stride, c.pad, part, tile_cfg=cfg, c_logical=c.cin)
             return rec
 
+        mean, invstd = torch.zeros(c.cin_store, device=self.dev), torch.ones(c.cin_store, device=self.dev)
+        x2 = torch.ones_like(x)
+        dpart = torch.empty(ops.conv2d_dgrad_stat_rows(x, c.cout, c.k, c.k, c.stride, c.pad, 2) * c.cin_store * 2,
+                            dtype=torch.float32, device=self.dev)
+
         def dgrad(cfg):
             def rec():
                 for _ in range(reps):
-                    ops.conv2d_dgrad(ctx, z, wt, x, c.stride, c.pad, tile_cfg=cfg, c_logical=c.cin)
+                    if self.fuse_bn_bwd:   # nearly every data gradient of the plan runs in this form
+                        ops.conv2d_dgrad_bnsums(ctx, z, wt, x, c.stride, c.pad, x2, mean, invstd, dpart, bn_mask=x2,
+                                                tile_cfg=cfg, c_logical=c.cin)
+                    else:
+                        ops.conv2d_dgrad(ctx, z, wt, x, c.stride, c.pad, tile_cfg=cfg, c_logical=c.cin)
             return rec
         cfgs = (0, 1, 2, 3) if c.cout > 64 else (1, 2, 3)
         t_f = {cfg: self._time_program(fwd(cfg)) / reps for cfg in cfgs}
@@ -404,10 +416,11 @@ class ResNetEngine:
             xm = torch.empty((n_, h_, w_, c_.cin_store), dtype=T, device="meta")
             # sized for the smallest row tile, whichever tiling is picked
             stat_elems[0] = max(stat_elems[0],
-                                ops.conv2d_fwd_stat_rows(xm, c_.cout, c_.k, c_.k, c_.stride, c_.pad, 2) * c_.cout * 2)
+                                ops.conv2d_fwd_stat_rows(xm, c_.cout, c_.k, c_.k, c_.stride, c_.pad, 2) * c_.cout * 2,
+                                ops.conv2d_dgrad_stat_rows(xm, c_.cout, c_.k, c_.k, c_.stride, c_.pad, 2) * c_.cin_store * 2)
             tiles[c_.name] = self._tune_conv(c_, n_, h_, w_) if self.autotune else (-1, -1)
         stat_partial = act(max(stat_elems[0], 2), dtype=torch.float32)
-        bn_scratch = act(2 * max(c_.cout for c_, _ in conv_inputs), dtype=torch.float32)
+        bn_scratch = act(3 * max(max(c_.cout, c_.cin_store) for c_, _ in conv_inputs), dtype=torch.float32)
 
         def conv_bn_fwd(c, name, x, z, y, residual=None, relu=True):
             if not self.fuse_bn_stats:
@@ -434,6 +447,22 @@ class ResNetEngine:
         def conv_dgrad(c, dy, dx, **kw):
             ops.conv2d_dgrad(ctx, dy, self._wt(c.name + ".weight"), dx, c.stride, c.pad, c_logical=c.cin,
                              tile_cfg=tiles.get(c.name, (-1, -1))[1], **kw)
+
+        # data gradient -> BatchNorm backward pairs: conv_dgrad_bn leaves dx gated by the ReLU of the
+        # BatchNorm `name` (output `relu_out`, input `z`) together with its two reductions; bn_bwd_sums
+        # is that BatchNorm's backward from there (finalize + apply)
+        def conv_dgrad_bn(c, dy, dx, name, z, relu_out, **kw):
+            o, ch = self._bn_off[name]
+            return ops.conv2d_dgrad_bnsums(ctx, dy, self._wt(c.name + ".weight"), dx, c.stride, c.pad, z,
+                                           bn_save[o:o + ch], bn_save[nbn + o:nbn + o + ch], stat_partial,
+                                           bn_mask=relu_out, c_logical=c.cin,
+                                           tile_cfg=tiles.get(c.name, (-1, -1))[1], **kw)
+
+        def bn_bwd_sums(name, g, x, dx, rb):
+            o, c = self._bn_off[name]
+            ops.bn_bwd_partials(ctx, g, x, dx, self._view(self.params, name + ".weight"), bn_save[o:o + c],
+                                bn_save[nbn + o:nbn + o + c], self._view(self.grads, name + ".weight"),
+                                self._view(self.grads, name + ".bias"), stat_partial, rb, bn_scratch)
 
         prog = ops.Program()
         marks = []  # (launch index one past the layer, 'fwd' | 'bwd', layer name): checkpoint positions
@@ -493,40 +522,68 @@ class ResNetEngine:
             g_out = galloc((B, Hl, Wl, self.feat))
             ops.avgpool_bwd(ctx, g_pooled, g_out)
             gfree(g_pooled)
-            for blk, (H, W, Ho, Wo), sv in zip(reversed(self.blocks), reversed(shapes), reversed(saved)):
+            # g_rb: g_out is already gated by the block's final ReLU and stat_partial holds g_rb row tiles of
+            # the sums of this block's bn3 (left by the c1 data gradient of the block after it); None = neither
+            g_rb = None
+            fuse = self.fuse_bn_bwd
+            for bi in range(len(self.blocks) - 1, -1, -1):
+                blk, (H, W, Ho, Wo), sv = self.blocks[bi], shapes[bi], saved[bi]
                 xin, z1, a1, z2, a2, z3, zd, out = sv
                 P, pre = blk.planes, blk.prefix
                 dz3 = galloc(z3.shape)
-                bn_bwd(pre + ".bn3", g_out, z3, dz3, out)
+                if g_rb is None:
+                    bn_bwd(pre + ".bn3", g_out, z3, dz3, out)
+                else:
+                    bn_bwd_sums(pre + ".bn3", g_out, z3, dz3, g_rb)
+                out_gate = out if g_rb is None else None   # what still has to gate g_out
                 conv_wgrad(blk.c3, a2, dz3)
                 g_a2 = galloc(a2.shape)
-                conv_dgrad(blk.c3, dz3, g_a2)
-                mark("bwd", pre + ".conv3")
-                gfree(dz3, True)
                 dz2 = galloc(z2.shape)
-                bn_bwd(pre + ".bn2", g_a2, z2, dz2, a2)
+                if fuse:
+                    rb = conv_dgrad_bn(blk.c3, dz3, g_a2, pre + ".bn2", z2, a2)
+                    mark("bwd", pre + ".conv3")
+                    bn_bwd_sums(pre + ".bn2", g_a2, z2, dz2, rb)
+                else:
+                    conv_dgrad(blk.c3, dz3, g_a2)
+                    mark("bwd", pre + ".conv3")
+                    bn_bwd(pre + ".bn2", g_a2, z2, dz2, a2)
+                gfree(dz3, True)
                 gfree(g_a2)
                 conv_wgrad(blk.c2, a1, dz2)
                 g_a1 = galloc(a1.shape)
-                conv_dgrad(blk.c2, dz2, g_a1)
-                mark("bwd", pre + ".conv2")
-                gfree(dz2, True)
                 dz1 = galloc(z1.shape)
-                bn_bwd(pre + ".bn1", g_a1, z1, dz1, a1)
+                if fuse:
+                    rb = conv_dgrad_bn(blk.c2, dz2, g_a1, pre + ".bn1", z1, a1)
+                    mark("bwd", pre + ".conv2")
+                    bn_bwd_sums(pre + ".bn1", g_a1, z1, dz1, rb)
+                else:
+                    conv_dgrad(blk.c2, dz2, g_a1)
+                    mark("bwd", pre + ".conv2")
+                    bn_bwd(pre + ".bn1", g_a1, z1, dz1, a1)
+                gfree(dz2, True)
                 gfree(g_a1)
                 conv_wgrad(blk.c1, xin, dz1)
                 gx = galloc(xin.shape)
+                # xin is the output of the block before (its bn3 + residual + ReLU), whose bn3 input is z3 there
+                prev = (self.blocks[bi - 1].prefix + ".bn3", saved[bi - 1][5]) if (fuse and bi > 0) else None
                 if blk.cd is not None:
                     dzd = galloc(zd.shape)
-                    bn_bwd(pre + ".downsample.1", g_out, zd, dzd, out)
+                    bn_bwd(pre + ".downsample.1", g_out, zd, dzd, out_gate)
                     conv_wgrad(blk.cd, xin, dzd)
                     gx_id = galloc(xin.shape)
                     conv_dgrad(blk.cd, dzd, gx_id)
                     gfree(dzd, True)
-                    conv_dgrad(blk.c1, dz1, gx, add=gx_id)
-                    gfree(gx_id)
+                    add_kw = dict(add=gx_id)
                 else:
-                    conv_dgrad(blk.c1, dz1, gx, add=g_out, mask=out)
+                    gx_id = None
+                    add_kw = dict(add=g_out, mask=out_gate)
+                if prev is not None:
+                    g_rb = conv_dgrad_bn(blk.c1, dz1, gx, prev[0], prev[1], xin, **add_kw)
+                else:
+                    conv_dgrad(blk.c1, dz1, gx, **add_kw)
+                    g_rb = None
+                if gx_id is not None:
+                    gfree(gx_id)
                 mark("bwd", pre + ".conv1")
                 gfree(dz1, True)
                 gfree(g_out)

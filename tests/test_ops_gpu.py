@@ -243,6 +243,62 @@ def test_bn_bwd(ctx, dtype, rows, C, masked):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", [CONV_CASES[0], CONV_CASES[1], CONV_CASES[3], CONV_CASES[4], CONV_CASES[6]])
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3])
+@pytest.mark.parametrize("with_add", [False, True])
+def test_conv_dgrad_with_bn_backward_sums(ctx, dtype, case, tile_cfg, with_add):
+    """The data-gradient convolution gates its output by the ReLU of the BatchNorm it flows into and
+    leaves that BatchNorm's two reductions; the BatchNorm backward starts from them.  Checked against
+    the oracle's dgrad -> (ReLU gate) -> BatchNorm backward chain on the same inputs."""
+    from sirius_amd import ops
+    N, H, W, C, K, R, S, st, pad = case
+    print("case", case, dtype, tile_cfg, with_add, flush=True)
+    g = _gen(22)
+    Ho, Wo = ops.conv_out_hw(H, W, R, S, st, pad)
+    dy = rnd((N, Ho, Wo, K), dtype, g)
+    w = rnd((K, R, S, C), dtype, g, (R * S * K) ** -0.5)
+    add = rnd((N, H, W, C), dtype, g) if with_add else None
+    z = (rnd((N, H, W, C), dtype, g) * 1.3 - 0.2).to(dtype)     # the BatchNorm's input
+    relu_out = rnd((N, H, W, C), dtype, g)                        # its ReLU output: only the sign matters
+    gamma = torch.rand(C, generator=g) + 0.5
+    z2 = z.float().reshape(-1, C)
+    mean, invstd = z2.mean(0), 1.0 / torch.sqrt(z2.var(0, unbiased=False) + 1e-5)
+    # oracle chain; the gradient is rounded to the storage type between the two operators
+    g_ref = O.conv2d_dgrad(dy, w, (N, H, W, C), st, pad)
+    if with_add:
+        g_ref = g_ref + add.float()
+    g_ref = g_ref.to(dtype)
+    dz_ref, dg_ref, db_ref = O.bn_bwd(g_ref, z, gamma, relu_mask=relu_out)
+    gated_ref = g_ref.float() * (relu_out.float() > 0)
+
+    d = lambda t: t.cuda() if t is not None else None
+    gx = torch.empty((N, H, W, C), dtype=dtype, device="cuda")
+    rb = ops.conv2d_dgrad_stat_rows(gx, K, R, S, st, pad, tile_cfg)
+    partial = torch.full((rb * C * 2,), float("nan"), device="cuda")
+    zd = z.cuda()
+    got_rb = ops.conv2d_dgrad_bnsums(ctx, dy.cuda(), ops.filter_transpose(ctx, w.cuda()), gx, st, pad, zd, mean.cuda(),
+                                     invstd.cuda(), partial, bn_mask=relu_out.cuda(), add=d(add), tile_cfg=tile_cfg)
+    assert got_rb == rb
+    dz = torch.empty_like(gx)
+    dg, db = torch.zeros(C, device="cuda"), torch.zeros(C, device="cuda")
+    scratch = torch.empty(3 * C, device="cuda")
+    ops.bn_bwd_partials(ctx, gx, zd, dz, gamma.cuda(), mean.cuda(), invstd.cuda(), dg, db, partial, rb, scratch)
+    torch.cuda.synchronize()
+    close(gx, gated_ref, dtype, "gated gradient")
+    assert ((gx.float().cpu() == 0) | (relu_out.float() > 0)).all(), "the gradient must be zero behind a closed ReLU"
+    # the sums are those of what was stored, exactly
+    g32 = gx.float().cpu().reshape(-1, C).double()
+    xhat = (z2 - mean).double() * invstd.double()
+    sums = partial.cpu().reshape(rb, C, 2).double().sum(0)
+    close(sums[:, 0].float(), g32.sum(0).float(), torch.float32, "sum g", rtol=1e-4)
+    close(sums[:, 1].float(), (g32 * xhat).sum(0).float(), torch.float32, "sum g*xhat", rtol=1e-4)
+    tol = 1e-3 if dtype == torch.float32 else 2e-2
+    close(dg, dg_ref, torch.float32, "bn dgamma", rtol=tol)
+    close(db, db_ref, torch.float32, "bn dbeta", rtol=tol)
+    close(dz, dz_ref, dtype, "bn dx", rtol=tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("shape", [(2, 16, 16, 64), (1, 7, 9, 8), (3, 112, 112, 16)])
 def test_maxpool(ctx, dtype, shape):
     from sirius_amd import ops
