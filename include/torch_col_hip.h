@@ -184,6 +184,48 @@ int tch_fill_zero(tch_context* ctx, void* ptr, int64_t bytes);
 int tch_bias_grad(tch_context* ctx, int dtype, const void* dy, float* dbias, int rows, int cols, int ld,
                   int accumulate);
 
+/* ---- transformer operators (Swin-B / GPT-2 steps) --------------------------------------
+ * The arithmetic restates torch.nn.LayerNorm / GELU / softmax / AdamW / Embedding as the reference's
+ * training scripts use them through torchvision and transformers (train/swin_b.py:38-45,
+ * train/gpt2.py:26-33; a readable statement of window attention: train/swin_b_tiny.py:8-172). */
+/* y = (x - mean) * rstd * gamma + beta over the last dimension of [rows, C] (C <= 1024); mean / rstd [rows]
+ * are kept for the backward. */
+int tch_layernorm_fwd(tch_context* ctx, int dtype, const void* x, void* y, const float* gamma, const float* beta,
+                      float* mean, float* rstd, int64_t rows, int C, float eps);
+/* partial: fp32 scratch of tch_layernorm_bwd_partial_rows(rows) * C * 2 floats; dgamma / dbeta (+)= */
+int tch_layernorm_bwd_partial_rows(int64_t rows);
+int tch_layernorm_bwd(tch_context* ctx, int dtype, const void* dy, const void* x, void* dx, const float* gamma,
+                      const float* mean, const float* rstd, float* dgamma, float* dbeta, int accumulate, int64_t rows,
+                      int C, float* partial);
+/* tanh_form 0: 0.5 x (1 + erf(x / sqrt 2)) (nn.GELU); 1: GPT-2's gelu_new.  n is a multiple of a 16-byte chunk. */
+int tch_gelu_fwd(tch_context* ctx, int dtype, const void* x, void* y, int64_t n, int tanh_form);
+int tch_gelu_bwd(tch_context* ctx, int dtype, const void* dy, const void* x, void* dx, int64_t n, int tanh_form);
+/* probs = softmax over the last dimension of scale * scores[batch, heads, Lq, Lk] + bias[heads, Lq, Lk]
+ * + mask[windows, Lq, Lk] (window = batch index % windows); bias and mask may be NULL; causal != 0 keeps keys
+ * j <= i only (Lq == Lk).  In place (probs == scores) is allowed. */
+int tch_attn_softmax_fwd(tch_context* ctx, int dtype, const void* scores, void* probs, int64_t batch, int heads, int Lq,
+                         int Lk, float scale, const float* bias, const float* mask, int windows, int causal);
+/* dscores = scale * probs * (dprobs - sum_j dprobs_j probs_j) per row; rows = batch * heads * Lq. */
+int tch_attn_softmax_bwd(tch_context* ctx, int dtype, const void* probs, const void* dprobs, void* dscores, int64_t rows,
+                         int Lk, float scale);
+/* torch.optim.AdamW (decoupled decay, bias correction) over a flat fp32 buffer; step_dev (int32, starts at 0)
+ * and scalars_dev (2 floats) live on the device so that a recorded program advances the step by itself. */
+int tch_adamw_step(tch_context* ctx, float* param, const float* grad, float* exp_avg, float* exp_avg_sq,
+                   void* shadow_bf16, int64_t n, double lr, double beta1, double beta2, double eps, double weight_decay,
+                   int* step_dev, float* scalars_dev);
+/* out[b, t, :] = wte[ids[b, t], :] + wpe[t, :]; backward: dwte[id] += dy rows (fp32 atomics), dwpe (+)= sum over b. */
+int tch_embedding_fwd(tch_context* ctx, int dtype, const int64_t* ids, const void* wte, const void* wpe, void* out, int B,
+                      int T, int C, int vocab);
+int tch_embedding_bwd(tch_context* ctx, int dtype, const int64_t* ids, const void* dy, float* dwte, float* dwpe, int B,
+                      int T, int C, int vocab, int accumulate_wpe);
+/* C[z](m, n) (+)= alpha * sum_k A[z](m, k) B[z](n, k), z = zo * batch_inner + zi; A(m, k) at
+ * a + zo * a_bo + zi * a_bi + m * a_rs + k * a_cs (elements), B alike with n; C row-major with ldc.
+ * One stride of each operand must be 1. */
+int tch_batched_gemm(tch_context* ctx, int dtype, const void* a, const void* b, void* c, int M, int N, int K,
+                     int64_t a_rs, int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t ldc, int batch_outer,
+                     int batch_inner, int64_t a_bo, int64_t a_bi, int64_t b_bo, int64_t b_bi, int64_t c_bo, int64_t c_bi,
+                     float alpha, int accumulate);
+
 /* ---- layout / precision ---------------------------------------------------------- */
 int tch_nchw_to_nhwc_pad(tch_context* ctx, int dtype, const float* x_nchw, void* y_nhwc, int N, int C, int H, int W,
                          int Cpad);

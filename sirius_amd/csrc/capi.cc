@@ -208,6 +208,62 @@ int tch_bn_bwd_partials(tch_context* ctx, int dtype, const void* g, const void* 
                          partial, row_blocks, scratch);
 }
 
+int tch_layernorm_fwd(tch_context* ctx, int dtype, const void* x, void* y, const float* gamma, const float* beta,
+                      float* mean, float* rstd, int64_t rows, int Cc, float eps) {
+  return layernorm_fwd(C(ctx), dtype, x, y, gamma, beta, mean, rstd, rows, Cc, eps);
+}
+
+int tch_layernorm_bwd_partial_rows(int64_t rows) { return layernorm_bwd_partial_rows(rows); }
+
+int tch_layernorm_bwd(tch_context* ctx, int dtype, const void* dy, const void* x, void* dx, const float* gamma,
+                      const float* mean, const float* rstd, float* dgamma, float* dbeta, int accumulate, int64_t rows,
+                      int Cc, float* partial) {
+  return layernorm_bwd(C(ctx), dtype, dy, x, dx, gamma, mean, rstd, dgamma, dbeta, accumulate, rows, Cc, partial);
+}
+
+int tch_gelu_fwd(tch_context* ctx, int dtype, const void* x, void* y, int64_t n, int tanh_form) {
+  return gelu_fwd(C(ctx), dtype, x, y, n, tanh_form);
+}
+
+int tch_gelu_bwd(tch_context* ctx, int dtype, const void* dy, const void* x, void* dx, int64_t n, int tanh_form) {
+  return gelu_bwd(C(ctx), dtype, dy, x, dx, n, tanh_form);
+}
+
+int tch_attn_softmax_fwd(tch_context* ctx, int dtype, const void* scores, void* probs, int64_t batch, int heads, int Lq,
+                         int Lk, float scale, const float* bias, const float* mask, int windows, int causal) {
+  return attn_softmax_fwd(C(ctx), dtype, scores, probs, batch, heads, Lq, Lk, scale, bias, mask, windows, causal);
+}
+
+int tch_attn_softmax_bwd(tch_context* ctx, int dtype, const void* probs, const void* dprobs, void* dscores, int64_t rows,
+                         int Lk, float scale) {
+  return attn_softmax_bwd(C(ctx), dtype, probs, dprobs, dscores, rows, Lk, scale);
+}
+
+int tch_adamw_step(tch_context* ctx, float* param, const float* grad, float* exp_avg, float* exp_avg_sq,
+                   void* shadow_bf16, int64_t n, double lr, double beta1, double beta2, double eps, double weight_decay,
+                   int* step_dev, float* scalars_dev) {
+  return adamw_step(C(ctx), param, grad, exp_avg, exp_avg_sq, shadow_bf16, n, lr, beta1, beta2, eps, weight_decay,
+                    step_dev, scalars_dev);
+}
+
+int tch_embedding_fwd(tch_context* ctx, int dtype, const int64_t* ids, const void* wte, const void* wpe, void* out, int B,
+                      int T, int Cc, int vocab) {
+  return embedding_fwd(C(ctx), dtype, ids, wte, wpe, out, B, T, Cc, vocab);
+}
+
+int tch_embedding_bwd(tch_context* ctx, int dtype, const int64_t* ids, const void* dy, float* dwte, float* dwpe, int B,
+                      int T, int Cc, int vocab, int accumulate_wpe) {
+  return embedding_bwd(C(ctx), dtype, ids, dy, dwte, dwpe, B, T, Cc, vocab, accumulate_wpe);
+}
+
+int tch_batched_gemm(tch_context* ctx, int dtype, const void* a, const void* b, void* c, int M, int N, int K,
+                     int64_t a_rs, int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t ldc, int batch_outer,
+                     int batch_inner, int64_t a_bo, int64_t a_bi, int64_t b_bo, int64_t b_bi, int64_t c_bo, int64_t c_bi,
+                     float alpha, int accumulate) {
+  return batched_gemm(C(ctx), dtype, a, b, c, M, N, K, a_rs, a_cs, b_rs, b_cs, ldc, batch_outer, batch_inner, a_bo, a_bi,
+                      b_bo, b_bi, c_bo, c_bi, alpha, accumulate);
+}
+
 int tch_conv2d_wgrad_pick_splits(int dtype, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad) {
   return conv2d_wgrad_pick_splits(shape(N, H, W, Cc, K, R, S, stride, pad), dtype);
 }

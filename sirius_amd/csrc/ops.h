@@ -63,6 +63,32 @@ int bn_bwd_partials(Context* ctx, int dtype, const void* g, const void* x, void*
                     const float* gamma, const float* save_mean, const float* save_invstd, float* dgamma,
                     float* dbeta, int accumulate, const float* partial, int row_blocks, float* scratch);
 
+// seq_ops.hip
+int layernorm_fwd(Context* ctx, int dtype, const void* x, void* y, const float* gamma, const float* beta, float* mean,
+                  float* rstd, int64_t rows, int C, float eps);
+int layernorm_bwd_partial_rows(int64_t rows);  // rows of [C][2] fp32 scratch layernorm_bwd needs
+int layernorm_bwd(Context* ctx, int dtype, const void* dy, const void* x, void* dx, const float* gamma,
+                  const float* mean, const float* rstd, float* dgamma, float* dbeta, int accumulate, int64_t rows,
+                  int C, float* partial);
+int gelu_fwd(Context* ctx, int dtype, const void* x, void* y, int64_t n, int tanh_form);
+int gelu_bwd(Context* ctx, int dtype, const void* dy, const void* x, void* dx, int64_t n, int tanh_form);
+int attn_softmax_fwd(Context* ctx, int dtype, const void* scores, void* probs, int64_t batch, int heads, int Lq, int Lk,
+                     float scale, const float* bias, const float* mask, int windows, int causal);
+int attn_softmax_bwd(Context* ctx, int dtype, const void* probs, const void* dprobs, void* dscores, int64_t rows, int Lk,
+                     float scale);
+int adamw_step(Context* ctx, float* param, const float* grad, float* exp_avg, float* exp_avg_sq, void* shadow_bf16,
+               int64_t n, double lr, double beta1, double beta2, double eps, double weight_decay, int* step_dev,
+               float* scalars_dev);
+int embedding_fwd(Context* ctx, int dtype, const int64_t* ids, const void* wte, const void* wpe, void* out, int B, int T,
+                  int C, int vocab);
+int embedding_bwd(Context* ctx, int dtype, const int64_t* ids, const void* dy, float* dwte, float* dwpe, int B, int T,
+                  int C, int vocab, int accumulate_wpe);
+
+// bgemm.hip
+int batched_gemm(Context* ctx, int dtype, const void* a, const void* b, void* c, int M, int N, int K, int64_t a_rs,
+                 int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t ldc, int batch_outer, int batch_inner, int64_t a_bo,
+                 int64_t a_bi, int64_t b_bo, int64_t b_bi, int64_t c_bo, int64_t c_bi, float alpha, int accumulate);
+
 // pool.hip
 int maxpool_fwd(Context* ctx, int dtype, const void* x, void* y, int32_t* index, int N, int H, int W, int C, int ksize,
                 int stride, int pad);

@@ -1,0 +1,602 @@
+// Row-wise and elementwise operators of the transformer training steps (Swin-B, GPT-2):
+// LayerNorm, GELU (exact erf and the tanh form), attention softmax (scale, additive bias,
+// window mask, causal), AdamW with a bf16 shadow copy, token + position embedding.
+// All HBM-bound: 16-byte chunks per lane, one wavefront per row for the row-wise ones.
+//
+// Restated arithmetic and its reference call sites (the arithmetic itself lives in PyTorch /
+// torchvision / transformers, which the reference calls):
+//   nn.LayerNorm(eps 1e-5), nn.GELU, window attention softmax with relative position bias
+//   and the shift mask                        train/swin_b_tiny.py:8-172, train/swin_b.py:38
+//   GPT-2 gelu_new, causal attention, wte + wpe   train/gpt2.py:26
+//   torch.optim.AdamW                         train/gpt2.py:31, train/swin_b.py:43 (variants)
+#include "kernels.h"
+#include "ops.h"
+
+namespace tch {
+namespace {
+
+unsigned flat_blocks(int64_t items, int64_t cap = 8192) {
+  int64_t b = (items + 255) / 256;
+  if (b > cap) b = cap;
+  if (b < 1) b = 1;
+  return static_cast<unsigned>(b);
+}
+
+// ---------------------------------------------------------------------------
+// LayerNorm over the last dimension of [rows, C]
+// ---------------------------------------------------------------------------
+constexpr int kLnMaxC = 1024;  // longest row: a lane holds 16 elements of it
+template <typename T>
+struct LnChunks {
+  static constexpr int kMax = kLnMaxC / 64 / Elem<T>::kPerChunk;  // 16-byte chunks per lane and row
+};
+
+struct LnArgs {
+  const void* x;
+  const void* dy;  // backward
+  void* out;       // forward: y   backward: dx
+  const float* gamma;
+  const float* beta;
+  float* mean;   // [rows]  forward: written   backward: read
+  float* rstd;   // [rows]
+  float* partial;  // backward: [gridDim.x][C][2] = per-workgroup (sum dy*xhat, sum dy)
+  int64_t rows;
+  int C, cc;
+  int rows_per_wg;
+  float eps;
+};
+
+// one wavefront per row; the row stays in registers between the passes
+template <typename T>
+__global__ __launch_bounds__(256) void ln_fwd_kernel(LnArgs p) {
+  constexpr int E = Elem<T>::kPerChunk;
+  constexpr int kLnMaxChunks = LnChunks<T>::kMax;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + wave;
+  if (row >= p.rows) return;
+  const uint4* src = static_cast<const uint4*>(p.x) + row * p.cc;
+  float v[kLnMaxChunks][E];
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < kLnMaxChunks; ++j) {
+    const int c = lane + j * 64;
+    if (c < p.cc) {
+      Chunk ch;
+      ch.u = src[c];
+      chunk_to_float<T>(ch, v[j]);
+#pragma unroll
+      for (int e = 0; e < E; ++e) s += v[j][e];
+    }
+  }
+  const float mean = wave_sum(s) / static_cast<float>(p.C);
+  float q = 0.f;
+#pragma unroll
+  for (int j = 0; j < kLnMaxChunks; ++j) {
+    if (lane + j * 64 < p.cc) {
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        const float d = v[j][e] - mean;
+        q += d * d;
+      }
+    }
+  }
+  const float rstd = 1.0f / sqrtf(wave_sum(q) / static_cast<float>(p.C) + p.eps);
+  if (lane == 0) {
+    p.mean[row] = mean;
+    p.rstd[row] = rstd;
+  }
+  uint4* dst = static_cast<uint4*>(p.out) + row * p.cc;
+#pragma unroll
+  for (int j = 0; j < kLnMaxChunks; ++j) {
+    const int c = lane + j * 64;
+    if (c < p.cc) {
+      float o[E];
+#pragma unroll
+      for (int e = 0; e < E; ++e) o[e] = (v[j][e] - mean) * rstd * p.gamma[c * E + e] + p.beta[c * E + e];
+      dst[c] = float_to_chunk<T>(o).u;
+    }
+  }
+}
+
+// dx per row; the column sums for dgamma / dbeta are kept per lane over the rows a wave
+// walks, then summed over the four waves through LDS: one partial row per workgroup
+template <typename T>
+__global__ __launch_bounds__(256) void ln_bwd_kernel(LnArgs p) {
+  constexpr int E = Elem<T>::kPerChunk;
+  constexpr int kLnMaxChunks = LnChunks<T>::kMax;
+  __shared__ float red[4][kLnMaxC * 2];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  float dg[kLnMaxChunks][E], db[kLnMaxChunks][E], gam[kLnMaxChunks][E];
+#pragma unroll
+  for (int j = 0; j < kLnMaxChunks; ++j)
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      dg[j][e] = db[j][e] = 0.f;
+      const int c = lane + j * 64;
+      gam[j][e] = c < p.cc ? p.gamma[c * E + e] : 0.f;
+    }
+  const int64_t r0 = static_cast<int64_t>(blockIdx.x) * p.rows_per_wg;
+  int64_t r1 = r0 + p.rows_per_wg;
+  if (r1 > p.rows) r1 = p.rows;
+  const float inv_c = 1.0f / static_cast<float>(p.C);
+  for (int64_t row = r0 + wave; row < r1; row += 4) {
+    const uint4* xs = static_cast<const uint4*>(p.x) + row * p.cc;
+    const uint4* gs = static_cast<const uint4*>(p.dy) + row * p.cc;
+    const float mean = p.mean[row], rstd = p.rstd[row];
+    float xh[kLnMaxChunks][E], g[kLnMaxChunks][E];
+    float a = 0.f, b = 0.f;
+#pragma unroll
+    for (int j = 0; j < kLnMaxChunks; ++j) {
+      const int c = lane + j * 64;
+      if (c < p.cc) {
+        Chunk cx, cg;
+        cx.u = xs[c];
+        cg.u = gs[c];
+        chunk_to_float<T>(cx, xh[j]);
+        chunk_to_float<T>(cg, g[j]);
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          xh[j][e] = (xh[j][e] - mean) * rstd;
+          dg[j][e] += g[j][e] * xh[j][e];
+          db[j][e] += g[j][e];
+          g[j][e] *= gam[j][e];
+          a += g[j][e];
+          b += g[j][e] * xh[j][e];
+        }
+      }
+    }
+    a = wave_sum(a) * inv_c;
+    b = wave_sum(b) * inv_c;
+    uint4* dst = static_cast<uint4*>(p.out) + row * p.cc;
+#pragma unroll
+    for (int j = 0; j < kLnMaxChunks; ++j) {
+      const int c = lane + j * 64;
+      if (c < p.cc) {
+        float o[E];
+#pragma unroll
+        for (int e = 0; e < E; ++e) o[e] = rstd * (g[j][e] - a - xh[j][e] * b);
+        dst[c] = float_to_chunk<T>(o).u;
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < kLnMaxChunks; ++j)
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      red[wave][((j * 64 + lane) * E + e) * 2] = dg[j][e];
+      red[wave][((j * 64 + lane) * E + e) * 2 + 1] = db[j][e];
+    }
+  __syncthreads();
+  // column col lives at chunk c = col / E -> (j = c / 64, lane = c % 64), element col % E
+  for (int col = threadIdx.x; col < p.C; col += 256) {
+    const int c = col / E, e = col - c * E;
+    const int j = c >> 6, l = c & 63;
+    const int at = ((j * 64 + l) * E + e) * 2;
+    const float sg = red[0][at] + red[1][at] + red[2][at] + red[3][at];
+    const float sb = red[0][at + 1] + red[1][at + 1] + red[2][at + 1] + red[3][at + 1];
+    float2* dst = reinterpret_cast<float2*>(p.partial + (static_cast<int64_t>(blockIdx.x) * p.C + col) * 2);
+    *dst = make_float2(sg, sb);
+  }
+}
+
+struct ColSumArgs {
+  const float* partial;  // [blocks][C][2]
+  float* out0;           // (+)= sum_b partial[b][c][0]
+  float* out1;           // (+)= sum_b partial[b][c][1]
+  int blocks, C, accumulate;
+};
+
+// 8 columns x 32 lanes per workgroup, fp64 sums in a fixed order
+__global__ __launch_bounds__(256) void col_sum_kernel(ColSumArgs p) {
+  __shared__ double red[32][8][2];
+  const int cl = threadIdx.x & 7, lane = threadIdx.x >> 3;
+  const int c = blockIdx.x * 8 + cl;
+  double s = 0.0, q = 0.0;
+  if (c < p.C) {
+    constexpr int U = 8;
+    for (int b = lane; b < p.blocks; b += U * 32) {
+      float2 v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int bb = b + u * 32;
+        v[u] = bb < p.blocks ? *reinterpret_cast<const float2*>(p.partial + (static_cast<int64_t>(bb) * p.C + c) * 2)
+                             : make_float2(0.f, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        s += v[u].x;
+        q += v[u].y;
+      }
+    }
+  }
+  red[lane][cl][0] = s;
+  red[lane][cl][1] = q;
+  __syncthreads();
+  for (int off = 16; off > 0; off >>= 1) {
+    if (lane < off) {
+      red[lane][cl][0] += red[lane + off][cl][0];
+      red[lane][cl][1] += red[lane + off][cl][1];
+    }
+    __syncthreads();
+  }
+  if (lane == 0 && c < p.C) {
+    const float a = static_cast<float>(red[0][cl][0]), b = static_cast<float>(red[0][cl][1]);
+    p.out0[c] = p.accumulate ? p.out0[c] + a : a;
+    p.out1[c] = p.accumulate ? p.out1[c] + b : b;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// GELU
+// ---------------------------------------------------------------------------
+struct GeluArgs {
+  const void* x;
+  const void* dy;  // backward
+  void* out;
+  int64_t chunks;
+  int tanh_form;
+};
+
+__device__ inline float gelu_value(float x, int tanh_form) {
+  if (tanh_form) {
+    const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+    return 0.5f * x * (1.0f + tanhf(u));
+  }
+  return 0.5f * x * (1.0f + erff(x * 0.7071067811865476f));
+}
+
+__device__ inline float gelu_slope(float x, int tanh_form) {
+  if (tanh_form) {
+    const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+    const float t = tanhf(u);
+    return 0.5f * (1.0f + t) + 0.5f * x * (1.0f - t * t) * 0.7978845608028654f * (1.0f + 3.0f * 0.044715f * x * x);
+  }
+  return 0.5f * (1.0f + erff(x * 0.7071067811865476f)) + x * 0.3989422804014327f * expf(-0.5f * x * x);
+}
+
+template <typename T, int BWD>
+__global__ __launch_bounds__(256) void gelu_kernel(GeluArgs p) {
+  constexpr int E = Elem<T>::kPerChunk;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < p.chunks; i += stride) {
+    Chunk cx;
+    cx.u = static_cast<const uint4*>(p.x)[i];
+    float x[E], o[E];
+    chunk_to_float<T>(cx, x);
+    if (BWD) {
+      Chunk cg;
+      cg.u = static_cast<const uint4*>(p.dy)[i];
+      float g[E];
+      chunk_to_float<T>(cg, g);
+#pragma unroll
+      for (int e = 0; e < E; ++e) o[e] = g[e] * gelu_slope(x[e], p.tanh_form);
+    } else {
+#pragma unroll
+      for (int e = 0; e < E; ++e) o[e] = gelu_value(x[e], p.tanh_form);
+    }
+    static_cast<uint4*>(p.out)[i] = float_to_chunk<T>(o).u;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// attention softmax over rows of [batch, heads, Lq, Lk]
+// ---------------------------------------------------------------------------
+struct SoftmaxArgs {
+  const void* s;      // forward: scores        backward: probabilities
+  const void* dp;     // backward: gradient of the probabilities
+  void* out;          // forward: probabilities backward: gradient of the scores
+  const float* bias;  // optional [heads][Lq][Lk], added after scaling
+  const float* mask;  // optional [windows][Lq][Lk], added after scaling; window = batch % windows
+  int64_t rows;       // batch * heads * Lq
+  int heads, Lq, Lk, windows, causal;
+  float scale;
+};
+
+// one wavefront per row, four rows per workgroup
+template <typename T, int BWD>
+__global__ __launch_bounds__(256) void attn_softmax_kernel(SoftmaxArgs p) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + wave;
+  if (row >= p.rows) return;
+  const T* src = static_cast<const T*>(p.s) + row * p.Lk;
+  T* dst = static_cast<T*>(p.out) + row * p.Lk;
+  if (BWD) {
+    const T* dp = static_cast<const T*>(p.dp) + row * p.Lk;
+    float dot = 0.f;
+    for (int j = lane; j < p.Lk; j += 64) dot += Elem<T>::load(src + j) * Elem<T>::load(dp + j);
+    dot = wave_sum(dot);
+    for (int j = lane; j < p.Lk; j += 64)
+      Elem<T>::store(dst + j, p.scale * Elem<T>::load(src + j) * (Elem<T>::load(dp + j) - dot));
+    return;
+  }
+  const int i = static_cast<int>(row % p.Lq);
+  const int64_t bh = row / p.Lq;
+  const int h = static_cast<int>(bh % p.heads);
+  const int64_t b = bh / p.heads;
+  const float* bias = p.bias ? p.bias + (static_cast<int64_t>(h) * p.Lq + i) * p.Lk : nullptr;
+  const float* mask = p.mask ? p.mask + (static_cast<int64_t>(b % p.windows) * p.Lq + i) * p.Lk : nullptr;
+  const int limit = p.causal ? (i + 1 < p.Lk ? i + 1 : p.Lk) : p.Lk;  // keys [0, limit) take part
+  auto logit = [&](int j) {
+    float v = Elem<T>::load(src + j) * p.scale;
+    if (bias) v += bias[j];
+    if (mask) v += mask[j];
+    return v;
+  };
+  float mx = -INFINITY;
+  for (int j = lane; j < limit; j += 64) mx = fmaxf(mx, logit(j));
+  mx = wave_max(mx);
+  float sum = 0.f;
+  for (int j = lane; j < limit; j += 64) sum += expf(logit(j) - mx);
+  sum = wave_sum(sum);
+  const float inv = 1.0f / sum;
+  for (int j = lane; j < p.Lk; j += 64) Elem<T>::store(dst + j, j < limit ? expf(logit(j) - mx) * inv : 0.f);
+}
+
+// ---------------------------------------------------------------------------
+// AdamW over a flat fp32 parameter buffer with a bf16 shadow
+// ---------------------------------------------------------------------------
+struct AdamTickArgs {
+  int* step;       // device step counter, incremented here
+  float* scalars;  // [0] = 1 - beta1^t, [1] = sqrt(1 - beta2^t)
+  double beta1, beta2;
+};
+
+__global__ void adamw_tick_kernel(AdamTickArgs p) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  const int t = *p.step + 1;
+  *p.step = t;
+  p.scalars[0] = static_cast<float>(1.0 - pow(p.beta1, static_cast<double>(t)));
+  p.scalars[1] = static_cast<float>(sqrt(1.0 - pow(p.beta2, static_cast<double>(t))));
+}
+
+struct AdamArgs {
+  float* param;
+  const float* grad;
+  float* m;
+  float* v;
+  uint16_t* shadow;
+  const float* scalars;
+  int64_t n;
+  // every constant is rounded to fp32 once, from the double the caller gave (1 - beta as well:
+  // 1 - 0.999f is off by 1e-5 relative)
+  float lr, beta2, one_minus_beta1, one_minus_beta2, eps, decay;
+};
+
+__global__ __launch_bounds__(256) void adamw_kernel(AdamArgs p) {
+  const float bc1 = p.scalars[0], bc2_sqrt = p.scalars[1];
+  const float step_size = p.lr / bc1;
+  const float decay = p.decay;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < p.n; i += stride) {
+    const float g = p.grad[i];
+    float w = p.param[i] * decay;
+    float m = p.m[i];
+    m = m + (g - m) * p.one_minus_beta1;
+    const float v = p.v[i] * p.beta2 + p.one_minus_beta2 * g * g;
+    const float denom = sqrtf(v) / bc2_sqrt + p.eps;
+    w -= step_size * (m / denom);
+    p.param[i] = w;
+    p.m[i] = m;
+    p.v[i] = v;
+    if (p.shadow) p.shadow[i] = float_to_bf16_bits(w);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// token + position embedding
+// ---------------------------------------------------------------------------
+struct EmbedArgs {
+  const int64_t* ids;  // [B*T]
+  const void* wte;     // [vocab][C]   (forward, T)
+  const void* wpe;     // [>=T][C]
+  void* out;           // [B*T][C]     (forward)
+  const void* dy;      // [B*T][C]     (backward)
+  float* dwte;         // [vocab][C] fp32, += (backward)
+  float* dwpe;         // [T][C] fp32, (+)= (backward)
+  int64_t tokens;
+  int T, C, cc, vocab, B, accumulate;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void embed_fwd_kernel(EmbedArgs p) {
+  constexpr int E = Elem<T>::kPerChunk;
+  const int64_t total = p.tokens * p.cc;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += stride) {
+    const int64_t tok = i / p.cc;
+    const int c = static_cast<int>(i - tok * p.cc);
+    const int t = static_cast<int>(tok % p.T);
+    int64_t id = p.ids[tok];
+    if (id < 0 || id >= p.vocab) id = 0;  // ids are validated on the host; never read outside the table
+    Chunk a, b;
+    a.u = static_cast<const uint4*>(p.wte)[id * p.cc + c];
+    b.u = static_cast<const uint4*>(p.wpe)[static_cast<int64_t>(t) * p.cc + c];
+    float va[E], vb[E];
+    chunk_to_float<T>(a, va);
+    chunk_to_float<T>(b, vb);
+#pragma unroll
+    for (int e = 0; e < E; ++e) va[e] += vb[e];
+    static_cast<uint4*>(p.out)[i] = float_to_chunk<T>(va).u;
+  }
+}
+
+// dwpe[t] = sum over the batch (fixed order); dwte[id] += dy row (fp32 atomics: rows that share a
+// token meet in an order that may differ between runs)
+template <typename T>
+__global__ __launch_bounds__(256) void embed_bwd_kernel(EmbedArgs p) {
+  constexpr int E = Elem<T>::kPerChunk;
+  const int64_t per_batch = static_cast<int64_t>(p.T) * p.cc;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < per_batch; i += stride) {
+    const int t = static_cast<int>(i / p.cc);
+    const int c = static_cast<int>(i - static_cast<int64_t>(t) * p.cc);
+    float acc[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) acc[e] = 0.f;
+    for (int b = 0; b < p.B; ++b) {
+      const int64_t tok = static_cast<int64_t>(b) * p.T + t;
+      Chunk g;
+      g.u = static_cast<const uint4*>(p.dy)[tok * p.cc + c];
+      float v[E];
+      chunk_to_float<T>(g, v);
+      int64_t id = p.ids[tok];
+      if (id < 0 || id >= p.vocab) id = 0;
+      float* row = p.dwte + id * p.C + c * E;
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        acc[e] += v[e];
+        atomicAdd(row + e, v[e]);
+      }
+    }
+    float* dst = p.dwpe + static_cast<int64_t>(t) * p.C + c * E;
+#pragma unroll
+    for (int e = 0; e < E; ++e) dst[e] = p.accumulate ? dst[e] + acc[e] : acc[e];
+  }
+}
+
+int check_rows(const char* what, int dtype, int64_t rows, int C) {
+  TCH_CHECK_ARG(dtype == kBF16 || dtype == kF32, std::string(what) + ": dtype must be f32(0) or bf16(1)");
+  const int E = dtype == kBF16 ? 8 : 4;
+  TCH_CHECK_ARG(rows > 0 && C > 0 && C % E == 0, std::string(what) + ": C must be a positive multiple of a 16-byte chunk");
+  return 0;
+}
+
+int ln_rows_per_wg(int64_t rows) {
+  int64_t r = (rows + 1023) / 1024;
+  r = (r + 3) / 4 * 4;
+  return static_cast<int>(r < 4 ? 4 : r);
+}
+
+}  // namespace
+
+int layernorm_bwd_partial_rows(int64_t rows) {
+  const int r = ln_rows_per_wg(rows);
+  return static_cast<int>((rows + r - 1) / r);
+}
+
+int layernorm_fwd(Context* ctx, int dtype, const void* x, void* y, const float* gamma, const float* beta, float* mean,
+                  float* rstd, int64_t rows, int C, float eps) {
+  if (int rc = check_rows("layernorm_fwd", dtype, rows, C)) return rc;
+  const int E = dtype == kBF16 ? 8 : 4;
+  TCH_CHECK_ARG(C <= kLnMaxC, "layernorm: rows longer than 1024 elements are not supported");
+  TCH_CHECK_ARG(x && y && gamma && beta && mean && rstd, "layernorm_fwd: null tensor");
+  LnArgs a{x, nullptr, y, gamma, beta, mean, rstd, nullptr, rows, C, C / E, 0, eps};
+  const double bytes = static_cast<double>(rows) * C * (dtype == kBF16 ? 4.0 : 8.0);
+  const dim3 grid(static_cast<unsigned>((rows + 3) / 4));
+  return dtype == kBF16 ? launch(ctx, ln_fwd_kernel<bf16>, grid, dim3(256), a, "ln_fwd_kernel<bf16>", bytes, 1)
+                        : launch(ctx, ln_fwd_kernel<float>, grid, dim3(256), a, "ln_fwd_kernel<f32>", bytes, 1);
+}
+
+int layernorm_bwd(Context* ctx, int dtype, const void* dy, const void* x, void* dx, const float* gamma,
+                  const float* mean, const float* rstd, float* dgamma, float* dbeta, int accumulate, int64_t rows,
+                  int C, float* partial) {
+  if (int rc = check_rows("layernorm_bwd", dtype, rows, C)) return rc;
+  const int E = dtype == kBF16 ? 8 : 4;
+  TCH_CHECK_ARG(C <= kLnMaxC, "layernorm: rows longer than 1024 elements are not supported");
+  TCH_CHECK_ARG(dy && x && dx && gamma && mean && rstd && dgamma && dbeta && partial, "layernorm_bwd: null tensor");
+  const int rpw = ln_rows_per_wg(rows);
+  const int blocks = static_cast<int>((rows + rpw - 1) / rpw);
+  LnArgs a{x, dy, dx, gamma, nullptr, const_cast<float*>(mean), const_cast<float*>(rstd), partial, rows, C, C / E, rpw, 0.f};
+  const double bytes = static_cast<double>(rows) * C * (dtype == kBF16 ? 6.0 : 12.0);
+  int rc = dtype == kBF16 ? launch(ctx, ln_bwd_kernel<bf16>, dim3(blocks), dim3(256), a, "ln_bwd_kernel<bf16>", bytes, 1)
+                          : launch(ctx, ln_bwd_kernel<float>, dim3(blocks), dim3(256), a, "ln_bwd_kernel<f32>", bytes, 1);
+  if (rc) return rc;
+  ColSumArgs s{partial, dgamma, dbeta, blocks, C, accumulate};
+  return launch(ctx, col_sum_kernel, dim3((C + 7) / 8), dim3(256), s, "col_sum_kernel", 8.0 * blocks * C, 1);
+}
+
+int gelu_fwd(Context* ctx, int dtype, const void* x, void* y, int64_t n, int tanh_form) {
+  TCH_CHECK_ARG(dtype == kBF16 || dtype == kF32, "gelu_fwd: dtype must be f32(0) or bf16(1)");
+  const int E = dtype == kBF16 ? 8 : 4;
+  TCH_CHECK_ARG(x && y && n > 0 && n % E == 0, "gelu_fwd: null tensor, or a size that is not a multiple of a 16-byte chunk");
+  GeluArgs a{x, nullptr, y, n / E, tanh_form};
+  const double bytes = static_cast<double>(n) * (dtype == kBF16 ? 4.0 : 8.0);
+  const dim3 grid(flat_blocks(a.chunks));
+  return dtype == kBF16 ? launch(ctx, gelu_kernel<bf16, 0>, grid, dim3(256), a, "gelu_kernel<bf16,fwd>", bytes, 1)
+                        : launch(ctx, gelu_kernel<float, 0>, grid, dim3(256), a, "gelu_kernel<f32,fwd>", bytes, 1);
+}
+
+int gelu_bwd(Context* ctx, int dtype, const void* dy, const void* x, void* dx, int64_t n, int tanh_form) {
+  TCH_CHECK_ARG(dtype == kBF16 || dtype == kF32, "gelu_bwd: dtype must be f32(0) or bf16(1)");
+  const int E = dtype == kBF16 ? 8 : 4;
+  TCH_CHECK_ARG(dy && x && dx && n > 0 && n % E == 0, "gelu_bwd: null tensor, or a size that is not a multiple of a 16-byte chunk");
+  GeluArgs a{x, dy, dx, n / E, tanh_form};
+  const double bytes = static_cast<double>(n) * (dtype == kBF16 ? 6.0 : 12.0);
+  const dim3 grid(flat_blocks(a.chunks));
+  return dtype == kBF16 ? launch(ctx, gelu_kernel<bf16, 1>, grid, dim3(256), a, "gelu_kernel<bf16,bwd>", bytes, 1)
+                        : launch(ctx, gelu_kernel<float, 1>, grid, dim3(256), a, "gelu_kernel<f32,bwd>", bytes, 1);
+}
+
+int attn_softmax_fwd(Context* ctx, int dtype, const void* scores, void* probs, int64_t batch, int heads, int Lq, int Lk,
+                     float scale, const float* bias, const float* mask, int windows, int causal) {
+  TCH_CHECK_ARG(dtype == kBF16 || dtype == kF32, "attn_softmax: dtype must be f32(0) or bf16(1)");
+  TCH_CHECK_ARG(scores && probs && batch > 0 && heads > 0 && Lq > 0 && Lk > 0, "attn_softmax_fwd: bad arguments");
+  TCH_CHECK_ARG(!mask || (windows > 0 && batch % windows == 0), "attn_softmax_fwd: batch must be a multiple of the windows");
+  TCH_CHECK_ARG(!causal || Lq == Lk, "attn_softmax_fwd: the causal form needs square score matrices");
+  SoftmaxArgs a{scores, nullptr, probs, bias, mask, batch * heads * Lq, heads, Lq, Lk, mask ? windows : 1, causal, scale};
+  const double bytes = static_cast<double>(a.rows) * Lk * (dtype == kBF16 ? 4.0 : 8.0);
+  const dim3 grid(static_cast<unsigned>((a.rows + 3) / 4));
+  return dtype == kBF16 ? launch(ctx, attn_softmax_kernel<bf16, 0>, grid, dim3(256), a, "attn_softmax_kernel<bf16,fwd>", bytes, 1)
+                        : launch(ctx, attn_softmax_kernel<float, 0>, grid, dim3(256), a, "attn_softmax_kernel<f32,fwd>", bytes, 1);
+}
+
+int attn_softmax_bwd(Context* ctx, int dtype, const void* probs, const void* dprobs, void* dscores, int64_t rows, int Lk,
+                     float scale) {
+  TCH_CHECK_ARG(dtype == kBF16 || dtype == kF32, "attn_softmax: dtype must be f32(0) or bf16(1)");
+  TCH_CHECK_ARG(probs && dprobs && dscores && rows > 0 && Lk > 0, "attn_softmax_bwd: bad arguments");
+  SoftmaxArgs a{probs, dprobs, dscores, nullptr, nullptr, rows, 1, 1, Lk, 1, 0, scale};
+  const double bytes = static_cast<double>(rows) * Lk * (dtype == kBF16 ? 6.0 : 12.0);
+  const dim3 grid(static_cast<unsigned>((rows + 3) / 4));
+  return dtype == kBF16 ? launch(ctx, attn_softmax_kernel<bf16, 1>, grid, dim3(256), a, "attn_softmax_kernel<bf16,bwd>", bytes, 1)
+                        : launch(ctx, attn_softmax_kernel<float, 1>, grid, dim3(256), a, "attn_softmax_kernel<f32,bwd>", bytes, 1);
+}
+
+int adamw_step(Context* ctx, float* param, const float* grad, float* exp_avg, float* exp_avg_sq, void* shadow_bf16,
+               int64_t n, double lr, double beta1, double beta2, double eps, double weight_decay, int* step_dev,
+               float* scalars_dev) {
+  TCH_CHECK_ARG(param && grad && exp_avg && exp_avg_sq && step_dev && scalars_dev && n > 0, "adamw_step: null tensor or empty");
+  AdamTickArgs t{step_dev, scalars_dev, beta1, beta2};
+  if (int rc = launch(ctx, adamw_tick_kernel, dim3(1), dim3(64), t, "adamw_tick_kernel", 12.0, 1)) return rc;
+  AdamArgs a{param,
+             grad,
+             exp_avg,
+             exp_avg_sq,
+             static_cast<uint16_t*>(shadow_bf16),
+             scalars_dev,
+             n,
+             static_cast<float>(lr),
+             static_cast<float>(beta2),
+             static_cast<float>(1.0 - beta1),
+             static_cast<float>(1.0 - beta2),
+             static_cast<float>(eps),
+             static_cast<float>(1.0 - lr * weight_decay)};
+  return launch(ctx, adamw_kernel, dim3(flat_blocks(n)), dim3(256), a, "adamw_kernel",
+                static_cast<double>(n) * (shadow_bf16 ? 30.0 : 28.0), 1);
+}
+
+int embedding_fwd(Context* ctx, int dtype, const int64_t* ids, const void* wte, const void* wpe, void* out, int B, int T,
+                  int C, int vocab) {
+  if (int rc = check_rows("embedding_fwd", dtype, static_cast<int64_t>(B) * T, C)) return rc;
+  TCH_CHECK_ARG(ids && wte && wpe && out && vocab > 0, "embedding_fwd: null tensor");
+  const int E = dtype == kBF16 ? 8 : 4;
+  EmbedArgs a{ids, wte, wpe, out, nullptr, nullptr, nullptr, static_cast<int64_t>(B) * T, T, C, C / E, vocab, B, 0};
+  const double bytes = static_cast<double>(a.tokens) * C * (dtype == kBF16 ? 6.0 : 12.0);
+  const dim3 grid(flat_blocks(a.tokens * a.cc));
+  return dtype == kBF16 ? launch(ctx, embed_fwd_kernel<bf16>, grid, dim3(256), a, "embed_fwd_kernel<bf16>", bytes, 1)
+                        : launch(ctx, embed_fwd_kernel<float>, grid, dim3(256), a, "embed_fwd_kernel<f32>", bytes, 1);
+}
+
+int embedding_bwd(Context* ctx, int dtype, const int64_t* ids, const void* dy, float* dwte, float* dwpe, int B, int T,
+                  int C, int vocab, int accumulate_wpe) {
+  if (int rc = check_rows("embedding_bwd", dtype, static_cast<int64_t>(B) * T, C)) return rc;
+  TCH_CHECK_ARG(ids && dy && dwte && dwpe && vocab > 0, "embedding_bwd: null tensor");
+  const int E = dtype == kBF16 ? 8 : 4;
+  EmbedArgs a{ids, nullptr, nullptr, nullptr, dy, dwte, dwpe, static_cast<int64_t>(B) * T, T, C, C / E, vocab, B,
+              accumulate_wpe};
+  const double bytes = static_cast<double>(a.tokens) * C * (dtype == kBF16 ? 2.0 : 4.0) + 8.0 * a.tokens * C;
+  const dim3 grid(flat_blocks(static_cast<int64_t>(T) * a.cc));
+  return dtype == kBF16 ? launch(ctx, embed_bwd_kernel<bf16>, grid, dim3(256), a, "embed_bwd_kernel<bf16>", bytes, 1)
+                        : launch(ctx, embed_bwd_kernel<float>, grid, dim3(256), a, "embed_bwd_kernel<f32>", bytes, 1);
+}
+
+}  // namespace tch

@@ -426,3 +426,109 @@ def cast_from_f32(ctx, src, dst):
 def cast_to_f32(ctx, src, dst):
     assert dst.dtype == torch.float32 and src.numel() == dst.numel()
     check(lib().tch_cast_to_f32(ctx.handle, dtype_code(src), _p(src), _p(dst), src.numel()), "tch_cast_to_f32")
+
+
+# ---------------------------------------------------------------------------
+# transformer operators (Swin-B / GPT-2 steps)
+# ---------------------------------------------------------------------------
+
+def layernorm_fwd(ctx, x, y, gamma, beta, mean, rstd, eps=1e-5):
+    C = x.shape[-1]
+    rows = x.numel() // C
+    assert y.shape == x.shape and y.dtype == x.dtype and x.is_contiguous() and y.is_contiguous()
+    assert gamma.numel() == C and beta.numel() == C and gamma.dtype == beta.dtype == torch.float32
+    assert mean.numel() == rows and rstd.numel() == rows and mean.dtype == rstd.dtype == torch.float32
+    check(lib().tch_layernorm_fwd(ctx.handle, dtype_code(x), _p(x), _p(y), _p(gamma), _p(beta), _p(mean), _p(rstd),
+                                  rows, C, eps), "tch_layernorm_fwd")
+
+
+def layernorm_bwd_partial_rows(rows):
+    return int(lib().tch_layernorm_bwd_partial_rows(rows))
+
+
+def layernorm_bwd(ctx, dy, x, dx, gamma, mean, rstd, dgamma, dbeta, partial, accumulate=False):
+    C = x.shape[-1]
+    rows = x.numel() // C
+    assert dy.shape == x.shape == dx.shape and dy.dtype == x.dtype == dx.dtype
+    assert partial.dtype == torch.float32 and partial.numel() >= layernorm_bwd_partial_rows(rows) * C * 2
+    check(lib().tch_layernorm_bwd(ctx.handle, dtype_code(x), _p(dy), _p(x), _p(dx), _p(gamma), _p(mean), _p(rstd),
+                                  _p(dgamma), _p(dbeta), int(accumulate), rows, C, _p(partial)), "tch_layernorm_bwd")
+
+
+def gelu_fwd(ctx, x, y, tanh_form=False):
+    assert y.shape == x.shape and y.dtype == x.dtype
+    check(lib().tch_gelu_fwd(ctx.handle, dtype_code(x), _p(x), _p(y), x.numel(), int(tanh_form)), "tch_gelu_fwd")
+
+
+def gelu_bwd(ctx, dy, x, dx, tanh_form=False):
+    assert dy.shape == x.shape == dx.shape and dy.dtype == x.dtype == dx.dtype
+    check(lib().tch_gelu_bwd(ctx.handle, dtype_code(x), _p(dy), _p(x), _p(dx), x.numel(), int(tanh_form)), "tch_gelu_bwd")
+
+
+def attn_softmax_fwd(ctx, scores, probs, scale=1.0, bias=None, mask=None, causal=False):
+    """scores / probs [batch, heads, Lq, Lk]; bias [heads, Lq, Lk] fp32; mask [windows, Lq, Lk] fp32."""
+    Bn, Hn, Lq, Lk = scores.shape
+    assert probs.shape == scores.shape and probs.dtype == scores.dtype and scores.is_contiguous()
+    windows = 1
+    if bias is not None:
+        assert tuple(bias.shape) == (Hn, Lq, Lk) and bias.dtype == torch.float32
+    if mask is not None:
+        assert tuple(mask.shape[1:]) == (Lq, Lk) and mask.dtype == torch.float32
+        windows = mask.shape[0]
+    check(lib().tch_attn_softmax_fwd(ctx.handle, dtype_code(scores), _p(scores), _p(probs), Bn, Hn, Lq, Lk, scale,
+                                     _p(bias), _p(mask), windows, int(causal)), "tch_attn_softmax_fwd")
+
+
+def attn_softmax_bwd(ctx, probs, dprobs, dscores, scale=1.0):
+    Lk = probs.shape[-1]
+    assert probs.shape == dprobs.shape == dscores.shape and probs.dtype == dprobs.dtype == dscores.dtype
+    check(lib().tch_attn_softmax_bwd(ctx.handle, dtype_code(probs), _p(probs), _p(dprobs), _p(dscores),
+                                     probs.numel() // Lk, Lk, scale), "tch_attn_softmax_bwd")
+
+
+def adamw_step(ctx, param, grad, exp_avg, exp_avg_sq, step_dev, scalars_dev, lr, beta1=0.9, beta2=0.999, eps=1e-8,
+               weight_decay=0.01, shadow=None):
+    n = param.numel()
+    for t in (grad, exp_avg, exp_avg_sq):
+        assert t.dtype == torch.float32 and t.numel() == n
+    assert param.dtype == torch.float32 and step_dev.dtype == torch.int32 and scalars_dev.dtype == torch.float32
+    assert step_dev.numel() >= 1 and scalars_dev.numel() >= 2
+    assert shadow is None or (shadow.dtype == torch.bfloat16 and shadow.numel() == n)
+    check(lib().tch_adamw_step(ctx.handle, _p(param), _p(grad), _p(exp_avg), _p(exp_avg_sq), _p(shadow), n, lr, beta1,
+                               beta2, eps, weight_decay, _p(step_dev), _p(scalars_dev)), "tch_adamw_step")
+
+
+def embedding_fwd(ctx, ids, wte, wpe, out):
+    B, T = ids.shape
+    vocab, C = wte.shape
+    assert ids.dtype == torch.int64 and wpe.shape[0] >= T and wpe.shape[1] == C
+    assert tuple(out.shape) == (B, T, C) and out.dtype == wte.dtype == wpe.dtype
+    check(lib().tch_embedding_fwd(ctx.handle, dtype_code(wte), _p(ids), _p(wte), _p(wpe), _p(out), B, T, C, vocab),
+          "tch_embedding_fwd")
+
+
+def embedding_bwd(ctx, ids, dy, dwte, dwpe, accumulate_wpe=False):
+    B, T = ids.shape
+    vocab, C = dwte.shape
+    assert tuple(dy.shape) == (B, T, C) and dwte.dtype == dwpe.dtype == torch.float32 and dwpe.shape[0] >= T
+    check(lib().tch_embedding_bwd(ctx.handle, dtype_code(dy), _p(ids), _p(dy), _p(dwte), _p(dwpe), B, T, C, vocab,
+                                  int(accumulate_wpe)), "tch_embedding_bwd")
+
+
+def batched_gemm(ctx, a, b, c, M, N, K, a_strides, b_strides, ldc, batch=(1, 1), a_batch=(0, 0), b_batch=(0, 0),
+                 c_batch=(0, 0), alpha=1.0, accumulate=False):
+    """C[z](m, n) (+)= alpha * sum_k A[z](m, k) * B[z](n, k); strides are (row, k) in elements, batch offsets are
+    (outer, inner) in elements, z = outer * batch[1] + inner.  The caller vouches that every address the
+    strides reach lies inside the tensors; what can be checked from the tensor sizes is checked here."""
+    assert a.dtype == b.dtype == c.dtype
+    bo, bi = batch
+
+    def extent(strides, rows, batch_off):
+        return (bo - 1) * batch_off[0] + (bi - 1) * batch_off[1] + (rows - 1) * strides[0] + (K - 1) * strides[1] + 1
+    assert extent(a_strides, M, a_batch) <= a.numel(), "batched_gemm: A reaches past its tensor"
+    assert extent(b_strides, N, b_batch) <= b.numel(), "batched_gemm: B reaches past its tensor"
+    assert (bo - 1) * c_batch[0] + (bi - 1) * c_batch[1] + (M - 1) * ldc + N <= c.numel(), \
+        "batched_gemm: C reaches past its tensor"
+    check(lib().tch_batched_gemm(ctx.handle, dtype_code(a), _p(a), _p(b), _p(c), M, N, K, a_strides[0], a_strides[1],
+                                 b_strides[0], b_strides[1], ldc, bo, bi, a_batch[0], a_batch[1], b_batch[0], b_batch[1],
+                                 c_batch[0], c_batch[1], alpha, int(accumulate)), "tch_batched_gemm")

@@ -1,0 +1,261 @@
+"""Transformer operators on the GPU (LayerNorm, GELU, attention softmax, AdamW, embedding, batched GEMM),
+called through the C ABI, against the CPU oracle (oracle/seq_ops.py) on the same seeded inputs.
+
+Tolerances: fp32 rtol 1e-3, bf16 rtol 2e-2 against the largest magnitude of the oracle tensor (the
+path's stated bound); tighter where an operator is purely elementwise.
+"""
+import pytest
+import torch
+
+from oracle import seq_ops as S
+
+pytestmark = pytest.mark.gpu
+
+RTOL = {torch.float32: 1e-3, torch.bfloat16: 2e-2}
+
+
+def _gen(seed):
+    g = torch.Generator()
+    g.manual_seed(seed)
+    return g
+
+
+def rnd(shape, dtype, g, scale=1.0):
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def close(got, ref, dtype, what, rtol=None):
+    rtol = RTOL[dtype] if rtol is None else rtol
+    got, ref = got.detach().float().cpu(), ref.detach().float()
+    assert got.shape == ref.shape, f"{what}: shape {tuple(got.shape)} vs {tuple(ref.shape)}"
+    assert torch.isfinite(got).all(), f"{what}: non-finite values"
+    scale = ref.abs().max().item() + 1e-12
+    err = (got - ref).abs().max().item()
+    assert err <= rtol * scale, f"{what}: max err {err:.3e} > {rtol:g} * {scale:.3e}"
+
+
+LN_CASES = [(8 * 49, 128), (3 * 197, 768), (1000, 1024), (5, 8), (4100, 256)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,C", LN_CASES)
+def test_layernorm(ctx, dtype, rows, C):
+    from sirius_amd import ops
+    print("case", rows, C, dtype, flush=True)
+    g = _gen(31)
+    x = (rnd((rows, C), dtype, g) * 1.5 + 0.3).to(dtype)
+    gamma, beta = torch.rand(C, generator=g) + 0.5, torch.randn(C, generator=g) * 0.2
+    y_ref, mean_ref, rstd_ref = S.layernorm(x, gamma, beta)
+    xd = x.cuda()
+    y = torch.empty_like(xd)
+    mean, rstd = torch.empty(rows, device="cuda"), torch.empty(rows, device="cuda")
+    ops.layernorm_fwd(ctx, xd, y, gamma.cuda(), beta.cuda(), mean, rstd)
+    dy = rnd((rows, C), dtype, g)
+    dx_ref, dg_ref, db_ref = S.layernorm_bwd(dy, x, gamma)
+    dx = torch.empty_like(xd)
+    dg, db = torch.full((C,), 3.0, device="cuda"), torch.full((C,), -2.0, device="cuda")
+    partial = torch.empty(ops.layernorm_bwd_partial_rows(rows) * C * 2, device="cuda")
+    ops.layernorm_bwd(ctx, dy.cuda(), xd, dx, gamma.cuda(), mean, rstd, dg, db, partial)
+    # accumulate on top
+    dg2, db2 = dg.clone(), db.clone()
+    torch.cuda.synchronize()
+    ops.layernorm_bwd(ctx, dy.cuda(), xd, dx, gamma.cuda(), mean, rstd, dg2, db2, partial, accumulate=True)
+    torch.cuda.synchronize()
+    close(mean, mean_ref, torch.float32, "ln mean", rtol=1e-4)
+    close(rstd, rstd_ref, torch.float32, "ln rstd", rtol=1e-4)
+    close(y, y_ref, dtype, "ln y", rtol=1e-4 if dtype == torch.float32 else 1e-2)
+    close(dx, dx_ref, dtype, "ln dx", rtol=1e-3 if dtype == torch.float32 else 1e-2)
+    close(dg, dg_ref, torch.float32, "ln dgamma", rtol=1e-3)
+    close(db, db_ref, torch.float32, "ln dbeta", rtol=1e-3)
+    close(dg2, 2 * dg_ref, torch.float32, "ln dgamma accumulated", rtol=1e-3)
+    close(db2, 2 * db_ref, torch.float32, "ln dbeta accumulated", rtol=1e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("tanh_form", [False, True])
+@pytest.mark.parametrize("n", [8, 4096 * 3 + 8, 1 << 20])
+def test_gelu(ctx, dtype, tanh_form, n):
+    from sirius_amd import ops
+    g = _gen(32)
+    x = rnd((n,), dtype, g, 2.0)
+    x[:8] = torch.tensor([0.0, -0.0, 1e-4, -1e-4, 6.0, -6.0, 12.0, -12.0]).to(dtype)
+    dy = rnd((n,), dtype, g)
+    y, dx = torch.empty(n, dtype=dtype, device="cuda"), torch.empty(n, dtype=dtype, device="cuda")
+    ops.gelu_fwd(ctx, x.cuda(), y, tanh_form)
+    ops.gelu_bwd(ctx, dy.cuda(), x.cuda(), dx, tanh_form)
+    torch.cuda.synchronize()
+    tol = 1e-5 if dtype == torch.float32 else 8e-3   # bf16: one rounding of the output
+    close(y, S.gelu(x, tanh_form), dtype, "gelu", rtol=tol)
+    close(dx, S.gelu_bwd(dy, x, tanh_form), dtype, "gelu bwd", rtol=tol)
+
+
+SOFTMAX_CASES = [
+    # batch, heads, L, windows (0: no mask), bias, causal
+    (8, 4, 49, 4, True, False),     # Swin window attention with the shift mask
+    (6, 3, 49, 0, True, False),     # unshifted block
+    (2, 12, 128, 0, False, True),   # GPT-2, short
+    (1, 2, 1024, 0, False, True),   # GPT-2 sequence length
+    (3, 1, 7, 0, False, False),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", SOFTMAX_CASES)
+def test_attn_softmax(ctx, dtype, case):
+    from sirius_amd import ops
+    Bn, Hn, L, nW, with_bias, causal = case
+    print("case", case, dtype, flush=True)
+    g = _gen(33)
+    s = rnd((Bn, Hn, L, L), dtype, g, 3.0)
+    bias = torch.randn(Hn, L, L, generator=g) if with_bias else None
+    mask = torch.where(torch.rand(nW, L, L, generator=g) > 0.6, -100.0, 0.0) if nW else None
+    scale = 0.17
+    p_ref = S.attn_softmax(s, scale, bias, mask, causal)
+    d = lambda t: t.cuda() if t is not None else None
+    p = torch.empty((Bn, Hn, L, L), dtype=dtype, device="cuda")
+    ops.attn_softmax_fwd(ctx, s.cuda(), p, scale, d(bias), d(mask), causal)
+    torch.cuda.synchronize()
+    close(p, p_ref, dtype, "softmax", rtol=1e-5 if dtype == torch.float32 else 8e-3)
+    if causal:
+        assert torch.all(p.float().cpu().triu(1) == 0), "keys after the query must get probability zero"
+    # in place
+    s2 = s.cuda()
+    ops.attn_softmax_fwd(ctx, s2, s2, scale, d(bias), d(mask), causal)
+    torch.cuda.synchronize()
+    assert torch.equal(s2, p), "in-place softmax must match the out-of-place one bit for bit"
+    # backward from the kernel's own (rounded) probabilities
+    dp = rnd((Bn, Hn, L, L), dtype, g)
+    pf = p.float().cpu()
+    ds_ref = scale * pf * (dp.float() - (dp.float() * pf).sum(-1, keepdim=True))
+    ds = torch.empty_like(p)
+    ops.attn_softmax_bwd(ctx, p, dp.cuda(), ds, scale)
+    torch.cuda.synchronize()
+    close(ds, ds_ref, dtype, "softmax bwd", rtol=1e-4 if dtype == torch.float32 else 1e-2)
+    if dtype == torch.float32:
+        close(ds, S.attn_softmax_bwd(s, dp, scale, bias, mask, causal), dtype, "softmax bwd vs autograd", rtol=1e-4)
+
+
+@pytest.mark.parametrize("n", [5, 1000, (1 << 20) + 3])
+@pytest.mark.parametrize("with_shadow", [False, True])
+def test_adamw(ctx, n, with_shadow):
+    from sirius_amd import ops
+    g = _gen(34)
+    p0 = torch.randn(n, generator=g)
+    grads = [torch.randn(n, generator=g) * (0.1 + i) for i in range(3)]
+    hp = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.05)
+    p_ref, m_ref, v_ref = S.adamw(p0, grads, hp["lr"], hp["beta1"], hp["beta2"], hp["eps"], hp["weight_decay"])
+    p, m, v = p0.cuda(), torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+    step, scal = torch.zeros(1, dtype=torch.int32, device="cuda"), torch.zeros(2, device="cuda")
+    shadow = torch.empty(n, dtype=torch.bfloat16, device="cuda") if with_shadow else None
+    for gi in grads:
+        ops.adamw_step(ctx, p, gi.cuda(), m, v, step, scal, shadow=shadow, **hp)
+        torch.cuda.synchronize()
+    assert step.item() == 3
+    close(p, p_ref, torch.float32, "adamw param", rtol=1e-5)
+    close(m, m_ref, torch.float32, "adamw exp_avg", rtol=1e-5)
+    close(v, v_ref, torch.float32, "adamw exp_avg_sq", rtol=1e-5)
+    if with_shadow:
+        assert torch.equal(shadow, p.to(torch.bfloat16)), "the bf16 shadow is the rounded parameter, bit for bit"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,T,C,vocab", [(2, 16, 64, 101), (3, 37, 768, 5000), (1, 1, 8, 3)])
+def test_embedding(ctx, dtype, B, T, C, vocab):
+    from sirius_amd import ops
+    g = _gen(35)
+    wte, wpe = rnd((vocab, C), dtype, g), rnd((T + 3, C), dtype, g)
+    ids = torch.randint(0, vocab, (B, T), generator=g)
+    if B * T > 4:
+        ids.view(-1)[:4] = ids.view(-1)[0]   # a token that repeats
+    out = torch.empty((B, T, C), dtype=dtype, device="cuda")
+    ops.embedding_fwd(ctx, ids.cuda(), wte.cuda(), wpe.cuda(), out)
+    torch.cuda.synchronize()
+    close(out, S.embedding(ids, wte, wpe), dtype, "embedding", rtol=1e-6 if dtype == torch.float32 else 8e-3)
+    dy = rnd((B, T, C), dtype, g)
+    dwte_ref, dwpe_ref = S.embedding_bwd(ids, dy, vocab, T + 3)
+    dwte = torch.zeros((vocab, C), device="cuda")
+    dwpe = torch.full((T + 3, C), 9.0, device="cuda")
+    ops.embedding_bwd(ctx, ids.cuda(), dy.cuda(), dwte, dwpe)
+    torch.cuda.synchronize()
+    close(dwte, dwte_ref, torch.float32, "dwte", rtol=1e-5)
+    close(dwpe[:T], dwpe_ref[:T], torch.float32, "dwpe", rtol=1e-5)
+    assert torch.all(dwpe[T:] == 9.0), "positions past the sequence are not touched"
+
+
+def _attention_layouts(B, H, T, D):
+    """Offsets of head h of sample b inside a packed [B, T, 3, H, D] projection (GPT-2's c_attn output)."""
+    C = H * D
+    return dict(row=3 * C, batch=(T * 3 * C, D), q0=0, k0=C, v0=2 * C)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,H,T,D", [(2, 3, 49, 32), (1, 2, 200, 64), (2, 2, 64, 64), (1, 1, 5, 8)])
+def test_batched_gemm_attention_products(ctx, dtype, B, H, T, D):
+    """Every product of an attention layer and of its backward, on strided views of one packed qkv tensor,
+    against einsum on the CPU: Q K^T, P V, P^T dO, dO V^T, dS K, dS^T Q."""
+    from sirius_amd import ops
+    print("case", B, H, T, D, dtype, flush=True)
+    g = _gen(36)
+    C = H * D
+    qkv = rnd((B, T, 3, H, D), dtype, g)
+    q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3).float() for i in range(3))     # [B, H, T, D]
+    lay = _attention_layouts(B, H, T, D)
+    qkv_d = qkv.cuda()
+    flat = qkv_d.view(-1)
+    qv, kv, vv = flat[lay["q0"]:], flat[lay["k0"]:], flat[lay["v0"]:]
+    sb = (H * T * T, T * T)   # scores [B, H, T, T]
+    ob = (T * C, D)           # output [B, T, H, D]
+    tol = 1e-3 if dtype == torch.float32 else 2e-2
+
+    s = torch.full((B, H, T, T), 7.0, dtype=dtype, device="cuda")
+    ops.batched_gemm(ctx, qv, kv, s, T, T, D, (lay["row"], 1), (lay["row"], 1), T, (B, H), lay["batch"], lay["batch"], sb,
+                     alpha=0.25)
+    torch.cuda.synchronize()
+    close(s, 0.25 * torch.einsum("bhtd,bhsd->bhts", q, k), dtype, "Q K^T", rtol=tol)
+
+    p = rnd((B, H, T, T), dtype, g, 0.2)
+    p_d = p.cuda()
+    o = torch.empty((B, T, H, D), dtype=dtype, device="cuda")
+    ops.batched_gemm(ctx, p_d, vv, o, T, D, T, (T, 1), (1, lay["row"]), C, (B, H), sb, lay["batch"], ob)
+    torch.cuda.synchronize()
+    o_ref = torch.einsum("bhts,bhsd->bthd", p.float(), v)
+    close(o, o_ref, dtype, "P V", rtol=tol)
+
+    do = rnd((B, T, H, D), dtype, g)
+    do_d = do.cuda()
+    dof = do.float().permute(0, 2, 1, 3)                                        # [B, H, T, D]
+    dqkv = torch.zeros((B, T, 3, H, D), dtype=dtype, device="cuda")
+    dflat = dqkv.view(-1)
+    # dV[s, d] = sum_t P[t, s] dO[t, d]
+    ops.batched_gemm(ctx, p_d, do_d, dflat[lay["v0"]:], T, D, T, (1, T), (1, C), lay["row"], (B, H), sb, ob, lay["batch"])
+    # dP[t, s] = sum_d dO[t, d] V[s, d]
+    dp = torch.empty((B, H, T, T), dtype=dtype, device="cuda")
+    ops.batched_gemm(ctx, do_d, vv, dp, T, T, D, (C, 1), (lay["row"], 1), T, (B, H), ob, lay["batch"], sb)
+    ds = rnd((B, H, T, T), dtype, g, 0.3)
+    ds_d = ds.cuda()
+    # dQ[t, d] = sum_s dS[t, s] K[s, d];  dK[s, d] = sum_t dS[t, s] Q[t, d]
+    ops.batched_gemm(ctx, ds_d, kv, dflat[lay["q0"]:], T, D, T, (T, 1), (1, lay["row"]), lay["row"], (B, H), sb,
+                     lay["batch"], lay["batch"])
+    ops.batched_gemm(ctx, ds_d, qv, dflat[lay["k0"]:], T, D, T, (1, T), (1, lay["row"]), lay["row"], (B, H), sb,
+                     lay["batch"], lay["batch"])
+    torch.cuda.synchronize()
+    close(dp, torch.einsum("bhtd,bhsd->bhts", dof, v), dtype, "dO V^T", rtol=tol)
+    got = dqkv.float().cpu()
+    close(got[:, :, 2], torch.einsum("bhts,bhtd->bshd", p.float(), dof), dtype, "P^T dO", rtol=tol)
+    close(got[:, :, 0], torch.einsum("bhts,bhsd->bthd", ds.float(), k), dtype, "dS K", rtol=tol)
+    close(got[:, :, 1], torch.einsum("bhts,bhtd->bshd", ds.float(), q), dtype, "dS^T Q", rtol=tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_batched_gemm_accumulate_and_edges(ctx, dtype):
+    """Sizes off every tile edge, an unaligned base, accumulate on top of existing values."""
+    from sirius_amd import ops
+    g = _gen(37)
+    M, N, K = 70, 33, 45
+    a, b = rnd((M * K + 1,), dtype, g), rnd((N, K), dtype, g)
+    a_d = a.cuda()
+    c = torch.ones((M, N), dtype=dtype, device="cuda")
+    ops.batched_gemm(ctx, a_d[1:], b.cuda(), c, M, N, K, (K, 1), (K, 1), N, accumulate=True, alpha=0.5)
+    torch.cuda.synchronize()
+    ref = 1.0 + 0.5 * a[1:].float().view(M, K) @ b.float().t()
+    close(c, ref, dtype, "accumulate", rtol=1e-3 if dtype == torch.float32 else 2e-2)
