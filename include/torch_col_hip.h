@@ -175,6 +175,13 @@ int tch_avgpool_bwd(tch_context* ctx, int dtype, const void* dy, void* dx, int N
  * dimension ld_dlogits) = (softmax - onehot) * grad_scale, grad_scale = loss_scale / rows. */
 int tch_softmax_ce_fwd_bwd(tch_context* ctx, int dtype, const float* logits, const int64_t* labels, float* loss_rows,
                            float* loss_mean, void* dlogits, int rows, int classes, int ld_dlogits, float grad_scale);
+/* The language-model form (GPT-2's output.loss, train/gpt2.py:93): rows as long as the vocabulary, logits with
+ * their own leading dimension, a row whose label is negative is ignored (zero loss, zero gradient);
+ * loss_mean = sum / valid_rows, dlogits = (softmax - onehot) * loss_scale / valid_rows.  Columns of dlogits
+ * from `classes` up to ld_dlogits are not written. */
+int tch_softmax_ce_lm(tch_context* ctx, int dtype, const float* logits, int ld_logits, const int64_t* labels,
+                      float* loss_rows, float* loss_mean, void* dlogits, int ld_dlogits, int rows, int classes,
+                      int valid_rows, float loss_scale);
 /* g += wd*p; buf = momentum*buf + g; p -= lr*buf; shadow_bf16 (may be NULL) = bf16(p) */
 int tch_sgd_momentum_step(tch_context* ctx, float* param, const float* grad, float* momentum_buf, void* shadow_bf16,
                           int64_t n, float lr, float momentum, float weight_decay);
@@ -192,9 +199,11 @@ int tch_bias_grad(tch_context* ctx, int dtype, const void* dy, float* dbias, int
  * are kept for the backward. */
 int tch_layernorm_fwd(tch_context* ctx, int dtype, const void* x, void* y, const float* gamma, const float* beta,
                       float* mean, float* rstd, int64_t rows, int C, float eps);
-/* partial: fp32 scratch of tch_layernorm_bwd_partial_rows(rows) * C * 2 floats; dgamma / dbeta (+)= */
+/* dx = LayerNorm'(dy) (+ residual, laid out like dx, may be NULL: the gradient that bypasses the LayerNorm);
+ * partial: fp32 scratch of tch_layernorm_bwd_partial_rows(rows) * C * 2 floats; dgamma / dbeta (+)= */
 int tch_layernorm_bwd_partial_rows(int64_t rows);
-int tch_layernorm_bwd(tch_context* ctx, int dtype, const void* dy, const void* x, void* dx, const float* gamma,
+int tch_layernorm_bwd(tch_context* ctx, int dtype, const void* dy, const void* x, void* dx, const void* residual,
+                      const float* gamma,
                       const float* mean, const float* rstd, float* dgamma, float* dbeta, int accumulate, int64_t rows,
                       int C, float* partial);
 /* tanh_form 0: 0.5 x (1 + erf(x / sqrt 2)) (nn.GELU); 1: GPT-2's gelu_new.  n is a multiple of a 16-byte chunk. */

@@ -215,10 +215,12 @@ int tch_layernorm_fwd(tch_context* ctx, int dtype, const void* x, void* y, const
 
 int tch_layernorm_bwd_partial_rows(int64_t rows) { return layernorm_bwd_partial_rows(rows); }
 
-int tch_layernorm_bwd(tch_context* ctx, int dtype, const void* dy, const void* x, void* dx, const float* gamma,
+int tch_layernorm_bwd(tch_context* ctx, int dtype, const void* dy, const void* x, void* dx, const void* residual,
+                      const float* gamma,
                       const float* mean, const float* rstd, float* dgamma, float* dbeta, int accumulate, int64_t rows,
                       int Cc, float* partial) {
-  return layernorm_bwd(C(ctx), dtype, dy, x, dx, gamma, mean, rstd, dgamma, dbeta, accumulate, rows, Cc, partial);
+  return layernorm_bwd(C(ctx), dtype, dy, x, dx, residual, gamma, mean, rstd, dgamma, dbeta, accumulate, rows, Cc,
+                       partial);
 }
 
 int tch_gelu_fwd(tch_context* ctx, int dtype, const void* x, void* y, int64_t n, int tanh_form) {
@@ -319,6 +321,13 @@ int tch_softmax_ce_fwd_bwd(tch_context* ctx, int dtype, const float* logits, con
                            float* loss_mean, void* dlogits, int rows, int classes, int ld_dlogits, float grad_scale) {
   return softmax_ce_fwd_bwd(C(ctx), dtype, logits, labels, loss_rows, loss_mean, dlogits, rows, classes, ld_dlogits,
                             grad_scale);
+}
+
+int tch_softmax_ce_lm(tch_context* ctx, int dtype, const float* logits, int ld_logits, const int64_t* labels,
+                      float* loss_rows, float* loss_mean, void* dlogits, int ld_dlogits, int rows, int classes,
+                      int valid_rows, float loss_scale) {
+  return softmax_ce_lm(C(ctx), dtype, logits, ld_logits, labels, loss_rows, loss_mean, dlogits, ld_dlogits, rows, classes,
+                       valid_rows, loss_scale);
 }
 
 int tch_sgd_momentum_step(tch_context* ctx, float* param, const float* grad, float* momentum_buf, void* shadow_bf16,

@@ -47,17 +47,68 @@ __global__ __launch_bounds__(64) void softmax_ce_kernel(CeArgs p) {
   }
 }
 
+// Language-model form: one workgroup per row (vocabulary-sized rows), logits with their own leading
+// dimension, rows whose label is negative are ignored (zero loss, zero gradient).
+struct CeWideArgs {
+  const float* logits;
+  const int64_t* labels;
+  float* loss_rows;
+  void* dlogits;
+  int rows, classes, ld_logits, ld_dlogits;
+  float grad_scale;
+};
+
+__device__ inline float block_reduce(float v, bool take_max, float* scratch) {
+  v = take_max ? wave_max(v) : wave_sum(v);
+  const int wave = threadIdx.x >> 6;
+  __syncthreads();  // scratch may still be read from the previous reduction
+  if ((threadIdx.x & 63) == 0) scratch[wave] = v;
+  __syncthreads();
+  float r = scratch[0];
+#pragma unroll
+  for (int w = 1; w < 4; ++w) r = take_max ? fmaxf(r, scratch[w]) : r + scratch[w];
+  return r;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_ce_wide_kernel(CeWideArgs p) {
+  __shared__ float scratch[4];
+  const int row = blockIdx.x;
+  const int tid = threadIdx.x;
+  const float* z = p.logits + static_cast<int64_t>(row) * p.ld_logits;
+  T* g = static_cast<T*>(p.dlogits) + static_cast<int64_t>(row) * p.ld_dlogits;
+  const int64_t label = p.labels[row];
+  if (label < 0 || label >= p.classes) {
+    if (tid == 0) p.loss_rows[row] = 0.f;
+    for (int c = tid; c < p.classes; c += 256) Elem<T>::store(g + c, 0.f);
+    return;
+  }
+  float mx = -INFINITY;
+  for (int c = tid; c < p.classes; c += 256) mx = fmaxf(mx, z[c]);
+  mx = block_reduce(mx, true, scratch);
+  float sum = 0.f;
+  for (int c = tid; c < p.classes; c += 256) sum += expf(z[c] - mx);
+  sum = block_reduce(sum, false, scratch);
+  if (tid == 0) p.loss_rows[row] = mx + logf(sum) - z[label];
+  const float inv = 1.f / sum;
+  for (int c = tid; c < p.classes; c += 256) {
+    const float sm = expf(z[c] - mx) * inv;
+    Elem<T>::store(g + c, (sm - (c == label ? 1.f : 0.f)) * p.grad_scale);
+  }
+}
+
 struct MeanArgs {
   const float* in;
   float* out;
   int n;
+  float divisor;
 };
 
 __global__ __launch_bounds__(64) void mean_kernel(MeanArgs p) {
   float s = 0.f;
   for (int i = threadIdx.x; i < p.n; i += 64) s += p.in[i];
   s = wave_sum(s);
-  if (threadIdx.x == 0) *p.out = s / static_cast<float>(p.n);
+  if (threadIdx.x == 0) *p.out = s / p.divisor;
 }
 
 struct SgdArgs {
@@ -179,7 +230,26 @@ int softmax_ce_fwd_bwd(Context* ctx, int dtype, const float* logits, const int64
   int rc = dtype == kBF16 ? launch(ctx, softmax_ce_kernel<bf16>, dim3(rows), dim3(64), a, "softmax_ce_kernel<bf16>", bytes, 1)
                           : launch(ctx, softmax_ce_kernel<float>, dim3(rows), dim3(64), a, "softmax_ce_kernel<f32>", bytes, 1);
   if (rc) return rc;
-  MeanArgs m{loss_rows, loss_mean, rows};
+  MeanArgs m{loss_rows, loss_mean, rows, static_cast<float>(rows)};
+  return launch(ctx, mean_kernel, dim3(1), dim3(64), m, "mean_kernel", 4.0 * rows, 1);
+}
+
+int softmax_ce_lm(Context* ctx, int dtype, const float* logits, int ld_logits, const int64_t* labels, float* loss_rows,
+                  float* loss_mean, void* dlogits, int ld_dlogits, int rows, int classes, int valid_rows,
+                  float loss_scale) {
+  TCH_CHECK_ARG(dtype == kBF16 || dtype == kF32, "softmax_ce_lm: dtype must be f32(0) or bf16(1)");
+  TCH_CHECK_ARG(logits && labels && loss_rows && loss_mean && dlogits, "softmax_ce_lm: null tensor");
+  TCH_CHECK_ARG(rows > 0 && classes > 0 && ld_logits >= classes && ld_dlogits >= classes && valid_rows > 0 &&
+                    valid_rows <= rows,
+                "softmax_ce_lm: bad shape");
+  CeWideArgs a{logits, labels, loss_rows, dlogits, rows, classes, ld_logits, ld_dlogits,
+               loss_scale / static_cast<float>(valid_rows)};
+  const double bytes = static_cast<double>(rows) * classes * (4.0 + (dtype == kBF16 ? 2.0 : 4.0));
+  int rc = dtype == kBF16
+               ? launch(ctx, softmax_ce_wide_kernel<bf16>, dim3(rows), dim3(256), a, "softmax_ce_wide_kernel<bf16>", bytes, 1)
+               : launch(ctx, softmax_ce_wide_kernel<float>, dim3(rows), dim3(256), a, "softmax_ce_wide_kernel<f32>", bytes, 1);
+  if (rc) return rc;
+  MeanArgs m{loss_rows, loss_mean, rows, static_cast<float>(valid_rows)};
   return launch(ctx, mean_kernel, dim3(1), dim3(64), m, "mean_kernel", 4.0 * rows, 1);
 }
 

@@ -67,7 +67,7 @@ int bn_bwd_partials(Context* ctx, int dtype, const void* g, const void* x, void*
 int layernorm_fwd(Context* ctx, int dtype, const void* x, void* y, const float* gamma, const float* beta, float* mean,
                   float* rstd, int64_t rows, int C, float eps);
 int layernorm_bwd_partial_rows(int64_t rows);  // rows of [C][2] fp32 scratch layernorm_bwd needs
-int layernorm_bwd(Context* ctx, int dtype, const void* dy, const void* x, void* dx, const float* gamma,
+int layernorm_bwd(Context* ctx, int dtype, const void* dy, const void* x, void* dx, const void* residual, const float* gamma,
                   const float* mean, const float* rstd, float* dgamma, float* dbeta, int accumulate, int64_t rows,
                   int C, float* partial);
 int gelu_fwd(Context* ctx, int dtype, const void* x, void* y, int64_t n, int tanh_form);
@@ -100,6 +100,10 @@ int avgpool_bwd(Context* ctx, int dtype, const void* dy, void* dx, int N, int HW
 // loss_optim.hip
 int softmax_ce_fwd_bwd(Context* ctx, int dtype, const float* logits, const int64_t* labels, float* loss_rows,
                        float* loss_mean, void* dlogits, int rows, int classes, int ld_dlogits, float grad_scale);
+// vocabulary-sized rows; rows with a negative label are ignored; mean over valid_rows
+int softmax_ce_lm(Context* ctx, int dtype, const float* logits, int ld_logits, const int64_t* labels, float* loss_rows,
+                  float* loss_mean, void* dlogits, int ld_dlogits, int rows, int classes, int valid_rows,
+                  float loss_scale);
 int sgd_momentum_step(Context* ctx, float* param, const float* grad, float* momentum_buf, void* shadow_bf16,
                       int64_t n, float lr, float momentum, float weight_decay);
 int grad_accumulate(Context* ctx, float* global, float* grad, int64_t n);

@@ -34,6 +34,7 @@ struct LnChunks {
 struct LnArgs {
   const void* x;
   const void* dy;  // backward
+  const void* add; // backward, optional: added to dx (the residual branch's gradient)
   void* out;       // forward: y   backward: dx
   const float* gamma;
   const float* beta;
@@ -155,6 +156,14 @@ __global__ __launch_bounds__(256) void ln_bwd_kernel(LnArgs p) {
         float o[E];
 #pragma unroll
         for (int e = 0; e < E; ++e) o[e] = rstd * (g[j][e] - a - xh[j][e] * b);
+        if (p.add) {
+          Chunk cr;
+          cr.u = (static_cast<const uint4*>(p.add) + row * p.cc)[c];
+          float r[E];
+          chunk_to_float<T>(cr, r);
+#pragma unroll
+          for (int e = 0; e < E; ++e) o[e] += r[e];
+        }
         dst[c] = float_to_chunk<T>(o).u;
       }
     }
@@ -480,14 +489,14 @@ int layernorm_fwd(Context* ctx, int dtype, const void* x, void* y, const float* 
   const int E = dtype == kBF16 ? 8 : 4;
   TCH_CHECK_ARG(C <= kLnMaxC, "layernorm: rows longer than 1024 elements are not supported");
   TCH_CHECK_ARG(x && y && gamma && beta && mean && rstd, "layernorm_fwd: null tensor");
-  LnArgs a{x, nullptr, y, gamma, beta, mean, rstd, nullptr, rows, C, C / E, 0, eps};
+  LnArgs a{x, nullptr, nullptr, y, gamma, beta, mean, rstd, nullptr, rows, C, C / E, 0, eps};
   const double bytes = static_cast<double>(rows) * C * (dtype == kBF16 ? 4.0 : 8.0);
   const dim3 grid(static_cast<unsigned>((rows + 3) / 4));
   return dtype == kBF16 ? launch(ctx, ln_fwd_kernel<bf16>, grid, dim3(256), a, "ln_fwd_kernel<bf16>", bytes, 1)
                         : launch(ctx, ln_fwd_kernel<float>, grid, dim3(256), a, "ln_fwd_kernel<f32>", bytes, 1);
 }
 
-int layernorm_bwd(Context* ctx, int dtype, const void* dy, const void* x, void* dx, const float* gamma,
+int layernorm_bwd(Context* ctx, int dtype, const void* dy, const void* x, void* dx, const void* residual, const float* gamma,
                   const float* mean, const float* rstd, float* dgamma, float* dbeta, int accumulate, int64_t rows,
                   int C, float* partial) {
   if (int rc = check_rows("layernorm_bwd", dtype, rows, C)) return rc;
@@ -496,7 +505,8 @@ int layernorm_bwd(Context* ctx, int dtype, const void* dy, const void* x, void* 
   TCH_CHECK_ARG(dy && x && dx && gamma && mean && rstd && dgamma && dbeta && partial, "layernorm_bwd: null tensor");
   const int rpw = ln_rows_per_wg(rows);
   const int blocks = static_cast<int>((rows + rpw - 1) / rpw);
-  LnArgs a{x, dy, dx, gamma, nullptr, const_cast<float*>(mean), const_cast<float*>(rstd), partial, rows, C, C / E, rpw, 0.f};
+  LnArgs a{x,    dy,   residual, dx, gamma, nullptr, const_cast<float*>(mean), const_cast<float*>(rstd), partial,
+           rows, C,    C / E,    rpw, 0.f};
   const double bytes = static_cast<double>(rows) * C * (dtype == kBF16 ? 6.0 : 12.0);
   int rc = dtype == kBF16 ? launch(ctx, ln_bwd_kernel<bf16>, dim3(blocks), dim3(256), a, "ln_bwd_kernel<bf16>", bytes, 1)
                           : launch(ctx, ln_bwd_kernel<float>, dim3(blocks), dim3(256), a, "ln_bwd_kernel<f32>", bytes, 1);

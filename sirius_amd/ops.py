@@ -356,6 +356,17 @@ def softmax_ce_fwd_bwd(ctx, logits, labels, loss_rows, loss_mean, dlogits, loss_
                                        float(loss_scale) / rows), "tch_softmax_ce_fwd_bwd")
 
 
+def softmax_ce_lm(ctx, logits, labels, loss_rows, loss_mean, dlogits, classes, valid_rows, loss_scale=1.0):
+    """logits [rows, ld] fp32 and dlogits [rows, ld'] with ld, ld' >= classes; labels < 0 are ignored."""
+    rows = logits.shape[0]
+    assert logits.dtype == torch.float32 and labels.dtype == torch.int64 and labels.numel() == rows
+    assert logits.stride(0) == logits.shape[1] >= classes and dlogits.stride(0) == dlogits.shape[1] >= classes
+    assert dlogits.shape[0] == rows and loss_rows.numel() >= rows
+    check(lib().tch_softmax_ce_lm(ctx.handle, dtype_code(dlogits), _p(logits), logits.shape[1], _p(labels), _p(loss_rows),
+                                  _p(loss_mean), _p(dlogits), dlogits.shape[1], rows, classes, int(valid_rows),
+                                  float(loss_scale)), "tch_softmax_ce_lm")
+
+
 def sgd_momentum_step(ctx, param, grad, buf, lr, momentum, weight_decay, shadow=None):
     n = param.numel()
     assert param.dtype == grad.dtype == buf.dtype == torch.float32 and grad.numel() == n and buf.numel() == n
@@ -446,12 +457,13 @@ def layernorm_bwd_partial_rows(rows):
     return int(lib().tch_layernorm_bwd_partial_rows(rows))
 
 
-def layernorm_bwd(ctx, dy, x, dx, gamma, mean, rstd, dgamma, dbeta, partial, accumulate=False):
+def layernorm_bwd(ctx, dy, x, dx, gamma, mean, rstd, dgamma, dbeta, partial, accumulate=False, residual=None):
     C = x.shape[-1]
     rows = x.numel() // C
     assert dy.shape == x.shape == dx.shape and dy.dtype == x.dtype == dx.dtype
     assert partial.dtype == torch.float32 and partial.numel() >= layernorm_bwd_partial_rows(rows) * C * 2
-    check(lib().tch_layernorm_bwd(ctx.handle, dtype_code(x), _p(dy), _p(x), _p(dx), _p(gamma), _p(mean), _p(rstd),
+    assert residual is None or (residual.shape == x.shape and residual.dtype == x.dtype)
+    check(lib().tch_layernorm_bwd(ctx.handle, dtype_code(x), _p(dy), _p(x), _p(dx), _p(residual), _p(gamma), _p(mean), _p(rstd),
                                   _p(dgamma), _p(dbeta), int(accumulate), rows, C, _p(partial)), "tch_layernorm_bwd")
 
 

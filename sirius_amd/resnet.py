@@ -23,6 +23,7 @@ import math
 import torch
 
 from . import ops
+from .engine_base import EngineBase
 
 STEM_CIN_PAD = 8
 
@@ -45,26 +46,16 @@ class _Block:
     pass
 
 
-class ResNetEngine:
+class ResNetEngine(EngineBase):
     def __init__(self, depths=(3, 8, 36, 3), num_classes=1000, width=64, dtype=torch.bfloat16, image_size=224,
                  lr=0.1, momentum=0.9, weight_decay=1e-4, bn_momentum=0.1, bn_eps=1e-5, stream=None, allocator=None,
                  overlap_wgrad=True, fuse_bn_stats=True, fuse_bn_bwd=True, autotune=False):
-        if not torch.cuda.is_available():
-            raise RuntimeError("ResNetEngine runs on the GPU only; there is no CPU path")
-        assert dtype in (torch.bfloat16, torch.float32)
+        self._init_engine(dtype, stream, allocator)
         assert num_classes % 8 == 0, "class count must be a multiple of one 16-byte chunk"
-        self.dtype, self.image_size, self.num_classes = dtype, image_size, num_classes
+        self.image_size, self.num_classes = image_size, num_classes
         self.lr, self.momentum, self.weight_decay = lr, momentum, weight_decay
         self.bn_momentum, self.bn_eps = bn_momentum, bn_eps
-        self.dev = torch.device("cuda", torch.cuda.current_device())
-        self.ctx = ops.Context(stream if stream is not None else torch.cuda.current_stream())
         self.depths, self.width = tuple(depths), width
-        # allocator(shape, dtype) -> uninitialised device tensor; the shared HBM pool plugs in here
-        # (torch_col.pool_empty), torch's own allocator is the default
-        self._alloc = allocator if allocator is not None else (
-            lambda shape, dtype: torch.empty(shape, dtype=dtype, device=self.dev))
-        self._hook = None
-        self._cut_exception = None
         # weight gradients depend only on dy and the saved input: recorded on a second lane so that
         # they run beside the data-gradient chain (each kernel alone leaves CUs idle at batch 64);
         # costs the recycling of the dy buffers (they stay alive until the lanes join)
@@ -133,10 +124,6 @@ class ResNetEngine:
         for name, c in self._bn_names:
             self._bn_off[name] = (o, c)
             o += c
-        self._plans = {}
-        self._opt_prog = None
-        self._acc_prog = None
-        self._opt_global_prog = None
 
     # ------------------------------------------------------------------ parameter table
     def _add_param(self, name, kind, shape, store_shape):
@@ -606,69 +593,6 @@ class ResNetEngine:
         plan.bytes = sum(t.numel() * t.element_size() for t in keep)
         return plan
 
-    def plan(self, batch, loss_scale=1.0):
-        key = (int(batch), float(loss_scale))
-        p = self._plans.get(key)
-        if p is None:
-            # plans of other batch sizes own activation memory: drop them first
-            for k in [k for k in self._plans if k[0] != key[0]]:
-                del self._plans[k]
-            p = self._plans[key] = self._build_plan(*key)
-        return p
-
-    def release_activations(self):
-        """Drop every plan (and with it all activation / gradient-scratch memory)."""
-        n = sum(p.bytes for p in self._plans.values())
-        # an exception in flight may still hold a plan through its traceback: with an allocator
-        # that can release a block under a live tensor, give the memory back now
-        release = getattr(self._alloc, "release", None)
-        if release is not None:
-            self.ctx.synchronize()
-            for p in self._plans.values():
-                for t in p.keep:
-                    release(t)
-                p.keep = []
-        self._plans.clear()
-        self._last_plan = None
-        return n
-
-    def last_loss(self):
-        """Mean loss of the most recent micro-batch (nan once its plan has been released)."""
-        p = getattr(self, "_last_plan", None)
-        if p is None or not p.keep:
-            return float("nan")
-        self.ctx.synchronize()
-        return float(p.loss.item())
-
-    def set_checkpoint_hook(self, fn):
-        """fn(phase, layer name) runs between the launch segments of forward_backward, once per
-        layer and direction: the place of the forward / backward module hooks of the reference
-        (torch_col/colocate_ctrl.py:360-402).  An exception raised by fn ends the step there."""
-        self._hook = fn
-
-    def set_cut_exception(self, exc_type):
-        """Raise exc_type from forward_backward when the reject flag cut the replay short (the
-        control thread killed the batch on receipt of a request): what the reference's autograd
-        engine hook does with EngineColocateAdjustL1Exception (csrc/mem_tagging.cc:54-58)."""
-        self._cut_exception = exc_type
-
-    def _run_plan(self, p):
-        if self._hook is None:
-            cut = self.ctx.run(p.prog)
-        else:
-            first, cut = 0, False
-            for idx, phase, name in p.marks:
-                cut = self.ctx.run(p.prog, first, idx) or cut
-                first = idx
-                self._hook(phase, name)
-                if cut and self._cut_exception is not None:
-                    break
-            if first < len(p.prog) and not (cut and self._cut_exception is not None):
-                cut = self.ctx.run(p.prog, first, len(p.prog)) or cut
-        if cut and self._cut_exception is not None:
-            raise self._cut_exception("launches rejected: batch killed on request")
-        return cut
-
     # ------------------------------------------------------------------ the step
     def forward_backward(self, x, y, loss_scale=1.0):
         """x [B,3,S,S] fp32 and y [B] int64 on the GPU.  Returns (plan, cut_short)."""
@@ -683,61 +607,7 @@ class ResNetEngine:
         p = self.plan(batch, loss_scale)
         return p, self._run_plan(p)
 
-    def _flat_prog(self, fn):
-        prog = ops.Program()
-        self.ctx.begin_record(prog)
-        try:
-            fn()
-        finally:
-            self.ctx.end_record()
-        return prog
-
-    def ensure_global_grads(self):
-        if self.global_grads is None:
-            self.global_grads = self._alloc((self.n_store,), torch.float32).zero_()
-
-    def zero_global_grads(self):
-        if self.global_grads is not None:
-            ops.fill_zero(self.ctx, self.global_grads)
-
-    def synchronize(self):
-        self.ctx.synchronize()
-
-    def zero_grad(self):
-        ops.fill_zero(self.ctx, self.grads)
-
-    def discard_partial_grads(self):
-        """After a killed micro-batch: its gradients are partial.  Every backward overwrites the
-        whole gradient buffer, so zeroing is only for the reader of grads_dict()."""
-        ops.fill_zero(self.ctx, self.grads)
-
-    def accumulate(self):
-        """global += grads; grads = 0   (GradAccumulator.accumulate)"""
-        self.ensure_global_grads()
-        if self._acc_prog is None:
-            self._acc_prog = self._flat_prog(lambda: ops.grad_accumulate(self.ctx, self.global_grads, self.grads))
-        return self.ctx.run(self._acc_prog)
-
-    def optimizer_step(self, use_global=False, zero_global=True):
-        """SGD-momentum over the flat buffers; with use_global the accumulated gradients are
-        consumed and zeroed (GradAccumulator.step)."""
-        if use_global:
-            if self.global_grads is None:
-                raise RuntimeError("optimizer_step(use_global=True) before any accumulate()")
-            if self._opt_global_prog is None:
-                def rec():
-                    ops.sgd_momentum_step(self.ctx, self.params, self.global_grads, self.momentum_buf, self.lr,
-                                          self.momentum, self.weight_decay, shadow=self.shadow)
-                    self._refresh_transposed()
-                self._opt_global_prog = self._flat_prog(rec)
-            cut = self.ctx.run(self._opt_global_prog)
-            if zero_global:
-                ops.fill_zero(self.ctx, self.global_grads)
-            return cut
-        if self._opt_prog is None:
-            def rec():
-                ops.sgd_momentum_step(self.ctx, self.params, self.grads, self.momentum_buf, self.lr, self.momentum,
-                                      self.weight_decay, shadow=self.shadow)
-                self._refresh_transposed()
-            self._opt_prog = self._flat_prog(rec)
-        return self.ctx.run(self._opt_prog)
+    def _record_optimizer(self, grads):
+        ops.sgd_momentum_step(self.ctx, self.params, grads, self.momentum_buf, self.lr, self.momentum,
+                              self.weight_decay, shadow=self.shadow)
+        self._refresh_transposed()

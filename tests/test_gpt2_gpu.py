@@ -1,0 +1,107 @@
+"""GPT-2 training step on the GPU (sirius_amd.gpt2.GPT2Engine, every kernel through the C ABI) against the
+CPU oracle (oracle/gpt2.py, itself pinned against transformers' GPT2LMHeadModel) on the same seeded
+weights and token ids: loss, every gradient, and the weights after a few optimizer steps.
+
+Tolerances: fp32 rtol 1e-3, bf16 rtol 2e-2 of the largest magnitude of the oracle tensor.
+"""
+import pytest
+import torch
+
+from oracle import gpt2 as G
+
+pytestmark = pytest.mark.gpu
+
+CFG = dict(vocab=97, n_pos=40, n_embd=64, n_layer=2, n_head=4)   # vocabulary padded to 128 inside the engine
+T = 32
+
+
+def _ids(B, seed):
+    g = torch.Generator()
+    g.manual_seed(seed)
+    return torch.randint(0, CFG["vocab"], (B, T), generator=g)
+
+
+def _state(seed=0):
+    sd = G.make_state_dict(CFG["vocab"], CFG["n_pos"], CFG["n_embd"], CFG["n_layer"], seed=seed)
+    g = torch.Generator()
+    g.manual_seed(seed + 100)
+    for k, v in sd.items():       # biases and LayerNorm parameters away from their trivial initial values
+        if v.dim() == 1:
+            v.add_(torch.randn(v.shape, generator=g) * 0.1)
+    return sd
+
+
+def _rel(got, ref):
+    return (got.float() - ref.float()).abs().max().item() / (ref.float().abs().max().item() + 1e-12)
+
+
+def _engine(dtype, **kw):
+    from sirius_amd.gpt2 import GPT2Engine
+    return GPT2Engine(seq_len=T, dtype=dtype, **CFG, **kw)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-3), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("B", [1, 3])
+def test_loss_and_gradients(dtype, tol, B):
+    print("case", dtype, B, flush=True)
+    sd = _state()
+    if dtype == torch.bfloat16:   # both sides start from weights that bf16 holds exactly
+        sd = {k: v.to(torch.bfloat16).float() for k, v in sd.items()}
+    ids = _ids(B, 1)
+    loss_ref, grads_ref = G.loss_and_grads(sd, ids, CFG["n_head"], CFG["n_layer"], loss_scale=0.5)
+    eng = _engine(dtype)
+    eng.load_state_dict(sd)
+    rt = eng.state_dict()
+    for k in sd:
+        assert torch.equal(rt[k], sd[k]), f"state dict round trip: {k}"
+    p, cut = eng.forward_backward(ids.cuda(), loss_scale=0.5)
+    assert not cut
+    loss = eng.last_loss()
+    assert abs(loss - loss_ref.item()) <= tol * abs(loss_ref.item()), (loss, loss_ref.item())
+    logits_ref = G.forward(sd, ids, CFG["n_head"], CFG["n_layer"]).reshape(B * T, -1)
+    assert _rel(p.logits[:, :CFG["vocab"]].cpu(), logits_ref) <= tol
+    grads = eng.grads_dict()
+    for k, ref in grads_ref.items():
+        assert torch.isfinite(grads[k]).all(), k
+        assert _rel(grads[k], ref) <= tol, (k, _rel(grads[k], ref))
+    # padding rows of the token embedding never receive a gradient
+    pad = eng._view(eng.grads, "transformer.wte.weight").view(eng.vocab_pad, -1)[CFG["vocab"]:]
+    assert torch.all(pad == 0)
+
+
+@pytest.mark.parametrize("optimizer", ["adamw", "sgd"])
+def test_training_steps_fp32(optimizer):
+    sd = _state(2)
+    batches = [_ids(2, 10 + i) for i in range(3)]
+    hp = dict(lr=1e-3, weight_decay=0.01) if optimizer == "adamw" else dict(lr=0.05, weight_decay=1e-4)
+    losses_ref, sd_ref = G.train_steps(sd, batches, CFG["n_head"], CFG["n_layer"], optimizer=optimizer, **hp)
+    eng = _engine(torch.float32, optimizer=optimizer, **hp)
+    eng.load_state_dict(sd)
+    losses = []
+    for ids in batches:
+        eng.forward_backward(ids.cuda())
+        losses.append(eng.last_loss())
+        eng.optimizer_step()
+    got = eng.state_dict()
+    for a, b in zip(losses, losses_ref):
+        assert abs(a - b) <= 1e-3 * abs(b), (losses, losses_ref)
+    for k, ref in sd_ref.items():
+        # what moved must have moved the same way: compare the update, not only the weight
+        assert _rel(got[k] - sd[k], ref - sd[k]) <= 2e-2, (k, _rel(got[k] - sd[k], ref - sd[k]))
+        assert _rel(got[k], ref) <= 1e-3, k
+
+
+def test_accumulated_micro_batches_match_one_batch():
+    """Two micro-batches with the loss scaled by 1/2 and accumulated give the gradient of the whole batch
+    (the reference's GradAccumulator + scale_loss: torch_col/accumulate.py:8-51, dynamic_batch.py:112-120)."""
+    sd = _state(3)
+    ids = _ids(4, 20)
+    _, grads_ref = G.loss_and_grads(sd, ids, CFG["n_head"], CFG["n_layer"])
+    eng = _engine(torch.float32)
+    eng.load_state_dict(sd)
+    for part in (ids[:2], ids[2:]):
+        eng.forward_backward(part.cuda(), loss_scale=0.5)
+        eng.accumulate()
+    got = eng.grads_dict(use_global=True)
+    for k, ref in grads_ref.items():
+        assert _rel(got[k], ref) <= 1e-3, (k, _rel(got[k], ref))

@@ -59,8 +59,12 @@ def test_layernorm(ctx, dtype, rows, C):
     # accumulate on top
     dg2, db2 = dg.clone(), db.clone()
     torch.cuda.synchronize()
-    ops.layernorm_bwd(ctx, dy.cuda(), xd, dx, gamma.cuda(), mean, rstd, dg2, db2, partial, accumulate=True)
+    res = rnd((rows, C), dtype, g)
+    dx_res = torch.empty_like(xd)
+    ops.layernorm_bwd(ctx, dy.cuda(), xd, dx_res, gamma.cuda(), mean, rstd, dg2, db2, partial, accumulate=True,
+                      residual=res.cuda())
     torch.cuda.synchronize()
+    close(dx_res, dx_ref + res.float(), dtype, "ln dx + residual", rtol=1e-3 if dtype == torch.float32 else 1e-2)
     close(mean, mean_ref, torch.float32, "ln mean", rtol=1e-4)
     close(rstd, rstd_ref, torch.float32, "ln rstd", rtol=1e-4)
     close(y, y_ref, dtype, "ln y", rtol=1e-4 if dtype == torch.float32 else 1e-2)
