@@ -188,8 +188,13 @@ int tch_sgd_momentum_step(tch_context* ctx, float* param, const float* grad, flo
 /* global += grad; grad = 0   (pytorch/torch_col/accumulate.py:20-24) */
 int tch_grad_accumulate(tch_context* ctx, float* global, float* grad, int64_t n);
 int tch_fill_zero(tch_context* ctx, void* ptr, int64_t bytes);
+/* dbias[c] (+)= sum over rows of dy[r, c] (dy with leading dimension ld) */
 int tch_bias_grad(tch_context* ctx, int dtype, const void* dy, float* dbias, int rows, int cols, int ld,
                   int accumulate);
+/* The same with fp32 scratch memory (workspace_floats >= 2 * cols is useful, 64 * cols is the most it takes): with
+ * thousands of rows (tokens) the rows are cut into slabs that separate workgroups sum, in a fixed order. */
+int tch_bias_grad_ws(tch_context* ctx, int dtype, const void* dy, float* dbias, int rows, int cols, int ld,
+                     int accumulate, float* workspace, int64_t workspace_floats);
 
 /* ---- transformer operators (Swin-B / GPT-2 steps) --------------------------------------
  * The arithmetic restates torch.nn.LayerNorm / GELU / softmax / AdamW / Embedding as the reference's
@@ -214,9 +219,11 @@ int tch_gelu_bwd(tch_context* ctx, int dtype, const void* dy, const void* x, voi
  * j <= i only (Lq == Lk).  In place (probs == scores) is allowed. */
 int tch_attn_softmax_fwd(tch_context* ctx, int dtype, const void* scores, void* probs, int64_t batch, int heads, int Lq,
                          int Lk, float scale, const float* bias, const float* mask, int windows, int causal);
-/* dscores = scale * probs * (dprobs - sum_j dprobs_j probs_j) per row; rows = batch * heads * Lq. */
+/* dscores = scale * probs * (dprobs - sum_j dprobs_j probs_j) per row; rows = batch * heads * Lq.  causal != 0:
+ * dprobs beyond the query's own position is never read and dscores there is zero.  In place (dscores == dprobs)
+ * is allowed. */
 int tch_attn_softmax_bwd(tch_context* ctx, int dtype, const void* probs, const void* dprobs, void* dscores, int64_t rows,
-                         int Lk, float scale);
+                         int Lq, int Lk, float scale, int causal);
 /* torch.optim.AdamW (decoupled decay, bias correction) over a flat fp32 buffer; step_dev (int32, starts at 0)
  * and scalars_dev (2 floats) live on the device so that a recorded program advances the step by itself. */
 int tch_adamw_step(tch_context* ctx, float* param, const float* grad, float* exp_avg, float* exp_avg_sq,
@@ -229,11 +236,13 @@ int tch_embedding_bwd(tch_context* ctx, int dtype, const int64_t* ids, const voi
                       int T, int C, int vocab, int accumulate_wpe);
 /* C[z](m, n) (+)= alpha * sum_k A[z](m, k) B[z](n, k), z = zo * batch_inner + zi; A(m, k) at
  * a + zo * a_bo + zi * a_bi + m * a_rs + k * a_cs (elements), B alike with n; C row-major with ldc.
- * One stride of each operand must be 1. */
+ * One stride of each operand must be 1.  causal (square problems under a causal mask): 0 nothing is known;
+ * 1 only C(m, n) with n <= m is wanted (tiles wholly above the diagonal are left unwritten); 2 A(m, k) = 0 for
+ * k > m; 3 A(m, k) = 0 for k < m (the reduction is cut to the part that can be non-zero). */
 int tch_batched_gemm(tch_context* ctx, int dtype, const void* a, const void* b, void* c, int M, int N, int K,
                      int64_t a_rs, int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t ldc, int batch_outer,
                      int batch_inner, int64_t a_bo, int64_t a_bi, int64_t b_bo, int64_t b_bi, int64_t c_bo, int64_t c_bi,
-                     float alpha, int accumulate);
+                     float alpha, int accumulate, int causal);
 
 /* ---- layout / precision ---------------------------------------------------------- */
 int tch_nchw_to_nhwc_pad(tch_context* ctx, int dtype, const float* x_nchw, void* y_nhwc, int N, int C, int H, int W,

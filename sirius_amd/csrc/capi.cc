@@ -237,8 +237,8 @@ int tch_attn_softmax_fwd(tch_context* ctx, int dtype, const void* scores, void* 
 }
 
 int tch_attn_softmax_bwd(tch_context* ctx, int dtype, const void* probs, const void* dprobs, void* dscores, int64_t rows,
-                         int Lk, float scale) {
-  return attn_softmax_bwd(C(ctx), dtype, probs, dprobs, dscores, rows, Lk, scale);
+                         int Lq, int Lk, float scale, int causal) {
+  return attn_softmax_bwd(C(ctx), dtype, probs, dprobs, dscores, rows, Lq, Lk, scale, causal);
 }
 
 int tch_adamw_step(tch_context* ctx, float* param, const float* grad, float* exp_avg, float* exp_avg_sq,
@@ -261,9 +261,9 @@ int tch_embedding_bwd(tch_context* ctx, int dtype, const int64_t* ids, const voi
 int tch_batched_gemm(tch_context* ctx, int dtype, const void* a, const void* b, void* c, int M, int N, int K,
                      int64_t a_rs, int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t ldc, int batch_outer,
                      int batch_inner, int64_t a_bo, int64_t a_bi, int64_t b_bo, int64_t b_bi, int64_t c_bo, int64_t c_bi,
-                     float alpha, int accumulate) {
+                     float alpha, int accumulate, int causal) {
   return batched_gemm(C(ctx), dtype, a, b, c, M, N, K, a_rs, a_cs, b_rs, b_cs, ldc, batch_outer, batch_inner, a_bo, a_bi,
-                      b_bo, b_bi, c_bo, c_bi, alpha, accumulate);
+                      b_bo, b_bi, c_bo, c_bi, alpha, accumulate, causal);
 }
 
 int tch_conv2d_wgrad_pick_splits(int dtype, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad) {
@@ -328,6 +328,11 @@ int tch_softmax_ce_lm(tch_context* ctx, int dtype, const float* logits, int ld_l
                       int valid_rows, float loss_scale) {
   return softmax_ce_lm(C(ctx), dtype, logits, ld_logits, labels, loss_rows, loss_mean, dlogits, ld_dlogits, rows, classes,
                        valid_rows, loss_scale);
+}
+
+int tch_bias_grad_ws(tch_context* ctx, int dtype, const void* dy, float* dbias, int rows, int cols, int ld,
+                     int accumulate, float* workspace, int64_t workspace_floats) {
+  return bias_grad(C(ctx), dtype, dy, dbias, rows, cols, ld, accumulate, workspace, workspace_floats);
 }
 
 int tch_sgd_momentum_step(tch_context* ctx, float* param, const float* grad, float* momentum_buf, void* shadow_bf16,

@@ -198,6 +198,8 @@ struct BiasGradArgs {
   const void* dy;
   float* dbias;
   int rows, cols, ld, accumulate;
+  float* partial;     // tall form with row slabs: [slabs][cols] partial sums instead of dbias
+  int rows_per_slab;  // tall form: rows one workgroup (blockIdx.y) covers
 };
 
 // one lane per column; rows are few (the batch)
@@ -209,6 +211,60 @@ __global__ __launch_bounds__(256) void bias_grad_kernel(BiasGradArgs p) {
   const T* src = static_cast<const T*>(p.dy) + c;
   for (int r = 0; r < p.rows; ++r) s += Elem<T>::load(src + static_cast<int64_t>(r) * p.ld);
   p.dbias[c] = p.accumulate ? p.dbias[c] + s : s;
+}
+
+// many rows (tokens): 8 chunk columns x 32 row lanes per workgroup, 16-byte loads, the row lanes
+// meet in LDS in a fixed order
+template <typename T>
+__global__ __launch_bounds__(256) void bias_grad_tall_kernel(BiasGradArgs p) {
+  constexpr int E = Elem<T>::kPerChunk;
+  __shared__ float red[32][8 * E + 1];
+  const int tx = threadIdx.x & 7, ty = threadIdx.x >> 3;
+  const int col = (blockIdx.x * 8 + tx) * E;
+  float s[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) s[e] = 0.f;
+  const int r_begin = blockIdx.y * p.rows_per_slab;
+  const int r_end = r_begin + p.rows_per_slab < p.rows ? r_begin + p.rows_per_slab : p.rows;
+  if (col < p.cols) {
+    const T* src = static_cast<const T*>(p.dy) + col;
+    for (int r = r_begin + ty; r < r_end; r += 32) {
+      Chunk c;
+      c.u = *reinterpret_cast<const uint4*>(src + static_cast<int64_t>(r) * p.ld);
+      float v[E];
+      chunk_to_float<T>(c, v);
+#pragma unroll
+      for (int e = 0; e < E; ++e) s[e] += v[e];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < E; ++e) red[ty][tx * E + e] = s[e];
+  __syncthreads();
+  if (threadIdx.x < 8 * E) {
+    const int c = blockIdx.x * 8 * E + threadIdx.x;
+    if (c < p.cols) {
+      float t = 0.f;
+      for (int y = 0; y < 32; ++y) t += red[y][threadIdx.x];
+      if (p.partial)
+        p.partial[static_cast<int64_t>(blockIdx.y) * p.cols + c] = t;
+      else
+        p.dbias[c] = p.accumulate ? p.dbias[c] + t : t;
+    }
+  }
+}
+
+struct SlabSumArgs {
+  const float* partial;  // [slabs][cols]
+  float* out;
+  int slabs, cols, accumulate;
+};
+
+__global__ __launch_bounds__(256) void slab_sum_kernel(SlabSumArgs p) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= p.cols) return;
+  float t = 0.f;
+  for (int s = 0; s < p.slabs; ++s) t += p.partial[static_cast<int64_t>(s) * p.cols + c];
+  p.out[c] = p.accumulate ? p.out[c] + t : t;
 }
 
 unsigned flat_blocks(int64_t n_vec) {
@@ -275,11 +331,35 @@ int fill_zero(Context* ctx, void* ptr, int64_t bytes) {
                 static_cast<double>(bytes), 1);
 }
 
-int bias_grad(Context* ctx, int dtype, const void* dy, float* dbias, int rows, int cols, int ld, int accumulate) {
+int bias_grad(Context* ctx, int dtype, const void* dy, float* dbias, int rows, int cols, int ld, int accumulate,
+              float* workspace, int64_t workspace_floats) {
   TCH_CHECK_ARG(dtype == kBF16 || dtype == kF32, "bias_grad: dtype must be f32(0) or bf16(1)");
   TCH_CHECK_ARG(dy && dbias && rows > 0 && cols > 0 && ld >= cols, "bias_grad: bad arguments");
-  BiasGradArgs a{dy, dbias, rows, cols, ld, accumulate};
+  BiasGradArgs a{dy, dbias, rows, cols, ld, accumulate, nullptr, rows};
   const double bytes = static_cast<double>(rows) * cols * (dtype == kBF16 ? 2.0 : 4.0);
+  const int E = dtype == kBF16 ? 8 : 4;
+  if (rows >= 256 && cols % E == 0 && ld % E == 0 && (reinterpret_cast<uintptr_t>(dy) & 15) == 0) {
+    // with scratch memory the rows are cut into slabs (more workgroups), summed by a second small launch
+    int slabs = 1;
+    if (workspace) {
+      slabs = rows / 256;
+      if (slabs > 64) slabs = 64;
+      if (static_cast<int64_t>(slabs) * cols > workspace_floats) slabs = static_cast<int>(workspace_floats / cols);
+      if (slabs < 1) slabs = 1;
+    }
+    if (slabs > 1) {
+      a.partial = workspace;
+      a.rows_per_slab = (rows + slabs - 1) / slabs;
+      slabs = (rows + a.rows_per_slab - 1) / a.rows_per_slab;
+    }
+    const dim3 grid((cols / E + 7) / 8, slabs);
+    int rc = dtype == kBF16
+                 ? launch(ctx, bias_grad_tall_kernel<bf16>, grid, dim3(256), a, "bias_grad_tall_kernel<bf16>", bytes, 1)
+                 : launch(ctx, bias_grad_tall_kernel<float>, grid, dim3(256), a, "bias_grad_tall_kernel<f32>", bytes, 1);
+    if (rc || slabs == 1) return rc;
+    SlabSumArgs s{workspace, dbias, slabs, cols, accumulate};
+    return launch(ctx, slab_sum_kernel, dim3((cols + 255) / 256), dim3(256), s, "slab_sum_kernel", 4.0 * slabs * cols, 1);
+  }
   return dtype == kBF16 ? launch(ctx, bias_grad_kernel<bf16>, dim3((cols + 255) / 256), dim3(256), a, "bias_grad_kernel<bf16>", bytes, 1)
                         : launch(ctx, bias_grad_kernel<float>, dim3((cols + 255) / 256), dim3(256), a, "bias_grad_kernel<f32>", bytes, 1);
 }

@@ -74,8 +74,8 @@ int gelu_fwd(Context* ctx, int dtype, const void* x, void* y, int64_t n, int tan
 int gelu_bwd(Context* ctx, int dtype, const void* dy, const void* x, void* dx, int64_t n, int tanh_form);
 int attn_softmax_fwd(Context* ctx, int dtype, const void* scores, void* probs, int64_t batch, int heads, int Lq, int Lk,
                      float scale, const float* bias, const float* mask, int windows, int causal);
-int attn_softmax_bwd(Context* ctx, int dtype, const void* probs, const void* dprobs, void* dscores, int64_t rows, int Lk,
-                     float scale);
+int attn_softmax_bwd(Context* ctx, int dtype, const void* probs, const void* dprobs, void* dscores, int64_t rows, int Lq,
+                     int Lk, float scale, int causal);
 int adamw_step(Context* ctx, float* param, const float* grad, float* exp_avg, float* exp_avg_sq, void* shadow_bf16,
                int64_t n, double lr, double beta1, double beta2, double eps, double weight_decay, int* step_dev,
                float* scalars_dev);
@@ -87,7 +87,7 @@ int embedding_bwd(Context* ctx, int dtype, const int64_t* ids, const void* dy, f
 // bgemm.hip
 int batched_gemm(Context* ctx, int dtype, const void* a, const void* b, void* c, int M, int N, int K, int64_t a_rs,
                  int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t ldc, int batch_outer, int batch_inner, int64_t a_bo,
-                 int64_t a_bi, int64_t b_bo, int64_t b_bi, int64_t c_bo, int64_t c_bi, float alpha, int accumulate);
+                 int64_t a_bi, int64_t b_bo, int64_t b_bi, int64_t c_bo, int64_t c_bi, float alpha, int accumulate, int causal);
 
 // pool.hip
 int maxpool_fwd(Context* ctx, int dtype, const void* x, void* y, int32_t* index, int N, int H, int W, int C, int ksize,
@@ -108,7 +108,8 @@ int sgd_momentum_step(Context* ctx, float* param, const float* grad, float* mome
                       int64_t n, float lr, float momentum, float weight_decay);
 int grad_accumulate(Context* ctx, float* global, float* grad, int64_t n);
 int fill_zero(Context* ctx, void* ptr, int64_t bytes);
-int bias_grad(Context* ctx, int dtype, const void* dy, float* dbias, int rows, int cols, int ld, int accumulate);
+int bias_grad(Context* ctx, int dtype, const void* dy, float* dbias, int rows, int cols, int ld, int accumulate,
+              float* workspace = nullptr, int64_t workspace_floats = 0);
 
 // layout.hip
 int nchw_to_nhwc_pad(Context* ctx, int dtype, const float* x_nchw, void* y_nhwc, int N, int C, int H, int W, int Cpad);

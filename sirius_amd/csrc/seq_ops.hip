@@ -310,12 +310,16 @@ __global__ __launch_bounds__(256) void attn_softmax_kernel(SoftmaxArgs p) {
   const T* src = static_cast<const T*>(p.s) + row * p.Lk;
   T* dst = static_cast<T*>(p.out) + row * p.Lk;
   if (BWD) {
+    // causal: probabilities beyond the query's own position are zero and dp there is never read (it
+    // may be unwritten memory)
+    const int i = static_cast<int>(row % p.Lq);
+    const int limit = p.causal ? (i + 1 < p.Lk ? i + 1 : p.Lk) : p.Lk;
     const T* dp = static_cast<const T*>(p.dp) + row * p.Lk;
     float dot = 0.f;
-    for (int j = lane; j < p.Lk; j += 64) dot += Elem<T>::load(src + j) * Elem<T>::load(dp + j);
+    for (int j = lane; j < limit; j += 64) dot += Elem<T>::load(src + j) * Elem<T>::load(dp + j);
     dot = wave_sum(dot);
     for (int j = lane; j < p.Lk; j += 64)
-      Elem<T>::store(dst + j, p.scale * Elem<T>::load(src + j) * (Elem<T>::load(dp + j) - dot));
+      Elem<T>::store(dst + j, j < limit ? p.scale * Elem<T>::load(src + j) * (Elem<T>::load(dp + j) - dot) : 0.f);
     return;
   }
   const int i = static_cast<int>(row % p.Lq);
@@ -550,11 +554,12 @@ int attn_softmax_fwd(Context* ctx, int dtype, const void* scores, void* probs, i
                         : launch(ctx, attn_softmax_kernel<float, 0>, grid, dim3(256), a, "attn_softmax_kernel<f32,fwd>", bytes, 1);
 }
 
-int attn_softmax_bwd(Context* ctx, int dtype, const void* probs, const void* dprobs, void* dscores, int64_t rows, int Lk,
-                     float scale) {
+int attn_softmax_bwd(Context* ctx, int dtype, const void* probs, const void* dprobs, void* dscores, int64_t rows, int Lq,
+                     int Lk, float scale, int causal) {
   TCH_CHECK_ARG(dtype == kBF16 || dtype == kF32, "attn_softmax: dtype must be f32(0) or bf16(1)");
-  TCH_CHECK_ARG(probs && dprobs && dscores && rows > 0 && Lk > 0, "attn_softmax_bwd: bad arguments");
-  SoftmaxArgs a{probs, dprobs, dscores, nullptr, nullptr, rows, 1, 1, Lk, 1, 0, scale};
+  TCH_CHECK_ARG(probs && dprobs && dscores && rows > 0 && Lk > 0 && Lq > 0 && rows % Lq == 0, "attn_softmax_bwd: bad arguments");
+  TCH_CHECK_ARG(!causal || Lq == Lk, "attn_softmax_bwd: the causal form needs square score matrices");
+  SoftmaxArgs a{probs, dprobs, dscores, nullptr, nullptr, rows, 1, Lq, Lk, 1, causal, scale};
   const double bytes = static_cast<double>(rows) * Lk * (dtype == kBF16 ? 6.0 : 12.0);
   const dim3 grid(static_cast<unsigned>((rows + 3) / 4));
   return dtype == kBF16 ? launch(ctx, attn_softmax_kernel<bf16, 1>, grid, dim3(256), a, "attn_softmax_kernel<bf16,bwd>", bytes, 1)

@@ -218,6 +218,7 @@ class GPT2Engine(EngineBase):
                 sp = int(ops.lib().tch_conv2d_wgrad_pick_splits(code, R, 1, 1, Cin, K, 1, 1, 1, 0))
                 ws_bytes = max(ws_bytes, ops.conv2d_wgrad_workspace_bytes(code, K, 1, 1, Cin, sp))
         wg_ws = act(ws_bytes // 4, dtype=torch.float32)
+        bias_ws = act(64 * 4 * C, dtype=torch.float32)   # row-slab partial sums of the bias gradients
 
         def ln_stats(i):
             return ln_mean[i * R:(i + 1) * R], ln_rstd[i * R:(i + 1) * R]
@@ -243,7 +244,7 @@ class GPT2Engine(EngineBase):
         def lin_bwd(name, x, dy, dx):
             """dW, db from (x, dy); dx = dy W"""
             ops.conv2d_wgrad(ctx, as4(x), as4(dy), self._view(self.grads, name + ".weight"), 1, 0, workspace=wg_ws)
-            ops.bias_grad(ctx, dy, self._view(self.grads, name + ".bias"))
+            ops.bias_grad(ctx, dy, self._view(self.grads, name + ".bias"), workspace=bias_ws)
             ops.conv2d_dgrad(ctx, as4(dy), self._wt(name + ".weight"), as4(dx), 1, 0)
 
         # strides / batch offsets of head h of sample b inside the packed projection and the score tensor
@@ -271,10 +272,12 @@ class GPT2Engine(EngineBase):
                 lin_fwd(pre + "attn.c_attn", a, qkv)
                 flat = qkv.view(-1)
                 P = act(B, H, T, T)
-                ops.batched_gemm(ctx, flat, flat[C:], P, T, T, D, (qkv_row, 1), (qkv_row, 1), T, (B, H), qkv_b, qkv_b, s_b)
+                ops.batched_gemm(ctx, flat, flat[C:], P, T, T, D, (qkv_row, 1), (qkv_row, 1), T, (B, H), qkv_b, qkv_b, s_b,
+                                 causal=1)
                 ops.attn_softmax_fwd(ctx, P, P, scale, causal=True)
                 o = act(R, C)
-                ops.batched_gemm(ctx, P, flat[2 * C:], o, T, D, T, (T, 1), (1, qkv_row), C, (B, H), s_b, qkv_b, o_b)
+                ops.batched_gemm(ctx, P, flat[2 * C:], o, T, D, T, (T, 1), (1, qkv_row), C, (B, H), s_b, qkv_b, o_b,
+                                 causal=2)
                 h1 = act(R, C)
                 lin_fwd(pre + "attn.c_proj", o, h1, add=h)
                 m, f1, f2 = act(R, C), act(R, 4 * C), act(R, 4 * C)
@@ -318,13 +321,15 @@ class GPT2Engine(EngineBase):
                 ln_bwd(pre + "ln_2", 2 * i + 1, d_m, h1, g1, residual=g)
                 # attention
                 lin_bwd(pre + "attn.c_proj", o, g1, d_o)
-                ops.batched_gemm(ctx, P, d_o, gflat[2 * C:], T, D, T, (1, T), (1, C), qkv_row, (B, H), s_b, o_b, qkv_b)
-                ops.batched_gemm(ctx, d_o, flat[2 * C:], dP, T, T, D, (C, 1), (qkv_row, 1), T, (B, H), o_b, qkv_b, s_b)
-                ops.attn_softmax_bwd(ctx, P, dP, dP, scale)
+                ops.batched_gemm(ctx, P, d_o, gflat[2 * C:], T, D, T, (1, T), (1, C), qkv_row, (B, H), s_b, o_b, qkv_b,
+                                 causal=3)
+                ops.batched_gemm(ctx, d_o, flat[2 * C:], dP, T, T, D, (C, 1), (qkv_row, 1), T, (B, H), o_b, qkv_b, s_b,
+                                 causal=1)
+                ops.attn_softmax_bwd(ctx, P, dP, dP, scale, causal=True)
                 ops.batched_gemm(ctx, dP, flat[C:], gflat, T, D, T, (T, 1), (1, qkv_row), qkv_row, (B, H), s_b, qkv_b,
-                                 qkv_b)
+                                 qkv_b, causal=2)
                 ops.batched_gemm(ctx, dP, flat, gflat[C:], T, D, T, (1, T), (1, qkv_row), qkv_row, (B, H), s_b, qkv_b,
-                                 qkv_b)
+                                 qkv_b, causal=3)
                 d_a = d_m   # free again
                 lin_bwd(pre + "attn.c_attn", a, g_qkv, d_a)
                 g_next = d_o

@@ -384,9 +384,14 @@ def fill_zero(ctx, t):
     check(lib().tch_fill_zero(ctx.handle, _p(t), t.numel() * t.element_size()), "tch_fill_zero")
 
 
-def bias_grad(ctx, dy, dbias, cols=None, accumulate=False):
+def bias_grad(ctx, dy, dbias, cols=None, accumulate=False, workspace=None):
     rows, ld = dy.shape
     cols = ld if cols is None else cols
+    if workspace is not None:
+        assert workspace.dtype == torch.float32
+        check(lib().tch_bias_grad_ws(ctx.handle, dtype_code(dy), _p(dy), _p(dbias), rows, cols, ld, int(accumulate),
+                                     _p(workspace), workspace.numel()), "tch_bias_grad_ws")
+        return
     check(lib().tch_bias_grad(ctx.handle, dtype_code(dy), _p(dy), _p(dbias), rows, cols, ld, int(accumulate)),
           "tch_bias_grad")
 
@@ -491,11 +496,11 @@ def attn_softmax_fwd(ctx, scores, probs, scale=1.0, bias=None, mask=None, causal
                                      _p(bias), _p(mask), windows, int(causal)), "tch_attn_softmax_fwd")
 
 
-def attn_softmax_bwd(ctx, probs, dprobs, dscores, scale=1.0):
-    Lk = probs.shape[-1]
+def attn_softmax_bwd(ctx, probs, dprobs, dscores, scale=1.0, causal=False):
+    Lq, Lk = probs.shape[-2:]
     assert probs.shape == dprobs.shape == dscores.shape and probs.dtype == dprobs.dtype == dscores.dtype
     check(lib().tch_attn_softmax_bwd(ctx.handle, dtype_code(probs), _p(probs), _p(dprobs), _p(dscores),
-                                     probs.numel() // Lk, Lk, scale), "tch_attn_softmax_bwd")
+                                     probs.numel() // Lk, Lq, Lk, scale, int(causal)), "tch_attn_softmax_bwd")
 
 
 def adamw_step(ctx, param, grad, exp_avg, exp_avg_sq, step_dev, scalars_dev, lr, beta1=0.9, beta2=0.999, eps=1e-8,
@@ -528,7 +533,7 @@ def embedding_bwd(ctx, ids, dy, dwte, dwpe, accumulate_wpe=False):
 
 
 def batched_gemm(ctx, a, b, c, M, N, K, a_strides, b_strides, ldc, batch=(1, 1), a_batch=(0, 0), b_batch=(0, 0),
-                 c_batch=(0, 0), alpha=1.0, accumulate=False):
+                 c_batch=(0, 0), alpha=1.0, accumulate=False, causal=0):
     """C[z](m, n) (+)= alpha * sum_k A[z](m, k) * B[z](n, k); strides are (row, k) in elements, batch offsets are
     (outer, inner) in elements, z = outer * batch[1] + inner.  The caller vouches that every address the
     strides reach lies inside the tensors; what can be checked from the tensor sizes is checked here."""
@@ -543,4 +548,4 @@ def batched_gemm(ctx, a, b, c, M, N, K, a_strides, b_strides, ldc, batch=(1, 1),
         "batched_gemm: C reaches past its tensor"
     check(lib().tch_batched_gemm(ctx.handle, dtype_code(a), _p(a), _p(b), _p(c), M, N, K, a_strides[0], a_strides[1],
                                  b_strides[0], b_strides[1], ldc, bo, bi, a_batch[0], a_batch[1], b_batch[0], b_batch[1],
-                                 c_batch[0], c_batch[1], alpha, int(accumulate)), "tch_batched_gemm")
+                                 c_batch[0], c_batch[1], alpha, int(accumulate), int(causal)), "tch_batched_gemm")

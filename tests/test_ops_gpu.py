@@ -395,14 +395,27 @@ def test_layout_and_cast(ctx, dtype):
     assert torch.equal(dst.cpu(), src.to(dtype)) and torch.equal(back.cpu(), src.to(dtype).float())
 
 
-def test_bias_grad(ctx):
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,cols", [(16, 1000), (8192, 2304), (1000, 72), (257, 8)])
+def test_bias_grad(ctx, dtype, rows, cols):
+    """few rows (a batch of logits) and many rows (tokens of a transformer projection)"""
     from sirius_amd import ops
     g = _gen(13)
-    dy = rnd((16, 1000), torch.bfloat16, g)
-    db = torch.zeros(1000, device="cuda")
+    dy = rnd((rows, cols), dtype, g)
+    db = torch.ones(cols, device="cuda")
     ops.bias_grad(ctx, dy.cuda(), db)
     torch.cuda.synchronize()
-    close(db, dy.float().sum(0), torch.float32, "bias grad", rtol=1e-5)
+    close(db, dy.double().sum(0).float(), torch.float32, "bias grad", rtol=1e-5)
+    ops.bias_grad(ctx, dy.cuda(), db, accumulate=True)
+    torch.cuda.synchronize()
+    close(db, 2 * dy.double().sum(0).float(), torch.float32, "bias grad accumulated", rtol=1e-5)
+    # with scratch memory (rows summed in slabs); a scratch too small for two slabs falls back to one
+    for floats in (64 * cols, 3 * cols, cols):
+        ws = torch.full((floats,), float("nan"), device="cuda")
+        db2 = torch.ones(cols, device="cuda")
+        ops.bias_grad(ctx, dy.cuda(), db2, accumulate=True, workspace=ws)
+        torch.cuda.synchronize()
+        close(db2, 1 + dy.double().sum(0).float(), torch.float32, "bias grad with scratch", rtol=1e-5)
 
 
 def test_program_record_replay(ctx):

@@ -137,6 +137,15 @@ def test_attn_softmax(ctx, dtype, case):
     close(ds, ds_ref, dtype, "softmax bwd", rtol=1e-4 if dtype == torch.float32 else 1e-2)
     if dtype == torch.float32:
         close(ds, S.attn_softmax_bwd(s, dp, scale, bias, mask, causal), dtype, "softmax bwd vs autograd", rtol=1e-4)
+    if causal:
+        # the causal form never reads dp beyond the query's own position: poison it
+        poisoned = dp.clone().float()
+        poisoned[..., torch.triu(torch.ones(L, L, dtype=torch.bool), 1)] = float("nan")
+        ds2 = torch.full_like(p, 5.0)
+        ops.attn_softmax_bwd(ctx, p, poisoned.to(dtype).cuda(), ds2, scale, causal=True)
+        torch.cuda.synchronize()
+        close(ds2, ds_ref, dtype, "causal softmax bwd", rtol=1e-4 if dtype == torch.float32 else 1e-2)
+        assert torch.all(ds2.float().cpu().triu(1) == 0)
 
 
 @pytest.mark.parametrize("n", [5, 1000, (1 << 20) + 3])
@@ -248,6 +257,39 @@ def test_batched_gemm_attention_products(ctx, dtype, B, H, T, D):
     close(got[:, :, 2], torch.einsum("bhts,bhtd->bshd", p.float(), dof), dtype, "P^T dO", rtol=tol)
     close(got[:, :, 0], torch.einsum("bhts,bhsd->bthd", ds.float(), k), dtype, "dS K", rtol=tol)
     close(got[:, :, 1], torch.einsum("bhts,bhtd->bshd", ds.float(), q), dtype, "dS^T Q", rtol=tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,D", [(200, 64), (64, 16), (130, 32)])
+def test_batched_gemm_causal_forms(ctx, dtype, T, D):
+    """What a causal mask leaves of a square problem: (1) only the lower triangle of the output is wanted and the
+    tiles above the diagonal stay untouched; (2) / (3) A is lower / upper triangular and the reduction is cut."""
+    from sirius_amd import ops
+    g = _gen(38)
+    tol = 1e-3 if dtype == torch.float32 else 2e-2
+    Z = 3
+    q, k = rnd((Z, T, D), dtype, g), rnd((Z, T, D), dtype, g)
+    s = torch.full((Z, T, T), 7.0, dtype=dtype, device="cuda")
+    ops.batched_gemm(ctx, q.cuda(), k.cuda(), s, T, T, D, (D, 1), (D, 1), T, (Z, 1), (T * D, 0), (T * D, 0), (T * T, 0),
+                     causal=1)
+    torch.cuda.synchronize()
+    ref = torch.einsum("ztd,zsd->zts", q.float(), k.float())
+    low = torch.tril(torch.ones(T, T, dtype=torch.bool))
+    got = s.float().cpu()
+    close(got * low, ref * low, dtype, "lower triangle", rtol=tol)
+    tiles = (torch.arange(T)[None, :] // 64) > (torch.arange(T)[:, None] // 64)      # tiles wholly above the diagonal
+    assert torch.all(got[:, tiles] == 7.0), "tiles above the diagonal must be left unwritten"
+    p_low = (rnd((Z, T, T), dtype, g, 0.3).float() * low).to(dtype)
+    v = rnd((Z, T, D), dtype, g)
+    o = torch.empty((Z, T, D), dtype=dtype, device="cuda")
+    ops.batched_gemm(ctx, p_low.cuda(), v.cuda(), o, T, D, T, (T, 1), (1, D), D, (Z, 1), (T * T, 0), (T * D, 0),
+                     (T * D, 0), causal=2)
+    o_t = torch.empty((Z, T, D), dtype=dtype, device="cuda")
+    ops.batched_gemm(ctx, p_low.cuda(), v.cuda(), o_t, T, D, T, (1, T), (1, D), D, (Z, 1), (T * T, 0), (T * D, 0),
+                     (T * D, 0), causal=3)
+    torch.cuda.synchronize()
+    close(o, torch.einsum("zts,zsd->ztd", p_low.float(), v.float()), dtype, "P V, lower-triangular P", rtol=tol)
+    close(o_t, torch.einsum("zts,ztd->zsd", p_low.float(), v.float()), dtype, "P^T dO, lower-triangular P", rtol=tol)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
