@@ -174,6 +174,7 @@ class EventManager:
 
 def initialize_sgd_optimizer(model, optimizer=None):
     """util.py:182-191 pre-creates zero gradients and momentum buffers so that memory is stable
-    from the first step; the engine allocates both flat buffers when it is built, so this only
-    checks that they exist."""
-    assert model.grads is not None and model.momentum_buf is not None
+    from the first step; the engine allocates its flat gradient and optimizer-state buffers when it is
+    built, so this only checks that they exist."""
+    state = [getattr(model, n, None) for n in ("momentum_buf", "exp_avg")]
+    assert model.grads is not None and any(t is not None for t in state)
