@@ -22,6 +22,16 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_FLOPS = 2.5e15   # MI355X dense bf16 MFMA
 PEAK_HBM_BYTES = 8.0e12    # MI355X HBM3E
 METRIC = "ResNet-152 bf16 bs64 train images/sec on 1 GPU; conv MFMA util %"
+# HBM bytes per launch of the kernels that can top the step, from two rocprofv3 --pmc runs of this file
+# (FETCH_SIZE and WRITE_SIZE, KiB per dispatch, scaled by what the same counters read for the --calibrate
+# copy of known size: factors 2.000 and 1.000); the summary is profiles/resnet152_bf16_bs64_step_kernel_stats_and_traffic.txt
+MEASURED_TRAFFIC_MIB = {
+    "wgrad_kernel<bf16,128x128>": 27.97 + 24.29,
+    "bn_apply_kernel<bf16,bwd>": 36.33 + 17.76,
+    "bn_apply_kernel<bf16,fwd>": 28.19 + 17.76,
+    "igemm2_kernel<bf16,dgrad,128x64,3buf>": 58.22 + 21.16,
+    "igemm2_kernel<bf16,fwd,128x64,3buf>": 31.84 + 18.31,
+}
 
 
 def cpu_baseline(batch, timed_steps):
@@ -89,9 +99,51 @@ def handover(batch):
     return res
 
 
+def gpt2_step(batch=8, seq_len=1024, warmup=2, steps=5):
+    """BASELINE configs[4]'s training side: GPT-2 small (124.4 M parameters), bf16 compute with fp32 master
+    weights, token ids uniform in [0, 50257) of shape [8, 1024], AdamW.  Reported beside the headline figure."""
+    import torch
+    from sirius_amd.gpt2 import GPT2Engine
+    eng = GPT2Engine(seq_len=seq_len, dtype=torch.bfloat16, optimizer="adamw")
+    eng.init_normal(0)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(2)
+    ids = torch.randint(0, eng.vocab, (batch, seq_len), device="cuda", generator=g)
+    for _ in range(warmup):
+        eng.forward_backward(ids)
+        eng.optimizer_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        eng.forward_backward(ids)
+        eng.optimizer_step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    plan = eng.plan(batch)
+    rows = eng.ctx.profile(plan.prog, 1) + eng.ctx.profile(eng._opt_prog, 1)
+    rows.sort(key=lambda r: -r["total_ms"])
+    gemm = [r for r in rows if not r["work_is_bytes"]]
+    flops = sum(r["work"] for r in gemm)
+    res = {
+        "workload": f"GPT-2 small training step, bf16, ids [{batch}, {seq_len}], AdamW(lr 1e-3, wd 0.01)",
+        "tokens_per_s": batch * seq_len / dt, "ms_per_step": dt * 1e3, "loss_after_run": eng.last_loss(),
+        "parameters": eng.num_parameters(), "launches_per_step": len(plan.prog) + len(eng._opt_prog),
+        "mfma_tflop_per_step": flops / 1e12,
+        "mfma_kernel_ms_per_step": sum(r["total_ms"] for r in gemm),
+        "mfma_util": flops / (sum(r["total_ms"] for r in gemm) * 1e-3) / PEAK_BF16_FLOPS,
+        "breakdown": [{"kernel": r["name"], "ms_per_step": round(r["total_ms"], 4), "launches": r["launches"]}
+                      for r in rows[:8]],
+    }
+    del eng, plan
+    torch.cuda.empty_cache()
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--no-handover", action="store_true", help="skip the 64 -> 16 -> 64 handover measurement")
+    ap.add_argument("--no-gpt2", action="store_true", help="skip the GPT-2 step measurement")
+    ap.add_argument("--only-gpt2", action="store_true", help="run the GPT-2 step measurement alone (for profiling it)")
     ap.add_argument("--no-autotune", action="store_true", help="keep the library's tiling heuristic")
     ap.add_argument("--no-overlap", action="store_true", help="record weight gradients on the main lane (one stream)")
     ap.add_argument("--calibrate", action="store_true",
@@ -113,6 +165,9 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs the GPU; there is no CPU fallback"
     torch.cuda.set_device(0)
+    if args.only_gpt2:
+        print(json.dumps({"gpt2": gpt2_step(steps=args.steps, warmup=args.warmup)}), flush=True)
+        return
     B = args.batch
     eng = ResNetEngine((3, 8, 36, 3), 1000, 64, dtype=torch.bfloat16, image_size=224, lr=0.1, momentum=0.9,
                        weight_decay=1e-4, overlap_wgrad=not args.no_overlap, autotune=not args.no_autotune)
@@ -167,7 +222,8 @@ def main():
         "peak": peak / (1e9 if top["work_is_bytes"] else 1e12),
         "unit": "GB/s" if top["work_is_bytes"] else "TFLOP/s",
         "frac": achieved / peak,
-        "traffic": None,
+        "traffic": MEASURED_TRAFFIC_MIB[top["name"]] * 2 ** 20 if top["name"] in MEASURED_TRAFFIC_MIB else None,
+        "traffic_unit": "bytes per launch (HBM, rocprofv3 FETCH_SIZE + WRITE_SIZE, calibrated)",
         "avg_launch_us": per_launch_s * 1e6,
         "launches_per_step": top["launches"] // reps,
         "share_of_step_kernel_time": top["total_ms"] / reps / total_ms,
@@ -207,13 +263,18 @@ def main():
         out["cpu_baseline"] = cpu_baseline(B, args.cpu_steps)
     else:
         out["cpu_baseline"] = None
+    del eng, plan, x, y
+    torch.cuda.empty_cache()
     if not args.no_handover:
-        del eng, plan, x, y
-        torch.cuda.empty_cache()
         try:
             out["handover"] = handover(B)
         except Exception as e:  # the headline figure stands on its own; say what went wrong
             out["handover"] = {"error": repr(e)}
+    if not args.no_gpt2:
+        try:
+            out["gpt2"] = gpt2_step()
+        except Exception as e:
+            out["gpt2"] = {"error": repr(e)}
     print(json.dumps(out), flush=True)
 
 
