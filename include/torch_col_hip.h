@@ -130,6 +130,25 @@ int tch_conv2d_dgrad_bnsums(tch_context* ctx, int dtype, const void* dy, const v
                             const float* bn_invstd, float* bn_partial);
 int tch_conv2d_dgrad_stat_rows(int dtype, int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
                                int tile_cfg);
+/* Convolution + the whole front half of the BatchNorm next to it, in one call: the sums as above, and the
+ * per-channel coefficients from them (by the workgroup that finishes a column tile last, or by a finalize launch
+ * when there are more than 256 row tiles).  counters: >= ceil(channels / 64) ints, zero before the call, zero
+ * after it.  Forward: save_mean / save_invstd / running statistics are updated, coef = scale[K], shift[K];
+ * finish with tch_bn_apply_fwd.  Data gradient: dgamma / dbeta (+)=, coef = [3][C]; finish with tch_bn_apply_bwd. */
+int tch_conv2d_fwd_bn(tch_context* ctx, int dtype, const void* x, const void* w, void* y, int N, int H, int W, int C,
+                      int K, int R, int S, int stride, int pad, int tile_cfg, int c_logical, float* bn_partial,
+                      int* counters, const float* gamma, const float* beta, float* running_mean, float* running_var,
+                      float* save_mean, float* save_invstd, float momentum, float eps, float* coef);
+int tch_conv2d_dgrad_bn(tch_context* ctx, int dtype, const void* dy, const void* wt, void* dx, const void* add,
+                        const void* mask, int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
+                        int tile_cfg, int c_logical, const void* bn_mask, const void* bn_x, const float* bn_mean,
+                        const float* bn_invstd, float* bn_partial, int* counters, const float* gamma, float* dgamma,
+                        float* dbeta, int accumulate, float* coef);
+/* y = relu?(x * scale + shift (+ residual)), coef = scale[C], shift[C];  dx = c0 * g + c1 * x + c2, coef = [3][C] */
+int tch_bn_apply_fwd(tch_context* ctx, int dtype, const void* x, void* y, const void* residual, int relu, int64_t rows,
+                     int C, const float* coef);
+int tch_bn_apply_bwd(tch_context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int C,
+                     const float* coef);
 /* dw[K,R,S,C] (fp32) (+)= sum over pixels of dy x x.  splits > 1 needs a workspace of
  * tch_conv2d_wgrad_workspace_bytes(); splits <= 0 lets the library choose (query with _pick_splits). */
 int tch_conv2d_wgrad_pick_splits(int dtype, int N, int H, int W, int C, int K, int R, int S, int stride, int pad);

@@ -358,6 +358,56 @@ int bn_fwd_train(Context* ctx, int dtype, const void* x, void* y, const void* re
                                  "bn_apply_kernel<f32,fwd>", apply_bytes, 1);
 }
 
+int bn_fwd_finalize(Context* ctx, const float* partial, int row_blocks, int C, int64_t rows, const float* gamma,
+                    const float* beta, float* running_mean, float* running_var, float* save_mean, float* save_invstd,
+                    float* coef, float momentum, float eps) {
+  TCH_CHECK_ARG(partial && gamma && beta && save_mean && save_invstd && coef && row_blocks >= 1 && C > 0 && rows > 0,
+                "bn_fwd_finalize: bad arguments");
+  TCH_CHECK_ARG((running_mean == nullptr) == (running_var == nullptr), "bn_fwd_finalize: running stats come in pairs");
+  FwdFinalizeArgs f{partial, row_blocks, C, rows, gamma, beta, running_mean, running_var, save_mean, save_invstd,
+                    coef,    coef + C,   momentum, eps};
+  return launch(ctx, bn_fwd_finalize_kernel, dim3((C + 7) / 8), dim3(256), f, "bn_fwd_finalize_kernel",
+                8.0 * row_blocks * C, 1);
+}
+
+int bn_bwd_finalize(Context* ctx, const float* partial, int row_blocks, int C, int64_t rows, const float* gamma,
+                    const float* save_mean, const float* save_invstd, float* dgamma, float* dbeta, float* coef,
+                    int accumulate) {
+  TCH_CHECK_ARG(partial && gamma && save_mean && save_invstd && dgamma && dbeta && coef && row_blocks >= 1 && C > 0 &&
+                    rows > 0,
+                "bn_bwd_finalize: bad arguments");
+  BwdFinalizeArgs f{partial, row_blocks, C, rows, gamma, save_mean, save_invstd, dgamma, dbeta, coef, accumulate};
+  return launch(ctx, bn_bwd_finalize_kernel, dim3((C + 7) / 8), dim3(256), f, "bn_bwd_finalize_kernel",
+                8.0 * row_blocks * C, 1);
+}
+
+int bn_apply_fwd(Context* ctx, int dtype, const void* x, void* y, const void* residual, int relu, int64_t rows, int C,
+                 const float* coef) {
+  if (int rc = check_common(rows, C, dtype)) return rc;
+  TCH_CHECK_ARG(x && y && coef, "bn_apply_fwd: null tensor");
+  Geometry g = geometry(rows, C, dtype);
+  const double tensor_bytes = static_cast<double>(rows) * C * (dtype == kBF16 ? 2.0 : 4.0);
+  ApplyArgs a{x, residual, nullptr, y, coef, coef + C, nullptr, rows * g.cc, FastDiv(g.cc), relu};
+  const double apply_bytes = tensor_bytes * (residual ? 3.0 : 2.0);
+  return dtype == kBF16 ? launch(ctx, bn_apply_kernel<bf16, 0>, dim3(apply_blocks(a.chunks)), dim3(256), a,
+                                 "bn_apply_kernel<bf16,fwd>", apply_bytes, 1)
+                        : launch(ctx, bn_apply_kernel<float, 0>, dim3(apply_blocks(a.chunks)), dim3(256), a,
+                                 "bn_apply_kernel<f32,fwd>", apply_bytes, 1);
+}
+
+int bn_apply_bwd(Context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int C,
+                 const float* coef) {
+  if (int rc = check_common(rows, C, dtype)) return rc;
+  TCH_CHECK_ARG(g && x && dx && coef, "bn_apply_bwd: null tensor");
+  Geometry geo = geometry(rows, C, dtype);
+  const double tensor_bytes = static_cast<double>(rows) * C * (dtype == kBF16 ? 2.0 : 4.0);
+  ApplyArgs a{g, nullptr, x, dx, coef, coef + C, coef + 2 * C, rows * geo.cc, FastDiv(geo.cc), 0};
+  return dtype == kBF16 ? launch(ctx, bn_apply_kernel<bf16, 1>, dim3(apply_blocks(a.chunks)), dim3(256), a,
+                                 "bn_apply_kernel<bf16,bwd>", tensor_bytes * 3.0, 1)
+                        : launch(ctx, bn_apply_kernel<float, 1>, dim3(apply_blocks(a.chunks)), dim3(256), a,
+                                 "bn_apply_kernel<f32,bwd>", tensor_bytes * 3.0, 1);
+}
+
 int bn_fwd_train_partials(Context* ctx, int dtype, const void* x, void* y, const void* residual, int relu,
                           int64_t rows, int C, const float* gamma, const float* beta, float* running_mean,
                           float* running_var, float* save_mean, float* save_invstd, float momentum, float eps,

@@ -191,7 +191,7 @@ int tch_conv2d_dgrad_bnsums(tch_context* ctx, int dtype, const void* dy, const v
                             const void* mask, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad,
                             int tile_cfg, int c_logical, const void* bn_mask, const void* bn_x, const float* bn_mean,
                             const float* bn_invstd, float* bn_partial) {
-  BnBwdSums bn{bn_mask, bn_x, bn_mean, bn_invstd, bn_partial};
+  BnBwdSums bn{bn_mask, bn_x, bn_mean, bn_invstd, bn_partial, nullptr};
   return conv2d_dgrad(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad, c_logical), dy, w, dx, add, mask, tile_cfg,
                       &bn);
 }
@@ -264,6 +264,36 @@ int tch_batched_gemm(tch_context* ctx, int dtype, const void* a, const void* b, 
                      float alpha, int accumulate, int causal) {
   return batched_gemm(C(ctx), dtype, a, b, c, M, N, K, a_rs, a_cs, b_rs, b_cs, ldc, batch_outer, batch_inner, a_bo, a_bi,
                       b_bo, b_bi, c_bo, c_bi, alpha, accumulate, causal);
+}
+
+int tch_conv2d_fwd_bn(tch_context* ctx, int dtype, const void* x, const void* w, void* y, int N, int H, int W, int Cc,
+                      int K, int R, int S, int stride, int pad, int tile_cfg, int c_logical, float* bn_partial,
+                      int* counters, const float* gamma, const float* beta, float* running_mean, float* running_var,
+                      float* save_mean, float* save_invstd, float momentum, float eps, float* coef) {
+  BnFinalize fin{counters, gamma, beta, running_mean, running_var, save_mean, save_invstd, coef, momentum, eps, 0};
+  return conv2d_fwd(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad, c_logical), x, w, y, nullptr, nullptr, nullptr,
+                    0, tile_cfg, bn_partial, &fin);
+}
+
+int tch_conv2d_dgrad_bn(tch_context* ctx, int dtype, const void* dy, const void* w, void* dx, const void* add,
+                        const void* mask, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad,
+                        int tile_cfg, int c_logical, const void* bn_mask, const void* bn_x, const float* bn_mean,
+                        const float* bn_invstd, float* bn_partial, int* counters, const float* gamma, float* dgamma,
+                        float* dbeta, int accumulate, float* coef) {
+  BnFinalize fin{counters, gamma, nullptr, nullptr, nullptr, dgamma, dbeta, coef, 0.f, 0.f, accumulate};
+  BnBwdSums bn{bn_mask, bn_x, bn_mean, bn_invstd, bn_partial, &fin};
+  return conv2d_dgrad(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad, c_logical), dy, w, dx, add, mask, tile_cfg,
+                      &bn);
+}
+
+int tch_bn_apply_fwd(tch_context* ctx, int dtype, const void* x, void* y, const void* residual, int relu, int64_t rows,
+                     int Cc, const float* coef) {
+  return bn_apply_fwd(C(ctx), dtype, x, y, residual, relu, rows, Cc, coef);
+}
+
+int tch_bn_apply_bwd(tch_context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int Cc,
+                     const float* coef) {
+  return bn_apply_bwd(C(ctx), dtype, g, x, dx, rows, Cc, coef);
 }
 
 int tch_conv2d_wgrad_pick_splits(int dtype, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad) {

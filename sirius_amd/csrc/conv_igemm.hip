@@ -56,6 +56,19 @@ struct IgemmArgs {
   const void* bn_x;         // DGRAD with stats: input of the BatchNorm this gradient flows into, laid out like out
   const float* bn_mean;     // DGRAD with stats: that BatchNorm's saved batch mean / inverse std per column
   const float* bn_invstd;
+  // Optional, with stats: the workgroup that finishes a column tile last also turns the sums into the
+  // BatchNorm's per-channel coefficients (no finalize launch).  fin_counters: one int per column tile,
+  // zero before the launch; the finishing workgroup leaves it zero again.
+  int* fin_counters;
+  const float* fin_gamma;
+  const float* fin_beta;     // FWD
+  float* fin_running_mean;   // FWD, may be null (then fin_running_var is null too)
+  float* fin_running_var;
+  float* fin_out0;           // FWD: saved batch mean         DGRAD: dgamma
+  float* fin_out1;           // FWD: saved inverse std        DGRAD: dbeta
+  float* fin_coef;           // FWD: scale[C], shift[C]       DGRAD: coef[3][C] (dx = c0*g + c1*x + c2)
+  float fin_momentum, fin_eps;
+  int fin_accumulate;        // DGRAD: dgamma / dbeta +=
   int N, H, W, C;     // x side
   int Ho, Wo, K;      // y side
   int R, S, stride, stride_log2, pad;
@@ -135,6 +148,97 @@ struct TapWalker {
     }
   }
 };
+
+// Called by every workgroup after it has stored its row of partial sums: the one that arrives last at
+// the column tile's counter sums all tiles_m rows of its BN columns (fp64, fixed order) and writes
+// the BatchNorm coefficients.  Nobody waits for anybody: a workgroup that is not last just leaves.
+// Visibility across the chip's L2 slices without flushing them (a device-scope fence per workgroup
+// writes back every dirty line of its L2 slice, the convolution's own output included, and costs
+// more than the whole kernel): the partial sums are published with device-scope atomic exchanges,
+// whose result the publishing thread waits for before the barrier that precedes the counter bump,
+// and the finishing workgroup reads them with device-scope atomic loads.  Atomics execute at the
+// point all slices share.
+template <int MODE, int BN, int NT>
+__device__ inline void finalize_column_tile(const IgemmArgs& p, float* stage, int tid, int n0) {
+  __shared__ int last_arrival;
+  __syncthreads();
+  if (tid == 0) {
+    int* counter = p.fin_counters + n0 / BN;
+    const int prev = atomicAdd(counter, 1);
+    last_arrival = prev == p.tiles_m - 1;
+    if (last_arrival) *counter = 0;  // every other workgroup of this column tile has been here already
+  }
+  __syncthreads();
+  if (!last_arrival) return;
+
+  constexpr int PARTS = NT / BN;   // row tiles are dealt round-robin to PARTS threads per column
+  const int cl = tid % BN, part = tid / BN;
+  double s_part = 0.0, q_part = 0.0;
+  if (n0 + cl < p.gemm_n) {
+    constexpr int U = 8;
+    for (int b = part; b < p.tiles_m; b += U * PARTS) {
+      unsigned long long v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int bb = b + u * PARTS;
+        v[u] = bb < p.tiles_m
+                   ? __hip_atomic_load(reinterpret_cast<const unsigned long long*>(
+                                           p.stats + (static_cast<int64_t>(bb) * p.gemm_n + n0 + cl) * 2),
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                   : 0ull;
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        s_part += __uint_as_float(static_cast<uint32_t>(v[u]));
+        q_part += __uint_as_float(static_cast<uint32_t>(v[u] >> 32));
+      }
+    }
+  }
+  double* red = reinterpret_cast<double*>(stage);  // [PARTS][BN][2]
+  red[(part * BN + cl) * 2] = s_part;
+  red[(part * BN + cl) * 2 + 1] = q_part;
+  __syncthreads();
+  const int c = n0 + tid;
+  if (tid >= BN || c >= p.gemm_n) return;
+  double s = 0.0, q = 0.0;
+#pragma unroll
+  for (int k = 0; k < PARTS; ++k) {
+    s += red[(k * BN + tid) * 2];
+    q += red[(k * BN + tid) * 2 + 1];
+  }
+  const double n = static_cast<double>(p.gemm_m);
+  const int C = p.gemm_n;
+  if (MODE == kFwd) {
+    // s = sum x, q = sum x^2  (torch.nn.BatchNorm2d in training mode: biased variance normalises,
+    // the unbiased one goes into running_var)
+    const double mean = s / n;
+    double var = q / n - mean * mean;
+    if (var < 0.0) var = 0.0;
+    const float invstd = 1.0f / sqrtf(static_cast<float>(var) + p.fin_eps);
+    p.fin_out0[c] = static_cast<float>(mean);
+    p.fin_out1[c] = invstd;
+    if (p.fin_running_mean) {
+      const double unbiased = p.gemm_m > 1 ? var * n / (n - 1.0) : var;
+      p.fin_running_mean[c] = (1.f - p.fin_momentum) * p.fin_running_mean[c] + p.fin_momentum * static_cast<float>(mean);
+      p.fin_running_var[c] = (1.f - p.fin_momentum) * p.fin_running_var[c] + p.fin_momentum * static_cast<float>(unbiased);
+    }
+    const float sc = p.fin_gamma[c] * invstd;
+    p.fin_coef[c] = sc;
+    p.fin_coef[C + c] = p.fin_beta[c] - static_cast<float>(mean) * sc;
+  } else {
+    // s = sum g, q = sum g * xhat
+    const float db = static_cast<float>(s), dg = static_cast<float>(q);
+    p.fin_out1[c] = p.fin_accumulate ? p.fin_out1[c] + db : db;
+    p.fin_out0[c] = p.fin_accumulate ? p.fin_out0[c] + dg : dg;
+    const double invstd = p.bn_invstd[c];
+    const double scale = static_cast<double>(p.fin_gamma[c]) * invstd;
+    const double cb = -scale * invstd * (q / n);
+    const double c0 = -scale * (s / n) - cb * p.bn_mean[c];
+    p.fin_coef[c] = static_cast<float>(scale);
+    p.fin_coef[C + c] = static_cast<float>(cb);
+    p.fin_coef[2 * C + c] = static_cast<float>(c0);
+  }
+}
 
 // The accumulators of one workgroup tile, one 32-row band (index tm) at a time:
 // lanes write float4 groups into the staging tile [WM*32][BN + pad], then every
@@ -327,9 +431,18 @@ __device__ inline void finish_tile(const IgemmArgs& p, f32x16_t (&acc)[TM][TN], 
       const int col = n0 + tid;
       if (col < p.gemm_n) {
         float2* dst = reinterpret_cast<float2*>(p.stats + (static_cast<int64_t>(tile_m) * p.gemm_n + col) * 2);
-        *dst = make_float2(a, b);
+        if (p.fin_counters) {
+          // published for the workgroup that finishes this column tile (see finalize_column_tile)
+          const unsigned long long bits = static_cast<unsigned long long>(__float_as_uint(a)) |
+                                          (static_cast<unsigned long long>(__float_as_uint(b)) << 32);
+          const unsigned long long old = atomicExch(reinterpret_cast<unsigned long long*>(dst), bits);
+          asm volatile("" ::"v"(old));  // wait for the exchange itself, not only for its issue
+        } else {
+          *dst = make_float2(a, b);
+        }
       }
     }
+    if (p.fin_counters) finalize_column_tile<MODE, BN, NT>(p, stage, tid, n0);
   }
 }
 
@@ -1106,12 +1219,37 @@ void conv_output_hw(const ConvShape& s, int* Ho, int* Wo) {
   *Wo = (s.W + 2 * s.pad - s.S) / s.stride + 1;
 }
 
+namespace {
+
+bool check_finalize(const BnFinalize* f, bool forward) {
+  return f->counters && f->gamma && f->out0 && f->out1 && f->coef && (!forward || f->beta) &&
+         ((f->running_mean == nullptr) == (f->running_var == nullptr));
+}
+
+void bind_finalize(IgemmArgs& a, const BnFinalize* f) {
+  a.fin_counters = f->counters;
+  a.fin_gamma = f->gamma;
+  a.fin_beta = f->beta;
+  a.fin_running_mean = f->running_mean;
+  a.fin_running_var = f->running_var;
+  a.fin_out0 = f->out0;
+  a.fin_out1 = f->out1;
+  a.fin_coef = f->coef;
+  a.fin_momentum = f->momentum;
+  a.fin_eps = f->eps;
+  a.fin_accumulate = f->accumulate;
+}
+
+}  // namespace
+
 int conv2d_fwd(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* w, void* y, const void* add,
-               const void* mask, const float* bias, int out_f32, int tile_cfg, float* bn_partial) {
+               const void* mask, const float* bias, int out_f32, int tile_cfg, float* bn_partial,
+               const BnFinalize* finalize) {
   IgemmArgs a{};
   if (int rc = fill_common(a, s, dtype)) return rc;
   TCH_CHECK_ARG(x && w && y, "conv2d_fwd: null tensor");
   TCH_CHECK_ARG(!(bn_partial && out_f32), "conv2d_fwd: statistics are taken of outputs stored in the compute type");
+  TCH_CHECK_ARG(!finalize || (bn_partial && check_finalize(finalize, true)), "conv2d_fwd: incomplete BatchNorm finalize operands");
   a.stats = bn_partial;
   const int eb = dtype == kBF16 ? 2 : 4;
   a.a_src = x;
@@ -1130,8 +1268,15 @@ int conv2d_fwd(Context* ctx, int dtype, const ConvShape& s, const void* x, const
   a.div_plane = FastDiv(a.Ho * a.Wo);
   a.div_width = FastDiv(a.Wo);
   if (tile_cfg < 0) tile_cfg = pick_tile(a.gemm_m, a.gemm_n, 1);
-  return dtype == kBF16 ? launch_mode<bf16, kFwd>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo))
-                        : launch_mode<float, kFwd>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo));
+  const int row_tiles = (a.gemm_m + (tile_cfg >= 2 ? 64 : 128) - 1) / (tile_cfg >= 2 ? 64 : 128);
+  const bool in_kernel = finalize && row_tiles <= kBnFinalizeInKernelTiles;
+  if (in_kernel) bind_finalize(a, finalize);
+  int rc = dtype == kBF16 ? launch_mode<bf16, kFwd>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo))
+                          : launch_mode<float, kFwd>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo));
+  if (rc || !finalize || in_kernel) return rc;
+  return bn_fwd_finalize(ctx, bn_partial, row_tiles, s.K, a.gemm_m, finalize->gamma, finalize->beta,
+                         finalize->running_mean, finalize->running_var, finalize->out0, finalize->out1, finalize->coef,
+                         finalize->momentum, finalize->eps);
 }
 
 int conv2d_fwd_stat_rows(const ConvShape& s, int dtype, int tile_cfg) {
@@ -1159,6 +1304,7 @@ int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, co
   TCH_CHECK_ARG(dy && wt && dx, "conv2d_dgrad: null tensor");
   if (bn) {
     TCH_CHECK_ARG(bn->x && bn->mean && bn->invstd && bn->partial, "conv2d_dgrad: incomplete BatchNorm operands");
+    TCH_CHECK_ARG(!bn->finalize || check_finalize(bn->finalize, false), "conv2d_dgrad: incomplete BatchNorm finalize operands");
     a.stats = bn->partial;
     a.bn_mask = bn->mask;
     a.bn_x = bn->x;
@@ -1181,8 +1327,15 @@ int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, co
   a.div_plane = FastDiv(s.H * s.W);
   a.div_width = FastDiv(s.W);
   if (tile_cfg < 0) tile_cfg = pick_tile(a.gemm_m, a.gemm_n, 1);
-  return dtype == kBF16 ? launch_mode<bf16, kDgrad>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo))
-                        : launch_mode<float, kDgrad>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo));
+  const BnFinalize* finalize = bn ? bn->finalize : nullptr;
+  const int row_tiles = (a.gemm_m + (tile_cfg >= 2 ? 64 : 128) - 1) / (tile_cfg >= 2 ? 64 : 128);
+  const bool in_kernel = finalize && row_tiles <= kBnFinalizeInKernelTiles;
+  if (in_kernel) bind_finalize(a, finalize);
+  int rc = dtype == kBF16 ? launch_mode<bf16, kDgrad>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo))
+                          : launch_mode<float, kDgrad>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo));
+  if (rc || !finalize || in_kernel) return rc;
+  return bn_bwd_finalize(ctx, bn->partial, row_tiles, s.C, a.gemm_m, finalize->gamma, bn->mean, bn->invstd,
+                         finalize->out0, finalize->out1, finalize->coef, finalize->accumulate);
 }
 
 int64_t conv2d_wgrad_workspace_bytes(const ConvShape& s, int dtype, int splits) {

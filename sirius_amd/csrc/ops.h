@@ -20,9 +20,27 @@ struct ConvShape {
 
 void conv_output_hw(const ConvShape& s, int* Ho, int* Wo);
 
+// Turns the sums a convolution epilogue leaves into the BatchNorm's per-channel coefficients as part of the
+// convolution call: inside the kernel (the workgroup that finishes a column tile last does it) when there
+// are at most kBnFinalizeInKernelTiles row tiles, by a finalize launch otherwise.
+constexpr int kBnFinalizeInKernelTiles = 256;
+struct BnFinalize {
+  int* counters;        // >= ceil(C / 64) ints, zero before the call; left zero
+  const float* gamma;
+  const float* beta;    // forward
+  float* running_mean;  // forward, may be null together with running_var
+  float* running_var;
+  float* out0;          // forward: saved batch mean      backward: dgamma
+  float* out1;          // forward: saved inverse std     backward: dbeta
+  float* coef;          // forward: scale[C], shift[C]    backward: coef[3][C]
+  float momentum, eps;  // forward
+  int accumulate;       // backward: dgamma / dbeta +=
+};
+
 // conv_igemm.hip
 int conv2d_fwd(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* w, void* y, const void* add,
-               const void* mask, const float* bias, int out_f32, int tile_cfg, float* bn_partial = nullptr);
+               const void* mask, const float* bias, int out_f32, int tile_cfg, float* bn_partial = nullptr,
+               const BnFinalize* finalize = nullptr);
 // rows of partial statistics conv2d_fwd writes for this shape and tiling (one per row tile)
 int conv2d_fwd_stat_rows(const ConvShape& s, int dtype, int tile_cfg);
 // The two reductions of a BatchNorm backward, taken in the epilogue of the data-gradient
@@ -33,6 +51,7 @@ struct BnBwdSums {
   const float* mean;    // saved batch statistics, one per channel of dx
   const float* invstd;
   float* partial;       // [conv2d_dgrad_stat_rows][C][2]
+  const BnFinalize* finalize;  // optional
 };
 int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, const void* w, void* dx,
                  const void* add, const void* mask, int tile_cfg, const BnBwdSums* bn = nullptr);
@@ -57,6 +76,17 @@ int bn_fwd_train_partials(Context* ctx, int dtype, const void* x, void* y, const
 int bn_bwd(Context* ctx, int dtype, const void* dy, const void* relu_mask, const void* x, void* dx, int64_t rows,
            int C, const float* gamma, const float* save_mean, const float* save_invstd, float* dgamma, float* dbeta,
            int accumulate, float* workspace);
+// pieces of the above for callers whose sums come from a convolution epilogue
+int bn_fwd_finalize(Context* ctx, const float* partial, int row_blocks, int C, int64_t rows, const float* gamma,
+                    const float* beta, float* running_mean, float* running_var, float* save_mean, float* save_invstd,
+                    float* coef, float momentum, float eps);
+int bn_bwd_finalize(Context* ctx, const float* partial, int row_blocks, int C, int64_t rows, const float* gamma,
+                    const float* save_mean, const float* save_invstd, float* dgamma, float* dbeta, float* coef,
+                    int accumulate);
+int bn_apply_fwd(Context* ctx, int dtype, const void* x, void* y, const void* residual, int relu, int64_t rows, int C,
+                 const float* coef);
+int bn_apply_bwd(Context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int C,
+                 const float* coef);
 // the same from the sums a convolution epilogue left ([row_blocks][C][2]); g is already gated by the
 // ReLU; scratch: 3*C floats
 int bn_bwd_partials(Context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int C,

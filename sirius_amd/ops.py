@@ -220,6 +220,61 @@ def conv2d_dgrad_bnsums(ctx, dy, wt, dx, stride, pad, bn_x, bn_mean, bn_invstd, 
     return rb
 
 
+def conv2d_fwd_bn(ctx, x, w, y, stride, pad, partial, counters, gamma, beta, running_mean, running_var, save_mean,
+                  save_invstd, coef, momentum=0.1, eps=1e-5, tile_cfg=-1, c_logical=0):
+    """conv2d_fwd + batch statistics + the BatchNorm's scale / shift (coef [2, K]); finish with bn_apply_fwd."""
+    N, H, W, C = x.shape
+    K, R, S, C2 = w.shape
+    assert C == C2 and w.dtype == x.dtype == y.dtype
+    Ho, Wo = conv_out_hw(H, W, R, S, stride, pad)
+    assert tuple(y.shape) == (N, Ho, Wo, K)
+    rb = conv2d_fwd_stat_rows(x, K, R, S, stride, pad, tile_cfg)
+    assert partial.dtype == torch.float32 and partial.numel() >= rb * K * 2
+    assert counters.dtype == torch.int32 and counters.numel() >= (K + 63) // 64 and coef.numel() >= 2 * K
+    for t in (gamma, beta, save_mean, save_invstd):
+        assert t.dtype == torch.float32 and t.numel() == K
+    check(lib().tch_conv2d_fwd_bn(ctx.handle, dtype_code(x), _p(x), _p(w), _p(y), N, H, W, C, K, R, S, stride, pad,
+                                  tile_cfg, c_logical, _p(partial), _p(counters), _p(gamma), _p(beta), _p(running_mean),
+                                  _p(running_var), _p(save_mean), _p(save_invstd), momentum, eps, _p(coef)),
+          "tch_conv2d_fwd_bn")
+
+
+def conv2d_dgrad_bn(ctx, dy, wt, dx, stride, pad, bn_x, bn_mean, bn_invstd, partial, counters, gamma, dgamma, dbeta, coef,
+                    bn_mask=None, add=None, mask=None, accumulate=False, tile_cfg=-1, c_logical=0):
+    """conv2d_dgrad_bnsums + dgamma / dbeta + the coefficients of the BatchNorm input gradient (coef [3, C]);
+    finish with bn_apply_bwd."""
+    N, H, W, C = dx.shape
+    C2, R, S, K = wt.shape
+    assert C == C2
+    Ho, Wo = conv_out_hw(H, W, R, S, stride, pad)
+    assert tuple(dy.shape) == (N, Ho, Wo, K) and dy.dtype == wt.dtype == dx.dtype
+    for t in (add, mask, bn_mask, bn_x):
+        assert t is None or (t.shape == dx.shape and t.dtype == dx.dtype)
+    assert bn_x is not None and bn_mean.numel() == C and bn_invstd.numel() == C
+    rb = conv2d_dgrad_stat_rows(dx, K, R, S, stride, pad, tile_cfg)
+    assert partial.dtype == torch.float32 and partial.numel() >= rb * C * 2
+    assert counters.dtype == torch.int32 and counters.numel() >= (C + 63) // 64 and coef.numel() >= 3 * C
+    check(lib().tch_conv2d_dgrad_bn(ctx.handle, dtype_code(dy), _p(dy), _p(wt), _p(dx), _p(add), _p(mask),
+                                    N, H, W, C, K, R, S, stride, pad, tile_cfg, c_logical, _p(bn_mask), _p(bn_x),
+                                    _p(bn_mean), _p(bn_invstd), _p(partial), _p(counters), _p(gamma), _p(dgamma),
+                                    _p(dbeta), int(accumulate), _p(coef)), "tch_conv2d_dgrad_bn")
+
+
+def bn_apply_fwd(ctx, x, y, coef, residual=None, relu=True):
+    C = x.shape[-1]
+    assert y.shape == x.shape and y.dtype == x.dtype and coef.numel() >= 2 * C
+    assert residual is None or (residual.shape == x.shape and residual.dtype == x.dtype)
+    check(lib().tch_bn_apply_fwd(ctx.handle, dtype_code(x), _p(x), _p(y), _p(residual), int(relu), x.numel() // C, C,
+                                 _p(coef)), "tch_bn_apply_fwd")
+
+
+def bn_apply_bwd(ctx, g, x, dx, coef):
+    C = x.shape[-1]
+    assert g.shape == x.shape == dx.shape and g.dtype == x.dtype == dx.dtype and coef.numel() >= 3 * C
+    check(lib().tch_bn_apply_bwd(ctx.handle, dtype_code(x), _p(g), _p(x), _p(dx), x.numel() // C, C, _p(coef)),
+          "tch_bn_apply_bwd")
+
+
 def conv2d_wgrad_splits(x, K, R, S, stride, pad):
     N, H, W, C = x.shape
     return int(lib().tch_conv2d_wgrad_pick_splits(dtype_code(x), N, H, W, C, K, R, S, stride, pad))

@@ -49,7 +49,7 @@ class _Block:
 class ResNetEngine(EngineBase):
     def __init__(self, depths=(3, 8, 36, 3), num_classes=1000, width=64, dtype=torch.bfloat16, image_size=224,
                  lr=0.1, momentum=0.9, weight_decay=1e-4, bn_momentum=0.1, bn_eps=1e-5, stream=None, allocator=None,
-                 overlap_wgrad=True, fuse_bn_stats=True, fuse_bn_bwd=True, autotune=False):
+                 overlap_wgrad=True, fuse_bn_stats=True, fuse_bn_bwd=True, fuse_bn_finalize=False, autotune=False):
         self._init_engine(dtype, stream, allocator)
         assert num_classes % 8 == 0, "class count must be a multiple of one 16-byte chunk"
         self.image_size, self.num_classes = image_size, num_classes
@@ -64,6 +64,12 @@ class ResNetEngine(EngineBase):
         # fuse_bn_bwd: a data-gradient convolution whose output flows into a BatchNorm(+ReLU) backward applies
         # the ReLU gate and takes that BatchNorm's two reductions in its epilogue (no reduction pass)
         self.fuse_bn_bwd = fuse_bn_bwd
+        # fuse_bn_finalize: the convolution that leaves the sums also turns them into the BatchNorm's
+        # coefficients (its last workgroup per column tile), so that only the apply launch follows.
+        # Off by default: measured on MI355X at batch 64, the tail it adds to every convolution (two
+        # round trips of device-scope atomics, then a few batches of uncached loads in one workgroup)
+        # costs as much as the finalize launch it saves (20.2 ms per step against 19.3 ms)
+        self.fuse_bn_finalize = fuse_bn_finalize
         # autotune: when a plan is built, time each distinct convolution shape with every tiling and
         # keep the fastest (forward and data gradient separately); off = the library's heuristic
         self.autotune = autotune
@@ -408,14 +414,22 @@ class ResNetEngine(EngineBase):
             tiles[c_.name] = self._tune_conv(c_, n_, h_, w_) if self.autotune else (-1, -1)
         stat_partial = act(max(stat_elems[0], 2), dtype=torch.float32)
         bn_scratch = act(3 * max(max(c_.cout, c_.cin_store) for c_, _ in conv_inputs), dtype=torch.float32)
+        bn_counters = act(max(max(c_.cout, c_.cin_store) for c_, _ in conv_inputs) // 64 + 1, dtype=torch.int32).zero_()
 
         def conv_bn_fwd(c, name, x, z, y, residual=None, relu=True):
             if not self.fuse_bn_stats:
                 conv_fwd(c, x, z)
                 return bn_fwd(name, z, y, residual=residual, relu=relu)
+            o, ch = self._bn_off[name]
+            if self.fuse_bn_finalize:
+                ops.conv2d_fwd_bn(ctx, x, self._w(c.name + ".weight"), z, c.stride, c.pad, stat_partial, bn_counters,
+                                  self._view(self.params, name + ".weight"), self._view(self.params, name + ".bias"),
+                                  self.running_mean[o:o + ch], self.running_var[o:o + ch], bn_save[o:o + ch],
+                                  bn_save[nbn + o:nbn + o + ch], bn_scratch, momentum=self.bn_momentum, eps=self.bn_eps,
+                                  tile_cfg=tiles[c.name][0], c_logical=c.cin)
+                return ops.bn_apply_fwd(ctx, z, y, bn_scratch, residual=residual, relu=relu)
             rb = ops.conv2d_fwd_bnstats(ctx, x, self._w(c.name + ".weight"), z, c.stride, c.pad, stat_partial,
                                         tile_cfg=tiles[c.name][0], c_logical=c.cin)
-            o, ch = self._bn_off[name]
             ops.bn_fwd_train_partials(ctx, z, y, self._view(self.params, name + ".weight"),
                                       self._view(self.params, name + ".bias"), self.running_mean[o:o + ch],
                                       self.running_var[o:o + ch], bn_save[o:o + ch], bn_save[nbn + o:nbn + o + ch],
@@ -440,12 +454,21 @@ class ResNetEngine(EngineBase):
         # is that BatchNorm's backward from there (finalize + apply)
         def conv_dgrad_bn(c, dy, dx, name, z, relu_out, **kw):
             o, ch = self._bn_off[name]
+            if self.fuse_bn_finalize:
+                ops.conv2d_dgrad_bn(ctx, dy, self._wt(c.name + ".weight"), dx, c.stride, c.pad, z, bn_save[o:o + ch],
+                                    bn_save[nbn + o:nbn + o + ch], stat_partial, bn_counters,
+                                    self._view(self.params, name + ".weight"), self._view(self.grads, name + ".weight"),
+                                    self._view(self.grads, name + ".bias"), bn_scratch, bn_mask=relu_out,
+                                    c_logical=c.cin, tile_cfg=tiles.get(c.name, (-1, -1))[1], **kw)
+                return -1   # the coefficients are in bn_scratch already
             return ops.conv2d_dgrad_bnsums(ctx, dy, self._wt(c.name + ".weight"), dx, c.stride, c.pad, z,
                                            bn_save[o:o + ch], bn_save[nbn + o:nbn + o + ch], stat_partial,
                                            bn_mask=relu_out, c_logical=c.cin,
                                            tile_cfg=tiles.get(c.name, (-1, -1))[1], **kw)
 
         def bn_bwd_sums(name, g, x, dx, rb):
+            if rb == -1:
+                return ops.bn_apply_bwd(ctx, g, x, dx, bn_scratch)
             o, c = self._bn_off[name]
             ops.bn_bwd_partials(ctx, g, x, dx, self._view(self.params, name + ".weight"), bn_save[o:o + c],
                                 bn_save[nbn + o:nbn + o + c], self._view(self.grads, name + ".weight"),
@@ -590,6 +613,7 @@ class ResNetEngine(EngineBase):
         plan.marks = marks
         plan.keep = keep
         plan.logits = logits
+        plan.bn_save = bn_save   # [2][sum of BatchNorm widths]: saved batch mean, then inverse std
         plan.bytes = sum(t.numel() * t.element_size() for t in keep)
         return plan
 

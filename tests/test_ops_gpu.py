@@ -216,6 +216,55 @@ def test_conv_with_bn_statistics(ctx, dtype, case, tile_cfg):
     close(sm, mean_ref, torch.float32, "bn mean", rtol=tol)
     close(si, invstd_ref, torch.float32, "bn invstd", rtol=tol)
     close(y, y_ref, dtype, "bn y", rtol=tol)
+    # the same with the coefficients computed as part of the convolution call; twice, on the same counters
+    counters = torch.zeros(K // 64 + 1, dtype=torch.int32, device="cuda")
+    for _ in range(2):
+        rm2, rv2 = torch.zeros(K, device="cuda"), torch.ones(K, device="cuda")
+        sm2, si2 = torch.empty(K, device="cuda"), torch.empty(K, device="cuda")
+        coef = torch.full((2 * K,), float("nan"), device="cuda")
+        z2, y2 = torch.empty_like(z), torch.empty_like(z)
+        partial.fill_(float("nan"))
+        ops.conv2d_fwd_bn(ctx, xd, wd, z2, st, pad, partial, counters, gamma.cuda(), beta.cuda(), rm2, rv2, sm2, si2, coef,
+                          tile_cfg=tile_cfg)
+        ops.bn_apply_fwd(ctx, z2, y2, coef, relu=True)
+        torch.cuda.synchronize()
+        assert torch.equal(z2, z) and torch.all(counters == 0)
+        close(sm2, sm.cpu(), torch.float32, "fused finalize: mean", rtol=1e-6)
+        close(si2, si.cpu(), torch.float32, "fused finalize: invstd", rtol=1e-6)
+        close(rm2, rm.cpu(), torch.float32, "fused finalize: running mean", rtol=1e-6)
+        close(rv2, rv.cpu(), torch.float32, "fused finalize: running var", rtol=1e-6)
+        close(y2, y.float().cpu(), dtype, "fused finalize: y", rtol=1e-6 if dtype == torch.float32 else 8e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_conv_bn_finalize_with_many_row_tiles(ctx, dtype):
+    """More row tiles than one workgroup should sum (> 256): the convolution call finishes the coefficients
+    with a launch of its own; same results, same interface."""
+    from sirius_amd import ops
+    N, H, W, C, K = 2, 96, 96, 64, 64     # 18432 output rows: 288 tiles of 64 rows
+    g = _gen(23)
+    x = rnd((N, H, W, C), dtype, g)
+    w = rnd((K, 1, 1, C), dtype, g, C ** -0.5)
+    gamma, beta = torch.rand(K, generator=g) + 0.5, torch.randn(K, generator=g) * 0.1
+    z_ref = O.conv2d_fwd(x, w, 1, 0).to(dtype)
+    rm_ref, rv_ref = torch.zeros(K), torch.ones(K)
+    y_ref, mean_ref, invstd_ref = O.bn_fwd_train(z_ref, gamma, beta, rm_ref, rv_ref, relu=True)
+    xd, wd = x.cuda(), w.cuda()
+    assert ops.conv2d_fwd_stat_rows(xd, K, 1, 1, 1, 0, 2) > 256
+    partial = torch.empty(ops.conv2d_fwd_stat_rows(xd, K, 1, 1, 1, 0, 2) * K * 2, device="cuda")
+    counters = torch.zeros(2, dtype=torch.int32, device="cuda")
+    z, y = (torch.empty(z_ref.shape, dtype=dtype, device="cuda") for _ in range(2))
+    rm, rv = torch.zeros(K, device="cuda"), torch.ones(K, device="cuda")
+    sm, si, coef = torch.empty(K, device="cuda"), torch.empty(K, device="cuda"), torch.empty(2 * K, device="cuda")
+    ops.conv2d_fwd_bn(ctx, xd, wd, z, 1, 0, partial, counters, gamma.cuda(), beta.cuda(), rm, rv, sm, si, coef, tile_cfg=2)
+    ops.bn_apply_fwd(ctx, z, y, coef, relu=True)
+    torch.cuda.synchronize()
+    tol = 1e-3 if dtype == torch.float32 else 2e-2
+    close(sm, mean_ref, torch.float32, "bn mean", rtol=tol)
+    close(si, invstd_ref, torch.float32, "bn invstd", rtol=tol)
+    close(rv, rv_ref, torch.float32, "running var", rtol=tol)
+    close(y, y_ref, dtype, "bn y", rtol=tol)
+    assert torch.all(counters == 0)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -296,6 +345,22 @@ def test_conv_dgrad_with_bn_backward_sums(ctx, dtype, case, tile_cfg, with_add):
     close(dg, dg_ref, torch.float32, "bn dgamma", rtol=tol)
     close(db, db_ref, torch.float32, "bn dbeta", rtol=tol)
     close(dz, dz_ref, dtype, "bn dx", rtol=tol)
+    # the same with the coefficients computed as part of the convolution call; twice, on the same counters
+    counters = torch.zeros(C // 64 + 1, dtype=torch.int32, device="cuda")
+    for _ in range(2):
+        gx2, dz2 = torch.empty_like(gx), torch.empty_like(gx)
+        dg2, db2 = torch.zeros(C, device="cuda"), torch.zeros(C, device="cuda")
+        coef = torch.full((3 * C,), float("nan"), device="cuda")
+        partial.fill_(float("nan"))
+        ops.conv2d_dgrad_bn(ctx, dy.cuda(), ops.filter_transpose(ctx, w.cuda()), gx2, st, pad, zd, mean.cuda(),
+                            invstd.cuda(), partial, counters, gamma.cuda(), dg2, db2, coef, bn_mask=relu_out.cuda(),
+                            add=d(add), tile_cfg=tile_cfg)
+        ops.bn_apply_bwd(ctx, gx2, zd, dz2, coef)
+        torch.cuda.synchronize()
+        assert torch.equal(gx2, gx) and torch.all(counters == 0)
+        close(dg2, dg.cpu(), torch.float32, "fused finalize: dgamma", rtol=1e-6)
+        close(db2, db.cpu(), torch.float32, "fused finalize: dbeta", rtol=1e-6)
+        close(dz2, dz.float().cpu(), dtype, "fused finalize: dx", rtol=1e-5 if dtype == torch.float32 else 8e-3)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
