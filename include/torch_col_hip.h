@@ -219,7 +219,7 @@ int tch_bias_grad_ws(tch_context* ctx, int dtype, const void* dy, float* dbias, 
  * The arithmetic restates torch.nn.LayerNorm / GELU / softmax / AdamW / Embedding as the reference's
  * training scripts use them through torchvision and transformers (train/swin_b.py:38-45,
  * train/gpt2.py:26-33; a readable statement of window attention: train/swin_b_tiny.py:8-172). */
-/* y = (x - mean) * rstd * gamma + beta over the last dimension of [rows, C] (C <= 1024); mean / rstd [rows]
+/* y = (x - mean) * rstd * gamma + beta over the last dimension of [rows, C] (C <= 2048); mean / rstd [rows]
  * are kept for the backward. */
 int tch_layernorm_fwd(tch_context* ctx, int dtype, const void* x, void* y, const float* gamma, const float* beta,
                       float* mean, float* rstd, int64_t rows, int C, float eps);
@@ -262,6 +262,28 @@ int tch_batched_gemm(tch_context* ctx, int dtype, const void* a, const void* b, 
                      int64_t a_rs, int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t ldc, int batch_outer,
                      int batch_inner, int64_t a_bo, int64_t a_bi, int64_t b_bo, int64_t b_bi, int64_t c_bo, int64_t c_bi,
                      float alpha, int accumulate, int causal);
+
+/* Swin-B data movement (train/swin_b_tiny.py:8-19,116-131; patch merging and shift as in torchvision's swin_b,
+ * train/swin_b.py:38).
+ * reverse == 0: dst[windows of window x window tokens] = roll(src[B,H,W,C], -shift) partitioned;
+ * reverse != 0: dst[B,H,W,C] = roll(un-partitioned src, +shift) (+ add, laid out like dst).  Each direction is
+ * also the gradient of the other. */
+int tch_window_partition(tch_context* ctx, int dtype, const void* src, void* dst, const void* add, int B, int H, int W,
+                         int C, int window, int shift, int reverse);
+/* reverse == 0: dst[B,H/2,W/2,4C] = concat(src[0::2,0::2], src[1::2,0::2], src[0::2,1::2], src[1::2,1::2]);
+ * reverse != 0: the inverse permutation (its gradient). */
+int tch_patch_merge_gather(tch_context* ctx, int dtype, const void* src, void* dst, int B, int H, int W, int C,
+                           int reverse);
+/* bias[h, i, j] = table[index[i, j], h] (index int32 [tokens * tokens]); scatter: dtable[e, h] (+)= sum of
+ * dbias[h, i, j] over the (i, j) with index[i, j] == e. */
+int tch_relpos_bias_gather(tch_context* ctx, const float* table, const int32_t* index, float* bias, int heads,
+                           int tokens, int entries);
+int tch_relpos_bias_scatter(tch_context* ctx, const float* dbias, const int32_t* index, float* dtable, int heads,
+                            int tokens, int entries, int accumulate);
+/* out[c] (+)= sum over rows of x[r, c], any width; workspace: tch_column_sum_workspace_floats(rows, cols) floats */
+int64_t tch_column_sum_workspace_floats(int rows, int cols);
+int tch_column_sum(tch_context* ctx, int dtype, const void* x, float* out, int rows, int cols, int accumulate,
+                   float* workspace);
 
 /* ---- layout / precision ---------------------------------------------------------- */
 int tch_nchw_to_nhwc_pad(tch_context* ctx, int dtype, const float* x_nchw, void* y_nhwc, int N, int C, int H, int W,

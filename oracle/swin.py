@@ -1,0 +1,177 @@
+"""Swin Transformer training-step oracle on CPU fp32 (test infrastructure only; see oracle/__init__.py).
+
+A plain torch statement of the model the reference trains with ``models.swin_b`` (train/swin_b.py:38-45,
+83-95).  torchvision is not importable here, so its exact wiring is not pinned; the block mathematics follows
+the reference's own readable statement, train/swin_b_tiny.py: window_partition / window_reverse (:8-19), the
+relative position index and bias gather (:35-59), scaled q k^T + bias (+ mask) -> softmax -> @ v -> proj
+(:49-76), pre-norm block with cyclic shift by roll (:104-137) -- and tests/golden/swin_block.npz holds
+input/output vectors written by that file's own WindowAttention and SwinTransformerBlock.  What the toy does
+not have is restated from the Swin paper / torchvision's documented behaviour and pinned by brute force in
+tests/test_swin_oracle.py: the attention mask of shifted windows, patch merging (2x2 neighbourhood
+concatenated in the order (even,even), (odd,even), (even,odd), (odd,odd) -> LayerNorm -> Linear without bias),
+patch embedding (4x4 stride-4 convolution -> LayerNorm), final LayerNorm -> mean over tokens -> Linear.
+Parameter names follow torchvision's state dict so that a real checkpoint would load unchanged.
+"""
+import math
+
+import torch
+import torch.nn.functional as F
+
+
+def relative_position_index(ws):
+    """train/swin_b_tiny.py:35-46"""
+    coords = torch.stack(torch.meshgrid([torch.arange(ws), torch.arange(ws)], indexing="ij"))
+    flat = torch.flatten(coords, 1)
+    rel = (flat[:, :, None] - flat[:, None, :]).permute(1, 2, 0).contiguous()
+    rel[:, :, 0] += ws - 1
+    rel[:, :, 1] += ws - 1
+    rel[:, :, 0] *= 2 * ws - 1
+    return rel.sum(-1)
+
+
+def window_partition(x, ws):
+    B, H, W, C = x.shape
+    return x.view(B, H // ws, ws, W // ws, ws, C).permute(0, 1, 3, 2, 4, 5).contiguous().view(-1, ws * ws, C)
+
+
+def window_reverse(win, ws, B, H, W):
+    C = win.shape[-1]
+    return win.view(B, H // ws, W // ws, ws, ws, C).permute(0, 1, 3, 2, 4, 5).contiguous().view(B, H, W, C)
+
+
+def shift_mask(H, W, ws, shift):
+    """[nW, ws*ws, ws*ws] of 0 / -100: after the cyclic shift a window may hold tokens of regions that are not
+    neighbours in the image; pairs from different regions must not attend to each other."""
+    img = torch.zeros(H, W)
+    cnt = 0
+    for hs in (slice(0, -ws), slice(-ws, -shift), slice(-shift, None)):
+        for wsl in (slice(0, -ws), slice(-ws, -shift), slice(-shift, None)):
+            img[hs, wsl] = cnt
+            cnt += 1
+    win = window_partition(img.view(1, H, W, 1), ws).squeeze(-1)          # [nW, ws*ws]
+    diff = win.unsqueeze(1) - win.unsqueeze(2)
+    return torch.where(diff != 0, torch.tensor(-100.0), torch.tensor(0.0))
+
+
+def config(embed=128, depths=(2, 2, 18, 2), heads=(4, 8, 16, 32), window=7, patch=4, image=224, classes=1000):
+    return dict(embed=embed, depths=tuple(depths), heads=tuple(heads), window=window, patch=patch, image=image,
+                classes=classes)
+
+
+def param_shapes(cfg):
+    """torchvision's swin_b state-dict names -> shapes"""
+    C, shapes = cfg["embed"], {}
+    shapes["features.0.0.weight"] = (C, 3, cfg["patch"], cfg["patch"])
+    shapes["features.0.0.bias"] = (C,)
+    shapes["features.0.2.weight"] = shapes["features.0.2.bias"] = (C,)
+    n_table = (2 * cfg["window"] - 1) ** 2
+    for s, (depth, heads) in enumerate(zip(cfg["depths"], cfg["heads"])):
+        f = 1 + 2 * s
+        for i in range(depth):
+            p = f"features.{f}.{i}."
+            shapes[p + "norm1.weight"] = shapes[p + "norm1.bias"] = (C,)
+            shapes[p + "attn.qkv.weight"], shapes[p + "attn.qkv.bias"] = (3 * C, C), (3 * C,)
+            shapes[p + "attn.proj.weight"], shapes[p + "attn.proj.bias"] = (C, C), (C,)
+            shapes[p + "attn.relative_position_bias_table"] = (n_table, heads)
+            shapes[p + "norm2.weight"] = shapes[p + "norm2.bias"] = (C,)
+            shapes[p + "mlp.0.weight"], shapes[p + "mlp.0.bias"] = (4 * C, C), (4 * C,)
+            shapes[p + "mlp.3.weight"], shapes[p + "mlp.3.bias"] = (C, 4 * C), (C,)
+        if s + 1 < len(cfg["depths"]):
+            p = f"features.{f + 1}."
+            shapes[p + "norm.weight"] = shapes[p + "norm.bias"] = (4 * C,)
+            shapes[p + "reduction.weight"] = (2 * C, 4 * C)
+            C *= 2
+    shapes["norm.weight"] = shapes["norm.bias"] = (C,)
+    shapes["head.weight"], shapes["head.bias"] = (cfg["classes"], C), (cfg["classes"],)
+    return shapes
+
+
+def make_state_dict(cfg, seed=0):
+    """trunc_normal(0.02)-like weights (plain normal here), zero biases, LayerNorm gamma 1 / beta 0; then every
+    1-D parameter is moved off its trivial value so that it takes part in a parity check."""
+    g = torch.Generator()
+    g.manual_seed(seed)
+    sd = {}
+    for k, shp in param_shapes(cfg).items():
+        if len(shp) == 1:
+            base = 1.0 if ("norm" in k and k.endswith("weight")) or k == "features.0.2.weight" else 0.0
+            sd[k] = base + torch.randn(shp, generator=g) * 0.1
+        else:
+            sd[k] = torch.randn(shp, generator=g) * 0.02
+    return sd
+
+
+def block(sd, p, x, heads, ws, shift, use_mask=True):
+    """One SwinTransformerBlock on x [B, H, W, C] (train/swin_b_tiny.py:104-137; with use_mask the attention mask
+    of shifted windows that the full model adds and the toy leaves out)."""
+    B, H, W, C = x.shape
+    if ws >= H:             # window covers the image: no shift (train/swin_b_tiny.py:99-101)
+        ws, shift = H, 0
+    D = C // heads
+    h = F.layer_norm(x, (C,), sd[p + "norm1.weight"], sd[p + "norm1.bias"], 1e-5)
+    if shift:
+        h = torch.roll(h, shifts=(-shift, -shift), dims=(1, 2))
+    win = window_partition(h, ws)                                                   # [B_, N, C]
+    B_, N, _ = win.shape
+    qkv = F.linear(win, sd[p + "attn.qkv.weight"], sd[p + "attn.qkv.bias"]).reshape(B_, N, 3, heads, D).permute(2, 0, 3, 1, 4)
+    q, k, v = qkv[0] * D ** -0.5, qkv[1], qkv[2]
+    attn = q @ k.transpose(-2, -1)
+    idx = relative_position_index(ws).view(-1)
+    bias = sd[p + "attn.relative_position_bias_table"][idx].view(N, N, heads).permute(2, 0, 1)
+    attn = attn + bias.unsqueeze(0)
+    if shift and use_mask:
+        m = shift_mask(H, W, ws, shift)
+        nW = m.shape[0]
+        attn = (attn.view(B_ // nW, nW, heads, N, N) + m.unsqueeze(1).unsqueeze(0)).view(B_, heads, N, N)
+    attn = torch.softmax(attn, dim=-1)
+    o = (attn @ v).transpose(1, 2).reshape(B_, N, C)
+    o = F.linear(o, sd[p + "attn.proj.weight"], sd[p + "attn.proj.bias"])
+    o = window_reverse(o, ws, B, H, W)
+    if shift:
+        o = torch.roll(o, shifts=(shift, shift), dims=(1, 2))
+    x = x + o
+    m = F.layer_norm(x, (C,), sd[p + "norm2.weight"], sd[p + "norm2.bias"], 1e-5)
+    m = F.gelu(F.linear(m, sd[p + "mlp.0.weight"], sd[p + "mlp.0.bias"]))
+    return x + F.linear(m, sd[p + "mlp.3.weight"], sd[p + "mlp.3.bias"])
+
+
+def patch_merging(sd, p, x):
+    C = x.shape[-1]
+    x = torch.cat([x[:, 0::2, 0::2], x[:, 1::2, 0::2], x[:, 0::2, 1::2], x[:, 1::2, 1::2]], dim=-1)
+    x = F.layer_norm(x, (4 * C,), sd[p + "norm.weight"], sd[p + "norm.bias"], 1e-5)
+    return F.linear(x, sd[p + "reduction.weight"])
+
+
+def forward(sd, images, cfg):
+    """images [B, 3, S, S] -> logits [B, classes]"""
+    x = F.conv2d(images, sd["features.0.0.weight"], sd["features.0.0.bias"], stride=cfg["patch"]).permute(0, 2, 3, 1)
+    x = F.layer_norm(x, (x.shape[-1],), sd["features.0.2.weight"], sd["features.0.2.bias"], 1e-5)
+    for s, (depth, heads) in enumerate(zip(cfg["depths"], cfg["heads"])):
+        f = 1 + 2 * s
+        for i in range(depth):
+            x = block(sd, f"features.{f}.{i}.", x, heads, cfg["window"], 0 if i % 2 == 0 else cfg["window"] // 2)
+        if s + 1 < len(cfg["depths"]):
+            x = patch_merging(sd, f"features.{f + 1}.", x)
+    x = F.layer_norm(x, (x.shape[-1],), sd["norm.weight"], sd["norm.bias"], 1e-5)
+    return F.linear(x.mean(dim=(1, 2)), sd["head.weight"], sd["head.bias"])
+
+
+def loss_and_grads(sd, images, labels, cfg, loss_scale=1.0):
+    leaf = {k: v.detach().clone().float().requires_grad_(True) for k, v in sd.items()}
+    loss = F.cross_entropy(forward(leaf, images.float(), cfg), labels)
+    (loss * loss_scale).backward()
+    return loss.detach(), {k: v.grad for k, v in leaf.items()}
+
+
+def train_steps(sd, batches, cfg, lr=1e-3, weight_decay=0.05):
+    """AdamW (PyTorch defaults for betas / eps) steps; returns (losses, final state dict)."""
+    leaf = {k: v.detach().clone().float().requires_grad_(True) for k, v in sd.items()}
+    opt = torch.optim.AdamW(list(leaf.values()), lr=lr, weight_decay=weight_decay)
+    losses = []
+    for images, labels in batches:
+        opt.zero_grad(set_to_none=False)
+        loss = F.cross_entropy(forward(leaf, images.float(), cfg), labels)
+        loss.backward()
+        opt.step()
+        losses.append(loss.item())
+    return losses, {k: v.detach() for k, v in leaf.items()}

@@ -296,6 +296,33 @@ int tch_bn_apply_bwd(tch_context* ctx, int dtype, const void* g, const void* x, 
   return bn_apply_bwd(C(ctx), dtype, g, x, dx, rows, Cc, coef);
 }
 
+int tch_window_partition(tch_context* ctx, int dtype, const void* src, void* dst, const void* add, int B, int H, int W,
+                         int Cc, int window, int shift, int reverse) {
+  return window_partition(C(ctx), dtype, src, dst, add, B, H, W, Cc, window, shift, reverse);
+}
+
+int tch_patch_merge_gather(tch_context* ctx, int dtype, const void* src, void* dst, int B, int H, int W, int Cc,
+                           int reverse) {
+  return patch_merge_gather(C(ctx), dtype, src, dst, B, H, W, Cc, reverse);
+}
+
+int tch_relpos_bias_gather(tch_context* ctx, const float* table, const int32_t* index, float* bias, int heads,
+                           int tokens, int entries) {
+  return relpos_bias_gather(C(ctx), table, index, bias, heads, tokens, entries);
+}
+
+int tch_relpos_bias_scatter(tch_context* ctx, const float* dbias, const int32_t* index, float* dtable, int heads,
+                            int tokens, int entries, int accumulate) {
+  return relpos_bias_scatter(C(ctx), dbias, index, dtable, heads, tokens, entries, accumulate);
+}
+
+int64_t tch_column_sum_workspace_floats(int rows, int cols) { return column_sum_workspace_floats(rows, cols); }
+
+int tch_column_sum(tch_context* ctx, int dtype, const void* x, float* out, int rows, int cols, int accumulate,
+                   float* workspace) {
+  return column_sum(C(ctx), dtype, x, out, rows, cols, accumulate, workspace);
+}
+
 int tch_conv2d_wgrad_pick_splits(int dtype, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad) {
   return conv2d_wgrad_pick_splits(shape(N, H, W, Cc, K, R, S, stride, pad), dtype);
 }

@@ -114,6 +114,17 @@ int embedding_fwd(Context* ctx, int dtype, const int64_t* ids, const void* wte, 
 int embedding_bwd(Context* ctx, int dtype, const int64_t* ids, const void* dy, float* dwte, float* dwpe, int B, int T,
                   int C, int vocab, int accumulate_wpe);
 
+// swin_ops.hip
+int window_partition(Context* ctx, int dtype, const void* src, void* dst, const void* add, int B, int H, int W, int C,
+                     int window, int shift, int reverse);
+int patch_merge_gather(Context* ctx, int dtype, const void* src, void* dst, int B, int H, int W, int C, int reverse);
+int relpos_bias_gather(Context* ctx, const float* table, const int32_t* index, float* bias, int heads, int tokens,
+                       int entries);
+int relpos_bias_scatter(Context* ctx, const float* dbias, const int32_t* index, float* dtable, int heads, int tokens,
+                        int entries, int accumulate);
+int64_t column_sum_workspace_floats(int rows, int cols);
+int column_sum(Context* ctx, int dtype, const void* x, float* out, int rows, int cols, int accumulate, float* workspace);
+
 // bgemm.hip
 int batched_gemm(Context* ctx, int dtype, const void* a, const void* b, void* c, int M, int N, int K, int64_t a_rs,
                  int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t ldc, int batch_outer, int batch_inner, int64_t a_bo,

@@ -25,7 +25,7 @@ unsigned flat_blocks(int64_t items, int64_t cap = 8192) {
 // ---------------------------------------------------------------------------
 // LayerNorm over the last dimension of [rows, C]
 // ---------------------------------------------------------------------------
-constexpr int kLnMaxC = 1024;  // longest row: a lane holds 16 elements of it
+constexpr int kLnMaxC = 2048;  // longest row: a lane holds 32 elements of it
 template <typename T>
 struct LnChunks {
   static constexpr int kMax = kLnMaxC / 64 / Elem<T>::kPerChunk;  // 16-byte chunks per lane and row
@@ -491,7 +491,7 @@ int layernorm_fwd(Context* ctx, int dtype, const void* x, void* y, const float* 
                   float* rstd, int64_t rows, int C, float eps) {
   if (int rc = check_rows("layernorm_fwd", dtype, rows, C)) return rc;
   const int E = dtype == kBF16 ? 8 : 4;
-  TCH_CHECK_ARG(C <= kLnMaxC, "layernorm: rows longer than 1024 elements are not supported");
+  TCH_CHECK_ARG(C <= kLnMaxC, "layernorm: rows longer than 2048 elements are not supported");
   TCH_CHECK_ARG(x && y && gamma && beta && mean && rstd, "layernorm_fwd: null tensor");
   LnArgs a{x, nullptr, nullptr, y, gamma, beta, mean, rstd, nullptr, rows, C, C / E, 0, eps};
   const double bytes = static_cast<double>(rows) * C * (dtype == kBF16 ? 4.0 : 8.0);
@@ -505,7 +505,7 @@ int layernorm_bwd(Context* ctx, int dtype, const void* dy, const void* x, void* 
                   int C, float* partial) {
   if (int rc = check_rows("layernorm_bwd", dtype, rows, C)) return rc;
   const int E = dtype == kBF16 ? 8 : 4;
-  TCH_CHECK_ARG(C <= kLnMaxC, "layernorm: rows longer than 1024 elements are not supported");
+  TCH_CHECK_ARG(C <= kLnMaxC, "layernorm: rows longer than 2048 elements are not supported");
   TCH_CHECK_ARG(dy && x && dx && gamma && mean && rstd && dgamma && dbeta && partial, "layernorm_bwd: null tensor");
   const int rpw = ln_rows_per_wg(rows);
   const int blocks = static_cast<int>((rows + rpw - 1) / rpw);

@@ -604,3 +604,56 @@ def batched_gemm(ctx, a, b, c, M, N, K, a_strides, b_strides, ldc, batch=(1, 1),
     check(lib().tch_batched_gemm(ctx.handle, dtype_code(a), _p(a), _p(b), _p(c), M, N, K, a_strides[0], a_strides[1],
                                  b_strides[0], b_strides[1], ldc, bo, bi, a_batch[0], a_batch[1], b_batch[0], b_batch[1],
                                  c_batch[0], c_batch[1], alpha, int(accumulate), int(causal)), "tch_batched_gemm")
+
+
+# ---------------------------------------------------------------------------
+# Swin-B data movement
+# ---------------------------------------------------------------------------
+
+def window_partition(ctx, src, dst, window, shift, reverse=False, add=None, image_shape=None):
+    """reverse=False: src [B,H,W,C] -> dst [B*nW*window*window, C] (cyclic shift by -shift, then windows);
+    reverse=True: src windows -> dst [B,H,W,C] (+ add).  image_shape = (B, H, W, C) when neither tensor says."""
+    B, H, W, C = image_shape if image_shape is not None else (dst.shape if reverse else src.shape)
+    assert src.numel() == dst.numel() == B * H * W * C and src.dtype == dst.dtype
+    assert add is None or (add.numel() == dst.numel() and add.dtype == dst.dtype)
+    check(lib().tch_window_partition(ctx.handle, dtype_code(src), _p(src), _p(dst), _p(add), B, H, W, C, window, shift,
+                                     int(reverse)), "tch_window_partition")
+
+
+def patch_merge_gather(ctx, src, dst, image_shape, reverse=False):
+    """image_shape = (B, H, W, C) of the unmerged side; the merged side is [B, H/2, W/2, 4C]."""
+    B, H, W, C = image_shape
+    assert src.numel() == dst.numel() == B * H * W * C and src.dtype == dst.dtype
+    check(lib().tch_patch_merge_gather(ctx.handle, dtype_code(src), _p(src), _p(dst), B, H, W, C, int(reverse)),
+          "tch_patch_merge_gather")
+
+
+def relpos_bias_gather(ctx, table, index, bias):
+    entries, heads = table.shape
+    nn = index.numel()
+    tokens = int(round(nn ** 0.5))
+    assert tokens * tokens == nn and index.dtype == torch.int32 and bias.numel() == heads * nn
+    assert table.dtype == bias.dtype == torch.float32
+    check(lib().tch_relpos_bias_gather(ctx.handle, _p(table), _p(index), _p(bias), heads, tokens, entries),
+          "tch_relpos_bias_gather")
+
+
+def relpos_bias_scatter(ctx, dbias, index, dtable, accumulate=False):
+    entries, heads = dtable.shape
+    nn = index.numel()
+    tokens = int(round(nn ** 0.5))
+    assert dbias.numel() == heads * nn and dbias.dtype == dtable.dtype == torch.float32 and index.dtype == torch.int32
+    check(lib().tch_relpos_bias_scatter(ctx.handle, _p(dbias), _p(index), _p(dtable), heads, tokens, entries,
+                                        int(accumulate)), "tch_relpos_bias_scatter")
+
+
+def column_sum_workspace_floats(rows, cols):
+    return int(lib().tch_column_sum_workspace_floats(rows, cols))
+
+
+def column_sum(ctx, x, out, workspace, accumulate=False):
+    rows, cols = x.shape
+    assert out.numel() == cols and out.dtype == workspace.dtype == torch.float32 and x.is_contiguous()
+    assert workspace.numel() >= column_sum_workspace_floats(rows, cols)
+    check(lib().tch_column_sum(ctx.handle, dtype_code(x), _p(x), _p(out), rows, cols, int(accumulate), _p(workspace)),
+          "tch_column_sum")
