@@ -139,11 +139,53 @@ def gpt2_step(batch=8, seq_len=1024, warmup=2, steps=5):
     return res
 
 
+def swin_b_step(batch=32, warmup=2, steps=5):
+    """BASELINE configs[3]: Swin-B (87.77 M parameters), bf16 compute with fp32 master weights, images
+    [32, 3, 224, 224] N(0,1), AdamW(lr 1e-3, wd 0.05), stochastic depth 0.  Reported beside the headline figure."""
+    import torch
+    from sirius_amd.swin import SwinEngine
+    eng = SwinEngine(dtype=torch.bfloat16)
+    eng.init_normal(0)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(3)
+    x = torch.randn(batch, 3, 224, 224, device="cuda", generator=g)
+    y = torch.randint(0, 1000, (batch,), device="cuda", generator=g)
+    for _ in range(warmup):
+        eng.forward_backward(x, y)
+        eng.optimizer_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        eng.forward_backward(x, y)
+        eng.optimizer_step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    plan = eng.plan(batch)
+    rows = eng.ctx.profile(plan.prog, 1) + eng.ctx.profile(eng._opt_prog, 1)
+    rows.sort(key=lambda r: -r["total_ms"])
+    gemm = [r for r in rows if not r["work_is_bytes"]]
+    flops = sum(r["work"] for r in gemm)
+    res = {
+        "workload": f"Swin-B training step, bf16, images [{batch}, 3, 224, 224], AdamW(lr 1e-3, wd 0.05)",
+        "images_per_s": batch / dt, "ms_per_step": dt * 1e3, "loss_after_run": eng.last_loss(),
+        "parameters": eng.num_parameters(), "launches_per_step": len(plan.prog) + len(eng._opt_prog),
+        "mfma_tflop_per_step": flops / 1e12,
+        "mfma_util": flops / (sum(r["total_ms"] for r in gemm) * 1e-3) / PEAK_BF16_FLOPS,
+        "breakdown": [{"kernel": r["name"], "ms_per_step": round(r["total_ms"], 4), "launches": r["launches"]}
+                      for r in rows[:8]],
+    }
+    del eng, plan
+    torch.cuda.empty_cache()
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--no-handover", action="store_true", help="skip the 64 -> 16 -> 64 handover measurement")
     ap.add_argument("--no-gpt2", action="store_true", help="skip the GPT-2 step measurement")
     ap.add_argument("--only-gpt2", action="store_true", help="run the GPT-2 step measurement alone (for profiling it)")
+    ap.add_argument("--no-swin", action="store_true", help="skip the Swin-B step measurement")
+    ap.add_argument("--only-swin", action="store_true", help="run the Swin-B step measurement alone (for profiling it)")
     ap.add_argument("--no-autotune", action="store_true", help="keep the library's tiling heuristic")
     ap.add_argument("--no-overlap", action="store_true", help="record weight gradients on the main lane (one stream)")
     ap.add_argument("--calibrate", action="store_true",
@@ -167,6 +209,9 @@ def main():
     torch.cuda.set_device(0)
     if args.only_gpt2:
         print(json.dumps({"gpt2": gpt2_step(steps=args.steps, warmup=args.warmup)}), flush=True)
+        return
+    if args.only_swin:
+        print(json.dumps({"swin_b": swin_b_step(steps=args.steps, warmup=args.warmup)}), flush=True)
         return
     B = args.batch
     eng = ResNetEngine((3, 8, 36, 3), 1000, 64, dtype=torch.bfloat16, image_size=224, lr=0.1, momentum=0.9,
@@ -275,6 +320,11 @@ def main():
             out["gpt2"] = gpt2_step()
         except Exception as e:
             out["gpt2"] = {"error": repr(e)}
+    if not args.no_swin:
+        try:
+            out["swin_b"] = swin_b_step()
+        except Exception as e:
+            out["swin_b"] = {"error": repr(e)}
     print(json.dumps(out), flush=True)
 
 

@@ -210,6 +210,35 @@ def test_gpt2_handover_8_2_8_on_gpu(clean_runtime, monkeypatch, tmp_path):
     assert tc.GetXQueueSizeAllStreams() == 0
 
 
+def test_swin_handover_16_4_16_on_gpu(clean_runtime, monkeypatch, tmp_path):
+    """The handover with the Swin engine (the reference's train/swin_b.py under colocate-l1)."""
+    tc = clean_runtime
+    from sirius_amd.train import swin_b as script
+    env = {"COLTRAIN_MODE": "colocate-l1", "COLTRAIN_HOOK_MODE": "xsched-sync", "COLTRAIN_USE_XSCHED": "1",
+           "COLTRAIN_HAS_INFER_SERVER": "1", "COLTRAIN_USE_SHARED_TENSOR": "1",
+           "COLTRAIN_SHARED_TENSOR_POOL_GB": "2", "COLTRAIN_PROFILE_LOG_PATH": str(tmp_path / "train-profile.csv")}
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    peer = script.PeerScript({3: ("l1", 4), 10: ("exit", 16)}, delay_ms=1.0)
+    try:
+        out = script.train(1, 16, dataset_size=16 * 8, dtype=torch.bfloat16, peer=peer, num_distinct_samples=32,
+                           embed=32, depths=(2, 2), heads=(2, 4), window=4, patch=2, image_size=32, num_classes=16)
+    finally:
+        peer.stop()
+    stat = out["trainer"].get_last_epoch_stat()
+    assert stat.finished_sample == 16 * 8
+    assert [k for _, k, _ in peer.sent] == ["l1", "exit"]
+    req, fin = tc.get_adjust_request_time_stamp(), tc.get_adjust_done_time_stamp()
+    assert len(req) == 1 and len(fin) == 1 and 0 <= (fin[0] - req[0]) / 1e3 < 50.0
+    import csv
+    rows = [r for r in csv.DictReader(open(out["profile"])) if r["name"].startswith("batch_0")]
+    sizes = [int(r["name"].split("_")[-1]) for r in rows]
+    assert sizes[0] == 16 and 4 in sizes and sizes[-1] > 4
+    assert sum(s for r, s in zip(rows, sizes) if r["tag"] == "finish") == 16 * 8
+    assert all(torch.isfinite(v).all() for v in out["model"].state_dict().values())
+    assert tc.GetXQueueSizeAllStreams() == 0
+
+
 def test_torch_allocations_through_the_pool_hook(clean_runtime):
     """torch's own allocations land in the pool through the allocator hook
     (tch_pool_malloc / tch_pool_free in the shape torch's pluggable allocator binds; the

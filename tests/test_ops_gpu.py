@@ -50,6 +50,7 @@ CONV_CASES = [
     (3, 7, 7, 32, 40, 3, 3, 1, 1),        # ragged: rows, cols and reduction all off-tile
     (5, 1, 1, 64, 1000, 1, 1, 1, 0),      # fully connected as a 1x1 convolution
     (1, 9, 11, 16, 24, 3, 3, 1, 1),       # non-square
+    (2, 16, 16, 8, 32, 4, 4, 4, 0),       # patch embedding: 4x4 patches, stride 4, channels padded to one chunk
 ]
 
 
