@@ -18,6 +18,7 @@ recorded program of hand-written kernels per batch size:
 
 torch supplies device memory and streams only.  Dropout is off (probabilities 0).
 """
+import contextlib
 import math
 
 import torch
@@ -41,8 +42,12 @@ class _Plan:
 class GPT2Engine(EngineBase):
     def __init__(self, vocab=50257, n_pos=1024, n_embd=768, n_layer=12, n_head=12, seq_len=1024, dtype=torch.bfloat16,
                  optimizer="adamw", lr=1e-3, weight_decay=0.01, betas=(0.9, 0.999), eps=1e-8, momentum=0.9,
-                 stream=None, allocator=None):
+                 stream=None, allocator=None, overlap_wgrad=True):
         self._init_engine(dtype, stream, allocator)
+        # weight and bias gradients depend only on a saved activation and on a gradient that stays put until
+        # the layer is done: recorded on a second lane, they run beside the data-gradient chain; the lanes
+        # meet at the end of every layer, before its gradient buffers are handed round again
+        self.overlap_wgrad = overlap_wgrad
         assert n_embd % n_head == 0 and n_embd % 8 == 0 and seq_len <= n_pos
         assert optimizer in ("adamw", "sgd")
         self.vocab, self.n_pos, self.C, self.n_layer, self.n_head = vocab, n_pos, n_embd, n_layer, n_head
@@ -241,10 +246,14 @@ class GPT2Engine(EngineBase):
             ops.conv2d_fwd(ctx, as4(x), self._w(name + ".weight"), as4(y), 1, 0,
                            bias=self._view(self.params, name + ".bias"), add=None if add is None else as4(add))
 
+        def side():
+            return ctx.side_lane(wait_main=True) if self.overlap_wgrad else contextlib.nullcontext()
+
         def lin_bwd(name, x, dy, dx):
             """dW, db from (x, dy); dx = dy W"""
-            ops.conv2d_wgrad(ctx, as4(x), as4(dy), self._view(self.grads, name + ".weight"), 1, 0, workspace=wg_ws)
-            ops.bias_grad(ctx, dy, self._view(self.grads, name + ".bias"), workspace=bias_ws)
+            with side():
+                ops.conv2d_wgrad(ctx, as4(x), as4(dy), self._view(self.grads, name + ".weight"), 1, 0, workspace=wg_ws)
+                ops.bias_grad(ctx, dy, self._view(self.grads, name + ".bias"), workspace=bias_ws)
             ops.conv2d_dgrad(ctx, as4(dy), self._wt(name + ".weight"), as4(dx), 1, 0)
 
         # strides / batch offsets of head h of sample b inside the packed projection and the score tensor
@@ -303,8 +312,9 @@ class GPT2Engine(EngineBase):
             g_f1, g_f2, g_qkv = act(R, 4 * C), act(R, 4 * C), act(R, 3 * C)
             dP = act(B, H, T, T)
             d_hf, g = g_c[0], g_c[1]
-            ops.conv2d_wgrad(ctx, as4(hf), as4(dlogits), self._view(self.grads, "transformer.wte.weight"), 1, 0,
-                             workspace=wg_ws)
+            with side():
+                ops.conv2d_wgrad(ctx, as4(hf), as4(dlogits), self._view(self.grads, "transformer.wte.weight"), 1, 0,
+                                 workspace=wg_ws)
             ops.conv2d_dgrad(ctx, as4(dlogits), self._wt("transformer.wte.weight"), as4(d_hf), 1, 0)
             ln_bwd("transformer.ln_f", 2 * L, d_hf, h, g)
             mark("bwd", "ln_f")
@@ -335,6 +345,8 @@ class GPT2Engine(EngineBase):
                 g_next = d_o
                 ln_bwd(pre + "ln_1", 2 * i, d_a, h_in, g_next, residual=g1)
                 g = g_next
+                if self.overlap_wgrad:
+                    ctx.join()
                 mark("bwd", f"h.{i}")
             # tied weights: the scattered embedding gradient lands on top of the head's weight gradient
             ops.embedding_bwd(ctx, plan.ids, g.view(B, T, C), self._view(self.grads, "transformer.wte.weight").view(Vp, C),

@@ -19,6 +19,7 @@ adds: the attention mask of shifted windows, patch merging, patch embedding.
 
 torch supplies device memory and streams only.  Stochastic depth and dropout are off.
 """
+import contextlib
 import math
 
 import torch
@@ -69,8 +70,11 @@ def shifted_window_mask(H, W, ws, shift):
 class SwinEngine(EngineBase):
     def __init__(self, embed=128, depths=(2, 2, 18, 2), heads=(4, 8, 16, 32), window=7, patch=4, image_size=224,
                  num_classes=1000, dtype=torch.bfloat16, lr=1e-3, weight_decay=0.05, betas=(0.9, 0.999), eps=1e-8,
-                 stream=None, allocator=None):
+                 stream=None, allocator=None, overlap_wgrad=True):
         self._init_engine(dtype, stream, allocator)
+        # weight / bias / bias-table gradients on a second lane beside the data-gradient chain; the lanes meet
+        # at the end of every block, before its gradient buffers are handed round again
+        self.overlap_wgrad = overlap_wgrad
         assert len(depths) == len(heads) and image_size % patch == 0 and num_classes % 8 == 0 and embed % 8 == 0
         self.embed, self.depths, self.heads = embed, tuple(depths), tuple(heads)
         self.window, self.patch, self.image_size, self.num_classes = window, patch, image_size, num_classes
@@ -285,10 +289,14 @@ class SwinEngine(EngineBase):
                            bias=self._view(self.params, name + ".bias") if bias else None,
                            add=None if add is None else as4(add))
 
+        def side():
+            return ctx.side_lane(wait_main=True) if self.overlap_wgrad else contextlib.nullcontext()
+
         def lin_bwd(name, x, dy, dx, bias=True):
-            ops.conv2d_wgrad(ctx, as4(x), as4(dy), self._view(self.grads, name + ".weight"), 1, 0, workspace=wg_ws)
-            if bias:
-                ops.bias_grad(ctx, dy, self._view(self.grads, name + ".bias"), workspace=bias_ws)
+            with side():
+                ops.conv2d_wgrad(ctx, as4(x), as4(dy), self._view(self.grads, name + ".weight"), 1, 0, workspace=wg_ws)
+                if bias:
+                    ops.bias_grad(ctx, dy, self._view(self.grads, name + ".bias"), workspace=bias_ws)
             if dx is not None:
                 ops.conv2d_dgrad(ctx, as4(dy), self._wt(name + ".weight"), as4(dx), 1, 0)
 
@@ -296,7 +304,9 @@ class SwinEngine(EngineBase):
         def flat(n):
             return act(n)
         s_n1 = flat(max_rc)                                    # LayerNorm output before it is gathered
-        g_bufs = [flat(max_rc) for _ in range(4)]              # gradients of [rows, C] tensors, handed round
+        # gradients of [rows, C] tensors, handed round; six, so that inside a block nothing the second lane
+        # still reads (the block's incoming gradient, the gathered projection gradient) is written again
+        g_bufs = [flat(max_rc) for _ in range(6)]
         g_3c, g_4c_a, g_4c_b = flat(3 * max_rc), flat(4 * max_rc), flat(4 * max_rc)
         max_scores = max(B * (st["R"] // st["ws"]) ** 2 * st["heads"] * st["ws"] ** 4 for st in self.stages)
         d_scores = flat(max_scores)
@@ -443,23 +453,26 @@ class SwinEngine(EngineBase):
                     # g is the gradient of the merged tokens [rows/4, 2C]
                     xm, nm, mstats = merges[si]
                     pre = f"features.{st['f'] + 1}."
-                    spare = [k for k in range(4) if k != gi]
+                    spare = [k for k in range(len(g_bufs)) if k != gi]
                     d_nm = v2(g_4c_a, rows // 4, 4 * C)
-                    ops.conv2d_wgrad(ctx, as4(nm), as4(g), self._view(self.grads, pre + "reduction.weight"), 1, 0,
-                                     workspace=wg_ws)
+                    with side():
+                        ops.conv2d_wgrad(ctx, as4(nm), as4(g), self._view(self.grads, pre + "reduction.weight"), 1, 0,
+                                         workspace=wg_ws)
                     ops.conv2d_dgrad(ctx, as4(g), self._wt(pre + "reduction.weight"), as4(d_nm), 1, 0)
                     d_xm = v2(g_4c_b, rows // 4, 4 * C)
                     ln_bwd(pre + "norm", d_nm, xm, d_xm, mstats)
                     gi = spare[0]
                     g = v2(g_bufs[gi], rows, C)
                     ops.patch_merge_gather(ctx, d_xm, g, (B, R, R, C), reverse=True)
+                    if self.overlap_wgrad:
+                        ctx.join()
                     mark("bwd", pre[:-1])
                 for i in range(st["depth"] - 1, -1, -1):
                     bi -= 1
                     _, _, shift, x_in, xw, qkv, Pm, o, x1, n2, f1, f2, stats1, stats2 = saved_blocks[bi]
                     pre = f"features.{st['f']}.{i}."
-                    spare = [k for k in range(4) if k != gi]
-                    t_a, t_b, t_c = (v2(g_bufs[k], rows, C) for k in spare)
+                    spare = [k for k in range(len(g_bufs)) if k != gi]
+                    t_a, t_b, t_c, t_d, t_e = (v2(g_bufs[k], rows, C) for k in spare)
                     d_f2, d_f1, d_qkv = v2(g_4c_a, rows, 4 * C), v2(g_4c_b, rows, 4 * C), v2(g_3c, rows, 3 * C)
                     fq, fg = qkv.view(-1), d_qkv.view(-1)
                     dP = d_scores[:B_ * Hh * N * N].view(B_, Hh, N, N)
@@ -481,32 +494,38 @@ class SwinEngine(EngineBase):
                     ops.batched_gemm(ctx, d_o, fq[2 * C:], dP, N, N, D, (C, 1), (qkv_row, 1), N, (B_, Hh), o_b, qkv_b, s_b)
                     ops.attn_softmax_bwd(ctx, Pm, dP, dP, 1.0)
                     dbias = dbias_buf[:Hh * N * N]
-                    ops.column_sum(ctx, dP.view(B_, Hh * N * N), dbias, colsum_ws)
-                    ops.relpos_bias_scatter(ctx, dbias, st["index_dev"],
-                                            self._view(self.grads, pre + "attn.relative_position_bias_table"))
+                    with side():
+                        ops.column_sum(ctx, dP.view(B_, Hh * N * N), dbias, colsum_ws)
+                        ops.relpos_bias_scatter(ctx, dbias, st["index_dev"],
+                                                self._view(self.grads, pre + "attn.relative_position_bias_table"))
                     ops.batched_gemm(ctx, dP, fq[C:], fg, N, D, N, (N, 1), (1, qkv_row), qkv_row, (B_, Hh), s_b, qkv_b, qkv_b,
                                      alpha=scale)
                     ops.batched_gemm(ctx, dP, fq, fg[C:], N, D, N, (1, N), (1, qkv_row), qkv_row, (B_, Hh), s_b, qkv_b, qkv_b,
                                      alpha=scale)
-                    d_xw = t_a
+                    d_xw = t_d
                     lin_bwd(pre + "attn.qkv", xw, d_qkv, d_xw)
                     if whole:
                         d_n1 = d_xw
                     else:
                         d_n1 = t_c
                         ops.window_partition(ctx, d_xw, d_n1, ws, shift, reverse=True, image_shape=(B, R, R, C))
-                    # the new running gradient goes where neither d_n1 nor g1 lives
-                    g_next = v2(g_bufs[gi], rows, C)          # the old running gradient is dead by now
+                    # the new running gradient goes into a buffer of its own: the old one may still be read by
+                    # this block's first weight gradient on the second lane
+                    g_next = t_e
                     ln_bwd(pre + "norm1", d_n1, x_in, g_next, stats1, residual=g1)
-                    g = g_next
+                    g, gi = g_next, spare[4]
+                    if self.overlap_wgrad:
+                        ctx.join()
                     mark("bwd", pre[:-1])
             # patch embedding: LayerNorm, then the 4x4 stride-4 convolution (no data gradient: it is the input)
-            spare = [k for k in range(4) if k != gi]
+            spare = [k for k in range(len(g_bufs)) if k != gi]
             d_e0 = v2(g_bufs[spare[0]], rows0, C0)
             ln_bwd("features.0.2", g, e0, d_e0, embed_stats)
             ops.conv2d_wgrad(ctx, x0, d_e0.view(B, R0, R0, C0), self._view(self.grads, "features.0.0.weight"), P, 0,
                              workspace=wg_ws, c_logical=3)
             ops.bias_grad(ctx, d_e0, self._view(self.grads, "features.0.0.bias"), workspace=bias_ws)
+            if self.overlap_wgrad:
+                ctx.join()
             mark("bwd", "features.0")
         finally:
             ctx.end_record()
