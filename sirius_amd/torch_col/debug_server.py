@@ -36,6 +36,17 @@ class DebugServer:
     def infer_exit(self, batch_size: int):
         return self._send(CtrlEvent.kInferExit, batch_size)
 
+    # -- task switching (the controller's pair of commands, server/control/controller.cc:207-260)
+    def interrupt_train(self):
+        cmd_id = self._cmd_ids[CtrlEvent.kInterruptTrain] = self._cmd_ids.get(CtrlEvent.kInterruptTrain, 0) + 1
+        self._inf_tra_comm.put_inf2tra(_C.PyCtrlMsgEntry(cmd_id, CtrlEvent.kInterruptTrain, 0), 0)
+        return cmd_id
+
+    def resume_train(self):
+        cmd_id = self._cmd_ids[CtrlEvent.kResumeTrain] = self._cmd_ids.get(CtrlEvent.kResumeTrain, 0) + 1
+        self._inf_tra_comm.put_inf2tra(_C.PyCtrlMsgEntry(cmd_id, CtrlEvent.kResumeTrain, 0), 0)
+        return cmd_id
+
     # -- requests in megabytes, through the server's own arithmetic (server/train_adjuster.cc)
     def require_memory_mb(self, required_mem_mb: float, adjuster=None):
         """Inference needs required_mem_mb more: shrink training by ceil(MB / slope) samples."""

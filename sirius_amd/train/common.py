@@ -21,7 +21,8 @@ def cleanup():
 
 
 class PeerScript:
-    """Stand-in inference server: `at` maps a micro-batch index to ('l1' | 'l2' | 'exit', batch size).
+    """Stand-in inference server: `at` maps a micro-batch index to ('l1' | 'l2' | 'exit', batch size) or to
+    ('switch', milliseconds until the resume).
     The command is sent from a side thread `delay_ms` after the micro-batch began, so that it lands
     while kernels are queued, as a real request would."""
 
@@ -40,6 +41,15 @@ class PeerScript:
         def fire():
             time.sleep(self.delay_ms / 1e3)
             t = torch_col.get_unix_timestamp_us()
+            if kind == "switch":
+                # task switch: interrupt now, resume `bs` milliseconds later (training stands still in
+                # between, so no micro-batch index could trigger the resume)
+                self.server.interrupt_train()
+                self.sent.append((t, "interrupt", 0))
+                time.sleep(bs / 1e3)
+                self.server.resume_train()
+                self.sent.append((torch_col.get_unix_timestamp_us(), "resume", 0))
+                return
             {"l1": self.server.colocate_l1, "l2": self.server.colocate_l2,
              "exit": self.server.infer_exit}[kind](bs)
             self.sent.append((t, kind, bs))

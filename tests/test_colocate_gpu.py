@@ -264,3 +264,35 @@ def test_torch_allocations_through_the_pool_hook(clean_runtime):
     finally:
         torch.cuda.synchronize()
         L.tch_pool_shutdown(0)
+
+
+def test_task_switch_interrupt_and_resume_on_gpu(clean_runtime, monkeypatch, tmp_path):
+    """taskswitch-l1 (the reference's second control flow: csrc/control_stub.cc:186-400, colocate_ctrl.py:117-301,
+    trainer.py:244-248): the peer interrupts training in the middle of a micro-batch; the batch is killed, all
+    activation memory goes back to the pool, kInterruptTrainDone is sent; training stands still until
+    kResumeTrain, answers kResumeTrainDone and finishes every sample."""
+    tc = clean_runtime
+    from sirius_amd.train import resnet152 as script
+    env = {"COLTRAIN_MODE": "taskswitch-l1", "COLTRAIN_HOOK_MODE": "xsched-sync", "COLTRAIN_USE_XSCHED": "1",
+           "COLTRAIN_HAS_INFER_SERVER": "1", "COLTRAIN_USE_SHARED_TENSOR": "1",
+           "COLTRAIN_SHARED_TENSOR_POOL_GB": "2", "COLTRAIN_PROFILE_LOG_PATH": str(tmp_path / "train-profile.csv")}
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    pause_ms = 30.0
+    peer = script.PeerScript({3: ("switch", pause_ms)}, delay_ms=1.0)
+    try:
+        out = script.train(1, 64, dataset_size=64 * 8, dtype=torch.bfloat16, peer=peer, num_distinct_samples=64, **SMALL)
+        events = [(t, m.event) for t, m in peer.server.received]
+    finally:
+        peer.stop()
+    stat = out["trainer"].get_last_epoch_stat()
+    assert stat.finished_sample == 64 * 8 and stat.killed_batch >= 1
+    assert [k for _, k, _ in peer.sent] == ["interrupt", "resume"]
+    t_int, t_res = peer.sent[0][0], peer.sent[1][0]
+    done = [t for t, e in events if e == tc.CtrlEvent.kInterruptTrainDone]
+    resumed = [t for t, e in events if e == tc.CtrlEvent.kResumeTrainDone]
+    assert len(done) == 1 and len(resumed) == 1
+    assert 0 <= (done[0] - t_int) / 1e3 < 50.0, "interrupt -> done within the handover bound"
+    assert resumed[0] >= t_res and (resumed[0] - t_int) / 1e3 >= pause_ms
+    assert all(torch.isfinite(v).all() for v in out["model"].state_dict().values())
+    assert tc.GetXQueueSizeAllStreams() == 0
