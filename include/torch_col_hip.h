@@ -96,6 +96,18 @@ void tch_SetRejectCudaCalls(int reject);            /* xsched_ctrl.cc:196-198 */
 void tch_SetXQueueShape(int queue_length, int sync_interval);
 size_t tch_GetXQueueInFlight(uint64_t hip_stream);
 
+/* ---- compute-unit partitioning (the reference's SMPartitioner, common/sm_partition.cc:26-112, with compute
+ * units in the place of TPCs; csrc/init.cc:43-71 installs it) ------------------------------------------
+ * init: total_cus <= 0 asks the current device; training may use between min and max compute units.
+ * train_avail(required) = min(max, max(min, total - required)).  A context with a limit n launches on streams
+ * whose CU mask keeps the highest-numbered n compute units (the other tenant keeps the lowest); 0 lifts the
+ * limit.  Changing the limit between two program runs is ordered like any two launches of the context. */
+int tch_cu_partition_init(int total_cus, int min_train_cus, int max_train_cus);
+int tch_cu_partition_total(void);
+int tch_cu_partition_train_avail(int infer_required_cus);
+int tch_context_set_cu_limit(tch_context* ctx, int n_cus);
+int tch_context_get_cu_limit(tch_context* ctx);
+
 /* ---- convolution (implicit GEMM on MFMA) ---------------------------------------- */
 /* y[N,Ho,Wo,K] = conv(x[N,H,W,C], w[K,R,S,C]) (+ bias[K]) (+ add, optionally gated by mask > 0).
  * out_f32 != 0 stores y as fp32 whatever dtype is.  tile_cfg: -1 auto, 0 = 128x128, 1 = 128x64, 2 = 64x64,

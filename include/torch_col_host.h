@@ -117,6 +117,11 @@ int tch_update_current_batch_size(int batch_size);
 /* field: 0 pid, 1 rank, 2 world size, 3 init bs, 4 current bs, 5 target bs, 6 target bs unpublished, 7 first epoch done */
 int tch_train_info_get_field(int id, int field);
 int tch_train_info_set_field(int id, int field, int value);
+/* Compute units the inference side wants on `device` (shared-memory board; the reference's
+ * SMPartitioner::Set/Add/Dec/GetInferRequiredTpcNum, common/sm_partition.cc:60-76).  add returns the new value. */
+int tch_infer_required_cus_get(int device);
+int tch_infer_required_cus_set(int device, int n);
+int tch_infer_required_cus_add(int device, int delta);
 int tch_train_info_is_valid(int id);
 int tch_train_info_model_name(int id, char* out, int cap);
 

@@ -125,12 +125,38 @@ int tch_program_run(tch_context* ctx, const tch_program* prog, int64_t first, in
   // the stream may have been registered after the context was made
   ctx->ctx.queue = queue_for_stream(reinterpret_cast<uint64_t>(ctx->ctx.stream));
   const uint64_t before = ctx->ctx.rejected.load();
+  // with a compute-unit limit the launches go to another stream than the caller's: order them behind
+  // what the caller's stream holds, and what the caller does next behind them
+  const bool limited = ctx->ctx.cu_limit > 0 && first < last;
+  if (limited)
+    if (int rc = ctx->ctx.depend(ctx->ctx.stream, ctx->ctx.main_stream())) return rc;
   for (int64_t i = first; i < last; ++i) {
     int rc = ctx->ctx.dispatch(prog->prog.launches[static_cast<size_t>(i)]);
     if (rc) return rc;
   }
+  if (limited)
+    if (int rc = ctx->ctx.depend(ctx->ctx.main_stream(), ctx->ctx.stream)) return rc;
   return ctx->ctx.rejected.load() != before ? 1 : 0;
 }
+
+int tch_cu_partition_init(int total_cus, int min_train_cus, int max_train_cus) {
+  return cu_partition_init(total_cus, min_train_cus, max_train_cus);
+}
+int tch_cu_partition_total(void) { return cu_partition_total(); }
+int tch_cu_partition_train_avail(int infer_required_cus) { return cu_partition_train_avail(infer_required_cus); }
+int tch_context_set_cu_limit(tch_context* ctx, int n_cus) {
+  if (!ctx) {
+    set_error("tch_context_set_cu_limit: null context");
+    return -22;
+  }
+  if (ctx->ctx.recording) {
+    set_error("tch_context_set_cu_limit: context is recording");
+    return -16;
+  }
+  ctx->ctx.queue = queue_for_stream(reinterpret_cast<uint64_t>(ctx->ctx.stream));
+  return ctx->ctx.set_cu_limit(n_cus);
+}
+int tch_context_get_cu_limit(tch_context* ctx) { return ctx ? ctx->ctx.cu_limit : -22; }
 
 uint64_t tch_RegisterStream(uint64_t hip_stream) { return register_stream(hip_stream); }
 int tch_UnRegisterStream(uint64_t hip_stream) { return unregister_stream(hip_stream); }

@@ -34,6 +34,7 @@ const char* last_error() { return g_error.c_str(); }
 
 LaunchQueue::LaunchQueue(hipStream_t stream, int queue_length, int sync_interval)
     : stream_(stream),
+      launch_stream_(stream),
       queue_length_(queue_length < 1 ? 1 : static_cast<size_t>(queue_length)),
       sync_interval_(sync_interval < 1 ? 1 : static_cast<uint64_t>(sync_interval)) {
   if (hipGetDevice(&device_) != hipSuccess) device_ = 0;
@@ -52,20 +53,42 @@ LaunchQueue::~LaunchQueue() {
   for (auto e : free_events_) (void)hipEventDestroy(e);
 }
 
-void LaunchQueue::submit(const LaunchRecord& rec) {
+void LaunchQueue::submit(const LaunchRecord& rec, hipStream_t on) {
   {
     std::lock_guard<std::mutex> lock(mu_);
     wait_.emplace_back();
     wait_.back().rec = rec;
+    wait_.back().on = on;
   }
   cv_work_.notify_one();
+}
+
+void LaunchQueue::submit_dependency(hipStream_t from, hipStream_t to) {
+  {
+    std::lock_guard<std::mutex> lock(mu_);
+    wait_.emplace_back();
+    wait_.back().is_dependency = true;
+    wait_.back().on = from;
+    wait_.back().to = to;
+  }
+  cv_work_.notify_one();
+}
+
+void LaunchQueue::chain(hipStream_t from, hipStream_t to) {
+  if (from == to) return;
+  hipEvent_t ev = take_event();
+  if (!ev || hipEventRecord(ev, from) != hipSuccess || hipStreamWaitEvent(to, ev, 0) != hipSuccess)
+    error_.store(static_cast<int>(hipErrorUnknown));
+  // the event may be recorded again once the wait is enqueued (the wait holds its own reference to the
+  // recorded state)
+  if (ev) free_events_.push_back(ev);
 }
 
 size_t LaunchQueue::clear() {
   std::lock_guard<std::mutex> lock(mu_);
   size_t removed = 0;
   for (auto it = wait_.begin(); it != wait_.end();) {
-    if (!it->is_sync) {
+    if (!it->is_sync && !it->is_dependency) {
       it = wait_.erase(it);
       ++removed;
     } else {
@@ -90,6 +113,8 @@ int LaunchQueue::synchronize() {
 size_t LaunchQueue::size() {
   std::lock_guard<std::mutex> lock(mu_);
   size_t n = 0;
+  // stream dependencies count: whoever waits for the queue to empty before giving the stream work of
+  // its own (copies, read-backs) relies on the trailing dependency of a compute-unit-limited run
   for (auto& it : wait_)
     if (!it.is_sync) ++n;
   return n;
@@ -127,7 +152,7 @@ void LaunchQueue::drain_log_until(size_t keep) {
         log_.pop_front();
       }
     } else {
-      hipError_t e = hipStreamSynchronize(stream_);
+      hipError_t e = hipStreamSynchronize(launch_stream_);
       if (e != hipSuccess) error_.store(static_cast<int>(e));
       log_.clear();
     }
@@ -135,10 +160,15 @@ void LaunchQueue::drain_log_until(size_t keep) {
   in_flight_.store(log_.size());
 }
 
-void LaunchQueue::launch_one(const LaunchRecord& rec) {
+void LaunchQueue::launch_one(const LaunchRecord& rec, hipStream_t on) {
   if (log_.size() >= queue_length_) drain_log_until(queue_length_ - 1);
+  hipStream_t target = on ? on : stream_;
+  if (target != launch_stream_) {
+    chain(launch_stream_, target);
+    launch_stream_ = target;
+  }
   void* args[1] = {const_cast<unsigned char*>(rec.args)};
-  hipError_t e = hipLaunchKernel(rec.fn, rec.grid, rec.block, args, 0, stream_);
+  hipError_t e = hipLaunchKernel(rec.fn, rec.grid, rec.block, args, 0, launch_stream_);
   if (e != hipSuccess) {
     error_.store(static_cast<int>(e));
     return;
@@ -147,7 +177,7 @@ void LaunchQueue::launch_one(const LaunchRecord& rec) {
   hipEvent_t ev = nullptr;
   if (idx - last_sync_idx_ >= sync_interval_) {
     ev = take_event();
-    if (ev && hipEventRecord(ev, stream_) == hipSuccess) {
+    if (ev && hipEventRecord(ev, launch_stream_) == hipSuccess) {
       last_sync_idx_ = idx;
     } else if (ev) {
       free_events_.push_back(ev);
@@ -173,8 +203,14 @@ void LaunchQueue::worker_loop() {
       item = wait_.front();
       wait_.pop_front();
     }
+    if (item.is_dependency) {
+      // the source of a dependency that names the launch stream of the moment is wherever the last launch went
+      chain(item.on, item.to);
+      continue;
+    }
     if (item.is_sync) {
-      hipError_t e = hipStreamSynchronize(stream_);
+      hipError_t e = hipStreamSynchronize(launch_stream_);
+      if (e == hipSuccess && launch_stream_ != stream_) e = hipStreamSynchronize(stream_);
       if (e != hipSuccess) error_.store(static_cast<int>(e));
       for (auto& l : log_)
         if (l.event) free_events_.push_back(l.event);
@@ -186,7 +222,7 @@ void LaunchQueue::worker_loop() {
       }
       cv_done_.notify_all();
     } else {
-      launch_one(item.rec);
+      launch_one(item.rec, item.on);
     }
   }
   // release waiters that raced with shutdown
@@ -230,7 +266,52 @@ int Context::record_join() {
   return 0;
 }
 
+int Context::depend(hipStream_t from, hipStream_t to) {
+  if (from == to) return 0;
+  if (queue) {
+    queue->submit_dependency(from, to);
+    return 0;
+  }
+  hipEvent_t e = next_event();
+  if (!e || hipEventRecord(e, from) != hipSuccess || hipStreamWaitEvent(to, e, 0) != hipSuccess) {
+    set_error("stream dependency failed");
+    return -5;
+  }
+  return 0;
+}
+
+int Context::set_cu_limit(int n_cus) {
+  const int total = cu_partition_total();
+  if (n_cus <= 0 || (total > 0 && n_cus >= total)) n_cus = 0;
+  if (n_cus == cu_limit) return 0;
+  hipStream_t new_main = stream, new_side = side;
+  if (n_cus > 0) {
+    new_main = cu_partition_stream(n_cus, 0);
+    new_side = cu_partition_stream(n_cus, 1);
+    if (!new_main || !new_side) return -5;
+  }
+  // what the old pair of streams holds comes first
+  hipStream_t old_main = main_stream(), old_side = cu_limit > 0 ? masked_side : side;
+  if (int rc = depend(old_main, new_main)) return rc;
+  if (side_dirty && old_side) {
+    if (int rc = depend(old_side, new_main)) return rc;
+    side_dirty = false;
+  }
+  cu_limit = n_cus;
+  masked_main = n_cus > 0 ? new_main : nullptr;
+  masked_side = n_cus > 0 ? new_side : nullptr;
+  return 0;
+}
+
 int Context::synchronize() {
+  if (masked_side && hipStreamSynchronize(masked_side) != hipSuccess) {
+    set_error("side stream synchronize failed");
+    return -5;
+  }
+  if (masked_main && hipStreamSynchronize(masked_main) != hipSuccess) {
+    set_error("stream synchronize failed");
+    return -5;
+  }
   if (side && hipStreamSynchronize(side) != hipSuccess) {
     set_error("side stream synchronize failed");
     return -5;
@@ -249,14 +330,17 @@ int Context::dispatch(const LaunchRecord& rec) {
     return 0;
   }
   if (queue) {
-    // behind the preemptible queue everything runs in program order on the one registered stream
-    if (rec.fn) queue->submit(rec);
+    // behind the preemptible queue everything runs in program order on one stream: the registered one, or
+    // the one that carries the compute-unit limit of the moment
+    if (rec.fn) queue->submit(rec, cu_limit > 0 ? masked_main : nullptr);
     return 0;
   }
+  hipStream_t main = main_stream();
   if (rec.op == kOpJoin) {
     if (side_dirty) {
+      hipStream_t s = cu_limit > 0 ? masked_side : side;
       hipEvent_t e = next_event();
-      if (!e || hipEventRecord(e, side) != hipSuccess || hipStreamWaitEvent(stream, e, 0) != hipSuccess) {
+      if (!e || hipEventRecord(e, s) != hipSuccess || hipStreamWaitEvent(main, e, 0) != hipSuccess) {
         set_error("join of the side stream failed");
         return -5;
       }
@@ -265,21 +349,89 @@ int Context::dispatch(const LaunchRecord& rec) {
     return 0;
   }
   if (rec.lane == 1) {
-    if (!side && hipStreamCreateWithFlags(&side, hipStreamNonBlocking) != hipSuccess) {
+    if (cu_limit == 0 && !side && hipStreamCreateWithFlags(&side, hipStreamNonBlocking) != hipSuccess) {
       set_error("hipStreamCreateWithFlags failed");
       return -5;
     }
+    hipStream_t s = cu_limit > 0 ? masked_side : side;
     if (rec.op == kOpLaunchAfter) {
       hipEvent_t e = next_event();
-      if (!e || hipEventRecord(e, stream) != hipSuccess || hipStreamWaitEvent(side, e, 0) != hipSuccess) {
+      if (!e || hipEventRecord(e, main) != hipSuccess || hipStreamWaitEvent(s, e, 0) != hipSuccess) {
         set_error("fork to the side stream failed");
         return -5;
       }
     }
     side_dirty = true;
-    return launch_now(side, rec);
+    return launch_now(s, rec);
   }
-  return launch_now(stream, rec);
+  return launch_now(main, rec);
+}
+
+// ---------------------------------------------------------------------------
+// compute-unit partitioning
+// ---------------------------------------------------------------------------
+namespace {
+std::mutex g_cu_mu;
+int g_cu_total = 0, g_cu_min = 1, g_cu_max = 0;
+std::map<std::pair<int, int>, hipStream_t> g_cu_streams;
+}  // namespace
+
+int cu_partition_init(int total_cus, int min_train_cus, int max_train_cus) {
+  std::lock_guard<std::mutex> lock(g_cu_mu);
+  if (total_cus <= 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+      set_error("cu_partition_init: cannot read the compute-unit count of the device");
+      return -5;
+    }
+    total_cus = n;
+  }
+  g_cu_total = total_cus;
+  g_cu_min = min_train_cus < 1 ? 1 : min_train_cus;
+  g_cu_max = (max_train_cus <= 0 || max_train_cus > total_cus) ? total_cus : max_train_cus;
+  if (g_cu_min > g_cu_max) {
+    set_error("cu_partition_init: min_train_cus exceeds max_train_cus");
+    return -22;
+  }
+  return 0;
+}
+
+int cu_partition_total() {
+  std::lock_guard<std::mutex> lock(g_cu_mu);
+  return g_cu_total;
+}
+
+int cu_partition_train_avail(int infer_required_cus) {
+  std::lock_guard<std::mutex> lock(g_cu_mu);
+  if (g_cu_total <= 0) return 0;
+  if (infer_required_cus < 0) infer_required_cus = 0;
+  int res = g_cu_total - infer_required_cus;
+  if (res < g_cu_min) res = g_cu_min;
+  if (res > g_cu_max) res = g_cu_max;
+  return res;
+}
+
+hipStream_t cu_partition_stream(int n_cus, int lane) {
+  std::lock_guard<std::mutex> lock(g_cu_mu);
+  if (g_cu_total <= 0 || n_cus <= 0 || n_cus > g_cu_total) {
+    set_error("cu_partition_stream: partitioning is not initialised or the share is out of range");
+    return nullptr;
+  }
+  auto key = std::make_pair(n_cus, lane);
+  auto it = g_cu_streams.find(key);
+  if (it != g_cu_streams.end()) return it->second;
+  // training keeps the highest-numbered compute units, the other tenant the lowest (sm_partition.cc:92-94)
+  const int words = (g_cu_total + 31) / 32;
+  std::vector<uint32_t> mask(static_cast<size_t>(words), 0u);
+  for (int cu = g_cu_total - n_cus; cu < g_cu_total; ++cu) mask[static_cast<size_t>(cu / 32)] |= 1u << (cu % 32);
+  hipStream_t s = nullptr;
+  if (hipExtStreamCreateWithCUMask(&s, static_cast<uint32_t>(words), mask.data()) != hipSuccess) {
+    set_error("hipExtStreamCreateWithCUMask failed");
+    return nullptr;
+  }
+  g_cu_streams[key] = s;
+  return s;
 }
 
 int submit(Context* ctx, const void* fn, dim3 grid, dim3 block, const void* args, size_t arg_bytes,

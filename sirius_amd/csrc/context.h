@@ -33,7 +33,12 @@ class LaunchQueue {
   LaunchQueue(const LaunchQueue&) = delete;
   LaunchQueue& operator=(const LaunchQueue&) = delete;
 
-  void submit(const LaunchRecord& rec);
+  // `on` (optional): the stream to launch on instead of the registered one (a stream restricted to a
+  // share of the compute units); the worker chains the streams with events whenever `on` changes,
+  // so program order holds across them.
+  void submit(const LaunchRecord& rec, hipStream_t on = nullptr);
+  // Queued in order with the launches: everything given to `to` afterwards waits for what `from` holds now.
+  void submit_dependency(hipStream_t from, hipStream_t to);
   // Erase every launch that has not been handed to the hardware queue yet.
   size_t clear();
   // Wait until everything submitted before this call has finished on the GPU.
@@ -50,7 +55,10 @@ class LaunchQueue {
  private:
   struct Item {
     bool is_sync = false;
+    bool is_dependency = false;
     uint64_t sync_ticket = 0;
+    hipStream_t on = nullptr;    // launch stream override / dependency source
+    hipStream_t to = nullptr;    // dependency target
     LaunchRecord rec;
   };
   struct Logged {
@@ -58,11 +66,13 @@ class LaunchQueue {
     hipEvent_t event;  // nullptr unless this command carries a sync point
   };
   void worker_loop();
-  void launch_one(const LaunchRecord& rec);
+  void launch_one(const LaunchRecord& rec, hipStream_t on);
+  void chain(hipStream_t from, hipStream_t to);
   void drain_log_until(size_t keep);
   hipEvent_t take_event();
 
   hipStream_t stream_;
+  hipStream_t launch_stream_;  // worker-private: where the last launch went
   const size_t queue_length_;
   const uint64_t sync_interval_;
   int device_ = 0;
@@ -99,6 +109,15 @@ class Context {
   hipStream_t stream;
   // second stream (default priority) for lane-1 launches of a replayed program; made on first use
   hipStream_t side = nullptr;
+  // Compute-unit share: with a limit in force the launches go to a pair of streams whose CU mask keeps
+  // the highest-numbered `cu_limit` compute units (made once per limit, kept for the process); 0 = no
+  // limit, launches go to `stream` / `side`.
+  int cu_limit = 0;
+  hipStream_t masked_main = nullptr, masked_side = nullptr;
+  int set_cu_limit(int n_cus);
+  hipStream_t main_stream() const { return cu_limit > 0 ? masked_main : stream; }
+  // everything given to `to` afterwards waits for what `from` holds now (direct or through the queue)
+  int depend(hipStream_t from, hipStream_t to);
   bool side_dirty = false;  // lane 1 was given work since the last join
   // recording state: the lane new launches are stamped with, and whether the next lane-1 launch
   // has to wait for lane 0
@@ -146,6 +165,15 @@ size_t queue_size_all_streams();
 void set_reject_calls(bool reject);
 bool query_reject_calls();
 void set_queue_shape(int queue_length, int sync_interval);
+
+// ---- compute-unit partitioning between training and a colocated tenant (the reference's SMPartitioner,
+// common/sm_partition.cc:26-112, with compute units in the place of TPCs) ----
+int cu_partition_init(int total_cus, int min_train_cus, int max_train_cus);  // total_cus <= 0: ask the device
+int cu_partition_total();
+// max(min, total - required) capped at max: what training may use while the other tenant needs `required`
+int cu_partition_train_avail(int infer_required_cus);
+// a stream (default priority) whose CU mask keeps the highest-numbered n compute units; lane 0 / 1
+hipStream_t cu_partition_stream(int n_cus, int lane);
 
 const char* last_error();
 

@@ -260,6 +260,22 @@ int tch_train_info_set_field(int id, int field, int value) {
   communicator()->update_field(id, static_cast<TrainInfoField>(field), value);
   return 0;
 }
+int tch_infer_required_cus_get(int device) {
+  NEED_COMM();
+  if (device < 0 || device >= kMaxDeviceNum) return fail("bad device");
+  return communicator()->infer_required_cus(device);
+}
+int tch_infer_required_cus_set(int device, int n) {
+  NEED_COMM();
+  if (device < 0 || device >= kMaxDeviceNum || n < 0) return fail("bad device or compute-unit count");
+  communicator()->set_infer_required_cus(device, n);
+  return 0;
+}
+int tch_infer_required_cus_add(int device, int delta) {
+  NEED_COMM();
+  if (device < 0 || device >= kMaxDeviceNum) return fail("bad device");
+  return communicator()->add_infer_required_cus(device, delta);
+}
 int tch_train_info_is_valid(int id) {
   NEED_COMM();
   if (id < 0 || id >= kMaxDeviceNum) return fail("bad board slot");

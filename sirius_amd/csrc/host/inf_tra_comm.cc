@@ -65,6 +65,7 @@ InfTraCommunicator* InfTraCommunicator::create(bool is_server, bool cleanup, int
       init_shared_mutex(&l->train_info_mu[i]);
       memset(&l->train_info[i], 0, sizeof(TrainInfo));
       l->train_info[i].train_pid = -1;
+      l->infer_required_cus[i] = 0;
     }
     seg->mark_ready();
   } else if (c->layout_->train_world_size < train_world_size) {

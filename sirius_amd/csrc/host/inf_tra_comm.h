@@ -87,6 +87,9 @@ struct InfTraLayout {
   ShmMsgQueue mq[kNumDirection][kMaxDeviceNum];
   pthread_mutex_t train_info_mu[kMaxDeviceNum];
   TrainInfo train_info[kMaxDeviceNum];
+  // compute units the inference side wants for itself on each device, read by the trainer before it
+  // launches (the tpc_datas[...].infer_required_tpc_num of the reference, common/sm_partition.cc:60-76)
+  int infer_required_cus[kMaxDeviceNum];
 };
 
 class InfTraCommunicator {
@@ -122,6 +125,12 @@ class InfTraCommunicator {
   std::vector<int> get_field_vec(TrainInfoField f);
   void update_field_vec(TrainInfoField f, const std::vector<int>& values);
   std::vector<pid_t> train_pids();
+  // ---- compute-unit demand of the inference side (relaxed atomics on the shared int) ----
+  int infer_required_cus(int device) { return __atomic_load_n(&layout_->infer_required_cus[device], __ATOMIC_RELAXED); }
+  void set_infer_required_cus(int device, int n) { __atomic_store_n(&layout_->infer_required_cus[device], n, __ATOMIC_RELAXED); }
+  int add_infer_required_cus(int device, int delta) {
+    return __atomic_add_fetch(&layout_->infer_required_cus[device], delta, __ATOMIC_RELAXED);
+  }
 
  private:
   InfTraCommunicator() = default;

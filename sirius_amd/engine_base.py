@@ -80,7 +80,19 @@ class EngineBase:
         engine hook does with EngineColocateAdjustL1Exception (csrc/mem_tagging.cc:54-58)."""
         self._cut_exception = exc_type
 
+    def set_cu_share_provider(self, fn):
+        """fn() -> compute units training may use right now (0 = all); asked before every launch segment,
+        as the reference sets the TPC mask of the training stream before each launch
+        (common/sm_partition.cc:108-112)."""
+        self._cu_share = fn
+
+    def _apply_cu_share(self):
+        fn = getattr(self, "_cu_share", None)
+        if fn is not None:
+            self.ctx.set_cu_limit(fn())
+
     def _run_plan(self, p):
+        self._apply_cu_share()
         if self._hook is None:
             cut = self.ctx.run(p.prog)
         else:
@@ -89,6 +101,7 @@ class EngineBase:
                 cut = self.ctx.run(p.prog, first, idx) or cut
                 first = idx
                 self._hook(phase, name)
+                self._apply_cu_share()
                 if cut and self._cut_exception is not None:
                     break
             if first < len(p.prog) and not (cut and self._cut_exception is not None):

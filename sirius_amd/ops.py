@@ -121,6 +121,14 @@ class Context:
     def join(self):
         check(lib().tch_context_join(self.handle), "tch_context_join")
 
+    def set_cu_limit(self, n_cus):
+        """From the next launch on, run on at most n_cus compute units (0 lifts the limit); needs
+        tch_cu_partition_init.  Ordered with what was launched before."""
+        check(lib().tch_context_set_cu_limit(self.handle, int(n_cus)), "tch_context_set_cu_limit")
+
+    def cu_limit(self):
+        return int(lib().tch_context_get_cu_limit(self.handle))
+
     def profile(self, program, reps=1):
         """Per-kernel HIP-event timing of `reps` replays: list of dicts with name, total_ms,
         launches, work (algorithmic flops or bytes, summed) and work_is_bytes."""

@@ -11,7 +11,7 @@ import threading
 import time
 import weakref
 
-from .._lib import CtrlMsg, TorchColHipError, check_host, lib
+from .._lib import CtrlMsg, TorchColHipError, check, check_host, lib
 
 # ---------------------------------------------------------------------------------- enums
 
@@ -437,13 +437,42 @@ def GetNcclStreams():
     return []
 
 
-def SMPartitionInit(stream):
-    """csrc/init.cc:43-71: compute-unit partitioning between the two tenants is not part of this
-    path; the call is accepted so the reference's stream registration sequence runs unchanged."""
-    return None
+_cu_partition = {"on": False}
+
+
+def SMPartitionInit(stream=None, min_train_cus=8, max_train_cus=0, total_cus=0):
+    """csrc/init.cc:43-71: from now on the training launches are confined to the compute units the inference
+    side leaves (its demand sits on the shared board, common/sm_partition.cc:60-76).  Compute units take the
+    place of the reference's TPCs; the confinement is a CU-masked stream per share instead of a mask per launch.
+    `stream` is accepted for the reference's call shape (the engines' contexts pick the masked streams)."""
+    check(lib().tch_cu_partition_init(int(total_cus), int(min_train_cus), int(max_train_cus)), "tch_cu_partition_init")
+    _cu_partition["on"] = True
+
+
+def sm_partition_enabled():
+    return _cu_partition["on"]
+
+
+def sm_partition_total():
+    return int(lib().tch_cu_partition_total())
+
+
+def set_infer_required_cus(n, device=0):
+    """SMPartitioner::SetInferRequiredTpcNum (the inference side's call; the stand-in peer uses it)."""
+    check_host(lib().tch_infer_required_cus_set(int(device), int(n)), "tch_infer_required_cus_set")
+
+
+def get_train_avail_cus(device=0):
+    """SMPartitioner::GetTrainAvailTpcNum: what training may use right now."""
+    required = lib().tch_infer_required_cus_get(int(device))
+    return int(lib().tch_cu_partition_train_avail(max(0, int(required))))
 
 
 def monitor_sm_partition(interval):
+    """The reference starts a thread that logs the partition every `interval` seconds (csrc/init.cc:60-70);
+    here: one line with the state of the moment."""
+    if _cu_partition["on"]:
+        info(f"[CU partition] total {sm_partition_total()} train may use {get_train_avail_cus()}")
     return None
 
 

@@ -36,6 +36,10 @@ class DebugServer:
     def infer_exit(self, batch_size: int):
         return self._send(CtrlEvent.kInferExit, batch_size)
 
+    # -- compute units the inference side wants for itself (SMPartitioner::SetInferRequiredTpcNum)
+    def set_infer_required_cus(self, n: int, device: int = 0):
+        _C.set_infer_required_cus(n, device)
+
     # -- task switching (the controller's pair of commands, server/control/controller.cc:207-260)
     def interrupt_train(self):
         cmd_id = self._cmd_ids[CtrlEvent.kInterruptTrain] = self._cmd_ids.get(CtrlEvent.kInterruptTrain, 0) + 1

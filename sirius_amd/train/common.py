@@ -22,7 +22,7 @@ def cleanup():
 
 class PeerScript:
     """Stand-in inference server: `at` maps a micro-batch index to ('l1' | 'l2' | 'exit', batch size) or to
-    ('switch', milliseconds until the resume).
+    ('switch', milliseconds until the resume), or to ('cus', compute units inference wants for itself).
     The command is sent from a side thread `delay_ms` after the micro-batch began, so that it lands
     while kernels are queued, as a real request would."""
 
@@ -50,13 +50,20 @@ class PeerScript:
                 self.server.resume_train()
                 self.sent.append((torch_col.get_unix_timestamp_us(), "resume", 0))
                 return
-            {"l1": self.server.colocate_l1, "l2": self.server.colocate_l2,
-             "exit": self.server.infer_exit}[kind](bs)
+            {"l1": self.server.colocate_l1, "l2": self.server.colocate_l2, "exit": self.server.infer_exit,
+             "cus": self.server.set_infer_required_cus}[kind](bs)
             self.sent.append((t, kind, bs))
         threading.Thread(target=fire, daemon=True).start()
 
     def stop(self):
         self.server.stop()
+
+
+def attach_cu_partition(model):
+    """With COLTRAIN_DYNAMIC_SM_PARTITION the engine asks the shared board before every launch segment how
+    many compute units training may use (csrc/init.cc:43-71 + common/sm_partition.cc:96-112)."""
+    if torch_col.sm_partition_enabled():
+        model.set_cu_share_provider(torch_col.get_train_avail_cus)
 
 
 def run_epochs(tag, model, iter_train_fn, col_ctrl, train_mode, num_epoch: int, batch_size: int,

@@ -15,7 +15,7 @@ import torch
 from .. import torch_col
 from ..swin import SwinEngine
 from ..torch_col import MemoryPool, dynamic_batch
-from .common import PeerScript, run_epochs, setup
+from .common import PeerScript, attach_cu_partition, run_epochs, setup
 
 
 def train(num_epoch: int, batch_size: int, global_batch_size: Optional[int] = None, dataset_size: int = 1000,
@@ -35,6 +35,7 @@ def train(num_epoch: int, batch_size: int, global_batch_size: Optional[int] = No
 
     col_ctrl = torch_col.create_colocate_ctrl(train_mode, hook_mode, num_epoch, batch_size)
     col_ctrl.register_pytorch_hook([model])
+    attach_cu_partition(model)
     enable_grad_accumulator = global_batch_size is not None or col_ctrl.train_mode.is_colocate()
     checkpoint_micro_batch = col_ctrl.train_mode.is_kill_batch()
     train_dataset, batch_manager = torch_col.init_dynamic_batch(

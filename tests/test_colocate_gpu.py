@@ -145,7 +145,8 @@ def _handover(tc, monkeypatch, tmp_path, hook_mode):
     sizes = []
     orig = tc.Trainer.train_one_epoch
     try:
-        out = script.train(1, 64, global_batch_size=None, dataset_size=64 * 8, dtype=torch.bfloat16,
+        # long enough that plenty of samples are left when the peer leaves, however fast the steps are
+        out = script.train(1, 64, global_batch_size=None, dataset_size=64 * 16, dtype=torch.bfloat16,
                            peer=peer, num_distinct_samples=64, **SMALL)
     finally:
         peer.stop()
@@ -159,7 +160,7 @@ def test_handover_64_16_64_on_gpu(clean_runtime, monkeypatch, tmp_path, hook_mod
     out, peer = _handover(tc, monkeypatch, tmp_path, hook_mode)
     trainer, model, ctrl = out["trainer"], out["model"], out["ctrl"]
     stat = trainer.get_last_epoch_stat()
-    assert stat.finished_sample == 64 * 8                      # every sample trained exactly once
+    assert stat.finished_sample == 64 * 16                     # every sample trained exactly once
     assert [k for _, k, _ in peer.sent] == ["l1", "exit"]
     req, fin = tc.get_adjust_request_time_stamp(), tc.get_adjust_done_time_stamp()
     assert len(req) == 1 and len(fin) == 1
@@ -174,7 +175,7 @@ def test_handover_64_16_64_on_gpu(clean_runtime, monkeypatch, tmp_path, hook_mod
     # 64 -> 16 -> 64; the first batch after the peer left is what remains of its global batch (64 or 48)
     assert sizes[0] == 64 and 16 in sizes and sizes[-1] > 16
     assert sum(s for r, s in zip([r for r in rows if r["name"].startswith("batch_0")], sizes)
-               if r["tag"] == "finish") == 64 * 8
+               if r["tag"] == "finish") == 64 * 16
     sd = model.state_dict()
     assert all(torch.isfinite(v).all() for v in sd.values())
     assert tc.GetXQueueSizeAllStreams() == 0
@@ -295,4 +296,42 @@ def test_task_switch_interrupt_and_resume_on_gpu(clean_runtime, monkeypatch, tmp
     assert 0 <= (done[0] - t_int) / 1e3 < 50.0, "interrupt -> done within the handover bound"
     assert resumed[0] >= t_res and (resumed[0] - t_int) / 1e3 >= pause_ms
     assert all(torch.isfinite(v).all() for v in out["model"].state_dict().values())
+    assert tc.GetXQueueSizeAllStreams() == 0
+
+
+def test_dynamic_compute_unit_partition_under_the_colocation_protocol(clean_runtime, monkeypatch, tmp_path):
+    """COLTRAIN_DYNAMIC_SM_PARTITION=1 (the reference's dynamic SM partition, csrc/init.cc:43-71): the stream is
+    registered for preemption (launches pass through the queue) and the engine follows the demand the peer writes
+    on the board: 192 compute units wanted -> training on the rest, demand withdrawn -> all of them again.
+    Every sample is trained; the shares the engine asked for are the expected ones.
+    (The model lives in pool memory: everything that reads it comes before the runtime is shut down, which
+    unmaps the pool.)"""
+    tc = clean_runtime
+    from sirius_amd.train import resnet152 as script
+    env = {"COLTRAIN_MODE": "colocate-l1", "COLTRAIN_HOOK_MODE": "xsched-sync", "COLTRAIN_USE_XSCHED": "1",
+           "COLTRAIN_HAS_INFER_SERVER": "1", "COLTRAIN_USE_SHARED_TENSOR": "1", "COLTRAIN_DYNAMIC_SM_PARTITION": "1",
+           "COLTRAIN_SHARED_TENSOR_POOL_GB": "2", "COLTRAIN_PROFILE_LOG_PATH": str(tmp_path / "train-profile.csv")}
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    seen = []
+    real = tc.get_train_avail_cus
+
+    def spy(device=0):
+        n = real(device)
+        seen.append(n)
+        return n
+    monkeypatch.setattr(tc, "get_train_avail_cus", spy)
+    peer = script.PeerScript({2: ("cus", 192), 5: ("cus", 0)}, delay_ms=0.5)
+    try:
+        out = script.train(1, 16, dataset_size=16 * 8, dtype=torch.bfloat16, peer=peer, num_distinct_samples=32,
+                           **SMALL)
+    finally:
+        peer.stop()
+    total = tc.sm_partition_total()
+    assert out["trainer"].get_last_epoch_stat().finished_sample == 16 * 8
+    assert set(seen) == {total, total - 192}, set(seen)
+    first_low = seen.index(total - 192)
+    assert seen[0] == total and total in seen[first_low:], "all compute units before the demand and after it is withdrawn"
+    assert all(torch.isfinite(v).all() for v in out["model"].state_dict().values())
+    out["model"].ctx.set_cu_limit(0)
     assert tc.GetXQueueSizeAllStreams() == 0
