@@ -281,6 +281,179 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(ApplyArgs p) {
   }
 }
 
+// Finalize + apply in ONE launch, for layers whose sums come in few rows (the 14x14 and 7x7 stages, where a
+// launch costs more than the work): a workgroup owns 64 channels and a slab of rows; it first sums the
+// per-tile partials of its 64 channels itself (every workgroup of a column block repeats that sum, in the
+// same fixed order, from L2: row_blocks x 512 bytes), then applies.  The workgroups of slab 0 also write the
+// per-channel outputs (saved statistics, running statistics / dgamma, dbeta).
+constexpr int kFusedCols = 64;
+constexpr int kFusedMaxRowBlocks = 256;
+
+struct FinApplyArgs {
+  const float* partial;
+  int row_blocks, C;
+  int64_t rows;
+  const float* gamma;
+  const float* beta;      // forward
+  float* running_mean;    // forward (may be null)
+  float* running_var;
+  float* save_mean;       // forward: written   backward: read
+  float* save_invstd;
+  float* dgamma;          // backward
+  float* dbeta;
+  float momentum, eps;
+  int accumulate;
+  const void* a;          // forward: x         backward: g
+  const void* b;          // forward: residual (may be null)   backward: x
+  void* out;
+  int relu;
+  int rows_per_slab;
+};
+
+template <typename T, int BWD>
+__global__ __launch_bounds__(256) void bn_fin_apply_kernel(FinApplyArgs p) {
+  constexpr int E = Elem<T>::kPerChunk;
+  constexpr int CPR = kFusedCols / E;     // chunks of this workgroup's channels per row
+  constexpr int RPP = 256 / CPR;          // rows per pass
+  __shared__ double red[8][32][4];
+  __shared__ float coef[3][kFusedCols];
+  const int tid = threadIdx.x;
+  const int c0 = blockIdx.x * kFusedCols;
+  {
+    const int pr = tid & 31, part = tid >> 5;
+    double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
+    constexpr int U = 8;
+    for (int b = part; b < p.row_blocks; b += 8 * U) {
+      float4 v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int bb = b + 8 * u;
+        v[u] = bb < p.row_blocks
+                   ? *reinterpret_cast<const float4*>(p.partial + (static_cast<int64_t>(bb) * p.C + c0 + 2 * pr) * 2)
+                   : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        s0 += v[u].x;
+        q0 += v[u].y;
+        s1 += v[u].z;
+        q1 += v[u].w;
+      }
+    }
+    red[part][pr][0] = s0;
+    red[part][pr][1] = q0;
+    red[part][pr][2] = s1;
+    red[part][pr][3] = q1;
+  }
+  __syncthreads();
+  if (tid < kFusedCols) {
+    const int c = c0 + tid;
+    double s = 0.0, q = 0.0;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      s += red[k][tid >> 1][(tid & 1) * 2];
+      q += red[k][tid >> 1][(tid & 1) * 2 + 1];
+    }
+    const double n = static_cast<double>(p.rows);
+    const bool writer = blockIdx.y == 0;
+    if (!BWD) {
+      const double mean = s / n;
+      double var = q / n - mean * mean;
+      if (var < 0.0) var = 0.0;
+      const float invstd = 1.0f / sqrtf(static_cast<float>(var) + p.eps);
+      const float sc = p.gamma[c] * invstd;
+      coef[0][tid] = sc;
+      coef[1][tid] = p.beta[c] - static_cast<float>(mean) * sc;
+      if (writer) {
+        p.save_mean[c] = static_cast<float>(mean);
+        p.save_invstd[c] = invstd;
+        if (p.running_mean) {
+          const double unbiased = p.rows > 1 ? var * n / (n - 1.0) : var;
+          p.running_mean[c] = (1.f - p.momentum) * p.running_mean[c] + p.momentum * static_cast<float>(mean);
+          p.running_var[c] = (1.f - p.momentum) * p.running_var[c] + p.momentum * static_cast<float>(unbiased);
+        }
+      }
+    } else {
+      const double invstd = p.save_invstd[c];
+      const double scale = static_cast<double>(p.gamma[c]) * invstd;
+      const double cb = -scale * invstd * (q / n);
+      const double cz = -scale * (s / n) - cb * p.save_mean[c];
+      coef[0][tid] = static_cast<float>(scale);
+      coef[1][tid] = static_cast<float>(cb);
+      coef[2][tid] = static_cast<float>(cz);
+      if (writer) {
+        const float db = static_cast<float>(s), dg = static_cast<float>(q);
+        p.dbeta[c] = p.accumulate ? p.dbeta[c] + db : db;
+        p.dgamma[c] = p.accumulate ? p.dgamma[c] + dg : dg;
+      }
+    }
+  }
+  __syncthreads();
+
+  const int tx = tid % CPR, ty = tid / CPR;
+  float k0[E], k1[E], k2[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    k0[e] = coef[0][tx * E + e];
+    k1[e] = coef[1][tx * E + e];
+    k2[e] = BWD ? coef[2][tx * E + e] : 0.f;
+  }
+  const int64_t cc = p.C / E;                    // chunks per full row
+  const int64_t col_chunk = c0 / E + tx;
+  const int64_t r0 = static_cast<int64_t>(blockIdx.y) * p.rows_per_slab;
+  int64_t r1 = r0 + p.rows_per_slab;
+  if (r1 > p.rows) r1 = p.rows;
+  for (int64_t r = r0 + ty; r < r1; r += RPP) {
+    const int64_t i = r * cc + col_chunk;
+    Chunk ca;
+    ca.u = static_cast<const uint4*>(p.a)[i];
+    float va[E], vo[E];
+    chunk_to_float<T>(ca, va);
+    if (BWD) {
+      Chunk cx;
+      cx.u = static_cast<const uint4*>(p.b)[i];
+      float vx[E];
+      chunk_to_float<T>(cx, vx);
+#pragma unroll
+      for (int e = 0; e < E; ++e) vo[e] = k0[e] * va[e] + k1[e] * vx[e] + k2[e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < E; ++e) vo[e] = va[e] * k0[e] + k1[e];
+      if (p.b) {
+        Chunk cr;
+        cr.u = static_cast<const uint4*>(p.b)[i];
+        float vr[E];
+        chunk_to_float<T>(cr, vr);
+#pragma unroll
+        for (int e = 0; e < E; ++e) vo[e] += vr[e];
+      }
+      if (p.relu) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) vo[e] = vo[e] > 0.f ? vo[e] : 0.f;
+      }
+    }
+    static_cast<uint4*>(p.out)[i] = float_to_chunk<T>(vo).u;
+  }
+}
+
+// rows per slab so that the grid has about 1024 workgroups, at least 32 rows each
+int fused_rows_per_slab(int64_t rows, int C) {
+  const int col_blocks = C / kFusedCols;
+  int64_t slabs = 1024 / col_blocks;
+  if (slabs < 1) slabs = 1;
+  int64_t rps = (rows + slabs - 1) / slabs;
+  if (rps < 32) rps = 32;
+  return static_cast<int>(rps);
+}
+
+bool use_fused_finalize() {
+  static const bool on = [] {
+    const char* e = getenv("TCH_BN_FUSED_FINALIZE");
+    return !e || atoi(e) != 0;
+  }();
+  return on;
+}
+
 struct Geometry {
   int cc, ccb, col_blocks, rowlanes, row_blocks;
   int64_t rows_per_block;
@@ -417,6 +590,16 @@ int bn_fwd_train_partials(Context* ctx, int dtype, const void* x, void* y, const
                 "bn_fwd_train_partials: null tensor");
   TCH_CHECK_ARG(row_blocks >= 1, "bn_fwd_train_partials: no partial statistics");
   TCH_CHECK_ARG((running_mean == nullptr) == (running_var == nullptr), "bn_fwd_train: running stats come in pairs");
+  const double eb0 = dtype == kBF16 ? 2.0 : 4.0;
+  if (use_fused_finalize() && row_blocks <= kFusedMaxRowBlocks && C % kFusedCols == 0) {
+    FinApplyArgs a{partial, row_blocks, C,        rows,    gamma,   beta, running_mean, running_var,
+                   save_mean, save_invstd, nullptr, nullptr, momentum, eps,  0,            x,
+                   residual, y,           relu,    fused_rows_per_slab(rows, C)};
+    const dim3 grid(C / kFusedCols, static_cast<unsigned>((rows + a.rows_per_slab - 1) / a.rows_per_slab));
+    const double bytes = static_cast<double>(rows) * C * eb0 * (residual ? 3.0 : 2.0);
+    return dtype == kBF16 ? launch(ctx, bn_fin_apply_kernel<bf16, 0>, grid, dim3(256), a, "bn_fin_apply_kernel<bf16,fwd>", bytes, 1)
+                          : launch(ctx, bn_fin_apply_kernel<float, 0>, grid, dim3(256), a, "bn_fin_apply_kernel<f32,fwd>", bytes, 1);
+  }
   Geometry g = geometry(rows, C, dtype);
   float* scale = scratch;
   float* shift = scratch + C;
@@ -472,6 +655,15 @@ int bn_bwd_partials(Context* ctx, int dtype, const void* g, const void* x, void*
   TCH_CHECK_ARG(g && x && dx && gamma && save_mean && save_invstd && dgamma && dbeta && partial && scratch,
                 "bn_bwd_partials: null tensor");
   TCH_CHECK_ARG(row_blocks >= 1, "bn_bwd_partials: no partial sums");
+  if (use_fused_finalize() && row_blocks <= kFusedMaxRowBlocks && C % kFusedCols == 0) {
+    FinApplyArgs a{partial, row_blocks, C, rows, gamma, nullptr, nullptr, nullptr, const_cast<float*>(save_mean),
+                   const_cast<float*>(save_invstd), dgamma, dbeta, 0.f, 0.f, accumulate, g, x, dx, 0,
+                   fused_rows_per_slab(rows, C)};
+    const dim3 grid(C / kFusedCols, static_cast<unsigned>((rows + a.rows_per_slab - 1) / a.rows_per_slab));
+    const double bytes = static_cast<double>(rows) * C * (dtype == kBF16 ? 2.0 : 4.0) * 3.0;
+    return dtype == kBF16 ? launch(ctx, bn_fin_apply_kernel<bf16, 1>, grid, dim3(256), a, "bn_fin_apply_kernel<bf16,bwd>", bytes, 1)
+                          : launch(ctx, bn_fin_apply_kernel<float, 1>, grid, dim3(256), a, "bn_fin_apply_kernel<f32,bwd>", bytes, 1);
+  }
   Geometry geo = geometry(rows, C, dtype);
   float* coef = scratch;
   BwdFinalizeArgs f{partial, row_blocks, C, rows, gamma, save_mean, save_invstd, dgamma, dbeta, coef, accumulate};
