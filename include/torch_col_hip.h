@@ -275,6 +275,20 @@ int tch_batched_gemm(tch_context* ctx, int dtype, const void* a, const void* b, 
                      int batch_inner, int64_t a_bo, int64_t a_bi, int64_t b_bo, int64_t b_bi, int64_t c_bo, int64_t c_bi,
                      float alpha, int accumulate, int causal);
 
+/* Attention of the GPT-2 step as one fused pass: o = softmax(scale * q k^T [+ causal mask]) v per head, the
+ * [T, T] scores never leave the chip (what transformers' GPT2Attention computes inside train/gpt2.py:26 with
+ * the benchmark's dropout of 0).  bf16 only (dtype 1), heads 64 wide, T a multiple of 128.  q, k, v (and dq, dk,
+ * dv) share one layout: element (b, t, h, d) at b * qkv_bs + t * qkv_rs + 64 h + d, so the three may be views of
+ * one packed [B, T, 3C] projection; o and dout likewise with o_bs / o_rs.  lse [B * H][T] fp32 receives the
+ * natural log-sum-exp of the scaled scores; the backward reads it back, fills delta [B * H][T] (row sums of
+ * dout * o) and writes dq, dk, dv in two launches without atomics. */
+int tch_flash_attn_fwd(tch_context* ctx, int dtype, const void* q, const void* k, const void* v, void* o, float* lse,
+                       int B, int H, int T, int64_t qkv_rs, int64_t qkv_bs, int64_t o_rs, int64_t o_bs, float scale,
+                       int causal);
+int tch_flash_attn_bwd(tch_context* ctx, int dtype, const void* q, const void* k, const void* v, const void* o,
+                       const void* dout, const float* lse, float* delta, void* dq, void* dk, void* dv, int B, int H,
+                       int T, int64_t qkv_rs, int64_t qkv_bs, int64_t o_rs, int64_t o_bs, float scale, int causal);
+
 /* Swin-B data movement (train/swin_b_tiny.py:8-19,116-131; patch merging and shift as in torchvision's swin_b,
  * train/swin_b.py:38).
  * reverse == 0: dst[windows of window x window tokens] = roll(src[B,H,W,C], -shift) partitioned;

@@ -69,6 +69,19 @@ def attn_softmax_bwd(scores, dprobs, scale, bias=None, mask=None, causal=False):
     return ds
 
 
+def attention(q, k, v, scale, causal=False):
+    """q, k, v [B, heads, T, d] -> (context [B, heads, T, d], log-sum-exp of the scaled scores [B, heads, T]):
+    the scores / mask / softmax / context chain of transformers' GPT2Attention as train/gpt2.py:26 runs it."""
+    z = attn_logits(q.float() @ k.float().transpose(-1, -2), scale, causal=causal)
+    return torch.softmax(z, dim=-1) @ v.float(), torch.logsumexp(z, dim=-1)
+
+
+def attention_bwd(q, k, v, dout, scale, causal=False):
+    qs, ks, vs = (t.float().clone().requires_grad_(True) for t in (q, k, v))
+    o, _ = attention(qs, ks, vs, scale, causal)
+    return torch.autograd.grad(o, (qs, ks, vs), dout.float())
+
+
 def adamw(param, grads, lr, beta1, beta2, eps, weight_decay):
     """torch.optim.AdamW over one flat parameter, one step per entry of `grads`."""
     p = param.clone().requires_grad_(True)

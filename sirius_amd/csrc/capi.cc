@@ -292,6 +292,19 @@ int tch_batched_gemm(tch_context* ctx, int dtype, const void* a, const void* b, 
                       b_bo, b_bi, c_bo, c_bi, alpha, accumulate, causal);
 }
 
+int tch_flash_attn_fwd(tch_context* ctx, int dtype, const void* q, const void* k, const void* v, void* o, float* lse,
+                       int B, int H, int T, int64_t qkv_rs, int64_t qkv_bs, int64_t o_rs, int64_t o_bs, float scale,
+                       int causal) {
+  return flash_attn_fwd(C(ctx), dtype, q, k, v, o, lse, B, H, T, qkv_rs, qkv_bs, o_rs, o_bs, scale, causal);
+}
+
+int tch_flash_attn_bwd(tch_context* ctx, int dtype, const void* q, const void* k, const void* v, const void* o,
+                       const void* dout, const float* lse, float* delta, void* dq, void* dk, void* dv, int B, int H,
+                       int T, int64_t qkv_rs, int64_t qkv_bs, int64_t o_rs, int64_t o_bs, float scale, int causal) {
+  return flash_attn_bwd(C(ctx), dtype, q, k, v, o, dout, lse, delta, dq, dk, dv, B, H, T, qkv_rs, qkv_bs, o_rs, o_bs,
+                        scale, causal);
+}
+
 int tch_conv2d_fwd_bn(tch_context* ctx, int dtype, const void* x, const void* w, void* y, int N, int H, int W, int Cc,
                       int K, int R, int S, int stride, int pad, int tile_cfg, int c_logical, float* bn_partial,
                       int* counters, const float* gamma, const float* beta, float* running_mean, float* running_var,

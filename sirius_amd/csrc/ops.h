@@ -130,6 +130,14 @@ int batched_gemm(Context* ctx, int dtype, const void* a, const void* b, void* c,
                  int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t ldc, int batch_outer, int batch_inner, int64_t a_bo,
                  int64_t a_bi, int64_t b_bo, int64_t b_bi, int64_t c_bo, int64_t c_bi, float alpha, int accumulate, int causal);
 
+// flash_attn.hip -- attention without the score matrix (bf16, heads 64 wide, T a multiple of 128); head h of
+// sample b starts at column 64 h of row b * bs; lse and delta are [B * H][T] fp32
+int flash_attn_fwd(Context* ctx, int dtype, const void* q, const void* k, const void* v, void* o, float* lse, int B,
+                   int H, int T, int64_t qkv_rs, int64_t qkv_bs, int64_t o_rs, int64_t o_bs, float scale, int causal);
+int flash_attn_bwd(Context* ctx, int dtype, const void* q, const void* k, const void* v, const void* o, const void* dout,
+                   const float* lse, float* delta, void* dq, void* dk, void* dv, int B, int H, int T, int64_t qkv_rs,
+                   int64_t qkv_bs, int64_t o_rs, int64_t o_bs, float scale, int causal);
+
 // pool.hip
 int maxpool_fwd(Context* ctx, int dtype, const void* x, void* y, int32_t* index, int N, int H, int W, int C, int ksize,
                 int stride, int pad);

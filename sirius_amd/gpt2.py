@@ -9,8 +9,10 @@ recorded program of hand-written kernels per batch size:
   output head on MFMA); bf16 mode keeps a flat bf16 shadow the kernels read;
 * the vocabulary is padded to a multiple of 128 rows of zeros (they never receive a gradient), so the
   output head and its two gradients run on the direct-to-LDS GEMM kernel;
-* attention is four batched strided GEMMs on the packed [B, T, 3, heads, head_dim] projection and a
-  causal softmax over materialised [B, heads, T, T] scores (kept for the backward);
+* attention reads the packed [B, T, 3, heads, head_dim] projection in place: in bf16 with heads 64 wide
+  and a sequence length that is a multiple of 128 it is one fused launch forward (scores never leave the
+  chip, the log-sum-exp is kept) and two backward; otherwise batched strided GEMMs and a causal softmax
+  over materialised [B, heads, T, T] scores (kept for the backward);
 * backward is written out by hand; the gradient that bypasses a LayerNorm is added inside the
   LayerNorm backward; the token embedding receives the head's weight gradient and then the scattered
   embedding gradient (tied weights);
@@ -42,12 +44,13 @@ class _Plan:
 class GPT2Engine(EngineBase):
     def __init__(self, vocab=50257, n_pos=1024, n_embd=768, n_layer=12, n_head=12, seq_len=1024, dtype=torch.bfloat16,
                  optimizer="adamw", lr=1e-3, weight_decay=0.01, betas=(0.9, 0.999), eps=1e-8, momentum=0.9,
-                 stream=None, allocator=None, overlap_wgrad=True):
+                 stream=None, allocator=None, overlap_wgrad=True, fused_attention=True):
         self._init_engine(dtype, stream, allocator)
         # weight and bias gradients depend only on a saved activation and on a gradient that stays put until
         # the layer is done: recorded on a second lane, they run beside the data-gradient chain; the lanes
         # meet at the end of every layer, before its gradient buffers are handed round again
         self.overlap_wgrad = overlap_wgrad
+        self.fused_attention = fused_attention
         assert n_embd % n_head == 0 and n_embd % 8 == 0 and seq_len <= n_pos
         assert optimizer in ("adamw", "sgd")
         self.vocab, self.n_pos, self.C, self.n_layer, self.n_head = vocab, n_pos, n_embd, n_layer, n_head
@@ -260,6 +263,8 @@ class GPT2Engine(EngineBase):
         qkv_row, qkv_b = 3 * C, (T * 3 * C, D)
         s_b, o_b = (H * T * T, T * T), (T * C, D)
         scale = 1.0 / math.sqrt(D)
+        # one fused pass per direction where the kernel's shape limits hold; the three-launch chain otherwise
+        fused = self.fused_attention and self.dtype == torch.bfloat16 and D == 64 and T % 128 == 0
 
         prog = ops.Program()
         marks = []
@@ -280,13 +285,19 @@ class GPT2Engine(EngineBase):
                 ln_fwd(pre + "ln_1", 2 * i, h, a)
                 lin_fwd(pre + "attn.c_attn", a, qkv)
                 flat = qkv.view(-1)
-                P = act(B, H, T, T)
-                ops.batched_gemm(ctx, flat, flat[C:], P, T, T, D, (qkv_row, 1), (qkv_row, 1), T, (B, H), qkv_b, qkv_b, s_b,
-                                 causal=1)
-                ops.attn_softmax_fwd(ctx, P, P, scale, causal=True)
                 o = act(R, C)
-                ops.batched_gemm(ctx, P, flat[2 * C:], o, T, D, T, (T, 1), (1, qkv_row), C, (B, H), s_b, qkv_b, o_b,
-                                 causal=2)
+                if fused:
+                    # P is the log-sum-exp here: all the backward needs to rebuild the probabilities
+                    P = act(B * H, T, dtype=torch.float32)
+                    ops.flash_attn_fwd(ctx, flat, flat[C:], flat[2 * C:], o.view(-1), P, B, H, T, (qkv_row, T * qkv_row),
+                                       (C, T * C), scale, causal=True)
+                else:
+                    P = act(B, H, T, T)
+                    ops.batched_gemm(ctx, flat, flat[C:], P, T, T, D, (qkv_row, 1), (qkv_row, 1), T, (B, H), qkv_b, qkv_b,
+                                     s_b, causal=1)
+                    ops.attn_softmax_fwd(ctx, P, P, scale, causal=True)
+                    ops.batched_gemm(ctx, P, flat[2 * C:], o, T, D, T, (T, 1), (1, qkv_row), C, (B, H), s_b, qkv_b, o_b,
+                                     causal=2)
                 h1 = act(R, C)
                 lin_fwd(pre + "attn.c_proj", o, h1, add=h)
                 m, f1, f2 = act(R, C), act(R, 4 * C), act(R, 4 * C)
@@ -310,7 +321,7 @@ class GPT2Engine(EngineBase):
             # ================= backward =================
             g_c = [act(R, C) for _ in range(4)]       # gradients of [R, C] tensors, handed round
             g_f1, g_f2, g_qkv = act(R, 4 * C), act(R, 4 * C), act(R, 3 * C)
-            dP = act(B, H, T, T)
+            dP = act(B * H, T, dtype=torch.float32) if fused else act(B, H, T, T)   # fused: the delta scratch
             d_hf, g = g_c[0], g_c[1]
             with side():
                 ops.conv2d_wgrad(ctx, as4(hf), as4(dlogits), self._view(self.grads, "transformer.wte.weight"), 1, 0,
@@ -331,15 +342,20 @@ class GPT2Engine(EngineBase):
                 ln_bwd(pre + "ln_2", 2 * i + 1, d_m, h1, g1, residual=g)
                 # attention
                 lin_bwd(pre + "attn.c_proj", o, g1, d_o)
-                ops.batched_gemm(ctx, P, d_o, gflat[2 * C:], T, D, T, (1, T), (1, C), qkv_row, (B, H), s_b, o_b, qkv_b,
-                                 causal=3)
-                ops.batched_gemm(ctx, d_o, flat[2 * C:], dP, T, T, D, (C, 1), (qkv_row, 1), T, (B, H), o_b, qkv_b, s_b,
-                                 causal=1)
-                ops.attn_softmax_bwd(ctx, P, dP, dP, scale, causal=True)
-                ops.batched_gemm(ctx, dP, flat[C:], gflat, T, D, T, (T, 1), (1, qkv_row), qkv_row, (B, H), s_b, qkv_b,
-                                 qkv_b, causal=2)
-                ops.batched_gemm(ctx, dP, flat, gflat[C:], T, D, T, (1, T), (1, qkv_row), qkv_row, (B, H), s_b, qkv_b,
-                                 qkv_b, causal=3)
+                if fused:
+                    ops.flash_attn_bwd(ctx, flat, flat[C:], flat[2 * C:], o.view(-1), d_o.view(-1), P, dP, gflat,
+                                       gflat[C:], gflat[2 * C:], B, H, T, (qkv_row, T * qkv_row), (C, T * C), scale,
+                                       causal=True)
+                else:
+                    ops.batched_gemm(ctx, P, d_o, gflat[2 * C:], T, D, T, (1, T), (1, C), qkv_row, (B, H), s_b, o_b, qkv_b,
+                                     causal=3)
+                    ops.batched_gemm(ctx, d_o, flat[2 * C:], dP, T, T, D, (C, 1), (qkv_row, 1), T, (B, H), o_b, qkv_b, s_b,
+                                     causal=1)
+                    ops.attn_softmax_bwd(ctx, P, dP, dP, scale, causal=True)
+                    ops.batched_gemm(ctx, dP, flat[C:], gflat, T, D, T, (T, 1), (1, qkv_row), qkv_row, (B, H), s_b, qkv_b,
+                                     qkv_b, causal=2)
+                    ops.batched_gemm(ctx, dP, flat, gflat[C:], T, D, T, (1, T), (1, qkv_row), qkv_row, (B, H), s_b, qkv_b,
+                                     qkv_b, causal=3)
                 d_a = d_m   # free again
                 lin_bwd(pre + "attn.c_attn", a, g_qkv, d_a)
                 g_next = d_o

@@ -614,6 +614,38 @@ def batched_gemm(ctx, a, b, c, M, N, K, a_strides, b_strides, ldc, batch=(1, 1),
                                  c_batch[0], c_batch[1], alpha, int(accumulate), int(causal)), "tch_batched_gemm")
 
 
+def _flash_check(name, t, B, H, T, strides):
+    rs, bs = strides
+    assert t.dtype == torch.bfloat16, f"flash attention: {name} must be bf16"
+    assert (B - 1) * bs + (T - 1) * rs + H * 64 <= t.numel(), f"flash attention: {name} reaches past its tensor"
+
+
+def flash_attn_fwd(ctx, q, k, v, o, lse, B, H, T, qkv_strides, o_strides, scale, causal=True):
+    """o = softmax(scale * q k^T [+ causal mask]) v per head without the [T, T] scores in memory (bf16, heads 64
+    wide, T a multiple of 128).  q, k, v are views that start at head 0 of sample 0; element (b, t, h, d) sits at
+    b * strides[1] + t * strides[0] + 64 h + d, so the three may be slices of one packed projection.  lse
+    [B * H, T] fp32 receives the log-sum-exp of the scaled scores for the backward."""
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _flash_check(name, t, B, H, T, qkv_strides)
+    _flash_check("o", o, B, H, T, o_strides)
+    assert lse.dtype == torch.float32 and lse.numel() >= B * H * T
+    check(lib().tch_flash_attn_fwd(ctx.handle, dtype_code(q), _p(q), _p(k), _p(v), _p(o), _p(lse), B, H, T, qkv_strides[0],
+                                   qkv_strides[1], o_strides[0], o_strides[1], scale, int(causal)), "tch_flash_attn_fwd")
+
+
+def flash_attn_bwd(ctx, q, k, v, o, dout, lse, delta, dq, dk, dv, B, H, T, qkv_strides, o_strides, scale, causal=True):
+    """Gradients of flash_attn_fwd; dq, dk, dv are laid out like q, k, v and o, dout like o.  delta [B * H, T]
+    fp32 is scratch (row sums of dout * o)."""
+    for name, t in (("q", q), ("k", k), ("v", v), ("dq", dq), ("dk", dk), ("dv", dv)):
+        _flash_check(name, t, B, H, T, qkv_strides)
+    for name, t in (("o", o), ("dout", dout)):
+        _flash_check(name, t, B, H, T, o_strides)
+    assert lse.dtype == delta.dtype == torch.float32 and lse.numel() >= B * H * T and delta.numel() >= B * H * T
+    check(lib().tch_flash_attn_bwd(ctx.handle, dtype_code(q), _p(q), _p(k), _p(v), _p(o), _p(dout), _p(lse), _p(delta),
+                                   _p(dq), _p(dk), _p(dv), B, H, T, qkv_strides[0], qkv_strides[1], o_strides[0],
+                                   o_strides[1], scale, int(causal)), "tch_flash_attn_bwd")
+
+
 # ---------------------------------------------------------------------------
 # Swin-B data movement
 # ---------------------------------------------------------------------------

@@ -305,3 +305,66 @@ def test_batched_gemm_accumulate_and_edges(ctx, dtype):
     torch.cuda.synchronize()
     ref = 1.0 + 0.5 * a[1:].float().view(M, K) @ b.float().t()
     close(c, ref, dtype, "accumulate", rtol=1e-3 if dtype == torch.float32 else 2e-2)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,H,T,packed", [(2, 3, 256, True), (1, 2, 128, False), (1, 1, 512, True)])
+def test_flash_attention(ctx, B, H, T, packed, causal):
+    """Fused attention forward and backward against the oracle's scores -> softmax -> context chain.  The
+    oracle sees the same bf16-rounded inputs; bf16 tolerance (2e-2 of the largest magnitude per tensor)."""
+    from sirius_amd import ops
+    D, C = 64, H * 64
+    g = _gen(40 + T + B)
+    dtype = torch.bfloat16
+    scale = 1.0 / 8.0
+    if packed:
+        qkv = rnd((B, T, 3 * C), dtype, g)
+        q, k, v = qkv[..., :C], qkv[..., C:2 * C], qkv[..., 2 * C:]
+        dev = qkv.cuda()
+        flat = dev.view(-1)
+        dq_, dk_, dv_ = flat, flat[C:], flat[2 * C:]
+        strides = (3 * C, T * 3 * C)
+        dgrad = torch.zeros_like(dev)
+        gflat = dgrad.view(-1)
+        gq, gk, gv = gflat, gflat[C:], gflat[2 * C:]
+    else:
+        q, k, v = (rnd((B, T, C), dtype, g) for _ in range(3))
+        dq_, dk_, dv_ = (t.cuda().view(-1) for t in (q, k, v))
+        strides = (C, T * C)
+        gq, gk, gv = (torch.zeros(B * T * C, dtype=dtype, device="cuda") for _ in range(3))
+    dout = rnd((B, T, C), dtype, g)
+
+    def heads(t):
+        return t.reshape(B, T, H, D).permute(0, 2, 1, 3)
+    o_ref, lse_ref = S.attention(heads(q), heads(k), heads(v), scale, causal)
+    dq_ref, dk_ref, dv_ref = S.attention_bwd(heads(q), heads(k), heads(v), heads(dout), scale, causal)
+
+    o = torch.zeros(B, T, C, dtype=dtype, device="cuda")
+    lse = torch.zeros(B * H, T, dtype=torch.float32, device="cuda")
+    delta = torch.zeros(B * H, T, dtype=torch.float32, device="cuda")
+    ops.flash_attn_fwd(ctx, dq_, dk_, dv_, o.view(-1), lse, B, H, T, strides, (C, T * C), scale, causal)
+    ctx.synchronize()
+    close(heads(o.cpu()), o_ref, dtype, "context")
+    close(lse.view(B, H, T), lse_ref, torch.float32, "log-sum-exp", rtol=2e-3)
+    d_dev = dout.cuda()
+    ops.flash_attn_bwd(ctx, dq_, dk_, dv_, o.view(-1), d_dev.view(-1), lse, delta, gq, gk, gv, B, H, T, strides,
+                       (C, T * C), scale, causal)
+    ctx.synchronize()
+    delta_ref = (heads(dout).float() * o_ref).sum(-1)
+    close(delta.view(B, H, T), delta_ref, dtype, "delta")
+    if packed:
+        got = dgrad.cpu()
+        got_q, got_k, got_v = got[..., :C], got[..., C:2 * C], got[..., 2 * C:]
+    else:
+        got_q, got_k, got_v = (t.cpu().view(B, T, C) for t in (gq, gk, gv))
+    close(heads(got_q), dq_ref, dtype, "dq")
+    close(heads(got_k), dk_ref, dtype, "dk")
+    close(heads(got_v), dv_ref, dtype, "dv")
+
+
+def test_flash_attention_rejects_bad_shapes(ctx):
+    from sirius_amd import ops
+    t = torch.zeros(2 * 100 * 64, dtype=torch.bfloat16, device="cuda")
+    lse = torch.zeros(2 * 100, dtype=torch.float32, device="cuda")
+    with pytest.raises(Exception, match="multiple of 128"):
+        ops.flash_attn_fwd(ctx, t, t, t, t, lse, 2, 1, 100, (64, 100 * 64), (64, 100 * 64), 0.125)

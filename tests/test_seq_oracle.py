@@ -66,6 +66,42 @@ def test_gelu_forms():
         assert torch.allclose(got.double(), num, atol=1e-5)
 
 
+def test_attention_brute_force():
+    """attention() against scalar loops on a tiny causal problem, and its gradients against central differences."""
+    g = torch.Generator().manual_seed(5)
+    B, H, T, d = 1, 2, 5, 3
+    q, k, v = (torch.randn(B, H, T, d, generator=g, dtype=torch.float64) for _ in range(3))
+    scale = 0.7
+    o, lse = S.attention(q.float(), k.float(), v.float(), scale, causal=True)
+
+    def brute(q, k, v):
+        out = torch.zeros(B, H, T, d, dtype=torch.float64)
+        ls = torch.zeros(B, H, T, dtype=torch.float64)
+        for b in range(B):
+            for h in range(H):
+                for i in range(T):
+                    w = [math.exp(scale * sum(q[b, h, i, e] * k[b, h, j, e] for e in range(d))) for j in range(i + 1)]
+                    tot = sum(w)
+                    ls[b, h, i] = math.log(tot)
+                    for e in range(d):
+                        out[b, h, i, e] = sum(w[j] * v[b, h, j, e] for j in range(i + 1)) / tot
+        return out, ls
+    ob, lb = brute(q, k, v)
+    assert torch.allclose(o.double(), ob, atol=1e-5) and torch.allclose(lse.double(), lb, atol=1e-5)
+    dout = torch.randn(B, H, T, d, generator=g, dtype=torch.float64)
+    dq, dk, dv = S.attention_bwd(q.float(), k.float(), v.float(), dout.float(), scale, causal=True)
+    eps = 1e-5
+    for name, t, got in (("q", q, dq), ("k", k, dk), ("v", v, dv)):
+        for idx in [(0, 0, 4, 1), (0, 1, 2, 0), (0, 1, 0, 2)]:
+            tp, tm = t.clone(), t.clone()
+            tp[idx] += eps
+            tm[idx] -= eps
+            args_p = [tp if n == name else x for n, x in (("q", q), ("k", k), ("v", v))]
+            args_m = [tm if n == name else x for n, x in (("q", q), ("k", k), ("v", v))]
+            num = ((brute(*args_p)[0] - brute(*args_m)[0]) * dout).sum().item() / (2 * eps)
+            assert abs(got[idx].item() - num) <= 1e-4 * max(1.0, abs(num)), (name, idx, got[idx].item(), num)
+
+
 def test_attn_softmax_brute_force():
     g = _gen(2)
     Bn, Hn, L, nW = 4, 2, 5, 2
