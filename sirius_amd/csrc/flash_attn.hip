@@ -165,8 +165,13 @@ __global__ __launch_bounds__(256) void flash_query_kernel(FlashArgs p) {
   unsigned char* kt = lds;
   unsigned char* vt = lds + kTileB;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5;
-  const int qb = gridDim.x - 1 - blockIdx.x;   // long rows of a causal problem first
-  const int bh = blockIdx.y;
+  // Workgroup ids go to the XCDs round-robin and all of them are resident at once, so the order is the
+  // placement: the blocks of one head keep one residue of the id modulo 8 (one XCD, one L2 for its keys and
+  // values), and the long blocks of a causal problem come first so that each compute unit's share of
+  // consecutive ids mixes long and short ones.
+  const int nbh = gridDim.x / (p.T / kFixed);
+  const int qb = p.T / kFixed - 1 - blockIdx.x / nbh;
+  const int bh = blockIdx.x % nbh;
   const int b = bh / p.H, h = bh - b * p.H;
   const int64_t qkv_off = b * p.qkv_bs + h * kHd, o_off = b * p.o_bs + h * kHd;
   const int q0 = qb * kFixed, qw0 = q0 + 32 * wave;
@@ -300,8 +305,9 @@ __global__ __launch_bounds__(256) void flash_key_kernel(FlashArgs p) {
   unsigned char* qt = lds;
   unsigned char* dot = lds + kTileB;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5;
-  const int kblk = blockIdx.x;
-  const int bh = blockIdx.y;
+  const int nbh = gridDim.x / (p.T / kFixed);   // placement as in flash_query_kernel: early keys see most queries
+  const int kblk = blockIdx.x / nbh;
+  const int bh = blockIdx.x % nbh;
   const int b = bh / p.H, h = bh - b * p.H;
   const int64_t qkv_off = b * p.qkv_bs + h * kHd, o_off = b * p.o_bs + h * kHd;
   const int k0 = kblk * kFixed, kw0 = k0 + 32 * wave;
@@ -399,7 +405,7 @@ int check_geometry(const char* who, int dtype, int B, int H, int T, int64_t qkv_
   const std::string w(who);
   TCH_CHECK_ARG(dtype == kBF16, w + ": bf16 only");
   TCH_CHECK_ARG(B >= 1 && H >= 1 && T >= kFixed && T % kFixed == 0, w + ": the sequence length must be a multiple of 128");
-  TCH_CHECK_ARG(static_cast<int64_t>(B) * H <= 65535, w + ": too many heads for one grid");
+  TCH_CHECK_ARG(static_cast<int64_t>(B) * H * (T / kFixed) < (1ll << 31), w + ": too many blocks for one grid");
   TCH_CHECK_ARG(qkv_rs >= static_cast<int64_t>(H) * kHd && o_rs >= static_cast<int64_t>(H) * kHd,
                 w + ": row strides shorter than the heads");
   TCH_CHECK_ARG(qkv_rs % 8 == 0 && qkv_bs % 8 == 0 && o_rs % 8 == 0 && o_bs % 8 == 0,
@@ -429,7 +435,7 @@ int flash_attn_fwd(Context* ctx, int dtype, const void* q, const void* k, const 
   a.H = H;
   a.T = T;
   a.scale = scale;
-  const dim3 grid(T / kFixed, B * H);
+  const dim3 grid(static_cast<unsigned>(T / kFixed) * B * H);
   const double flops = 4.0 * B * H * static_cast<double>(T) * T * kHd * (causal ? 0.5 : 1.0);
   return causal ? launch(ctx, flash_query_kernel<true, false>, grid, dim3(256), a, "flash_attn_fwd<causal>", flops, 0)
                 : launch(ctx, flash_query_kernel<false, false>, grid, dim3(256), a, "flash_attn_fwd<full>", flops, 0);
@@ -461,7 +467,7 @@ int flash_attn_bwd(Context* ctx, int dtype, const void* q, const void* k, const 
   a.H = H;
   a.T = T;
   a.scale = scale;
-  const dim3 grid(T / kFixed, B * H);
+  const dim3 grid(static_cast<unsigned>(T / kFixed) * B * H);
   const double pair = 2.0 * B * H * static_cast<double>(T) * T * kHd * (causal ? 0.5 : 1.0);   // one T x T x 64 product
   // the dQ launch leaves delta for the dK / dV launch
   int rc = causal ? launch(ctx, flash_query_kernel<true, true>, grid, dim3(256), a, "flash_attn_dq<causal>", 3.0 * pair, 0)
