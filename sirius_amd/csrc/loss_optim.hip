@@ -97,6 +97,93 @@ __global__ __launch_bounds__(256) void softmax_ce_wide_kernel(CeWideArgs p) {
   }
 }
 
+// The same with the whole row held in registers: 1024 threads keep up to 16 four-float pieces each (rows up
+// to 65536 classes), so the logits are read once and the gradient written once.  Needs 16-byte aligned rows
+// on both sides and room for the last piece (the columns between `classes` and the next multiple of four
+// receive zeros).
+constexpr int kRowPieces = 16;
+
+__device__ inline float block_reduce_1024(float v, bool take_max, float* scratch) {
+  v = take_max ? wave_max(v) : wave_sum(v);
+  __syncthreads();   // the previous reduction's readers are done
+  if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float r = scratch[0];
+#pragma unroll
+  for (int w = 1; w < 16; ++w) r = take_max ? fmaxf(r, scratch[w]) : r + scratch[w];
+  return r;
+}
+
+template <typename T>
+__global__ __launch_bounds__(1024) void softmax_ce_row_kernel(CeWideArgs p) {
+  __shared__ float scratch[16];
+  const int row = blockIdx.x;
+  const int tid = threadIdx.x;
+  const float4* z = reinterpret_cast<const float4*>(p.logits + static_cast<int64_t>(row) * p.ld_logits);
+  T* g = static_cast<T*>(p.dlogits) + static_cast<int64_t>(row) * p.ld_dlogits;
+  const int pieces = (p.classes + 3) >> 2;
+  const int64_t label = p.labels[row];
+  const bool ignored = label < 0 || label >= p.classes;
+  float v[kRowPieces][4];
+  float mx = -INFINITY;
+  if (!ignored) {
+#pragma unroll
+    for (int i = 0; i < kRowPieces; ++i) {
+      const int pc = tid + 1024 * i;
+      if (pc < pieces) {
+        const float4 t = z[pc];
+        v[i][0] = t.x;
+        v[i][1] = t.y;
+        v[i][2] = t.z;
+        v[i][3] = t.w;
+        if (pc == pieces - 1) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (pc * 4 + e >= p.classes) v[i][e] = -INFINITY;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[i][e] = -INFINITY;
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) mx = fmaxf(mx, v[i][e]);
+    }
+  }
+  mx = block_reduce_1024(mx, true, scratch);
+  float sum = 0.f;
+  if (!ignored) {
+#pragma unroll
+    for (int i = 0; i < kRowPieces; ++i)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v[i][e] = __expf(v[i][e] - mx);
+        sum += v[i][e];
+      }
+  }
+  sum = block_reduce_1024(sum, false, scratch);
+  if (tid == 0) p.loss_rows[row] = ignored ? 0.f : mx + logf(sum) - p.logits[static_cast<int64_t>(row) * p.ld_logits + label];
+  const float mul = ignored ? 0.f : p.grad_scale / sum;
+#pragma unroll
+  for (int i = 0; i < kRowPieces; ++i) {
+    const int pc = tid + 1024 * i;
+    if (pc >= pieces) continue;
+    float o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      o[e] = ignored ? 0.f : v[i][e] * mul;
+      if (pc * 4 + e == label) o[e] -= p.grad_scale;
+    }
+    if constexpr (sizeof(T) == 2) {
+      uint2 w;
+      w.x = float_to_bf16_bits(o[0]) | (static_cast<uint32_t>(float_to_bf16_bits(o[1])) << 16);
+      w.y = float_to_bf16_bits(o[2]) | (static_cast<uint32_t>(float_to_bf16_bits(o[3])) << 16);
+      *reinterpret_cast<uint2*>(g + pc * 4) = w;
+    } else {
+      *reinterpret_cast<float4*>(g + pc * 4) = make_float4(o[0], o[1], o[2], o[3]);
+    }
+  }
+}
+
 struct MeanArgs {
   const float* in;
   float* out;
@@ -301,9 +388,21 @@ int softmax_ce_lm(Context* ctx, int dtype, const float* logits, int ld_logits, c
   CeWideArgs a{logits, labels, loss_rows, dlogits, rows, classes, ld_logits, ld_dlogits,
                loss_scale / static_cast<float>(valid_rows)};
   const double bytes = static_cast<double>(rows) * classes * (4.0 + (dtype == kBF16 ? 2.0 : 4.0));
-  int rc = dtype == kBF16
-               ? launch(ctx, softmax_ce_wide_kernel<bf16>, dim3(rows), dim3(256), a, "softmax_ce_wide_kernel<bf16>", bytes, 1)
-               : launch(ctx, softmax_ce_wide_kernel<float>, dim3(rows), dim3(256), a, "softmax_ce_wide_kernel<f32>", bytes, 1);
+  const int padded = (classes + 3) / 4 * 4;
+  const int eb = dtype == kBF16 ? 2 : 4;
+  const bool in_registers = padded <= kRowPieces * 4096 && padded <= ld_logits && padded <= ld_dlogits && ld_logits % 4 == 0 &&
+                            (static_cast<int64_t>(ld_dlogits) * eb) % 16 == 0 &&
+                            (reinterpret_cast<uintptr_t>(logits) & 15) == 0 && (reinterpret_cast<uintptr_t>(dlogits) & 15) == 0;
+  int rc;
+  if (in_registers) {
+    rc = dtype == kBF16
+             ? launch(ctx, softmax_ce_row_kernel<bf16>, dim3(rows), dim3(1024), a, "softmax_ce_row_kernel<bf16>", bytes, 1)
+             : launch(ctx, softmax_ce_row_kernel<float>, dim3(rows), dim3(1024), a, "softmax_ce_row_kernel<f32>", bytes, 1);
+  } else {
+    rc = dtype == kBF16
+             ? launch(ctx, softmax_ce_wide_kernel<bf16>, dim3(rows), dim3(256), a, "softmax_ce_wide_kernel<bf16>", bytes, 1)
+             : launch(ctx, softmax_ce_wide_kernel<float>, dim3(rows), dim3(256), a, "softmax_ce_wide_kernel<f32>", bytes, 1);
+  }
   if (rc) return rc;
   MeanArgs m{loss_rows, loss_mean, rows, static_cast<float>(valid_rows)};
   return launch(ctx, mean_kernel, dim3(1), dim3(64), m, "mean_kernel", 4.0 * rows, 1);

@@ -368,3 +368,31 @@ def test_flash_attention_rejects_bad_shapes(ctx):
     lse = torch.zeros(2 * 100, dtype=torch.float32, device="cuda")
     with pytest.raises(Exception, match="multiple of 128"):
         ops.flash_attn_fwd(ctx, t, t, t, t, lse, 2, 1, 100, (64, 100 * 64), (64, 100 * 64), 0.125)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,classes,ld", [(37, 50257, 50304), (64, 97, 128), (19, 1001, 1001), (8, 70001, 70008)])
+def test_softmax_ce_lm(ctx, dtype, rows, classes, ld):
+    """Language-model cross entropy (mean over rows with a label >= 0) and its gradient against torch's CPU
+    cross_entropy with ignore_index; covers the rows-in-registers kernel (aligned rows of at most 65536 classes)
+    and the looping one (unaligned leading dimension, longer rows)."""
+    from sirius_amd import ops
+    g = _gen(rows + classes)
+    z = torch.randn(rows, ld, generator=g) * 3.0
+    labels = torch.randint(0, classes, (rows,), generator=g)
+    labels[::5] = -100
+    valid = int((labels >= 0).sum())
+    zr = z[:, :classes].clone().requires_grad_(True)
+    loss_ref = torch.nn.functional.cross_entropy(zr, labels, ignore_index=-100) * 0.5
+    (g_ref,) = torch.autograd.grad(loss_ref, zr)
+    zd = z.cuda()
+    dl = torch.full((rows, ld), 7.0, dtype=dtype, device="cuda")
+    loss_rows = torch.zeros(rows, device="cuda")
+    loss = torch.zeros(1, device="cuda")
+    ops.softmax_ce_lm(ctx, zd, labels.cuda(), loss_rows, loss, dl, classes, valid, loss_scale=0.5)
+    ctx.synchronize()
+    assert abs(loss.item() * 0.5 - loss_ref.item()) <= 1e-4 * abs(loss_ref.item()), (loss.item(), loss_ref.item())
+    close(dl[:, :classes], g_ref, dtype, "dlogits")
+    assert torch.all(dl[labels.cuda() < 0][:, :classes] == 0)
+    pad = dl[:, (classes + 3) // 4 * 4:]
+    assert torch.all(pad == 7.0), "columns beyond the last four-float piece are not touched"
