@@ -289,6 +289,25 @@ int tch_flash_attn_bwd(tch_context* ctx, int dtype, const void* q, const void* k
                        const void* dout, const float* lse, float* delta, void* dq, void* dk, void* dv, int B, int H,
                        int T, int64_t qkv_rs, int64_t qkv_bs, int64_t o_rs, int64_t o_bs, float scale, int causal);
 
+/* Window attention of the Swin-B step in one launch per direction (train/swin_b_tiny.py:94-110: q k^T * scale +
+ * relative position bias (+ shift mask), softmax, @ v; torchvision's shifted_window_attention for
+ * train/swin_b.py:38).  bf16 only, heads 32 wide (C = 32 heads), N <= 64 tokens per window.
+ * qkv [windows * N][3C] is the packed projection of the window-partitioned tokens, o / dout [windows * N][C];
+ * probs and ds are [windows * heads][N][64] (key rows padded to 64; the forward stores the probabilities there,
+ * the backward reads them and stores the gradient of the logits, whose sum over the windows is the bias
+ * gradient); bias [heads][64][64] fp32 holds -inf in the key columns from N on (tch_relpos_bias_gather_pairs
+ * with negative indices there); mask [nW][64][64] fp32 or null, window w uses mask w % nW. */
+int tch_window_attn_fwd(tch_context* ctx, int dtype, const void* qkv, void* o, void* probs, const float* bias,
+                        const float* mask, int windows, int heads, int N, int C, int nW, float scale);
+int tch_window_attn_bwd(tch_context* ctx, int dtype, const void* qkv, const void* probs, const void* dout, void* dqkv,
+                        void* ds, int windows, int heads, int N, int C, float scale);
+/* tch_relpos_bias_gather / _scatter over an explicit list of (query, key) pairs instead of tokens^2: index[pair]
+ * < 0 marks padding (gathers -inf, takes no gradient). */
+int tch_relpos_bias_gather_pairs(tch_context* ctx, const float* table, const int32_t* index, float* bias, int heads,
+                                 int pairs, int entries);
+int tch_relpos_bias_scatter_pairs(tch_context* ctx, const float* dbias, const int32_t* index, float* dtable, int heads,
+                                  int pairs, int entries, int accumulate);
+
 /* Swin-B data movement (train/swin_b_tiny.py:8-19,116-131; patch merging and shift as in torchvision's swin_b,
  * train/swin_b.py:38).
  * reverse == 0: dst[windows of window x window tokens] = roll(src[B,H,W,C], -shift) partitioned;

@@ -292,6 +292,26 @@ int tch_batched_gemm(tch_context* ctx, int dtype, const void* a, const void* b, 
                       b_bo, b_bi, c_bo, c_bi, alpha, accumulate, causal);
 }
 
+int tch_window_attn_fwd(tch_context* ctx, int dtype, const void* qkv, void* o, void* probs, const float* bias,
+                        const float* mask, int windows, int heads, int N, int Cc, int nW, float scale) {
+  return window_attn_fwd(C(ctx), dtype, qkv, o, probs, bias, mask, windows, heads, N, Cc, nW, scale);
+}
+
+int tch_window_attn_bwd(tch_context* ctx, int dtype, const void* qkv, const void* probs, const void* dout, void* dqkv,
+                        void* ds, int windows, int heads, int N, int Cc, float scale) {
+  return window_attn_bwd(C(ctx), dtype, qkv, probs, dout, dqkv, ds, windows, heads, N, Cc, scale);
+}
+
+int tch_relpos_bias_gather_pairs(tch_context* ctx, const float* table, const int32_t* index, float* bias, int heads,
+                                 int pairs, int entries) {
+  return relpos_bias_gather_pairs(C(ctx), table, index, bias, heads, pairs, entries);
+}
+
+int tch_relpos_bias_scatter_pairs(tch_context* ctx, const float* dbias, const int32_t* index, float* dtable, int heads,
+                                  int pairs, int entries, int accumulate) {
+  return relpos_bias_scatter_pairs(C(ctx), dbias, index, dtable, heads, pairs, entries, accumulate);
+}
+
 int tch_flash_attn_fwd(tch_context* ctx, int dtype, const void* q, const void* k, const void* v, void* o, float* lse,
                        int B, int H, int T, int64_t qkv_rs, int64_t qkv_bs, int64_t o_rs, int64_t o_bs, float scale,
                        int causal) {

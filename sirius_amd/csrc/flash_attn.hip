@@ -22,6 +22,7 @@
 // probabilities rounded to bf16 for the second product (as the unfused path stores them).  The backward
 // recomputes the probabilities from the saved log-sum-exp; dQ and (dK, dV) are two launches so that nothing is
 // accumulated atomically and results do not depend on scheduling.
+#include "attn_frag.h"
 #include "kernels.h"
 #include "ops.h"
 
@@ -36,11 +37,6 @@ constexpr int kRowB = 144;       // LDS bytes per tile row: 64 bf16 + 16 bytes, 
 constexpr int kTileB = kWalk * kRowB;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
-
-typedef short short4_t __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) short4_t* lds_short4_ptr;
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-typedef float f32x2_t __attribute__((ext_vector_type(2)));
 
 struct FlashArgs {
   const bf16* q;
@@ -59,12 +55,6 @@ struct FlashArgs {
   float scale;
 };
 
-__device__ inline uint32_t pack_bf16(float a, float b) {
-  f32x2_t v = {a, b};
-  bf16x2_t r = __builtin_convertvector(v, bf16x2_t);
-  return __builtin_bit_cast(uint32_t, r);
-}
-
 // a [64][64] bf16 tile: global -> registers (two 16-byte chunks per thread) -> LDS rows of kRowB bytes
 __device__ inline void tile_load(const bf16* base, int64_t rs, int tid, Chunk (&r)[2]) {
 #pragma unroll
@@ -81,57 +71,11 @@ __device__ inline void tile_store(unsigned char* lds, int tid, const Chunk (&r)[
   }
 }
 
-// operand fragment whose MFMA rows are tile rows row0 .. row0+31 and whose reduction index is the head
-// dimension: lane holds 8 consecutive columns 16 ks + 8 (lane / 32) of row row0 + lane % 32
-__device__ inline Chunk frag_rows(const unsigned char* lds, int row0, int ks, int lane) {
-  Chunk c;
-  c.u = *reinterpret_cast<const uint4*>(lds + (row0 + (lane & 31)) * kRowB + (ks * 16 + 8 * (lane >> 5)) * 2);
-  return c;
-}
-
-// operand fragment whose MFMA rows are the columns 32 ct .. 32 ct + 31 of the tile and whose reduction index
-// runs over the 16 tile rows from row0 in the accumulator's order: element 4t + i of lane half h is row
-// row0 + 8t + 4h + i
-__device__ inline Chunk frag_cols(const unsigned char* lds, int row0, int ct, int lane) {
-  const int grp = lane >> 4, q16 = lane & 15;
-  Chunk c;
-#pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    const int row = row0 + 8 * t + 4 * (grp >> 1) + (q16 >> 2);
-    const int col = 32 * ct + 16 * (grp & 1) + 4 * (q16 & 3);
-    union {
-      short4_t s;
-      uint32_t w[2];
-    } v;
-    v.s = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_short4_ptr)(lds + row * kRowB + col * 2));
-    c.w[2 * t] = v.w[0];
-    c.w[2 * t + 1] = v.w[1];
-  }
-  return c;
-}
-
 // this wave's fragments of 32 fixed rows (row = first + lane % 32): 4 chunks cover the lane half's 32 columns
 __device__ inline void load_fixed(const bf16* base, int64_t rs, int first, int lane, Chunk (&f)[4]) {
   const bf16* row = base + static_cast<int64_t>(first + (lane & 31)) * rs + 8 * (lane >> 5);
 #pragma unroll
   for (int ks = 0; ks < 4; ++ks) f[ks].u = *reinterpret_cast<const uint4*>(row + ks * 16);
-}
-
-// registers 8s .. 8s+7 of an accumulator as the second operand of the next product
-__device__ inline Chunk pack_slab(const float* p) {
-  Chunk c;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) c.w[i] = pack_bf16(p[2 * i], p[2 * i + 1]);
-  return c;
-}
-
-__device__ inline void zero_acc(f32x16_t& a) {
-#pragma unroll
-  for (int e = 0; e < 16; ++e) a[e] = 0.f;
-}
-
-__device__ inline f32x16_t mma16(const Chunk& first, const Chunk& second, f32x16_t acc) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(first.h, second.h, acc, 0, 0, 0);
 }
 
 // acc[ct] holds the transposed result: column 32 ct + 8 (r / 4) + 4 (lane / 32) + r % 4 of fixed row lane % 32.
@@ -227,11 +171,11 @@ __global__ __launch_bounds__(256) void flash_query_kernel(FlashArgs p) {
     for (int t = 0; t < 2; ++t) {
       zero_acc(s[t]);
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) s[t] = mma16(frag_rows(kt, 32 * t, ks, lane), qf[ks], s[t]);
+      for (int ks = 0; ks < 4; ++ks) s[t] = mma16(frag_rows<kRowB>(kt, 32 * t, ks, lane), qf[ks], s[t]);
       if (DQ) {
         zero_acc(dp[t]);
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) dp[t] = mma16(frag_rows(vt, 32 * t, ks, lane), dof[ks], dp[t]);
+        for (int ks = 0; ks < 4; ++ks) dp[t] = mma16(frag_rows<kRowB>(vt, 32 * t, ks, lane), dof[ks], dp[t]);
       }
     }
     const bool diagonal = CAUSAL && k0 + kWalk - 1 > qw0;   // some key of the tile lies beyond some query
@@ -281,7 +225,7 @@ __global__ __launch_bounds__(256) void flash_query_kernel(FlashArgs p) {
       for (int sl = 0; sl < 2; ++sl) {
         const Chunk pc = pack_slab(&pr[t][8 * sl]);
 #pragma unroll
-        for (int ct = 0; ct < 2; ++ct) acc[ct] = mma16(frag_cols(second, 32 * t + 16 * sl, ct, lane), pc, acc[ct]);
+        for (int ct = 0; ct < 2; ++ct) acc[ct] = mma16(frag_cols<kRowB>(second, 32 * t + 16 * sl, ct, lane), pc, acc[ct]);
       }
   }
 
@@ -357,8 +301,8 @@ __global__ __launch_bounds__(256) void flash_key_kernel(FlashArgs p) {
       zero_acc(dp[t]);
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
-        s[t] = mma16(frag_rows(qt, 32 * t, ks, lane), kf[ks], s[t]);
-        dp[t] = mma16(frag_rows(dot, 32 * t, ks, lane), vf[ks], dp[t]);
+        s[t] = mma16(frag_rows<kRowB>(qt, 32 * t, ks, lane), kf[ks], s[t]);
+        dp[t] = mma16(frag_rows<kRowB>(dot, 32 * t, ks, lane), vf[ks], dp[t]);
       }
     }
     const bool diagonal = CAUSAL && q0 < kw0 + 31;   // some staged query lies before some key of this wave
@@ -388,8 +332,8 @@ __global__ __launch_bounds__(256) void flash_key_kernel(FlashArgs p) {
         const Chunk dc = pack_slab(&ds[t][8 * sl]);
 #pragma unroll
         for (int ct = 0; ct < 2; ++ct) {
-          dv[ct] = mma16(frag_cols(dot, 32 * t + 16 * sl, ct, lane), pc, dv[ct]);
-          dk[ct] = mma16(frag_cols(qt, 32 * t + 16 * sl, ct, lane), dc, dk[ct]);
+          dv[ct] = mma16(frag_cols<kRowB>(dot, 32 * t + 16 * sl, ct, lane), pc, dv[ct]);
+          dk[ct] = mma16(frag_cols<kRowB>(qt, 32 * t + 16 * sl, ct, lane), dc, dk[ct]);
         }
       }
   }

@@ -122,6 +122,12 @@ int relpos_bias_gather(Context* ctx, const float* table, const int32_t* index, f
                        int entries);
 int relpos_bias_scatter(Context* ctx, const float* dbias, const int32_t* index, float* dtable, int heads, int tokens,
                         int entries, int accumulate);
+// the same over an arbitrary list of (query, key) pairs, e.g. rows padded to 64 keys: a negative index is padding
+// (gathers -inf, receives no gradient)
+int relpos_bias_gather_pairs(Context* ctx, const float* table, const int32_t* index, float* bias, int heads, int pairs,
+                             int entries);
+int relpos_bias_scatter_pairs(Context* ctx, const float* dbias, const int32_t* index, float* dtable, int heads, int pairs,
+                              int entries, int accumulate);
 int64_t column_sum_workspace_floats(int rows, int cols);
 int column_sum(Context* ctx, int dtype, const void* x, float* out, int rows, int cols, int accumulate, float* workspace);
 
@@ -137,6 +143,14 @@ int flash_attn_fwd(Context* ctx, int dtype, const void* q, const void* k, const 
 int flash_attn_bwd(Context* ctx, int dtype, const void* q, const void* k, const void* v, const void* o, const void* dout,
                    const float* lse, float* delta, void* dq, void* dk, void* dv, int B, int H, int T, int64_t qkv_rs,
                    int64_t qkv_bs, int64_t o_rs, int64_t o_bs, float scale, int causal);
+
+// window_attn.hip -- Swin window attention in one launch per direction (bf16, heads 32 wide, N <= 64 tokens):
+// qkv [windows * N][3C], o / dout [windows * N][C], probs and ds [windows * heads][N][64], bias [heads][64][64]
+// with -inf beyond key N, mask [nW][64][64] or null (window w of an image uses mask w % nW)
+int window_attn_fwd(Context* ctx, int dtype, const void* qkv, void* o, void* probs, const float* bias, const float* mask,
+                    int windows, int heads, int N, int C, int nW, float scale);
+int window_attn_bwd(Context* ctx, int dtype, const void* qkv, const void* probs, const void* dout, void* dqkv, void* ds,
+                    int windows, int heads, int N, int C, float scale);
 
 // pool.hip
 int maxpool_fwd(Context* ctx, int dtype, const void* x, void* y, int32_t* index, int N, int H, int W, int C, int ksize,

@@ -138,7 +138,8 @@ __global__ __launch_bounds__(256) void relpos_gather_kernel(RelPosArgs p) {
   const int e = blockIdx.x * 256 + threadIdx.x;
   if (e >= p.heads * p.nn) return;
   const int h = e / p.nn, ij = e - h * p.nn;
-  p.bias[e] = p.table[p.index[ij] * p.heads + h];
+  const int idx = p.index[ij];
+  p.bias[e] = idx < 0 ? -INFINITY : p.table[idx * p.heads + h];   // a negative index marks padding: masked out
 }
 
 // one wavefront per (table entry, head): the (i, j) pairs that point at the entry are summed in index order
@@ -223,6 +224,22 @@ int relpos_bias_scatter(Context* ctx, const float* dbias, const int32_t* index, 
                         int entries, int accumulate) {
   TCH_CHECK_ARG(dbias && index && dtable && heads > 0 && tokens > 0 && entries > 0, "relpos_bias_scatter: bad arguments");
   RelPosArgs a{nullptr, index, nullptr, dbias, dtable, heads, tokens * tokens, entries, accumulate};
+  return launch(ctx, relpos_scatter_kernel, dim3(entries * heads), dim3(64), a, "relpos_scatter_kernel",
+                4.0 * entries * heads * a.nn, 1);
+}
+
+int relpos_bias_gather_pairs(Context* ctx, const float* table, const int32_t* index, float* bias, int heads, int pairs,
+                             int entries) {
+  TCH_CHECK_ARG(table && index && bias && heads > 0 && pairs > 0 && entries > 0, "relpos_bias_gather_pairs: bad arguments");
+  RelPosArgs a{table, index, bias, nullptr, nullptr, heads, pairs, entries, 0};
+  return launch(ctx, relpos_gather_kernel, dim3((heads * a.nn + 255) / 256), dim3(256), a, "relpos_gather_kernel",
+                8.0 * heads * a.nn, 1);
+}
+
+int relpos_bias_scatter_pairs(Context* ctx, const float* dbias, const int32_t* index, float* dtable, int heads, int pairs,
+                              int entries, int accumulate) {
+  TCH_CHECK_ARG(dbias && index && dtable && heads > 0 && pairs > 0 && entries > 0, "relpos_bias_scatter_pairs: bad arguments");
+  RelPosArgs a{nullptr, index, nullptr, dbias, dtable, heads, pairs, entries, accumulate};
   return launch(ctx, relpos_scatter_kernel, dim3(entries * heads), dim3(64), a, "relpos_scatter_kernel",
                 4.0 * entries * heads * a.nn, 1);
 }

@@ -687,6 +687,51 @@ def relpos_bias_scatter(ctx, dbias, index, dtable, accumulate=False):
                                         int(accumulate)), "tch_relpos_bias_scatter")
 
 
+def relpos_bias_gather_pairs(ctx, table, index, bias):
+    """bias[h, pair] = table[index[pair], h], -inf where index[pair] < 0 (padding)."""
+    entries, heads = table.shape
+    assert index.dtype == torch.int32 and bias.numel() == heads * index.numel()
+    assert table.dtype == bias.dtype == torch.float32
+    check(lib().tch_relpos_bias_gather_pairs(ctx.handle, _p(table), _p(index), _p(bias), heads, index.numel(), entries),
+          "tch_relpos_bias_gather_pairs")
+
+
+def relpos_bias_scatter_pairs(ctx, dbias, index, dtable, accumulate=False):
+    """dtable[entry, h] (+)= sum of dbias[h, pair] over the pairs with index[pair] == entry."""
+    entries, heads = dtable.shape
+    assert dbias.numel() == heads * index.numel() and dbias.dtype == dtable.dtype == torch.float32
+    assert index.dtype == torch.int32
+    check(lib().tch_relpos_bias_scatter_pairs(ctx.handle, _p(dbias), _p(index), _p(dtable), heads, index.numel(), entries,
+                                              int(accumulate)), "tch_relpos_bias_scatter_pairs")
+
+
+def window_attn_fwd(ctx, qkv, o, probs, bias, mask, windows, heads, N, scale):
+    """Window attention forward in one launch (bf16, heads 32 wide, N <= 64): qkv [windows * N, 3C] ->
+    o [windows * N, C]; probs [windows * heads, N, 64] keeps the probabilities; bias [heads, 64, 64] fp32 with -inf
+    from key column N on; mask [nW, 64, 64] fp32 or None."""
+    C = heads * 32
+    assert qkv.dtype == o.dtype == probs.dtype == torch.bfloat16 and bias.dtype == torch.float32
+    assert qkv.numel() == windows * N * 3 * C and o.numel() == windows * N * C
+    assert probs.numel() == windows * heads * N * 64 and bias.numel() == heads * 64 * 64
+    nW = 1
+    if mask is not None:
+        assert mask.dtype == torch.float32 and mask.numel() % (64 * 64) == 0
+        nW = mask.numel() // (64 * 64)
+    check(lib().tch_window_attn_fwd(ctx.handle, dtype_code(qkv), _p(qkv), _p(o), _p(probs), _p(bias), _p(mask), windows,
+                                    heads, N, C, nW, scale), "tch_window_attn_fwd")
+
+
+def window_attn_bwd(ctx, qkv, probs, dout, dqkv, ds, windows, heads, N, scale):
+    """Gradients of window_attn_fwd: dqkv like qkv, ds [windows * heads, N, 64] = gradient of the logits (its sum
+    over the windows is the bias gradient in the padded pair layout)."""
+    C = heads * 32
+    assert qkv.dtype == probs.dtype == dout.dtype == dqkv.dtype == ds.dtype == torch.bfloat16
+    assert qkv.numel() == dqkv.numel() == windows * N * 3 * C and dout.numel() == windows * N * C
+    assert probs.numel() == ds.numel() == windows * heads * N * 64
+    check(lib().tch_window_attn_bwd(ctx.handle, dtype_code(qkv), _p(qkv), _p(probs), _p(dout), _p(dqkv), _p(ds), windows,
+                                    heads, N, C, scale), "tch_window_attn_bwd")
+
+
 def column_sum_workspace_floats(rows, cols):
     return int(lib().tch_column_sum_workspace_floats(rows, cols))
 

@@ -70,11 +70,12 @@ def shifted_window_mask(H, W, ws, shift):
 class SwinEngine(EngineBase):
     def __init__(self, embed=128, depths=(2, 2, 18, 2), heads=(4, 8, 16, 32), window=7, patch=4, image_size=224,
                  num_classes=1000, dtype=torch.bfloat16, lr=1e-3, weight_decay=0.05, betas=(0.9, 0.999), eps=1e-8,
-                 stream=None, allocator=None, overlap_wgrad=True):
+                 stream=None, allocator=None, overlap_wgrad=True, fused_attention=True):
         self._init_engine(dtype, stream, allocator)
         # weight / bias / bias-table gradients on a second lane beside the data-gradient chain; the lanes meet
         # at the end of every block, before its gradient buffers are handed round again
         self.overlap_wgrad = overlap_wgrad
+        self.fused_attention = fused_attention
         assert len(depths) == len(heads) and image_size % patch == 0 and num_classes % 8 == 0 and embed % 8 == 0
         self.embed, self.depths, self.heads = embed, tuple(depths), tuple(heads)
         self.window, self.patch, self.image_size, self.num_classes = window, patch, image_size, num_classes
@@ -308,12 +309,20 @@ class SwinEngine(EngineBase):
         # still reads (the block's incoming gradient, the gathered projection gradient) is written again
         g_bufs = [flat(max_rc) for _ in range(6)]
         g_3c, g_4c_a, g_4c_b = flat(3 * max_rc), flat(4 * max_rc), flat(4 * max_rc)
-        max_scores = max(B * (st["R"] // st["ws"]) ** 2 * st["heads"] * st["ws"] ** 4 for st in self.stages)
+        # One launch per direction for the attention of a block where the kernel's limits hold (bf16, heads 32
+        # wide and even in number, at most 64 tokens per window): score rows are then padded to 64 keys.
+        for st in self.stages:
+            st["fused"] = (self.fused_attention and self.dtype == torch.bfloat16 and st["C"] // st["heads"] == 32 and
+                           st["heads"] % 2 == 0 and st["ws"] ** 2 <= 64)
+            st["keys_ld"] = 64 if st["fused"] else st["ws"] ** 2      # leading dimension of a score row
+            st["bias_elems"] = st["heads"] * (64 * 64 if st["fused"] else st["ws"] ** 4)
+        max_scores = max(B * (st["R"] // st["ws"]) ** 2 * st["heads"] * st["ws"] ** 2 * st["keys_ld"] for st in self.stages)
         d_scores = flat(max_scores)
-        max_bias = max(st["heads"] * st["ws"] ** 4 for st in self.stages)
+        max_bias = max(st["bias_elems"] for st in self.stages)
         bias_buf = act(max_bias, dtype=torch.float32)
         dbias_buf = act(max_bias, dtype=torch.float32)
-        colsum_ws = act(max(ops.column_sum_workspace_floats(B * (st["R"] // st["ws"]) ** 2, st["heads"] * st["ws"] ** 4)
+        colsum_ws = act(max(ops.column_sum_workspace_floats(B * (st["R"] // st["ws"]) ** 2,
+                                                            st["heads"] * st["ws"] ** 2 * st["keys_ld"])
                             for st in self.stages), dtype=torch.float32)
 
         def v2(buf, r, c):
@@ -335,7 +344,18 @@ class SwinEngine(EngineBase):
             keep.append(st["index_dev"])
             shift = ws // 2 if ws < st["R"] else 0
             st["shift"] = shift
-            st["mask_dev"] = shifted_window_mask(st["R"], st["R"], ws, shift).to(dev) if shift else None
+            mask = shifted_window_mask(st["R"], st["R"], ws, shift) if shift else None
+            if st["fused"]:
+                # (query, key) pairs in rows of 64 keys: -1 = padding (gathers -inf, which masks the padded keys)
+                pairs = torch.full((64, 64), -1, dtype=torch.int32)
+                pairs[:ws * ws, :ws * ws] = st["index"].to(torch.int32)
+                st["pairs_dev"] = pairs.reshape(-1).to(dev)
+                keep.append(st["pairs_dev"])
+                if mask is not None:
+                    padded = torch.zeros(mask.shape[0], 64, 64)
+                    padded[:, :ws * ws, :ws * ws] = mask
+                    mask = padded
+            st["mask_dev"] = mask.contiguous().to(dev) if mask is not None else None
             if st["mask_dev"] is not None:
                 keep.append(st["mask_dev"])
 
@@ -381,15 +401,22 @@ class SwinEngine(EngineBase):
                     qkv = act(rows, 3 * C)
                     lin_fwd(pre + "attn.qkv", xw, qkv)
                     fq = qkv.view(-1)
-                    Pm = act(B_, Hh, N, N)
-                    ops.batched_gemm(ctx, fq, fq[C:], Pm, N, N, D, (qkv_row, 1), (qkv_row, 1), N, (B_, Hh), qkv_b, qkv_b, s_b,
-                                     alpha=scale)
-                    bias = bias_buf[:Hh * N * N].view(Hh, N, N)
-                    ops.relpos_bias_gather(ctx, self._view(self.params, pre + "attn.relative_position_bias_table"),
-                                           st["index_dev"], bias)
-                    ops.attn_softmax_fwd(ctx, Pm, Pm, 1.0, bias=bias, mask=st["mask_dev"] if shift else None)
                     o = act(rows, C)
-                    ops.batched_gemm(ctx, Pm, fq[2 * C:], o, N, D, N, (N, 1), (1, qkv_row), C, (B_, Hh), s_b, qkv_b, o_b)
+                    if st["fused"]:
+                        Pm = act(B_ * Hh, N, 64)
+                        bias = bias_buf[:Hh * 64 * 64]
+                        ops.relpos_bias_gather_pairs(ctx, self._view(self.params, pre + "attn.relative_position_bias_table"),
+                                                     st["pairs_dev"], bias)
+                        ops.window_attn_fwd(ctx, qkv, o, Pm, bias, st["mask_dev"] if shift else None, B_, Hh, N, scale)
+                    else:
+                        Pm = act(B_, Hh, N, N)
+                        ops.batched_gemm(ctx, fq, fq[C:], Pm, N, N, D, (qkv_row, 1), (qkv_row, 1), N, (B_, Hh), qkv_b, qkv_b,
+                                         s_b, alpha=scale)
+                        bias = bias_buf[:Hh * N * N].view(Hh, N, N)
+                        ops.relpos_bias_gather(ctx, self._view(self.params, pre + "attn.relative_position_bias_table"),
+                                               st["index_dev"], bias)
+                        ops.attn_softmax_fwd(ctx, Pm, Pm, 1.0, bias=bias, mask=st["mask_dev"] if shift else None)
+                        ops.batched_gemm(ctx, Pm, fq[2 * C:], o, N, D, N, (N, 1), (1, qkv_row), C, (B_, Hh), s_b, qkv_b, o_b)
                     x1 = act(rows, C)
                     if whole:
                         lin_fwd(pre + "attn.proj", o, x1, add=x)
@@ -475,7 +502,7 @@ class SwinEngine(EngineBase):
                     t_a, t_b, t_c, t_d, t_e = (v2(g_bufs[k], rows, C) for k in spare)
                     d_f2, d_f1, d_qkv = v2(g_4c_a, rows, 4 * C), v2(g_4c_b, rows, 4 * C), v2(g_3c, rows, 3 * C)
                     fq, fg = qkv.view(-1), d_qkv.view(-1)
-                    dP = d_scores[:B_ * Hh * N * N].view(B_, Hh, N, N)
+                    dP = d_scores[:B_ * Hh * N * st["keys_ld"]].view(B_, Hh, N, st["keys_ld"])
                     # MLP
                     lin_bwd(pre + "mlp.3", f2, g, d_f2)
                     ops.gelu_bwd(ctx, d_f2, f1, d_f1, tanh_form=False)
@@ -490,18 +517,26 @@ class SwinEngine(EngineBase):
                         ops.window_partition(ctx, g1, d_pr, ws, shift, image_shape=(B, R, R, C))
                     d_o = t_c
                     lin_bwd(pre + "attn.proj", o, d_pr, d_o)
-                    ops.batched_gemm(ctx, Pm, d_o, fg[2 * C:], N, D, N, (1, N), (1, C), qkv_row, (B_, Hh), s_b, o_b, qkv_b)
-                    ops.batched_gemm(ctx, d_o, fq[2 * C:], dP, N, N, D, (C, 1), (qkv_row, 1), N, (B_, Hh), o_b, qkv_b, s_b)
-                    ops.attn_softmax_bwd(ctx, Pm, dP, dP, 1.0)
-                    dbias = dbias_buf[:Hh * N * N]
-                    with side():
-                        ops.column_sum(ctx, dP.view(B_, Hh * N * N), dbias, colsum_ws)
-                        ops.relpos_bias_scatter(ctx, dbias, st["index_dev"],
-                                                self._view(self.grads, pre + "attn.relative_position_bias_table"))
-                    ops.batched_gemm(ctx, dP, fq[C:], fg, N, D, N, (N, 1), (1, qkv_row), qkv_row, (B_, Hh), s_b, qkv_b, qkv_b,
-                                     alpha=scale)
-                    ops.batched_gemm(ctx, dP, fq, fg[C:], N, D, N, (1, N), (1, qkv_row), qkv_row, (B_, Hh), s_b, qkv_b, qkv_b,
-                                     alpha=scale)
+                    if st["fused"]:
+                        ops.window_attn_bwd(ctx, qkv, Pm, d_o, d_qkv, dP, B_, Hh, N, scale)
+                        dbias = dbias_buf[:Hh * N * 64]
+                        with side():
+                            ops.column_sum(ctx, dP.view(B_, Hh * N * 64), dbias, colsum_ws)
+                            ops.relpos_bias_scatter_pairs(ctx, dbias, st["pairs_dev"][:N * 64],
+                                                          self._view(self.grads, pre + "attn.relative_position_bias_table"))
+                    else:
+                        ops.batched_gemm(ctx, Pm, d_o, fg[2 * C:], N, D, N, (1, N), (1, C), qkv_row, (B_, Hh), s_b, o_b, qkv_b)
+                        ops.batched_gemm(ctx, d_o, fq[2 * C:], dP, N, N, D, (C, 1), (qkv_row, 1), N, (B_, Hh), o_b, qkv_b, s_b)
+                        ops.attn_softmax_bwd(ctx, Pm, dP, dP, 1.0)
+                        dbias = dbias_buf[:Hh * N * N]
+                        with side():
+                            ops.column_sum(ctx, dP.view(B_, Hh * N * N), dbias, colsum_ws)
+                            ops.relpos_bias_scatter(ctx, dbias, st["index_dev"],
+                                                    self._view(self.grads, pre + "attn.relative_position_bias_table"))
+                        ops.batched_gemm(ctx, dP, fq[C:], fg, N, D, N, (N, 1), (1, qkv_row), qkv_row, (B_, Hh), s_b, qkv_b,
+                                         qkv_b, alpha=scale)
+                        ops.batched_gemm(ctx, dP, fq, fg[C:], N, D, N, (1, N), (1, qkv_row), qkv_row, (B_, Hh), s_b, qkv_b,
+                                         qkv_b, alpha=scale)
                     d_xw = t_d
                     lin_bwd(pre + "attn.qkv", xw, d_qkv, d_xw)
                     if whole:

@@ -105,6 +105,77 @@ def _engine(cfg, dtype, **kw):
                       patch=cfg["patch"], image_size=cfg["image"], num_classes=cfg["classes"], dtype=dtype, **kw)
 
 
+def _padded_pairs(index, N):
+    """[64 * 64] int32: the bias-table entry of (query, key) in rows padded to 64 keys, -1 for padding."""
+    pad = torch.full((64, 64), -1, dtype=torch.int32)
+    pad[:N, :N] = index.to(torch.int32)
+    return pad.reshape(-1)
+
+
+@pytest.mark.parametrize("ws,heads,windows,nW,shifted", [(7, 4, 8, 4, True), (7, 2, 3, 1, False), (4, 6, 6, 2, True),
+                                                         (8, 2, 2, 1, False)])
+def test_fused_window_attention(ctx, ws, heads, windows, nW, shifted):
+    """One-launch window attention (forward, backward, bias gradient through the padded pair layout) against
+    the oracle's scores -> (+ bias, + mask) softmax -> context chain on the same bf16 inputs; bf16 bound 2e-2 of
+    the largest magnitude per tensor (4e-2 for the bias-table gradient, a sum of bf16-rounded logit gradients)."""
+    from oracle import seq_ops as Q
+    from sirius_amd import ops
+    dtype = torch.bfloat16
+    N, D, C = ws * ws, 32, heads * 32
+    g = _gen(ws * 100 + heads)
+    qkv = torch.randn(windows * N, 3 * C, generator=g).to(dtype)
+    dout = torch.randn(windows * N, C, generator=g).to(dtype)
+    table = torch.randn((2 * ws - 1) ** 2, heads, generator=g) * 0.5
+    index = S.relative_position_index(ws)
+    mask = None
+    if shifted:
+        mask = torch.where(torch.rand(nW, N, N, generator=g) < 0.3, torch.tensor(-100.0), torch.tensor(0.0))
+        mask[:, torch.arange(N), torch.arange(N)] = 0.0
+    scale = D ** -0.5
+
+    def heads_of(t):   # [windows * N, C] -> [windows, heads, N, D]
+        return t.float().cpu().view(windows, N, heads, D).permute(0, 2, 1, 3)
+    q, k, v = (heads_of(qkv[:, i * C:(i + 1) * C]).clone().requires_grad_(True) for i in range(3))
+    tab = table.clone().requires_grad_(True)
+    bias = tab[index.reshape(-1)].view(N, N, heads).permute(2, 0, 1)
+    probs_ref = Q.attn_softmax(q @ k.transpose(-1, -2), scale, bias, mask)
+    o_ref = (probs_ref @ v).permute(0, 2, 1, 3).reshape(windows * N, C)
+    dq_ref, dk_ref, dv_ref, dtab_ref = torch.autograd.grad(o_ref, (q, k, v, tab), dout.float())
+
+    pairs = _padded_pairs(index, N).cuda()
+    bias_pad = torch.zeros(heads, 64, 64, device="cuda")
+    ops.relpos_bias_gather_pairs(ctx, table.cuda(), pairs, bias_pad)
+    mask_pad = None
+    if mask is not None:
+        mask_pad = torch.zeros(nW, 64, 64)
+        mask_pad[:, :N, :N] = mask
+        mask_pad = mask_pad.cuda()
+    qkv_d, o = qkv.cuda(), torch.zeros(windows * N, C, dtype=dtype, device="cuda")
+    probs = torch.full((windows * heads, N, 64), 9.0, dtype=dtype, device="cuda")
+    ops.window_attn_fwd(ctx, qkv_d, o, probs, bias_pad, mask_pad, windows, heads, N, scale)
+    ctx.synchronize()
+    got_bias = bias_pad.cpu()
+    assert torch.equal(got_bias[:, :N, :N], bias.detach()) and torch.all(got_bias[:, :N, N:] == float("-inf"))
+    assert _rel(o, o_ref.detach()) <= 2e-2, ("context", _rel(o, o_ref.detach()))
+    assert _rel(probs.view(windows, heads, N, 64)[..., :N], probs_ref.detach()) <= 2e-2
+    assert torch.all(probs[..., N:] == 0), "padded key columns hold zero probability"
+
+    dqkv = torch.zeros_like(qkv_d)
+    ds = torch.full((windows * heads, N, 64), 9.0, dtype=dtype, device="cuda")
+    ops.window_attn_bwd(ctx, qkv_d, probs, dout.cuda(), dqkv, ds, windows, heads, N, scale)
+    dbias = torch.zeros(heads * N * 64, device="cuda")
+    ws_buf = torch.zeros(ops.column_sum_workspace_floats(windows, heads * N * 64), device="cuda")
+    ops.column_sum(ctx, ds.view(windows, heads * N * 64), dbias, ws_buf)
+    dtab = torch.zeros(table.shape, device="cuda")
+    ops.relpos_bias_scatter_pairs(ctx, dbias, pairs[:N * 64].contiguous(), dtab)
+    ctx.synchronize()
+    for name, lo, ref in (("dq", 0, dq_ref), ("dk", C, dk_ref), ("dv", 2 * C, dv_ref)):
+        err = _rel(heads_of(dqkv[:, lo:lo + C]), ref)
+        assert err <= 2e-2, (name, err)
+    assert torch.all(ds[..., N:] == 0)
+    assert _rel(dtab, dtab_ref) <= 4e-2, ("bias table gradient", _rel(dtab, dtab_ref))
+
+
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-3), (torch.bfloat16, 2e-2)])
 @pytest.mark.parametrize("name", list(CFGS))
 def test_loss_and_gradients(dtype, tol, name):
@@ -166,3 +237,31 @@ def test_swin_b_parameter_count():
     from sirius_amd.swin import SwinEngine
     eng = SwinEngine(dtype=torch.bfloat16)
     assert eng.num_parameters() == 87_768_224
+
+
+def test_fused_attention_step():
+    """The window7 configuration in bf16 has heads 32 wide: the engine takes the one-launch window attention.
+    Loss and gradients against the oracle at the bf16 bound, for the fused engine and for the same engine on
+    the unfused chain, and the two against each other."""
+    cfg = S.config(**CFGS["window7"])
+    sd = S.make_state_dict(cfg, seed=2)
+    sd = {k: (v.to(torch.bfloat16).float() if v.is_floating_point() else v) for k, v in sd.items()}
+    g = _gen(11)
+    x = torch.randn(2, 3, cfg["image"], cfg["image"], generator=g)
+    y = torch.randint(0, cfg["classes"], (2,), generator=g)
+    loss_ref, grads_ref = S.loss_and_grads(sd, x, y, cfg)
+    losses = []
+    for fused in (True, False):
+        eng = _engine(cfg, torch.bfloat16, fused_attention=fused)
+        eng.load_state_dict(sd)
+        p, cut = eng.forward_backward(x.cuda(), y.cuda())
+        assert not cut
+        loss, grads = eng.last_loss(), {k: v.clone() for k, v in eng.grads_dict().items()}
+        names = [r["name"] for r in eng.ctx.profile(p.prog, 1)]
+        assert any("window_attn" in n for n in names) == fused, names
+        assert abs(loss - loss_ref.item()) <= 2e-2 * abs(loss_ref.item()), (fused, loss, loss_ref.item())
+        for k, ref in grads_ref.items():
+            tol = 4e-2 if "relative_position_bias_table" in k else 2e-2   # sums of bf16-rounded logit gradients
+            assert _rel(grads[k], ref) <= tol, (fused, k, _rel(grads[k], ref))
+        losses.append(loss)
+    assert abs(losses[0] - losses[1]) <= 5e-3 * abs(losses[1])
