@@ -26,10 +26,6 @@ unsigned flat_blocks(int64_t items, int64_t cap = 8192) {
 // LayerNorm over the last dimension of [rows, C]
 // ---------------------------------------------------------------------------
 constexpr int kLnMaxC = 2048;  // longest row: a lane holds 32 elements of it
-template <typename T>
-struct LnChunks {
-  static constexpr int kMax = kLnMaxC / 64 / Elem<T>::kPerChunk;  // 16-byte chunks per lane and row
-};
 
 struct LnArgs {
   const void* x;
@@ -47,21 +43,43 @@ struct LnArgs {
   float eps;
 };
 
-// one wavefront per row; the row stays in registers between the passes
+// L lanes per row (L = 64: one wavefront per row, NCH 16-byte chunks per lane; L = 16 or 32: short rows, 64 / L
+// rows per wavefront, one chunk per lane); the row stays in registers between the passes
+template <int L>
+__device__ inline float row_sum(float v) {
+#pragma unroll
+  for (int off = L / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
 template <typename T>
+__device__ inline void load_params(const float* src, int c, float* out) {
+  constexpr int E = Elem<T>::kPerChunk;
+#pragma unroll
+  for (int e = 0; e < E; e += 4) {
+    const float4 t = *reinterpret_cast<const float4*>(src + c * E + e);
+    out[e] = t.x;
+    out[e + 1] = t.y;
+    out[e + 2] = t.z;
+    out[e + 3] = t.w;
+  }
+}
+
+template <typename T, int NCH, int L>
 __global__ __launch_bounds__(256) void ln_fwd_kernel(LnArgs p) {
   constexpr int E = Elem<T>::kPerChunk;
-  constexpr int kLnMaxChunks = LnChunks<T>::kMax;
+  constexpr int RPW = 64 / L;   // rows per wavefront
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int64_t row = static_cast<int64_t>(blockIdx.x) * 4 + wave;
-  if (row >= p.rows) return;
+  const int sub = lane % L;
+  const int64_t row = (static_cast<int64_t>(blockIdx.x) * 4 + wave) * RPW + lane / L;
+  const bool live = row < p.rows;
   const uint4* src = static_cast<const uint4*>(p.x) + row * p.cc;
-  float v[kLnMaxChunks][E];
+  float v[NCH][E];
   float s = 0.f;
 #pragma unroll
-  for (int j = 0; j < kLnMaxChunks; ++j) {
-    const int c = lane + j * 64;
-    if (c < p.cc) {
+  for (int j = 0; j < NCH; ++j) {
+    const int c = sub + j * L;
+    if (live && c < p.cc) {
       Chunk ch;
       ch.u = src[c];
       chunk_to_float<T>(ch, v[j]);
@@ -69,11 +87,11 @@ __global__ __launch_bounds__(256) void ln_fwd_kernel(LnArgs p) {
       for (int e = 0; e < E; ++e) s += v[j][e];
     }
   }
-  const float mean = wave_sum(s) / static_cast<float>(p.C);
+  const float mean = row_sum<L>(s) / static_cast<float>(p.C);
   float q = 0.f;
 #pragma unroll
-  for (int j = 0; j < kLnMaxChunks; ++j) {
-    if (lane + j * 64 < p.cc) {
+  for (int j = 0; j < NCH; ++j) {
+    if (live && sub + j * L < p.cc) {
 #pragma unroll
       for (int e = 0; e < E; ++e) {
         const float d = v[j][e] - mean;
@@ -81,55 +99,68 @@ __global__ __launch_bounds__(256) void ln_fwd_kernel(LnArgs p) {
       }
     }
   }
-  const float rstd = 1.0f / sqrtf(wave_sum(q) / static_cast<float>(p.C) + p.eps);
-  if (lane == 0) {
+  const float rstd = 1.0f / sqrtf(row_sum<L>(q) / static_cast<float>(p.C) + p.eps);
+  if (!live) return;
+  if (sub == 0) {
     p.mean[row] = mean;
     p.rstd[row] = rstd;
   }
   uint4* dst = static_cast<uint4*>(p.out) + row * p.cc;
 #pragma unroll
-  for (int j = 0; j < kLnMaxChunks; ++j) {
-    const int c = lane + j * 64;
+  for (int j = 0; j < NCH; ++j) {
+    const int c = sub + j * L;
     if (c < p.cc) {
-      float o[E];
+      float o[E], ga[E], be[E];
+      load_params<T>(p.gamma, c, ga);
+      load_params<T>(p.beta, c, be);
 #pragma unroll
-      for (int e = 0; e < E; ++e) o[e] = (v[j][e] - mean) * rstd * p.gamma[c * E + e] + p.beta[c * E + e];
+      for (int e = 0; e < E; ++e) o[e] = (v[j][e] - mean) * rstd * ga[e] + be[e];
       dst[c] = float_to_chunk<T>(o).u;
     }
   }
 }
 
-// dx per row; the column sums for dgamma / dbeta are kept per lane over the rows a wave
-// walks, then summed over the four waves through LDS: one partial row per workgroup
-template <typename T>
+// dx per row; the column sums for dgamma / dbeta are kept per lane over the rows its row group walks, then
+// summed over the 4 * 64 / L row groups of the workgroup through LDS: one partial row per workgroup
+template <typename T, int NCH, int L>
 __global__ __launch_bounds__(256) void ln_bwd_kernel(LnArgs p) {
   constexpr int E = Elem<T>::kPerChunk;
-  constexpr int kLnMaxChunks = LnChunks<T>::kMax;
-  __shared__ float red[4][kLnMaxC * 2];
+  constexpr int RPW = 64 / L;
+  constexpr int GROUPS = 4 * RPW;
+  constexpr int COLS = NCH * L * E;      // columns a row group covers
+  __shared__ float red[GROUPS][COLS * 2];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  float dg[kLnMaxChunks][E], db[kLnMaxChunks][E], gam[kLnMaxChunks][E];
+  const int sub = lane % L, group = wave * RPW + lane / L;
+  float dg[NCH][E], db[NCH][E], gam[NCH][E];
 #pragma unroll
-  for (int j = 0; j < kLnMaxChunks; ++j)
+  for (int j = 0; j < NCH; ++j) {
+    const int c = sub + j * L;
 #pragma unroll
-    for (int e = 0; e < E; ++e) {
-      dg[j][e] = db[j][e] = 0.f;
-      const int c = lane + j * 64;
-      gam[j][e] = c < p.cc ? p.gamma[c * E + e] : 0.f;
-    }
+    for (int e = 0; e < E; ++e) dg[j][e] = db[j][e] = gam[j][e] = 0.f;
+    if (c < p.cc) load_params<T>(p.gamma, c, gam[j]);
+  }
   const int64_t r0 = static_cast<int64_t>(blockIdx.x) * p.rows_per_wg;
   int64_t r1 = r0 + p.rows_per_wg;
   if (r1 > p.rows) r1 = p.rows;
   const float inv_c = 1.0f / static_cast<float>(p.C);
-  for (int64_t row = r0 + wave; row < r1; row += 4) {
+  // rows_per_wg is a multiple of GROUPS, so the groups of a wavefront stay in step (the row sums below are
+  // taken by all lanes); a group beyond the last row works on nothing
+  for (int64_t base = r0; base < r1; base += GROUPS) {
+    const int64_t row = base + group;
+    const bool live = row < r1;
     const uint4* xs = static_cast<const uint4*>(p.x) + row * p.cc;
     const uint4* gs = static_cast<const uint4*>(p.dy) + row * p.cc;
-    const float mean = p.mean[row], rstd = p.rstd[row];
-    float xh[kLnMaxChunks][E], g[kLnMaxChunks][E];
+    float mean = 0.f, rstd = 0.f;
+    if (live) {
+      mean = p.mean[row];
+      rstd = p.rstd[row];
+    }
+    float xh[NCH][E], g[NCH][E];
     float a = 0.f, b = 0.f;
 #pragma unroll
-    for (int j = 0; j < kLnMaxChunks; ++j) {
-      const int c = lane + j * 64;
-      if (c < p.cc) {
+    for (int j = 0; j < NCH; ++j) {
+      const int c = sub + j * L;
+      if (live && c < p.cc) {
         Chunk cx, cg;
         cx.u = xs[c];
         cg.u = gs[c];
@@ -146,12 +177,13 @@ __global__ __launch_bounds__(256) void ln_bwd_kernel(LnArgs p) {
         }
       }
     }
-    a = wave_sum(a) * inv_c;
-    b = wave_sum(b) * inv_c;
+    a = row_sum<L>(a) * inv_c;
+    b = row_sum<L>(b) * inv_c;
+    if (!live) continue;
     uint4* dst = static_cast<uint4*>(p.out) + row * p.cc;
 #pragma unroll
-    for (int j = 0; j < kLnMaxChunks; ++j) {
-      const int c = lane + j * 64;
+    for (int j = 0; j < NCH; ++j) {
+      const int c = sub + j * L;
       if (c < p.cc) {
         float o[E];
 #pragma unroll
@@ -169,20 +201,21 @@ __global__ __launch_bounds__(256) void ln_bwd_kernel(LnArgs p) {
     }
   }
 #pragma unroll
-  for (int j = 0; j < kLnMaxChunks; ++j)
+  for (int j = 0; j < NCH; ++j)
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-      red[wave][((j * 64 + lane) * E + e) * 2] = dg[j][e];
-      red[wave][((j * 64 + lane) * E + e) * 2 + 1] = db[j][e];
+      red[group][((j * L + sub) * E + e) * 2] = dg[j][e];
+      red[group][((j * L + sub) * E + e) * 2 + 1] = db[j][e];
     }
   __syncthreads();
-  // column col lives at chunk c = col / E -> (j = c / 64, lane = c % 64), element col % E
+  // column col lives at chunk c = col / E = j * L + sub, element col % E: position col of a group's row
   for (int col = threadIdx.x; col < p.C; col += 256) {
-    const int c = col / E, e = col - c * E;
-    const int j = c >> 6, l = c & 63;
-    const int at = ((j * 64 + l) * E + e) * 2;
-    const float sg = red[0][at] + red[1][at] + red[2][at] + red[3][at];
-    const float sb = red[0][at + 1] + red[1][at + 1] + red[2][at + 1] + red[3][at + 1];
+    float sg = 0.f, sb = 0.f;
+#pragma unroll
+    for (int gidx = 0; gidx < GROUPS; ++gidx) {
+      sg += red[gidx][col * 2];
+      sb += red[gidx][col * 2 + 1];
+    }
     float2* dst = reinterpret_cast<float2*>(p.partial + (static_cast<int64_t>(blockIdx.x) * p.C + col) * 2);
     *dst = make_float2(sg, sb);
   }
@@ -474,10 +507,42 @@ int check_rows(const char* what, int dtype, int64_t rows, int C) {
   return 0;
 }
 
+// rows per workgroup of the backward: about 1024 workgroups, a multiple of 16 (the most rows a workgroup takes
+// in one pass, with 16 lanes per row)
 int ln_rows_per_wg(int64_t rows) {
   int64_t r = (rows + 1023) / 1024;
-  r = (r + 3) / 4 * 4;
-  return static_cast<int>(r < 4 ? 4 : r);
+  r = (r + 15) / 16 * 16;
+  return static_cast<int>(r);
+}
+
+// lanes per row and chunks per lane for rows of cc 16-byte chunks
+struct LnShape {
+  int lanes, nch;
+};
+LnShape ln_shape(int cc) {
+  if (cc <= 16) return {16, 1};
+  if (cc <= 32) return {32, 1};
+  return {64, (cc + 63) / 64};
+}
+
+template <typename T, bool BWD>
+void (*ln_kernel_for(LnShape sh))(LnArgs) {
+  if (sh.lanes == 16) return BWD ? ln_bwd_kernel<T, 1, 16> : ln_fwd_kernel<T, 1, 16>;
+  if (sh.lanes == 32) return BWD ? ln_bwd_kernel<T, 1, 32> : ln_fwd_kernel<T, 1, 32>;
+  switch (sh.nch) {
+    case 1:
+      return BWD ? ln_bwd_kernel<T, 1, 64> : ln_fwd_kernel<T, 1, 64>;
+    case 2:
+      return BWD ? ln_bwd_kernel<T, 2, 64> : ln_fwd_kernel<T, 2, 64>;
+    case 3:
+      return BWD ? ln_bwd_kernel<T, 3, 64> : ln_fwd_kernel<T, 3, 64>;
+    default:
+      break;
+  }
+  if constexpr (sizeof(T) == 2) return BWD ? ln_bwd_kernel<T, 4, 64> : ln_fwd_kernel<T, 4, 64>;
+  if (sh.nch <= 4) return BWD ? ln_bwd_kernel<T, 4, 64> : ln_fwd_kernel<T, 4, 64>;
+  if (sh.nch <= 6) return BWD ? ln_bwd_kernel<T, 6, 64> : ln_fwd_kernel<T, 6, 64>;
+  return BWD ? ln_bwd_kernel<T, 8, 64> : ln_fwd_kernel<T, 8, 64>;
 }
 
 }  // namespace
@@ -495,9 +560,10 @@ int layernorm_fwd(Context* ctx, int dtype, const void* x, void* y, const float* 
   TCH_CHECK_ARG(x && y && gamma && beta && mean && rstd, "layernorm_fwd: null tensor");
   LnArgs a{x, nullptr, nullptr, y, gamma, beta, mean, rstd, nullptr, rows, C, C / E, 0, eps};
   const double bytes = static_cast<double>(rows) * C * (dtype == kBF16 ? 4.0 : 8.0);
-  const dim3 grid(static_cast<unsigned>((rows + 3) / 4));
-  return dtype == kBF16 ? launch(ctx, ln_fwd_kernel<bf16>, grid, dim3(256), a, "ln_fwd_kernel<bf16>", bytes, 1)
-                        : launch(ctx, ln_fwd_kernel<float>, grid, dim3(256), a, "ln_fwd_kernel<f32>", bytes, 1);
+  const LnShape sh = ln_shape(a.cc);
+  const dim3 grid(static_cast<unsigned>((rows + 4 * (64 / sh.lanes) - 1) / (4 * (64 / sh.lanes))));
+  return dtype == kBF16 ? launch(ctx, ln_kernel_for<bf16, false>(sh), grid, dim3(256), a, "ln_fwd_kernel<bf16>", bytes, 1)
+                        : launch(ctx, ln_kernel_for<float, false>(sh), grid, dim3(256), a, "ln_fwd_kernel<f32>", bytes, 1);
 }
 
 int layernorm_bwd(Context* ctx, int dtype, const void* dy, const void* x, void* dx, const void* residual, const float* gamma,
@@ -512,8 +578,9 @@ int layernorm_bwd(Context* ctx, int dtype, const void* dy, const void* x, void* 
   LnArgs a{x,    dy,   residual, dx, gamma, nullptr, const_cast<float*>(mean), const_cast<float*>(rstd), partial,
            rows, C,    C / E,    rpw, 0.f};
   const double bytes = static_cast<double>(rows) * C * (dtype == kBF16 ? 6.0 : 12.0);
-  int rc = dtype == kBF16 ? launch(ctx, ln_bwd_kernel<bf16>, dim3(blocks), dim3(256), a, "ln_bwd_kernel<bf16>", bytes, 1)
-                          : launch(ctx, ln_bwd_kernel<float>, dim3(blocks), dim3(256), a, "ln_bwd_kernel<f32>", bytes, 1);
+  const LnShape sh = ln_shape(a.cc);
+  int rc = dtype == kBF16 ? launch(ctx, ln_kernel_for<bf16, true>(sh), dim3(blocks), dim3(256), a, "ln_bwd_kernel<bf16>", bytes, 1)
+                          : launch(ctx, ln_kernel_for<float, true>(sh), dim3(blocks), dim3(256), a, "ln_bwd_kernel<f32>", bytes, 1);
   if (rc) return rc;
   ColSumArgs s{partial, dgamma, dbeta, blocks, C, accumulate};
   return launch(ctx, col_sum_kernel, dim3((C + 7) / 8), dim3(256), s, "col_sum_kernel", 8.0 * blocks * C, 1);
