@@ -168,6 +168,11 @@ int64_t tch_conv2d_wgrad_workspace_bytes(int dtype, int K, int R, int S, int C, 
 int tch_conv2d_wgrad(tch_context* ctx, int dtype, const void* x, const void* dy, float* dw, float* workspace,
                      int splits, int accumulate, int N, int H, int W, int C, int K, int R, int S, int stride,
                      int pad, int tile_cfg, int c_logical);
+/* The same, and dbias[K] (fp32) (+)= sum over pixels of dy: weight and bias gradient of a linear layer
+ * (torch.nn.Linear's backward under train/gpt2.py:26 and train/swin_b.py:38) in one pass over dy. */
+int tch_conv2d_wgrad_bias(tch_context* ctx, int dtype, const void* x, const void* dy, float* dw, float* dbias,
+                          float* workspace, int splits, int accumulate, int N, int H, int W, int C, int K, int R, int S,
+                          int stride, int pad, int tile_cfg, int c_logical);
 
 /* ---- BatchNorm (training mode) with fused ReLU / residual ---------------------- */
 int64_t tch_bn_workspace_bytes(int dtype, int64_t rows, int C);

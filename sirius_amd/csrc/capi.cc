@@ -398,6 +398,14 @@ int tch_conv2d_wgrad(tch_context* ctx, int dtype, const void* x, const void* dy,
   return conv2d_wgrad(C(ctx), dtype, s, x, dy, dw, workspace, splits, accumulate, tile_cfg);
 }
 
+int tch_conv2d_wgrad_bias(tch_context* ctx, int dtype, const void* x, const void* dy, float* dw, float* dbias,
+                          float* workspace, int splits, int accumulate, int N, int H, int W, int Cc, int K, int R, int S,
+                          int stride, int pad, int tile_cfg, int c_logical) {
+  ConvShape s = shape(N, H, W, Cc, K, R, S, stride, pad, c_logical);
+  if (splits <= 0) splits = workspace ? conv2d_wgrad_pick_splits(s, dtype) : 1;
+  return conv2d_wgrad(C(ctx), dtype, s, x, dy, dw, workspace, splits, accumulate, tile_cfg, dbias);
+}
+
 int64_t tch_bn_workspace_bytes(int dtype, int64_t rows, int Cc) { return bn_workspace_bytes(rows, Cc, dtype); }
 
 int tch_bn_fwd_train(tch_context* ctx, int dtype, const void* x, void* y, const void* residual, int relu,

@@ -51,6 +51,7 @@ struct IgemmArgs {
   const void* add;    // optional addend, laid out like out (FWD/DGRAD)
   const void* mask;   // optional: addend counts only where mask > 0
   const float* bias;  // optional per-column bias (FWD)
+  float* dbias;       // WGRAD, optional: column sums of dy (the gradient of that bias), [splits][K] partials or final
   float* stats;       // optional: per (row tile, column) pair of sums over the stored output (see finish_tile)
   const void* bn_mask;      // DGRAD with stats, optional: the stored output is zeroed where bn_mask <= 0
   const void* bn_x;         // DGRAD with stats: input of the BatchNorm this gradient flows into, laid out like out
@@ -710,11 +711,27 @@ __global__ __launch_bounds__(WM* WN * 64) void wgrad_kernel(IgemmArgs p) {
     }
   };
 
+  // The bias gradient of a linear layer is the column sum of dy: the workgroups of the first column tile add
+  // up the dy chunks they stage anyway (every pixel of the split passes through exactly once).
+  const bool sum_dy = p.dbias != nullptr && tile_n == 0;
+  float bsum[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) bsum[e] = 0.f;
+
   auto store_tiles = [&](int buf, const Chunk* ra, const Chunk* rb) {
 #pragma unroll
     for (int i = 0; i < A_PT; ++i) lds_a[(buf * BKP + a_prow + i * (NT / CA)) * LDA + a_cc] = ra[i].u;
 #pragma unroll
     for (int i = 0; i < B_PT; ++i) lds_b[(buf * BKP + b_prow + i * (NT / CB)) * LDB + b_cc] = rb[i].u;
+    if (sum_dy) {
+#pragma unroll
+      for (int i = 0; i < A_PT; ++i) {
+        float v[E];
+        chunk_to_float<T>(ra[i], v);
+#pragma unroll
+        for (int e = 0; e < E; ++e) bsum[e] += v[e];
+      }
+    }
   };
 
   f32x16_t acc[TM][TN];
@@ -819,6 +836,21 @@ __global__ __launch_bounds__(WM* WN * 64) void wgrad_kernel(IgemmArgs p) {
     }
     store_floats<E>(dst, v);
   });
+  if (sum_dy) {
+    // NT / CA threads hold partial sums of the same E channels: through LDS, then one thread per channel
+    float* red = reinterpret_cast<float*>(lds);
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < E; ++e) red[a_prow * BM + a_cc * E + e] = bsum[e];
+    __syncthreads();
+    if (tid < BM && m0 + tid < p.gemm_m) {
+      float s = 0.f;
+#pragma unroll
+      for (int r = 0; r < NT / CA; ++r) s += red[r * BM + tid];
+      float* dst = p.dbias + (p.splits > 1 ? static_cast<int64_t>(split) * p.gemm_m : 0) + m0 + tid;
+      *dst = accumulate ? *dst + s : s;
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -1049,9 +1081,22 @@ struct ReduceArgs {
   int64_t n;
   int splits;
   int accumulate;
+  // optional second, short vector reduced by the workgroups from first_blocks on (the bias gradient)
+  const float* partial2;
+  float* out2;
+  int n2;
+  unsigned first_blocks;
 };
 
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(ReduceArgs p) {
+  if (blockIdx.x >= p.first_blocks) {
+    const int i = (blockIdx.x - p.first_blocks) * 256 + threadIdx.x;
+    if (i >= p.n2) return;
+    float s = 0.f;
+    for (int k = 0; k < p.splits; ++k) s += p.partial2[static_cast<int64_t>(k) * p.n2 + i];
+    p.out2[i] = p.accumulate ? p.out2[i] + s : s;
+    return;
+  }
   int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
   if (i >= p.n) return;
   float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -1341,7 +1386,8 @@ int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, co
 int64_t conv2d_wgrad_workspace_bytes(const ConvShape& s, int dtype, int splits) {
   if (splits <= 1) return 0;
   (void)dtype;
-  return static_cast<int64_t>(splits) * s.K * s.R * s.S * s.C * 4;
+  // partial filters, then partial column sums of dy for callers that also want the bias gradient
+  return static_cast<int64_t>(splits) * (static_cast<int64_t>(s.K) * s.R * s.S * s.C + s.K) * 4;
 }
 
 int conv2d_wgrad_pick_splits(const ConvShape& s, int dtype) {
@@ -1366,7 +1412,7 @@ int conv2d_wgrad_pick_splits(const ConvShape& s, int dtype) {
 }
 
 int conv2d_wgrad(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* dy, float* dw, float* workspace,
-                 int splits, int accumulate, int tile_cfg) {
+                 int splits, int accumulate, int tile_cfg, float* dbias) {
   IgemmArgs a{};
   if (int rc = fill_common(a, s, dtype)) return rc;
   TCH_CHECK_ARG(x && dy && dw, "conv2d_wgrad: null tensor");
@@ -1388,6 +1434,8 @@ int conv2d_wgrad(Context* ctx, int dtype, const ConvShape& s, const void* x, con
   a.k_per_split = per;
   a.accumulate = accumulate;
   a.out = splits > 1 ? static_cast<void*>(workspace) : static_cast<void*>(dw);
+  float* dbias_partial = workspace ? workspace + static_cast<int64_t>(splits) * a.gemm_m * a.gemm_n : nullptr;
+  a.dbias = !dbias ? nullptr : splits > 1 ? dbias_partial : dbias;
   a.div_plane = FastDiv(a.Ho * a.Wo);
   a.div_width = FastDiv(a.Wo);
   if (tile_cfg < 0) {
@@ -1397,9 +1445,11 @@ int conv2d_wgrad(Context* ctx, int dtype, const ConvShape& s, const void* x, con
                           : launch_mode<float, kWgrad>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo));
   if (rc) return rc;
   if (splits > 1) {
-    ReduceArgs r{workspace, dw, static_cast<int64_t>(a.gemm_m) * a.gemm_n, splits, accumulate};
+    ReduceArgs r{workspace, dw, static_cast<int64_t>(a.gemm_m) * a.gemm_n, splits, accumulate, dbias_partial, dbias,
+                 dbias ? a.gemm_m : 0, 0u};
     TCH_CHECK_ARG(r.n % 4 == 0, "conv2d_wgrad: filter size must be a multiple of 4");
-    unsigned blocks = static_cast<unsigned>((r.n / 4 + 255) / 256);
+    r.first_blocks = static_cast<unsigned>((r.n / 4 + 255) / 256);
+    const unsigned blocks = r.first_blocks + static_cast<unsigned>((r.n2 + 255) / 256);
     return launch(ctx, splitk_reduce_kernel, dim3(blocks), dim3(256), r, "splitk_reduce_kernel",
                   4.0 * r.n * (splits + 1 + (accumulate ? 1 : 0)), 1);
   }

@@ -58,8 +58,9 @@ int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, co
 int conv2d_dgrad_stat_rows(const ConvShape& s, int dtype, int tile_cfg);
 int conv2d_wgrad_pick_splits(const ConvShape& s, int dtype);
 int64_t conv2d_wgrad_workspace_bytes(const ConvShape& s, int dtype, int splits);
+// dbias (optional, [K] fp32): also the column sums of dy, i.e. the gradient of a bias added to the output
 int conv2d_wgrad(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* dy, float* dw,
-                 float* workspace, int splits, int accumulate, int tile_cfg);
+                 float* workspace, int splits, int accumulate, int tile_cfg, float* dbias = nullptr);
 
 // bn.hip -- training-mode BatchNorm over [rows, C] with fused ReLU / residual
 int bn_partial_rows(int64_t rows, int C, int dtype);  // number of row blocks the reductions use

@@ -226,7 +226,6 @@ class GPT2Engine(EngineBase):
                 sp = int(ops.lib().tch_conv2d_wgrad_pick_splits(code, R, 1, 1, Cin, K, 1, 1, 1, 0))
                 ws_bytes = max(ws_bytes, ops.conv2d_wgrad_workspace_bytes(code, K, 1, 1, Cin, sp))
         wg_ws = act(ws_bytes // 4, dtype=torch.float32)
-        bias_ws = act(64 * 4 * C, dtype=torch.float32)   # row-slab partial sums of the bias gradients
 
         def ln_stats(i):
             return ln_mean[i * R:(i + 1) * R], ln_rstd[i * R:(i + 1) * R]
@@ -255,8 +254,8 @@ class GPT2Engine(EngineBase):
         def lin_bwd(name, x, dy, dx):
             """dW, db from (x, dy); dx = dy W"""
             with side():
-                ops.conv2d_wgrad(ctx, as4(x), as4(dy), self._view(self.grads, name + ".weight"), 1, 0, workspace=wg_ws)
-                ops.bias_grad(ctx, dy, self._view(self.grads, name + ".bias"), workspace=bias_ws)
+                ops.conv2d_wgrad(ctx, as4(x), as4(dy), self._view(self.grads, name + ".weight"), 1, 0, workspace=wg_ws,
+                                 dbias=self._view(self.grads, name + ".bias"))
             ops.conv2d_dgrad(ctx, as4(dy), self._wt(name + ".weight"), as4(dx), 1, 0)
 
         # strides / batch offsets of head h of sample b inside the packed projection and the score tensor

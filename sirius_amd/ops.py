@@ -292,7 +292,9 @@ def conv2d_wgrad_workspace_bytes(dtype, K, R, S, C, splits):
     return int(lib().tch_conv2d_wgrad_workspace_bytes(dtype, K, R, S, C, splits))
 
 
-def conv2d_wgrad(ctx, x, dy, dw, stride, pad, workspace=None, splits=0, accumulate=False, tile_cfg=-1, c_logical=0):
+def conv2d_wgrad(ctx, x, dy, dw, stride, pad, workspace=None, splits=0, accumulate=False, tile_cfg=-1, c_logical=0,
+                 dbias=None):
+    """dw (+)= dy^T x over the pixels; with dbias [K] fp32 also dbias (+)= column sums of dy."""
     N, H, W, C = x.shape
     K, R, S, C2 = dw.shape
     assert C == C2 and dw.dtype == torch.float32
@@ -303,6 +305,12 @@ def conv2d_wgrad(ctx, x, dy, dw, stride, pad, workspace=None, splits=0, accumula
             splits = conv2d_wgrad_splits(x, K, R, S, stride, pad)
         need = conv2d_wgrad_workspace_bytes(dtype_code(x), K, R, S, C, splits)
         assert workspace.numel() * workspace.element_size() >= need, "wgrad workspace too small"
+    if dbias is not None:
+        assert dbias.dtype == torch.float32 and dbias.numel() == K
+        check(lib().tch_conv2d_wgrad_bias(ctx.handle, dtype_code(x), _p(x), _p(dy), _p(dw), _p(dbias), _p(workspace),
+                                          splits, int(accumulate), N, H, W, C, K, R, S, stride, pad, tile_cfg, c_logical),
+              "tch_conv2d_wgrad_bias")
+        return
     check(lib().tch_conv2d_wgrad(ctx.handle, dtype_code(x), _p(x), _p(dy), _p(dw), _p(workspace), splits,
                                  int(accumulate), N, H, W, C, K, R, S, stride, pad, tile_cfg, c_logical),
           "tch_conv2d_wgrad")

@@ -295,9 +295,8 @@ class SwinEngine(EngineBase):
 
         def lin_bwd(name, x, dy, dx, bias=True):
             with side():
-                ops.conv2d_wgrad(ctx, as4(x), as4(dy), self._view(self.grads, name + ".weight"), 1, 0, workspace=wg_ws)
-                if bias:
-                    ops.bias_grad(ctx, dy, self._view(self.grads, name + ".bias"), workspace=bias_ws)
+                ops.conv2d_wgrad(ctx, as4(x), as4(dy), self._view(self.grads, name + ".weight"), 1, 0, workspace=wg_ws,
+                                 dbias=self._view(self.grads, name + ".bias") if bias else None)
             if dx is not None:
                 ops.conv2d_dgrad(ctx, as4(dy), self._wt(name + ".weight"), as4(dx), 1, 0)
 

@@ -142,10 +142,19 @@ def test_conv_wgrad(ctx, dtype, case, splits):
     ops.conv2d_wgrad(ctx, x.cuda(), dy.cuda(), dw, st, pad, workspace=ws, splits=splits)
     torch.cuda.synchronize()
     close(dw, ref, dtype, "conv wgrad", rtol=1e-3 if dtype == torch.float32 else 5e-3)
-    # accumulate: a second pass adds the same gradient on top
-    ops.conv2d_wgrad(ctx, x.cuda(), dy.cuda(), dw, st, pad, workspace=ws, splits=splits, accumulate=True)
+    # accumulate: a second pass adds the same gradient on top; this one also asks for the bias gradient
+    # (column sums of dy), first plain into a filled buffer, then accumulated
+    db_ref = dy.float().sum(dim=(0, 1, 2))
+    db = torch.full((K,), -3.0, dtype=torch.float32, device="cuda")
+    dw2 = torch.full((K, R, S, C), 7.0, dtype=torch.float32, device="cuda")
+    ops.conv2d_wgrad(ctx, x.cuda(), dy.cuda(), dw2, st, pad, workspace=ws, splits=splits, dbias=db)
+    torch.cuda.synchronize()
+    assert torch.equal(dw2, dw), "asking for the bias gradient changes the filter gradient"
+    close(db, db_ref, torch.float32, "bias gradient", rtol=1e-4)
+    ops.conv2d_wgrad(ctx, x.cuda(), dy.cuda(), dw, st, pad, workspace=ws, splits=splits, accumulate=True, dbias=db)
     torch.cuda.synchronize()
     close(dw, 2 * ref, dtype, "conv wgrad accumulate", rtol=1e-3 if dtype == torch.float32 else 5e-3)
+    close(db, 2 * db_ref, torch.float32, "bias gradient accumulate", rtol=1e-4)
 
 
 BN_CASES = [(2 * 14 * 14, 64), (4 * 28 * 28, 128), (3 * 7 * 7, 2048), (37, 8), (100000, 64)]
