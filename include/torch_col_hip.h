@@ -313,6 +313,12 @@ int tch_relpos_bias_gather_pairs(tch_context* ctx, const float* table, const int
 int tch_relpos_bias_scatter_pairs(tch_context* ctx, const float* dbias, const int32_t* index, float* dtable, int heads,
                                   int pairs, int entries, int accumulate);
 
+/* The scatter through the inverse of the index, built once by the caller: table entry e receives the pairs
+ * list[ptr[e]] .. list[ptr[e + 1] - 1] (pair numbers below `pairs`, ptr non-decreasing, both on the device),
+ * summed in list order. */
+int tch_relpos_bias_scatter_csr(tch_context* ctx, const float* dbias, const int32_t* ptr, const int32_t* list,
+                                float* dtable, int heads, int pairs, int entries, int accumulate);
+
 /* Swin-B data movement (train/swin_b_tiny.py:8-19,116-131; patch merging and shift as in torchvision's swin_b,
  * train/swin_b.py:38).
  * reverse == 0: dst[windows of window x window tokens] = roll(src[B,H,W,C], -shift) partitioned;

@@ -312,6 +312,11 @@ int tch_relpos_bias_scatter_pairs(tch_context* ctx, const float* dbias, const in
   return relpos_bias_scatter_pairs(C(ctx), dbias, index, dtable, heads, pairs, entries, accumulate);
 }
 
+int tch_relpos_bias_scatter_csr(tch_context* ctx, const float* dbias, const int32_t* ptr, const int32_t* list,
+                                float* dtable, int heads, int pairs, int entries, int accumulate) {
+  return relpos_bias_scatter_csr(C(ctx), dbias, ptr, list, dtable, heads, pairs, entries, accumulate);
+}
+
 int tch_flash_attn_fwd(tch_context* ctx, int dtype, const void* q, const void* k, const void* v, void* o, float* lse,
                        int B, int H, int T, int64_t qkv_rs, int64_t qkv_bs, int64_t o_rs, int64_t o_bs, float scale,
                        int causal) {

@@ -437,7 +437,7 @@ int bias_grad(Context* ctx, int dtype, const void* dy, float* dbias, int rows, i
   BiasGradArgs a{dy, dbias, rows, cols, ld, accumulate, nullptr, rows};
   const double bytes = static_cast<double>(rows) * cols * (dtype == kBF16 ? 2.0 : 4.0);
   const int E = dtype == kBF16 ? 8 : 4;
-  if (rows >= 256 && cols % E == 0 && ld % E == 0 && (reinterpret_cast<uintptr_t>(dy) & 15) == 0) {
+  if (rows >= 32 && cols % E == 0 && ld % E == 0 && (reinterpret_cast<uintptr_t>(dy) & 15) == 0) {
     // with scratch memory the rows are cut into slabs (more workgroups), summed by a second small launch
     int slabs = 1;
     if (workspace) {

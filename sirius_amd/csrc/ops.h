@@ -129,6 +129,10 @@ int relpos_bias_gather_pairs(Context* ctx, const float* table, const int32_t* in
                              int entries);
 int relpos_bias_scatter_pairs(Context* ctx, const float* dbias, const int32_t* index, float* dtable, int heads, int pairs,
                               int entries, int accumulate);
+// scatter through the inverse of the index (ptr [entries + 1], list of pair numbers per entry; the caller
+// vouches that every listed pair is below `pairs` and ptr is non-decreasing)
+int relpos_bias_scatter_csr(Context* ctx, const float* dbias, const int32_t* ptr, const int32_t* list, float* dtable,
+                            int heads, int pairs, int entries, int accumulate);
 int64_t column_sum_workspace_floats(int rows, int cols);
 int column_sum(Context* ctx, int dtype, const void* x, float* out, int rows, int cols, int accumulate, float* workspace);
 

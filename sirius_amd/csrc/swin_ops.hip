@@ -155,6 +155,30 @@ __global__ __launch_bounds__(64) void relpos_scatter_kernel(RelPosArgs p) {
   }
 }
 
+// the same from a precomputed inverse of the index: entry e receives the pairs list[ptr[e] .. ptr[e+1]), summed
+// by one wavefront per (entry, head) in a fixed order
+struct RelPosCsrArgs {
+  const float* dbias;    // [heads][pairs]
+  const int32_t* ptr;    // [entries + 1]
+  const int32_t* list;   // [ptr[entries]] pair numbers
+  float* dtable;         // [entries][heads]
+  int heads, pairs, entries, accumulate;
+};
+
+__global__ __launch_bounds__(256) void relpos_scatter_csr_kernel(RelPosCsrArgs p) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (t >= p.entries * p.heads) return;
+  const int entry = t / p.heads, h = t - entry * p.heads;
+  const int end = p.ptr[entry + 1];
+  float s = 0.f;
+  for (int i = p.ptr[entry] + lane; i < end; i += 64) s += p.dbias[static_cast<int64_t>(h) * p.pairs + p.list[i]];
+  s = wave_sum(s);
+  if (lane == 0) {
+    float* dst = p.dtable + t;
+    *dst = p.accumulate ? *dst + s : s;
+  }
+}
+
 struct ColSumArgs {
   const void* x;   // [rows][cols], T
   float* partial;  // [slabs][cols]
@@ -242,6 +266,14 @@ int relpos_bias_scatter_pairs(Context* ctx, const float* dbias, const int32_t* i
   RelPosArgs a{nullptr, index, nullptr, dbias, dtable, heads, pairs, entries, accumulate};
   return launch(ctx, relpos_scatter_kernel, dim3(entries * heads), dim3(64), a, "relpos_scatter_kernel",
                 4.0 * entries * heads * a.nn, 1);
+}
+
+int relpos_bias_scatter_csr(Context* ctx, const float* dbias, const int32_t* ptr, const int32_t* list, float* dtable,
+                            int heads, int pairs, int entries, int accumulate) {
+  TCH_CHECK_ARG(dbias && ptr && list && dtable && heads > 0 && pairs > 0 && entries > 0, "relpos_bias_scatter_csr: bad arguments");
+  RelPosCsrArgs a{dbias, ptr, list, dtable, heads, pairs, entries, accumulate};
+  return launch(ctx, relpos_scatter_csr_kernel, dim3((entries * heads + 3) / 4), dim3(256), a,
+                "relpos_scatter_csr_kernel", 8.0 * heads * pairs, 1);
 }
 
 int64_t column_sum_workspace_floats(int rows, int cols) {

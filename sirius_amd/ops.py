@@ -713,6 +713,28 @@ def relpos_bias_scatter_pairs(ctx, dbias, index, dtable, accumulate=False):
                                               int(accumulate)), "tch_relpos_bias_scatter_pairs")
 
 
+def relpos_inverse_index(index, entries):
+    """(ptr [entries + 1], list) int32 on the CPU: list[ptr[e]:ptr[e + 1]] are the positions of `index` (any
+    shape, negative = padding) that hold e, in ascending order."""
+    flat = index.reshape(-1).to(torch.int64).cpu()
+    pos = torch.nonzero(flat >= 0).reshape(-1)
+    order = torch.argsort(flat[pos], stable=True)
+    counts = torch.bincount(flat[pos], minlength=entries)
+    assert counts.numel() == entries, "index refers to entries beyond the table"
+    ptr = torch.zeros(entries + 1, dtype=torch.int64)
+    ptr[1:] = torch.cumsum(counts, 0)
+    return ptr.to(torch.int32), pos[order].to(torch.int32)
+
+
+def relpos_bias_scatter_csr(ctx, dbias, ptr, pair_list, dtable, pairs, accumulate=False):
+    """dtable[e, h] (+)= sum of dbias[h, pair] over pair in list[ptr[e]:ptr[e + 1]] (relpos_inverse_index)."""
+    entries, heads = dtable.shape
+    assert dbias.numel() == heads * pairs and dbias.dtype == dtable.dtype == torch.float32
+    assert ptr.dtype == pair_list.dtype == torch.int32 and ptr.numel() == entries + 1
+    check(lib().tch_relpos_bias_scatter_csr(ctx.handle, _p(dbias), _p(ptr), _p(pair_list), _p(dtable), heads, pairs,
+                                            entries, int(accumulate)), "tch_relpos_bias_scatter_csr")
+
+
 def window_attn_fwd(ctx, qkv, o, probs, bias, mask, windows, heads, N, scale):
     """Window attention forward in one launch (bf16, heads 32 wide, N <= 64): qkv [windows * N, 3C] ->
     o [windows * N, C]; probs [windows * heads, N, 64] keeps the probabilities; bias [heads, 64, 64] fp32 with -inf

@@ -349,6 +349,9 @@ class SwinEngine(EngineBase):
                 pairs = torch.full((64, 64), -1, dtype=torch.int32)
                 pairs[:ws * ws, :ws * ws] = st["index"].to(torch.int32)
                 st["pairs_dev"] = pairs.reshape(-1).to(dev)
+                ptr, plist = ops.relpos_inverse_index(pairs[:ws * ws], (2 * self.window - 1) ** 2)
+                st["inv_ptr_dev"], st["inv_list_dev"] = ptr.to(dev), plist.to(dev)
+                keep += [st["inv_ptr_dev"], st["inv_list_dev"]]
                 keep.append(st["pairs_dev"])
                 if mask is not None:
                     padded = torch.zeros(mask.shape[0], 64, 64)
@@ -520,9 +523,12 @@ class SwinEngine(EngineBase):
                         ops.window_attn_bwd(ctx, qkv, Pm, d_o, d_qkv, dP, B_, Hh, N, scale)
                         dbias = dbias_buf[:Hh * N * 64]
                         with side():
-                            ops.column_sum(ctx, dP.view(B_, Hh * N * 64), dbias, colsum_ws)
-                            ops.relpos_bias_scatter_pairs(ctx, dbias, st["pairs_dev"][:N * 64],
-                                                          self._view(self.grads, pre + "attn.relative_position_bias_table"))
+                            # the sum over the windows in 16-byte pieces (rows are a multiple of 8 wide), then
+                            # each table entry collects its pairs through the inverse index
+                            ops.bias_grad(ctx, dP.view(B_, Hh * N * 64), dbias, workspace=colsum_ws)
+                            ops.relpos_bias_scatter_csr(ctx, dbias, st["inv_ptr_dev"], st["inv_list_dev"],
+                                                        self._view(self.grads, pre + "attn.relative_position_bias_table")
+                                                        .view(-1, Hh), N * 64)
                     else:
                         ops.batched_gemm(ctx, Pm, d_o, fg[2 * C:], N, D, N, (1, N), (1, C), qkv_row, (B_, Hh), s_b, o_b, qkv_b)
                         ops.batched_gemm(ctx, d_o, fq[2 * C:], dP, N, N, D, (C, 1), (qkv_row, 1), N, (B_, Hh), o_b, qkv_b, s_b)

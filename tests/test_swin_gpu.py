@@ -168,7 +168,14 @@ def test_fused_window_attention(ctx, ws, heads, windows, nW, shifted):
     ops.column_sum(ctx, ds.view(windows, heads * N * 64), dbias, ws_buf)
     dtab = torch.zeros(table.shape, device="cuda")
     ops.relpos_bias_scatter_pairs(ctx, dbias, pairs[:N * 64].contiguous(), dtab)
+    # the same through the inverse index (entry -> its pairs), on top of a filled table
+    ptr, plist = ops.relpos_inverse_index(pairs[:N * 64].view(N, 64), table.shape[0])
+    assert int(ptr[-1]) == N * N and torch.equal(pairs.cpu()[plist.long()].long(),
+                                                 torch.repeat_interleave(torch.arange(table.shape[0]), (ptr[1:] - ptr[:-1]).long()))
+    dtab2 = torch.ones(table.shape, device="cuda")
+    ops.relpos_bias_scatter_csr(ctx, dbias, ptr.cuda(), plist.cuda(), dtab2, N * 64, accumulate=True)
     ctx.synchronize()
+    assert _rel(dtab2 - 1.0, dtab.cpu()) <= 1e-5
     for name, lo, ref in (("dq", 0, dq_ref), ("dk", C, dk_ref), ("dv", 2 * C, dv_ref)):
         err = _rel(heads_of(dqkv[:, lo:lo + C]), ref)
         assert err <= 2e-2, (name, err)
