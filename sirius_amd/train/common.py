@@ -31,6 +31,7 @@ class PeerScript:
         self.at = dict(at)
         self.delay_ms = delay_ms
         self.sent = []
+        self._threads = []
 
     def on_batch(self, idx):
         cmd = self.at.pop(idx, None)
@@ -53,9 +54,14 @@ class PeerScript:
             {"l1": self.server.colocate_l1, "l2": self.server.colocate_l2, "exit": self.server.infer_exit,
              "cus": self.server.set_infer_required_cus}[kind](bs)
             self.sent.append((t, kind, bs))
-        threading.Thread(target=fire, daemon=True).start()
+        t = threading.Thread(target=fire, daemon=True)
+        self._threads.append(t)
+        t.start()
 
     def stop(self):
+        # a command still on its way must not reach the communicator after the runtime is shut down
+        for t in self._threads:
+            t.join(timeout=5.0)
         self.server.stop()
 
 
