@@ -56,19 +56,20 @@ struct FlashArgs {
 };
 
 // a [64][64] bf16 tile: global -> registers (two 16-byte chunks per thread) -> LDS rows of kRowB bytes
-__device__ inline void tile_load(const bf16* base, int64_t rs, int tid, Chunk (&r)[2]) {
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int q = tid + 256 * i;
-    r[i].u = *reinterpret_cast<const uint4*>(base + static_cast<int64_t>(q >> 3) * rs + (q & 7) * 8);
-  }
+struct TileRegs {
+  uint4 lo, hi;   // rows tid / 8 and 32 + tid / 8, slot tid % 8 (plain members: an array here ends up in scratch)
+};
+__device__ inline TileRegs tile_load(const bf16* base, int64_t rs, int tid) {
+  const bf16* src = base + static_cast<int64_t>(tid >> 3) * rs + (tid & 7) * 8;
+  TileRegs r;
+  r.lo = *reinterpret_cast<const uint4*>(src);
+  r.hi = *reinterpret_cast<const uint4*>(src + 32 * rs);
+  return r;
 }
-__device__ inline void tile_store(unsigned char* lds, int tid, const Chunk (&r)[2]) {
-#pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int q = tid + 256 * i;
-    *reinterpret_cast<uint4*>(lds + (q >> 3) * kRowB + (q & 7) * 16) = r[i].u;
-  }
+__device__ inline void tile_store(unsigned char* lds, int tid, const TileRegs& r) {
+  unsigned char* dst = lds + (tid >> 3) * kRowB + (tid & 7) * 16;
+  *reinterpret_cast<uint4*>(dst) = r.lo;
+  *reinterpret_cast<uint4*>(dst + 32 * kRowB) = r.hi;
 }
 
 // this wave's fragments of 32 fixed rows (row = first + lane % 32): 4 chunks cover the lane half's 32 columns
@@ -144,9 +145,8 @@ __global__ __launch_bounds__(256) void flash_query_kernel(FlashArgs p) {
   const int steps = CAUSAL ? (q0 + kFixed) / kWalk : p.T / kWalk;
   const bf16* kbase = p.k + qkv_off;
   const bf16* vbase = p.v + qkv_off;
-  Chunk rk[2], rv[2];
-  tile_load(kbase, p.qkv_rs, tid, rk);
-  tile_load(vbase, p.qkv_rs, tid, rv);
+  TileRegs rk = tile_load(kbase, p.qkv_rs, tid);
+  TileRegs rv = tile_load(vbase, p.qkv_rs, tid);
 
   f32x16_t acc[2];
   zero_acc(acc[0]);
@@ -159,9 +159,11 @@ __global__ __launch_bounds__(256) void flash_query_kernel(FlashArgs p) {
     tile_store(kt, tid, rk);
     tile_store(vt, tid, rv);
     __syncthreads();
-    if (kb + 1 < steps) {
-      tile_load(kbase + static_cast<int64_t>(kb + 1) * kWalk * p.qkv_rs, p.qkv_rs, tid, rk);
-      tile_load(vbase + static_cast<int64_t>(kb + 1) * kWalk * p.qkv_rs, p.qkv_rs, tid, rv);
+    {
+      // the last step fetches its own tile again rather than branching around the loads
+      const int64_t next = static_cast<int64_t>(kb + 1 < steps ? kb + 1 : kb) * kWalk * p.qkv_rs;
+      rk = tile_load(kbase + next, p.qkv_rs, tid);
+      rv = tile_load(vbase + next, p.qkv_rs, tid);
     }
     const int k0 = kb * kWalk;
     if (CAUSAL && k0 > qw0 + 31) continue;   // nothing of this tile is visible to this wave's queries
@@ -181,33 +183,40 @@ __global__ __launch_bounds__(256) void flash_query_kernel(FlashArgs p) {
     const bool diagonal = CAUSAL && k0 + kWalk - 1 > qw0;   // some key of the tile lies beyond some query
     float pr[2][16];
     if (!DQ) {
+      // running maximum on the raw scores (the scale is positive), then exp2(s * c - m * c) as one fused
+      // multiply-add and one exponential per score
       float bmax = -INFINITY;
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          float v = s[t][r] * c;
+          float v = s[t][r];
           if (diagonal && k0 + 32 * t + 8 * (r >> 2) + 4 * half + (r & 3) > query) v = -INFINITY;
           pr[t][r] = v;
           bmax = fmaxf(bmax, v);
         }
       bmax = fmaxf(bmax, __shfl_xor(bmax, 32, 64));
       const float m_new = fmaxf(m, bmax);
-      const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+      const bool moved = m_new != m;
+      const float alpha = __builtin_amdgcn_exp2f((m - m_new) * c);
       m = m_new;
+      const float mc = m_new * c;
       float sum = 0.f;
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          pr[t][r] = __builtin_amdgcn_exp2f(pr[t][r] - m_new);
+          pr[t][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(pr[t][r], c, -mc));
           sum += pr[t][r];
         }
       l = l * alpha + sum;
+      // after the first tiles the maxima seldom move: the accumulators are rescaled only when one in the wave did
+      if (__any(moved)) {
 #pragma unroll
-      for (int ct = 0; ct < 2; ++ct)
+        for (int ct = 0; ct < 2; ++ct)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) acc[ct][e] *= alpha;
+          for (int e = 0; e < 16; ++e) acc[ct][e] *= alpha;
+      }
     } else {
 #pragma unroll
       for (int t = 0; t < 2; ++t)
@@ -233,7 +242,7 @@ __global__ __launch_bounds__(256) void flash_query_kernel(FlashArgs p) {
   if (!DQ) {
     l += __shfl_xor(l, 32, 64);
     mul = 1.f / l;
-    if (half == 0) p.lse[static_cast<int64_t>(bh) * p.T + query] = (m + __builtin_amdgcn_logf(l)) * kLn2;
+    if (half == 0) p.lse[static_cast<int64_t>(bh) * p.T + query] = m * p.scale + __builtin_amdgcn_logf(l) * kLn2;
   }
   __syncthreads();   // every wave is done with the tiles: the space becomes four output patches
   store_fixed(acc, mul, lds + wave * 32 * kRowB, p.out + (DQ ? qkv_off : o_off), DQ ? p.qkv_rs : p.o_rs, qw0, lane);
@@ -267,11 +276,11 @@ __global__ __launch_bounds__(256) void flash_key_kernel(FlashArgs p) {
   const bf16* dobase = p.dout + o_off;
   const float* lse = p.lse + static_cast<int64_t>(bh) * p.T;
   const float* dlt = p.delta + static_cast<int64_t>(bh) * p.T;
-  Chunk rq[2], rd[2];
+  TileRegs rq, rd;
   float rstat = 0.f;
   auto fetch = [&](int qb) {
-    tile_load(qbase + static_cast<int64_t>(qb) * kWalk * p.qkv_rs, p.qkv_rs, tid, rq);
-    tile_load(dobase + static_cast<int64_t>(qb) * kWalk * p.o_rs, p.o_rs, tid, rd);
+    rq = tile_load(qbase + static_cast<int64_t>(qb) * kWalk * p.qkv_rs, p.qkv_rs, tid);
+    rd = tile_load(dobase + static_cast<int64_t>(qb) * kWalk * p.o_rs, p.o_rs, tid);
     if (tid < kWalk) rstat = lse[qb * kWalk + tid] * kLog2e;
     else if (tid < 2 * kWalk) rstat = dlt[qb * kWalk + tid - kWalk];
   };
@@ -290,7 +299,7 @@ __global__ __launch_bounds__(256) void flash_key_kernel(FlashArgs p) {
     tile_store(dot, tid, rd);
     if (tid < 2 * kWalk) stat[tid >> 6][tid & 63] = rstat;
     __syncthreads();
-    if (qb + 1 < steps) fetch(qb + 1);
+    fetch(qb + 1 < steps ? qb + 1 : qb);   // the last step fetches its own tile again: no branch around the loads
     const int q0 = qb * kWalk;
     if (CAUSAL && q0 + kWalk - 1 < kw0) continue;   // every staged query lies before this wave's keys
 
