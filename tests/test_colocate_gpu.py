@@ -3,7 +3,7 @@ memory, checkpoint hooks, and the 64 -> 16 -> 64 handover with an in-process pee
 
 Bars: offsets and integer bookkeeping bit-exact against the CPU model of the pool; the engine on
 pool memory bit-exact against the engine on torch memory (same kernels, same inputs); handover
-request -> AdjustL1Done under 50 ms (BASELINE's bound for the path)."""
+request -> AdjustL1Done under 50 ms (the bound the reference states for the path)."""
 import ctypes
 import os
 import random
