@@ -134,3 +134,28 @@ def test_fused_attention_step():
             assert _rel(grads[k], ref) <= 2e-2, (fused, k, _rel(grads[k], ref))
         results.append((loss, grads))
     assert abs(results[0][0] - results[1][0]) <= 5e-3 * abs(results[1][0])
+
+
+def test_gpt2_small_widths_two_layers():
+    """GPT-2 small's real widths (768 channels, 12 heads of 64, vocabulary 50 257 padded to 50 304, tied head) at two
+    layers and 2 x 128 tokens in bf16: the shapes the benchmark step runs (fused attention, cross entropy with
+    the row in registers, projections on the direct-to-LDS kernel), against the oracle at the bf16 bound."""
+    from sirius_amd.gpt2 import GPT2Engine
+    cfg = dict(vocab=50257, n_pos=128, n_embd=768, n_layer=2, n_head=12)
+    sd = G.make_state_dict(cfg["vocab"], cfg["n_pos"], cfg["n_embd"], cfg["n_layer"], seed=4)
+    sd = {k: v.to(torch.bfloat16).float() for k, v in sd.items()}
+    g = torch.Generator()
+    g.manual_seed(12)
+    ids = torch.randint(0, cfg["vocab"], (2, 128), generator=g)
+    loss_ref, grads_ref = G.loss_and_grads(sd, ids, cfg["n_head"], cfg["n_layer"])
+    eng = GPT2Engine(seq_len=128, dtype=torch.bfloat16, **cfg)
+    eng.load_state_dict(sd)
+    p, cut = eng.forward_backward(ids.cuda())
+    assert not cut
+    loss, grads = eng.last_loss(), eng.grads_dict()
+    assert abs(loss - loss_ref.item()) <= 2e-2 * abs(loss_ref.item()), (loss, loss_ref.item())
+    worst = max((_rel(grads[k], ref), k) for k, ref in grads_ref.items())
+    print("worst gradient", worst, flush=True)
+    for k, ref in grads_ref.items():
+        assert torch.isfinite(grads[k]).all(), k
+        assert _rel(grads[k], ref) <= 2e-2, (k, _rel(grads[k], ref))
