@@ -1051,26 +1051,32 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm2_kernel(IgemmArgs p) {
   constexpr int WAIT_IMM = (AHEAD & 0xF) | ((AHEAD >> 4) << 14) | (0x7 << 4) | (0xF << 8);
   static_assert(AHEAD < 64, "vmcnt range");
 
+  // One step = wait until only the newer tiles' loads are outstanding (then this wave's part of tile kt has
+  // landed; near the end fewer newer tiles exist, so wait for everything), barrier (every wave's part is in
+  // LDS and every wave is done with tile kt-1), request the tile NBUF-1 steps ahead into the buffer that just
+  // became free, multiply.  The main loop takes NBUF steps per trip with the buffer index a constant and the
+  // multiply outside every conditional (inside one, the compiler moves the 64 accumulators between register
+  // classes in every step); the last nk % NBUF steps follow one by one.
+  auto step = [&](int kt, int u) {
+    if (kt + NBUF - 1 <= nk)
+      __builtin_amdgcn_s_waitcnt(WAIT_IMM);
+    else
+      __builtin_amdgcn_s_waitcnt((0x7 << 4) | (0xF << 8));
+    __syncthreads();
+    if (kt + NBUF - 1 < nk) issue_loads((u + NBUF - 1) % NBUF);
+    compute(u);
+  };
 #pragma unroll
   for (int s = 0; s < NBUF - 1; ++s)
     if (s < nk) issue_loads(s);
-  for (int kt0 = 0; kt0 < nk; kt0 += NBUF) {
+  int kt0 = 0;
+  for (; kt0 + NBUF <= nk; kt0 += NBUF) {
 #pragma unroll
-    for (int u = 0; u < NBUF; ++u) {
-      const int kt = kt0 + u;
-      if (kt < nk) {
-        // tile kt has landed for this wave once only the newer tiles' loads are outstanding; near the
-        // end fewer newer tiles exist, so wait for everything
-        if (kt + NBUF - 1 <= nk)
-          __builtin_amdgcn_s_waitcnt(WAIT_IMM);
-        else
-          __builtin_amdgcn_s_waitcnt((0x7 << 4) | (0xF << 8));
-        __syncthreads();  // every wave's part of tile kt is in LDS, and every wave is done with tile kt-1
-        if (kt + NBUF - 1 < nk) issue_loads((u + NBUF - 1) % NBUF);
-        compute(u);
-      }
-    }
+    for (int u = 0; u < NBUF; ++u) step(kt0 + u, u);
   }
+#pragma unroll
+  for (int u = 0; u < NBUF - 1; ++u)
+    if (kt0 + u < nk) step(kt0 + u, u);
 
   finish_tile<T, MODE, WM, WN, TM, TN>(p, acc, reinterpret_cast<float*>(lds), tid, m0, n0, tile_m);
 }
