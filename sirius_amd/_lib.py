@@ -8,7 +8,8 @@ import os
 import re
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libtorch_col_hip.so")
+# TCH_LIBRARY_PATH names another build of the same library (e.g. to compare two builds on one machine)
+LIB_PATH = os.environ.get("TCH_LIBRARY_PATH") or os.path.join(_HERE, "lib", "libtorch_col_hip.so")
 INCLUDE_DIR = os.path.join(os.path.dirname(_HERE), "include")
 HEADERS = ("torch_col_hip.h", "torch_col_host.h")
 
