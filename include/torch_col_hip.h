@@ -72,7 +72,9 @@ typedef struct tch_kernel_stat {
   double total_ms;    /* summed HIP-event time of its launches over all repetitions */
   double work;        /* summed ALGORITHMIC work of those launches: flops or bytes */
   int64_t launches;
-  int work_is_bytes;  /* 1: work counts bytes (HBM-bound kernel), 0: flops (MFMA-bound) */
+  int work_is_bytes;  /* 1: work counts bytes (HBM-bound kernel), 0: flops (MFMA kernel) */
+  double bytes;       /* summed ALGORITHMIC bytes of those launches (equals work when work counts bytes; 0 where a
+                         flops-annotated kernel states none): flops / peak against bytes / bandwidth tells which roof binds */
 } tch_kernel_stat;
 /* Replays prog `reps` times directly on the context's stream (not through a launch queue)
  * with a HIP event between any two launches; one row per kernel name. */

@@ -23,7 +23,7 @@ class TorchColHipError(RuntimeError):
 class KernelStat(ctypes.Structure):
     """Mirror of tch_kernel_stat (include/torch_col_hip.h)."""
     _fields_ = [("name", ctypes.c_char * 96), ("total_ms", ctypes.c_double), ("work", ctypes.c_double),
-                ("launches", ctypes.c_int64), ("work_is_bytes", ctypes.c_int)]
+                ("launches", ctypes.c_int64), ("work_is_bytes", ctypes.c_int), ("bytes", ctypes.c_double)]
 
 
 class CtrlMsg(ctypes.Structure):

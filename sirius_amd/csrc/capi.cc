@@ -519,6 +519,7 @@ extern "C" int tch_program_profile(tch_context* ctx, const tch_program* prog, in
     o.work = s.work;
     o.launches = s.launches;
     o.work_is_bytes = s.work_is_bytes;
+    o.bytes = s.bytes;
   }
   *n_out = n;
   return 0;

@@ -435,7 +435,7 @@ hipStream_t cu_partition_stream(int n_cus, int lane) {
 }
 
 int submit(Context* ctx, const void* fn, dim3 grid, dim3 block, const void* args, size_t arg_bytes,
-           const char* name, double work, int work_is_bytes) {
+           const char* name, double work, int work_is_bytes, double bytes) {
   if (!ctx) {
     set_error("null context");
     return -22;
@@ -452,6 +452,7 @@ int submit(Context* ctx, const void* fn, dim3 grid, dim3 block, const void* args
   rec.name = name;
   rec.work = work;
   rec.work_is_bytes = work_is_bytes;
+  rec.bytes = work_is_bytes ? work : bytes;
   memcpy(rec.args, args, arg_bytes);
   rec.lane = 0;
   rec.op = kOpLaunch;
@@ -510,6 +511,7 @@ int profile_program(Context* ctx, const Program& prog, int reps, std::vector<Ker
       k.work += l.work;
       k.launches += 1;
       k.work_is_bytes = l.work_is_bytes;
+      k.bytes += l.bytes;
     }
   }
   for (auto e : ev) (void)hipEventDestroy(e);

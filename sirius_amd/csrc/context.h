@@ -145,6 +145,7 @@ struct KernelStat {
   double work = 0.0;  // sum of the algorithmic work of the launches
   int64_t launches = 0;
   int work_is_bytes = 1;
+  double bytes = 0.0;  // sum of the algorithmic bytes of the launches (0 where a flops-annotated launch gave none)
 };
 
 // Replays prog `reps` times directly on the context's stream with a HIP event between any

@@ -1139,6 +1139,19 @@ const char* igemm_name() {
   return name.c_str();
 }
 
+// Algorithmic bytes of one convolution launch: each operand read once, the result written once (the partial
+// results of a split reduction are the kernel's own choice and do not count).  Many of these layers do fewer
+// flops per byte than the chip can feed, so the profiler is told the bytes beside the flops.
+template <int MODE>
+double conv_bytes(const IgemmArgs& a, int eb) {
+  const double x = static_cast<double>(a.N) * a.H * a.W * a.C, y = static_cast<double>(a.N) * a.Ho * a.Wo * a.K;
+  const double w = static_cast<double>(a.K) * a.R * a.S * a.C;
+  if (MODE == kWgrad) return (x + y) * eb + w * 4;
+  const double out = MODE == kFwd ? y : x;
+  const int extra = (a.add ? 1 : 0) + (a.add && a.mask ? 1 : 0) + (a.bn_x ? 1 : 0) + (a.bn_mask ? 1 : 0);
+  return ((MODE == kFwd ? x : y) + w + out * extra) * eb + out * (a.out_f32 ? 4 : eb);
+}
+
 template <typename T, int MODE, int WM, int WN, int TM, int TN>
 int launch_cfg(Context* ctx, IgemmArgs& a, double flops) {
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
@@ -1151,10 +1164,11 @@ int launch_cfg(Context* ctx, IgemmArgs& a, double flops) {
   }
   const dim3 grid(static_cast<unsigned>(wgs)), block(WM * WN * 64);
   if constexpr (MODE == kWgrad)
-    return launch(ctx, wgrad_kernel<T, WM, WN, TM, TN>, grid, block, a, igemm_name<T, MODE, WM, WN, TM, TN>(), flops, 0);
+    return launch(ctx, wgrad_kernel<T, WM, WN, TM, TN>, grid, block, a, igemm_name<T, MODE, WM, WN, TM, TN>(), flops, 0,
+                  conv_bytes<MODE>(a, sizeof(T)));
   else
     return launch(ctx, igemm_kernel<T, MODE, WM, WN, TM, TN>, grid, block, a, igemm_name<T, MODE, WM, WN, TM, TN>(),
-                  flops, 0);
+                  flops, 0, conv_bytes<MODE>(a, sizeof(T)));
 }
 
 template <int MODE, int WM, int WN, int TM, int TN, int NBUF>
@@ -1170,7 +1184,7 @@ int launch_cfg2(Context* ctx, IgemmArgs& a, double flops) {
     return -22;
   }
   return launch(ctx, igemm2_kernel<MODE, WM, WN, TM, TN, NBUF>, dim3(static_cast<unsigned>(wgs)), dim3(WM * WN * 64), a,
-                name.c_str(), flops, 0);
+                name.c_str(), flops, 0, conv_bytes<MODE>(a, 2));
 }
 
 // TCH_IGEMM2 = 0 keeps every convolution on igemm_kernel; 2 or 3 picks the number of LDS tiles

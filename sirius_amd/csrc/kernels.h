@@ -188,6 +188,9 @@ struct LaunchRecord {
   const char* name;
   double work;
   int work_is_bytes;
+  // for a launch annotated with flops: its algorithmic bytes as well (0 = not given), so that a reader can
+  // tell which of the two roofs binds it
+  double bytes;
   // A recorded program is a valid serial order of launches.  `lane` 1 marks launches that may
   // run beside the lane-0 ones on a second stream; `op` says how the lanes meet:
   //   kOpLaunch       plain launch on its lane
@@ -202,16 +205,16 @@ enum LaunchOp : int { kOpLaunch = 0, kOpLaunchAfter = 1, kOpJoin = 2 };
 class Context;  // defined in context.h
 
 int submit(Context* ctx, const void* fn, dim3 grid, dim3 block, const void* args, size_t arg_bytes,
-           const char* name, double work, int work_is_bytes);
+           const char* name, double work, int work_is_bytes, double bytes = 0.0);
 
 // name must have static storage duration
 template <typename Args>
 inline int launch(Context* ctx, void (*kernel)(Args), dim3 grid, dim3 block, const Args& args,
-                  const char* name = "kernel", double work = 0.0, int work_is_bytes = 1) {
+                  const char* name = "kernel", double work = 0.0, int work_is_bytes = 1, double bytes = 0.0) {
   static_assert(sizeof(Args) <= sizeof(LaunchRecord::args), "kernel argument struct too large");
   static_assert(std::is_trivially_copyable<Args>::value, "kernel arguments must be POD");
   return submit(ctx, reinterpret_cast<const void*>(kernel), grid, block, &args, sizeof(Args), name, work,
-                work_is_bytes);
+                work_is_bytes, bytes);
 }
 
 void set_error(const std::string& msg);

@@ -131,7 +131,8 @@ class Context:
 
     def profile(self, program, reps=1):
         """Per-kernel HIP-event timing of `reps` replays: list of dicts with name, total_ms,
-        launches, work (algorithmic flops or bytes, summed) and work_is_bytes."""
+        launches, work (algorithmic flops or bytes, summed), work_is_bytes and bytes (algorithmic bytes,
+        summed; 0 where a kernel annotated with flops states none)."""
         from ._lib import KernelStat
         cap = 256
         buf = (KernelStat * cap)()
@@ -139,7 +140,7 @@ class Context:
         check(lib().tch_program_profile(self.handle, program.handle, reps, buf, cap, ctypes.byref(n)),
               "tch_program_profile")
         return [dict(name=buf[i].name.decode(), total_ms=buf[i].total_ms, launches=int(buf[i].launches),
-                     work=buf[i].work, work_is_bytes=bool(buf[i].work_is_bytes)) for i in range(n.value)]
+                     work=buf[i].work, work_is_bytes=bool(buf[i].work_is_bytes), bytes=buf[i].bytes) for i in range(n.value)]
 
 
 # ---------------------------------------------------------------------------
