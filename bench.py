@@ -288,7 +288,7 @@ def main():
                   if r["total_ms"] > 0 else None,
                   **({} if r["work_is_bytes"] or r["total_ms"] <= 0 else
                      {"GB/s": round(r["bytes"] / (r["total_ms"] * 1e-3) / 1e9, 2)})}
-                 for r in rows[:12]]
+                 for r in rows[:24]]
 
     out = {
         "metric": METRIC,

@@ -125,23 +125,29 @@ struct FwdFinalizeArgs {
   float momentum, eps;
 };
 
-// Sum the per-row-block partials of one channel: 8 channels x 32 lanes per workgroup, each
-// lane strides over the row blocks in fp64, then a tree over the 32 lanes through LDS.
+// Sum the per-row-block partials of one channel: 8 channels x 128 lanes per workgroup (thread = lane * 8 +
+// channel, so the 8 channels of a row block are one 64-byte piece).  What this costs is its count of
+// dependent round trips to L2, so every lane requests 16 row blocks at once: up to 2048 row blocks are one
+// trip.  The lanes add up in fp64 in a fixed order: own values, the 8 lanes of a wavefront by exchange, the
+// 16 wavefronts through LDS.
+constexpr int kFinalizeThreads = 1024;
 __device__ inline bool finalize_sums(const float* partial, int row_blocks, int C, int c, int lane, double* s_out,
                                      double* q_out) {
-  __shared__ double red[32][8][2];
+  constexpr int LANES = kFinalizeThreads / 8, WAVES = kFinalizeThreads / 64;
+  __shared__ double red[WAVES][8][2];
   double s = 0.0, q = 0.0;
   if (c < C) {
-    // eight loads in flight per lane: what this loop costs is its count of dependent round trips
-    constexpr int U = 8;
-    for (int b = lane; b < row_blocks; b += U * 32) {
+    constexpr int U = 16;
+    for (int b = lane; b < row_blocks; b += U * LANES) {
       float2 v[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const int bb = b + u * 32;
-        v[u] = bb < row_blocks ? *reinterpret_cast<const float2*>(partial + (static_cast<int64_t>(bb) * C + c) * 2)
-                               : make_float2(0.f, 0.f);
+        const int bb = b + u * LANES;   // past the end: the last row block again, counted as zero
+        v[u] = *reinterpret_cast<const float2*>(partial + (static_cast<int64_t>(bb < row_blocks ? bb : row_blocks - 1) * C + c) * 2);
       }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (b + u * LANES >= row_blocks) v[u] = make_float2(0.f, 0.f);
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         s += v[u].x;
@@ -149,23 +155,29 @@ __device__ inline bool finalize_sums(const float* partial, int row_blocks, int C
       }
     }
   }
-  const int cl = threadIdx.x & 7;
-  red[lane][cl][0] = s;
-  red[lane][cl][1] = q;
-  __syncthreads();
-  for (int off = 16; off > 0; off >>= 1) {
-    if (lane < off) {
-      red[lane][cl][0] += red[lane + off][cl][0];
-      red[lane][cl][1] += red[lane + off][cl][1];
-    }
-    __syncthreads();
+#pragma unroll
+  for (int off = 8; off < 64; off <<= 1) {
+    s += __shfl_xor(s, off, 64);
+    q += __shfl_xor(q, off, 64);
   }
-  *s_out = red[0][cl][0];
-  *q_out = red[0][cl][1];
+  const int cl = threadIdx.x & 7, wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) < 8) {
+    red[wave][cl][0] = s;
+    red[wave][cl][1] = q;
+  }
+  __syncthreads();
+  s = q = 0.0;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) {
+    s += red[w][cl][0];
+    q += red[w][cl][1];
+  }
+  *s_out = s;
+  *q_out = q;
   return lane == 0 && c < C;
 }
 
-__global__ __launch_bounds__(256) void bn_fwd_finalize_kernel(FwdFinalizeArgs p) {
+__global__ __launch_bounds__(kFinalizeThreads) void bn_fwd_finalize_kernel(FwdFinalizeArgs p) {
   const int c = blockIdx.x * 8 + (threadIdx.x & 7);
   double s, q;
   if (!finalize_sums(p.partial, p.row_blocks, p.C, c, threadIdx.x >> 3, &s, &q)) return;
@@ -199,7 +211,7 @@ struct BwdFinalizeArgs {
   int accumulate;
 };
 
-__global__ __launch_bounds__(256) void bn_bwd_finalize_kernel(BwdFinalizeArgs p) {
+__global__ __launch_bounds__(kFinalizeThreads) void bn_bwd_finalize_kernel(BwdFinalizeArgs p) {
   const int c = blockIdx.x * 8 + (threadIdx.x & 7);
   double s1, s2;
   if (!finalize_sums(p.partial, p.row_blocks, p.C, c, threadIdx.x >> 3, &s1, &s2)) return;
@@ -322,18 +334,27 @@ __global__ __launch_bounds__(256) void bn_fin_apply_kernel(FinApplyArgs p) {
   {
     const int pr = tid & 31, part = tid >> 5;
     double s0 = 0.0, q0 = 0.0, s1 = 0.0, q1 = 0.0;
-    constexpr int U = 8;
+    constexpr int U = 16;   // 128 row blocks per round trip
+    // uniform base + 32-bit lane offset: one address register per request
+    const float* base = p.partial + static_cast<int64_t>(c0) * 2;
+    const uint32_t stride = static_cast<uint32_t>(p.C) * 2;   // floats per row block
     for (int b = part; b < p.row_blocks; b += 8 * U) {
       float4 v[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
+        // every request is made (a row block past the end repeats the last one and counts as zero): a
+        // conditional request would be a branch of its own
         const int bb = b + 8 * u;
-        v[u] = bb < p.row_blocks
-                   ? *reinterpret_cast<const float4*>(p.partial + (static_cast<int64_t>(bb) * p.C + c0 + 2 * pr) * 2)
-                   : make_float4(0.f, 0.f, 0.f, 0.f);
+        const uint32_t off = static_cast<uint32_t>(bb < p.row_blocks ? bb : p.row_blocks - 1) * stride + 4u * pr;
+        v[u] = *reinterpret_cast<const float4*>(base + off);
       }
 #pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (b + 8 * u >= p.row_blocks) v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
       for (int u = 0; u < U; ++u) {
+        // keeps the conversions to fp64 next to their additions (hoisted, they would cost 2 registers per value)
+        if (u % 4 == 0) __builtin_amdgcn_sched_barrier(0);
         s0 += v[u].x;
         q0 += v[u].y;
         s1 += v[u].z;
@@ -403,29 +424,20 @@ __global__ __launch_bounds__(256) void bn_fin_apply_kernel(FinApplyArgs p) {
   const int64_t r0 = static_cast<int64_t>(blockIdx.y) * p.rows_per_slab;
   int64_t r1 = r0 + p.rows_per_slab;
   if (r1 > p.rows) r1 = p.rows;
-  for (int64_t r = r0 + ty; r < r1; r += RPP) {
-    const int64_t i = r * cc + col_chunk;
-    Chunk ca;
-    ca.u = static_cast<const uint4*>(p.a)[i];
-    float va[E], vo[E];
+  const bool has_b = BWD || p.b != nullptr;
+  auto finish = [&](int64_t i, const Chunk& ca, const Chunk& cb) {
+    float va[E], vb[E], vo[E];
     chunk_to_float<T>(ca, va);
+    chunk_to_float<T>(cb, vb);
     if (BWD) {
-      Chunk cx;
-      cx.u = static_cast<const uint4*>(p.b)[i];
-      float vx[E];
-      chunk_to_float<T>(cx, vx);
 #pragma unroll
-      for (int e = 0; e < E; ++e) vo[e] = k0[e] * va[e] + k1[e] * vx[e] + k2[e];
+      for (int e = 0; e < E; ++e) vo[e] = k0[e] * va[e] + k1[e] * vb[e] + k2[e];
     } else {
 #pragma unroll
       for (int e = 0; e < E; ++e) vo[e] = va[e] * k0[e] + k1[e];
       if (p.b) {
-        Chunk cr;
-        cr.u = static_cast<const uint4*>(p.b)[i];
-        float vr[E];
-        chunk_to_float<T>(cr, vr);
 #pragma unroll
-        for (int e = 0; e < E; ++e) vo[e] += vr[e];
+        for (int e = 0; e < E; ++e) vo[e] += vb[e];
       }
       if (p.relu) {
 #pragma unroll
@@ -433,6 +445,21 @@ __global__ __launch_bounds__(256) void bn_fin_apply_kernel(FinApplyArgs p) {
       }
     }
     static_cast<uint4*>(p.out)[i] = float_to_chunk<T>(vo).u;
+  };
+  // two rows per trip: both rows' chunks are requested before either is used
+  for (int64_t r = r0 + ty; r < r1; r += 2 * RPP) {
+    const int64_t i0 = r * cc + col_chunk, i1 = i0 + RPP * cc;
+    const bool second = r + RPP < r1;
+    Chunk a0, a1, b0 = zero_chunk(), b1 = zero_chunk();
+    a0.u = static_cast<const uint4*>(p.a)[i0];
+    if (has_b) b0.u = static_cast<const uint4*>(p.b)[i0];
+    a1 = a0;
+    if (second) {
+      a1.u = static_cast<const uint4*>(p.a)[i1];
+      if (has_b) b1.u = static_cast<const uint4*>(p.b)[i1];
+    }
+    finish(i0, a0, b0);
+    if (second) finish(i1, a1, b1);
   }
 }
 
@@ -520,7 +547,7 @@ int bn_fwd_train(Context* ctx, int dtype, const void* x, void* y, const void* re
   if (rc) return rc;
   FwdFinalizeArgs f{partial, g.row_blocks, C, rows, gamma, beta, running_mean, running_var, save_mean, save_invstd,
                     scale,   shift,        momentum, eps};
-  rc = launch(ctx, bn_fwd_finalize_kernel, dim3((C + 7) / 8), dim3(256), f, "bn_fwd_finalize_kernel",
+  rc = launch(ctx, bn_fwd_finalize_kernel, dim3((C + 7) / 8), dim3(kFinalizeThreads), f, "bn_fwd_finalize_kernel",
               8.0 * g.row_blocks * C, 1);
   if (rc) return rc;
   ApplyArgs a{x, residual, nullptr, y, scale, shift, nullptr, rows * g.cc, FastDiv(g.cc), relu};
@@ -539,7 +566,7 @@ int bn_fwd_finalize(Context* ctx, const float* partial, int row_blocks, int C, i
   TCH_CHECK_ARG((running_mean == nullptr) == (running_var == nullptr), "bn_fwd_finalize: running stats come in pairs");
   FwdFinalizeArgs f{partial, row_blocks, C, rows, gamma, beta, running_mean, running_var, save_mean, save_invstd,
                     coef,    coef + C,   momentum, eps};
-  return launch(ctx, bn_fwd_finalize_kernel, dim3((C + 7) / 8), dim3(256), f, "bn_fwd_finalize_kernel",
+  return launch(ctx, bn_fwd_finalize_kernel, dim3((C + 7) / 8), dim3(kFinalizeThreads), f, "bn_fwd_finalize_kernel",
                 8.0 * row_blocks * C, 1);
 }
 
@@ -550,7 +577,7 @@ int bn_bwd_finalize(Context* ctx, const float* partial, int row_blocks, int C, i
                     rows > 0,
                 "bn_bwd_finalize: bad arguments");
   BwdFinalizeArgs f{partial, row_blocks, C, rows, gamma, save_mean, save_invstd, dgamma, dbeta, coef, accumulate};
-  return launch(ctx, bn_bwd_finalize_kernel, dim3((C + 7) / 8), dim3(256), f, "bn_bwd_finalize_kernel",
+  return launch(ctx, bn_bwd_finalize_kernel, dim3((C + 7) / 8), dim3(kFinalizeThreads), f, "bn_bwd_finalize_kernel",
                 8.0 * row_blocks * C, 1);
 }
 
@@ -605,7 +632,7 @@ int bn_fwd_train_partials(Context* ctx, int dtype, const void* x, void* y, const
   float* shift = scratch + C;
   FwdFinalizeArgs f{partial, row_blocks, C, rows, gamma, beta, running_mean, running_var, save_mean, save_invstd,
                     scale,   shift,      momentum, eps};
-  int rc = launch(ctx, bn_fwd_finalize_kernel, dim3((C + 7) / 8), dim3(256), f, "bn_fwd_finalize_kernel",
+  int rc = launch(ctx, bn_fwd_finalize_kernel, dim3((C + 7) / 8), dim3(kFinalizeThreads), f, "bn_fwd_finalize_kernel",
                   8.0 * row_blocks * C, 1);
   if (rc) return rc;
   const double eb = dtype == kBF16 ? 2.0 : 4.0;
@@ -638,7 +665,7 @@ int bn_bwd(Context* ctx, int dtype, const void* dy, const void* relu_mask, const
                                    tensor_bytes * in_tensors, 1);
   if (rc) return rc;
   BwdFinalizeArgs f{partial, g.row_blocks, C, rows, gamma, save_mean, save_invstd, dgamma, dbeta, coef, accumulate};
-  rc = launch(ctx, bn_bwd_finalize_kernel, dim3((C + 7) / 8), dim3(256), f, "bn_bwd_finalize_kernel",
+  rc = launch(ctx, bn_bwd_finalize_kernel, dim3((C + 7) / 8), dim3(kFinalizeThreads), f, "bn_bwd_finalize_kernel",
               8.0 * g.row_blocks * C, 1);
   if (rc) return rc;
   ApplyArgs a{dy, relu_mask, x, dx, coef, coef + C, coef + 2 * C, rows * g.cc, FastDiv(g.cc), 0};
@@ -667,7 +694,7 @@ int bn_bwd_partials(Context* ctx, int dtype, const void* g, const void* x, void*
   Geometry geo = geometry(rows, C, dtype);
   float* coef = scratch;
   BwdFinalizeArgs f{partial, row_blocks, C, rows, gamma, save_mean, save_invstd, dgamma, dbeta, coef, accumulate};
-  int rc = launch(ctx, bn_bwd_finalize_kernel, dim3((C + 7) / 8), dim3(256), f, "bn_bwd_finalize_kernel",
+  int rc = launch(ctx, bn_bwd_finalize_kernel, dim3((C + 7) / 8), dim3(kFinalizeThreads), f, "bn_bwd_finalize_kernel",
                   8.0 * row_blocks * C, 1);
   if (rc) return rc;
   const double eb = dtype == kBF16 ? 2.0 : 4.0;

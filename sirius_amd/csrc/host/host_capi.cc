@@ -305,7 +305,11 @@ tch_stub* tch_stub_create(int kind, int batch_size) {
   s->stub->start();
   return s;
 }
-void tch_stub_destroy(tch_stub* s) { delete s; }
+void tch_stub_destroy(tch_stub* s) {
+  // the control thread calls into the derived class: it has to be gone before any destructor runs
+  if (s && s->stub) s->stub->stop();
+  delete s;
+}
 void tch_stub_stop(tch_stub* s) { if (s) s->stub->stop(); }
 int tch_stub_cmd(tch_stub* s) { return s ? s->stub->cmd() : -1; }
 void tch_stub_set_cmd(tch_stub* s, int cmd) { if (s) s->stub->set_cmd(cmd); }
