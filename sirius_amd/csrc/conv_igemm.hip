@@ -1418,10 +1418,14 @@ int conv2d_wgrad_pick_splits(const ConvShape& s, int dtype) {
   const int gemm_m = s.K, gemm_n = s.R * s.S * s.C;
   int64_t tiles = tiles_for(gemm_m, gemm_n, 128, 128);
   if (tiles < 8) tiles = tiles_for(gemm_m, gemm_n, 64, 64);
-  static const int target_wgs = [] {
+  // Workgroups to aim for.  The weight gradients run beside the data-gradient chain on a second stream: a
+  // launch that does not fill the chip by itself shares it better, and every split costs a partial filter
+  // written and read again, so filters of few tiles over short reductions aim lower than wide or long products.
+  static const int target_env = [] {
     const char* e = getenv("TCH_WGRAD_WGS");
-    return e && atoi(e) > 0 ? atoi(e) : 384;
+    return e && atoi(e) > 0 ? atoi(e) : 0;
   }();
+  const int target_wgs = target_env ? target_env : (tiles <= 64 && pixels <= 16384) ? 192 : 384;
   int64_t want = (target_wgs + tiles - 1) / tiles;
   int64_t max_by_k = pixels / (4 * BK);  // at least four reduction steps per split
   if (max_by_k < 1) max_by_k = 1;
@@ -1459,7 +1463,11 @@ int conv2d_wgrad(Context* ctx, int dtype, const ConvShape& s, const void* x, con
   a.div_plane = FastDiv(a.Ho * a.Wo);
   a.div_width = FastDiv(a.Wo);
   if (tile_cfg < 0) {
-    tile_cfg = (a.gemm_m >= 128 && a.gemm_n >= 128 && tiles_for(a.gemm_m, a.gemm_n, 128, 128) * splits >= 256) ? 0 : 2;
+    static const int big_from = [] {
+      const char* e = getenv("TCH_WGRAD_BIG_TILE_WGS");
+      return e && atoi(e) > 0 ? atoi(e) : 128;
+    }();
+    tile_cfg = (a.gemm_m >= 128 && a.gemm_n >= 128 && tiles_for(a.gemm_m, a.gemm_n, 128, 128) * splits >= big_from) ? 0 : 2;
   }
   int rc = dtype == kBF16 ? launch_mode<bf16, kWgrad>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo))
                           : launch_mode<float, kWgrad>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo));
