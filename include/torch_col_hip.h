@@ -113,7 +113,10 @@ int tch_context_get_cu_limit(tch_context* ctx);
 /* ---- convolution (implicit GEMM on MFMA) ---------------------------------------- */
 /* y[N,Ho,Wo,K] = conv(x[N,H,W,C], w[K,R,S,C]) (+ bias[K]) (+ add, optionally gated by mask > 0).
  * out_f32 != 0 stores y as fp32 whatever dtype is.  tile_cfg: -1 auto, 0 = 128x128, 1 = 128x64, 2 = 64x64,
- * 3 = 64x64 on the register-staged kernel even where the direct-to-LDS kernel applies.
+ * 3 = 64x64 on the register-staged kernel even where the direct-to-LDS kernel applies, 5 = 128x64 with the
+ * activation side of all nine taps of a channel block held in LDS as one patch (bf16, 3x3, stride 1, pad 1,
+ * channels a multiple of 64, rows of at most 63 pixels; any other convolution runs tiling 1 for it).  The patch
+ * kernel adds up channel block by channel block, the others tap by tap: results agree to rounding, not bit for bit.
  * c_logical: input channels that carry data when C is zero-padded to a chunk (0 = C); it only enters the
  * algorithmic-work figure the profiler reports, never the arithmetic. */
 int tch_conv2d_fwd(tch_context* ctx, int dtype, const void* x, const void* w, void* y, const void* add,

@@ -1081,6 +1081,200 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm2_kernel(IgemmArgs p) {
   finish_tile<T, MODE, WM, WN, TM, TN>(p, acc, reinterpret_cast<float*>(lds), tid, m0, n0, tile_m);
 }
 
+// ---------------------------------------------------------------------------
+// 3x3, stride 1, pad 1 (forward and data gradient), 128 x 64*TN tile: the activation side of the nine
+// taps of a channel block is ONE patch in LDS.  The 128 output pixels of a tile are consecutive in the
+// flattened (image, row, column) order, and the input pixel of tap (r, s) lies (r-1)*W + (s-1) places
+// further in the same order, so the patch is the contiguous range of pixels from W+1 before the tile to
+// W+1 behind it (128 + 2W + 2 rows of 64 channels), loaded once per channel block instead of nine
+// shifted copies of the tile.  A tap that falls outside its image (the zero padding) reads a row of
+// zeros kept in LDS instead.  The filter tiles stream per (channel block, tap) as in igemm2_kernel,
+// three in flight; the patch of the next channel block is requested at the first tap of this one.
+// The reduction runs channel block by channel block (taps innermost), so sums round differently from
+// igemm2_kernel's tap-major order.
+// ---------------------------------------------------------------------------
+constexpr int vmcnt_imm(int n) { return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8); }
+
+template <int MODE, int TN, int NBUF, int P_LD>
+__global__ __launch_bounds__(256) void igemm3_kernel(IgemmArgs p) {
+  using T = bf16;
+  constexpr int E = 8, WM = 2, WN = 2, TM = 2, NW = 4;
+  static_assert(NBUF >= 2 && NBUF <= 4, "filter tiles in flight");
+  constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
+  constexpr int B_LD = BN / 8 / NW;
+  constexpr int PATCH_BYTES = P_LD * 32 * kRowBytes2, B_BYTES = BN * kRowBytes2;
+  constexpr int B_OFF = 2 * PATCH_BYTES, ZERO_OFF = B_OFF + NBUF * B_BYTES;
+  constexpr int STAGE_BYTES = WM * 32 * (BN + kStagePad) * 4;
+  constexpr int LDS_BYTES = ZERO_OFF + kRowBytes2 > STAGE_BYTES ? ZERO_OFF + kRowBytes2 : STAGE_BYTES;
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[LDS_BYTES];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  uint32_t id = xcd_remap(blockIdx.x, gridDim.x);
+  const int tile_m = id / p.tiles_n;
+  const int tile_n = id - tile_m * p.tiles_n;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  const int in_c = (MODE == kFwd) ? p.C : p.K;
+  const int cblocks = in_c / kStep2;
+  const int nk = 9 * cblocks;
+  const int W = p.W, H = p.H, halo = W + 1;
+
+  // ---- loaders: patch rows (wave * P_LD + j) * 8 + lane / 8, filter rows as in igemm2_kernel ----
+  const int sub_row = lane >> 3, slot = lane & 7;
+  int p_off[P_LD];
+#pragma unroll
+  for (int j = 0; j < P_LD; ++j) {
+    const int prow = (wave * P_LD + j) * 8 + sub_row;
+    const int chunk = slot ^ ((prow >> 1) & 7);
+    const int grow = m0 - halo + prow;
+    const bool ok = grow >= 0 && grow < p.gemm_m && prow < BM + 2 * halo;
+    p_off[j] = ok ? (grow * in_c + chunk * E) * 2 : static_cast<int>(kOutOfRange);
+  }
+  int b_off[B_LD];
+#pragma unroll
+  for (int j = 0; j < B_LD; ++j) {
+    const int trow = (wave * B_LD + j) * 8 + sub_row;
+    const int chunk = slot ^ ((trow >> 1) & 7);
+    const int row = n0 + trow;
+    b_off[j] = row < p.gemm_n ? (row * p.gemm_k + chunk * E) * 2 : static_cast<int>(kOutOfRange);
+  }
+  const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(p.a_src, p.a_bytes);
+  const __amdgpu_buffer_rsrc_t rsrc_b = make_rsrc(p.b_src, p.b_bytes);
+  auto issue_patch = [&](int cb) {
+    unsigned char* dst = lds + (cb & 1) * PATCH_BYTES + wave * P_LD * 1024;
+#pragma unroll
+    for (int j = 0; j < P_LD; ++j) load_to_lds(rsrc_a, dst + j * 1024, p_off[j], cb * kRowBytes2);
+  };
+  auto issue_filter = [&](int cb, int tap, int buf) {
+    unsigned char* dst = lds + B_OFF + buf * B_BYTES + wave * B_LD * 1024;
+    const int soff = (tap * in_c + cb * kStep2) * 2;
+#pragma unroll
+    for (int j = 0; j < B_LD; ++j) load_to_lds(rsrc_b, dst + j * 1024, b_off[j], soff);
+  };
+
+  // ---- the rows this lane feeds to the MFMAs and which of their nine taps lie inside the image ----
+  const int frag_row = lane & 31, frag_half = lane >> 5;
+  uint32_t taps[TM];
+#pragma unroll
+  for (int tm = 0; tm < TM; ++tm) {
+    const int row = m0 + (wm * TM + tm) * 32 + frag_row;
+    uint32_t bits = 0;
+    if (row < p.gemm_m) {
+      uint32_t img, pix, oh, ow;
+      p.div_plane.divmod(static_cast<uint32_t>(row), img, pix);
+      p.div_width.divmod(pix, oh, ow);
+#pragma unroll
+      for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int s2 = 0; s2 < 3; ++s2) {
+          const int ih = (MODE == kFwd) ? static_cast<int>(oh) + r - 1 : static_cast<int>(oh) + 1 - r;
+          const int iw = (MODE == kFwd) ? static_cast<int>(ow) + s2 - 1 : static_cast<int>(ow) + 1 - s2;
+          if (static_cast<unsigned>(ih) < static_cast<unsigned>(H) && static_cast<unsigned>(iw) < static_cast<unsigned>(W))
+            bits |= 1u << (r * 3 + s2);
+        }
+    }
+    taps[tm] = bits;
+  }
+
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
+  const int swz = (frag_row >> 1) & 7;
+  const uint32_t b_rd = lds_base + B_OFF + (wn * TN * 32 + frag_row) * kRowBytes2 + swz * 16;
+
+  // One step = one (channel block, tap).  pa[tm]: LDS address of this lane's patch row for the tap (slot
+  // swizzle of that row included), or of the zero row.
+  auto compute = [&](uint32_t patch_base, int tap, int buf) {
+    const int r = tap / 3, s2 = tap - 3 * r;
+    const int tapoff = (MODE == kFwd) ? r * W + s2 : (2 - r) * W + (2 - s2);
+    uint32_t pa[TM];
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm) {
+      const uint32_t prow = static_cast<uint32_t>((wm * TM + tm) * 32 + frag_row + tapoff);
+      const uint32_t in_patch = patch_base + prow * kRowBytes2 + ((prow >> 1) & 7) * 16;
+      pa[tm] = ((taps[tm] >> tap) & 1u) ? in_patch : lds_base + ZERO_OFF;
+    }
+    const uint32_t pb0 = b_rd + buf * B_BYTES;
+    auto read_frags = [&](int kk, uint4_t* fa, uint4_t* fb) {
+      const uint32_t cx = (2 * kk + frag_half) * 16;
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) asm volatile("ds_read_b128 %0, %1" : "=v"(fa[tm]) : "v"(pa[tm] ^ cx));
+      const uint32_t pb = pb0 ^ cx;
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn)
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fb[tn]) : "v"(pb), "n"(tn * 32 * kRowBytes2));
+    };
+    auto multiply = [&](uint4_t* fa, uint4_t* fb) {
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm) asm volatile("" : "+v"(fa[tm]));
+#pragma unroll
+      for (int tn = 0; tn < TN; ++tn) asm volatile("" : "+v"(fb[tn]));
+#pragma unroll
+      for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+          acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, fb[tn]),
+                                                                __builtin_bit_cast(bf16x8_t, fa[tm]), acc[tm][tn], 0, 0, 0);
+    };
+    uint4_t fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+    read_frags(0, fa0, fb0);
+    read_frags(1, fa1, fb1);
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(TM + TN));
+    multiply(fa0, fb0);
+    read_frags(2, fa0, fb0);
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(TM + TN));
+    multiply(fa1, fb1);
+    read_frags(3, fa1, fb1);
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(TM + TN));
+    multiply(fa0, fb0);
+    asm volatile("s_waitcnt lgkmcnt(0)");
+    multiply(fa1, fb1);
+  };
+
+  // Requests leave in this order: patch 0, filters 0 .. NBUF-2; then at step kt, behind its barrier, filter
+  // kt + NBUF-1 (into the buffer step kt-1 read) and, at the first tap of a channel block, the next block's
+  // patch.  They land in order, so "filter kt has landed" (and every patch requested before it) is a count
+  // of the requests made after it: the NBUF-2 filters behind it, and the patch requested at tap 0 when this
+  // is one of the taps 1 .. NBUF-1.  (Over the last steps fewer filters follow: wait for everything.)
+  constexpr int AHEAD = NBUF - 1;
+  if (tid < 8) *reinterpret_cast<uint4*>(lds + ZERO_OFF + tid * 16) = make_uint4(0u, 0u, 0u, 0u);
+  issue_patch(0);
+#pragma unroll
+  for (int t = 0; t < AHEAD; ++t) issue_filter(0, t, t);
+  for (int cb = 0; cb < cblocks; ++cb) {
+    const uint32_t patch_base = lds_base + (cb & 1) * PATCH_BYTES;
+    const bool next_patch = cb + 1 < cblocks;
+#pragma unroll
+    for (int tap = 0; tap < 9; ++tap) {
+      const int kt = cb * 9 + tap;
+      if (kt + AHEAD > nk)
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+      else if (tap >= 1 && tap <= AHEAD && next_patch)
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((NBUF - 2) * B_LD + P_LD));
+      else
+        __builtin_amdgcn_s_waitcnt(vmcnt_imm((NBUF - 2) * B_LD));
+      __syncthreads();
+      // 9 taps per channel block: with three buffers the buffer of a step is a constant of the unrolled loop
+      const int buf = NBUF == 3 ? tap % 3 : kt % NBUF;
+      const int buf_ahead = NBUF == 3 ? (tap + AHEAD) % 3 : (kt + AHEAD) % NBUF;
+      if (kt + AHEAD < nk) issue_filter(tap + AHEAD >= 9 ? cb + 1 : cb, (tap + AHEAD) % 9, buf_ahead);
+      if (tap == 0 && next_patch) issue_patch(cb + 1);
+      compute(patch_base, tap, buf);
+    }
+  }
+
+  finish_tile<T, MODE, WM, WN, TM, TN>(p, acc, reinterpret_cast<float*>(lds), tid, m0, n0, tile_m);
+}
+
 struct ReduceArgs {
   const float* partial;
   float* out;
@@ -1187,6 +1381,39 @@ int launch_cfg2(Context* ctx, IgemmArgs& a, double flops) {
                 name.c_str(), flops, 0, conv_bytes<MODE>(a, 2));
 }
 
+// The 3x3 patch kernel: stride 1, pad 1, input channels in blocks of 64, rows short enough for the patch
+template <int MODE>
+bool patch_kernel_fits(const IgemmArgs& a) {
+  const int in_c = MODE == kFwd ? a.C : a.K;
+  return a.R == 3 && a.S == 3 && a.stride == 1 && a.pad == 1 && a.H == a.Ho && a.W == a.Wo && in_c % kStep2 == 0 &&
+         128 + 2 * (a.W + 1) <= 256;
+}
+
+template <int MODE, int TN, int NBUF, int P_LD>
+int launch_cfg3_rows(Context* ctx, IgemmArgs& a, double flops) {
+  constexpr int BM = 128, BN = 64 * TN;
+  static const std::string name = std::string("igemm3_kernel<bf16,") + (MODE == kFwd ? "fwd," : "dgrad,") +
+                                  std::to_string(BM) + "x" + std::to_string(BN) + "," + std::to_string(NBUF) + "buf,patch" +
+                                  std::to_string(P_LD * 32) + ">";
+  a.tiles_m = (a.gemm_m + BM - 1) / BM;
+  a.tiles_n = (a.gemm_n + BN - 1) / BN;
+  const int64_t wgs = static_cast<int64_t>(a.tiles_m) * a.tiles_n;
+  if (wgs <= 0 || wgs > 0x7fffffff) {
+    set_error("igemm: grid out of range");
+    return -22;
+  }
+  return launch(ctx, igemm3_kernel<MODE, TN, NBUF, P_LD>, dim3(static_cast<unsigned>(wgs)), dim3(256), a, name.c_str(), flops, 0,
+                conv_bytes<MODE>(a, 2));
+}
+
+template <int MODE, int TN, int NBUF>
+int launch_cfg3(Context* ctx, IgemmArgs& a, double flops) {
+  const int rows = 128 + 2 * (a.W + 1);   // patch rows, loaded 32 at a time
+  if (rows <= 160) return launch_cfg3_rows<MODE, TN, NBUF, 5>(ctx, a, flops);
+  if (rows <= 192) return launch_cfg3_rows<MODE, TN, NBUF, 6>(ctx, a, flops);
+  return launch_cfg3_rows<MODE, TN, NBUF, 8>(ctx, a, flops);
+}
+
 // TCH_IGEMM2 = 0 keeps every convolution on igemm_kernel; 2 or 3 picks the number of LDS tiles
 // in flight of igemm2_kernel (default: 2 for 128x128, 3 for 128x64)
 int igemm2_setting() {
@@ -1202,6 +1429,12 @@ int launch_mode(Context* ctx, IgemmArgs& a, int tile_cfg, double flops) {
   if constexpr (sizeof(T) == 2 && (MODE == kFwd || MODE == kDgrad)) {
     const int in_c = MODE == kFwd ? a.C : a.K;
     const int setting = igemm2_setting();
+    if (tile_cfg == 5) {   // 128 x 64 with the 3x3 patch in LDS; convolutions it does not fit run as tiling 1
+      // (measured and not built: a 128 x 128 tile with two or three filter tiles in flight and four filter
+      // tiles for this one were 4-30 % slower on every 3x3 layer of ResNet-152 at batch 64)
+      if (setting != 0 && patch_kernel_fits<MODE>(a)) return launch_cfg3<MODE, 1, 3>(ctx, a, flops);
+      tile_cfg = 1;
+    }
     if (setting != 0 && in_c % kStep2 == 0 && a.R * a.S <= 32 && tile_cfg >= 0 && tile_cfg <= 2) {
       if (tile_cfg == 0)
         return setting == 3 ? launch_cfg2<MODE, 2, 2, 2, 2, 3>(ctx, a, flops) : launch_cfg2<MODE, 2, 2, 2, 2, 2>(ctx, a, flops);
@@ -1210,6 +1443,7 @@ int launch_mode(Context* ctx, IgemmArgs& a, int tile_cfg, double flops) {
       return setting == 2 ? launch_cfg2<MODE, 2, 2, 1, 1, 2>(ctx, a, flops) : launch_cfg2<MODE, 2, 2, 1, 1, 3>(ctx, a, flops);
     }
   }
+  if (tile_cfg == 5) tile_cfg = 1;
   switch (tile_cfg) {
     case 0:
       return launch_cfg<T, MODE, 2, 2, 2, 2>(ctx, a, flops);  // 128 x 128
@@ -1226,6 +1460,9 @@ double conv_flops(const ConvShape& s, int Ho, int Wo) {
   const int c = (s.c_logical > 0 && s.c_logical < s.C) ? s.c_logical : s.C;
   return 2.0 * s.N * Ho * Wo * static_cast<double>(s.K) * s.R * s.S * c;
 }
+
+// rows of the workgroup tile of a tiling number (5 = the 3x3 patch kernel, or tiling 1 where it does not fit)
+int tile_rows(int tile_cfg) { return tile_cfg == 5 ? 128 : tile_cfg >= 2 ? 64 : 128; }
 
 int64_t tiles_for(int m, int n, int bm, int bn) {
   return static_cast<int64_t>((m + bm - 1) / bm) * ((n + bn - 1) / bn);
@@ -1333,7 +1570,7 @@ int conv2d_fwd(Context* ctx, int dtype, const ConvShape& s, const void* x, const
   a.div_plane = FastDiv(a.Ho * a.Wo);
   a.div_width = FastDiv(a.Wo);
   if (tile_cfg < 0) tile_cfg = pick_tile(a.gemm_m, a.gemm_n, 1);
-  const int row_tiles = (a.gemm_m + (tile_cfg >= 2 ? 64 : 128) - 1) / (tile_cfg >= 2 ? 64 : 128);
+  const int row_tiles = (a.gemm_m + tile_rows(tile_cfg) - 1) / tile_rows(tile_cfg);
   const bool in_kernel = finalize && row_tiles <= kBnFinalizeInKernelTiles;
   if (in_kernel) bind_finalize(a, finalize);
   int rc = dtype == kBF16 ? launch_mode<bf16, kFwd>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo))
@@ -1350,7 +1587,7 @@ int conv2d_fwd_stat_rows(const ConvShape& s, int dtype, int tile_cfg) {
   conv_output_hw(s, &Ho, &Wo);
   const int gemm_m = s.N * Ho * Wo;
   if (tile_cfg < 0) tile_cfg = pick_tile(gemm_m, s.K, 1);
-  const int bm = tile_cfg >= 2 ? 64 : 128;
+  const int bm = tile_rows(tile_cfg);
   return (gemm_m + bm - 1) / bm;
 }
 
@@ -1358,7 +1595,7 @@ int conv2d_dgrad_stat_rows(const ConvShape& s, int dtype, int tile_cfg) {
   (void)dtype;
   const int gemm_m = s.N * s.H * s.W;
   if (tile_cfg < 0) tile_cfg = pick_tile(gemm_m, s.C, 1);
-  const int bm = tile_cfg >= 2 ? 64 : 128;
+  const int bm = tile_rows(tile_cfg);
   return (gemm_m + bm - 1) / bm;
 }
 
@@ -1393,7 +1630,7 @@ int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, co
   a.div_width = FastDiv(s.W);
   if (tile_cfg < 0) tile_cfg = pick_tile(a.gemm_m, a.gemm_n, 1);
   const BnFinalize* finalize = bn ? bn->finalize : nullptr;
-  const int row_tiles = (a.gemm_m + (tile_cfg >= 2 ? 64 : 128) - 1) / (tile_cfg >= 2 ? 64 : 128);
+  const int row_tiles = (a.gemm_m + tile_rows(tile_cfg) - 1) / tile_rows(tile_cfg);
   const bool in_kernel = finalize && row_tiles <= kBnFinalizeInKernelTiles;
   if (in_kernel) bind_finalize(a, finalize);
   int rc = dtype == kBF16 ? launch_mode<bf16, kDgrad>(ctx, a, tile_cfg, conv_flops(s, a.Ho, a.Wo))

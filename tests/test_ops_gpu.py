@@ -51,12 +51,16 @@ CONV_CASES = [
     (5, 1, 1, 64, 1000, 1, 1, 1, 0),      # fully connected as a 1x1 convolution
     (1, 9, 11, 16, 24, 3, 3, 1, 1),       # non-square
     (2, 16, 16, 8, 32, 4, 4, 4, 0),       # patch embedding: 4x4 patches, stride 4, channels padded to one chunk
+    (3, 14, 14, 128, 96, 3, 3, 1, 1),     # 3x3 over two channel blocks, tiles that span images, ragged columns
+    (1, 28, 28, 64, 64, 3, 3, 1, 1),      # 3x3 with 28-pixel rows (the longer patch of tiling 5)
+    (1, 56, 56, 64, 64, 3, 3, 1, 1),      # 3x3 with 56-pixel rows (the longest patch)
+    (2, 7, 7, 128, 64, 3, 3, 1, 1),       # 3x3 on 7x7 images: every tile holds image borders
 ]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", CONV_CASES)
-@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3])
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3, 5])
 def test_conv_fwd(ctx, dtype, case, tile_cfg):
     from sirius_amd import ops
     N, H, W, C, K, R, S, st, pad = case
@@ -90,7 +94,7 @@ def test_conv_fwd_epilogue(ctx, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", CONV_CASES)
-@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3])
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3, 5])
 def test_conv_dgrad(ctx, dtype, case, tile_cfg):
     from sirius_amd import ops
     N, H, W, C, K, R, S, st, pad = case
@@ -189,8 +193,8 @@ def test_bn_fwd(ctx, dtype, rows, C, fuse):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("case", [CONV_CASES[0], CONV_CASES[2], CONV_CASES[3], CONV_CASES[5], CONV_CASES[6]])
-@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3])
+@pytest.mark.parametrize("case", [CONV_CASES[0], CONV_CASES[2], CONV_CASES[3], CONV_CASES[5], CONV_CASES[6], CONV_CASES[10], CONV_CASES[13]])
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3, 5])
 def test_conv_with_bn_statistics(ctx, dtype, case, tile_cfg):
     """The convolution leaves per-tile sums of its stored output; BatchNorm starts from them.
     Checked against the oracle's conv -> BatchNorm(train) on the same inputs; the statistics must be
@@ -302,8 +306,8 @@ def test_bn_bwd(ctx, dtype, rows, C, masked):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("case", [CONV_CASES[0], CONV_CASES[1], CONV_CASES[3], CONV_CASES[4], CONV_CASES[6]])
-@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3])
+@pytest.mark.parametrize("case", [CONV_CASES[0], CONV_CASES[1], CONV_CASES[3], CONV_CASES[4], CONV_CASES[6], CONV_CASES[10], CONV_CASES[13]])
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3, 5])
 @pytest.mark.parametrize("with_add", [False, True])
 def test_conv_dgrad_with_bn_backward_sums(ctx, dtype, case, tile_cfg, with_add):
     """The data-gradient convolution gates its output by the ReLU of the BatchNorm it flows into and
