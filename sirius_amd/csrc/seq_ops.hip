@@ -144,59 +144,74 @@ __global__ __launch_bounds__(256) void ln_bwd_kernel(LnArgs p) {
   if (r1 > p.rows) r1 = p.rows;
   const float inv_c = 1.0f / static_cast<float>(p.C);
   // rows_per_wg is a multiple of GROUPS, so the groups of a wavefront stay in step (the row sums below are
-  // taken by all lanes); a group beyond the last row works on nothing
-  for (int64_t base = r0; base < r1; base += GROUPS) {
-    const int64_t row = base + group;
-    const bool live = row < r1;
-    const uint4* xs = static_cast<const uint4*>(p.x) + row * p.cc;
-    const uint4* gs = static_cast<const uint4*>(p.dy) + row * p.cc;
-    float mean = 0.f, rstd = 0.f;
-    if (live) {
-      mean = p.mean[row];
-      rstd = p.rstd[row];
-    }
-    float xh[NCH][E], g[NCH][E];
-    float a = 0.f, b = 0.f;
+  // taken by all lanes); a group beyond the last row works on nothing.  A group takes R rows per trip and
+  // requests the chunks of all of them before it uses any: a trip costs one round trip to memory, not R.
+  constexpr int R = 2;
+  for (int64_t base = r0; base < r1; base += R * GROUPS) {
+    bool live[R];
+    float mean[R], rstd[R];
+    Chunk cx[R][NCH], cg[R][NCH], cr[R][NCH];
 #pragma unroll
-    for (int j = 0; j < NCH; ++j) {
-      const int c = sub + j * L;
-      if (live && c < p.cc) {
-        Chunk cx, cg;
-        cx.u = xs[c];
-        cg.u = gs[c];
-        chunk_to_float<T>(cx, xh[j]);
-        chunk_to_float<T>(cg, g[j]);
+    for (int q = 0; q < R; ++q) {
+      const int64_t row = base + q * GROUPS + group;
+      live[q] = row < r1;
+      mean[q] = rstd[q] = 0.f;
+      if (live[q]) {
+        mean[q] = p.mean[row];
+        rstd[q] = p.rstd[row];
+      }
 #pragma unroll
-        for (int e = 0; e < E; ++e) {
-          xh[j][e] = (xh[j][e] - mean) * rstd;
-          dg[j][e] += g[j][e] * xh[j][e];
-          db[j][e] += g[j][e];
-          g[j][e] *= gam[j][e];
-          a += g[j][e];
-          b += g[j][e] * xh[j][e];
+      for (int j = 0; j < NCH; ++j) {
+        const int c = sub + j * L;
+        cx[q][j] = cg[q][j] = cr[q][j] = zero_chunk();
+        if (live[q] && c < p.cc) {
+          cx[q][j].u = (static_cast<const uint4*>(p.x) + row * p.cc)[c];
+          cg[q][j].u = (static_cast<const uint4*>(p.dy) + row * p.cc)[c];
+          if (p.add) cr[q][j].u = (static_cast<const uint4*>(p.add) + row * p.cc)[c];
         }
       }
     }
-    a = row_sum<L>(a) * inv_c;
-    b = row_sum<L>(b) * inv_c;
-    if (!live) continue;
-    uint4* dst = static_cast<uint4*>(p.out) + row * p.cc;
 #pragma unroll
-    for (int j = 0; j < NCH; ++j) {
-      const int c = sub + j * L;
-      if (c < p.cc) {
-        float o[E];
+    for (int q = 0; q < R; ++q) {
+      const int64_t row = base + q * GROUPS + group;
+      float xh[NCH][E], g[NCH][E];
+      float a = 0.f, b = 0.f;
 #pragma unroll
-        for (int e = 0; e < E; ++e) o[e] = rstd * (g[j][e] - a - xh[j][e] * b);
-        if (p.add) {
-          Chunk cr;
-          cr.u = (static_cast<const uint4*>(p.add) + row * p.cc)[c];
-          float r[E];
-          chunk_to_float<T>(cr, r);
+      for (int j = 0; j < NCH; ++j) {
+        const int c = sub + j * L;
+        chunk_to_float<T>(cx[q][j], xh[j]);
+        chunk_to_float<T>(cg[q][j], g[j]);
+        if (live[q] && c < p.cc) {
 #pragma unroll
-          for (int e = 0; e < E; ++e) o[e] += r[e];
+          for (int e = 0; e < E; ++e) {
+            xh[j][e] = (xh[j][e] - mean[q]) * rstd[q];
+            dg[j][e] += g[j][e] * xh[j][e];
+            db[j][e] += g[j][e];
+            g[j][e] *= gam[j][e];
+            a += g[j][e];
+            b += g[j][e] * xh[j][e];
+          }
         }
-        dst[c] = float_to_chunk<T>(o).u;
+      }
+      a = row_sum<L>(a) * inv_c;
+      b = row_sum<L>(b) * inv_c;
+      if (!live[q]) continue;
+      uint4* dst = static_cast<uint4*>(p.out) + row * p.cc;
+#pragma unroll
+      for (int j = 0; j < NCH; ++j) {
+        const int c = sub + j * L;
+        if (c < p.cc) {
+          float o[E];
+#pragma unroll
+          for (int e = 0; e < E; ++e) o[e] = rstd[q] * (g[j][e] - a - xh[j][e] * b);
+          if (p.add) {
+            float r[E];
+            chunk_to_float<T>(cr[q][j], r);
+#pragma unroll
+            for (int e = 0; e < E; ++e) o[e] += r[e];
+          }
+          dst[c] = float_to_chunk<T>(o).u;
+        }
       }
     }
   }
