@@ -26,11 +26,12 @@ METRIC = "ResNet-152 bf16 bs64 train images/sec on 1 GPU; conv MFMA util %"
 # (FETCH_SIZE and WRITE_SIZE, KiB per dispatch, scaled by what the same counters read for the --calibrate
 # copy of known size: factors 2.000 and 1.000); the summary is profiles/resnet152_bf16_bs64_step_kernel_stats_and_traffic.txt
 MEASURED_TRAFFIC_MIB = {
-    "wgrad_kernel<bf16,128x128>": 27.97 + 24.29,
-    "igemm2_kernel<bf16,dgrad,128x128,2buf>": 83.11 + 33.00,
-    "igemm2_kernel<bf16,dgrad,128x64,3buf>": 54.53 + 27.18,
-    "igemm2_kernel<bf16,fwd,128x128,2buf>": 26.50 + 26.83,
-    "igemm2_kernel<bf16,fwd,128x64,3buf>": 40.45 + 15.49,
+    "wgrad_kernel<bf16,128x128>": 31.79 + 13.77,
+    "igemm2_kernel<bf16,dgrad,128x128,2buf>": 83.54 + 28.00,
+    "igemm2_kernel<bf16,dgrad,128x64,3buf>": 63.10 + 31.49,
+    "igemm2_kernel<bf16,fwd,128x128,2buf>": 30.03 + 22.89,
+    "igemm2_kernel<bf16,fwd,128x64,3buf>": 35.10 + 18.06,
+    "igemm3_kernel<bf16,dgrad,128x64,3buf,patch160>": 29.72 + 5.90,
     "bn_apply_kernel<bf16,bwd>": 72.04 + 34.61,
     "bn_apply_kernel<bf16,fwd>": 54.69 + 36.09,
 }
