@@ -24,7 +24,8 @@ class PeerScript:
     """Stand-in inference server: `at` maps a micro-batch index to ('l1' | 'l2' | 'exit', batch size) or to
     ('switch', milliseconds until the resume), or to ('cus', compute units inference wants for itself).
     The command is sent from a side thread `delay_ms` after the micro-batch began, so that it lands
-    while kernels are queued, as a real request would."""
+    while kernels are queued, as a real request would; with `delay_ms` <= 0 it is sent on the spot, before
+    the micro-batch's first launch (no thread, no dependence on how the threads are scheduled)."""
 
     def __init__(self, at, delay_ms=5.0, verbose=False):
         self.server = torch_col.DebugServer(1, verbose=verbose)
@@ -54,6 +55,9 @@ class PeerScript:
             {"l1": self.server.colocate_l1, "l2": self.server.colocate_l2, "exit": self.server.infer_exit,
              "cus": self.server.set_infer_required_cus}[kind](bs)
             self.sent.append((t, kind, bs))
+        if self.delay_ms <= 0:
+            fire()
+            return
         t = threading.Thread(target=fire, daemon=True)
         self._threads.append(t)
         t.start()

@@ -53,6 +53,7 @@ def clean_runtime(monkeypatch):
     tc.torch_col_shutdown()
     tc.reset_for_tests()
     yield tc
+    torch.cuda.synchronize()      # also behind a failed test nothing may be running when the pool is unmapped
     tc.UnRegisterAllStreams()
     tc.SetRejectCudaCalls(False)
     tc.reset_for_tests()
@@ -321,7 +322,8 @@ def test_dynamic_compute_unit_partition_under_the_colocation_protocol(clean_runt
         seen.append(n)
         return n
     monkeypatch.setattr(tc, "get_train_avail_cus", spy)
-    peer = script.PeerScript({2: ("cus", 192), 5: ("cus", 0)}, delay_ms=0.5)
+    # sent on the spot: the shares the engine sees must not depend on how a side thread is scheduled
+    peer = script.PeerScript({2: ("cus", 192), 5: ("cus", 0)}, delay_ms=0)
     try:
         out = script.train(1, 16, dataset_size=16 * 8, dtype=torch.bfloat16, peer=peer, num_distinct_samples=32,
                            **SMALL)
