@@ -255,7 +255,7 @@ def main():
     rows = eng.ctx.profile(plan.prog, reps) + eng.ctx.profile(eng._opt_prog, reps)
     rows.sort(key=lambda r: -r["total_ms"])
     total_ms = sum(r["total_ms"] for r in rows) / reps
-    conv = [r for r in rows if r["name"].startswith(("igemm_kernel", "igemm2_kernel", "wgrad_kernel"))]
+    conv = [r for r in rows if r["name"].startswith(("igemm_kernel", "igemm2_kernel", "igemm3_kernel", "wgrad_kernel"))]
     conv_ms = sum(r["total_ms"] for r in conv) / reps
     conv_flops = sum(r["work"] for r in conv) / reps
     top = rows[0]
