@@ -250,6 +250,55 @@ def test_conv_with_bn_statistics(ctx, dtype, case, tile_cfg):
         close(y2, y.float().cpu(), dtype, "fused finalize: y", rtol=1e-6 if dtype == torch.float32 else 8e-3)
 
 
+def test_bn_finalize_over_more_row_tiles_than_one_trip(ctx):
+    """2 400 row tiles of 64 rows: the finalize kernels' lanes take more than one trip over their row tiles
+    (a trip covers 2 048).  Forward statistics and backward sums against the oracle."""
+    from sirius_amd import ops
+    dtype = torch.bfloat16
+    N, H, W, C, K = 6, 160, 160, 64, 64     # 153 600 output rows
+    g = _gen(29)
+    x = rnd((N, H, W, C), dtype, g)
+    w = rnd((K, 1, 1, C), dtype, g, C ** -0.5)
+    gamma, beta = torch.rand(K, generator=g) + 0.5, torch.randn(K, generator=g) * 0.1
+    z_ref = O.conv2d_fwd(x, w, 1, 0).to(dtype)
+    y_ref, mean_ref, invstd_ref = O.bn_fwd_train(z_ref, gamma, beta, torch.zeros(K), torch.ones(K), relu=True)
+    xd, wd = x.cuda(), w.cuda()
+    z = torch.empty(z_ref.shape, dtype=dtype, device="cuda")
+    rb = ops.conv2d_fwd_stat_rows(xd, K, 1, 1, 1, 0, 2)
+    assert rb == 2400
+    partial = torch.full((rb * K * 2,), float("nan"), device="cuda")
+    ops.conv2d_fwd_bnstats(ctx, xd, wd, z, 1, 0, partial, tile_cfg=2)
+    y = torch.empty_like(z)
+    rm, rv = torch.zeros(K, device="cuda"), torch.ones(K, device="cuda")
+    sm, si = torch.empty(K, device="cuda"), torch.empty(K, device="cuda")
+    scratch = torch.empty(2 * K, device="cuda")
+    ops.bn_fwd_train_partials(ctx, z, y, gamma.cuda(), beta.cuda(), rm, rv, sm, si, partial, rb, scratch, relu=True)
+    torch.cuda.synchronize()
+    close(sm, mean_ref, torch.float32, "bn mean", rtol=2e-2)
+    close(si, invstd_ref, torch.float32, "bn invstd", rtol=2e-2)
+    close(y, y_ref, dtype, "bn y", rtol=2e-2)
+    z32 = z.float().cpu().reshape(-1, K).double()
+    close(sm, z32.mean(0).float(), torch.float32, "mean of the stored output", rtol=1e-5)
+    # backward: data gradient of a 1x1 convolution behind that BatchNorm + ReLU, sums over 2 400 row tiles
+    dy2 = rnd((N, H, W, K), dtype, g)
+    w2 = rnd((K, 1, 1, K), dtype, g, K ** -0.5)
+    g_ref = O.conv2d_dgrad(dy2, w2, (N, H, W, K), 1, 0)
+    dz_ref, dg_ref, db_ref = O.bn_bwd(g_ref, z_ref, gamma, relu_mask=y_ref)
+    gx = torch.empty((N, H, W, K), dtype=dtype, device="cuda")
+    rb2 = ops.conv2d_dgrad_stat_rows(gx, K, 1, 1, 1, 0, 2)
+    assert rb2 == 2400
+    partial2 = torch.full((rb2 * K * 2,), float("nan"), device="cuda")
+    ops.conv2d_dgrad_bnsums(ctx, dy2.cuda(), ops.filter_transpose(ctx, w2.cuda()), gx, 1, 0, z, sm, si, partial2,
+                            bn_mask=y, tile_cfg=2)
+    dz = torch.empty_like(z)
+    dgm, dbt = torch.empty(K, device="cuda"), torch.empty(K, device="cuda")
+    ops.bn_bwd_partials(ctx, gx, z, dz, gamma.cuda(), sm, si, dgm, dbt, partial2, rb2, torch.empty(3 * K, device="cuda"))
+    torch.cuda.synchronize()
+    close(dgm, dg_ref, torch.float32, "bn dgamma", rtol=2e-2)
+    close(dbt, db_ref, torch.float32, "bn dbeta", rtol=2e-2)
+    close(dz, dz_ref, dtype, "bn dz", rtol=2e-2)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_conv_bn_finalize_with_many_row_tiles(ctx, dtype):
     """More row tiles than one workgroup should sum (> 256): the convolution call finishes the coefficients
