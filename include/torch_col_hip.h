@@ -117,6 +117,7 @@ int tch_context_get_cu_limit(tch_context* ctx);
  * activation side of all nine taps of a channel block held in LDS as one patch (bf16, 3x3, stride 1, pad 1,
  * channels a multiple of 64, rows of at most 63 pixels; any other convolution runs tiling 1 for it).  The patch
  * kernel adds up channel block by channel block, the others tap by tap: results agree to rounding, not bit for bit.
+ * 6 / 7 = tilings 1 / 2 with two LDS tiles in flight instead of three (more workgroups per CU).
  * c_logical: input channels that carry data when C is zero-padded to a chunk (0 = C); it only enters the
  * algorithmic-work figure the profiler reports, never the arithmetic. */
 int tch_conv2d_fwd(tch_context* ctx, int dtype, const void* x, const void* w, void* y, const void* add,

@@ -1435,6 +1435,13 @@ int launch_mode(Context* ctx, IgemmArgs& a, int tile_cfg, double flops) {
       if (setting != 0 && patch_kernel_fits<MODE>(a)) return launch_cfg3<MODE, 1, 3>(ctx, a, flops);
       tile_cfg = 1;
     }
+    // 6 / 7: tilings 1 / 2 with two LDS tiles in flight instead of three (48 / 32 KB of LDS: three or four
+    // workgroups per CU, which the memory-bound data gradients of the large feature maps prefer)
+    if (tile_cfg == 6 || tile_cfg == 7) {
+      if (setting != 0 && in_c % kStep2 == 0 && a.R * a.S <= 32)
+        return tile_cfg == 6 ? launch_cfg2<MODE, 2, 2, 2, 1, 2>(ctx, a, flops) : launch_cfg2<MODE, 2, 2, 1, 1, 2>(ctx, a, flops);
+      tile_cfg -= 5;
+    }
     if (setting != 0 && in_c % kStep2 == 0 && a.R * a.S <= 32 && tile_cfg >= 0 && tile_cfg <= 2) {
       if (tile_cfg == 0)
         return setting == 3 ? launch_cfg2<MODE, 2, 2, 2, 2, 3>(ctx, a, flops) : launch_cfg2<MODE, 2, 2, 2, 2, 2>(ctx, a, flops);
@@ -1444,6 +1451,7 @@ int launch_mode(Context* ctx, IgemmArgs& a, int tile_cfg, double flops) {
     }
   }
   if (tile_cfg == 5) tile_cfg = 1;
+  if (tile_cfg == 6 || tile_cfg == 7) tile_cfg -= 5;
   switch (tile_cfg) {
     case 0:
       return launch_cfg<T, MODE, 2, 2, 2, 2>(ctx, a, flops);  // 128 x 128
@@ -1462,7 +1470,7 @@ double conv_flops(const ConvShape& s, int Ho, int Wo) {
 }
 
 // rows of the workgroup tile of a tiling number (5 = the 3x3 patch kernel, or tiling 1 where it does not fit)
-int tile_rows(int tile_cfg) { return tile_cfg == 5 ? 128 : tile_cfg >= 2 ? 64 : 128; }
+int tile_rows(int tile_cfg) { return (tile_cfg == 5 || tile_cfg == 6) ? 128 : tile_cfg >= 2 ? 64 : 128; }
 
 int64_t tiles_for(int m, int n, int bm, int bn) {
   return static_cast<int64_t>((m + bm - 1) / bm) * ((n + bn - 1) / bn);

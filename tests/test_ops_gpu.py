@@ -60,7 +60,7 @@ CONV_CASES = [
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", CONV_CASES)
-@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3, 5])
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3, 5, 6, 7])
 def test_conv_fwd(ctx, dtype, case, tile_cfg):
     from sirius_amd import ops
     N, H, W, C, K, R, S, st, pad = case
@@ -94,7 +94,7 @@ def test_conv_fwd_epilogue(ctx, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", CONV_CASES)
-@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3, 5])
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3, 5, 6, 7])
 def test_conv_dgrad(ctx, dtype, case, tile_cfg):
     from sirius_amd import ops
     N, H, W, C, K, R, S, st, pad = case
@@ -194,7 +194,7 @@ def test_bn_fwd(ctx, dtype, rows, C, fuse):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", [CONV_CASES[0], CONV_CASES[2], CONV_CASES[3], CONV_CASES[5], CONV_CASES[6], CONV_CASES[10], CONV_CASES[13]])
-@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3, 5])
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3, 5, 6, 7])
 def test_conv_with_bn_statistics(ctx, dtype, case, tile_cfg):
     """The convolution leaves per-tile sums of its stored output; BatchNorm starts from them.
     Checked against the oracle's conv -> BatchNorm(train) on the same inputs; the statistics must be
@@ -356,7 +356,7 @@ def test_bn_bwd(ctx, dtype, rows, C, masked):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", [CONV_CASES[0], CONV_CASES[1], CONV_CASES[3], CONV_CASES[4], CONV_CASES[6], CONV_CASES[10], CONV_CASES[13]])
-@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3, 5])
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3, 5, 6, 7])
 @pytest.mark.parametrize("with_add", [False, True])
 def test_conv_dgrad_with_bn_backward_sums(ctx, dtype, case, tile_cfg, with_add):
     """The data-gradient convolution gates its output by the ReLU of the BatchNorm it flows into and
