@@ -1293,19 +1293,40 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(ReduceArgs p) {
     const int i = (blockIdx.x - p.first_blocks) * 256 + threadIdx.x;
     if (i >= p.n2) return;
     float s = 0.f;
-    for (int k = 0; k < p.splits; ++k) s += p.partial2[static_cast<int64_t>(k) * p.n2 + i];
+    constexpr int U2 = 8;
+    for (int k0 = 0; k0 < p.splits; k0 += U2) {
+      float v[U2];
+#pragma unroll
+      for (int u = 0; u < U2; ++u) v[u] = p.partial2[static_cast<int64_t>(k0 + u < p.splits ? k0 + u : p.splits - 1) * p.n2 + i];
+#pragma unroll
+      for (int u = 0; u < U2; ++u)
+        if (k0 + u < p.splits) s += v[u];
+    }
     p.out2[i] = p.accumulate ? p.out2[i] + s : s;
     return;
   }
   int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
   if (i >= p.n) return;
+  // Eight partials are requested before any is added (a request past the last split repeats it and does not
+  // count): the kernel costs its dependent round trips to memory, one per trip here instead of one per split.
+  // The additions keep the order of the splits.
   float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
-  for (int k = 0; k < p.splits; ++k) {
-    float4 v = *reinterpret_cast<const float4*>(p.partial + static_cast<int64_t>(k) * p.n + i);
-    s.x += v.x;
-    s.y += v.y;
-    s.z += v.z;
-    s.w += v.w;
+  constexpr int U = 8;
+  for (int k0 = 0; k0 < p.splits; k0 += U) {
+    float4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int k = k0 + u < p.splits ? k0 + u : p.splits - 1;
+      v[u] = *reinterpret_cast<const float4*>(p.partial + static_cast<int64_t>(k) * p.n + i);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (k0 + u < p.splits) {
+        s.x += v[u].x;
+        s.y += v[u].y;
+        s.z += v[u].z;
+        s.w += v[u].w;
+      }
   }
   float4* o = reinterpret_cast<float4*>(p.out + i);
   if (p.accumulate) {
