@@ -28,6 +28,22 @@ __global__ __launch_bounds__(256) void nchw_to_nhwc_kernel(NchwArgs p) {
   Elem<T>::store(static_cast<T*>(p.y) + i, v);
 }
 
+// The same for at most one chunk of channels per pixel (images: 3 -> one 16-byte chunk): a thread makes one
+// pixel, reads its channels from the planes (neighbouring threads read neighbouring addresses of each plane)
+// and stores the chunk at once.
+template <typename T>
+__global__ __launch_bounds__(256) void nchw_to_nhwc_chunk_kernel(NchwArgs p) {
+  constexpr int E = Elem<T>::kPerChunk;
+  const int64_t pix = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  const int64_t plane = static_cast<int64_t>(p.H) * p.W;
+  if (pix >= p.N * plane) return;
+  const int64_t n = pix / plane, hw = pix - n * plane;
+  float v[E];
+#pragma unroll
+  for (int c = 0; c < E; ++c) v[c] = c < p.C ? p.x[(n * p.C + c) * plane + hw] : 0.f;
+  static_cast<uint4*>(p.y)[pix] = float_to_chunk<T>(v).u;
+}
+
 struct CastArgs {
   const void* src;
   void* dst;
@@ -79,6 +95,33 @@ __global__ __launch_bounds__(256) void filter_transpose_kernel(TransposeArgs p) 
   const int rs = static_cast<int>(t / tiles_k);
   const T* src = static_cast<const T*>(p.src) + off;
   T* dst = static_cast<T*>(p.dst) + off;
+  // 16-byte accesses where the filter allows them (K, C and the offset multiples of a chunk): a thread moves one
+  // chunk of a tile row in, one chunk of a transposed row out; element by element otherwise
+  constexpr int E = Elem<T>::kPerChunk;
+  constexpr int TPR = 32 / E;   // threads per tile row
+  if (K % E == 0 && C % E == 0 && off % E == 0) {
+    const int row = threadIdx.x / TPR, seg = threadIdx.x % TPR;
+    if (threadIdx.x < 32 * TPR) {
+      const int k = tk * 32 + row, c = tc * 32 + seg * E;
+      if (k < K && c < C) {
+        union { uint4 u; T e[E]; } v;
+        v.u = *reinterpret_cast<const uint4*>(src + (static_cast<int64_t>(k) * RS + rs) * C + c);
+#pragma unroll
+        for (int e = 0; e < E; ++e) tile[row][seg * E + e] = v.e[e];
+      }
+    }
+    __syncthreads();
+    if (threadIdx.x < 32 * TPR) {
+      const int c = tc * 32 + row, k = tk * 32 + seg * E;
+      if (c < C && k < K) {
+        union { uint4 u; T e[E]; } v;
+#pragma unroll
+        for (int e = 0; e < E; ++e) v.e[e] = tile[seg * E + e][row];
+        *reinterpret_cast<uint4*>(dst + (static_cast<int64_t>(c) * RS + rs) * K + k) = v.u;
+      }
+    }
+    return;
+  }
   const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -108,6 +151,11 @@ int nchw_to_nhwc_pad(Context* ctx, int dtype, const float* x_nchw, void* y_nhwc,
   NchwArgs a{x_nchw, y_nhwc, N, C, H, W, Cpad, static_cast<int64_t>(N) * H * W * Cpad};
   dim3 grid(static_cast<unsigned>((a.total + 255) / 256));
   const double bytes = static_cast<double>(N) * H * W * (C * 4.0 + Cpad * (dtype == kBF16 ? 2.0 : 4.0));
+  if (Cpad == (dtype == kBF16 ? 8 : 4)) {
+    const dim3 pixels(static_cast<unsigned>((static_cast<int64_t>(N) * H * W + 255) / 256));
+    return dtype == kBF16 ? launch(ctx, nchw_to_nhwc_chunk_kernel<bf16>, pixels, dim3(256), a, "nchw_to_nhwc_kernel<bf16>", bytes, 1)
+                          : launch(ctx, nchw_to_nhwc_chunk_kernel<float>, pixels, dim3(256), a, "nchw_to_nhwc_kernel<f32>", bytes, 1);
+  }
   return dtype == kBF16 ? launch(ctx, nchw_to_nhwc_kernel<bf16>, grid, dim3(256), a, "nchw_to_nhwc_kernel<bf16>", bytes, 1)
                         : launch(ctx, nchw_to_nhwc_kernel<float>, grid, dim3(256), a, "nchw_to_nhwc_kernel<f32>", bytes, 1);
 }
