@@ -49,7 +49,8 @@ class _Block:
 class ResNetEngine(EngineBase):
     def __init__(self, depths=(3, 8, 36, 3), num_classes=1000, width=64, dtype=torch.bfloat16, image_size=224,
                  lr=0.1, momentum=0.9, weight_decay=1e-4, bn_momentum=0.1, bn_eps=1e-5, stream=None, allocator=None,
-                 overlap_wgrad=True, fuse_bn_stats=True, fuse_bn_bwd=True, fuse_bn_finalize=False, autotune=False):
+                 overlap_wgrad=True, fuse_bn_stats=True, fuse_bn_bwd=True, fuse_bn_finalize=False, autotune=False,
+                 retain_gradients=False):
         self._init_engine(dtype, stream, allocator)
         assert num_classes % 8 == 0, "class count must be a multiple of one 16-byte chunk"
         self.image_size, self.num_classes = image_size, num_classes
@@ -73,6 +74,10 @@ class ResNetEngine(EngineBase):
         # autotune: when a plan is built, time each distinct convolution shape with every tiling and
         # keep the fastest (forward and data gradient separately); off = the library's heuristic
         self.autotune = autotune
+        # retain_gradients: no gradient buffer of a plan is handed out twice, and the plan lists every
+        # intermediate tensor of the step by name (plan.tensors): for inspection layer by layer; the launches,
+        # their order and their tilings are those of the ordinary plan
+        self.retain_gradients = retain_gradients
         self._tile_cache = {}
         self.tile_timings = {}   # what the tuner measured: {shape key: {"fwd_ms": {cfg: ms}, "dgrad_ms": {cfg: ms}}}
 
@@ -329,7 +334,7 @@ class ResNetEngine(EngineBase):
 
         def gfree(t, read_by_wgrad=False):
             # a buffer the side lane still reads must not be handed out again before the join
-            if read_by_wgrad and self.overlap_wgrad:
+            if (read_by_wgrad and self.overlap_wgrad) or self.retain_gradients:
                 return
             free.setdefault(t.numel(), []).append(t.reshape(-1))
 
@@ -479,6 +484,7 @@ class ResNetEngine(EngineBase):
 
         prog = ops.Program()
         marks = []  # (launch index one past the layer, 'fwd' | 'bwd', layer name): checkpoint positions
+        named = {}  # retain_gradients: every intermediate tensor of the step by name
 
         def mark(phase, name):
             marks.append((len(prog), phase, name))
@@ -514,6 +520,7 @@ class ResNetEngine(EngineBase):
                 conv_bn_fwd(blk.c3, pre + ".bn3", a2, z3, out, residual=idn, relu=True)
                 mark("fwd", pre + ".bn3")
                 saved.append((x, z1, a1, z2, a2, z3, zd, out))
+                named[pre] = dict(x=x, z1=z1, a1=a1, z2=z2, a2=a2, z3=z3, zd=zd, idn=idn, out=out)
                 x = out
             pooled = act(B, self.feat)
             ops.avgpool_fwd(ctx, x, pooled)
@@ -534,6 +541,8 @@ class ResNetEngine(EngineBase):
                              g_pooled.view(B, 1, 1, self.feat), 1, 0)
             g_out = galloc((B, Hl, Wl, self.feat))
             ops.avgpool_bwd(ctx, g_pooled, g_out)
+            named["head"] = dict(x0=x0, z0=z0, a0=a0, p0=p0, p0_idx=p0_idx, pooled=pooled, logits=logits,
+                                 dlogits=dlogits, g_pooled=g_pooled, g_feat=g_out)
             gfree(g_pooled)
             # g_rb: g_out is already gated by the block's final ReLU and stat_partial holds g_rb row tiles of
             # the sums of this block's bn3 (left by the c1 data gradient of the block after it); None = neither
@@ -598,6 +607,11 @@ class ResNetEngine(EngineBase):
                 if gx_id is not None:
                     gfree(gx_id)
                 mark("bwd", pre + ".conv1")
+                # g_out_gated: g_out arrived with this block's final ReLU applied (by the data gradient that wrote it);
+                # gx_gated: gx leaves with the ReLU of the block before applied
+                named[pre].update(g_out=g_out, g_out_gated=out_gate is None, dz3=dz3, g_a2=g_a2, dz2=dz2, g_a1=g_a1,
+                                  dz1=dz1, gx=gx, gx_gated=prev is not None, dzd=dzd if blk.cd is not None else None,
+                                  gx_id=gx_id)
                 gfree(dz1, True)
                 gfree(g_out)
                 g_out = gx
@@ -608,6 +622,7 @@ class ResNetEngine(EngineBase):
             bn_bwd("bn1", g_a0, z0, dz0, a0)
             gfree(g_a0)
             conv_wgrad(self.stem, x0, dz0)
+            named["head"].update(g_p0=g_out, g_a0=g_a0, dz0=dz0)
             gfree(dz0, True)
             ctx.join()
         finally:
@@ -616,6 +631,8 @@ class ResNetEngine(EngineBase):
         plan.marks = marks
         plan.keep = keep
         plan.logits = logits
+        plan.tensors = named if self.retain_gradients else None
+        plan.tiles = tiles
         plan.bn_save = bn_save   # [2][sum of BatchNorm widths]: saved batch mean, then inverse std
         plan.bytes = sum(t.numel() * t.element_size() for t in keep)
         return plan

@@ -337,3 +337,42 @@ def test_dynamic_compute_unit_partition_under_the_colocation_protocol(clean_runt
     assert all(torch.isfinite(v).all() for v in out["model"].state_dict().values())
     out["model"].ctx.set_cu_limit(0)
     assert tc.GetXQueueSizeAllStreams() == 0
+
+
+def test_handover_64_16_64_on_the_real_resnet152(clean_runtime, monkeypatch, tmp_path):
+    """BASELINE configs[2] at its real size: ResNet-152 (depths 3/8/36/3, 224 x 224, 1000 classes) in bf16 from the
+    shared pool, micro-batches of 64; the peer asks for memory at micro-batch 10 (target 16) and leaves at
+    micro-batch 20 (back to 64).  Every sample is trained exactly once, the batch sizes go 64 -> 16 -> 64,
+    gigabytes of activations go back to the pool, and request -> kColocateAdjustL1Done stays under 50 ms."""
+    tc = clean_runtime
+    from sirius_amd.train import resnet152 as script
+    env = {"COLTRAIN_MODE": "colocate-l1", "COLTRAIN_HOOK_MODE": "xsched-sync", "COLTRAIN_USE_XSCHED": "1",
+           "COLTRAIN_HAS_INFER_SERVER": "1", "COLTRAIN_USE_SHARED_TENSOR": "1",
+           "COLTRAIN_SHARED_TENSOR_POOL_GB": "48", "COLTRAIN_PROFILE_LOG_PATH": str(tmp_path / "train-profile.csv")}
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    n_samples = 64 * 24
+    peer = script.PeerScript({10: ("l1", 16), 20: ("exit", 64)}, delay_ms=3.0)
+    try:
+        out = script.train(1, 64, dataset_size=n_samples, dtype=torch.bfloat16, peer=peer, num_distinct_samples=64)
+    finally:
+        peer.stop()
+    stat, ctrl = out["trainer"].get_last_epoch_stat(), out["ctrl"]
+    assert stat.finished_sample == n_samples
+    assert [(k, bs) for _, k, bs in peer.sent] == [("l1", 16), ("exit", 64)]
+    req, fin = tc.get_adjust_request_time_stamp(), tc.get_adjust_done_time_stamp()
+    assert len(req) == 1 and len(fin) == 1
+    latency_ms = (fin[0] - req[0]) / 1e3
+    print(f"ResNet-152 64->16 adjust latency {latency_ms:.2f} ms, {ctrl.last_adjust}", flush=True)
+    assert 0 <= latency_ms < 50.0
+    assert ctrl.last_adjust["released_bytes"] > 4 << 30, "a batch-64 plan holds more than 6 GB of activations"
+    import csv
+    rows = [r for r in csv.DictReader(open(out["profile"])) if r["name"].startswith("batch_0")]
+    sizes = [int(r["name"].split("_")[-1]) for r in rows]
+    assert sizes[:10] == [64] * 10 and 16 in sizes and sizes[-1] == 64
+    first16, last16 = sizes.index(16), len(sizes) - 1 - sizes[::-1].index(16)
+    assert all(s <= 16 for s in sizes[first16:last16 + 1]), sizes
+    assert sum(s for r, s in zip(rows, sizes) if r["tag"] == "finish") == n_samples
+    assert stat.killed_batch >= 1
+    assert all(torch.isfinite(v).all() for v in out["model"].state_dict().values())
+    assert tc.GetXQueueSizeAllStreams() == 0

@@ -159,3 +159,53 @@ def test_gpt2_small_widths_two_layers():
     for k, ref in grads_ref.items():
         assert torch.isfinite(grads[k]).all(), k
         assert _rel(grads[k], ref) <= 2e-2, (k, _rel(grads[k], ref))
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-3), (torch.bfloat16, 2e-2)])
+def test_gpt2_small_full_depth_1024_tokens(dtype, tol):
+    """BASELINE configs[4]'s model as it is benchmarked -- 12 layers, 768 channels, 12 heads, vocabulary 50 257, a
+    1024-token causal context -- at batch 1 (the oracle runs on the CPU): logits, loss and every gradient of the
+    first step against oracle/gpt2.py on the same seeded weights and token ids; then two more AdamW steps, the
+    loss of each against the oracle's."""
+    from sirius_amd.gpt2 import GPT2Engine
+    cfg = dict(vocab=50257, n_pos=1024, n_embd=768, n_layer=12, n_head=12)
+    sd = G.make_state_dict(cfg["vocab"], cfg["n_pos"], cfg["n_embd"], cfg["n_layer"], seed=5)
+    g = torch.Generator()
+    g.manual_seed(105)
+    for k, v in sd.items():
+        if v.dim() == 1:
+            v.add_(torch.randn(v.shape, generator=g) * 0.05)
+    if dtype == torch.bfloat16:
+        sd = {k: v.to(torch.bfloat16).float() for k, v in sd.items()}
+    batches = [torch.randint(0, cfg["vocab"], (1, 1024), generator=g) for _ in range(3)]
+    ids = batches[0]
+    loss_ref, grads_ref = G.loss_and_grads(sd, ids, cfg["n_head"], cfg["n_layer"])
+    eng = GPT2Engine(seq_len=1024, dtype=dtype, lr=1e-4, weight_decay=0.01, **cfg)
+    assert eng.num_parameters() == 124_439_808
+    eng.load_state_dict(sd)
+    p, cut = eng.forward_backward(ids.cuda())
+    assert not cut
+    loss, grads = eng.last_loss(), eng.grads_dict()
+    assert abs(loss - loss_ref.item()) <= tol * abs(loss_ref.item()), (loss, loss_ref.item())
+    logits_ref = G.forward(sd, ids, cfg["n_head"], cfg["n_layer"]).reshape(1024, -1)
+    assert _rel(p.logits[:, :cfg["vocab"]].cpu(), logits_ref) <= tol
+    errs = sorted(((_rel(grads[k], ref), k) for k, ref in grads_ref.items()), reverse=True)
+    print("GPT-2 small", dtype, "loss", loss, "oracle", loss_ref.item(), "worst gradients", errs[:4], flush=True)
+    for e, k in errs:
+        assert torch.isfinite(grads[k]).all(), k
+        assert e <= tol, (k, e)
+    if dtype == torch.bfloat16:
+        names = [r["name"] for r in eng.ctx.profile(p.prog, 1)]
+        assert any("flash" in n for n in names), "the benchmark shape runs the fused attention kernels"
+        eng.forward_backward(ids.cuda())
+    losses_ref, _ = G.train_steps(sd, batches, cfg["n_head"], cfg["n_layer"], optimizer="adamw", lr=1e-4,
+                                  weight_decay=0.01)
+    losses = [loss]
+    eng.optimizer_step()
+    for b in batches[1:]:
+        eng.forward_backward(b.cuda())
+        losses.append(eng.last_loss())
+        eng.optimizer_step()
+    print("losses", losses, "oracle", losses_ref, flush=True)
+    for a, b in zip(losses, losses_ref):
+        assert abs(a - b) <= tol * abs(b), (losses, losses_ref)
