@@ -64,7 +64,10 @@ void StubBase::start() {
   thread_.reset(new std::thread([this] {
     while (running_.load()) {
       CtrlMsgEntry msg;
-      if (communicator()->timed_get(1000, kInf2Tra, config_rank(), &msg)) process_ctrl_msg(config_rank(), msg);
+      // a counted reference per wait: a shutdown on another thread cannot unmap the queue under this one
+      auto comm = communicator();
+      if (!comm) break;
+      if (comm->timed_get(1000, kInf2Tra, config_rank(), &msg)) process_ctrl_msg(config_rank(), msg);
     }
   }));
 }
@@ -90,7 +93,7 @@ void StubBase::set_cmd(int c) {
 }
 
 void StubBase::reply(uint64_t id, int event, int value) {
-  if (communicator()) communicator()->put(CtrlMsgEntry{id, event, value}, kTra2Inf, config_rank());
+  if (auto comm = communicator()) comm->put(CtrlMsgEntry{id, event, value}, kTra2Inf, config_rank());
 }
 
 void StubBase::train_start() {
@@ -122,8 +125,8 @@ bool StubBase::can_exit_after_infer_workload_done() {
 }
 
 void StubBase::set_train_first_epoch_done() {
-  if (config().has_colocated_infer_server && communicator())
-    communicator()->update_field(config_rank(), kFieldFirstEpochDone, 1);
+  if (!config().has_colocated_infer_server) return;
+  if (auto comm = communicator()) comm->update_field(config_rank(), kFieldFirstEpochDone, 1);
 }
 
 size_t StubBase::kill_in_flight_batch(int64_t* wait_ms) {
@@ -150,15 +153,15 @@ void DummyStub::process_ctrl_msg(int, const CtrlMsgEntry& msg) {
 // ---------------------------------------------------------------------------
 int ColocateStub::target_batch_size() {
   std::lock_guard<std::mutex> l(mutex_);
-  if (config().has_colocated_infer_server && communicator())
-    return communicator()->get_field(config_rank(), kFieldTargetBatchSize);
+  if (config().has_colocated_infer_server)
+    if (auto comm = communicator()) return comm->get_field(config_rank(), kFieldTargetBatchSize);
   return input_batch_size_;
 }
 
 int ColocateStub::unpub_target_batch_size() {
   std::lock_guard<std::mutex> l(mutex_);
-  if (config().has_colocated_infer_server && communicator())
-    return communicator()->get_field(config_rank(), kFieldTargetBatchSizeUnpublished);
+  if (config().has_colocated_infer_server)
+    if (auto comm = communicator()) return comm->get_field(config_rank(), kFieldTargetBatchSizeUnpublished);
   return input_batch_size_;
 }
 
@@ -188,10 +191,11 @@ void ColocateStub::process_ctrl_msg(int, const CtrlMsgEntry& msg) {
       break;
     }
     case kInferExit: {
-      if (config_rank() != 0 || !communicator()) break;
+      auto comm = communicator();
+      if (config_rank() != 0 || !comm) break;
       if (config().is_colocate_l1 && will_killed_batch_reconfig_.load(std::memory_order_acquire)) break;
-      std::vector<int> cur = communicator()->get_field_vec(kFieldTargetBatchSize);
-      std::vector<int> unpub = communicator()->get_field_vec(kFieldTargetBatchSizeUnpublished);
+      std::vector<int> cur = comm->get_field_vec(kFieldTargetBatchSize);
+      std::vector<int> unpub = comm->get_field_vec(kFieldTargetBatchSizeUnpublished);
       bool all_same = true;
       for (size_t i = 0; i < cur.size() && i < unpub.size(); ++i) all_same = all_same && cur[i] == unpub[i];
       if (!all_same && DynamicBatchDistributor::get()) DynamicBatchDistributor::get()->distribute_batch(true, false, false);

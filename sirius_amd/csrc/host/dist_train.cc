@@ -222,9 +222,10 @@ void DynamicBatchDistributor::distribute_batch(bool check, bool to_all, bool at_
 void DynamicBatchDistributor::distribute_without_lock(bool check, bool to_all, bool at_begin) {
   DistTrainLayout* l = DistTrainSync::layout();
   const int world = DistTrainSync::world_size();
-  const bool has_server = config().has_colocated_infer_server && communicator() != nullptr;
+  auto comm = config().has_colocated_infer_server ? communicator() : nullptr;
+  const bool has_server = comm != nullptr;
   std::vector<int> target_bs_unpub;
-  if (has_server) target_bs_unpub = communicator()->get_field_vec(kFieldTargetBatchSizeUnpublished);
+  if (has_server) target_bs_unpub = comm->get_field_vec(kFieldTargetBatchSizeUnpublished);
 
   const bool do_distribute = !(lazy_ || (!at_begin && policy_ == DistributePolicy::kFix));
   int num_unproc = l->num_unproc;
@@ -248,7 +249,7 @@ void DynamicBatchDistributor::distribute_without_lock(bool check, bool to_all, b
     }
     if (!ongoing.empty()) distribute_impl(ongoing, target_bs, num_unproc);
   }
-  if (has_server) communicator()->update_field_vec(kFieldTargetBatchSize, target_bs_unpub);
+  if (has_server) comm->update_field_vec(kFieldTargetBatchSize, target_bs_unpub);
 }
 
 void DynamicBatchDistributor::distribute_impl(const std::vector<int>& ongoing, const std::vector<int>& target_bs,

@@ -181,18 +181,21 @@ void tch_InfTraCommunicator_Shutdown(void) {
 }
 int tch_InfTraCommunicator_IsInitialized(void) { return communicator() != nullptr; }
 
-#define NEED_COMM() \
-  if (!communicator()) return fail("InfTraCommunicator has not been initialized")
+// one counted reference for the whole entry point: the segment stays mapped until it returns, also when another
+// thread shuts the communicator down meanwhile
+#define NEED_COMM()            \
+  auto comm = communicator();  \
+  if (!comm) return fail("InfTraCommunicator has not been initialized")
 
 int tch_mq_put(int d, int id, const tch_ctrl_msg* msg) {
   NEED_COMM();
   if (!dir_ok(d) || !msg) return fail("tch_mq_put: bad arguments");
-  return communicator()->put(to_msg(msg), static_cast<Direction>(d), id) ? 0 : fail("tch_mq_put: bad rank");
+  return comm->put(to_msg(msg), static_cast<Direction>(d), id) ? 0 : fail("tch_mq_put: bad rank");
 }
 int tch_mq_put_all(int d, const tch_ctrl_msg* msg) {
   NEED_COMM();
   if (!dir_ok(d) || !msg) return fail("tch_mq_put_all: bad arguments");
-  communicator()->put_all(to_msg(msg), static_cast<Direction>(d));
+  comm->put_all(to_msg(msg), static_cast<Direction>(d));
   return 0;
 }
 int tch_mq_put_all_vec(int d, const tch_ctrl_msg* msgs, int n) {
@@ -200,27 +203,27 @@ int tch_mq_put_all_vec(int d, const tch_ctrl_msg* msgs, int n) {
   if (!dir_ok(d) || !msgs) return fail("tch_mq_put_all_vec: bad arguments");
   std::vector<CtrlMsgEntry> v;
   for (int i = 0; i < n; ++i) v.push_back(to_msg(&msgs[i]));
-  return communicator()->put_all(v, static_cast<Direction>(d)) ? 0 : fail("one message per training rank is required");
+  return comm->put_all(v, static_cast<Direction>(d)) ? 0 : fail("one message per training rank is required");
 }
 int tch_mq_block_get(int d, int id, tch_ctrl_msg* out) {
   NEED_COMM();
-  if (!dir_ok(d) || !out || id < 0 || id >= communicator()->world_size()) return fail("tch_mq_block_get: bad arguments");
-  from_msg(communicator()->block_get(static_cast<Direction>(d), id), out);
+  if (!dir_ok(d) || !out || id < 0 || id >= comm->world_size()) return fail("tch_mq_block_get: bad arguments");
+  from_msg(comm->block_get(static_cast<Direction>(d), id), out);
   return 0;
 }
 int tch_mq_try_get(int d, int id, tch_ctrl_msg* out) {
   NEED_COMM();
-  if (!dir_ok(d) || !out || id < 0 || id >= communicator()->world_size()) return fail("tch_mq_try_get: bad arguments");
+  if (!dir_ok(d) || !out || id < 0 || id >= comm->world_size()) return fail("tch_mq_try_get: bad arguments");
   CtrlMsgEntry m;
-  if (!communicator()->try_get(static_cast<Direction>(d), id, &m)) return 0;
+  if (!comm->try_get(static_cast<Direction>(d), id, &m)) return 0;
   from_msg(m, out);
   return 1;
 }
 int tch_mq_timed_get(int d, int id, uint32_t timeout_ms, tch_ctrl_msg* out) {
   NEED_COMM();
-  if (!dir_ok(d) || !out || id < 0 || id >= communicator()->world_size()) return fail("tch_mq_timed_get: bad arguments");
+  if (!dir_ok(d) || !out || id < 0 || id >= comm->world_size()) return fail("tch_mq_timed_get: bad arguments");
   CtrlMsgEntry m;
-  if (!communicator()->timed_get(timeout_ms, static_cast<Direction>(d), id, &m)) return 0;
+  if (!comm->timed_get(timeout_ms, static_cast<Direction>(d), id, &m)) return 0;
   from_msg(m, out);
   return 1;
 }
@@ -228,63 +231,63 @@ int tch_mq_timed_get_from_any(int d, uint32_t timeout_ms, int* id, tch_ctrl_msg*
   NEED_COMM();
   if (!dir_ok(d) || !out || !id) return fail("tch_mq_timed_get_from_any: bad arguments");
   CtrlMsgEntry m;
-  if (!communicator()->timed_get_from_any(timeout_ms, static_cast<Direction>(d), id, &m)) return 0;
+  if (!comm->timed_get_from_any(timeout_ms, static_cast<Direction>(d), id, &m)) return 0;
   from_msg(m, out);
   return 1;
 }
-void tch_mq_clear(void) { if (communicator()) communicator()->clear(); }
+void tch_mq_clear(void) { if (auto comm = communicator()) comm->clear(); }
 
 int tch_init_train_info(int init_bs, int cur_bs, const char* model_name) {
   if (!config().has_colocated_infer_server) return 0;  // nothing to publish to (main.pyx:485-515)
   NEED_COMM();
   pid_t pid = getpid();
   int rank = config().train_rank, world = config().train_world_size;
-  if (!communicator()->set_train_info(rank, &pid, &rank, &world, &init_bs, &cur_bs, model_name))
+  if (!comm->set_train_info(rank, &pid, &rank, &world, &init_bs, &cur_bs, model_name))
     return fail("init_train_info: board slot rejected the update");
   return 0;
 }
 int tch_update_current_batch_size(int bs) {
   if (!config().has_colocated_infer_server) return 0;
   NEED_COMM();
-  communicator()->update_field(config().train_rank, kFieldCurrentBatchSize, bs);
+  comm->update_field(config().train_rank, kFieldCurrentBatchSize, bs);
   return 0;
 }
 int tch_train_info_get_field(int id, int field) {
   NEED_COMM();
   if (id < 0 || id >= kMaxDeviceNum || field < 0 || field > kFieldFirstEpochDone) return fail("bad board slot or field");
-  return communicator()->get_field(id, static_cast<TrainInfoField>(field));
+  return comm->get_field(id, static_cast<TrainInfoField>(field));
 }
 int tch_train_info_set_field(int id, int field, int value) {
   NEED_COMM();
   if (id < 0 || id >= kMaxDeviceNum || field < 0 || field > kFieldFirstEpochDone) return fail("bad board slot or field");
-  communicator()->update_field(id, static_cast<TrainInfoField>(field), value);
+  comm->update_field(id, static_cast<TrainInfoField>(field), value);
   return 0;
 }
 int tch_infer_required_cus_get(int device) {
   NEED_COMM();
   if (device < 0 || device >= kMaxDeviceNum) return fail("bad device");
-  return communicator()->infer_required_cus(device);
+  return comm->infer_required_cus(device);
 }
 int tch_infer_required_cus_set(int device, int n) {
   NEED_COMM();
   if (device < 0 || device >= kMaxDeviceNum || n < 0) return fail("bad device or compute-unit count");
-  communicator()->set_infer_required_cus(device, n);
+  comm->set_infer_required_cus(device, n);
   return 0;
 }
 int tch_infer_required_cus_add(int device, int delta) {
   NEED_COMM();
   if (device < 0 || device >= kMaxDeviceNum) return fail("bad device");
-  return communicator()->add_infer_required_cus(device, delta);
+  return comm->add_infer_required_cus(device, delta);
 }
 int tch_train_info_is_valid(int id) {
   NEED_COMM();
   if (id < 0 || id >= kMaxDeviceNum) return fail("bad board slot");
-  return communicator()->train_info_valid(id) ? 1 : 0;
+  return comm->train_info_valid(id) ? 1 : 0;
 }
 int tch_train_info_model_name(int id, char* out, int cap) {
   NEED_COMM();
   if (id < 0 || id >= kMaxDeviceNum || !out || cap < 1) return fail("bad arguments");
-  TrainInfo t = communicator()->get_train_info(id);
+  TrainInfo t = comm->get_train_info(id);
   strncpy(out, t.model_name, cap - 1);
   out[cap - 1] = 0;
   return static_cast<int>(strlen(out));

@@ -2,11 +2,17 @@
 
 #include <string.h>
 
+#include <mutex>
+
 namespace tch {
 namespace host {
 
 namespace {
-std::unique_ptr<InfTraCommunicator> g_comm;
+std::mutex g_comm_mu;
+std::shared_ptr<InfTraCommunicator> g_comm;   // read and replaced under g_comm_mu only
+
+// longest a blocking get sleeps before it looks at closed() again
+constexpr int64_t kWakeMs = 50;
 
 void push(ShmMsgQueue* q, const CtrlMsgEntry& m) {
   if (q->count == kMqCapacity) {  // never expected: drop the oldest rather than block the sender
@@ -120,7 +126,10 @@ bool InfTraCommunicator::put_all(const std::vector<CtrlMsgEntry>& msgs, Directio
 CtrlMsgEntry InfTraCommunicator::block_get(Direction d, int id) {
   ShmMsgQueue* q = &layout_->mq[d][id];
   ShmLock lock(&q->mu);
-  while (q->count == 0) cond_wait_ms(&q->cond, &q->mu, -1);
+  while (q->count == 0) {
+    if (closed()) return CtrlMsgEntry{0, -1, 0};
+    cond_wait_ms(&q->cond, &q->mu, kWakeMs);
+  }
   return pop(q);
 }
 
@@ -138,8 +147,8 @@ bool InfTraCommunicator::timed_get(uint32_t timeout_ms, Direction d, int id, Ctr
   const int64_t deadline = unix_timestamp_ms() + timeout_ms;
   while (q->count == 0) {
     int64_t left = deadline - unix_timestamp_ms();
-    if (left <= 0) return false;
-    cond_wait_ms(&q->cond, &q->mu, left);
+    if (left <= 0 || closed()) return false;
+    cond_wait_ms(&q->cond, &q->mu, left < kWakeMs ? left : kWakeMs);
   }
   *msg = pop(q);
   return true;
@@ -159,10 +168,10 @@ bool InfTraCommunicator::timed_get_from_any(uint32_t timeout_ms, Direction d, in
       }
     }
     int64_t left = deadline - unix_timestamp_ms();
-    if (left <= 0) return false;
+    if (left <= 0 || closed()) return false;
     // a sender signals the group condition after releasing the queue lock; poll at a
     // bounded interval so a signal that slipped in between is never waited on for long
-    cond_wait_ms(&layout_->group_cond[d], &layout_->group_mu[d], left < 50 ? left : 50);
+    cond_wait_ms(&layout_->group_cond[d], &layout_->group_mu[d], left < kWakeMs ? left : kWakeMs);
   }
 }
 
@@ -170,6 +179,7 @@ std::pair<int, CtrlMsgEntry> InfTraCommunicator::block_get_from_any(Direction d)
   int id = 0;
   CtrlMsgEntry m{};
   while (!timed_get_from_any(1000, d, &id, &m)) {
+    if (closed()) return {-1, CtrlMsgEntry{0, -1, 0}};
   }
   return {id, m};
 }
@@ -264,9 +274,13 @@ std::vector<pid_t> InfTraCommunicator::train_pids() {
   return out;
 }
 
-InfTraCommunicator* communicator() { return g_comm.get(); }
+std::shared_ptr<InfTraCommunicator> communicator() {
+  std::lock_guard<std::mutex> l(g_comm_mu);
+  return g_comm;
+}
 
 bool communicator_init(bool is_server, bool cleanup, int train_world_size, std::string* err) {
+  std::lock_guard<std::mutex> l(g_comm_mu);
   if (g_comm) {
     if (err) *err = "InfTraCommunicator has already been initialized";
     return false;
@@ -275,7 +289,18 @@ bool communicator_init(bool is_server, bool cleanup, int train_world_size, std::
   return g_comm != nullptr;
 }
 
-void communicator_shutdown() { g_comm.reset(); }
+void communicator_shutdown() {
+  // The instance is taken out of the global first, so no new caller can find it; callers that are inside it
+  // hold references of their own.  close() makes the blocked ones return within kWakeMs, and the segment is
+  // unmapped (and, on the creating side, unlinked) by whichever thread drops the last reference -- never
+  // under a thread that still waits on a mutex or condition variable inside the mapping.
+  std::shared_ptr<InfTraCommunicator> last;
+  {
+    std::lock_guard<std::mutex> l(g_comm_mu);
+    last.swap(g_comm);
+  }
+  if (last) last->close();
+}
 
 }  // namespace host
 }  // namespace tch

@@ -99,6 +99,12 @@ class InfTraCommunicator {
   static InfTraCommunicator* create(bool is_server, bool cleanup, int train_world_size, std::string* err);
   ~InfTraCommunicator();
 
+  // Ask every blocking get of THIS process to return (block_get: a message with event -1; the *_from_any
+  // form: rank -1) at its next wake-up, which is at most 50 ms away.  Called by communicator_shutdown(); the
+  // segment itself stays mapped until the last holder of the shared_ptr lets go.
+  void close() { closed_.store(true, std::memory_order_release); }
+  bool closed() const { return closed_.load(std::memory_order_acquire); }
+
   int world_size() const { return layout_->train_world_size; }
 
   // ---- message queues ----
@@ -136,10 +142,13 @@ class InfTraCommunicator {
   InfTraCommunicator() = default;
   std::unique_ptr<ShmSegment> seg_;
   InfTraLayout* layout_ = nullptr;
+  std::atomic<bool> closed_{false};   // process-local: not part of the shared layout
 };
 
-// process-wide instance used by the stubs and the batch distributor
-InfTraCommunicator* communicator();
+// Process-wide instance used by the stubs and the batch distributor.  Every caller gets a counted reference:
+// whoever is inside a call (a control thread waiting in timed_get, a side thread in put) keeps the segment
+// mapped for the length of that call, whatever another thread shuts down meanwhile.  Null when not initialised.
+std::shared_ptr<InfTraCommunicator> communicator();
 bool communicator_init(bool is_server, bool cleanup, int train_world_size, std::string* err);
 void communicator_shutdown();
 

@@ -66,7 +66,10 @@ class PeerScript:
         # a command still on its way must not reach the communicator after the runtime is shut down
         for t in self._threads:
             t.join(timeout=5.0)
+        alive = [t for t in self._threads if t.is_alive()]
         self.server.stop()
+        if alive:
+            raise RuntimeError(f"PeerScript.stop: {len(alive)} command thread(s) still running after 5 s")
 
 
 def attach_cu_partition(model):
