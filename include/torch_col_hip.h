@@ -174,6 +174,18 @@ int64_t tch_conv2d_wgrad_workspace_bytes(int dtype, int K, int R, int S, int C, 
 int tch_conv2d_wgrad(tch_context* ctx, int dtype, const void* x, const void* dy, float* dw, float* workspace,
                      int splits, int accumulate, int N, int H, int W, int C, int K, int R, int S, int stride,
                      int pad, int tile_cfg, int c_logical);
+/* tch_conv2d_wgrad for callers that cannot allocate device memory and hold no workspace of their own: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  Same kernels and same result, bit for bit, as tch_conv2d_wgrad with the same split count; the
+ * split-K partials live in a static device buffer of tch_conv2d_wgrad_static_capacity_bytes() (64 MiB) that is
+ * part of the library's code object on every GPU it runs on.  The call allocates and frees nothing.  splits <= 0:
+ * the library's choice, lowered to what the buffer holds; an explicit split count whose partials
+ * (splits * (K*R*S*C + K) * 4 bytes) exceed the buffer is rejected with an error.  All calls on one GPU share the
+ * buffer: calls that overlap on one GPU (two streams, two threads) race. */
+int64_t tch_conv2d_wgrad_static_capacity_bytes(void);
+int tch_conv2d_wgrad_static(tch_context* ctx, int dtype, const void* x, const void* dy, float* dw, int splits,
+                            int accumulate, int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
+                            int tile_cfg, int c_logical);
 /* The same, and dbias[K] (fp32) (+)= sum over pixels of dy: weight and bias gradient of a linear layer
  * (torch.nn.Linear's backward under train/gpt2.py:26 and train/swin_b.py:38) in one pass over dy. */
 int tch_conv2d_wgrad_bias(tch_context* ctx, int dtype, const void* x, const void* dy, float* dw, float* dbias,

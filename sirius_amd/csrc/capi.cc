@@ -403,6 +403,15 @@ int tch_conv2d_wgrad(tch_context* ctx, int dtype, const void* x, const void* dy,
   return conv2d_wgrad(C(ctx), dtype, s, x, dy, dw, workspace, splits, accumulate, tile_cfg);
 }
 
+int64_t tch_conv2d_wgrad_static_capacity_bytes(void) { return conv2d_wgrad_static_capacity_bytes(); }
+
+int tch_conv2d_wgrad_static(tch_context* ctx, int dtype, const void* x, const void* dy, float* dw, int splits,
+                            int accumulate, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad,
+                            int tile_cfg, int c_logical) {
+  return conv2d_wgrad_static(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad, c_logical), x, dy, dw, splits,
+                             accumulate, tile_cfg);
+}
+
 int tch_conv2d_wgrad_bias(tch_context* ctx, int dtype, const void* x, const void* dy, float* dw, float* dbias,
                           float* workspace, int splits, int accumulate, int N, int H, int W, int Cc, int K, int R, int S,
                           int stride, int pad, int tile_cfg, int c_logical) {

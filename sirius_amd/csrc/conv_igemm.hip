@@ -33,6 +33,7 @@
 #include "kernels.h"
 #include "ops.h"
 
+#include <mutex>
 #include <string>
 
 namespace tch {
@@ -1748,6 +1749,68 @@ int conv2d_wgrad(Context* ctx, int dtype, const ConvShape& s, const void* x, con
                   4.0 * r.n * (splits + 1 + (accumulate ? 1 : 0)), 1);
   }
   return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Weight gradient for callers that cannot allocate: the split-K partials go to a buffer that is part of the
+// library's own device image, so that no workspace is passed in and none is made.
+// ---------------------------------------------------------------------------------------------------------------
+}  // namespace tch
+
+// 64 MiB of fp32 partials per GPU, held from the moment the code object is loaded until the process ends.
+// Host code never touches this name: it is a host-side stand-in for a device symbol.  The device address comes
+// from hipGetSymbolAddress, once per device, and that pointer is what kernels and copies get.
+static constexpr int64_t kStaticScratchFloats = 16ll << 20;
+static __device__ __align__(256) float scratch[kStaticScratchFloats];
+
+namespace tch {
+
+namespace {
+constexpr int kScratchDevices = 16;
+std::mutex g_scratch_mu;
+float* g_scratch_ptr[kScratchDevices] = {};
+
+// The device address of `scratch` on the current device (every GPU holds its own copy at its own address).
+int static_scratch(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  TCH_CHECK_ARG(e == hipSuccess && dev >= 0 && dev < kScratchDevices,
+                std::string("conv2d_wgrad_static: hipGetDevice: ") + hipGetErrorString(e));
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    TCH_CHECK_ARG(e == hipSuccess && ptr, std::string("conv2d_wgrad_static: hipGetSymbolAddress: ") + hipGetErrorString(e));
+    g_scratch_ptr[dev] = static_cast<float*>(ptr);
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+}  // namespace
+
+int64_t conv2d_wgrad_static_capacity_bytes() { return kStaticScratchFloats * 4; }
+
+int conv2d_wgrad_static(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* dy, float* dw, int splits,
+                        int accumulate, int tile_cfg) {
+  const int64_t cap = conv2d_wgrad_static_capacity_bytes();
+  const int64_t per_split = conv2d_wgrad_workspace_bytes(s, dtype, 2) / 2;
+  TCH_CHECK_ARG(per_split > 0, "conv2d_wgrad_static: empty filter");
+  if (splits <= 0) {
+    // the library's own choice, lowered to what the buffer holds (one split needs no partials at all)
+    splits = conv2d_wgrad_pick_splits(s, dtype);
+    if (splits > cap / per_split) splits = static_cast<int>(cap / per_split);
+    if (splits < 2) splits = 1;
+  } else if (splits > 1 && conv2d_wgrad_workspace_bytes(s, dtype, splits) > cap) {
+    TCH_CHECK_ARG(false, "conv2d_wgrad_static: " + std::to_string(splits) + " splits of this filter need " +
+                             std::to_string(conv2d_wgrad_workspace_bytes(s, dtype, splits)) +
+                             " bytes of split-K partials, the static buffer holds " + std::to_string(cap));
+  }
+  float* ptr = nullptr;
+  if (splits > 1)
+    if (int rc = static_scratch(&ptr)) return rc;
+  // Every partial element the reduction reads is written by the split kernels of the same call first, so
+  // what an earlier call left in the buffer never shows; two calls that overlap on one GPU would race on it.
+  return conv2d_wgrad(ctx, dtype, s, x, dy, dw, ptr, splits, accumulate, tile_cfg);
 }
 
 }  // namespace tch

@@ -61,6 +61,10 @@ int64_t conv2d_wgrad_workspace_bytes(const ConvShape& s, int dtype, int splits);
 // dbias (optional, [K] fp32): also the column sums of dy, i.e. the gradient of a bias added to the output
 int conv2d_wgrad(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* dy, float* dw,
                  float* workspace, int splits, int accumulate, int tile_cfg, float* dbias = nullptr);
+// the same with the split-K partials in the library's static device buffer: no workspace, no allocation
+int64_t conv2d_wgrad_static_capacity_bytes();
+int conv2d_wgrad_static(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* dy, float* dw, int splits,
+                        int accumulate, int tile_cfg);
 
 // bn.hip -- training-mode BatchNorm over [rows, C] with fused ReLU / residual
 int bn_partial_rows(int64_t rows, int C, int dtype);  // number of row blocks the reductions use

@@ -317,6 +317,23 @@ def conv2d_wgrad(ctx, x, dy, dw, stride, pad, workspace=None, splits=0, accumula
           "tch_conv2d_wgrad")
 
 
+def conv2d_wgrad_static_capacity_bytes():
+    return int(lib().tch_conv2d_wgrad_static_capacity_bytes())
+
+
+def conv2d_wgrad_static(ctx, x, dy, dw, stride, pad, splits=0, accumulate=False, tile_cfg=-1, c_logical=0):
+    """conv2d_wgrad with the split-K partials in the library's static device buffer: nothing is allocated and no
+    workspace is passed (for callers that cannot allocate)."""
+    N, H, W, C = x.shape
+    K, R, S, C2 = dw.shape
+    assert C == C2 and dw.dtype == torch.float32
+    Ho, Wo = conv_out_hw(H, W, R, S, stride, pad)
+    assert tuple(dy.shape) == (N, Ho, Wo, K) and dy.dtype == x.dtype
+    check(lib().tch_conv2d_wgrad_static(ctx.handle, dtype_code(x), _p(x), _p(dy), _p(dw), splits, int(accumulate),
+                                        N, H, W, C, K, R, S, stride, pad, tile_cfg, c_logical),
+          "tch_conv2d_wgrad_static")
+
+
 # ---------------------------------------------------------------------------
 # BatchNorm
 # ---------------------------------------------------------------------------
