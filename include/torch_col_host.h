@@ -53,8 +53,15 @@ double tch_TorchColConfig_GetSharedTensorPoolGb(void);
 const char* tch_TorchColConfig_GetTrainProfileLogPath(void);
 
 /* ---- HBM pool (cython/main.pyx:228-279; common/cuda_allocator.cc:38-105,259-307) ---- */
+/* The process that initialises a pool creates its physical pages and its page table, a shared-memory segment
+ * "<prefix>_pages_pool_d<device>" (the PagesPool of common/cuda_allocator.cc:61-73: one pool, every page with
+ * its owner, visible to both processes), and serves the pages' dma-buf descriptors to peers.  Page size and
+ * unmapping policy of tch_pool_init come from COLTRAIN_POOL_PAGE_MB (default 32, CUDAMemPool::PageNbytes) and
+ * COLTRAIN_POOL_LAZY_UNMAP (default 0: FreeTrainLocals unmaps what it hands back); _ex states them. */
 int tch_pool_init(int device, uint64_t pool_bytes, int use_gpu);
+int tch_pool_init_ex(int device, uint64_t pool_bytes, int use_gpu, uint64_t page_bytes, int lazy_unmap);
 void tch_pool_shutdown(int device);
+uint64_t tch_pool_page_bytes(int device);
 int tch_pool_is_enabled(int device);
 /* number of pools this device has had so far: a holder of a pool pointer compares it with the value
  * at allocation time before freeing, so that a pointer into a pool that was shut down is dropped */
@@ -78,11 +85,27 @@ int64_t tch_pool_offset_of(int device, const void* ptr);
 /* counters (6 x u64): allocs, frees, driver maps, driver unmaps, slots that got their page back
  * without a driver call, stale mappings currently in place */
 void tch_pool_counters(int device, uint64_t* out6);
-/* FreeTrainLocals relabels pages and leaves their mappings in place (unmapping costs the driver
- * ~0.24 ms per 32 MB page, which would dominate a handover); this removes up to max_pages of
- * those stale mappings and returns how many it removed.  Never needed for correctness. */
+/* Lazy mode only: FreeTrainLocals relabels pages and leaves their mappings in place (removing a mapping costs
+ * the driver 0.26 ms whatever the page size); this removes up to max_pages of those stale mappings and returns
+ * how many it removed. */
 uint64_t tch_pool_trim(int device, uint64_t max_pages);
-/* the inference side as a fake peer needs it: label n FREE pages inference-owned / give back */
+uint64_t tch_pool_unmap_calls(int device); /* driver calls behind the unmaps (a run of neighbouring slots is one) */
+/* The pool from ANOTHER process (the inference side; the TVM-side allocator over the same PagesPool,
+ * common/cuda_allocator.cc:86-99): attach to the page table, claim FREE pages (lowest index first; returns how
+ * many, indices in pages_out), map a claimed page (its device address in this process; the descriptor comes from
+ * the pool's creator, who hands it only to the page's owner), unmap, give pages back (still-mapped ones are
+ * unmapped first), detach (gives back whatever is still owned). */
+int tch_pool_peer_attach(int device);
+void tch_pool_peer_detach(int device);
+int tch_pool_peer_num_pages(int device);
+uint64_t tch_pool_peer_page_bytes(int device);
+int tch_pool_peer_free_pages(int device);
+int tch_pool_peer_claim(int device, int n, int* pages_out);
+int tch_pool_peer_release(int device, const int* pages, int n);
+void* tch_pool_peer_map(int device, int page);
+int tch_pool_peer_unmap(int device, int page);
+/* the inference side inside the training process (a stand-in peer on a thread): label n FREE pages
+ * inference-owned / give back */
 int tch_pool_infer_claim_pages(int device, int n);
 int tch_pool_infer_release_pages(int device, int n);
 void tch_tag_model_start(int device);       /* main.pyx tag_model_start */

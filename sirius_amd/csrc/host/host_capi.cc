@@ -3,8 +3,11 @@
 // a message for tch_host_last_error().
 #include "../../../include/torch_col_host.h"
 
+#include <stdlib.h>
 #include <string.h>
 #include <unistd.h>
+
+#include <mutex>
 
 #include <string>
 
@@ -37,6 +40,23 @@ void from_msg(const CtrlMsgEntry& m, tch_ctrl_msg* out) {
 bool dir_ok(int d) { return d == kInf2Tra || d == kTra2Inf; }
 }  // namespace
 
+namespace {
+PoolOptions options_from_env() {
+  PoolOptions o;
+  if (const char* e = getenv("COLTRAIN_POOL_PAGE_MB"))
+    if (atoi(e) > 0) o.page_bytes = static_cast<size_t>(atoi(e)) << 20;
+  if (const char* e = getenv("COLTRAIN_POOL_LAZY_UNMAP")) o.lazy_unmap = atoi(e) != 0;
+  return o;
+}
+std::mutex g_peer_mu;
+std::shared_ptr<PoolPeer> g_peers[kMaxDeviceNum];
+std::shared_ptr<PoolPeer> peer(int device) {
+  if (device < 0 || device >= kMaxDeviceNum) return nullptr;
+  std::lock_guard<std::mutex> l(g_peer_mu);
+  return g_peers[device];
+}
+}  // namespace
+
 struct tch_stub {
   int kind;
   std::unique_ptr<StubBase> stub;
@@ -58,7 +78,7 @@ int tch_TorchColInit(int train_rank, int train_world_size, int use_gpu) {
   // one pool per device; a rank trains on the device of its own index (init.cc:23-28)
   if (c.use_shared_tensor && !pool(train_rank)) {
     const size_t bytes = static_cast<size_t>(c.shared_tensor_pool_gb * (1ull << 30));
-    if (!pool_init(train_rank, bytes, use_gpu != 0, &err)) return fail("pool init: " + err);
+    if (!pool_init(train_rank, bytes, use_gpu != 0, options_from_env(), &err)) return fail("pool init: " + err);
   }
   if (c.has_colocated_infer_server && !communicator()) {
     if (!communicator_init(false, false, train_world_size, &err)) return fail("communicator init: " + err);
@@ -104,23 +124,32 @@ const char* tch_TorchColConfig_GetTrainProfileLogPath(void) { return config().tr
 // ---------------------------------------------------------------------------
 int tch_pool_init(int device, uint64_t pool_bytes, int use_gpu) {
   std::string err;
-  if (!pool_init(device, pool_bytes, use_gpu != 0, &err)) return fail(err);
+  if (!pool_init(device, pool_bytes, use_gpu != 0, options_from_env(), &err)) return fail(err);
+  return 0;
+}
+int tch_pool_init_ex(int device, uint64_t pool_bytes, int use_gpu, uint64_t page_bytes, int lazy_unmap) {
+  std::string err;
+  PoolOptions o;
+  if (page_bytes) o.page_bytes = page_bytes;
+  o.lazy_unmap = lazy_unmap != 0;
+  if (!pool_init(device, pool_bytes, use_gpu != 0, o, &err)) return fail(err);
   return 0;
 }
 void tch_pool_shutdown(int device) { pool_shutdown(device); }
 int tch_pool_is_enabled(int device) { return pool(device) != nullptr; }
 uint64_t tch_pool_generation(int device) { return pool_generation(device); }
-uint64_t tch_cuda_memory_pool_infer_usage(int d) { return pool(d) ? pool(d)->stats().infer_usage : 0; }
-uint64_t tch_cuda_memory_pool_train_usage(int d) { return pool(d) ? pool(d)->stats().train_usage : 0; }
-uint64_t tch_cuda_memory_pool_train_peak_usage(int d) { return pool(d) ? pool(d)->stats().train_peak_usage : 0; }
-uint64_t tch_cuda_memory_pool_train_all_usage(int d) { return pool(d) ? pool(d)->stats().train_all_usage : 0; }
-uint64_t tch_cuda_memory_pool_free_train_local(int d) { return pool(d) ? pool(d)->empty_cache() : 0; }
-uint64_t tch_cuda_memory_pool_num_free_pages(int d) { return pool(d) ? pool(d)->stats().free_pages : 0; }
-uint64_t tch_cuda_memory_pool_nbytes(int d) { return pool(d) ? pool(d)->stats().pool_bytes : 0; }
-uint64_t tch_cuda_memory_pool_base(int d) { return pool(d) ? pool(d)->base() : 0; }
+uint64_t tch_pool_page_bytes(int d) { auto p = pool(d); return p ? p->page_bytes() : 0; }
+uint64_t tch_cuda_memory_pool_infer_usage(int d) { auto p = pool(d); return p ? p->stats().infer_usage : 0; }
+uint64_t tch_cuda_memory_pool_train_usage(int d) { auto p = pool(d); return p ? p->stats().train_usage : 0; }
+uint64_t tch_cuda_memory_pool_train_peak_usage(int d) { auto p = pool(d); return p ? p->stats().train_peak_usage : 0; }
+uint64_t tch_cuda_memory_pool_train_all_usage(int d) { auto p = pool(d); return p ? p->stats().train_all_usage : 0; }
+uint64_t tch_cuda_memory_pool_free_train_local(int d) { auto p = pool(d); return p ? p->empty_cache() : 0; }
+uint64_t tch_cuda_memory_pool_num_free_pages(int d) { auto p = pool(d); return p ? p->stats().free_pages : 0; }
+uint64_t tch_cuda_memory_pool_nbytes(int d) { auto p = pool(d); return p ? p->stats().pool_bytes : 0; }
+uint64_t tch_cuda_memory_pool_base(int d) { auto p = pool(d); return p ? p->base() : 0; }
 
 void* tch_pool_malloc(ptrdiff_t nbytes, int device, void* hip_stream) {
-  HbmPool* p = pool(device);
+  auto p = pool(device);
   if (!p) {
     fail("tch_pool_malloc: pool not initialised for this device");
     return nullptr;
@@ -134,21 +163,21 @@ void* tch_pool_malloc(ptrdiff_t nbytes, int device, void* hip_stream) {
 }
 
 void tch_pool_free(void* ptr, ptrdiff_t, int device, void*) {
-  HbmPool* p = pool(device);
+  auto p = pool(device);
   if (!p || !ptr) return;
   std::string err;
   if (!p->free(ptr, &err)) fail(err);
 }
 
 void tch_pool_record_stream(void* ptr, int device, void* hip_stream) {
-  if (HbmPool* p = pool(device)) p->record_stream(ptr, reinterpret_cast<uint64_t>(hip_stream));
+  if (auto p = pool(device)) p->record_stream(ptr, reinterpret_cast<uint64_t>(hip_stream));
 }
-uint64_t tch_pool_process_events(int device) { return pool(device) ? pool(device)->process_events() : 0; }
-int64_t tch_pool_offset_of(int device, const void* ptr) { return pool(device) ? pool(device)->offset_of(ptr) : -1; }
+uint64_t tch_pool_process_events(int device) { auto p = pool(device); return p ? p->process_events() : 0; }
+int64_t tch_pool_offset_of(int device, const void* ptr) { auto p = pool(device); return p ? p->offset_of(ptr) : -1; }
 void tch_pool_counters(int device, uint64_t* out6) {
   if (!out6) return;
   PoolStats s{};
-  if (pool(device)) s = pool(device)->stats();
+  if (auto p = pool(device)) s = p->stats();
   out6[0] = s.num_allocs;
   out6[1] = s.num_frees;
   out6[2] = s.num_maps;
@@ -156,17 +185,66 @@ void tch_pool_counters(int device, uint64_t* out6) {
   out6[4] = s.num_revives;
   out6[5] = s.stale_pages;
 }
-uint64_t tch_pool_trim(int device, uint64_t max_pages) { return pool(device) ? pool(device)->trim(max_pages) : 0; }
-int tch_pool_infer_claim_pages(int d, int n) { return pool(d) ? pool(d)->infer_claim_pages(n) : 0; }
-int tch_pool_infer_release_pages(int d, int n) { return pool(d) ? pool(d)->infer_release_pages(n) : 0; }
-void tch_tag_model_start(int d) { if (pool(d)) pool(d)->tag_model_start(); }
-void tch_tag_model_end(int d) { if (pool(d)) pool(d)->tag_model_end(); }
-int tch_tag_interm_memory(int d, void* ptr) { return pool(d) && pool(d)->tag_interm_memory(ptr) ? 1 : 0; }
-uint64_t tch_release_interm_memory(int d) { return pool(d) ? pool(d)->release_interm_memory() : 0; }
-void tch_untag_interm_memory(int d) { if (pool(d)) pool(d)->untag_interm_memory(); }
+uint64_t tch_pool_unmap_calls(int device) { auto p = pool(device); return p ? p->stats().num_unmap_calls : 0; }
+uint64_t tch_pool_trim(int device, uint64_t max_pages) { auto p = pool(device); return p ? p->trim(max_pages) : 0; }
+int tch_pool_infer_claim_pages(int d, int n) { auto p = pool(d); return p ? p->infer_claim_pages(n) : 0; }
+int tch_pool_infer_release_pages(int d, int n) { auto p = pool(d); return p ? p->infer_release_pages(n) : 0; }
+void tch_tag_model_start(int d) { if (auto p = pool(d)) p->tag_model_start(); }
+void tch_tag_model_end(int d) { if (auto p = pool(d)) p->tag_model_end(); }
+int tch_tag_interm_memory(int d, void* ptr) { auto p = pool(d); return p && p->tag_interm_memory(ptr) ? 1 : 0; }
+uint64_t tch_release_interm_memory(int d) { auto p = pool(d); return p ? p->release_interm_memory() : 0; }
+void tch_untag_interm_memory(int d) { if (auto p = pool(d)) p->untag_interm_memory(); }
 void tch_pool_null_backend_complete_events(int d, uint64_t upto) {
-  if (!pool(d)) return;
-  if (auto* nb = dynamic_cast<NullBackend*>(pool(d)->backend())) nb->completed_upto = upto;
+  auto p = pool(d);
+  if (!p) return;
+  if (auto* nb = dynamic_cast<NullBackend*>(p->backend())) nb->completed_upto = upto;
+}
+
+// ---- the pool as another process sees it ----
+int tch_pool_peer_attach(int device) {
+  if (device < 0 || device >= kMaxDeviceNum) return fail("bad device");
+  std::lock_guard<std::mutex> l(g_peer_mu);
+  if (g_peers[device]) return fail("this process is already attached to the pool of this device");
+  std::string err;
+  g_peers[device].reset(PoolPeer::attach(device, &err));
+  return g_peers[device] ? 0 : fail("tch_pool_peer_attach: " + err);
+}
+void tch_pool_peer_detach(int device) {
+  std::shared_ptr<PoolPeer> last;
+  std::lock_guard<std::mutex> l(g_peer_mu);
+  if (device >= 0 && device < kMaxDeviceNum) last.swap(g_peers[device]);
+}
+int tch_pool_peer_num_pages(int device) { auto p = peer(device); return p ? p->num_pages() : fail("not attached"); }
+uint64_t tch_pool_peer_page_bytes(int device) { auto p = peer(device); return p ? p->page_bytes() : 0; }
+int tch_pool_peer_free_pages(int device) { auto p = peer(device); return p ? p->free_pages() : fail("not attached"); }
+int tch_pool_peer_claim(int device, int n, int* pages_out) {
+  auto p = peer(device);
+  if (!p) return fail("tch_pool_peer_claim: not attached");
+  if (n < 0) return fail("tch_pool_peer_claim: negative page count");
+  return p->claim(n, pages_out);
+}
+int tch_pool_peer_release(int device, const int* pages, int n) {
+  auto p = peer(device);
+  if (!p) return fail("tch_pool_peer_release: not attached");
+  if (!pages || n < 0) return fail("tch_pool_peer_release: bad arguments");
+  return p->release(pages, n);
+}
+void* tch_pool_peer_map(int device, int page) {
+  auto p = peer(device);
+  if (!p) {
+    fail("tch_pool_peer_map: not attached");
+    return nullptr;
+  }
+  std::string err;
+  void* ptr = p->map(page, &err);
+  if (!ptr) fail("tch_pool_peer_map: " + err);
+  return ptr;
+}
+int tch_pool_peer_unmap(int device, int page) {
+  auto p = peer(device);
+  if (!p) return fail("tch_pool_peer_unmap: not attached");
+  std::string err;
+  return p->unmap(page, &err) ? 0 : fail("tch_pool_peer_unmap: " + err);
 }
 
 // ---------------------------------------------------------------------------

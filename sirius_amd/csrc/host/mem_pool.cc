@@ -1,62 +1,213 @@
 #include "mem_pool.h"
 
-#include <algorithm>
+#include <errno.h>
+#include <poll.h>
+#include <string.h>
+#include <sys/socket.h>
+#include <sys/un.h>
+#include <unistd.h>
 
-#include "shm.h"
+#include <algorithm>
 
 namespace tch {
 namespace host {
 
 namespace {
-std::unique_ptr<HbmPool> g_pools[kMaxDeviceNum];
+std::shared_ptr<HbmPool> g_pools[kMaxDeviceNum];
 std::mutex g_pools_mu;
 uint64_t g_generation[kMaxDeviceNum] = {};  // bumped per pool_init: tells a stale pointer from a live one
 
 inline size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// abstract unix socket "\0<name>": no file to clean up, gone with the last descriptor
+socklen_t abstract_addr(const std::string& name, sockaddr_un* a) {
+  memset(a, 0, sizeof(*a));
+  a->sun_family = AF_UNIX;
+  const size_t n = std::min(name.size(), sizeof(a->sun_path) - 2);
+  memcpy(a->sun_path + 1, name.data(), n);
+  return static_cast<socklen_t>(offsetof(sockaddr_un, sun_path) + 1 + n);
+}
+
+// one request of a peer: the descriptor of `page`; the answer is one status word, with the descriptor
+// attached (SCM_RIGHTS) when the status is 0
+struct FdRequest {
+  int32_t page;
+};
+
+bool send_status_fd(int sock, int32_t status, int fd) {
+  msghdr m{};
+  iovec io{&status, sizeof(status)};
+  m.msg_iov = &io;
+  m.msg_iovlen = 1;
+  alignas(cmsghdr) char ctl[CMSG_SPACE(sizeof(int))];
+  if (fd >= 0) {
+    m.msg_control = ctl;
+    m.msg_controllen = sizeof(ctl);
+    cmsghdr* h = CMSG_FIRSTHDR(&m);
+    h->cmsg_level = SOL_SOCKET;
+    h->cmsg_type = SCM_RIGHTS;
+    h->cmsg_len = CMSG_LEN(sizeof(int));
+    memcpy(CMSG_DATA(h), &fd, sizeof(int));
+  }
+  return sendmsg(sock, &m, MSG_NOSIGNAL) == static_cast<ssize_t>(sizeof(status));
+}
+
+bool recv_status_fd(int sock, int32_t* status, int* fd) {
+  msghdr m{};
+  iovec io{status, sizeof(*status)};
+  m.msg_iov = &io;
+  m.msg_iovlen = 1;
+  alignas(cmsghdr) char ctl[CMSG_SPACE(sizeof(int))];
+  m.msg_control = ctl;
+  m.msg_controllen = sizeof(ctl);
+  *fd = -1;
+  if (recvmsg(sock, &m, 0) != static_cast<ssize_t>(sizeof(*status))) return false;
+  for (cmsghdr* h = CMSG_FIRSTHDR(&m); h; h = CMSG_NXTHDR(&m, h))
+    if (h->cmsg_level == SOL_SOCKET && h->cmsg_type == SCM_RIGHTS) memcpy(fd, CMSG_DATA(h), sizeof(int));
+  return true;
+}
 }  // namespace
 
-HbmPool* HbmPool::create(int device, size_t pool_bytes, PoolBackend* backend, std::string* err) {
+std::string page_table_name(int device) { return default_shm_prefix() + "_pages_pool_d" + std::to_string(device); }
+
+HbmPool* HbmPool::create(int device, size_t pool_bytes, PoolBackend* backend, const PoolOptions& opt, std::string* err) {
   std::unique_ptr<PoolBackend> be(backend);
-  if (pool_bytes < kPageBytes) {
-    if (err) *err = "pool must hold at least one 32 MB page";
+  const size_t page = opt.page_bytes;
+  if (page < kSmallBlockBytes || page % kSmallBlockBytes != 0) {
+    if (err) *err = "the page size must be a multiple of 2 MB";
+    return nullptr;
+  }
+  if (pool_bytes < page) {
+    if (err) *err = "pool must hold at least one page";
+    return nullptr;
+  }
+  if (pool_bytes / page > static_cast<size_t>(kMaxPoolPages)) {
+    if (err) *err = "pool has more pages than the shared page table holds (" + std::to_string(kMaxPoolPages) + ")";
     return nullptr;
   }
   std::unique_ptr<HbmPool> p(new HbmPool());
   p->device_ = device;
-  p->num_pages_ = static_cast<int>(pool_bytes / kPageBytes);
-  p->pool_bytes_ = static_cast<size_t>(p->num_pages_) * kPageBytes;
+  p->page_bytes_ = page;
+  p->lazy_unmap_ = opt.lazy_unmap;
+  p->num_pages_ = static_cast<int>(pool_bytes / page);
+  p->pool_bytes_ = static_cast<size_t>(p->num_pages_) * page;
   p->va_bytes_ = p->pool_bytes_ * kVaRangeScale;
-  if (!be->reserve(p->va_bytes_, &p->base_, err)) return nullptr;
+  // The descriptor server's address first: it is taken while the process that made a pool of this name is
+  // alive, so a live pool is never taken over; a table left behind by a dead one is replaced.
+  sockaddr_un addr;
+  const socklen_t len = abstract_addr(page_table_name(device), &addr);
+  p->listen_fd_ = socket(AF_UNIX, SOCK_STREAM | SOCK_CLOEXEC, 0);
+  if (p->listen_fd_ < 0 || bind(p->listen_fd_, reinterpret_cast<sockaddr*>(&addr), len) != 0 ||
+      listen(p->listen_fd_, 16) != 0) {
+    if (err) *err = "a pool named " + page_table_name(device) + " is served by another process (" + strerror(errno) + ")";
+    return nullptr;
+  }
+  p->table_seg_.reset(ShmSegment::open(page_table_name(device), sizeof(PageTableLayout), true, true, err));
+  if (!p->table_seg_) return nullptr;
+  if (!p->table_seg_->created()) {
+    if (err) *err = "a page table named " + page_table_name(device) + " already exists";
+    return nullptr;
+  }
+  p->table_ = static_cast<PageTableLayout*>(p->table_seg_->base());
+  init_shared_mutex(&p->table_->mu);
+  p->table_->num_pages = p->num_pages_;
+  p->table_->page_bytes = page;
+  p->table_->creator_pid = static_cast<int>(getpid());
+  p->table_->has_device = be->has_device() ? 1 : 0;
+  if (!be->reserve(p->va_bytes_, page, &p->base_, err)) return nullptr;
   if (!be->create_pages(p->num_pages_, err)) return nullptr;
-  p->owner_.assign(p->num_pages_, kOwnerFree);
-  p->slot_page_.assign(p->va_bytes_ / kPageBytes, -1);
-  p->slot_live_.assign(p->va_bytes_ / kPageBytes, 0);
+  p->slot_page_.assign(p->va_bytes_ / page, -1);
+  p->slot_live_.assign(p->va_bytes_ / page, 0);
   p->page_slot_.assign(p->num_pages_, -1);
   // one eighth of the range for small blocks, the rest for large ones
-  const uint64_t small_bytes = round_up(p->va_bytes_ / 8, kPageBytes);
+  const uint64_t small_bytes = round_up(p->va_bytes_ / 8, page);
   p->small_.va_begin = p->small_.frontier = 0;
   p->small_.va_limit = small_bytes;
   p->large_.va_begin = p->large_.frontier = small_bytes;
   p->large_.va_limit = p->va_bytes_;
   p->backend_ = std::move(be);
+  p->serving_.store(true);
+  HbmPool* raw = p.get();
+  p->server_.reset(new std::thread([raw] { raw->serve_descriptors(); }));
+  p->table_seg_->mark_ready();
   return p.release();
 }
 
-HbmPool::~HbmPool() = default;
+HbmPool::~HbmPool() {
+  serving_.store(false);
+  if (server_) server_->join();
+  if (listen_fd_ >= 0) close(listen_fd_);
+}
+
+void HbmPool::set_owner(int page, PageOwner o) {
+  table_->owner[page] = o;
+  table_->owner_pid[page] = o == kOwnerFree ? 0 : static_cast<int32_t>(getpid());
+  table_->changes++;
+}
+
+void HbmPool::serve_descriptors() {
+  std::vector<pollfd> fds;
+  fds.push_back({listen_fd_, POLLIN, 0});
+  while (serving_.load()) {
+    const int n = poll(fds.data(), fds.size(), 50);
+    if (n <= 0) continue;
+    if (fds[0].revents & POLLIN) {
+      const int c = accept4(listen_fd_, nullptr, nullptr, SOCK_CLOEXEC);
+      if (c >= 0) fds.push_back({c, POLLIN, 0});
+    }
+    for (size_t i = 1; i < fds.size();) {
+      if (!(fds[i].revents & (POLLIN | POLLHUP | POLLERR))) {
+        ++i;
+        continue;
+      }
+      FdRequest rq{};
+      const ssize_t got = recv(fds[i].fd, &rq, sizeof(rq), MSG_DONTWAIT);
+      if (got != static_cast<ssize_t>(sizeof(rq))) {   // closed or broken: drop the peer
+        close(fds[i].fd);
+        fds.erase(fds.begin() + i);
+        continue;
+      }
+      // the descriptor of a page goes only to the process the table names as its owner
+      ucred cred{};
+      socklen_t cl = sizeof(cred);
+      getsockopt(fds[i].fd, SOL_SOCKET, SO_PEERCRED, &cred, &cl);
+      int32_t status = -1;
+      int fd = -1;
+      if (rq.page >= 0 && rq.page < num_pages_) {
+        bool owned;
+        {
+          ShmLock t(&table_->mu);
+          owned = table_->owner[rq.page] == kOwnerInfer && table_->owner_pid[rq.page] == static_cast<int32_t>(cred.pid);
+        }
+        if (owned) {
+          std::string err;
+          fd = backend_->export_fd(rq.page, &err);
+          status = fd >= 0 ? 0 : -2;
+        }
+      }
+      send_status_fd(fds[i].fd, status, fd);
+      if (fd >= 0) close(fd);
+      ++i;
+    }
+  }
+  for (size_t i = 1; i < fds.size(); ++i) close(fds[i].fd);
+}
 
 int HbmPool::take_free_page(std::string* err) {
   // lowest index first; a free page that still carries a stale mapping elsewhere is the last
   // resort, and loses that mapping before it is mapped anew (one page, one mapping)
+  // (called with the table locked)
   int stale = -1;
   for (int i = 0; i < num_pages_; ++i) {
-    if (owner_[i] != kOwnerFree) continue;
+    if (table_->owner[i] != kOwnerFree) continue;
     if (page_slot_[i] < 0) return i;
     if (stale < 0) stale = i;
   }
   if (stale >= 0) {
     const int64_t slot = page_slot_[stale];
-    if (!backend_->unmap(base_ + static_cast<uint64_t>(slot) * kPageBytes, stale, err)) return -1;
+    if (!backend_->unmap(base_ + static_cast<uint64_t>(slot) * page_bytes_, 1, err)) return -1;
     ++n_unmap_;
+    ++n_unmap_calls_;
     slot_page_[slot] = -1;
     page_slot_[stale] = -1;
   }
@@ -64,12 +215,19 @@ int HbmPool::take_free_page(std::string* err) {
 }
 
 bool HbmPool::ensure_mapped(uint64_t off, size_t n, std::string* err) {
-  const uint64_t first = off / kPageBytes, last = (off + n - 1) / kPageBytes;
+  const uint64_t first = off / page_bytes_, last = (off + n - 1) / page_bytes_;
+  {
+    bool all_live = true;
+    for (uint64_t s = first; s <= last && all_live; ++s) all_live = slot_live_[s] != 0;
+    if (all_live) return true;   // the common case touches no shared state
+  }
+  // ownership changes from here on: the table is locked against the other processes
+  ShmLock table_lock(&table_->mu);
   // a slot whose page was handed back but is still free gets it back without a driver call
   for (uint64_t s = first; s <= last; ++s) {
     const int page = slot_page_[s];
-    if (page >= 0 && !slot_live_[s] && owner_[page] == kOwnerFree) {
-      owner_[page] = kOwnerTrain;
+    if (page >= 0 && !slot_live_[s] && table_->owner[page] == kOwnerFree) {
+      set_owner(page, kOwnerTrain);
       slot_live_[s] = 1;
       ++n_revive_;
     }
@@ -82,14 +240,14 @@ bool HbmPool::ensure_mapped(uint64_t off, size_t n, std::string* err) {
   };
   auto count_free = [&] {
     int f = 0;
-    for (int i = 0; i < num_pages_; ++i) f += owner_[i] == kOwnerFree ? 1 : 0;
+    for (int i = 0; i < num_pages_; ++i) f += table_->owner[i] == kOwnerFree ? 1 : 0;
     return f;
   };
   int missing = count_missing();
   if (missing == 0) return true;
   if (count_free() < missing) {
     // pages cached under free blocks elsewhere may cover the shortfall
-    empty_cache_locked();
+    empty_cache_table_locked();
     missing = count_missing();
     const int free_pages = count_free();
     if (free_pages < missing) {
@@ -97,26 +255,41 @@ bool HbmPool::ensure_mapped(uint64_t off, size_t n, std::string* err) {
       return false;
     }
   }
+  // access rights are set once per run of newly mapped neighbours (the driver call costs the same for
+  // one page and for a hundred)
+  uint64_t run_first = 0, run_len = 0;
+  auto close_run = [&]() -> bool {
+    if (run_len == 0) return true;
+    const bool ok = backend_->set_access(base_ + run_first * page_bytes_, run_len * page_bytes_, err);
+    run_len = 0;
+    return ok;
+  };
   for (uint64_t s = first; s <= last; ++s) {
-    if (slot_live_[s]) continue;
+    if (slot_live_[s]) {
+      if (!close_run()) return false;
+      continue;
+    }
     if (slot_page_[s] >= 0) {
       // the page this slot used to hold now belongs to someone else: drop the stale mapping
       const int old = slot_page_[s];
-      if (!backend_->unmap(base_ + s * kPageBytes, old, err)) return false;
+      if (!backend_->unmap(base_ + s * page_bytes_, 1, err)) return false;
       ++n_unmap_;
+      ++n_unmap_calls_;
       page_slot_[old] = -1;
       slot_page_[s] = -1;
     }
     const int page = take_free_page(err);
     if (page < 0) return false;
-    if (!backend_->map(base_ + s * kPageBytes, page, err)) return false;
-    owner_[page] = kOwnerTrain;
+    if (!backend_->map(base_ + s * page_bytes_, page, err)) return false;
+    set_owner(page, kOwnerTrain);
     slot_page_[s] = page;
     page_slot_[page] = static_cast<int64_t>(s);
     slot_live_[s] = 1;
     ++n_map_;
+    if (run_len == 0) run_first = s;
+    ++run_len;
   }
-  return true;
+  return close_run();
 }
 
 bool HbmPool::alloc_in(Segment& s, size_t n, uint64_t stream, uint64_t* off_out, std::string* err) {
@@ -136,7 +309,7 @@ bool HbmPool::alloc_in(Segment& s, size_t n, uint64_t stream, uint64_t* off_out,
         s.blocks.erase(last);
       }
     }
-    const uint64_t new_frontier = round_up(start + n, kPageBytes);
+    const uint64_t new_frontier = round_up(start + n, page_bytes_);
     if (new_frontier > s.va_limit) {
       // put the trailing block back before failing
       if (start < s.frontier) {
@@ -274,50 +447,86 @@ size_t HbmPool::process_events() {
 }
 
 size_t HbmPool::empty_cache_locked() {
-  // Handing a page back is bookkeeping only: the page is relabelled FREE and its mapping into
-  // the training range is left in place ("stale").  Tearing a mapping down costs the driver
-  // about 0.24 ms per 32 MB page on MI355X -- 47 ms for the 6.5 GB a batch-64 ResNet-152 step
-  // gives up -- so it is kept off the handover path: the mapping is reused for free if the
-  // page is still FREE when the range grows again, and is only removed when the slot needs a
-  // different page, when the page is needed elsewhere, or by trim().
-  size_t bytes = 0;
-  bool quiesced = false;
+  ShmLock table_lock(&table_->mu);
+  return empty_cache_table_locked();
+}
+
+size_t HbmPool::empty_cache_table_locked() {
+  // Every page that lies wholly inside free blocks goes back as FREE.  Eager mode removes the page's
+  // mapping first, so that what the table calls FREE is mapped nowhere in this process and another
+  // process may take it: one driver call per run of neighbouring slots (0.26 ms per mapping in the run on
+  // MI355X, whatever the page size).  Lazy mode relabels only: the mapping stays (stale), is reused for
+  // free if the page is still FREE when the range grows again, and is removed when the slot needs
+  // another page, when the page is needed elsewhere, or by trim().
+  std::vector<uint64_t> slots;
   for (Segment* s : {&small_, &large_}) {
     for (auto& kv : s->blocks) {
       if (kv.second.allocated) continue;
-      const uint64_t lo = round_up(kv.first, kPageBytes);
-      const uint64_t hi = (kv.first + kv.second.size) / kPageBytes * kPageBytes;
-      for (uint64_t a = lo; a + kPageBytes <= hi; a += kPageBytes) {
-        const uint64_t slot = a / kPageBytes;
-        const int page = slot_page_[slot];
-        if (page < 0 || !slot_live_[slot]) continue;
-        if (!quiesced) {
-          // a freed block may still be read by launches in flight on its own stream (frees are
-          // stream ordered): nothing may be running when its pages change hands
-          backend_->quiesce();
-          quiesced = true;
-        }
-        slot_live_[slot] = 0;
-        owner_[page] = kOwnerFree;
-        bytes += kPageBytes;
+      const uint64_t lo = round_up(kv.first, page_bytes_);
+      const uint64_t hi = (kv.first + kv.second.size) / page_bytes_ * page_bytes_;
+      for (uint64_t a = lo; a + page_bytes_ <= hi; a += page_bytes_) {
+        const uint64_t slot = a / page_bytes_;
+        if (slot_page_[slot] >= 0 && slot_live_[slot]) slots.push_back(slot);
       }
     }
   }
-  return bytes;
+  if (slots.empty()) return 0;
+  // a freed block may still be read by launches in flight on its own stream (frees are stream
+  // ordered): nothing may be running when its pages change hands
+  backend_->quiesce();
+  std::sort(slots.begin(), slots.end());
+  if (!lazy_unmap_) {
+    for (size_t i = 0; i < slots.size();) {
+      size_t j = i + 1;
+      while (j < slots.size() && slots[j] == slots[j - 1] + 1) ++j;
+      std::string err;
+      if (backend_->unmap(base_ + slots[i] * page_bytes_, static_cast<int>(j - i), &err)) {
+        n_unmap_ += j - i;
+        ++n_unmap_calls_;
+        for (size_t k = i; k < j; ++k) {
+          page_slot_[slot_page_[slots[k]]] = -1;
+          set_owner(slot_page_[slots[k]], kOwnerFree);
+          slot_page_[slots[k]] = -1;
+          slot_live_[slots[k]] = 0;
+        }
+      } else {
+        // the driver refused: these pages stay with training (nothing was handed over)
+        for (size_t k = i; k < j; ++k) slots[k] = UINT64_MAX;
+      }
+      i = j;
+    }
+    size_t bytes = 0;
+    for (uint64_t sl : slots) bytes += sl == UINT64_MAX ? 0 : page_bytes_;
+    return bytes;
+  }
+  for (uint64_t slot : slots) {
+    slot_live_[slot] = 0;
+    set_owner(slot_page_[slot], kOwnerFree);
+  }
+  return slots.size() * page_bytes_;
 }
 
 size_t HbmPool::trim(size_t max_pages) {
   std::lock_guard<std::mutex> lock(mu_);
   size_t n = 0;
-  for (size_t slot = 0; slot < slot_page_.size() && n < max_pages; ++slot) {
-    const int page = slot_page_[slot];
-    if (page < 0 || slot_live_[slot]) continue;
+  for (size_t slot = 0; slot < slot_page_.size() && n < max_pages;) {
+    if (slot_page_[slot] < 0 || slot_live_[slot]) {
+      ++slot;
+      continue;
+    }
+    size_t end = slot + 1;
+    while (end < slot_page_.size() && end - slot < max_pages - n && slot_page_[end] >= 0 && !slot_live_[end]) ++end;
     std::string err;
-    if (!backend_->unmap(base_ + slot * kPageBytes, page, &err)) continue;
-    ++n_unmap_;
-    slot_page_[slot] = -1;
-    page_slot_[page] = -1;
-    ++n;
+    if (backend_->unmap(base_ + slot * page_bytes_, static_cast<int>(end - slot), &err)) {
+      n_unmap_ += end - slot;
+      ++n_unmap_calls_;
+      for (size_t k = slot; k < end; ++k) {
+        page_slot_[slot_page_[k]] = -1;
+        slot_page_[k] = -1;
+      }
+      n += end - slot;
+    }
+    slot = end;
   }
   return n;
 }
@@ -332,23 +541,28 @@ PoolStats HbmPool::stats() {
   std::lock_guard<std::mutex> lock(mu_);
   PoolStats st{};
   st.pool_bytes = pool_bytes_;
-  st.page_bytes = kPageBytes;
+  st.page_bytes = page_bytes_;
   st.train_usage = train_usage_;
   st.train_peak_usage = train_peak_;
   size_t train_pages = 0, infer_pages = 0, free_pages = 0;
-  for (uint8_t o : owner_) {
-    train_pages += o == kOwnerTrain;
-    infer_pages += o == kOwnerInfer;
-    free_pages += o == kOwnerFree;
+  {
+    ShmLock table_lock(&table_->mu);
+    for (int i = 0; i < num_pages_; ++i) {
+      const uint8_t o = table_->owner[i];
+      train_pages += o == kOwnerTrain;
+      infer_pages += o == kOwnerInfer;
+      free_pages += o == kOwnerFree;
+    }
   }
-  st.train_all_usage = train_pages * kPageBytes;
-  st.infer_usage = infer_pages * kPageBytes;
+  st.train_all_usage = train_pages * page_bytes_;
+  st.infer_usage = infer_pages * page_bytes_;
   st.free_pages = free_pages;
   st.num_allocs = n_alloc_;
   st.num_frees = n_free_;
   st.num_maps = n_map_;
   st.num_unmaps = n_unmap_;
   st.num_revives = n_revive_;
+  st.num_unmap_calls = n_unmap_calls_;
   for (size_t s = 0; s < slot_page_.size(); ++s) st.stale_pages += slot_page_[s] >= 0 && !slot_live_[s] ? 1 : 0;
   return st;
 }
@@ -361,10 +575,11 @@ int64_t HbmPool::offset_of(const void* ptr) const {
 
 int HbmPool::infer_claim_pages(int n) {
   std::lock_guard<std::mutex> lock(mu_);
+  ShmLock table_lock(&table_->mu);
   int moved = 0;
   for (int i = 0; i < num_pages_ && moved < n; ++i)
-    if (owner_[i] == kOwnerFree) {
-      owner_[i] = kOwnerInfer;
+    if (table_->owner[i] == kOwnerFree) {
+      set_owner(i, kOwnerInfer);
       ++moved;
     }
   return moved;
@@ -372,10 +587,12 @@ int HbmPool::infer_claim_pages(int n) {
 
 int HbmPool::infer_release_pages(int n) {
   std::lock_guard<std::mutex> lock(mu_);
+  ShmLock table_lock(&table_->mu);
+  const int32_t me = static_cast<int32_t>(getpid());
   int moved = 0;
   for (int i = num_pages_ - 1; i >= 0 && moved < n; --i)
-    if (owner_[i] == kOwnerInfer) {
-      owner_[i] = kOwnerFree;
+    if (table_->owner[i] == kOwnerInfer && table_->owner_pid[i] == me) {
+      set_owner(i, kOwnerFree);
       ++moved;
     }
   return moved;
@@ -429,12 +646,13 @@ void HbmPool::register_oom_handler(std::function<void()> fn) {
   oom_handlers_.push_back(std::move(fn));
 }
 
-HbmPool* pool(int device) {
+std::shared_ptr<HbmPool> pool(int device) {
   if (device < 0 || device >= kMaxDeviceNum) return nullptr;
-  return g_pools[device].get();
+  std::lock_guard<std::mutex> lock(g_pools_mu);
+  return g_pools[device];
 }
 
-bool pool_init(int device, size_t pool_bytes, bool use_gpu, std::string* err) {
+bool pool_init(int device, size_t pool_bytes, bool use_gpu, const PoolOptions& opt, std::string* err) {
   std::lock_guard<std::mutex> lock(g_pools_mu);
   if (device < 0 || device >= kMaxDeviceNum) {
     if (err) *err = "device id exceeds the supported device count";
@@ -445,7 +663,7 @@ bool pool_init(int device, size_t pool_bytes, bool use_gpu, std::string* err) {
     return false;
   }
   PoolBackend* be = use_gpu ? make_hip_vmm_backend(device) : new NullBackend();
-  g_pools[device].reset(HbmPool::create(device, pool_bytes, be, err));
+  g_pools[device].reset(HbmPool::create(device, pool_bytes, be, opt, err));
   if (g_pools[device]) ++g_generation[device];
   return g_pools[device] != nullptr;
 }
@@ -456,8 +674,148 @@ uint64_t pool_generation(int device) {
 }
 
 void pool_shutdown(int device) {
-  std::lock_guard<std::mutex> lock(g_pools_mu);
-  if (device >= 0 && device < kMaxDeviceNum) g_pools[device].reset();
+  // out of the table first; the pool itself goes when the last caller inside it has left
+  std::shared_ptr<HbmPool> last;
+  {
+    std::lock_guard<std::mutex> lock(g_pools_mu);
+    if (device >= 0 && device < kMaxDeviceNum) last.swap(g_pools[device]);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// PoolPeer: the page table and the pages as another process sees them
+// ---------------------------------------------------------------------------
+
+bool peer_map_descriptor(int device, int fd, size_t expect_bytes, void** ptr, std::string* err);   // mem_pool_hip.cc
+bool peer_unmap(void* ptr, std::string* err);
+
+PoolPeer* PoolPeer::attach(int device, std::string* err) {
+  std::unique_ptr<PoolPeer> p(new PoolPeer());
+  p->device_ = device;
+  p->seg_.reset(ShmSegment::open(page_table_name(device), sizeof(PageTableLayout), false, false, err));
+  if (!p->seg_) return nullptr;
+  p->table_ = static_cast<PageTableLayout*>(p->seg_->base());
+  sockaddr_un addr;
+  const socklen_t len = abstract_addr(page_table_name(device), &addr);
+  p->sock_ = socket(AF_UNIX, SOCK_STREAM | SOCK_CLOEXEC, 0);
+  if (p->sock_ < 0 || connect(p->sock_, reinterpret_cast<sockaddr*>(&addr), len) != 0) {
+    if (err) *err = std::string("descriptor server of the pool's creator: ") + strerror(errno);
+    return nullptr;
+  }
+  return p.release();
+}
+
+PoolPeer::~PoolPeer() {
+  std::vector<int> mine;
+  {
+    std::lock_guard<std::mutex> lock(mu_);
+    for (auto& kv : mapped_) {
+      std::string err;
+      peer_unmap(kv.second, &err);
+    }
+    mapped_.clear();
+  }
+  // whatever this process still owns goes back
+  if (table_) {
+    ShmLock t(&table_->mu);
+    const int32_t me = static_cast<int32_t>(getpid());
+    for (int i = 0; i < table_->num_pages; ++i)
+      if (table_->owner[i] == kOwnerInfer && table_->owner_pid[i] == me) {
+        table_->owner[i] = kOwnerFree;
+        table_->owner_pid[i] = 0;
+        table_->changes++;
+      }
+  }
+  if (sock_ >= 0) close(sock_);
+}
+
+int PoolPeer::free_pages() {
+  ShmLock t(&table_->mu);
+  int n = 0;
+  for (int i = 0; i < table_->num_pages; ++i) n += table_->owner[i] == kOwnerFree;
+  return n;
+}
+
+int PoolPeer::claim(int n, int* pages_out) {
+  ShmLock t(&table_->mu);
+  const int32_t me = static_cast<int32_t>(getpid());
+  int got = 0;
+  for (int i = 0; i < table_->num_pages && got < n; ++i)
+    if (table_->owner[i] == kOwnerFree) {
+      table_->owner[i] = kOwnerInfer;
+      table_->owner_pid[i] = me;
+      table_->changes++;
+      if (pages_out) pages_out[got] = i;
+      ++got;
+    }
+  return got;
+}
+
+int PoolPeer::release(const int* pages, int n) {
+  const int32_t me = static_cast<int32_t>(getpid());
+  int done = 0;
+  for (int k = 0; k < n; ++k) {
+    const int page = pages[k];
+    if (page < 0 || page >= table_->num_pages) continue;
+    std::string err;
+    unmap(page, &err);   // nothing of a page given back stays mapped here
+    ShmLock t(&table_->mu);
+    if (table_->owner[page] == kOwnerInfer && table_->owner_pid[page] == me) {
+      table_->owner[page] = kOwnerFree;
+      table_->owner_pid[page] = 0;
+      table_->changes++;
+      ++done;
+    }
+  }
+  return done;
+}
+
+int PoolPeer::fetch_fd(int page, std::string* err) {
+  FdRequest rq{page};
+  if (send(sock_, &rq, sizeof(rq), MSG_NOSIGNAL) != static_cast<ssize_t>(sizeof(rq))) {
+    if (err) *err = std::string("asking the pool's creator for a page descriptor: ") + strerror(errno);
+    return -1;
+  }
+  int32_t status = -1;
+  int fd = -1;
+  if (!recv_status_fd(sock_, &status, &fd)) {
+    if (err) *err = "the pool's creator closed the descriptor channel";
+    return -1;
+  }
+  if (status != 0 || fd < 0) {
+    if (fd >= 0) close(fd);
+    if (err) *err = status == -1 ? "the page table does not name this process as the owner of page " + std::to_string(page)
+                                 : "the pool's creator could not export page " + std::to_string(page);
+    return -1;
+  }
+  return fd;
+}
+
+void* PoolPeer::map(int page, std::string* err) {
+  std::lock_guard<std::mutex> lock(mu_);
+  auto it = mapped_.find(page);
+  if (it != mapped_.end()) return it->second;
+  if (!table_->has_device) {
+    if (err) *err = "this pool is the CPU model: its pages have no device memory";
+    return nullptr;
+  }
+  const int fd = fetch_fd(page, err);
+  if (fd < 0) return nullptr;
+  void* ptr = nullptr;
+  const bool ok = peer_map_descriptor(device_, fd, table_->page_bytes, &ptr, err);
+  close(fd);
+  if (!ok) return nullptr;
+  mapped_[page] = ptr;
+  return ptr;
+}
+
+bool PoolPeer::unmap(int page, std::string* err) {
+  std::lock_guard<std::mutex> lock(mu_);
+  auto it = mapped_.find(page);
+  if (it == mapped_.end()) return true;
+  const bool ok = peer_unmap(it->second, err);
+  mapped_.erase(it);
+  return ok;
 }
 
 }  // namespace host

@@ -199,6 +199,18 @@ def cuda_memory_pool_free_train_local(device_id):
     return int(lib().tch_cuda_memory_pool_free_train_local(device_id))
 
 
+def pool_counters(device_id):
+    c = (ctypes.c_uint64 * 6)()
+    lib().tch_pool_counters(device_id, c)
+    out = dict(zip(("allocs", "frees", "maps", "unmaps", "revives", "stale"), (int(v) for v in c)))
+    out["unmap_calls"] = int(lib().tch_pool_unmap_calls(device_id))
+    return out
+
+
+def pool_trim(device_id, max_pages=1 << 30):
+    return int(lib().tch_pool_trim(device_id, max_pages))
+
+
 def cuda_memory_pool_num_free_pages(device_id):
     return int(lib().tch_cuda_memory_pool_num_free_pages(device_id))
 

@@ -1,54 +1,183 @@
-"""Python half of the inference<->training handover (pytorch/torch_col/colocate_ctrl.py:30-572).
+"""Training's side of the handover protocol: when may a micro-batch be cut, what happens to the memory, what is
+answered.  Public names, exception types, event names and the `[Adjust L1 ...]` report line are those of the
+reference's controllers (pytorch/torch_col/colocate_ctrl.py:30-572); the bodies are written for this engine.
 
-The reference hangs forward / backward hooks on every leaf nn.Module; the step here is a recorded
-launch program cut into one segment per layer, and the same hook bodies run between segments
-(`engine.set_checkpoint_hook`).  Class names, the exceptions and where they are raised, the stage
-timings of the adjust line and the event names follow the reference.
+The engine's step is a recorded program of launches with a checkpoint after every layer.  A controller is
+therefore three small things:
+
+  * a *pending test*: "is the command that interrupts training set on the stub?"
+    (kColocateAdjustL1 for colocation, kInterruptTrain for task switching);
+  * a *checkpoint callback* the engine calls between launch segments, chosen by hook mode from one table
+    (_CHECKPOINT_STYLES): synchronise then look, look then kill the queued launches, or nothing at all because
+    the control thread kills on receipt and the engine raises when its launches are rejected;
+  * a *critical section* around the optimizer step (`steps_no_interrupt`), the same sequence for both
+    controllers: drain the launch queue, synchronise, announce the section to the stub, look once more -- and
+    after the section serve a command that arrived meanwhile, when nothing is in flight.
 """
 import abc
 import contextlib
 import os
 import time
-from typing import List, Optional, Union
+from typing import Callable, Optional, Union
 
 from . import _C, xsched
 from ._C import ColocateCtrlHookMode, CtrlEvent, TrainMode
 from .util import EventManager, MemoryPool
 
 
+class SwitchL1Exception(Exception):
+    pass
+
+
+class ColocateAdjustL1Exception(Exception):
+    pass
+
+
+class EngineColocateAdjustL1Exception(Exception):
+    pass
+
+
 def register_saved_tensor_hook():
-    """colocate_ctrl.py:18-27 tags every tensor autograd saves; activations here belong to the
-    engine's plan, which registers itself as their owner when it is hooked."""
+    """The reference tags every tensor autograd saves (colocate_ctrl.py:18-27); here a plan owns its
+    activations and the engine is registered as their owner when it is hooked."""
     return None
+
+
+# hook mode -> (synchronise before looking, kill the queued launches when the command is there)
+_CHECKPOINT_STYLES = {
+    ColocateCtrlHookMode.SYNC: (True, False),
+    ColocateCtrlHookMode.XSCHED_SYNC: (False, True),
+    ColocateCtrlHookMode.XSCHED_SYNC2: (False, True),
+}
 
 
 class CtrlBase(abc.ABC):
     _colocate_ctrl = None
 
+    #: what a cut raises and the first word of its message ("[Adjust XSCHED_SYNC FWD]" / "[Task Switch FWD]")
+    interrupt_exception = RuntimeError
+    interrupt_label = ""
+
     def __init__(self, train_mode: TrainMode, hook_mode: ColocateCtrlHookMode, num_epoch: int, batch_size: int):
         if CtrlBase._colocate_ctrl is not None:
             raise RuntimeError("Only one instance of Colocate Ctrl can be created.")
         CtrlBase._colocate_ctrl = self
-        self.train_mode = train_mode
-        self.hook_mode = hook_mode
-        self.input_batch_size = batch_size
-        self.num_epoch = num_epoch
+        self.train_mode, self.hook_mode = train_mode, hook_mode
+        self.num_epoch, self.input_batch_size = num_epoch, batch_size
         self._stub = None
         self._grad_fn = None
 
     @classmethod
     def _reset_singleton(cls):
-        """Lets one process build a second controller after the first was stopped (tests)."""
+        """One process may build a second controller after the first was stopped (tests)."""
         CtrlBase._colocate_ctrl = None
 
-    @abc.abstractmethod
+    # ---- what differs between the controllers ----
+    def _pending(self) -> bool:
+        """The command that interrupts training is waiting on the stub."""
+        return False
+
+    def _interruptible(self) -> bool:
+        """This train mode cuts micro-batches at all."""
+        return False
+
+    def _serve_after_step(self):
+        """A command arrived during the optimizer step; nothing is in flight now."""
+
+    # ---- the critical section around the optimizer step ----
+    @contextlib.contextmanager
     def steps_no_interrupt(self):
-        ...
+        if not self._interruptible():
+            self._begin_plain_section()
+            yield
+            self._end_plain_section()
+            return
+        where = 'before_critical_section'
+        if self.hook_mode.use_xsched():
+            # what is still queued in software has not started: it can be dropped instead of waited for
+            while xsched.get_xqueue_size() != 0:
+                if self._pending():
+                    xsched.kill_batch()
+                    raise self.interrupt_exception(where)
+        _C.SyncAllStreams()
+        if self._pending():
+            raise self.interrupt_exception(where)
+        self._stub.StepsNoInteruptBegin()
+        if self._pending():      # set between the look and the announcement
+            self._stub.StepsNoInteruptEnd()
+            raise self.interrupt_exception(where)
+        yield
+        _C.SyncAllStreams()
+        self._stub.StepsNoInteruptEnd()
+        if _C.get_train_world_size() == 1 and self._pending():
+            self._serve_after_step()
 
-    @abc.abstractmethod
+    def _begin_plain_section(self):
+        pass
+
+    def _end_plain_section(self):
+        pass
+
+    # ---- checkpoints between the launch segments of the engines ----
+    def _checkpoint(self) -> Callable[[str, str], None]:
+        """fn(phase, layer): runs after every layer of a forward / backward replay."""
+        style = _CHECKPOINT_STYLES.get(self.hook_mode)
+        if style is None:
+            raise RuntimeError(f"Unsupported hook_mode: {self.hook_mode.name}")
+        sync_first, kill_queue = style
+        mode = self.hook_mode.name if self.interrupt_label == "Adjust" else ""
+
+        def checkpoint(phase, layer):
+            if sync_first:
+                with EventManager.record_duration_event('sync_fwd' if phase == 'fwd' else 'sync_bwd'):
+                    _C.SyncAllStreams()
+            if not self._pending():
+                return
+            if kill_queue:
+                xsched.kill_batch()
+            tag = " ".join(w for w in (self.interrupt_label, mode, phase.upper()[:3]) if w)
+            raise self.interrupt_exception(f"[{tag}]")
+        return checkpoint
+
+    def get_fwd_hook(self):
+        cp = self._checkpoint()
+        return lambda module, input, output: cp('fwd', getattr(module, '__name__', ''))
+
+    def get_bwd_hook(self):
+        cp = self._checkpoint()
+        return lambda module, grad_input, grad_output: cp('bwd', getattr(module, '__name__', ''))
+
+    @classmethod
+    def register_fbward_hook(cls, module, fwd_hook, bwd_hook):
+        """The reference hangs the pair on every leaf module (colocate_ctrl.py:101-110); an engine is one leaf
+        that calls back per layer with ('fwd' | 'bwd', layer name)."""
+        if not _C.is_enable_fbward_hook() or not hasattr(module, "set_checkpoint_hook"):
+            return
+        module.set_checkpoint_hook(lambda phase, name: (fwd_hook if phase == 'fwd' else bwd_hook)(module, name, None))
+        _C.register_interm_memory_owner(module.release_activations)
+
     def register_pytorch_hook(self, module_list):
-        ...
+        if not self._interruptible():
+            return
+        if self.hook_mode == ColocateCtrlHookMode.XSCHED_SYNC2:
+            self._stub.EnableTorchColEngine()
+        if self.hook_mode == ColocateCtrlHookMode.XSCHED_SYNC2 and self.interrupt_label == "Adjust":
+            # the control thread kills on receipt; the engine notices its rejected launches and raises
+            print("SetUpTorchColEngine")
+            for engine in module_list:
+                if hasattr(engine, "set_cut_exception"):
+                    engine.set_cut_exception(EngineColocateAdjustL1Exception)
+                    _C.register_interm_memory_owner(engine.release_activations)
+            return
+        checkpoint = self._checkpoint()
+        if not _C.is_enable_fbward_hook():
+            return
+        for engine in module_list:
+            if hasattr(engine, "set_checkpoint_hook"):
+                engine.set_checkpoint_hook(checkpoint)
+                _C.register_interm_memory_owner(engine.release_activations)
 
+    # ---- release and reply ----
     def release_and_reply(self, barrier: Optional[bool] = None):
         if self.train_mode.is_colocate():
             return self.adjust()
@@ -70,6 +199,7 @@ class CtrlBase(abc.ABC):
     def unpub_target_batch_size(self):
         ...
 
+    # ---- life cycle ----
     def train_start(self):
         self._stub.train_start()
 
@@ -87,32 +217,17 @@ class CtrlBase(abc.ABC):
     def set_train_first_epoch_done(self):
         self._stub.set_train_first_epoch_done()
 
-    @classmethod
-    def register_fbward_hook(cls, module, fwd_hook, bwd_hook):
-        """colocate_ctrl.py:101-110: leaves get the hooks.  An engine is one leaf whose segments
-        call back with ('fwd' | 'bwd', layer name)."""
-        if not _C.is_enable_fbward_hook():
-            return
-        if hasattr(module, "set_checkpoint_hook"):
-            def hook(phase, name):
-                if phase == 'fwd':
-                    fwd_hook(module, name, None)
-                else:
-                    bwd_hook(module, name, None)
-            module.set_checkpoint_hook(hook)
-            _C.register_interm_memory_owner(module.release_activations)
 
-
-class SwitchL1Exception(Exception):
-    pass
-
-
-class ColocateAdjustL1Exception(Exception):
-    pass
-
-
-class EngineColocateAdjustL1Exception(Exception):
-    pass
+def _give_memory_back():
+    """The memory half of every reply: the plans' activations go back to the allocator, whole pages go back to
+    the pool (unmapped from this process unless the pool runs in lazy mode).  Returns
+    (activation bytes released, pool bytes returned, ms for the first, ms for the second)."""
+    t0 = time.time()
+    released = _C.release_interm_memory()
+    t1 = time.time()
+    returned = MemoryPool.empty_cache()
+    t2 = time.time()
+    return released, returned, (t1 - t0) * 1e3, (t2 - t1) * 1e3
 
 
 def _used_gb():
@@ -120,7 +235,10 @@ def _used_gb():
 
 
 class SwitchCtrl(CtrlBase):
-    """colocate_ctrl.py:117-301"""
+    """Task switching: inference interrupts training altogether and resumes it later
+    (colocate_ctrl.py:117-301)."""
+    interrupt_exception = SwitchL1Exception
+    interrupt_label = "Task Switch"
 
     def __init__(self, train_mode, hook_mode, num_epoch, batch_size):
         assert train_mode in {TrainMode.TASKSWITCH_L1, TrainMode.TASKSWITCH_L0}
@@ -128,77 +246,30 @@ class SwitchCtrl(CtrlBase):
         self._stub = _C.PySwitchStub()
         self._grad_fn = []
 
-    def _interrupted(self):
+    def _pending(self):
         return self._stub.cmd == CtrlEvent.kInterruptTrain
 
-    @contextlib.contextmanager
-    def steps_no_interrupt(self):
-        if self.train_mode == TrainMode.TASKSWITCH_L0:
-            yield
-            return
-        if self.hook_mode.use_xsched():
-            while xsched.get_xqueue_size() != 0:
-                if self._interrupted():
-                    xsched.kill_batch()
-                    raise SwitchL1Exception('before_critical_section')
-        _C.SyncAllStreams()
-        if self._interrupted():
-            raise SwitchL1Exception('before_critical_section')
-        self._stub.StepsNoInteruptBegin()
-        if self._interrupted():
-            self._stub.StepsNoInteruptEnd()
-            raise SwitchL1Exception('before_critical_section')
-        yield
-        _C.SyncAllStreams()
-        self._stub.StepsNoInteruptEnd()
-        if _C.get_train_world_size() == 1 and self._interrupted():
-            self.switch(barrier=False)
+    def _interruptible(self):
+        return self.train_mode != TrainMode.TASKSWITCH_L0
 
-    def register_pytorch_hook(self, module_list):
-        if self.train_mode == TrainMode.TASKSWITCH_L0:
-            return
-        if self.hook_mode == ColocateCtrlHookMode.XSCHED_SYNC2:
-            self._stub.EnableTorchColEngine()
-        for module in module_list:
-            CtrlBase.register_fbward_hook(module, self.get_fwd_hook(), self.get_bwd_hook())
-
-    def _hook(self, where):
-        sync = self.hook_mode == ColocateCtrlHookMode.SYNC
-        if not sync and not self.hook_mode.use_xsched():
-            raise RuntimeError(f"Unsupported hook_mode: {self.hook_mode.name}")
-
-        def hook(module, input, output):
-            if sync:
-                _C.SyncAllStreams()
-            if self._interrupted():
-                if not sync:
-                    xsched.kill_batch()
-                raise SwitchL1Exception(f"[Task Switch {where}]")
-        return hook
-
-    def get_fwd_hook(self):
-        return self._hook("FWD")
-
-    def get_bwd_hook(self):
-        return self._hook("BWD")
+    def _serve_after_step(self):
+        self.switch(barrier=False)
 
     def switch(self, barrier: bool):
-        if self.train_mode == TrainMode.TASKSWITCH_L1:
-            return self.switch_l1(barrier)
-        raise RuntimeError(f"Unsupported train_mode: {self.train_mode.name}")
+        if self.train_mode != TrainMode.TASKSWITCH_L1:
+            raise RuntimeError(f"Unsupported train_mode: {self.train_mode.name}")
+        return self.switch_l1(barrier)
 
     def switch_l1(self, barrier: bool):
-        t0 = time.time()
-        _C.release_interm_memory()
-        old_gpu_mem = MemoryPool.get_memory_usage()
-        MemoryPool.empty_cache()
-        cur_gpu_mem = MemoryPool.get_memory_usage()
-        succ = self.try_reply_interrupt(barrier)
-        t1 = time.time()
-        if succ:
-            print(f'[Switch L1 {(t1-t0)*1e3:.1f} ms] target batch_size: {self.target_batch_size}, '
-                  f'memory usage: {old_gpu_mem:.2f}GB -> {cur_gpu_mem:.2f}GB.', flush=True)
-        return succ
+        began = time.time()
+        before = MemoryPool.get_memory_usage()
+        _give_memory_back()
+        after = MemoryPool.get_memory_usage()
+        acknowledged = self.try_reply_interrupt(barrier)
+        if acknowledged:
+            print(f'[Switch L1 {(time.time() - began) * 1e3:.1f} ms] target batch_size: {self.target_batch_size}, '
+                  f'memory usage: {before:.2f}GB -> {after:.2f}GB.', flush=True)
+        return acknowledged
 
     def try_reply_interrupt(self, barrier):
         return self._stub.try_interrupt_train_done(barrier)
@@ -219,85 +290,35 @@ class SwitchCtrl(CtrlBase):
 
 
 class ColocateCtrl(CtrlBase):
-    """colocate_ctrl.py:310-503"""
+    """Colocation: inference asks for memory, training shrinks its batch (L1: at once, killing the micro-batch
+    in flight; L2: at the end of it) and grows back when told (colocate_ctrl.py:310-503)."""
+    interrupt_exception = ColocateAdjustL1Exception
+    interrupt_label = "Adjust"
 
     def __init__(self, train_mode, hook_mode, num_epoch, batch_size):
         assert train_mode in (TrainMode.COLOCATE_L1, TrainMode.COLOCATE_L2)
         super().__init__(train_mode, hook_mode, num_epoch, batch_size)
         self._stub = _C.PyColocateStub(batch_size)
         self._grad_fn = []
-        self.last_adjust = None  # stage timings (ms) and bytes of the most recent adjust
+        #: the most recent adjust: stage timings in ms, bytes released / returned, stale mappings left
+        self.last_adjust = None
 
-    def _adjust_l1_pending(self):
+    def _pending(self):
         return self._stub.cmd == CtrlEvent.kColocateAdjustL1
 
-    @contextlib.contextmanager
-    def steps_no_interrupt(self):
-        if self.train_mode == TrainMode.COLOCATE_L1:
-            # drain the launch queue first so that the critical section starts with nothing pending
-            if self.hook_mode.use_xsched():
-                while xsched.get_xqueue_size() != 0:
-                    if self._adjust_l1_pending():
-                        xsched.kill_batch()
-                        raise ColocateAdjustL1Exception('before_critical_section')
-            _C.SyncAllStreams()
-            if self._adjust_l1_pending():
-                raise ColocateAdjustL1Exception('before_critical_section')
-            self._stub.StepsNoInteruptBegin()
-            if self._adjust_l1_pending():
-                self._stub.StepsNoInteruptEnd()
-                raise ColocateAdjustL1Exception('before_critical_section')
-            yield
-            _C.SyncAllStreams()
-            self._stub.StepsNoInteruptEnd()
-            # a request that arrived during the step is served right after it: nothing is in flight
-            if _C.get_train_world_size() == 1 and self._adjust_l1_pending():
-                with EventManager.record_duration_event('adjust_after_step'):
-                    self.adjust()
-        else:
-            self._stub.StepsNoInteruptBegin()
-            yield
-            self._stub.StepsNoInteruptEnd()
+    def _interruptible(self):
+        return self.train_mode == TrainMode.COLOCATE_L1
 
-    def register_pytorch_hook(self, module_list):
-        if self.train_mode != TrainMode.COLOCATE_L1:
-            return
-        if self.hook_mode == ColocateCtrlHookMode.SYNC:
-            def fwd_hook(module, input, output):
-                with EventManager.record_duration_event('sync_fwd'):
-                    _C.SyncAllStreams()
-                    if self._adjust_l1_pending():
-                        raise ColocateAdjustL1Exception('[Adjust SYNC FWD]')
+    def _serve_after_step(self):
+        with EventManager.record_duration_event('adjust_after_step'):
+            self.adjust()
 
-            def bwd_hook(module, grad_input, grad_output):
-                with EventManager.record_duration_event('sync_bwd'):
-                    _C.SyncAllStreams()
-                    if self._adjust_l1_pending():
-                        raise ColocateAdjustL1Exception('[Adjust SYNC BWD]')
-        elif self.hook_mode == ColocateCtrlHookMode.XSCHED_SYNC2:
-            # the control thread kills on receipt; the engine notices the rejected launches
-            print("SetUpTorchColEngine")
-            self._stub.EnableTorchColEngine()
-            for module in module_list:
-                if hasattr(module, "set_cut_exception"):
-                    module.set_cut_exception(EngineColocateAdjustL1Exception)
-                    _C.register_interm_memory_owner(module.release_activations)
-            return
-        elif self.hook_mode.use_xsched():
-            # one event per layer would swamp the log at 310 segments a step: the checks are silent
-            def fwd_hook(module, input, output):
-                if self._adjust_l1_pending():
-                    xsched.kill_batch()
-                    raise ColocateAdjustL1Exception('[Adjust XSCHED_SYNC FWD]')
+    # L2 never cuts a micro-batch: its section only tells the stub that a step is running
+    def _begin_plain_section(self):
+        self._stub.StepsNoInteruptBegin()
 
-            def bwd_hook(module, grad_input, grad_output):
-                if self._adjust_l1_pending():
-                    xsched.kill_batch()
-                    raise ColocateAdjustL1Exception('[Adjust XSCHED_SYNC BWD]')
-        else:
-            raise RuntimeError(f"Unsupported hook_mode: {self.hook_mode.name}")
-        for module in module_list:
-            CtrlBase.register_fbward_hook(module, fwd_hook, bwd_hook)
+    def _end_plain_section(self):
+        self._stub.StepsNoInteruptEnd()
 
     def adjust(self):
         if self.train_mode == TrainMode.COLOCATE_L1:
@@ -307,41 +328,42 @@ class ColocateCtrl(CtrlBase):
         raise RuntimeError(f"Unsupported train_mode: {self.train_mode.name}")
 
     def adjust_l1(self):
-        """colocate_ctrl.py:413-445: release activations | return whole pages | reply | read usage."""
-        t0 = time.time()
+        """Release | return pages | reply | read usage: the four stage times of the report line
+        (colocate_ctrl.py:413-445)."""
         with EventManager.record_duration_event('adjust_l1'):
-            old_cached, old_alloc = _used_gb()
-            released = _C.release_interm_memory()
-            t1 = time.time()
-            freed = MemoryPool.empty_cache()
-            t2 = time.time()
+            cached0, alloc0 = _used_gb()
+            released, returned, release_ms, pages_ms = _give_memory_back()
+            t = time.time()
             self._stub.adjust_l1_done()
-            t3 = time.time()
-            cur_cached, cur_alloc = _used_gb()
-        t4 = time.time()
-        self.last_adjust = {"release_ms": (t1 - t0) * 1e3, "empty_cache_ms": (t2 - t1) * 1e3,
-                            "reply_ms": (t3 - t2) * 1e3, "stat_ms": (t4 - t3) * 1e3,
-                            "released_bytes": released, "pool_bytes_returned": freed}
+            reply_ms = (time.time() - t) * 1e3
+            t = time.time()
+            cached1, alloc1 = _used_gb()
+        stat_ms = (time.time() - t) * 1e3
+        # lazy pools answer first and take the mappings of the pages they gave away down afterwards
+        trimmed = MemoryPool.trim_stale_mappings()
+        self.last_adjust = {"release_ms": release_ms, "empty_cache_ms": pages_ms, "reply_ms": reply_ms,
+                            "stat_ms": stat_ms, "released_bytes": released, "pool_bytes_returned": returned,
+                            "trimmed_after_reply": trimmed, "stale_pages_after": MemoryPool.stale_pages()}
         print(f'[Rank {_C.get_train_rank()} | PID {os.getpid()} | {_C.get_unix_timestamp_us()/1000}]'
-              f' [Adjust L1 {(t1-t0)*1e3:.1f} | {(t2-t1)*1e3:.1f} | {(t3-t2)*1e3:.1f} | {(t4-t3)*1e3:.1f} ms]'
+              f' [Adjust L1 {release_ms:.1f} | {pages_ms:.1f} | {reply_ms:.1f} | {stat_ms:.1f} ms]'
               f' target batch_size: {self.target_batch_size},'
-              f' memory cached: {old_cached:.2f}GB -> {cur_cached:.2f}GB,'
-              f' memory allocated: {old_alloc:.2f}GB -> {cur_alloc:.2f}GB.', flush=True)
+              f' memory cached: {cached0:.2f}GB -> {cached1:.2f}GB,'
+              f' memory allocated: {alloc0:.2f}GB -> {alloc1:.2f}GB.', flush=True)
 
     def adjust_l2(self):
-        """colocate_ctrl.py:448-469"""
-        t0 = time.time()
+        """colocate_ctrl.py:448-469: nothing is in flight at the end of a micro-batch; cached pages go back."""
+        began = time.time()
         with EventManager.record_duration_event('adjust_l2'):
-            old_cached, old_alloc = _used_gb()
-            freed = MemoryPool.empty_cache()
+            cached0, alloc0 = _used_gb()
+            returned = MemoryPool.empty_cache()
             self._stub.adjust_l2_done()
-            cur_cached, cur_alloc = _used_gb()
-        t1 = time.time()
-        self.last_adjust = {"empty_cache_ms": (t1 - t0) * 1e3, "pool_bytes_returned": freed}
-        print(f'[{_C.get_unix_timestamp_us()/1000}] [Adjust L2 {(t1-t0)*1e3:.1f} ms]'
+            cached1, alloc1 = _used_gb()
+        took_ms = (time.time() - began) * 1e3
+        self.last_adjust = {"empty_cache_ms": took_ms, "pool_bytes_returned": returned}
+        print(f'[{_C.get_unix_timestamp_us()/1000}] [Adjust L2 {took_ms:.1f} ms]'
               f' target batch_size: {self.target_batch_size},'
-              f' memory cached: {old_cached:.2f}GB -> {cur_cached:.2f}GB,'
-              f' memory allocated: {old_alloc:.2f}GB -> {cur_alloc:.2f}GB.', flush=True)
+              f' memory cached: {cached0:.2f}GB -> {cached1:.2f}GB,'
+              f' memory allocated: {alloc0:.2f}GB -> {alloc1:.2f}GB.', flush=True)
 
     def report_batch_size(self, batch_size):
         self._stub.report_batch_size(batch_size)
@@ -362,21 +384,14 @@ class ColocateCtrl(CtrlBase):
 
 
 class DummyCtrl(CtrlBase):
-    """colocate_ctrl.py:506-553"""
+    """Training alone on the GPU: nobody interrupts (colocate_ctrl.py:506-553)."""
 
     def __init__(self, train_mode, hook_mode, num_epoch, batch_size):
         super().__init__(train_mode, hook_mode, num_epoch, batch_size)
         self._stub = _C.PyDummyStub()
         assert hook_mode == ColocateCtrlHookMode.NONE
 
-    @contextlib.contextmanager
-    def steps_no_interrupt(self):
-        yield
-
     def check_async_killed_batch(self):
-        pass
-
-    def register_pytorch_hook(self, module_list):
         pass
 
     def report_batch_size(self, batch_size):
@@ -397,12 +412,14 @@ class DummyCtrl(CtrlBase):
 def create_colocate_ctrl(train_mode: TrainMode, hook_mode: ColocateCtrlHookMode, num_epoch: int,
                          batch_size: int) -> Union[DummyCtrl, ColocateCtrl, SwitchCtrl]:
     if train_mode == TrainMode.NORMAL:
-        return DummyCtrl(train_mode, hook_mode, num_epoch, batch_size)
-    if train_mode.is_colocate():
-        return ColocateCtrl(train_mode, hook_mode, num_epoch, batch_size)
-    if train_mode.is_taskswitch() or train_mode == TrainMode.TASKSWITCH_L0:
-        return SwitchCtrl(train_mode, hook_mode, num_epoch, batch_size)
-    raise RuntimeError(f"Unsupported train_mode: {train_mode}")
+        kind = DummyCtrl
+    elif train_mode.is_colocate():
+        kind = ColocateCtrl
+    elif train_mode.is_taskswitch() or train_mode == TrainMode.TASKSWITCH_L0:
+        kind = SwitchCtrl
+    else:
+        raise RuntimeError(f"Unsupported train_mode: {train_mode}")
+    return kind(train_mode, hook_mode, num_epoch, batch_size)
 
 
 def get_colocate_ctrl() -> Union[DummyCtrl, ColocateCtrl, SwitchCtrl]:

@@ -84,6 +84,20 @@ class MemoryPool:
             torch.cuda.empty_cache()
         return 0
 
+    @classmethod
+    def stale_pages(cls):
+        """Mappings this process still holds over pages it gave back (lazy pools only; 0 otherwise)."""
+        if not _C.is_enable_shared_tensor():
+            return 0
+        return _C.pool_counters(_C.get_train_rank())["stale"]
+
+    @classmethod
+    def trim_stale_mappings(cls):
+        """Remove those mappings; returns how many.  A pool in eager mode has none."""
+        if not _C.is_enable_shared_tensor():
+            return 0
+        return _C.pool_trim(_C.get_train_rank())
+
 
 @dataclass
 class Event:

@@ -11,14 +11,19 @@ What pins each part (none of them has stored expectations in the reference's tes
   pool         configuration constants (common/cuda_allocator.cc:61-85) + determinism of offsets
 """
 import ctypes
+import json
 import multiprocessing as mp
 import os
 import random
+import subprocess
+import sys
 import time
 
 import pytest
 
 from sirius_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 from sirius_amd._lib import CtrlMsg, lib
 
 _PORT = [20000 + (os.getpid() % 5000) * 7]
@@ -692,11 +697,11 @@ def _counters(L):
     return dict(zip(("allocs", "frees", "maps", "unmaps", "revives", "stale"), (int(v) for v in c)))
 
 
-def test_pool_hands_pages_back_without_unmapping(fresh):
-    """Returning pages is bookkeeping: no driver unmap on the handover path; the mapping is reused
+def test_pool_lazy_mode_hands_pages_back_without_unmapping(fresh):
+    """Lazy mode: returning pages is bookkeeping, no driver unmap on the handover path; the mapping is reused
     when the page is still free at regrowth, and replaced when inference has taken the page."""
     L = fresh
-    assert L.tch_pool_init(0, 128 * MB, 0) == 0            # 4 pages
+    assert L.tch_pool_init_ex(0, 128 * MB, 0, 32 * MB, 1) == 0            # 4 pages, lazy unmapping
     try:
         a = L.tch_pool_malloc(64 * MB, 0, None)
         assert _counters(L)["maps"] == 2
@@ -724,6 +729,126 @@ def test_pool_hands_pages_back_without_unmapping(fresh):
         assert L.tch_pool_infer_release_pages(0, 3) == 3
     finally:
         L.tch_pool_shutdown(0)
+
+
+def test_pool_eager_mode_unmaps_what_it_hands_back(fresh):
+    """The default: a page the table calls FREE is mapped nowhere in the training process.  Neighbouring slots
+    go in one driver call; growing back maps again (no revival), and the offsets are the same as in lazy mode."""
+    L = fresh
+    assert L.tch_pool_init(0, 256 * MB, 0) == 0             # 8 pages of 32 MB, eager
+    try:
+        assert L.tch_pool_page_bytes(0) == 32 * MB
+        a = L.tch_pool_malloc(96 * MB, 0, None)
+        keep = L.tch_pool_malloc(32 * MB, 0, None)
+        b = L.tch_pool_malloc(64 * MB, 0, None)
+        assert _counters(L)["maps"] == 6
+        L.tch_pool_free(a, 0, 0, None)
+        L.tch_pool_free(b, 0, 0, None)
+        assert L.tch_cuda_memory_pool_free_train_local(0) == 160 * MB
+        c = _counters(L)
+        assert c["unmaps"] == 5 and c["stale"] == 0
+        assert L.tch_pool_unmap_calls(0) == 2                # two runs: slots 0-2 and slots 4-5
+        assert L.tch_cuda_memory_pool_num_free_pages(0) == 7 and L.tch_cuda_memory_pool_train_all_usage(0) == 32 * MB
+        a2 = L.tch_pool_malloc(96 * MB, 0, None)
+        assert a2 == a
+        c = _counters(L)
+        assert c["maps"] == 9 and c["revives"] == 0
+        assert L.tch_pool_trim(0, 100) == 0
+        L.tch_pool_free(a2, 0, 0, None)
+        L.tch_pool_free(keep, 0, 0, None)
+    finally:
+        L.tch_pool_shutdown(0)
+
+
+def test_pool_offsets_do_not_depend_on_the_unmapping_mode_and_scale_to_the_whole_part(fresh):
+    """The same trace gives the same offsets eager or lazy; a pool of 256 GB (the part has 288) follows it too,
+    and runs with 128 MB pages as well (a segment grows in whole pages, so placement then differs)."""
+    L = fresh
+    runs = {}
+    for name, (size, page, lazy) in {"eager": (1024 * MB, 32 * MB, 0), "lazy": (1024 * MB, 32 * MB, 1),
+                                     "big": (256 * 1024 * MB, 32 * MB, 0), "big128": (256 * 1024 * MB, 128 * MB, 0)}.items():
+        assert L.tch_pool_init_ex(0, size, 0, page, lazy) == 0, L.tch_host_last_error()
+        assert L.tch_cuda_memory_pool_num_free_pages(0) == size // page
+        runs[name] = _trace(L, 5)
+        L.tch_pool_shutdown(0)
+    assert runs["eager"] == runs["lazy"]
+    big_base = 256 * 1024 * MB          # start of the large segment: one eighth of 8 x 256 GB
+    small_base = 1024 * MB
+    rebased = [o if not isinstance(o, int) or o < small_base else o - small_base + big_base for o in runs["eager"]]
+    # the 1 GB pool runs out of pages where the big pool does not: compare up to the first failure
+    upto = next((i for i, o in enumerate(runs["eager"]) if o == -1), len(rebased))
+    def offsets_only(r):
+        return [o for o in r if isinstance(o, int)]
+    assert offsets_only(runs["big"][:upto]) == offsets_only(rebased[:upto])
+    assert -1 not in runs["big"] and -1 not in runs["big128"]
+    assert all(o % 1024 == 0 for o in offsets_only(runs["big128"]))
+    assert L.tch_pool_init_ex(0, 1024 * 1024 * MB, 0, 32 * MB, 0) < 0      # more pages than the table holds
+    assert b"page table" in L.tch_host_last_error()
+
+
+_PEER_CHILD = r"""
+import ctypes, json, os, sys
+sys.path.insert(0, sys.argv[1])
+from sirius_amd._lib import lib
+L = lib()
+out = {}
+assert L.tch_pool_peer_attach(0) == 0, L.tch_host_last_error()
+out["pages"], out["page_bytes"], out["free"] = L.tch_pool_peer_num_pages(0), L.tch_pool_peer_page_bytes(0), L.tch_pool_peer_free_pages(0)
+got = (ctypes.c_int * 16)()
+out["claimed"] = L.tch_pool_peer_claim(0, 5, got)
+out["indices"] = list(got)[:out["claimed"]]
+out["map"] = L.tch_pool_peer_map(0, got[0])
+out["map_error"] = L.tch_host_last_error().decode()
+print(json.dumps(out), flush=True)
+sys.stdin.readline()                      # the parent looks at the table, then lets us go on
+back = (ctypes.c_int * 2)(got[0], got[1])
+rel = L.tch_pool_peer_release(0, back, 2)
+print(json.dumps({"released": rel, "free": L.tch_pool_peer_free_pages(0)}), flush=True)
+sys.stdin.readline()
+os._exit(0)                               # dies holding three pages: detach never runs
+"""
+
+
+def test_pool_page_table_is_shared_with_another_process(fresh, tmp_path):
+    """The page table lives in shared memory: a separate process attaches, sees the same pages, claims FREE
+    ones (the trainer then cannot grow over them), gives some back, and the pages of a peer that died are
+    there to be taken back.  (CPU model: there is no device memory to map; the GPU test maps and writes.)"""
+    L = fresh
+    assert L.tch_pool_init(0, 256 * MB, 0) == 0              # 8 pages
+    child = None
+    try:
+        a = L.tch_pool_malloc(64 * MB, 0, None)              # pages 0, 1 -> training
+        child = subprocess.Popen([sys.executable, "-c", _PEER_CHILD, ROOT], stdin=subprocess.PIPE, stdout=subprocess.PIPE,
+                                 env=dict(os.environ), text=True)
+        first = json.loads(child.stdout.readline())
+        assert first["pages"] == 8 and first["page_bytes"] == 32 * MB and first["free"] == 6
+        assert first["claimed"] == 5 and first["indices"] == [2, 3, 4, 5, 6]
+        assert not first["map"] and "CPU model" in first["map_error"]
+        assert L.tch_cuda_memory_pool_infer_usage(0) == 5 * 32 * MB
+        assert L.tch_cuda_memory_pool_num_free_pages(0) == 1
+        assert L.tch_pool_malloc(64 * MB, 0, None) is None    # one page left: training cannot grow by two
+        child.stdin.write("\n")
+        child.stdin.flush()
+        second = json.loads(child.stdout.readline())
+        assert second == {"released": 2, "free": 3}
+        b = L.tch_pool_malloc(64 * MB, 0, None)               # now it can
+        assert b
+        assert L.tch_cuda_memory_pool_num_free_pages(0) == 1
+        child.stdin.write("\n")
+        child.stdin.flush()
+        child.wait(timeout=20)
+        # the in-process stand-in only ever gives back its own pages, not the dead peer's
+        assert L.tch_pool_infer_release_pages(0, 8) == 0
+        assert L.tch_cuda_memory_pool_infer_usage(0) == 3 * 32 * MB
+        L.tch_pool_free(a, 0, 0, None)
+        L.tch_pool_free(b, 0, 0, None)
+    finally:
+        if child is not None and child.poll() is None:
+            child.kill()
+        L.tch_pool_shutdown(0)
+    # a second pool of the same name can be made once the first is gone; a live one is not taken over
+    assert L.tch_pool_init(0, 64 * MB, 0) == 0
+    L.tch_pool_shutdown(0)
 
 
 def test_pool_cross_stream_free_is_deferred(fresh):

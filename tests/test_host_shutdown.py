@@ -34,7 +34,7 @@ def test_shutdown_under_blocked_waiters(tmp_path, sanitizer):
         out, _ = p.communicate()
         assert p.returncode == 0, out.decode()[-3000:]
     exe = str(tmp_path / "shutdown_race")
-    link = subprocess.run([hipcc, f"-fsanitize={sanitizer}", "-fno-gpu-sanitize"] + objs + ["-o", exe, "-lpthread", "-lrt"],
+    link = subprocess.run([hipcc, f"-fsanitize={sanitizer}", "-fno-gpu-sanitize"] + objs + ["-o", exe, "-lpthread", "-lrt", "-lhsa-runtime64"],
                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
     assert link.returncode == 0, link.stdout.decode()[-3000:]
     env = dict(os.environ, TSAN_OPTIONS="halt_on_error=1 exitcode=66", ASAN_OPTIONS="detect_leaks=0 exitcode=67")
