@@ -94,6 +94,13 @@ int tch_SyncStream(uint64_t hip_stream);            /* xsched_ctrl.cc:140-147 */
 int tch_SyncAllStreams(void);                       /* xsched_ctrl.cc:149-156 */
 int tch_QueryRejectCudaCalls(void);                 /* xsched_ctrl.cc:192-194 */
 void tch_SetRejectCudaCalls(int reject);            /* xsched_ctrl.cc:196-198 */
+/* Every registered queue stops handing launches to the hardware (what it already handed over runs on; with
+ * sync_hw the call returns when that has finished), until resumed; launches submitted meanwhile wait in
+ * order, or are dropped by tch_ResumeAllStreams(1).  Work another tenant submits to its own stream in between
+ * runs ahead of everything the queues hold: preemption between kernels
+ * (third_party/xsched/preempt/xqueue/xqueue.cpp:80-137 Suspend / Resume). */
+void tch_SuspendAllStreams(int sync_hw);
+void tch_ResumeAllStreams(int drop_commands);
 /* queue length / sync interval used by later tch_RegisterStream calls (reference: 16, 8) */
 void tch_SetXQueueShape(int queue_length, int sync_interval);
 size_t tch_GetXQueueInFlight(uint64_t hip_stream);
@@ -165,6 +172,11 @@ int tch_conv2d_dgrad_bn(tch_context* ctx, int dtype, const void* dy, const void*
 /* y = relu?(x * scale + shift (+ residual)), coef = scale[C], shift[C];  dx = c0 * g + c1 * x + c2, coef = [3][C] */
 int tch_bn_apply_fwd(tch_context* ctx, int dtype, const void* x, void* y, const void* residual, int relu, int64_t rows,
                      int C, const float* coef);
+/* Inference-mode BatchNorm (model.eval(): F.batch_norm with training=False, as the batch-1 ResNet-152 requests of
+ * the colocated inference side run it): coef = scale[C], shift[C] with scale = gamma / sqrt(running_var + eps),
+ * shift = beta - running_mean * scale; apply with tch_bn_apply_fwd. */
+int tch_bn_eval_coef(tch_context* ctx, const float* gamma, const float* beta, const float* running_mean,
+                     const float* running_var, float* coef, int C, float eps);
 int tch_bn_apply_bwd(tch_context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int C,
                      const float* coef);
 /* dw[K,R,S,C] (fp32) (+)= sum over pixels of dy x x.  splits > 1 needs a workspace of
@@ -283,11 +295,13 @@ int tch_attn_softmax_bwd(tch_context* ctx, int dtype, const void* probs, const v
 int tch_adamw_step(tch_context* ctx, float* param, const float* grad, float* exp_avg, float* exp_avg_sq,
                    void* shadow_bf16, int64_t n, double lr, double beta1, double beta2, double eps, double weight_decay,
                    int* step_dev, float* scalars_dev);
-/* out[b, t, :] = wte[ids[b, t], :] + wpe[t, :]; backward: dwte[id] += dy rows (fp32 atomics), dwpe (+)= sum over b. */
+/* out[b, t, :] = wte[ids[b, t], :] + wpe[t, :]; backward: dwte[id] += the dy rows of the positions that hold id,
+ * dwpe (+)= sum over b.  chain: 2 * B * T int32 of scratch; with it the rows that share a token are added up in
+ * position order by one thread (the same bits every run); NULL: fp32 atomics, order not fixed. */
 int tch_embedding_fwd(tch_context* ctx, int dtype, const int64_t* ids, const void* wte, const void* wpe, void* out, int B,
                       int T, int C, int vocab);
 int tch_embedding_bwd(tch_context* ctx, int dtype, const int64_t* ids, const void* dy, float* dwte, float* dwpe, int B,
-                      int T, int C, int vocab, int accumulate_wpe);
+                      int T, int C, int vocab, int accumulate_wpe, int32_t* chain);
 /* C[z](m, n) (+)= alpha * sum_k A[z](m, k) B[z](n, k), z = zo * batch_inner + zi; A(m, k) at
  * a + zo * a_bo + zi * a_bi + m * a_rs + k * a_cs (elements), B alike with n; C row-major with ldc.
  * One stride of each operand must be 1.  causal (square problems under a causal mask): 0 nothing is known;

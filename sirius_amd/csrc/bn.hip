@@ -518,6 +518,26 @@ unsigned apply_blocks(int64_t chunks) {
   return static_cast<unsigned>(b);
 }
 
+// Inference-mode BatchNorm as one scale and one shift per channel, from the running statistics:
+// y = (x - running_mean) / sqrt(running_var + eps) * gamma + beta = x * scale + shift.
+struct EvalCoefArgs {
+  const float* gamma;
+  const float* beta;
+  const float* mean;
+  const float* var;
+  float* coef;   // scale[C], then shift[C]
+  int C;
+  float eps;
+};
+
+__global__ void bn_eval_coef_kernel(EvalCoefArgs a) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= a.C) return;
+  const float scale = a.gamma[c] / sqrtf(a.var[c] + a.eps);
+  a.coef[c] = scale;
+  a.coef[a.C + c] = a.beta[c] - a.mean[c] * scale;
+}
+
 int check_common(int64_t rows, int C, int dtype) {
   TCH_CHECK_ARG(dtype == kBF16 || dtype == kF32, "bn: dtype must be f32(0) or bf16(1)");
   const int E = dtype == kBF16 ? 8 : 4;
@@ -599,6 +619,13 @@ int bn_apply_fwd(Context* ctx, int dtype, const void* x, void* y, const void* re
                                  "bn_apply_kernel<bf16,fwd>", apply_bytes, 1)
                         : launch(ctx, bn_apply_kernel<float, 0>, dim3(apply_blocks(a.chunks)), dim3(256), a,
                                  "bn_apply_kernel<f32,fwd>", apply_bytes, 1);
+}
+
+int bn_eval_coef(Context* ctx, const float* gamma, const float* beta, const float* running_mean,
+                 const float* running_var, float* coef, int C, float eps) {
+  TCH_CHECK_ARG(gamma && beta && running_mean && running_var && coef && C > 0, "bn_eval_coef: null tensor or no channels");
+  EvalCoefArgs a{gamma, beta, running_mean, running_var, coef, C, eps};
+  return launch(ctx, bn_eval_coef_kernel, dim3((C + 255) / 256), dim3(256), a, "bn_eval_coef_kernel", 24.0 * C, 1);
 }
 
 int bn_apply_bwd(Context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int C,

@@ -170,6 +170,8 @@ int tch_SyncStream(uint64_t hip_stream) { return sync_stream(hip_stream); }
 int tch_SyncAllStreams(void) { return sync_all_streams(); }
 int tch_QueryRejectCudaCalls(void) { return query_reject_calls() ? 1 : 0; }
 void tch_SetRejectCudaCalls(int reject) { set_reject_calls(reject != 0); }
+void tch_SuspendAllStreams(int sync_hw) { suspend_all_streams(sync_hw != 0); }
+void tch_ResumeAllStreams(int drop_commands) { resume_all_streams(drop_commands != 0); }
 void tch_SetXQueueShape(int queue_length, int sync_interval) { set_queue_shape(queue_length, sync_interval); }
 size_t tch_GetXQueueInFlight(uint64_t hip_stream) {
   auto q = queue_for_stream(hip_stream);
@@ -280,8 +282,8 @@ int tch_embedding_fwd(tch_context* ctx, int dtype, const int64_t* ids, const voi
 }
 
 int tch_embedding_bwd(tch_context* ctx, int dtype, const int64_t* ids, const void* dy, float* dwte, float* dwpe, int B,
-                      int T, int Cc, int vocab, int accumulate_wpe) {
-  return embedding_bwd(C(ctx), dtype, ids, dy, dwte, dwpe, B, T, Cc, vocab, accumulate_wpe);
+                      int T, int Cc, int vocab, int accumulate_wpe, int32_t* chain) {
+  return embedding_bwd(C(ctx), dtype, ids, dy, dwte, dwpe, B, T, Cc, vocab, accumulate_wpe, chain);
 }
 
 int tch_batched_gemm(tch_context* ctx, int dtype, const void* a, const void* b, void* c, int M, int N, int K,
@@ -353,6 +355,11 @@ int tch_conv2d_dgrad_bn(tch_context* ctx, int dtype, const void* dy, const void*
 int tch_bn_apply_fwd(tch_context* ctx, int dtype, const void* x, void* y, const void* residual, int relu, int64_t rows,
                      int Cc, const float* coef) {
   return bn_apply_fwd(C(ctx), dtype, x, y, residual, relu, rows, Cc, coef);
+}
+
+int tch_bn_eval_coef(tch_context* ctx, const float* gamma, const float* beta, const float* running_mean,
+                     const float* running_var, float* coef, int Cc, float eps) {
+  return bn_eval_coef(C(ctx), gamma, beta, running_mean, running_var, coef, Cc, eps);
 }
 
 int tch_bn_apply_bwd(tch_context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int Cc,

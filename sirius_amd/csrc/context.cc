@@ -47,6 +47,7 @@ LaunchQueue::~LaunchQueue() {
     stop_ = true;
   }
   cv_work_.notify_all();
+  cv_park_.notify_all();
   if (worker_.joinable()) worker_.join();
   for (auto& l : log_)
     if (l.event) (void)hipEventDestroy(l.event);
@@ -82,6 +83,28 @@ void LaunchQueue::chain(hipStream_t from, hipStream_t to) {
   // the event may be recorded again once the wait is enqueued (the wait holds its own reference to the
   // recorded state)
   if (ev) free_events_.push_back(ev);
+}
+
+void LaunchQueue::suspend(bool sync_hw) {
+  std::unique_lock<std::mutex> lock(mu_);
+  if (stop_) return;
+  if (suspended_ && parked_ && !sync_hw) return;
+  suspended_ = true;
+  parked_ = false;
+  park_sync_ = sync_hw;
+  cv_work_.notify_all();
+  cv_park_.wait(lock, [&] { return parked_ || stop_; });
+}
+
+void LaunchQueue::resume(bool drop_commands) {
+  {
+    std::lock_guard<std::mutex> lock(mu_);
+    if (drop_commands)
+      for (auto it = wait_.begin(); it != wait_.end();) it = (!it->is_sync && !it->is_dependency) ? wait_.erase(it) : it + 1;
+    suspended_ = false;
+    parked_ = false;
+  }
+  cv_work_.notify_all();
 }
 
 size_t LaunchQueue::clear() {
@@ -195,7 +218,24 @@ void LaunchQueue::worker_loop() {
     Item item;
     {
       std::unique_lock<std::mutex> lock(mu_);
-      cv_work_.wait(lock, [&] { return stop_ || !wait_.empty(); });
+      cv_work_.wait(lock, [&] { return stop_ || (suspended_ ? !parked_ : !wait_.empty()); });
+      if (suspended_ && !stop_) {
+        // park: nothing more goes to the hardware queue until resume()
+        const bool sync = park_sync_;
+        if (sync) {
+          lock.unlock();
+          hipError_t e = hipStreamSynchronize(launch_stream_);
+          if (e != hipSuccess) error_.store(static_cast<int>(e));
+          for (auto& l : log_)
+            if (l.event) free_events_.push_back(l.event);
+          log_.clear();
+          in_flight_.store(0);
+          lock.lock();
+        }
+        parked_ = true;
+        cv_park_.notify_all();
+        continue;
+      }
       if (wait_.empty()) {
         if (stop_) break;
         continue;
@@ -617,6 +657,24 @@ size_t queue_size_all_streams() {
   size_t total = 0;
   for (auto& kv : g_streams) total += kv.second->size();
   return total;
+}
+
+void suspend_all_streams(bool sync_hw) {
+  std::vector<std::shared_ptr<LaunchQueue>> qs;
+  {
+    std::lock_guard<std::mutex> lock(g_stream_mu);
+    for (auto& kv : g_streams) qs.push_back(kv.second);
+  }
+  for (auto& q : qs) q->suspend(sync_hw);
+}
+
+void resume_all_streams(bool drop_commands) {
+  std::vector<std::shared_ptr<LaunchQueue>> qs;
+  {
+    std::lock_guard<std::mutex> lock(g_stream_mu);
+    for (auto& kv : g_streams) qs.push_back(kv.second);
+  }
+  for (auto& q : qs) q->resume(drop_commands);
 }
 
 void set_reject_calls(bool reject) { g_reject.store(reject, std::memory_order_release); }

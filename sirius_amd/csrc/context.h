@@ -44,6 +44,12 @@ class LaunchQueue {
   // Wait until everything submitted before this call has finished on the GPU.
   // Returns 0 on success, a HIP error code otherwise.
   int synchronize();
+  // Stop handing launches to the hardware queue (what is already there runs on; with sync_hw the call
+  // returns once it has finished) / go on, optionally dropping what was queued meanwhile.  Another tenant's
+  // work submitted in between runs ahead of everything this queue still holds
+  // (third_party/xsched/preempt/xqueue/xqueue.cpp:80-137, Suspend / Resume).
+  void suspend(bool sync_hw);
+  void resume(bool drop_commands);
   // Launches still waiting in the software queue.
   size_t size();
   // Launches handed to the stream and not yet known to be complete.
@@ -82,6 +88,8 @@ class LaunchQueue {
   std::condition_variable cv_done_;
   std::deque<Item> wait_;
   bool stop_ = false;
+  bool suspended_ = false, parked_ = false, park_sync_ = false;
+  std::condition_variable cv_park_;
   uint64_t next_ticket_ = 1;
   uint64_t done_ticket_ = 0;
 
@@ -163,6 +171,8 @@ int sync_stream(uint64_t stream);
 int sync_all_streams();
 size_t queue_size(uint64_t stream);
 size_t queue_size_all_streams();
+void suspend_all_streams(bool sync_hw);
+void resume_all_streams(bool drop_commands);
 void set_reject_calls(bool reject);
 bool query_reject_calls();
 void set_queue_shape(int queue_length, int sync_interval);

@@ -90,6 +90,8 @@ int bn_bwd_finalize(Context* ctx, const float* partial, int row_blocks, int C, i
                     int accumulate);
 int bn_apply_fwd(Context* ctx, int dtype, const void* x, void* y, const void* residual, int relu, int64_t rows, int C,
                  const float* coef);
+int bn_eval_coef(Context* ctx, const float* gamma, const float* beta, const float* running_mean,
+                 const float* running_var, float* coef, int C, float eps);
 int bn_apply_bwd(Context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int C,
                  const float* coef);
 // the same from the sums a convolution epilogue left ([row_blocks][C][2]); g is already gated by the
@@ -117,7 +119,7 @@ int adamw_step(Context* ctx, float* param, const float* grad, float* exp_avg, fl
 int embedding_fwd(Context* ctx, int dtype, const int64_t* ids, const void* wte, const void* wpe, void* out, int B, int T,
                   int C, int vocab);
 int embedding_bwd(Context* ctx, int dtype, const int64_t* ids, const void* dy, float* dwte, float* dwpe, int B, int T,
-                  int C, int vocab, int accumulate_wpe);
+                  int C, int vocab, int accumulate_wpe, int32_t* chain);
 
 // swin_ops.hip
 int window_partition(Context* ctx, int dtype, const void* src, void* dst, const void* add, int B, int H, int W, int C,

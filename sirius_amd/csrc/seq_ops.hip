@@ -456,6 +456,8 @@ struct EmbedArgs {
   float* dwpe;         // [T][C] fp32, (+)= (backward)
   int64_t tokens;
   int T, C, cc, vocab, B, accumulate;
+  const int32_t* next_same;   // backward: chains of positions that hold the same token (nullptr: atomics)
+  const int32_t* first;
 };
 
 template <typename T>
@@ -481,37 +483,92 @@ __global__ __launch_bounds__(256) void embed_fwd_kernel(EmbedArgs p) {
   }
 }
 
-// dwpe[t] = sum over the batch (fixed order); dwte[id] += dy row (fp32 atomics: rows that share a
-// token meet in an order that may differ between runs)
+// Which positions hold the same token: next_same[i] = the next position after i with ids[i] (or -1),
+// first[i] = 1 when no earlier position holds it.  One thread per position, every thread walks all ids (they
+// sit in L2: 64 KB for 8192 tokens).
+struct ChainArgs {
+  const int64_t* ids;
+  int32_t* next_same;
+  int32_t* first;
+  int n;
+};
+
+__global__ __launch_bounds__(256) void embed_chain_kernel(ChainArgs p) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= p.n) return;
+  const int64_t id = p.ids[i];
+  int next = -1, first = 1;
+  for (int j = 0; j < i; ++j)
+    if (p.ids[j] == id) {
+      first = 0;
+      break;
+    }
+  for (int j = i + 1; j < p.n; ++j)
+    if (p.ids[j] == id) {
+      next = j;
+      break;
+    }
+  p.next_same[i] = next;
+  p.first[i] = first;
+}
+
+// dwpe[t] = sum over the batch (fixed order).  dwte[id] += sum of the dy rows of the positions that hold id,
+// added up in position order by the thread of the FIRST such position, which is the only writer of that row:
+// no atomics, the same bits every run.  (chain == nullptr: fp32 atomics per position instead; rows that share
+// a token then meet in an order that may differ between runs.)
 template <typename T>
 __global__ __launch_bounds__(256) void embed_bwd_kernel(EmbedArgs p) {
   constexpr int E = Elem<T>::kPerChunk;
+  const int32_t* next_same = p.next_same;
+  const int32_t* first = p.first;
   const int64_t per_batch = static_cast<int64_t>(p.T) * p.cc;
+  const int64_t total = p.tokens * p.cc;
   const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < per_batch; i += stride) {
-    const int t = static_cast<int>(i / p.cc);
-    const int c = static_cast<int>(i - static_cast<int64_t>(t) * p.cc);
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < total; i += stride) {
+    const int64_t tok = i / p.cc;
+    const int c = static_cast<int>(i - tok * p.cc);
+    if (i < per_batch) {   // position tok (< T) of every sequence: the position embedding's gradient
+      float acc[E];
+#pragma unroll
+      for (int e = 0; e < E; ++e) acc[e] = 0.f;
+      for (int b = 0; b < p.B; ++b) {
+        Chunk g;
+        g.u = static_cast<const uint4*>(p.dy)[(static_cast<int64_t>(b) * p.T + tok) * p.cc + c];
+        float v[E];
+        chunk_to_float<T>(g, v);
+#pragma unroll
+        for (int e = 0; e < E; ++e) acc[e] += v[e];
+      }
+      float* dst = p.dwpe + tok * p.C + c * E;
+#pragma unroll
+      for (int e = 0; e < E; ++e) dst[e] = p.accumulate ? dst[e] + acc[e] : acc[e];
+    }
+    int64_t id = p.ids[tok];
+    if (id < 0 || id >= p.vocab) id = 0;
+    float* row = p.dwte + id * p.C + c * E;
+    if (next_same == nullptr) {
+      Chunk g;
+      g.u = static_cast<const uint4*>(p.dy)[i];
+      float v[E];
+      chunk_to_float<T>(g, v);
+#pragma unroll
+      for (int e = 0; e < E; ++e) atomicAdd(row + e, v[e]);
+      continue;
+    }
+    if (!first[tok]) continue;
     float acc[E];
 #pragma unroll
     for (int e = 0; e < E; ++e) acc[e] = 0.f;
-    for (int b = 0; b < p.B; ++b) {
-      const int64_t tok = static_cast<int64_t>(b) * p.T + t;
+    for (int64_t j = tok; j >= 0; j = next_same[j]) {
       Chunk g;
-      g.u = static_cast<const uint4*>(p.dy)[tok * p.cc + c];
+      g.u = static_cast<const uint4*>(p.dy)[j * p.cc + c];
       float v[E];
       chunk_to_float<T>(g, v);
-      int64_t id = p.ids[tok];
-      if (id < 0 || id >= p.vocab) id = 0;
-      float* row = p.dwte + id * p.C + c * E;
 #pragma unroll
-      for (int e = 0; e < E; ++e) {
-        acc[e] += v[e];
-        atomicAdd(row + e, v[e]);
-      }
+      for (int e = 0; e < E; ++e) acc[e] += v[e];
     }
-    float* dst = p.dwpe + static_cast<int64_t>(t) * p.C + c * E;
 #pragma unroll
-    for (int e = 0; e < E; ++e) dst[e] = p.accumulate ? dst[e] + acc[e] : acc[e];
+    for (int e = 0; e < E; ++e) row[e] += acc[e];
   }
 }
 
@@ -676,7 +733,7 @@ int embedding_fwd(Context* ctx, int dtype, const int64_t* ids, const void* wte, 
   if (int rc = check_rows("embedding_fwd", dtype, static_cast<int64_t>(B) * T, C)) return rc;
   TCH_CHECK_ARG(ids && wte && wpe && out && vocab > 0, "embedding_fwd: null tensor");
   const int E = dtype == kBF16 ? 8 : 4;
-  EmbedArgs a{ids, wte, wpe, out, nullptr, nullptr, nullptr, static_cast<int64_t>(B) * T, T, C, C / E, vocab, B, 0};
+  EmbedArgs a{ids, wte, wpe, out, nullptr, nullptr, nullptr, static_cast<int64_t>(B) * T, T, C, C / E, vocab, B, 0, nullptr, nullptr};
   const double bytes = static_cast<double>(a.tokens) * C * (dtype == kBF16 ? 6.0 : 12.0);
   const dim3 grid(flat_blocks(a.tokens * a.cc));
   return dtype == kBF16 ? launch(ctx, embed_fwd_kernel<bf16>, grid, dim3(256), a, "embed_fwd_kernel<bf16>", bytes, 1)
@@ -684,14 +741,20 @@ int embedding_fwd(Context* ctx, int dtype, const int64_t* ids, const void* wte, 
 }
 
 int embedding_bwd(Context* ctx, int dtype, const int64_t* ids, const void* dy, float* dwte, float* dwpe, int B, int T,
-                  int C, int vocab, int accumulate_wpe) {
+                  int C, int vocab, int accumulate_wpe, int32_t* chain) {
   if (int rc = check_rows("embedding_bwd", dtype, static_cast<int64_t>(B) * T, C)) return rc;
   TCH_CHECK_ARG(ids && dy && dwte && dwpe && vocab > 0, "embedding_bwd: null tensor");
   const int E = dtype == kBF16 ? 8 : 4;
+  const int n = B * T;
   EmbedArgs a{ids, nullptr, nullptr, nullptr, dy, dwte, dwpe, static_cast<int64_t>(B) * T, T, C, C / E, vocab, B,
-              accumulate_wpe};
+              accumulate_wpe, chain, chain ? chain + n : nullptr};
+  if (chain) {
+    ChainArgs ca{ids, chain, chain + n, n};
+    if (int rc = launch(ctx, embed_chain_kernel, dim3((n + 255) / 256), dim3(256), ca, "embed_chain_kernel", 16.0 * n, 1))
+      return rc;
+  }
   const double bytes = static_cast<double>(a.tokens) * C * (dtype == kBF16 ? 2.0 : 4.0) + 8.0 * a.tokens * C;
-  const dim3 grid(flat_blocks(static_cast<int64_t>(T) * a.cc));
+  const dim3 grid(flat_blocks(a.tokens * a.cc));
   return dtype == kBF16 ? launch(ctx, embed_bwd_kernel<bf16>, grid, dim3(256), a, "embed_bwd_kernel<bf16>", bytes, 1)
                         : launch(ctx, embed_bwd_kernel<float>, grid, dim3(256), a, "embed_bwd_kernel<f32>", bytes, 1);
 }

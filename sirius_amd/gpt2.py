@@ -365,7 +365,7 @@ class GPT2Engine(EngineBase):
                 mark("bwd", f"h.{i}")
             # tied weights: the scattered embedding gradient lands on top of the head's weight gradient
             ops.embedding_bwd(ctx, plan.ids, g.view(B, T, C), self._view(self.grads, "transformer.wte.weight").view(Vp, C),
-                              self._view(self.grads, "transformer.wpe.weight"))
+                              self._view(self.grads, "transformer.wpe.weight"), chain=act(2 * B * T, dtype=torch.int32))
         finally:
             ctx.end_record()
         plan.prog, plan.marks, plan.keep, plan.logits = prog, marks, keep, logits

@@ -277,6 +277,14 @@ def bn_apply_fwd(ctx, x, y, coef, residual=None, relu=True):
                                  _p(coef)), "tch_bn_apply_fwd")
 
 
+def bn_eval_coef(ctx, gamma, beta, running_mean, running_var, coef, eps=1e-5):
+    """coef [2, C] fp32 = (scale, shift) of inference-mode BatchNorm from the running statistics."""
+    C = gamma.numel()
+    assert coef.dtype == torch.float32 and coef.numel() >= 2 * C
+    check(lib().tch_bn_eval_coef(ctx.handle, _p(gamma), _p(beta), _p(running_mean), _p(running_var), _p(coef), C,
+                                 float(eps)), "tch_bn_eval_coef")
+
+
 def bn_apply_bwd(ctx, g, x, dx, coef):
     C = x.shape[-1]
     assert g.shape == x.shape == dx.shape and g.dtype == x.dtype == dx.dtype and coef.numel() >= 3 * C
@@ -613,12 +621,15 @@ def embedding_fwd(ctx, ids, wte, wpe, out):
           "tch_embedding_fwd")
 
 
-def embedding_bwd(ctx, ids, dy, dwte, dwpe, accumulate_wpe=False):
+def embedding_bwd(ctx, ids, dy, dwte, dwpe, accumulate_wpe=False, chain=None):
+    """chain: int32 scratch of 2 * B * T elements; with it the result is the same bit for bit every run (rows that
+    share a token are added in position order), without it fp32 atomics decide the order."""
     B, T = ids.shape
     vocab, C = dwte.shape
     assert tuple(dy.shape) == (B, T, C) and dwte.dtype == dwpe.dtype == torch.float32 and dwpe.shape[0] >= T
+    assert chain is None or (chain.dtype == torch.int32 and chain.numel() >= 2 * B * T)
     check(lib().tch_embedding_bwd(ctx.handle, dtype_code(dy), _p(ids), _p(dy), _p(dwte), _p(dwpe), B, T, C, vocab,
-                                  int(accumulate_wpe)), "tch_embedding_bwd")
+                                  int(accumulate_wpe), _p(chain)), "tch_embedding_bwd")
 
 
 def batched_gemm(ctx, a, b, c, M, N, K, a_strides, b_strides, ldc, batch=(1, 1), a_batch=(0, 0), b_batch=(0, 0),

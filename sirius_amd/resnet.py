@@ -651,6 +651,84 @@ class ResNetEngine(EngineBase):
         p = self.plan(batch, loss_scale)
         return p, self._run_plan(p)
 
+    # ------------------------------------------------------------------ inference (model.eval())
+    def prepare_eval(self):
+        """Turn every BatchNorm into one scale and one shift per channel from its running statistics (what
+        model.eval() makes of it).  Run again whenever weights or statistics changed."""
+        if getattr(self, "_eval_coef", None) is None:
+            self._eval_coef = self._alloc((2 * self.running_mean.numel(),), torch.float32)
+        nbn = self.running_mean.numel()
+        for name, (o, c) in self._bn_off.items():
+            # (scale, shift) of a BatchNorm sit next to each other: coef[2o : 2o + 2c]
+            ops.bn_eval_coef(self.ctx, self._view(self.params, name + ".weight"), self._view(self.params, name + ".bias"),
+                             self.running_mean[o:o + c], self.running_var[o:o + c], self._eval_coef[2 * o:2 * o + 2 * c],
+                             eps=self.bn_eps)
+        assert 2 * nbn == self._eval_coef.numel()
+
+    def _build_eval_plan(self, B):
+        """Forward only, BatchNorm from the running statistics, nothing kept for a backward: the program of
+        one inference request (the batch-1 ResNet-152 requests that share the GPU with training)."""
+        T, ctx, S = self.dtype, self.ctx, self.image_size
+        plan = _Block()
+        keep = []
+
+        def act(*shape, dtype=T):
+            t = self._alloc(tuple(shape), dtype)
+            keep.append(t)
+            return t
+
+        def conv_bn(c, name, x, residual=None, relu=True):
+            Ho, Wo = ops.conv_out_hw(x.shape[1], x.shape[2], c.k, c.k, c.stride, c.pad)
+            z, y = act(B, Ho, Wo, c.cout), act(B, Ho, Wo, c.cout)
+            ops.conv2d_fwd(ctx, x, self._w(c.name + ".weight"), z, c.stride, c.pad, c_logical=c.cin)
+            o, ch = self._bn_off[name]
+            ops.bn_apply_fwd(ctx, z, y, self._eval_coef[2 * o:2 * o + 2 * ch], residual=residual, relu=relu)
+            return y
+
+        plan.x_in = act(B, 3, S, S, dtype=torch.float32)
+        prog = ops.Program()
+        ctx.begin_record(prog)
+        try:
+            x0 = act(B, S, S, STEM_CIN_PAD)
+            ops.nchw_to_nhwc_pad(ctx, plan.x_in, x0)
+            a0 = conv_bn(self.stem, "bn1", x0)
+            Hp, Wp = ops.conv_out_hw(a0.shape[1], a0.shape[2], 3, 3, 2, 1)
+            x = act(B, Hp, Wp, self.width)
+            idx = act(B, Hp, Wp, self.width, dtype=torch.int32)
+            ops.maxpool_fwd(ctx, a0, x, idx, 3, 2, 1)
+            for blk in self.blocks:
+                pre = blk.prefix
+                a1 = conv_bn(blk.c1, pre + ".bn1", x)
+                a2 = conv_bn(blk.c2, pre + ".bn2", a1)
+                idn = conv_bn(blk.cd, pre + ".downsample.1", x, relu=False) if blk.cd is not None else x
+                x = conv_bn(blk.c3, pre + ".bn3", a2, residual=idn, relu=True)
+            pooled = act(B, self.feat)
+            ops.avgpool_fwd(ctx, x, pooled)
+            plan.logits = act(B, self.num_classes, dtype=torch.float32)
+            ops.conv2d_fwd(ctx, pooled.view(B, 1, 1, self.feat), self._w("fc.weight"),
+                           plan.logits.view(B, 1, 1, self.num_classes), 1, 0, bias=self._view(self.params, "fc.bias"))
+        finally:
+            ctx.end_record()
+        plan.prog, plan.keep, plan.batch = prog, keep, B
+        plan.bytes = sum(t.numel() * t.element_size() for t in keep)
+        return plan
+
+    def eval_plan(self, batch):
+        plans = self.__dict__.setdefault("_eval_plans", {})
+        if batch not in plans:
+            if getattr(self, "_eval_coef", None) is None:
+                self.prepare_eval()
+            plans[batch] = self._build_eval_plan(batch)
+        return plans[batch]
+
+    def forward_eval(self, x):
+        """x [B,3,S,S] fp32 on the GPU -> the plan whose `logits` [B, classes] (fp32) the launches fill.  The
+        caller synchronises (ctx.synchronize()) before reading them."""
+        p = self.eval_plan(x.shape[0])
+        p.x_in.copy_(x, non_blocking=True)
+        self.ctx.run(p.prog)
+        return p
+
     def _record_optimizer(self, grads):
         ops.sgd_momentum_step(self.ctx, self.params, grads, self.momentum_buf, self.lr, self.momentum,
                               self.weight_decay, shadow=self.shadow)

@@ -63,6 +63,15 @@ def kill_batch(stream=None):
     return num_cmds
 
 
+def suspend_all_streams(sync_hw: bool = False):
+    """Training's queues stop handing launches to the hardware until resume_all_streams()."""
+    _C.lib().tch_SuspendAllStreams(int(sync_hw))
+
+
+def resume_all_streams(drop_commands: bool = False):
+    _C.lib().tch_ResumeAllStreams(int(drop_commands))
+
+
 def set_reject_cuda_calls(reject: bool):
     _C.SetRejectCudaCalls(reject)
 

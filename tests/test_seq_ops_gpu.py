@@ -193,6 +193,20 @@ def test_embedding(ctx, dtype, B, T, C, vocab):
     close(dwte, dwte_ref, torch.float32, "dwte", rtol=1e-5)
     close(dwpe[:T], dwpe_ref[:T], torch.float32, "dwpe", rtol=1e-5)
     assert torch.all(dwpe[T:] == 9.0), "positions past the sequence are not touched"
+    # with the chain scratch: the same values, on top of what the rows already hold (the tied head's gradient), and
+    # the same bits on every run -- one thread adds the rows of a repeated token in position order
+    base = rnd((vocab, C), torch.float32, g)
+    chain = torch.full((2 * B * T,), -7, dtype=torch.int32, device="cuda")
+    runs = []
+    for _ in range(3):
+        d = base.clone().cuda()
+        dp = torch.zeros((T + 3, C), device="cuda")
+        ops.embedding_bwd(ctx, ids.cuda(), dy.cuda(), d, dp, chain=chain)
+        torch.cuda.synchronize()
+        runs.append((d.clone(), dp.clone()))
+    close(runs[0][0] - base.cuda(), dwte_ref, torch.float32, "dwte (chained)", rtol=1e-4)
+    close(runs[0][1][:T], dwpe_ref[:T], torch.float32, "dwpe (chained)", rtol=1e-5)
+    assert all(torch.equal(runs[0][0], r[0]) and torch.equal(runs[0][1], r[1]) for r in runs[1:])
 
 
 def _attention_layouts(B, H, T, D):
