@@ -25,6 +25,10 @@ METRIC = "ResNet-152 bf16 bs64 train images/sec on 1 GPU; conv MFMA util %"
 # HBM bytes per launch of the kernels that can top the step, from two rocprofv3 --pmc runs of this file
 # (FETCH_SIZE and WRITE_SIZE, KiB per dispatch, scaled by what the same counters read for the --calibrate
 # copy of known size: factors 2.000 and 1.000); the summary is profiles/resnet152_bf16_bs64_step_kernel_stats_and_traffic.txt
+# The handover measurement: a pool of nearly the whole part in 128 MB pages (the reference's 32 MB page costs one
+# driver call per page on the way out: 9 GB take 68 ms there, 18 ms in 128 MB pages).
+HANDOVER_POOL_GB = 256
+HANDOVER_PAGE_MB = 128
 MEASURED_TRAFFIC_MIB = {
     "wgrad_kernel<bf16,128x128>": 31.79 + 13.77,
     "igemm2_kernel<bf16,dgrad,128x128,2buf>": 67.94 + 32.72,
@@ -35,6 +39,19 @@ MEASURED_TRAFFIC_MIB = {
     "bn_apply_kernel<bf16,bwd>": 72.04 + 34.61,
     "bn_apply_kernel<bf16,fwd>": 54.69 + 36.09,
 }
+
+
+def cpu_model():
+    """The host processor's name as the kernel reports it."""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    import platform
+    return platform.processor() or platform.machine()
 
 
 def cpu_baseline(batch, timed_steps):
@@ -49,8 +66,8 @@ def cpu_baseline(batch, timed_steps):
     t0 = time.perf_counter()
     R.train_steps(model, x, y, timed_steps)
     dt = time.perf_counter() - t0
-    return {"value": batch * timed_steps / dt, "unit": "images/s", "cores": cores, "kind": "port",
-            "sample": f"ResNet-152 fp32 batch {batch} @224, torch CPU oracle step, 1 warm-up + {timed_steps} timed steps"}
+    return {"value": batch * timed_steps / dt, "unit": "images/s", "cores": cores, "cpu_model": cpu_model(),
+            "kind": "port", "sample": f"ResNet-152 fp32 batch {batch} @224, torch CPU oracle step, 1 warm-up + {timed_steps} timed steps"}
 
 
 def handover(batch):
@@ -69,7 +86,8 @@ def handover(batch):
     tmp = tempfile.mkdtemp(prefix="tch_bench_")
     env = {"COLTRAIN_MODE": "colocate-l1", "COLTRAIN_HOOK_MODE": "xsched-sync", "COLTRAIN_USE_XSCHED": "1",
            "COLTRAIN_HAS_INFER_SERVER": "1", "COLTRAIN_USE_SHARED_TENSOR": "1",
-           "COLTRAIN_SHARED_TENSOR_POOL_GB": "48", "COLTRAIN_PROFILE_LOG_PATH": os.path.join(tmp, "train-profile.csv"),
+           "COLTRAIN_SHARED_TENSOR_POOL_GB": str(HANDOVER_POOL_GB), "COLTRAIN_POOL_PAGE_MB": str(HANDOVER_PAGE_MB),
+           "COLTRAIN_PROFILE_LOG_PATH": os.path.join(tmp, "train-profile.csv"),
            "SIRIUS_PORT": str(18000 + os.getpid() % 1000)}
     os.environ.update(env)
     peer = script.PeerScript({3: ("l1", 16), 14: ("exit", batch)}, delay_ms=8.0)
@@ -95,7 +113,48 @@ def handover(batch):
         "killed_batches": stat.killed_batch,
         "finished_samples": stat.finished_sample,
         "bound_ms": 50.0,
+        "pool_gb": HANDOVER_POOL_GB,
+        "page_mb": HANDOVER_PAGE_MB,
+        "unmapping": "eager: every page handed back is unmapped from training's address range before the reply",
+        "stale_pages_after": out["ctrl"].last_adjust.get("stale_pages_after"),
     }
+    del out
+    torch_col.reset_for_tests()
+    torch_col.torch_col_shutdown()
+    return res
+
+
+def through_plugin(batch, batches=30, skip=8):
+    """The same step through the plugin path, as the reference's train script drives it: colocate-l1 mode with the
+    allocator hook and the launch queue, micro-batches copied from pinned host memory (the next one ahead of
+    time on a copy stream), forward + backward + accumulate + optimizer, one synchronisation per micro-batch,
+    no inference peer.  Images per second over the micro-batch durations the profile records (the first
+    `skip` left out)."""
+    import contextlib
+    import csv
+    import tempfile
+
+    import torch
+    from sirius_amd import torch_col
+    from sirius_amd.train import resnet152 as script
+
+    tmp = tempfile.mkdtemp(prefix="tch_bench_")
+    os.environ.update({"COLTRAIN_MODE": "colocate-l1", "COLTRAIN_HOOK_MODE": "xsched-sync", "COLTRAIN_USE_XSCHED": "1",
+                       "COLTRAIN_HAS_INFER_SERVER": "0", "COLTRAIN_USE_SHARED_TENSOR": "1",
+                       "COLTRAIN_SHARED_TENSOR_POOL_GB": "48", "COLTRAIN_POOL_PAGE_MB": "32",
+                       "COLTRAIN_PROFILE_LOG_PATH": os.path.join(tmp, "train-profile.csv"),
+                       "SIRIUS_PORT": str(19000 + os.getpid() % 1000)})
+    with contextlib.redirect_stdout(sys.stderr):
+        out = script.train(1, batch, dataset_size=batch * batches, dtype=torch.bfloat16, num_distinct_samples=batch * 2)
+    rows = [r for r in csv.DictReader(open(out["profile"])) if r["name"].startswith("batch_0")]
+    dur = [float(r["duration"]) for r in rows][skip:]
+    t_first, t_last = float(rows[skip]["timestamp"]), float(rows[-1]["timestamp"]) + float(rows[-1]["duration"])
+    res = {"images_per_s": batch * len(dur) / ((t_last - t_first) * 1e-3), "micro_batches_timed": len(dur),
+           "ms_per_micro_batch": sum(dur) / len(dur),
+           "ms_per_micro_batch_wall": (t_last - t_first) / len(dur),
+           "note": "train script + Trainer + dataset: H2D copy of the next micro-batch overlapped on a copy stream, "
+                   "gradient accumulation, one synchronisation per micro-batch; wall = first timed micro-batch's "
+                   "begin to the last one's end, dataset and bookkeeping between micro-batches included"}
     del out
     torch_col.reset_for_tests()
     torch_col.torch_col_shutdown()
@@ -142,6 +201,81 @@ def gpt2_step(batch=8, seq_len=1024, warmup=2, steps=5):
     return res
 
 
+def interleaving(batch=8, seq_len=1024, rate_per_s=50.0, train_s=3.0):
+    """BASELINE configs[4] whole: the GPT-2 small training step (bf16, ids [8, 1024], AdamW) on a stream that is
+    registered with the launch queue, while batch-1 ResNet-152 forward-only requests arrive as a seeded Poisson
+    process at `rate_per_s` and suspend that queue for as long as each of them runs.  Reports the request
+    latencies (arrival to logits) and what the requests cost training: steps per second alone against steps
+    per second beside the requests, both over about `train_s` seconds of steps."""
+    import torch
+    from sirius_amd.gpt2 import GPT2Engine
+    from sirius_amd.resnet import ResNetEngine
+    from sirius_amd.serve import ColocatedInference, poisson_arrivals
+    from sirius_amd.torch_col import xsched
+    train_stream, infer_stream = torch.cuda.Stream(), torch.cuda.Stream()
+    xsched.register_stream(train_stream, False)
+    server = None
+    try:
+        eng = GPT2Engine(seq_len=seq_len, dtype=torch.bfloat16, optimizer="adamw", stream=train_stream)
+        eng.init_normal(0)
+        g = torch.Generator(device="cuda")
+        g.manual_seed(2)
+        ids = torch.randint(0, eng.vocab, (batch, seq_len), device="cuda", generator=g)
+
+        def run(seconds):
+            n = 0
+            with torch.cuda.stream(train_stream):
+                t0 = time.perf_counter()
+                while time.perf_counter() - t0 < seconds:
+                    eng.forward_backward(ids)
+                    eng.optimizer_step()
+                    n += 1
+                    if n % 8 == 0:
+                        eng.synchronize()      # keep the host no more than a few steps ahead of the device
+                eng.synchronize()
+                return n, time.perf_counter() - t0
+
+        run(0.2)
+        n_alone, s_alone = run(train_s)
+        infer = ResNetEngine(dtype=torch.bfloat16, stream=infer_stream)
+        infer.init_kaiming(seed=9)
+        arrivals = poisson_arrivals(rate_per_s, int(rate_per_s * train_s * 4) + 16, seed=7)
+        server = ColocatedInference(infer, arrivals, batch=1, preempt=True)
+        server.warm_up()
+        idle = []
+        for _ in range(20):                      # the request alone on the chip
+            t0 = time.perf_counter()
+            server._serve_one(t0)
+            idle.append(server.latencies_ms.pop())
+            server.service_ms.pop(), server.started_late_ms.pop()
+        server.start()
+        n_mixed, s_mixed = run(train_s)
+        served = len(server.latencies_ms)
+        server.stop()
+        lat = server.summary()
+        res = {
+            "workload": f"GPT-2 small training, bf16, ids [{batch}, {seq_len}], AdamW, beside batch-1 ResNet-152 bf16 "
+                        f"forward-only requests, Poisson {rate_per_s:g}/s (seed 7), each suspending training's launch queue",
+            "requests_served": served,
+            "infer_p50_ms": lat.get("p50_ms"), "infer_p99_ms": lat.get("p99_ms"), "infer_max_ms": lat.get("max_ms"),
+            "infer_alone_p50_ms": sorted(idle)[len(idle) // 2],
+            "train_ms_per_step_alone": s_alone / n_alone * 1e3,
+            "train_ms_per_step_interleaved": s_mixed / n_mixed * 1e3,
+            "train_slowdown": (s_mixed / n_mixed) / (s_alone / n_alone),
+            "tokens_per_s_interleaved": batch * seq_len * n_mixed / s_mixed,
+        }
+        del eng, infer
+        return res
+    finally:
+        if server is not None and server._thread is not None and server._thread.is_alive():
+            server._stop.set()
+            server._thread.join(10)
+        xsched.resume_all_streams()
+        torch.cuda.synchronize()
+        xsched.unregister_stream(train_stream)
+        torch.cuda.empty_cache()
+
+
 def swin_b_step(batch=32, warmup=2, steps=5):
     """BASELINE configs[3]: Swin-B (87.77 M parameters), bf16 compute with fp32 master weights, images
     [32, 3, 224, 224] N(0,1), AdamW(lr 1e-3, wd 0.05), stochastic depth 0.  Reported beside the headline figure."""
@@ -185,8 +319,10 @@ def swin_b_step(batch=32, warmup=2, steps=5):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--no-handover", action="store_true", help="skip the 64 -> 16 -> 64 handover measurement")
+    ap.add_argument("--no-plugin", action="store_true", help="skip the run of the same step through the train script")
     ap.add_argument("--no-gpt2", action="store_true", help="skip the GPT-2 step measurement")
     ap.add_argument("--only-gpt2", action="store_true", help="run the GPT-2 step measurement alone (for profiling it)")
+    ap.add_argument("--no-interleave", action="store_true", help="skip GPT-2 training beside Poisson ResNet-152 requests")
     ap.add_argument("--no-swin", action="store_true", help="skip the Swin-B step measurement")
     ap.add_argument("--only-swin", action="store_true", help="run the Swin-B step measurement alone (for profiling it)")
     ap.add_argument("--no-autotune", action="store_true", help="keep the library's tiling heuristic")
@@ -322,6 +458,11 @@ def main():
         out["cpu_baseline"] = None
     del eng, plan, x, y
     torch.cuda.empty_cache()
+    if not args.no_plugin:
+        try:
+            out["value_through_plugin"] = through_plugin(B)
+        except Exception as e:
+            out["value_through_plugin"] = {"error": repr(e)}
     if not args.no_handover:
         try:
             out["handover"] = handover(B)
@@ -332,6 +473,11 @@ def main():
             out["gpt2"] = gpt2_step()
         except Exception as e:
             out["gpt2"] = {"error": repr(e)}
+    if not args.no_gpt2 and not args.no_interleave:
+        try:
+            out["gpt2"]["interleaving"] = interleaving()
+        except Exception as e:
+            out["gpt2"]["interleaving"] = {"error": repr(e)}
     if not args.no_swin:
         try:
             out["swin_b"] = swin_b_step()

@@ -101,7 +101,9 @@ void tch_SetRejectCudaCalls(int reject);            /* xsched_ctrl.cc:196-198 */
  * (third_party/xsched/preempt/xqueue/xqueue.cpp:80-137 Suspend / Resume). */
 void tch_SuspendAllStreams(int sync_hw);
 void tch_ResumeAllStreams(int drop_commands);
-/* queue length / sync interval used by later tch_RegisterStream calls (reference: 16, 8) */
+/* queue length / sync interval used by later tch_RegisterStream calls (reference: 16, 8; default here: 16, 4 --
+ * the length bounds what a preempting tenant waits behind, the interval only sets how often the worker can
+ * notice that launches finished) */
 void tch_SetXQueueShape(int queue_length, int sync_interval);
 size_t tch_GetXQueueInFlight(uint64_t hip_stream);
 

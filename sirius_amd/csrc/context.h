@@ -33,9 +33,10 @@ class LaunchQueue {
   LaunchQueue(const LaunchQueue&) = delete;
   LaunchQueue& operator=(const LaunchQueue&) = delete;
 
-  // `on` (optional): the stream to launch on instead of the registered one (a stream restricted to a
-  // share of the compute units); the worker chains the streams with events whenever `on` changes,
-  // so program order holds across them.
+  // `on` (optional): the stream to launch on instead of the registered one (the second lane of a program, or a
+  // stream restricted to a share of the compute units).  Launches on different streams are ordered only by
+  // the dependencies the caller queues between them, exactly as when the caller launches directly; the bound
+  // on launches in flight holds over all streams together.
   void submit(const LaunchRecord& rec, hipStream_t on = nullptr);
   // Queued in order with the launches: everything given to `to` afterwards waits for what `from` holds now.
   void submit_dependency(hipStream_t from, hipStream_t to);
@@ -69,16 +70,22 @@ class LaunchQueue {
   };
   struct Logged {
     uint64_t idx;
-    hipEvent_t event;  // nullptr unless this command carries a sync point
+    hipEvent_t event;    // nullptr unless this command carries a sync point (of its own stream)
+    hipStream_t stream;  // where it was launched
+  };
+  struct StreamState {
+    hipStream_t stream;
+    uint64_t since_event;  // launches on the stream since its last sync point
   };
   void worker_loop();
   void launch_one(const LaunchRecord& rec, hipStream_t on);
   void chain(hipStream_t from, hipStream_t to);
   void drain_log_until(size_t keep);
+  void sync_everything();
+  StreamState& state_of(hipStream_t s);
   hipEvent_t take_event();
 
   hipStream_t stream_;
-  hipStream_t launch_stream_;  // worker-private: where the last launch went
   const size_t queue_length_;
   const uint64_t sync_interval_;
   int device_ = 0;
@@ -96,8 +103,8 @@ class LaunchQueue {
   // worker-private
   std::deque<Logged> log_;
   std::vector<hipEvent_t> free_events_;
+  std::vector<StreamState> streams_;  // every stream a launch went to since the last full synchronisation
   uint64_t next_idx_ = 0;
-  uint64_t last_sync_idx_ = 0;
 
   std::atomic<size_t> in_flight_{0};
   std::atomic<int> error_{0};

@@ -484,32 +484,54 @@ __global__ __launch_bounds__(256) void embed_fwd_kernel(EmbedArgs p) {
 }
 
 // Which positions hold the same token: next_same[i] = the next position after i with ids[i] (or -1),
-// first[i] = 1 when no earlier position holds it.  One thread per position, every thread walks all ids (they
-// sit in L2: 64 KB for 8192 tokens).
+// first[i] = 1 when no earlier position holds it.  A workgroup owns 64 positions (one per lane); the ids pass
+// through LDS in chunks of 4096 and each of the four wavefronts compares its quarter of a chunk against the
+// lane's id (every lane of a wavefront reads the same LDS word: a broadcast), without branches; the four
+// partial answers meet in LDS.  Ids outside the table count as 0, as in the kernels that use them.
 struct ChainArgs {
   const int64_t* ids;
   int32_t* next_same;
   int32_t* first;
-  int n;
+  int n, vocab;
 };
 
 __global__ __launch_bounds__(256) void embed_chain_kernel(ChainArgs p) {
-  const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i >= p.n) return;
-  const int64_t id = p.ids[i];
-  int next = -1, first = 1;
-  for (int j = 0; j < i; ++j)
-    if (p.ids[j] == id) {
-      first = 0;
-      break;
+  constexpr int kChunk = 4096;
+  __shared__ int32_t s_ids[kChunk];
+  __shared__ int32_t s_next[4][64];
+  __shared__ int32_t s_prev[4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int i = blockIdx.x * 64 + lane;
+  auto clamp_id = [&](int64_t v) { return (v < 0 || v >= p.vocab) ? 0 : static_cast<int32_t>(v); };
+  const int32_t id = i < p.n ? clamp_id(p.ids[i]) : -1;
+  int next = 0x7fffffff, prev = 0;
+  for (int base = 0; base < p.n; base += kChunk) {
+    const int len = min(kChunk, p.n - base);
+    __syncthreads();
+    for (int j = threadIdx.x; j < kChunk; j += 256) s_ids[j] = j < len ? clamp_id(p.ids[base + j]) : -2;
+    __syncthreads();
+    const int q0 = wave * (kChunk / 4);
+    for (int j = q0; j < q0 + kChunk / 4; j += 4) {
+      const int4 v = *reinterpret_cast<const int4*>(&s_ids[j]);
+      const int g = base + j;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int32_t w = e == 0 ? v.x : e == 1 ? v.y : e == 2 ? v.z : v.w;
+        const bool same = w == id;
+        prev |= (same && g + e < i) ? 1 : 0;
+        next = (same && g + e > i) ? min(next, g + e) : next;
+      }
     }
-  for (int j = i + 1; j < p.n; ++j)
-    if (p.ids[j] == id) {
-      next = j;
-      break;
-    }
-  p.next_same[i] = next;
-  p.first[i] = first;
+  }
+  s_next[wave][lane] = next;
+  s_prev[wave][lane] = prev;
+  __syncthreads();
+  if (wave == 0 && i < p.n) {
+    const int nx = min(min(s_next[0][lane], s_next[1][lane]), min(s_next[2][lane], s_next[3][lane]));
+    const int pv = s_prev[0][lane] | s_prev[1][lane] | s_prev[2][lane] | s_prev[3][lane];
+    p.next_same[i] = nx == 0x7fffffff ? -1 : nx;
+    p.first[i] = pv ? 0 : 1;
+  }
 }
 
 // dwpe[t] = sum over the batch (fixed order).  dwte[id] += sum of the dy rows of the positions that hold id,
@@ -749,8 +771,8 @@ int embedding_bwd(Context* ctx, int dtype, const int64_t* ids, const void* dy, f
   EmbedArgs a{ids, nullptr, nullptr, nullptr, dy, dwte, dwpe, static_cast<int64_t>(B) * T, T, C, C / E, vocab, B,
               accumulate_wpe, chain, chain ? chain + n : nullptr};
   if (chain) {
-    ChainArgs ca{ids, chain, chain + n, n};
-    if (int rc = launch(ctx, embed_chain_kernel, dim3((n + 255) / 256), dim3(256), ca, "embed_chain_kernel", 16.0 * n, 1))
+    ChainArgs ca{ids, chain, chain + n, n, vocab};
+    if (int rc = launch(ctx, embed_chain_kernel, dim3((n + 63) / 64), dim3(256), ca, "embed_chain_kernel", 16.0 * n, 1))
       return rc;
   }
   const double bytes = static_cast<double>(a.tokens) * C * (dtype == kBF16 ? 2.0 : 4.0) + 8.0 * a.tokens * C;

@@ -223,6 +223,9 @@ def _give_memory_back():
     the pool (unmapped from this process unless the pool runs in lazy mode).  Returns
     (activation bytes released, pool bytes returned, ms for the first, ms for the second)."""
     t0 = time.time()
+    from .dynamic_batch import DynamicBatchDataset      # the micro-batch copied ahead of time is memory too
+    if DynamicBatchDataset._dynamic_batch_dataset is not None:
+        DynamicBatchDataset._dynamic_batch_dataset._samples.drop_prefetched()
     released = _C.release_interm_memory()
     t1 = time.time()
     returned = MemoryPool.empty_cache()

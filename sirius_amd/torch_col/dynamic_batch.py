@@ -17,6 +17,7 @@ from __future__ import annotations
 
 import contextlib
 import dataclasses
+import os
 import sys
 import time
 from enum import Enum, IntEnum
@@ -104,24 +105,70 @@ class _HostSamples:
     def __init__(self, tensors: dict, pinned: bool):
         self.tensors = {k: (t.pin_memory() if pinned else t) for k, t in tensors.items()}
         self.resident = len(next(iter(self.tensors.values())))
+        self.pinned = pinned
+        self.prefetch = os.environ.get('COLTRAIN_PREFETCH_BATCH', '1') != '0'
+        self._copy_stream = None
+        self._ahead = None      # (first row, rows, device tensors, copy-done event) of the guessed next batch
 
     def rows_of(self, range_vec: RangeVec) -> torch.Tensor:
         return torch.cat([torch.arange(lo, hi) for lo, hi in range_vec]) % self.resident if range_vec \
             else torch.empty(0, dtype=torch.long)
+
+    def _copy_run(self, first: int, n: int, device) -> dict:
+        out = {}
+        for key, src in self.tensors.items():
+            dst = torch.empty((n, *src.shape[1:]), dtype=src.dtype, device=device)
+            dst.copy_(src[first:first + n], non_blocking=True)
+            out[key] = dst
+        return out
+
+    def _prefetch(self, first: int, n: int, device):
+        """Start copying rows [first, first + n) on the copy stream: the guess for the next micro-batch (the run
+        that follows this one, same size).  The copy stream first waits for the training stream, which is idle
+        here (a micro-batch ends with a synchronisation), so memory the allocator hands out again is not still in
+        use; the copy then runs beside the micro-batch that is launched next."""
+        if self._copy_stream is None:
+            self._copy_stream = torch.cuda.Stream(device=device)
+        self._copy_stream.wait_stream(torch.cuda.current_stream(device))
+        with torch.cuda.stream(self._copy_stream):
+            tensors = self._copy_run(first, n, device)
+            done = torch.cuda.Event()
+            done.record(self._copy_stream)
+        self._ahead = (first, n, tensors, done)
+
+    def drop_prefetched(self):
+        """Give the guessed batch's memory back (before memory is handed to inference)."""
+        if self._ahead is not None:
+            self._ahead[3].synchronize()
+            self._ahead = None
 
     def to_device(self, range_vec: RangeVec, device) -> dict:
         rows = self.rows_of(range_vec)
         n = rows.numel()
         # one ascending run is a slice of the pinned tensor: a single asynchronous copy, no gather on the host
         run = n > 0 and int(rows[-1]) - int(rows[0]) == n - 1 and bool((rows[1:] > rows[:-1]).all())
-        out = {}
-        for key, src in self.tensors.items():
-            dst = torch.empty((n, *src.shape[1:]), dtype=src.dtype, device=device)
-            if run:
-                dst.copy_(src[int(rows[0]):int(rows[0]) + n], non_blocking=True)
-            elif n:
-                dst.copy_(src.index_select(0, rows))
-            out[key] = dst
+        on_gpu = self.pinned and str(device).startswith('cuda')
+        ahead, self._ahead = self._ahead, None
+        if run and ahead is not None and ahead[:2] == (int(rows[0]), n):
+            torch.cuda.current_stream(device).wait_event(ahead[3])
+            out = ahead[2]
+        elif run:
+            if ahead is not None:
+                ahead[3].synchronize()
+            out = self._copy_run(int(rows[0]), n, device)
+        else:
+            if ahead is not None:
+                ahead[3].synchronize()
+            out = {}
+            for key, src in self.tensors.items():
+                dst = torch.empty((n, *src.shape[1:]), dtype=src.dtype, device=device)
+                if n:
+                    dst.copy_(src.index_select(0, rows))
+                out[key] = dst
+        if run and on_gpu and self.prefetch:
+            follow = (int(rows[-1]) + 1) % self.resident
+            if follow + n <= self.resident:
+                self._prefetch(follow, n, device)
         return out
 
 

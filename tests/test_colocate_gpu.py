@@ -54,6 +54,7 @@ def clean_runtime(monkeypatch):
     tc.reset_for_tests()
     yield tc
     torch.cuda.synchronize()      # also behind a failed test nothing may be running when the pool is unmapped
+    torch.cuda.set_stream(torch.cuda.default_stream())   # setup_colocate_training made its own stream current
     tc.UnRegisterAllStreams()
     tc.SetRejectCudaCalls(False)
     tc.reset_for_tests()
