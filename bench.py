@@ -327,6 +327,10 @@ def main():
     ap.add_argument("--only-swin", action="store_true", help="run the Swin-B step measurement alone (for profiling it)")
     ap.add_argument("--no-autotune", action="store_true", help="keep the library's tiling heuristic")
     ap.add_argument("--no-overlap", action="store_true", help="record weight gradients on the main lane (one stream)")
+    ap.add_argument("--group-wgrad", action="store_true", help="grouped weight-gradient launches instead of one per layer")
+    ap.add_argument("--wgrad-group-blocks", type=int, default=None, help="bottleneck blocks per grouped weight-gradient launch (0: a stage)")
+    ap.add_argument("--wgrad-group-wgs", type=int, default=None, help="workgroups a grouped weight-gradient launch aims for")
+    ap.add_argument("--wgrad-group-max-wgs", type=int, default=None, help="cap on the workgroups of a grouped weight-gradient launch")
     ap.add_argument("--calibrate", action="store_true",
                     help="also launch accumulate_kernel once over two 512 MiB buffers (reads 1 GiB, writes 1 GiB): "
                          "the known-size dispatch that scales FETCH_SIZE / WRITE_SIZE counter readings")
@@ -354,7 +358,11 @@ def main():
         return
     B = args.batch
     eng = ResNetEngine((3, 8, 36, 3), 1000, 64, dtype=torch.bfloat16, image_size=224, lr=0.1, momentum=0.9,
-                       weight_decay=1e-4, overlap_wgrad=not args.no_overlap, autotune=not args.no_autotune)
+                       weight_decay=1e-4, overlap_wgrad=not args.no_overlap, autotune=not args.no_autotune,
+                       group_wgrad=args.group_wgrad,
+                       **({} if args.wgrad_group_blocks is None else {"wgrad_group_blocks": args.wgrad_group_blocks}),
+                       **({} if args.wgrad_group_wgs is None else {"wgrad_group_wgs": args.wgrad_group_wgs}),
+                       **({} if args.wgrad_group_max_wgs is None else {"wgrad_group_max_wgs": args.wgrad_group_max_wgs}))
     eng.init_kaiming(seed=0)
     g = torch.Generator(device="cuda")
     g.manual_seed(1)

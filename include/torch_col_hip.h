@@ -188,6 +188,24 @@ int64_t tch_conv2d_wgrad_workspace_bytes(int dtype, int K, int R, int S, int C, 
 int tch_conv2d_wgrad(tch_context* ctx, int dtype, const void* x, const void* dy, float* dw, float* workspace,
                      int splits, int accumulate, int N, int H, int W, int C, int K, int R, int S, int stride,
                      int pad, int tile_cfg, int c_logical);
+/* The weight gradients (and optional bias gradients) of n convolutions as ONE launch over a table in device
+ * memory, plus one launch for the split reductions that remain: what a training step does once a stage's
+ * data-gradient chain has passed and every dy of the stage is at hand (the reference gets one cuDNN call per
+ * layer from autograd: train/resnet152.py:84-91; the result per layer is that of tch_conv2d_wgrad with the same
+ * split count, bit for bit).  shapes = n x {N, H, W, C, K, R, S, stride, pad}; x / dy / dw / dbias = n device
+ * addresses each (dbias may be NULL, or hold zeros for layers without a bias).
+ * _plan writes a split count per convolution so that the group yields about target_wgs (<= 0: 1024) workgroups
+ * of about equal length -- one split each, no partial filters at all, if the group is large enough -- and the
+ * bytes of `table` and `workspace` the call needs; it returns the tiling (0 = 128x128, 2 = 64x64) that
+ * tile_cfg < 0 stands for.  `table` is written by the call (synchronously) and read by the launches whenever
+ * they run: it must stay untouched for as long as a recorded program holds them.  max_wgs > 0 caps the launch at
+ * that many workgroups, each of which then takes every max_wgs-th tile of the group in turn: a launch that
+ * runs beside other kernels on a share of every compute unit instead of flooding the chip (same results). */
+int tch_conv2d_wgrad_group_plan(int dtype, int n, const int* shapes, int target_wgs, int tile_cfg, int* splits,
+                                int64_t* table_bytes, int64_t* workspace_bytes);
+int tch_conv2d_wgrad_group(tch_context* ctx, int dtype, int n, const int* shapes, const uint64_t* x, const uint64_t* dy,
+                           const uint64_t* dw, const uint64_t* dbias, const int* splits, int tile_cfg, int accumulate,
+                           float* workspace, void* table, int max_wgs);
 /* tch_conv2d_wgrad for callers that cannot allocate device memory and hold no workspace of their own: code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
  * reference.  Same kernels and same result, bit for bit, as tch_conv2d_wgrad with the same split count; the

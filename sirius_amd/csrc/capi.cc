@@ -2,6 +2,8 @@
 #include "../../include/torch_col_hip.h"
 
 #include "context.h"
+#include <vector>
+
 #include "ops.h"
 
 #include <stdio.h>
@@ -408,6 +410,41 @@ int tch_conv2d_wgrad(tch_context* ctx, int dtype, const void* x, const void* dy,
   ConvShape s = shape(N, H, W, Cc, K, R, S, stride, pad, c_logical);
   if (splits <= 0) splits = workspace ? conv2d_wgrad_pick_splits(s, dtype) : 1;
   return conv2d_wgrad(C(ctx), dtype, s, x, dy, dw, workspace, splits, accumulate, tile_cfg);
+}
+
+int tch_conv2d_wgrad_group_plan(int dtype, int n, const int* shapes, int target_wgs, int tile_cfg, int* splits,
+                                int64_t* table_bytes, int64_t* workspace_bytes) {
+  if (n <= 0 || !shapes || !splits) {
+    set_error("tch_conv2d_wgrad_group_plan: empty group");
+    return -22;
+  }
+  std::vector<ConvShape> v(static_cast<size_t>(n));
+  for (int i = 0; i < n; ++i) {
+    const int* q = shapes + 9 * i;
+    v[static_cast<size_t>(i)] = shape(q[0], q[1], q[2], q[3], q[4], q[5], q[6], q[7], q[8]);
+  }
+  return conv2d_wgrad_group_plan(dtype, n, v.data(), target_wgs, tile_cfg, splits, table_bytes, workspace_bytes);
+}
+
+int tch_conv2d_wgrad_group(tch_context* ctx, int dtype, int n, const int* shapes, const uint64_t* x, const uint64_t* dy,
+                           const uint64_t* dw, const uint64_t* dbias, const int* splits, int tile_cfg, int accumulate,
+                           float* workspace, void* table, int max_wgs) {
+  if (n <= 0 || !shapes || !x || !dy || !dw || !splits) {
+    set_error("tch_conv2d_wgrad_group: empty group or null array");
+    return -22;
+  }
+  std::vector<WgradGroupItem> v(static_cast<size_t>(n));
+  for (int i = 0; i < n; ++i) {
+    const int* q = shapes + 9 * i;
+    WgradGroupItem& it = v[static_cast<size_t>(i)];
+    it.shape = shape(q[0], q[1], q[2], q[3], q[4], q[5], q[6], q[7], q[8]);
+    it.x = reinterpret_cast<const void*>(x[i]);
+    it.dy = reinterpret_cast<const void*>(dy[i]);
+    it.dw = reinterpret_cast<float*>(dw[i]);
+    it.dbias = dbias ? reinterpret_cast<float*>(dbias[i]) : nullptr;
+    it.splits = splits[i];
+  }
+  return conv2d_wgrad_group(C(ctx), dtype, n, v.data(), tile_cfg, accumulate, workspace, table, max_wgs);
 }
 
 int64_t tch_conv2d_wgrad_static_capacity_bytes(void) { return conv2d_wgrad_static_capacity_bytes(); }

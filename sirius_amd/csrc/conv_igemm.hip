@@ -31,6 +31,9 @@
 // output columns: the epilogue moves them through LDS as 16-byte vectors and
 // writes (and reads the residual / mask) as full 16-byte chunks per lane.
 #include "kernels.h"
+#include <algorithm>
+#include <vector>
+
 #include "ops.h"
 
 #include <mutex>
@@ -625,8 +628,9 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm_kernel(IgemmArgs p) {
 // ---------------------------------------------------------------------------
 // weight gradient
 // ---------------------------------------------------------------------------
+// `id`: the workgroup's place among the tiles_m * tiles_n * splits workgroups of this weight gradient
 template <typename T, int WM, int WN, int TM, int TN>
-__global__ __launch_bounds__(WM* WN * 64) void wgrad_kernel(IgemmArgs p) {
+__device__ __forceinline__ void wgrad_body(const IgemmArgs& p, uint32_t id) {
   constexpr int E = Elem<T>::kPerChunk;
   constexpr int BKP = 4 * E;  // pixels per reduction step
   constexpr int BM = WM * TM * 32;
@@ -652,7 +656,6 @@ __global__ __launch_bounds__(WM* WN * 64) void wgrad_kernel(IgemmArgs p) {
   const int wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
 
-  uint32_t id = xcd_remap(blockIdx.x, gridDim.x);
   const int tiles_mn = p.tiles_m * p.tiles_n;
   const int split = id / tiles_mn;
   id -= split * tiles_mn;
@@ -851,6 +854,33 @@ __global__ __launch_bounds__(WM* WN * 64) void wgrad_kernel(IgemmArgs p) {
       float* dst = p.dbias + (p.splits > 1 ? static_cast<int64_t>(split) * p.gemm_m : 0) + m0 + tid;
       *dst = accumulate ? *dst + s : s;
     }
+  }
+}
+
+template <typename T, int WM, int WN, int TM, int TN>
+__global__ __launch_bounds__(WM* WN * 64) void wgrad_kernel(IgemmArgs p) {
+  wgrad_body<T, WM, WN, TM, TN>(p, xcd_remap(blockIdx.x, gridDim.x));
+}
+
+// The weight gradients of several convolutions in one launch.  `table` holds one argument block per convolution,
+// `map` one entry per workgroup: (which convolution, which of its workgroups).  Neighbouring entries of the map
+// are workgroups of the same convolution and split, so that after the XCD remap the workgroups that share
+// operand rows also share an L2.  Both arrays are read with wave-uniform addresses.
+// With fewer workgroups than entries a workgroup takes every gridDim.x-th entry: a launch that is meant to run
+// beside other kernels for a long time on a share of every CU instead of flooding the chip.
+struct WgradGroupArgs {
+  const IgemmArgs* table;
+  const uint2* map;
+  uint32_t entries;
+};
+
+template <typename T, int WM, int WN, int TM, int TN>
+__global__ __launch_bounds__(WM* WN * 64) void wgrad_group_kernel(WgradGroupArgs g) {
+  for (uint32_t gid = xcd_remap(blockIdx.x, gridDim.x); gid < g.entries; gid += gridDim.x) {
+    const uint2 e = g.map[gid];
+    const IgemmArgs p = g.table[__builtin_amdgcn_readfirstlane(e.x)];
+    wgrad_body<T, WM, WN, TM, TN>(p, __builtin_amdgcn_readfirstlane(e.y));
+    __syncthreads();   // the next entry's operand tiles overwrite what the epilogue staged in LDS
   }
 }
 
@@ -1289,9 +1319,9 @@ struct ReduceArgs {
   unsigned first_blocks;
 };
 
-__global__ __launch_bounds__(256) void splitk_reduce_kernel(ReduceArgs p) {
-  if (blockIdx.x >= p.first_blocks) {
-    const int i = (blockIdx.x - p.first_blocks) * 256 + threadIdx.x;
+__device__ __forceinline__ void splitk_reduce_body(const ReduceArgs& p, uint32_t block) {
+  if (block >= p.first_blocks) {
+    const int i = (block - p.first_blocks) * 256 + threadIdx.x;
     if (i >= p.n2) return;
     float s = 0.f;
     constexpr int U2 = 8;
@@ -1306,7 +1336,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(ReduceArgs p) {
     p.out2[i] = p.accumulate ? p.out2[i] + s : s;
     return;
   }
-  int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4;
+  int64_t i = (static_cast<int64_t>(block) * 256 + threadIdx.x) * 4;
   if (i >= p.n) return;
   // Eight partials are requested before any is added (a request past the last split repeats it and does not
   // count): the kernel costs its dependent round trips to memory, one per trip here instead of one per split.
@@ -1338,6 +1368,20 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(ReduceArgs p) {
     s.w += c.w;
   }
   *o = s;
+}
+
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(ReduceArgs p) { splitk_reduce_body(p, blockIdx.x); }
+
+// The split reductions of several weight gradients in one launch (table / map as in wgrad_group_kernel).
+struct ReduceGroupArgs {
+  const ReduceArgs* table;
+  const uint2* map;
+};
+
+__global__ __launch_bounds__(256) void splitk_reduce_group_kernel(ReduceGroupArgs g) {
+  const uint2 e = g.map[blockIdx.x];
+  const ReduceArgs p = g.table[__builtin_amdgcn_readfirstlane(e.x)];
+  splitk_reduce_body(p, __builtin_amdgcn_readfirstlane(e.y));
 }
 
 int ilog2_exact(int v) {
@@ -1747,6 +1791,220 @@ int conv2d_wgrad(Context* ctx, int dtype, const ConvShape& s, const void* x, con
     const unsigned blocks = r.first_blocks + static_cast<unsigned>((r.n2 + 255) / 256);
     return launch(ctx, splitk_reduce_kernel, dim3(blocks), dim3(256), r, "splitk_reduce_kernel",
                   4.0 * r.n * (splits + 1 + (accumulate ? 1 : 0)), 1);
+  }
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Grouped weight gradients: the weight gradients of several convolutions (a stage of a network, whose dy tensors
+// are all at hand once the data-gradient chain has passed) as ONE launch over a table, plus one launch for the
+// split reductions that are left.  Together the convolutions fill the chip, so each needs few splits or none:
+// long reduction loops, little or nothing written as partial filters, two launches instead of two per layer.
+// ---------------------------------------------------------------------------------------------------------------
+namespace {
+
+struct GroupLayout {
+  int64_t args_off = 0, red_off = 0, map_off = 0, rmap_off = 0, bytes = 0;
+  int64_t wgs = 0, reduce_blocks = 0, workspace_floats = 0;
+};
+
+int group_tile(int dtype, int n, const ConvShape* shapes, int tile_cfg) {
+  if (tile_cfg == 0 || tile_cfg == 2) return tile_cfg;
+  for (int i = 0; i < n; ++i)
+    if (shapes[i].K < 128 || shapes[i].R * shapes[i].S * shapes[i].C < 128) return 2;
+  return 0;
+}
+
+int64_t group_pixels(const ConvShape& s) {
+  int Ho, Wo;
+  conv_output_hw(s, &Ho, &Wo);
+  return static_cast<int64_t>(s.N) * Ho * Wo;
+}
+
+// what conv2d_wgrad makes of a requested split count: whole reduction steps per split, no empty tail splits
+void normalise_split(int64_t pixels, int BK, int want, int* splits, int* per) {
+  if (want < 1) want = 1;
+  int64_t p = (pixels + want - 1) / want;
+  p = (p + BK - 1) / BK * BK;
+  *per = static_cast<int>(p);
+  *splits = static_cast<int>((pixels + p - 1) / p);
+}
+
+GroupLayout group_layout(int dtype, int n, const ConvShape* shapes, const int* splits, int tile) {
+  const int BK = dtype == kBF16 ? 32 : 16;
+  const int bm = tile == 0 ? 128 : 64;
+  GroupLayout L;
+  for (int i = 0; i < n; ++i) {
+    const ConvShape& s = shapes[i];
+    int sp, per;
+    normalise_split(group_pixels(s), BK, splits[i], &sp, &per);
+    const int64_t filt = static_cast<int64_t>(s.K) * s.R * s.S * s.C;
+    L.wgs += tiles_for(s.K, s.R * s.S * s.C, bm, bm) * sp;
+    if (sp > 1) {
+      L.workspace_floats += sp * (filt + s.K);
+      L.reduce_blocks += (filt / 4 + 255) / 256 + (s.K + 255) / 256;
+    }
+  }
+  auto up = [](int64_t v) { return (v + 255) / 256 * 256; };
+  L.args_off = 0;
+  L.red_off = up(static_cast<int64_t>(n) * sizeof(IgemmArgs));
+  L.map_off = L.red_off + up(static_cast<int64_t>(n) * sizeof(ReduceArgs));
+  L.rmap_off = L.map_off + up(L.wgs * static_cast<int64_t>(sizeof(uint2)));
+  L.bytes = L.rmap_off + up(L.reduce_blocks * static_cast<int64_t>(sizeof(uint2)));
+  return L;
+}
+
+}  // namespace
+
+int conv2d_wgrad_group_plan(int dtype, int n, const ConvShape* shapes, int target_wgs, int tile_cfg, int* splits,
+                            int64_t* table_bytes, int64_t* workspace_bytes) {
+  TCH_CHECK_ARG(n > 0 && shapes && splits, "conv2d_wgrad_group_plan: empty group");
+  TCH_CHECK_ARG(dtype == kBF16 || dtype == kF32, "conv2d_wgrad_group_plan: dtype must be f32(0) or bf16(1)");
+  const int BK = dtype == kBF16 ? 32 : 16;
+  const int tile = group_tile(dtype, n, shapes, tile_cfg);
+  const int bm = tile == 0 ? 128 : 64;
+  if (target_wgs <= 0) target_wgs = 1024;
+  constexpr int64_t kMinSteps = 16;   // a split is at least this many reduction steps long
+  std::vector<int64_t> steps(n), tiles(n);
+  int64_t longest = 1;
+  for (int i = 0; i < n; ++i) {
+    const ConvShape& s = shapes[i];
+    TCH_CHECK_ARG(s.N > 0 && s.H > 0 && s.W > 0 && s.C > 0 && s.K > 0 && s.R > 0 && s.S > 0, "conv: non-positive dimension");
+    steps[i] = (group_pixels(s) + BK - 1) / BK;
+    tiles[i] = tiles_for(s.K, s.R * s.S * s.C, bm, bm);
+    longest = std::max(longest, steps[i]);
+  }
+  // Every workgroup runs about `len` reduction steps: the largest `len` that still yields target_wgs workgroups
+  // (none if the unsplit group already has that many).
+  auto wgs_at = [&](int64_t len) {
+    int64_t w = 0;
+    for (int i = 0; i < n; ++i) w += tiles[i] * ((steps[i] + len - 1) / len);
+    return w;
+  };
+  int64_t len = longest;
+  if (wgs_at(len) < target_wgs) {
+    int64_t lo = kMinSteps, hi = longest;   // wgs_at is non-increasing in len
+    while (lo < hi) {
+      const int64_t mid = (lo + hi + 1) / 2;
+      if (wgs_at(mid) >= target_wgs) lo = mid; else hi = mid - 1;
+    }
+    len = lo;
+  }
+  for (int i = 0; i < n; ++i) {
+    int sp, per;
+    normalise_split(group_pixels(shapes[i]), BK, static_cast<int>(std::min<int64_t>((steps[i] + len - 1) / len, 512)), &sp, &per);
+    splits[i] = sp;
+  }
+  const GroupLayout L = group_layout(dtype, n, shapes, splits, tile);
+  if (table_bytes) *table_bytes = L.bytes;
+  if (workspace_bytes) *workspace_bytes = std::max<int64_t>(L.workspace_floats * 4, 4);
+  return tile;
+}
+
+int conv2d_wgrad_group(Context* ctx, int dtype, int n, const WgradGroupItem* items, int tile_cfg, int accumulate,
+                       float* workspace, void* table, int max_wgs) {
+  TCH_CHECK_ARG(n > 0 && items && table, "conv2d_wgrad_group: empty group or no table");
+  const int eb = dtype == kBF16 ? 2 : 4;
+  const int BK = dtype == kBF16 ? 32 : 16;
+  std::vector<ConvShape> shapes(n);
+  std::vector<int> splits(n);
+  for (int i = 0; i < n; ++i) {
+    shapes[i] = items[i].shape;
+    splits[i] = items[i].splits;
+  }
+  const int tile = group_tile(dtype, n, shapes.data(), tile_cfg);
+  const int bm = tile == 0 ? 128 : 64;
+  const GroupLayout L = group_layout(dtype, n, shapes.data(), splits.data(), tile);
+  TCH_CHECK_ARG(L.workspace_floats == 0 || workspace, "conv2d_wgrad_group: split reductions need a workspace");
+  TCH_CHECK_ARG(L.wgs > 0 && L.wgs <= 0x7fffffff, "conv2d_wgrad_group: grid out of range");
+
+  std::vector<unsigned char> host(static_cast<size_t>(L.bytes), 0);
+  IgemmArgs* args = reinterpret_cast<IgemmArgs*>(host.data() + L.args_off);
+  ReduceArgs* reds = reinterpret_cast<ReduceArgs*>(host.data() + L.red_off);
+  uint2* map = reinterpret_cast<uint2*>(host.data() + L.map_off);
+  uint2* rmap = reinterpret_cast<uint2*>(host.data() + L.rmap_off);
+  double flops = 0.0, bytes = 0.0, red_bytes = 0.0;
+  int64_t ws_off = 0;
+  int n_red = 0;
+  std::vector<int> order(n);
+  for (int i = 0; i < n; ++i) order[i] = i;
+  for (int i = 0; i < n; ++i) {
+    IgemmArgs& a = args[i];
+    const WgradGroupItem& it = items[i];
+    if (int rc = fill_common(a, it.shape, dtype)) return rc;
+    TCH_CHECK_ARG(it.x && it.dy && it.dw, "conv2d_wgrad_group: null tensor");
+    const ConvShape& s = it.shape;
+    a.a_src = it.dy;
+    a.b_src = it.x;
+    a.a_bytes = static_cast<uint32_t>(static_cast<int64_t>(s.N) * a.Ho * a.Wo * s.K * eb);
+    a.b_bytes = static_cast<uint32_t>(static_cast<int64_t>(s.N) * s.H * s.W * s.C * eb);
+    a.gemm_m = s.K;
+    a.gemm_n = s.R * s.S * s.C;
+    a.gemm_k = s.N * a.Ho * a.Wo;
+    normalise_split(a.gemm_k, BK, it.splits, &a.splits, &a.k_per_split);
+    a.accumulate = accumulate;
+    a.tiles_m = (a.gemm_m + bm - 1) / bm;
+    a.tiles_n = (a.gemm_n + bm - 1) / bm;
+    a.div_plane = FastDiv(a.Ho * a.Wo);
+    a.div_width = FastDiv(a.Wo);
+    const int64_t filt = static_cast<int64_t>(a.gemm_m) * a.gemm_n;
+    if (a.splits > 1) {
+      float* part = workspace + ws_off;
+      float* bias_part = part + a.splits * filt;
+      ws_off += a.splits * (filt + a.gemm_m);
+      a.out = part;
+      a.dbias = it.dbias ? bias_part : nullptr;
+      TCH_CHECK_ARG(filt % 4 == 0, "conv2d_wgrad_group: filter size must be a multiple of 4");
+      ReduceArgs& r = reds[n_red];
+      r = ReduceArgs{part, it.dw, filt, a.splits, accumulate, bias_part, it.dbias, it.dbias ? a.gemm_m : 0, 0u};
+      r.first_blocks = static_cast<unsigned>((filt / 4 + 255) / 256);
+      red_bytes += 4.0 * filt * (a.splits + 1 + (accumulate ? 1 : 0));
+      ++n_red;
+    } else {
+      a.out = it.dw;
+      a.dbias = it.dbias;
+    }
+    flops += conv_flops(s, a.Ho, a.Wo);
+    bytes += conv_bytes<kWgrad>(a, eb);
+  }
+  // long workgroups first: what is left for the tail of the launch is short
+  std::stable_sort(order.begin(), order.end(), [&](int x, int y) { return args[x].k_per_split > args[y].k_per_split; });
+  int64_t w = 0;
+  for (int oi = 0; oi < n; ++oi) {
+    const int i = order[oi];
+    const int64_t cnt = static_cast<int64_t>(args[i].tiles_m) * args[i].tiles_n * args[i].splits;
+    for (int64_t j = 0; j < cnt; ++j) map[w++] = make_uint2(static_cast<unsigned>(i), static_cast<unsigned>(j));
+  }
+  TCH_CHECK_ARG(w == L.wgs, "conv2d_wgrad_group: workgroup count does not match the layout");
+  int64_t rb = 0;
+  for (int i = 0; i < n_red; ++i) {
+    const unsigned cnt = reds[i].first_blocks + static_cast<unsigned>((reds[i].n2 + 255) / 256);
+    for (unsigned j = 0; j < cnt; ++j) rmap[rb++] = make_uint2(static_cast<unsigned>(i), j);
+  }
+  TCH_CHECK_ARG(rb <= L.reduce_blocks, "conv2d_wgrad_group: reduction blocks do not match the layout");
+  // The table is written once, here; the launches (recorded or not) read it whenever they run.
+  hipError_t e = hipMemcpy(table, host.data(), host.size(), hipMemcpyHostToDevice);
+  TCH_CHECK_ARG(e == hipSuccess, std::string("conv2d_wgrad_group: table upload: ") + hipGetErrorString(e));
+
+  unsigned char* dev = static_cast<unsigned char*>(table);
+  WgradGroupArgs g{reinterpret_cast<const IgemmArgs*>(dev + L.args_off), reinterpret_cast<const uint2*>(dev + L.map_off),
+                   static_cast<uint32_t>(L.wgs)};
+  const dim3 grid(static_cast<unsigned>(max_wgs > 0 && max_wgs < L.wgs ? max_wgs : L.wgs)), block(256);
+  static const std::string names[2][2] = {{"wgrad_group_kernel<f32,128x128>", "wgrad_group_kernel<f32,64x64>"},
+                                          {"wgrad_group_kernel<bf16,128x128>", "wgrad_group_kernel<bf16,64x64>"}};
+  const char* name = names[dtype == kBF16 ? 1 : 0][tile == 0 ? 0 : 1].c_str();
+  int rc;
+  if (dtype == kBF16)
+    rc = tile == 0 ? launch(ctx, wgrad_group_kernel<bf16, 2, 2, 2, 2>, grid, block, g, name, flops, 0, bytes)
+                   : launch(ctx, wgrad_group_kernel<bf16, 2, 2, 1, 1>, grid, block, g, name, flops, 0, bytes);
+  else
+    rc = tile == 0 ? launch(ctx, wgrad_group_kernel<float, 2, 2, 2, 2>, grid, block, g, name, flops, 0, bytes)
+                   : launch(ctx, wgrad_group_kernel<float, 2, 2, 1, 1>, grid, block, g, name, flops, 0, bytes);
+  if (rc) return rc;
+  if (rb > 0) {
+    ReduceGroupArgs rg{reinterpret_cast<const ReduceArgs*>(dev + L.red_off), reinterpret_cast<const uint2*>(dev + L.rmap_off)};
+    return launch(ctx, splitk_reduce_group_kernel, dim3(static_cast<unsigned>(rb)), dim3(256), rg,
+                  "splitk_reduce_group_kernel", red_bytes, 1);
   }
   return 0;
 }

@@ -61,6 +61,23 @@ int64_t conv2d_wgrad_workspace_bytes(const ConvShape& s, int dtype, int splits);
 // dbias (optional, [K] fp32): also the column sums of dy, i.e. the gradient of a bias added to the output
 int conv2d_wgrad(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* dy, float* dw,
                  float* workspace, int splits, int accumulate, int tile_cfg, float* dbias = nullptr);
+// Several weight gradients as one launch (+ one for the split reductions that remain).  _plan picks a split
+// count per convolution so that the group yields about target_wgs workgroups of equal length (one split each if
+// the group is large enough without), says how large the device table and the workspace must be, and returns
+// the tiling (0 = 128x128, 2 = 64x64) it chose for tile_cfg < 0.
+struct WgradGroupItem {
+  ConvShape shape;
+  const void* x;
+  const void* dy;
+  float* dw;
+  float* dbias;  // optional
+  int splits;
+};
+int conv2d_wgrad_group_plan(int dtype, int n, const ConvShape* shapes, int target_wgs, int tile_cfg, int* splits,
+                            int64_t* table_bytes, int64_t* workspace_bytes);
+// max_wgs > 0: launch at most that many workgroups, each taking every max_wgs-th tile of the group
+int conv2d_wgrad_group(Context* ctx, int dtype, int n, const WgradGroupItem* items, int tile_cfg, int accumulate,
+                       float* workspace, void* table, int max_wgs = 0);
 // the same with the split-K partials in the library's static device buffer: no workspace, no allocation
 int64_t conv2d_wgrad_static_capacity_bytes();
 int conv2d_wgrad_static(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* dy, float* dw, int splits,

@@ -325,6 +325,54 @@ def conv2d_wgrad(ctx, x, dy, dw, stride, pad, workspace=None, splits=0, accumula
           "tch_conv2d_wgrad")
 
 
+def _wgrad_group_shapes(items):
+    import ctypes
+    flat = []
+    for it in items:
+        x, dy, dw, stride, pad = it[:5]
+        N, H, W, C = x.shape
+        K, R, S, C2 = dw.shape
+        assert C == C2 and dw.dtype == torch.float32 and dy.dtype == x.dtype
+        Ho, Wo = conv_out_hw(H, W, R, S, stride, pad)
+        assert tuple(dy.shape) == (N, Ho, Wo, K), (tuple(dy.shape), (N, Ho, Wo, K))
+        flat += [N, H, W, C, K, R, S, stride, pad]
+    return (ctypes.c_int * len(flat))(*flat)
+
+
+def conv2d_wgrad_group_plan(items, target_wgs=0, tile_cfg=-1):
+    """items: (x, dy, dw, stride, pad[, dbias]) per convolution (tensors may be on the meta device).  Returns
+    (splits per convolution, tiling, table bytes, workspace bytes) for conv2d_wgrad_group."""
+    import ctypes
+    n = len(items)
+    shapes = _wgrad_group_shapes(items)
+    splits = (ctypes.c_int * n)()
+    tb, wb = ctypes.c_int64(0), ctypes.c_int64(0)
+    tile = check(lib().tch_conv2d_wgrad_group_plan(dtype_code(items[0][0]), n, shapes, target_wgs, tile_cfg, splits,
+                                                   ctypes.byref(tb), ctypes.byref(wb)), "tch_conv2d_wgrad_group_plan")
+    return list(splits), tile, tb.value, wb.value
+
+
+def conv2d_wgrad_group(ctx, items, splits, tile_cfg, workspace, table, accumulate=False, max_wgs=0):
+    """The weight gradients of every (x, dy, dw, stride, pad[, dbias]) of `items` in one launch (+ one for the
+    split reductions): dw (+)= dy^T x, dbias (+)= column sums of dy.  `table` (uint8, device) and `workspace`
+    (fp32, device) sized by conv2d_wgrad_group_plan; the table is written here and must stay untouched while a
+    recorded program holds the launches.  max_wgs > 0: at most that many workgroups, which share the tiles out
+    among themselves (a launch that runs beside others instead of flooding the chip)."""
+    import ctypes
+    n = len(items)
+    assert n == len(splits) and table.dtype == torch.uint8 and table.is_cuda
+    shapes = _wgrad_group_shapes(items)
+    arr = ctypes.c_uint64 * n
+    xs = arr(*[it[0].data_ptr() for it in items])
+    dys = arr(*[it[1].data_ptr() for it in items])
+    dws = arr(*[it[2].data_ptr() for it in items])
+    with_bias = any(len(it) > 5 and it[5] is not None for it in items)
+    dbs = arr(*[(it[5].data_ptr() if len(it) > 5 and it[5] is not None else 0) for it in items]) if with_bias else None
+    sp = (ctypes.c_int * n)(*splits)
+    check(lib().tch_conv2d_wgrad_group(ctx.handle, dtype_code(items[0][0]), n, shapes, xs, dys, dws, dbs, sp, tile_cfg,
+                                       int(accumulate), _p(workspace), _p(table), max_wgs), "tch_conv2d_wgrad_group")
+
+
 def conv2d_wgrad_static_capacity_bytes():
     return int(lib().tch_conv2d_wgrad_static_capacity_bytes())
 

@@ -50,7 +50,8 @@ class ResNetEngine(EngineBase):
     def __init__(self, depths=(3, 8, 36, 3), num_classes=1000, width=64, dtype=torch.bfloat16, image_size=224,
                  lr=0.1, momentum=0.9, weight_decay=1e-4, bn_momentum=0.1, bn_eps=1e-5, stream=None, allocator=None,
                  overlap_wgrad=True, fuse_bn_stats=True, fuse_bn_bwd=True, fuse_bn_finalize=False, autotune=False,
-                 retain_gradients=False):
+                 retain_gradients=False, group_wgrad=False, wgrad_group_wgs=256, wgrad_group_blocks=2,
+                 wgrad_group_max_wgs=0):
         self._init_engine(dtype, stream, allocator)
         assert num_classes % 8 == 0, "class count must be a multiple of one 16-byte chunk"
         self.image_size, self.num_classes = image_size, num_classes
@@ -61,6 +62,19 @@ class ResNetEngine(EngineBase):
         # they run beside the data-gradient chain (each kernel alone leaves CUs idle at batch 64);
         # costs the recycling of the dy buffers (they stay alive until the lanes join)
         self.overlap_wgrad = overlap_wgrad
+        # group_wgrad: the weight gradients of the bottleneck convolutions are not launched layer by layer but
+        # collected, and launched together once the data-gradient chain has left a stage (or every
+        # wgrad_group_blocks blocks, if not 0): one launch over a table for all of them, sized for about
+        # wgrad_group_wgs workgroups of equal length, so that a layer is split only where a whole stage would
+        # not fill the chip.  Needs the second lane's rule that no dy buffer is handed out twice.  Off by default:
+        # measured on ResNet-152 at batch 64, the grouped launches need 2.4 ms of kernel time per step instead of
+        # 6.3 ms (745 against 320 TFLOP/s, no partial filters in stages 3 and 4, 300 launches fewer), but the step
+        # is 16.5-17.1 ms against 16.3 ms: the many short launches run in the gaps of the data-gradient chain,
+        # which is the critical path, while a launch that fills the chip holds that chain up for as long as it runs
+        # (also when it is capped to one workgroup per compute unit).
+        self.group_wgrad = group_wgrad and overlap_wgrad
+        self.wgrad_group_wgs, self.wgrad_group_blocks = wgrad_group_wgs, wgrad_group_blocks
+        self.wgrad_group_max_wgs = wgrad_group_max_wgs
         self.fuse_bn_stats = fuse_bn_stats
         # fuse_bn_bwd: a data-gradient convolution whose output flows into a BatchNorm(+ReLU) backward applies
         # the ReLU gate and takes that BatchNorm's two reductions in its epilogue (no reduction pass)
@@ -334,7 +348,7 @@ class ResNetEngine(EngineBase):
 
         def gfree(t, read_by_wgrad=False):
             # a buffer the side lane still reads must not be handed out again before the join
-            if (read_by_wgrad and self.overlap_wgrad) or self.retain_gradients:
+            if (read_by_wgrad and (self.overlap_wgrad or self.group_wgrad)) or self.retain_gradients:
                 return
             free.setdefault(t.numel(), []).append(t.reshape(-1))
 
@@ -444,7 +458,27 @@ class ResNetEngine(EngineBase):
                                       stat_partial, rb, bn_scratch, residual=residual, relu=relu,
                                       momentum=self.bn_momentum, eps=self.bn_eps)
 
-        def conv_wgrad(c, x, dy):
+        pending = []   # (convolution, its input, the gradient of its output): weight gradients not launched yet
+
+        def flush_wgrads():
+            if not pending:
+                return
+            items = [(x_, dy_, self._view(self.grads, c_.name + ".weight"), c_.stride, c_.pad) for c_, x_, dy_ in pending]
+            splits, tile, table_bytes, ws_bytes = ops.conv2d_wgrad_group_plan(items, self.wgrad_group_wgs)
+            table = act(table_bytes, dtype=torch.uint8)
+            ws = act(max(ws_bytes // 4, 1), dtype=torch.float32)
+            with ctx.side_lane(wait_main=True):
+                ops.conv2d_wgrad_group(ctx, items, splits, tile, ws, table, max_wgs=self.wgrad_group_max_wgs)
+            plan.wgrad_groups.append(dict(layers=[c_.name for c_, _, _ in pending], splits=splits, tile=tile,
+                                          workspace_bytes=ws_bytes))
+            pending.clear()
+
+        plan.wgrad_groups = []
+
+        def conv_wgrad(c, x, dy, grouped=False):
+            if grouped and self.group_wgrad:
+                pending.append((c, x, dy))
+                return
             if self.overlap_wgrad:
                 with ctx.side_lane(wait_main=True):
                     ops.conv2d_wgrad(ctx, x, dy, self._view(self.grads, c.name + ".weight"), c.stride, c.pad,
@@ -548,6 +582,7 @@ class ResNetEngine(EngineBase):
             # the sums of this block's bn3 (left by the c1 data gradient of the block after it); None = neither
             g_rb = None
             fuse = self.fuse_bn_bwd
+            since_flush = 0
             for bi in range(len(self.blocks) - 1, -1, -1):
                 blk, (H, W, Ho, Wo), sv = self.blocks[bi], shapes[bi], saved[bi]
                 xin, z1, a1, z2, a2, z3, zd, out = sv
@@ -558,7 +593,7 @@ class ResNetEngine(EngineBase):
                 else:
                     bn_bwd_sums(pre + ".bn3", g_out, z3, dz3, g_rb)
                 out_gate = out if g_rb is None else None   # what still has to gate g_out
-                conv_wgrad(blk.c3, a2, dz3)
+                conv_wgrad(blk.c3, a2, dz3, grouped=True)
                 g_a2 = galloc(a2.shape)
                 dz2 = galloc(z2.shape)
                 if fuse:
@@ -571,7 +606,7 @@ class ResNetEngine(EngineBase):
                     bn_bwd(pre + ".bn2", g_a2, z2, dz2, a2)
                 gfree(dz3, True)
                 gfree(g_a2)
-                conv_wgrad(blk.c2, a1, dz2)
+                conv_wgrad(blk.c2, a1, dz2, grouped=True)
                 g_a1 = galloc(a1.shape)
                 dz1 = galloc(z1.shape)
                 if fuse:
@@ -584,14 +619,14 @@ class ResNetEngine(EngineBase):
                     bn_bwd(pre + ".bn1", g_a1, z1, dz1, a1)
                 gfree(dz2, True)
                 gfree(g_a1)
-                conv_wgrad(blk.c1, xin, dz1)
+                conv_wgrad(blk.c1, xin, dz1, grouped=True)
                 gx = galloc(xin.shape)
                 # xin is the output of the block before (its bn3 + residual + ReLU), whose bn3 input is z3 there
                 prev = (self.blocks[bi - 1].prefix + ".bn3", saved[bi - 1][5]) if (fuse and bi > 0) else None
                 if blk.cd is not None:
                     dzd = galloc(zd.shape)
                     bn_bwd(pre + ".downsample.1", g_out, zd, dzd, out_gate)
-                    conv_wgrad(blk.cd, xin, dzd)
+                    conv_wgrad(blk.cd, xin, dzd, grouped=True)
                     gx_id = galloc(xin.shape)
                     conv_dgrad(blk.cd, dzd, gx_id)
                     gfree(dzd, True)
@@ -615,6 +650,11 @@ class ResNetEngine(EngineBase):
                 gfree(dz1, True)
                 gfree(g_out)
                 g_out = gx
+                since_flush += 1
+                if blk.cd is not None or (self.wgrad_group_blocks and since_flush >= self.wgrad_group_blocks):
+                    flush_wgrads()      # the stage ends here (its first block is the last one of the backward)
+                    since_flush = 0
+            flush_wgrads()
             g_a0 = galloc(a0.shape)
             ops.maxpool_bwd(ctx, g_out, p0_idx, g_a0, 3, 2, 1)
             gfree(g_out)

@@ -599,6 +599,10 @@ def get_train_info(id, field):
     return int(lib().tch_train_info_get_field(int(id), _TRAIN_INFO_FIELDS[field]))
 
 
+def train_info_is_valid(id):
+    return bool(lib().tch_train_info_is_valid(int(id)))
+
+
 def get_train_info_model_name(id):
     buf = ctypes.create_string_buffer(256)
     lib().tch_train_info_model_name(int(id), buf, 256)

@@ -18,6 +18,7 @@ from .dynamic_batch import (DynamicBatchDataset, MicroBatchManager, get_dynamic_
                             get_micro_batch_manager, init_dynamic_batch, BatchDistributePolicy)
 from .trainer import Trainer  # noqa: F401
 from .debug_server import DebugServer  # noqa: F401
+from .controller import Controller, ResourceManager, TrainStatus  # noqa: F401
 
 
 def setup_colocate_training(rank: int, world_size: int, will_use_nccl_comm: bool, init_nccl_process_group: bool):

@@ -161,6 +161,60 @@ def test_conv_wgrad(ctx, dtype, case, splits):
     close(db, 2 * db_ref, torch.float32, "bias gradient accumulate", rtol=1e-4)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("target_wgs,tile_cfg,max_wgs", [(0, -1, 0), (40, -1, 0), (300, 0, 0), (64, 2, 0), (0, -1, 37), (300, 0, 8)])
+def test_conv_wgrad_group(ctx, dtype, target_wgs, tile_cfg, max_wgs):
+    """Several weight gradients in one launch over a table: each layer's result equals the oracle's, and equals
+    the one-layer call with the same split count and tiling bit for bit (same kernel body, same split ranges,
+    same order of additions in the reduction); bias gradients ride along for the layers that ask.  max_wgs: the
+    launch is capped at that many workgroups, which share the tiles out among themselves."""
+    from sirius_amd import ops
+    cases = [c for c in CONV_CASES if c[7] in (1, 2)]
+    if tile_cfg == 0:
+        cases = [c for c in cases if c[4] >= 128 or c[3] * c[5] * c[6] >= 128]   # any shape runs, these fill tiles
+    g = _gen(11)
+    items, refs, singles = [], [], []
+    for i, (N, H, W, C, K, R, S, st, pad) in enumerate(cases):
+        Ho, Wo = ops.conv_out_hw(H, W, R, S, st, pad)
+        x = rnd((N, H, W, C), dtype, g)
+        dy = rnd((N, Ho, Wo, K), dtype, g, (N * Ho * Wo) ** -0.5)
+        dw = torch.full((K, R, S, C), float(i), dtype=torch.float32, device="cuda")
+        db = torch.full((K,), -1.0, dtype=torch.float32, device="cuda") if i % 2 == 0 else None
+        items.append((x.cuda(), dy.cuda(), dw, st, pad, db))
+        refs.append((O.conv2d_wgrad(x, dy, (K, R, S, C), st, pad), dy.float().sum(dim=(0, 1, 2))))
+    splits, tile, table_bytes, ws_bytes = ops.conv2d_wgrad_group_plan(items, target_wgs, tile_cfg)
+    print("group", dtype, target_wgs, tile_cfg, "->", tile, splits, table_bytes, ws_bytes, flush=True)
+    assert tile in (0, 2) and all(sp >= 1 for sp in splits)
+    if target_wgs == 0:
+        assert max(splits) > 1, "a small group is split to fill the chip"
+    table = torch.empty(table_bytes, dtype=torch.uint8, device="cuda")
+    ws = torch.full((max(ws_bytes // 4, 1),), float("nan"), dtype=torch.float32, device="cuda")
+    ops.conv2d_wgrad_group(ctx, items, splits, tile, ws, table, max_wgs=max_wgs)
+    torch.cuda.synchronize()
+    rt = 1e-3 if dtype == torch.float32 else 5e-3
+    for (x, dy, dw, st, pad, db), (ref, db_ref), sp, case in zip(items, refs, splits, cases):
+        close(dw, ref, dtype, f"grouped wgrad {case}", rtol=rt)
+        if db is not None:
+            close(db, db_ref, torch.float32, f"grouped bias gradient {case}", rtol=1e-4)
+        one = torch.empty_like(dw)
+        one_b = torch.empty_like(db) if db is not None else None
+        K, R, S, C = dw.shape
+        w1 = torch.empty(max(4, ops.conv2d_wgrad_workspace_bytes(ops.dtype_code(x), K, R, S, C, sp)) // 4,
+                         dtype=torch.float32, device="cuda")
+        ops.conv2d_wgrad(ctx, x, dy, one, st, pad, workspace=w1, splits=sp, tile_cfg=tile, dbias=one_b)
+        torch.cuda.synchronize()
+        assert torch.equal(one, dw), f"grouped and single launch differ for {case} at {sp} splits"
+        if db is not None:
+            assert torch.equal(one_b, db)
+    # a second run over the same table accumulates on top
+    ops.conv2d_wgrad_group(ctx, items, splits, tile, ws, table, accumulate=True, max_wgs=max_wgs)
+    torch.cuda.synchronize()
+    for (x, dy, dw, st, pad, db), (ref, db_ref), case in zip(items, refs, cases):
+        close(dw, 2 * ref, dtype, f"grouped wgrad accumulate {case}", rtol=rt)
+        if db is not None:
+            close(db, 2 * db_ref, torch.float32, f"grouped bias gradient accumulate {case}", rtol=1e-4)
+
+
 BN_CASES = [(2 * 14 * 14, 64), (4 * 28 * 28, 128), (3 * 7 * 7, 2048), (37, 8), (100000, 64)]
 
 

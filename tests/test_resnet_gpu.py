@@ -71,7 +71,7 @@ def engine_steps(eng, x, y, steps, micro_batches):
     return out
 
 
-def run_parity(depths, width, classes, image, batch, dtype, steps, micro_batches=1, direct_steps=0):
+def run_parity(depths, width, classes, image, batch, dtype, steps, micro_batches=1, direct_steps=0, **engine_kw):
     """HIP path and CPU path of the same precision on the same seeded weights and inputs, both
     measured against the fp64 oracle.  Per step: the loss is held to the DIRECT bound against
     the CPU path while the CPU path itself is that close to fp64; the worst and the median
@@ -83,7 +83,7 @@ def run_parity(depths, width, classes, image, batch, dtype, steps, micro_batches
     x, y = R.make_batch(batch, image, classes, seed=0)
     m64 = R.make_model(depths, classes, width, seed=0).double()
     mcpu = R.make_model(depths, classes, width, seed=0)
-    eng = ResNetEngine(depths, classes, width, dtype=dtype, image_size=image)
+    eng = ResNetEngine(depths, classes, width, dtype=dtype, image_size=image, **engine_kw)
     eng.load_state_dict(mcpu.state_dict())
     assert eng.num_parameters() == sum(p.numel() for p in mcpu.parameters())
     names = [k for k, _ in mcpu.named_parameters()]
@@ -132,6 +132,14 @@ def run_parity(depths, width, classes, image, batch, dtype, steps, micro_batches
 def test_fp32_four_stages_direct():
     """3 steps, every gradient / weight / statistic within 1e-3 of the CPU step"""
     run_parity((1, 1, 1, 1), 16, 16, 64, 4, torch.float32, 3, direct_steps=3)
+
+
+@pytest.mark.parametrize("blocks,wgs,cap", [(0, 1024, 0), (1, 8, 0), (2, 300, 16)])
+def test_fp32_grouped_weight_gradients(blocks, wgs, cap):
+    """the weight gradients of a stage (or of every `blocks` blocks) as one launch over a table, split to about
+    `wgs` workgroups, optionally capped: same bounds as the layer-by-layer plan"""
+    run_parity((2, 2, 2), 16, 16, 64, 8, torch.float32, 3, direct_steps=2, group_wgrad=True, wgrad_group_blocks=blocks,
+               wgrad_group_wgs=wgs, wgrad_group_max_wgs=cap)
 
 
 def test_fp32_identity_blocks():

@@ -206,3 +206,62 @@ def test_handover_64_16_64(colocate_env, capsys):
         lib().tch_pool_free(weights, 0, 0, None)
     finally:
         server.stop()
+
+
+def test_controller_command_ids_skip_rule_and_free_memory(colocate_env):
+    """The server's controller and resource manager as the stand-in peer restates them
+    (server/control/controller.cc:84-150,207-327,377-386; server/resource_manager.cc:22-87): command ids count
+    every call, nothing is sent to an idle trainer, a ColocateAdjust that finds no rank with an unpublished shrink
+    is skipped with id 0, the wait returns on a reply with an id >= the command's; free memory = pool - inference
+    - max(training now, training predicted) - margin."""
+    import time
+    tc = colocate_env
+    ctl = tc.Controller(1, colocate_level=1)
+    stub = None
+    try:
+        tc.torch_col_init(0, 1, use_gpu=False)
+        tc.init_train_info(64, 64, model_name="resnet152")
+        # idle trainer: ids are taken, nothing is sent
+        assert ctl.is_train_idle()
+        assert ctl.colocate_infer_require_adjust([48]) == 1 and ctl.colocate_adjust(8) == 2 and not ctl.sent
+        assert ctl.wait_colocate_adjust_done(2) is True          # idle: nothing to wait for
+        stub = tc.PyColocateStub(64)
+        stub.train_start()
+        assert ctl.wait_train_status(tc.TrainStatus.kRunning, 5.0)
+        assert ctl.target_batch_size == 64
+        # board: target 64, unpublished 64 -> no rank has a shrink pending: skipped, id 0, but the id is used up
+        assert ctl.colocate_adjust(8) == 0 and not ctl.sent
+        # inference asks for 4080 MB: 48 samples at 85 MB (server/train_adjuster.cc:535-538) -> target 16, id 4
+        cmd = ctl.infer_require_memory_mb(4080)
+        assert cmd == 4 and tc._C.get_train_info(0, "target_batch_size_unpublished") == 16
+        assert [(r, i, e, v) for _, r, i, e, v in ctl.sent] == [(0, 4, tc.CtrlEvent.kColocateAdjustL1, 16)]
+        for _ in range(2000):
+            if stub.cmd == tc.CtrlEvent.kColocateAdjustL1:
+                break
+            time.sleep(0.001)
+        assert stub.cmd == tc.CtrlEvent.kColocateAdjustL1 and stub.unpub_target_batch_size == 16 and stub.target_batch_size == 64
+        # now a shrink is pending (unpublished 16 < published 64): ColocateAdjust goes out, value = launcher target - 8
+        assert ctl.wait_colocate_adjust_done(cmd, timeout_s=0.05) is False
+        assert ctl.colocate_adjust(8) == 5 and ctl.sent[-1][2:] == (5, tc.CtrlEvent.kColocateAdjustL1, 8)
+        stub.adjust_l1_done()
+        assert ctl.wait_colocate_adjust_done(cmd, timeout_s=5.0) is True and ctl.adjust_done_ids[0] >= cmd
+        # resource manager on the pool of this environment (0.5 GB): training predicted at its new target
+        rm = tc.ResourceManager(train_memory_over_predict_mb=10.0)
+        pool_mb = tc._C.cuda_memory_pool_nbytes(0) / 1024 / 1024
+        assert pool_mb == 512.0
+        target = tc._C.get_train_info(0, "target_batch_size_unpublished")
+        assert rm.predict_train_memory_mb() == 1150 + 85 * target
+        blk = lib().tch_pool_malloc(96 * MB, 0, None)
+        assert rm.train_memory_mb() >= 96.0 and rm.infer_memory_mb() == 0.0
+        assert rm.free_memory_mb() == pool_mb - 0.0 - max(rm.train_memory_mb(), rm.predict_train_memory_mb()) - 10.0
+        assert rm.train_avail_memory_mb() == pool_mb - 10.0
+        lib().tch_pool_free(blk, 0, 0, None)
+        # inference leaves 1150 + 85 * 64 + 10 MB to training: back to the initial size, as kInferExit
+        cmd = ctl.infer_release_memory_mb(1150 + 85 * 64 + 10)
+        assert ctl.sent[-1][2:] == (cmd, tc.CtrlEvent.kInferExit, 64)
+        stub.train_end()
+        assert ctl.wait_train_status(tc.TrainStatus.kIdle, 5.0)
+    finally:
+        if stub is not None:
+            stub.stop()
+        ctl.stop()
