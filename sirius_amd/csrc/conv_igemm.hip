@@ -79,6 +79,7 @@ struct IgemmArgs {
   int R, S, stride, stride_log2, pad;
   int gemm_m, gemm_n, gemm_k;
   int tiles_m, tiles_n, splits;
+  int group_rows;   // FWD/DGRAD direct-to-LDS kernel: row tiles per group of the tile order (0 / 1: row-major)
   int k_per_split;  // multiple of BK
   int out_f32;      // FWD/DGRAD: store fp32 instead of T
   int accumulate;   // WGRAD with splits == 1: out += result
@@ -908,7 +909,7 @@ __device__ inline void load_to_lds(__amdgpu_buffer_rsrc_t rsrc, unsigned char* d
   __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)dst, 16, voff, soff, 0, 0);
 }
 
-template <int MODE, int WM, int WN, int TM, int TN, int NBUF>
+template <int MODE, int WM, int WN, int TM, int TN, int NBUF, int ROT = 0>
 __global__ __launch_bounds__(WM* WN * 64) void igemm2_kernel(IgemmArgs p) {
   using T = bf16;
   constexpr int E = 8;
@@ -930,8 +931,21 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm2_kernel(IgemmArgs p) {
   const int wm = wave / WN, wn = wave % WN;
 
   uint32_t id = xcd_remap(blockIdx.x, gridDim.x);
-  const int tile_m = id / p.tiles_n;
-  const int tile_n = id - tile_m * p.tiles_n;
+  int tile_m, tile_n;
+  if (p.group_rows > 1) {
+    // wide outputs: consecutive ids walk down group_rows row tiles before they move one column tile on, so that
+    // the tiles an XCD works on at one time form a squarish block (fewer distinct operand rows through its L2)
+    const uint32_t per_group = static_cast<uint32_t>(p.group_rows) * p.tiles_n;
+    const uint32_t grp = id / per_group;
+    const uint32_t local = id - grp * per_group;
+    const uint32_t first = grp * p.group_rows;
+    const uint32_t rows = min(static_cast<uint32_t>(p.group_rows), static_cast<uint32_t>(p.tiles_m) - first);
+    tile_n = local / rows;
+    tile_m = first + (local - tile_n * rows);
+  } else {
+    tile_m = id / p.tiles_n;
+    tile_n = id - tile_m * p.tiles_n;
+  }
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   const int in_h = (MODE == kFwd) ? p.H : p.Ho;
@@ -1097,17 +1111,57 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm2_kernel(IgemmArgs p) {
     if (kt + NBUF - 1 < nk) issue_loads((u + NBUF - 1) % NBUF);
     compute(u);
   };
+  if constexpr (ROT) {
+    // Rotated loop for the large tiles, whose workgroup has a compute unit to itself (nobody else fills the
+    // gap a barrier leaves): the barrier that hands over tile kt+1 sits BEFORE the last quarter of tile kt's
+    // multiplies, whose operands are in registers by then, and the first operand reads of tile kt+1 are issued
+    // in front of that quarter.  The matrix pipeline therefore has a quarter's multiplies to chew on while the
+    // barrier, the reads' latency and the issue of the next tile's loads pass.  Every wait stands behind a
+    // quarter's multiplies that were issued after the reads it waits for, and nothing is in flight at the loop
+    // edge.  Order of additions per accumulator: as in the plain loop (same results bit for bit).
+    static_assert(NBUF == 2, "the rotated loop keeps two tiles in LDS");
+    uint4_t fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+    issue_loads(0);
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    if (1 < nk) issue_loads(1);
+    read_frags(0, 0, fa0, fb0);
+    asm volatile("s_waitcnt lgkmcnt(0)");
+    auto body = [&](int kt, int u) {
+      read_frags(u, 1, fa1, fb1);
+      multiply(fa0, fb0);
+      asm volatile("s_waitcnt lgkmcnt(0)");
+      read_frags(u, 2, fa0, fb0);
+      multiply(fa1, fb1);
+      asm volatile("s_waitcnt lgkmcnt(0)");
+      read_frags(u, 3, fa1, fb1);
+      multiply(fa0, fb0);
+      // all of tile kt is in registers; tile kt+1 (the only loads outstanding) must have landed
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      if (kt + 1 < nk) read_frags(u ^ 1, 0, fa0, fb0);
+      multiply(fa1, fb1);
+      if (kt + 2 < nk) issue_loads(u);
+      asm volatile("s_waitcnt lgkmcnt(0)");
+    };
+    int kt0 = 0;
+    for (; kt0 + 2 <= nk; kt0 += 2) {
+      body(kt0, 0);
+      body(kt0 + 1, 1);
+    }
+    if (kt0 < nk) body(kt0, 0);
+    __syncthreads();   // the epilogue stages through the operand buffers: every wave is done reading them
+  } else {
 #pragma unroll
-  for (int s = 0; s < NBUF - 1; ++s)
-    if (s < nk) issue_loads(s);
-  int kt0 = 0;
-  for (; kt0 + NBUF <= nk; kt0 += NBUF) {
+    for (int s = 0; s < NBUF - 1; ++s)
+      if (s < nk) issue_loads(s);
+    int kt0 = 0;
+    for (; kt0 + NBUF <= nk; kt0 += NBUF) {
 #pragma unroll
-    for (int u = 0; u < NBUF; ++u) step(kt0 + u, u);
+      for (int u = 0; u < NBUF; ++u) step(kt0 + u, u);
+    }
+#pragma unroll
+    for (int u = 0; u < NBUF - 1; ++u)
+      if (kt0 + u < nk) step(kt0 + u, u);
   }
-#pragma unroll
-  for (int u = 0; u < NBUF - 1; ++u)
-    if (kt0 + u < nk) step(kt0 + u, u);
 
   finish_tile<T, MODE, WM, WN, TM, TN>(p, acc, reinterpret_cast<float*>(lds), tid, m0, n0, tile_m);
 }
@@ -1431,19 +1485,25 @@ int launch_cfg(Context* ctx, IgemmArgs& a, double flops) {
                   flops, 0, conv_bytes<MODE>(a, sizeof(T)));
 }
 
-template <int MODE, int WM, int WN, int TM, int TN, int NBUF>
+template <int MODE, int WM, int WN, int TM, int TN, int NBUF, int ROT = 0>
 int launch_cfg2(Context* ctx, IgemmArgs& a, double flops) {
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
   static const std::string name = std::string("igemm2_kernel<bf16,") + (MODE == kFwd ? "fwd," : "dgrad,") +
-                                  std::to_string(BM) + "x" + std::to_string(BN) + "," + std::to_string(NBUF) + "buf>";
+                                  std::to_string(BM) + "x" + std::to_string(BN) + "," + std::to_string(NBUF) + "buf" +
+                                  (WM * WN == 8 ? ",8w" : "") + (ROT ? ",rot>" : ">");
   a.tiles_m = (a.gemm_m + BM - 1) / BM;
   a.tiles_n = (a.gemm_n + BN - 1) / BN;
+  static const int group_env = [] {
+    const char* e = getenv("TCH_IGEMM_GROUP_ROWS");
+    return e ? atoi(e) : -1;
+  }();
+  a.group_rows = group_env >= 0 ? group_env : (a.tiles_n > 8 ? 4 : 0);
   int64_t wgs = static_cast<int64_t>(a.tiles_m) * a.tiles_n;
   if (wgs <= 0 || wgs > 0x7fffffff) {
     set_error("igemm: grid out of range");
     return -22;
   }
-  return launch(ctx, igemm2_kernel<MODE, WM, WN, TM, TN, NBUF>, dim3(static_cast<unsigned>(wgs)), dim3(WM * WN * 64), a,
+  return launch(ctx, igemm2_kernel<MODE, WM, WN, TM, TN, NBUF, ROT>, dim3(static_cast<unsigned>(wgs)), dim3(WM * WN * 64), a,
                 name.c_str(), flops, 0, conv_bytes<MODE>(a, 2));
 }
 
@@ -1501,6 +1561,15 @@ int launch_mode(Context* ctx, IgemmArgs& a, int tile_cfg, double flops) {
       if (setting != 0 && patch_kernel_fits<MODE>(a)) return launch_cfg3<MODE, 1, 3>(ctx, a, flops);
       tile_cfg = 1;
     }
+    // 9 / 10: 256 x 256 on eight wavefronts (128 x 64 each), two LDS tiles in flight, plain / rotated loop: for
+    // products with a thousand such tiles or more (measured on 65 536 x 4096 x 4096: 1.13-1.21 PFLOP/s rotated,
+    // 1.02 plain, 0.82-0.91 for 128 x 128; four wavefronts of 128 x 128 each: 0.99-1.05, and slower than 128 x 128
+    // on every layer of the three models, like this one)
+    if (tile_cfg == 9 || tile_cfg == 10) {
+      if (setting != 0 && in_c % kStep2 == 0 && a.R * a.S <= 32)
+        return tile_cfg == 9 ? launch_cfg2<MODE, 2, 4, 4, 2, 2>(ctx, a, flops) : launch_cfg2<MODE, 2, 4, 4, 2, 2, 1>(ctx, a, flops);
+      tile_cfg = 0;
+    }
     // 6 / 7: tilings 1 / 2 with two LDS tiles in flight instead of three (48 / 32 KB of LDS: three or four
     // workgroups per CU, which the memory-bound data gradients of the large feature maps prefer)
     if (tile_cfg == 6 || tile_cfg == 7) {
@@ -1518,6 +1587,7 @@ int launch_mode(Context* ctx, IgemmArgs& a, int tile_cfg, double flops) {
   }
   if (tile_cfg == 5) tile_cfg = 1;
   if (tile_cfg == 6 || tile_cfg == 7) tile_cfg -= 5;
+  if (tile_cfg == 9 || tile_cfg == 10) tile_cfg = 0;
   switch (tile_cfg) {
     case 0:
       return launch_cfg<T, MODE, 2, 2, 2, 2>(ctx, a, flops);  // 128 x 128
@@ -1536,10 +1606,28 @@ double conv_flops(const ConvShape& s, int Ho, int Wo) {
 }
 
 // rows of the workgroup tile of a tiling number (5 = the 3x3 patch kernel, or tiling 1 where it does not fit)
-int tile_rows(int tile_cfg) { return (tile_cfg == 5 || tile_cfg == 6) ? 128 : tile_cfg >= 2 ? 64 : 128; }
+int tile_rows(int tile_cfg) {
+  if (tile_cfg == 9 || tile_cfg == 10) return 256;
+  return (tile_cfg == 5 || tile_cfg == 6) ? 128 : tile_cfg >= 2 ? 64 : 128;
+}
 
 int64_t tiles_for(int m, int n, int bm, int bn) {
   return static_cast<int64_t>((m + bm - 1) / bm) * ((n + bn - 1) / bn);
+}
+
+// Whether the 256 x 256 tiling (10) is worth asking for: the kernel it needs is at hand (bf16, reduction in whole
+// 64-channel steps, few taps) and the product has at least four full rounds of such tiles.
+bool wants_huge_tile(int dtype, int gemm_m, int gemm_n, int in_c, int taps) {
+  return dtype == kBF16 && in_c % 64 == 0 && taps <= 32 && igemm2_setting() != 0 &&
+         tiles_for(gemm_m, gemm_n, 256, 256) >= 1024;
+}
+
+// The tiling that runs when `tile_cfg` is asked for: the 256 x 256 tilings exist for the direct-to-LDS kernel only
+// and stand for 128 x 128 elsewhere (the statistics' row tiles follow the tiling that runs).
+int effective_tile(int tile_cfg, int dtype, int in_c, int taps) {
+  if ((tile_cfg == 9 || tile_cfg == 10) && !(dtype == kBF16 && in_c % 64 == 0 && taps <= 32 && igemm2_setting() != 0))
+    return 0;
+  return tile_cfg;
 }
 
 // Enough workgroups to give each of the 256 CUs some, with bigger tiles as
@@ -1643,7 +1731,12 @@ int conv2d_fwd(Context* ctx, int dtype, const ConvShape& s, const void* x, const
   a.k_per_split = (a.gemm_k + 31) / 32 * 32;
   a.div_plane = FastDiv(a.Ho * a.Wo);
   a.div_width = FastDiv(a.Wo);
-  if (tile_cfg < 0) tile_cfg = pick_tile(a.gemm_m, a.gemm_n, 1);
+  if (tile_cfg < 0) {
+    tile_cfg = pick_tile(a.gemm_m, a.gemm_n, 1);
+    // statistics are sized by the caller for the heuristic's row tiles: leave those launches alone
+    if (!bn_partial && wants_huge_tile(dtype, a.gemm_m, a.gemm_n, s.C, s.R * s.S)) tile_cfg = 10;
+  }
+  tile_cfg = effective_tile(tile_cfg, dtype, s.C, s.R * s.S);
   const int row_tiles = (a.gemm_m + tile_rows(tile_cfg) - 1) / tile_rows(tile_cfg);
   const bool in_kernel = finalize && row_tiles <= kBnFinalizeInKernelTiles;
   if (in_kernel) bind_finalize(a, finalize);
@@ -1656,19 +1749,19 @@ int conv2d_fwd(Context* ctx, int dtype, const ConvShape& s, const void* x, const
 }
 
 int conv2d_fwd_stat_rows(const ConvShape& s, int dtype, int tile_cfg) {
-  (void)dtype;
   int Ho, Wo;
   conv_output_hw(s, &Ho, &Wo);
   const int gemm_m = s.N * Ho * Wo;
   if (tile_cfg < 0) tile_cfg = pick_tile(gemm_m, s.K, 1);
+  tile_cfg = effective_tile(tile_cfg, dtype, s.C, s.R * s.S);
   const int bm = tile_rows(tile_cfg);
   return (gemm_m + bm - 1) / bm;
 }
 
 int conv2d_dgrad_stat_rows(const ConvShape& s, int dtype, int tile_cfg) {
-  (void)dtype;
   const int gemm_m = s.N * s.H * s.W;
   if (tile_cfg < 0) tile_cfg = pick_tile(gemm_m, s.C, 1);
+  tile_cfg = effective_tile(tile_cfg, dtype, s.K, s.R * s.S);
   const int bm = tile_rows(tile_cfg);
   return (gemm_m + bm - 1) / bm;
 }
@@ -1702,7 +1795,11 @@ int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, co
   // 1x1 stride 1: dy is a dense [pixels][K] matrix in the same pixel order as dx
   a.div_plane = FastDiv(s.H * s.W);
   a.div_width = FastDiv(s.W);
-  if (tile_cfg < 0) tile_cfg = pick_tile(a.gemm_m, a.gemm_n, 1);
+  if (tile_cfg < 0) {
+    tile_cfg = pick_tile(a.gemm_m, a.gemm_n, 1);
+    if (!bn && wants_huge_tile(dtype, a.gemm_m, a.gemm_n, s.K, s.R * s.S)) tile_cfg = 10;
+  }
+  tile_cfg = effective_tile(tile_cfg, dtype, s.K, s.R * s.S);
   const BnFinalize* finalize = bn ? bn->finalize : nullptr;
   const int row_tiles = (a.gemm_m + tile_rows(tile_cfg) - 1) / tile_rows(tile_cfg);
   const bool in_kernel = finalize && row_tiles <= kBnFinalizeInKernelTiles;
