@@ -37,8 +37,10 @@ def test_shutdown_under_blocked_waiters(tmp_path, sanitizer):
     link = subprocess.run([hipcc, f"-fsanitize={sanitizer}", "-fno-gpu-sanitize"] + objs + ["-o", exe, "-lpthread", "-lrt", "-lhsa-runtime64"],
                           stdout=subprocess.PIPE, stderr=subprocess.STDOUT)
     assert link.returncode == 0, link.stdout.decode()[-3000:]
-    env = dict(os.environ, TSAN_OPTIONS="halt_on_error=1 exitcode=66", ASAN_OPTIONS="detect_leaks=0 exitcode=67")
-    env.pop("LD_PRELOAD", None)
+    # the environment is passed on as it is; verify_asan_link_order=0 lets the sanitizer runtime start behind
+    # whatever else the loader was asked to load first
+    env = dict(os.environ, TSAN_OPTIONS="halt_on_error=1 exitcode=66",
+               ASAN_OPTIONS="detect_leaks=0 exitcode=67 verify_asan_link_order=0")
     run = subprocess.run([exe, "20"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=240, env=env)
     text = run.stdout.decode()
     assert run.returncode == 0, text[-4000:]
