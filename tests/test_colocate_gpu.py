@@ -9,6 +9,7 @@ import os
 import random
 import subprocess
 import sys
+import time
 
 import pytest
 import torch
@@ -94,6 +95,73 @@ def test_pool_on_hip_vmm_matches_cpu_model(clean_runtime):
         assert float(b2[-1].item()) == 2.0
         del a, b2, c
         assert L.tch_cuda_memory_pool_train_usage(0) == 0
+    finally:
+        torch.cuda.synchronize()
+        L.tch_pool_shutdown(0)
+
+
+class _RawBytes:
+    """A span of device memory for torch to wrap without copying (CUDA array interface)."""
+
+    def __init__(self, ptr, nbytes):
+        self.__cuda_array_interface__ = {"shape": (nbytes,), "typestr": "|u1", "data": (ptr, False), "version": 2,
+                                         "strides": None}
+
+
+def test_pool_at_the_size_of_the_part(clean_runtime):
+    """A pool of 256 GB (what a 288 GB part leaves to the two tenants) in 128 MB pages: a trace of allocations
+    that fills 192 GB of it lands at the offsets the CPU model of the same pool gives, every block is real memory
+    (its first and last megabyte are written and read back), and handing everything back unmaps every page."""
+    L = lib()
+    tc = clean_runtime
+    torch.cuda.init()
+    GB = 1024 * MB
+    page = 128 * MB
+    sizes = [16 * GB, 40 * MB, 24 * GB, 3 * MB, 32 * GB, 8 * GB, 512, 48 * GB, 20 * GB, 100_000, 36 * GB, 16 * GB]
+
+    def run():
+        ptrs, offs = [], []
+        for i, n in enumerate(sizes):
+            p = L.tch_pool_malloc(n, 0, None)
+            assert p, (i, n, L.tch_host_last_error())
+            ptrs.append(p)
+            offs.append(L.tch_pool_offset_of(0, ctypes.c_void_p(p)))
+            if i in (2, 6):                      # holes in the middle: the next requests must find them
+                L.tch_pool_free(ptrs[i - 1], 0, 0, None)
+                ptrs[i - 1] = None
+        return ptrs, offs
+
+    assert L.tch_pool_init_ex(0, 256 * GB, 0, page, 0) == 0
+    cpu_ptrs, cpu_offs = run()
+    L.tch_pool_shutdown(0)
+    t0 = time.perf_counter()
+    assert L.tch_pool_init_ex(0, 256 * GB, 1, page, 0) == 0, L.tch_host_last_error()
+    init_s = time.perf_counter() - t0
+    try:
+        assert L.tch_cuda_memory_pool_nbytes(0) == 256 * GB and L.tch_pool_page_bytes(0) == page
+        ptrs, offs = run()
+        assert offs == cpu_offs
+        used = L.tch_cuda_memory_pool_train_all_usage(0)
+        assert used >= 190 * GB
+        for i, (p, n) in enumerate(zip(ptrs, sizes)):
+            if p is None or n < 2 * MB:
+                continue
+            for start in (0, n - MB):
+                view = torch.as_tensor(_RawBytes(p + start, MB), device="cuda:0").view(torch.float32)
+                view.fill_(float(i + 1))
+                assert float(view[-1].item()) == float(i + 1) and float(view[0].item()) == float(i + 1)
+        torch.cuda.synchronize()
+        for p in ptrs:
+            if p is not None:
+                L.tch_pool_free(p, 0, 0, None)
+        t0 = time.perf_counter()
+        freed = L.tch_cuda_memory_pool_free_train_local(0)
+        free_ms = (time.perf_counter() - t0) * 1e3
+        c = (ctypes.c_uint64 * 6)()
+        L.tch_pool_counters(0, c)
+        print(f"256 GB pool in 128 MB pages: init {init_s:.2f} s, {used / GB:.1f} GB in use, handed back {freed / GB:.1f} GB "
+              f"in {free_ms:.1f} ms ({int(c[3])} pages unmapped in {L.tch_pool_unmap_calls(0)} driver calls)", flush=True)
+        assert freed == used and L.tch_cuda_memory_pool_train_all_usage(0) == 0 and int(c[5]) == 0
     finally:
         torch.cuda.synchronize()
         L.tch_pool_shutdown(0)
