@@ -29,6 +29,14 @@ METRIC = "ResNet-152 bf16 bs64 train images/sec on 1 GPU; conv MFMA util %"
 # driver call per page on the way out: 9 GB take 68 ms there, 18 ms in 128 MB pages).
 HANDOVER_POOL_GB = 256
 HANDOVER_PAGE_MB = 128
+# Average launch duration of the same kernels INSIDE the step (both lanes sharing the chip), from the rocprofv3
+# --kernel-trace --stats run of this file summarised in the same profile: the one-launch-at-a-time replay below
+# is what this file can measure itself, the in-step figure is what the trace shows.
+PROFILE_FILE = "profiles/resnet152_bf16_bs64_step_kernel_stats_and_traffic.txt"
+MEASURED_IN_STEP_US = {
+    "wgrad_kernel<bf16,128x128>": 35.52,
+    "igemm2_kernel<bf16,dgrad,128x64,2buf>": 51.56,
+}
 MEASURED_TRAFFIC_MIB = {
     "wgrad_kernel<bf16,128x128>": 31.79 + 13.77,
     "igemm2_kernel<bf16,dgrad,128x128,2buf>": 67.94 + 32.72,
@@ -39,6 +47,43 @@ MEASURED_TRAFFIC_MIB = {
     "bn_apply_kernel<bf16,bwd>": 72.04 + 34.61,
     "bn_apply_kernel<bf16,fwd>": 54.69 + 36.09,
 }
+
+
+def grouped_wgrad_step(batch, x, y, steps, warmup, tile_cache):
+    """The same step with the weight gradients of a whole stage as ONE launch over a table
+    (`ResNetEngine(group_wgrad=True)`) instead of one launch (+ one split reduction) per layer: what the grouped
+    kernel does to the weight gradients' kernel time, and what it does to the step."""
+    import torch
+    from sirius_amd.resnet import ResNetEngine
+    eng = ResNetEngine((3, 8, 36, 3), 1000, 64, dtype=torch.bfloat16, image_size=224, lr=0.1, momentum=0.9,
+                       weight_decay=1e-4, autotune=True, group_wgrad=True, wgrad_group_blocks=0, wgrad_group_wgs=1024)
+    eng._tile_cache.update(tile_cache)          # the tilings the headline run measured
+    eng.init_kaiming(seed=0)
+    for _ in range(warmup):
+        eng.forward_backward(x, y)
+        eng.optimizer_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        eng.forward_backward(x, y)
+        eng.optimizer_step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    plan = eng.plan(batch)
+    rows = eng.ctx.profile(plan.prog, 1) + eng.ctx.profile(eng._opt_prog, 1)
+    wg = [r for r in rows if r["name"].startswith(("wgrad_", "splitk_reduce"))]
+    conv = [r for r in rows if r["name"].startswith(("igemm_kernel", "igemm2_kernel", "igemm3_kernel", "wgrad_"))]
+    grp = [r for r in rows if r["name"].startswith("wgrad_group_kernel<bf16,128x128>")]
+    res = {"ms_per_step": ms, "images_per_s": batch / (ms * 1e-3), "launches_per_step": len(plan.prog) + len(eng._opt_prog),
+           "wgrad_and_reduce_kernel_ms": sum(r["total_ms"] for r in wg),
+           "conv_mfma_util": sum(r["work"] for r in conv) / (sum(r["total_ms"] for r in conv) * 1e-3) / PEAK_BF16_FLOPS,
+           "wgrad_group_128x128_tflops": (sum(r["work"] for r in grp) / (sum(r["total_ms"] for r in grp) * 1e-3) / 1e12) if grp else None,
+           "groups": len(plan.wgrad_groups),
+           "layers_without_partial_filters": sum(sum(1 for sp in g["splits"] if sp == 1) for g in plan.wgrad_groups),
+           "layers_grouped": sum(len(g["splits"]) for g in plan.wgrad_groups)}
+    del eng, plan
+    torch.cuda.empty_cache()
+    return res
 
 
 def cpu_model():
@@ -327,6 +372,7 @@ def main():
     ap.add_argument("--only-swin", action="store_true", help="run the Swin-B step measurement alone (for profiling it)")
     ap.add_argument("--no-autotune", action="store_true", help="keep the library's tiling heuristic")
     ap.add_argument("--no-overlap", action="store_true", help="record weight gradients on the main lane (one stream)")
+    ap.add_argument("--no-grouped", action="store_true", help="skip the extra run of the step with grouped weight gradients")
     ap.add_argument("--group-wgrad", action="store_true", help="grouped weight-gradient launches instead of one per layer")
     ap.add_argument("--wgrad-group-blocks", type=int, default=None, help="bottleneck blocks per grouped weight-gradient launch (0: a stage)")
     ap.add_argument("--wgrad-group-wgs", type=int, default=None, help="workgroups a grouped weight-gradient launch aims for")
@@ -427,6 +473,13 @@ def main():
         "launches_per_step": top["launches"] // reps,
         "share_of_step_kernel_time": top["total_ms"] / reps / total_ms,
     }
+    if top["name"] in MEASURED_IN_STEP_US:
+        in_step_s = MEASURED_IN_STEP_US[top["name"]] * 1e-6
+        roofline["in_step"] = {"avg_launch_us": MEASURED_IN_STEP_US[top["name"]],
+                               "achieved": (nbytes if hbm_bound else flops) / in_step_s / (1e9 if hbm_bound else 1e12),
+                               "frac": (nbytes if hbm_bound else flops) / in_step_s / peak,
+                               "source": PROFILE_FILE + " (rocprofv3 --kernel-trace --stats of this file; the kernel shares the "
+                                         "chip with the other lane there, the replay above runs it alone)"}
     breakdown = [{"kernel": r["name"], "ms_per_step": round(r["total_ms"] / reps, 4), "launches": r["launches"] // reps,
                   ("GB/s" if r["work_is_bytes"] else "TFLOP/s"):
                       round(r["work"] / (r["total_ms"] * 1e-3) / (1e9 if r["work_is_bytes"] else 1e12), 2)
@@ -460,6 +513,11 @@ def main():
         "kernel_ms_per_step": total_ms,
         "breakdown": breakdown,
     }
+    if not args.no_grouped and not args.group_wgrad:
+        try:
+            out["grouped_wgrad"] = grouped_wgrad_step(B, x, y, max(4, args.steps // 2), 2, eng._tile_cache)
+        except Exception as e:
+            out["grouped_wgrad"] = {"error": repr(e)}
     if args.cpu_steps > 0:
         out["cpu_baseline"] = cpu_baseline(B, args.cpu_steps)
     else:
