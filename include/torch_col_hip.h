@@ -132,6 +132,14 @@ int tch_context_get_cu_limit(tch_context* ctx);
 int tch_conv2d_fwd(tch_context* ctx, int dtype, const void* x, const void* w, void* y, const void* add,
                    const void* mask, const float* bias, int out_f32, int N, int H, int W, int C, int K, int R, int S,
                    int stride, int pad, int tile_cfg, int c_logical);
+/* Convolution -> inference-mode BatchNorm (-> + residual) (-> ReLU) as ONE launch: y = relu?(conv(x, w) * scale[K]
+ * + shift[K] + residual?), everything after the convolution applied to the fp32 accumulators in the epilogue.
+ * scale / shift as tch_bn_eval_coef leaves them (model.eval(): F.batch_norm with training=False); what an
+ * inference graph compiler makes of torchvision's conv -> bn -> relu triples, and what the batch-1 ResNet-152
+ * requests of the colocated inference side run.  scale, shift, residual may be NULL. */
+int tch_conv2d_fwd_affine(tch_context* ctx, int dtype, const void* x, const void* w, void* y, const float* scale,
+                          const float* shift, const void* residual, int relu, int N, int H, int W, int C, int K, int R,
+                          int S, int stride, int pad, int tile_cfg, int c_logical);
 /* The convolution that feeds a BatchNorm (torchvision's conv -> bn pairs, train/resnet152.py:22): y as
  * above (no bias / addend), and per (row tile, output channel) the sum and the sum of squares of y as
  * stored: bn_partial[(tile * K + k) * 2 + {0,1}], tch_conv2d_fwd_stat_rows(...) row tiles.  Saves the

@@ -187,6 +187,13 @@ int tch_conv2d_fwd(tch_context* ctx, int dtype, const void* x, const void* w, vo
                     tile_cfg);
 }
 
+int tch_conv2d_fwd_affine(tch_context* ctx, int dtype, const void* x, const void* w, void* y, const float* scale,
+                          const float* shift, const void* residual, int relu, int N, int H, int W, int Cc, int K, int R,
+                          int S, int stride, int pad, int tile_cfg, int c_logical) {
+  return conv2d_fwd(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad, c_logical), x, w, y, residual, nullptr, shift, 0,
+                    tile_cfg, nullptr, nullptr, scale, relu);
+}
+
 int tch_conv2d_fwd_bnstats(tch_context* ctx, int dtype, const void* x, const void* w, void* y, int N, int H, int W,
                            int Cc, int K, int R, int S, int stride, int pad, int tile_cfg, int c_logical,
                            float* bn_partial) {

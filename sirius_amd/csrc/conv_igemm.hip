@@ -55,6 +55,8 @@ struct IgemmArgs {
   const void* add;    // optional addend, laid out like out (FWD/DGRAD)
   const void* mask;   // optional: addend counts only where mask > 0
   const float* bias;  // optional per-column bias (FWD)
+  const float* scale; // optional per-column factor applied before the bias (FWD: an inference-mode BatchNorm folded in)
+  int relu_out;       // FWD: the stored output is max(0, .) of everything above
   float* dbias;       // WGRAD, optional: column sums of dy (the gradient of that bias), [splits][K] partials or final
   float* stats;       // optional: per (row tile, column) pair of sums over the stored output (see finish_tile)
   const void* bn_mask;      // DGRAD with stats, optional: the stored output is zeroed where bn_mask <= 0
@@ -356,6 +358,10 @@ __device__ inline void finish_tile(const IgemmArgs& p, f32x16_t (&acc)[TM][TN], 
     const int row = m0 + tr, col = n0 + tc;
     if (row >= p.gemm_m || col >= p.gemm_n) return;
     const int64_t idx = static_cast<int64_t>(row) * p.gemm_n + col;
+    if (MODE == kFwd && p.scale) {
+#pragma unroll
+      for (int e = 0; e < E; ++e) v[e] *= p.scale[col + e];
+    }
     if (MODE == kFwd && p.bias) {
 #pragma unroll
       for (int e = 0; e < E; ++e) v[e] += p.bias[col + e];
@@ -376,6 +382,10 @@ __device__ inline void finish_tile(const IgemmArgs& p, f32x16_t (&acc)[TM][TN], 
       }
 #pragma unroll
       for (int e = 0; e < E; ++e) v[e] += a[e];
+    }
+    if (MODE == kFwd && p.relu_out) {
+#pragma unroll
+      for (int e = 0; e < E; ++e) v[e] = fmaxf(v[e], 0.f);
     }
     if (p.out_f32) {
       store_floats<E>(static_cast<float*>(p.out) + idx, v);
@@ -1708,9 +1718,12 @@ void bind_finalize(IgemmArgs& a, const BnFinalize* f) {
 
 int conv2d_fwd(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* w, void* y, const void* add,
                const void* mask, const float* bias, int out_f32, int tile_cfg, float* bn_partial,
-               const BnFinalize* finalize) {
+               const BnFinalize* finalize, const float* scale, int relu_out) {
   IgemmArgs a{};
   if (int rc = fill_common(a, s, dtype)) return rc;
+  TCH_CHECK_ARG(!((scale || relu_out) && bn_partial), "conv2d_fwd: statistics are taken of the plain convolution output");
+  a.scale = scale;
+  a.relu_out = relu_out ? 1 : 0;
   TCH_CHECK_ARG(x && w && y, "conv2d_fwd: null tensor");
   TCH_CHECK_ARG(!(bn_partial && out_f32), "conv2d_fwd: statistics are taken of outputs stored in the compute type");
   TCH_CHECK_ARG(!finalize || (bn_partial && check_finalize(finalize, true)), "conv2d_fwd: incomplete BatchNorm finalize operands");

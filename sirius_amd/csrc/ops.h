@@ -40,7 +40,7 @@ struct BnFinalize {
 // conv_igemm.hip
 int conv2d_fwd(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* w, void* y, const void* add,
                const void* mask, const float* bias, int out_f32, int tile_cfg, float* bn_partial = nullptr,
-               const BnFinalize* finalize = nullptr);
+               const BnFinalize* finalize = nullptr, const float* scale = nullptr, int relu_out = 0);
 // rows of partial statistics conv2d_fwd writes for this shape and tiling (one per row tile)
 int conv2d_fwd_stat_rows(const ConvShape& s, int dtype, int tile_cfg);
 // The two reductions of a BatchNorm backward, taken in the epilogue of the data-gradient

@@ -171,6 +171,23 @@ def conv2d_fwd_stat_rows(x, K, R, S, stride, pad, tile_cfg=-1):
     return int(lib().tch_conv2d_fwd_stat_rows(dtype_code(x), N, H, W, C, K, R, S, stride, pad, tile_cfg))
 
 
+def conv2d_fwd_affine(ctx, x, w, y, stride, pad, scale=None, shift=None, residual=None, relu=False, tile_cfg=-1,
+                      c_logical=0):
+    """y = relu?(conv(x, w) * scale + shift + residual?) in one launch (inference-mode BatchNorm folded into the
+    convolution's epilogue)."""
+    N, H, W, C = x.shape
+    K, R, S, C2 = w.shape
+    assert C == C2 and w.dtype == x.dtype == y.dtype
+    Ho, Wo = conv_out_hw(H, W, R, S, stride, pad)
+    assert tuple(y.shape) == (N, Ho, Wo, K)
+    for t in (scale, shift):
+        assert t is None or (t.dtype == torch.float32 and t.numel() == K)
+    assert residual is None or (residual.shape == y.shape and residual.dtype == y.dtype)
+    check(lib().tch_conv2d_fwd_affine(ctx.handle, dtype_code(x), _p(x), _p(w), _p(y), _p(scale), _p(shift), _p(residual),
+                                      int(relu), N, H, W, C, K, R, S, stride, pad, tile_cfg, c_logical),
+          "tch_conv2d_fwd_affine")
+
+
 def conv2d_fwd_bnstats(ctx, x, w, y, stride, pad, partial, tile_cfg=-1, c_logical=0):
     """conv2d_fwd that also leaves the per-row-tile BatchNorm sums of y in `partial`
     ([row tiles, K, 2] fp32); returns the number of row tiles."""

@@ -72,6 +72,9 @@ class ResNetEngine(EngineBase):
         # is 16.5-17.1 ms against 16.3 ms: the many short launches run in the gaps of the data-gradient chain,
         # which is the critical path, while a launch that fills the chip holds that chain up for as long as it runs
         # (also when it is capped to one workgroup per compute unit).
+        # fuse_eval_bn: the forward-only (inference) plan runs convolution + BatchNorm (+ residual) (+ ReLU) as one
+        # launch each instead of two
+        self.fuse_eval_bn = True
         self.group_wgrad = group_wgrad and overlap_wgrad
         self.wgrad_group_wgs, self.wgrad_group_blocks = wgrad_group_wgs, wgrad_group_blocks
         self.wgrad_group_max_wgs = wgrad_group_max_wgs
@@ -719,10 +722,17 @@ class ResNetEngine(EngineBase):
 
         def conv_bn(c, name, x, residual=None, relu=True):
             Ho, Wo = ops.conv_out_hw(x.shape[1], x.shape[2], c.k, c.k, c.stride, c.pad)
-            z, y = act(B, Ho, Wo, c.cout), act(B, Ho, Wo, c.cout)
-            ops.conv2d_fwd(ctx, x, self._w(c.name + ".weight"), z, c.stride, c.pad, c_logical=c.cin)
+            y = act(B, Ho, Wo, c.cout)
             o, ch = self._bn_off[name]
-            ops.bn_apply_fwd(ctx, z, y, self._eval_coef[2 * o:2 * o + 2 * ch], residual=residual, relu=relu)
+            coef = self._eval_coef[2 * o:2 * o + 2 * ch]
+            if self.fuse_eval_bn:
+                # the BatchNorm is a per-channel scale and shift here: applied to the accumulators in the epilogue
+                ops.conv2d_fwd_affine(ctx, x, self._w(c.name + ".weight"), y, c.stride, c.pad, scale=coef[:ch], shift=coef[ch:],
+                                      residual=residual, relu=relu, c_logical=c.cin)
+                return y
+            z = act(B, Ho, Wo, c.cout)
+            ops.conv2d_fwd(ctx, x, self._w(c.name + ".weight"), z, c.stride, c.pad, c_logical=c.cin)
+            ops.bn_apply_fwd(ctx, z, y, coef, residual=residual, relu=relu)
             return y
 
         plan.x_in = act(B, 3, S, S, dtype=torch.float32)

@@ -125,6 +125,42 @@ def test_conv_dgrad_residual(ctx, dtype):
     close(dx, ref, dtype, "conv dgrad + residual")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", [CONV_CASES[0], CONV_CASES[2], CONV_CASES[3], CONV_CASES[5], CONV_CASES[6], CONV_CASES[10]])
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 2, 5])
+def test_conv_fwd_with_inference_batchnorm_in_the_epilogue(ctx, dtype, case, tile_cfg):
+    """conv -> BatchNorm(eval) -> (+ residual) -> ReLU as one launch: scale, shift, residual and ReLU act on the
+    fp32 accumulators; against the oracle's convolution followed by the same arithmetic in fp32."""
+    from sirius_amd import ops
+    N, H, W, C, K, R, S, st, pad = case
+    g = _gen(23)
+    x = rnd((N, H, W, C), dtype, g)
+    w = rnd((K, R, S, C), dtype, g, (R * S * C) ** -0.5)
+    Ho, Wo = ops.conv_out_hw(H, W, R, S, st, pad)
+    res = rnd((N, Ho, Wo, K), dtype, g)
+    scale = torch.rand(K, generator=g) + 0.5
+    shift = torch.randn(K, generator=g)
+    conv = O.conv2d_fwd(x, w, st, pad)
+    for use_res, relu in ((False, True), (True, True), (True, False), (False, False)):
+        ref = conv * scale + shift + (res.float() if use_res else 0.0)
+        if relu:
+            ref = ref.clamp_min(0.0)
+        y = torch.full((N, Ho, Wo, K), -5.0, dtype=dtype, device="cuda")
+        ops.conv2d_fwd_affine(ctx, x.cuda(), w.cuda(), y, st, pad, scale=scale.cuda(), shift=shift.cuda(),
+                              residual=res.cuda() if use_res else None, relu=relu, tile_cfg=tile_cfg)
+        torch.cuda.synchronize()
+        close(y, ref, dtype, f"conv + affine (residual {use_res}, relu {relu})")
+        if relu:
+            assert float(y.float().min()) >= 0.0
+    # no scale, no shift: the plain convolution
+    y = torch.empty((N, Ho, Wo, K), dtype=dtype, device="cuda")
+    y2 = torch.empty_like(y)
+    ops.conv2d_fwd_affine(ctx, x.cuda(), w.cuda(), y, st, pad, tile_cfg=tile_cfg)
+    ops.conv2d_fwd(ctx, x.cuda(), w.cuda(), y2, st, pad, tile_cfg=tile_cfg)
+    torch.cuda.synchronize()
+    assert torch.equal(y, y2)
+
+
 @pytest.mark.parametrize("shape", [(1000, 128, 520), (2048, 192, 1024), (300, 64, 72), (1100, 64, 1200), (2900, 64, 2320)])
 def test_huge_tile_equals_the_128_tile(ctx, shape):
     """The 256 x 256 tilings (plain and rotated loop, eight wavefronts) on products with several such tiles and
