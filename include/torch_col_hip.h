@@ -150,10 +150,14 @@ int tch_conv2d_fwd_bnstats(tch_context* ctx, int dtype, const void* x, const voi
 int tch_conv2d_fwd_stat_rows(int dtype, int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
                              int tile_cfg);
 /* dx[N,H,W,C] = conv_transpose(dy[N,Ho,Wo,K], w) (+ add, optionally gated by mask > 0).
- * wt is the filter TRANSPOSED to [C][R][S][K] (tch_filter_transpose_batched). */
+ * wt is the filter TRANSPOSED to [C][R][S][K] (tch_filter_transpose_batched).
+ * add_stride (here and in the two forms below): 1 = `add` is laid out like dx; 2 = `add` is [N, ceil(H/2),
+ * ceil(W/2), C], the values of the even (h, w) of dx's grid, and counts there only: the data gradient of a
+ * stride-2 1x1 convolution (a ResNet downsample branch) is non-zero at those pixels alone, so it is computed on its
+ * own small grid (as the stride-1 data gradient over dy's pixels) and never blown up to dx's. */
 int tch_conv2d_dgrad(tch_context* ctx, int dtype, const void* dy, const void* wt, void* dx, const void* add,
                      const void* mask, int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
-                     int tile_cfg, int c_logical);
+                     int tile_cfg, int c_logical, int add_stride);
 /* The same where dx is the gradient behind a BatchNorm (+ReLU) whose input is bn_x (laid out like dx) and
  * whose ReLU output is bn_mask (may be NULL: no ReLU): dx is zeroed where bn_mask <= 0 before it is stored
  * and the epilogue leaves, per row tile and channel, sum(dx) and sum(dx * (bn_x - mean) * invstd) at
@@ -162,7 +166,7 @@ int tch_conv2d_dgrad(tch_context* ctx, int dtype, const void* dy, const void* wt
 int tch_conv2d_dgrad_bnsums(tch_context* ctx, int dtype, const void* dy, const void* wt, void* dx, const void* add,
                             const void* mask, int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
                             int tile_cfg, int c_logical, const void* bn_mask, const void* bn_x, const float* bn_mean,
-                            const float* bn_invstd, float* bn_partial);
+                            const float* bn_invstd, float* bn_partial, int add_stride);
 int tch_conv2d_dgrad_stat_rows(int dtype, int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
                                int tile_cfg);
 /* Convolution + the whole front half of the BatchNorm next to it, in one call: the sums as above, and the
@@ -178,7 +182,7 @@ int tch_conv2d_dgrad_bn(tch_context* ctx, int dtype, const void* dy, const void*
                         const void* mask, int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
                         int tile_cfg, int c_logical, const void* bn_mask, const void* bn_x, const float* bn_mean,
                         const float* bn_invstd, float* bn_partial, int* counters, const float* gamma, float* dgamma,
-                        float* dbeta, int accumulate, float* coef);
+                        float* dbeta, int accumulate, float* coef, int add_stride);
 /* y = relu?(x * scale + shift (+ residual)), coef = scale[C], shift[C];  dx = c0 * g + c1 * x + c2, coef = [3][C] */
 int tch_bn_apply_fwd(tch_context* ctx, int dtype, const void* x, void* y, const void* residual, int relu, int64_t rows,
                      int C, const float* coef);

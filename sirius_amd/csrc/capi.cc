@@ -220,17 +220,18 @@ int tch_bn_fwd_train_partials(tch_context* ctx, int dtype, const void* x, void* 
 
 int tch_conv2d_dgrad(tch_context* ctx, int dtype, const void* dy, const void* w, void* dx, const void* add,
                      const void* mask, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad,
-                     int tile_cfg, int c_logical) {
-  return conv2d_dgrad(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad, c_logical), dy, w, dx, add, mask, tile_cfg);
+                     int tile_cfg, int c_logical, int add_stride) {
+  return conv2d_dgrad(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad, c_logical), dy, w, dx, add, mask, tile_cfg,
+                      nullptr, add_stride);
 }
 
 int tch_conv2d_dgrad_bnsums(tch_context* ctx, int dtype, const void* dy, const void* w, void* dx, const void* add,
                             const void* mask, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad,
                             int tile_cfg, int c_logical, const void* bn_mask, const void* bn_x, const float* bn_mean,
-                            const float* bn_invstd, float* bn_partial) {
+                            const float* bn_invstd, float* bn_partial, int add_stride) {
   BnBwdSums bn{bn_mask, bn_x, bn_mean, bn_invstd, bn_partial, nullptr};
   return conv2d_dgrad(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad, c_logical), dy, w, dx, add, mask, tile_cfg,
-                      &bn);
+                      &bn, add_stride);
 }
 
 int tch_conv2d_dgrad_stat_rows(int dtype, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad,
@@ -354,11 +355,11 @@ int tch_conv2d_dgrad_bn(tch_context* ctx, int dtype, const void* dy, const void*
                         const void* mask, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad,
                         int tile_cfg, int c_logical, const void* bn_mask, const void* bn_x, const float* bn_mean,
                         const float* bn_invstd, float* bn_partial, int* counters, const float* gamma, float* dgamma,
-                        float* dbeta, int accumulate, float* coef) {
+                        float* dbeta, int accumulate, float* coef, int add_stride) {
   BnFinalize fin{counters, gamma, nullptr, nullptr, nullptr, dgamma, dbeta, coef, 0.f, 0.f, accumulate};
   BnBwdSums bn{bn_mask, bn_x, bn_mean, bn_invstd, bn_partial, &fin};
   return conv2d_dgrad(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad, c_logical), dy, w, dx, add, mask, tile_cfg,
-                      &bn);
+                      &bn, add_stride);
 }
 
 int tch_bn_apply_fwd(tch_context* ctx, int dtype, const void* x, void* y, const void* residual, int relu, int64_t rows,

@@ -54,6 +54,8 @@ struct IgemmArgs {
   void* out;          // FWD: y        DGRAD: dx       WGRAD: dw (fp32) or split partials
   const void* add;    // optional addend, laid out like out (FWD/DGRAD)
   const void* mask;   // optional: addend counts only where mask > 0
+  int add_sub;        // DGRAD: 1 = `add` lives on the stride-2 subsampled pixel grid [N, ceil(H/2), ceil(W/2), C] and
+                      // counts at the even (h, w) only (the data gradient of a strided 1x1 convolution, kept compact)
   const float* bias;  // optional per-column bias (FWD)
   const float* scale; // optional per-column factor applied before the bias (FWD: an inference-mode BatchNorm folded in)
   int relu_out;       // FWD: the stored output is max(0, .) of everything above
@@ -366,9 +368,19 @@ __device__ inline void finish_tile(const IgemmArgs& p, f32x16_t (&acc)[TM][TN], 
 #pragma unroll
       for (int e = 0; e < E; ++e) v[e] += p.bias[col + e];
     }
-    if (p.add) {
+    bool add_here = p.add != nullptr;
+    int64_t add_idx = idx;
+    if (MODE == kDgrad && p.add_sub && add_here) {
+      uint32_t img, rem, h, w;
+      p.div_plane.divmod(static_cast<uint32_t>(row), img, rem);
+      p.div_width.divmod(rem, h, w);
+      add_here = ((h | w) & 1u) == 0u;
+      const int64_t hs = (p.H + 1) >> 1, ws = (p.W + 1) >> 1;
+      add_idx = ((static_cast<int64_t>(img) * hs + (h >> 1)) * ws + (w >> 1)) * p.gemm_n + col;
+    }
+    if (add_here) {
       Chunk ca;
-      ca.u = *reinterpret_cast<const uint4*>(static_cast<const T*>(p.add) + idx);
+      ca.u = *reinterpret_cast<const uint4*>(static_cast<const T*>(p.add) + add_idx);
       float a[E];
       chunk_to_float<T>(ca, a);
       if (p.mask) {
@@ -1780,10 +1792,12 @@ int conv2d_dgrad_stat_rows(const ConvShape& s, int dtype, int tile_cfg) {
 }
 
 int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, const void* wt, void* dx,
-                 const void* add, const void* mask, int tile_cfg, const BnBwdSums* bn) {
+                 const void* add, const void* mask, int tile_cfg, const BnBwdSums* bn, int add_stride) {
   IgemmArgs a{};
   if (int rc = fill_common(a, s, dtype)) return rc;
   TCH_CHECK_ARG(dy && wt && dx, "conv2d_dgrad: null tensor");
+  TCH_CHECK_ARG(add_stride == 1 || add_stride == 2, "conv2d_dgrad: the addend's grid is the output's or every second pixel of it");
+  a.add_sub = (add && add_stride == 2) ? 1 : 0;
   if (bn) {
     TCH_CHECK_ARG(bn->x && bn->mean && bn->invstd && bn->partial, "conv2d_dgrad: incomplete BatchNorm operands");
     TCH_CHECK_ARG(!bn->finalize || check_finalize(bn->finalize, false), "conv2d_dgrad: incomplete BatchNorm finalize operands");

@@ -54,7 +54,7 @@ struct BnBwdSums {
   const BnFinalize* finalize;  // optional
 };
 int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, const void* w, void* dx,
-                 const void* add, const void* mask, int tile_cfg, const BnBwdSums* bn = nullptr);
+                 const void* add, const void* mask, int tile_cfg, const BnBwdSums* bn = nullptr, int add_stride = 1);
 int conv2d_dgrad_stat_rows(const ConvShape& s, int dtype, int tile_cfg);
 int conv2d_wgrad_pick_splits(const ConvShape& s, int dtype);
 int64_t conv2d_wgrad_workspace_bytes(const ConvShape& s, int dtype, int splits);

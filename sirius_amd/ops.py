@@ -203,8 +203,19 @@ def conv2d_fwd_bnstats(ctx, x, w, y, stride, pad, partial, tile_cfg=-1, c_logica
     return rb
 
 
-def conv2d_dgrad(ctx, dy, wt, dx, stride, pad, add=None, mask=None, tile_cfg=-1, c_logical=0):
-    """wt is the filter transposed to [C,R,S,K] (filter_transpose)."""
+def _check_addend(add, dx, add_stride):
+    """add is laid out like dx, or (add_stride 2) holds the even (h, w) of dx's grid only."""
+    assert add_stride in (1, 2)
+    if add is None:
+        return
+    N, H, W, C = dx.shape
+    want = (N, H, W, C) if add_stride == 1 else (N, (H + 1) // 2, (W + 1) // 2, C)
+    assert tuple(add.shape) == want and add.dtype == dx.dtype, (tuple(add.shape), want)
+
+
+def conv2d_dgrad(ctx, dy, wt, dx, stride, pad, add=None, mask=None, tile_cfg=-1, c_logical=0, add_stride=1):
+    """wt is the filter transposed to [C,R,S,K] (filter_transpose).  add_stride=2: `add` is [N, ceil(H/2), ceil(W/2), C]
+    and counts at the even pixels of dx's grid (the compact data gradient of a stride-2 1x1 convolution)."""
     w = wt
     N, H, W, C = dx.shape
     C2, R, S, K = wt.shape
@@ -212,10 +223,10 @@ def conv2d_dgrad(ctx, dy, wt, dx, stride, pad, add=None, mask=None, tile_cfg=-1,
     Ho, Wo = conv_out_hw(H, W, R, S, stride, pad)
     assert tuple(dy.shape) == (N, Ho, Wo, K)
     assert dy.dtype == w.dtype == dx.dtype
-    for t in (add, mask):
-        assert t is None or (t.shape == dx.shape and t.dtype == dx.dtype)
+    assert mask is None or (mask.shape == dx.shape and mask.dtype == dx.dtype)
+    _check_addend(add, dx, add_stride)
     check(lib().tch_conv2d_dgrad(ctx.handle, dtype_code(dy), _p(dy), _p(w), _p(dx), _p(add), _p(mask),
-                                 N, H, W, C, K, R, S, stride, pad, tile_cfg, c_logical), "tch_conv2d_dgrad")
+                                 N, H, W, C, K, R, S, stride, pad, tile_cfg, c_logical, add_stride), "tch_conv2d_dgrad")
 
 
 def conv2d_dgrad_stat_rows(dx, K, R, S, stride, pad, tile_cfg=-1):
@@ -224,7 +235,7 @@ def conv2d_dgrad_stat_rows(dx, K, R, S, stride, pad, tile_cfg=-1):
 
 
 def conv2d_dgrad_bnsums(ctx, dy, wt, dx, stride, pad, bn_x, bn_mean, bn_invstd, partial, bn_mask=None, add=None,
-                        mask=None, tile_cfg=-1, c_logical=0):
+                        mask=None, tile_cfg=-1, c_logical=0, add_stride=1):
     """conv2d_dgrad whose output is the gradient behind a BatchNorm(+ReLU) with input bn_x and ReLU output
     bn_mask: dx is stored already gated by the ReLU, and `partial` ([row tiles, C, 2] fp32) receives the two
     reductions of that BatchNorm's backward.  Returns the number of row tiles."""
@@ -234,15 +245,16 @@ def conv2d_dgrad_bnsums(ctx, dy, wt, dx, stride, pad, bn_x, bn_mean, bn_invstd, 
     Ho, Wo = conv_out_hw(H, W, R, S, stride, pad)
     assert tuple(dy.shape) == (N, Ho, Wo, K)
     assert dy.dtype == wt.dtype == dx.dtype
-    for t in (add, mask, bn_mask, bn_x):
+    for t in (mask, bn_mask, bn_x):
         assert t is None or (t.shape == dx.shape and t.dtype == dx.dtype)
+    _check_addend(add, dx, add_stride)
     assert bn_x is not None and bn_mean.numel() == C and bn_invstd.numel() == C
     assert bn_mean.dtype == bn_invstd.dtype == torch.float32
     rb = conv2d_dgrad_stat_rows(dx, K, R, S, stride, pad, tile_cfg)
     assert partial.dtype == torch.float32 and partial.numel() >= rb * C * 2
     check(lib().tch_conv2d_dgrad_bnsums(ctx.handle, dtype_code(dy), _p(dy), _p(wt), _p(dx), _p(add), _p(mask),
                                         N, H, W, C, K, R, S, stride, pad, tile_cfg, c_logical, _p(bn_mask), _p(bn_x),
-                                        _p(bn_mean), _p(bn_invstd), _p(partial)), "tch_conv2d_dgrad_bnsums")
+                                        _p(bn_mean), _p(bn_invstd), _p(partial), add_stride), "tch_conv2d_dgrad_bnsums")
     return rb
 
 
@@ -266,7 +278,7 @@ def conv2d_fwd_bn(ctx, x, w, y, stride, pad, partial, counters, gamma, beta, run
 
 
 def conv2d_dgrad_bn(ctx, dy, wt, dx, stride, pad, bn_x, bn_mean, bn_invstd, partial, counters, gamma, dgamma, dbeta, coef,
-                    bn_mask=None, add=None, mask=None, accumulate=False, tile_cfg=-1, c_logical=0):
+                    bn_mask=None, add=None, mask=None, accumulate=False, tile_cfg=-1, c_logical=0, add_stride=1):
     """conv2d_dgrad_bnsums + dgamma / dbeta + the coefficients of the BatchNorm input gradient (coef [3, C]);
     finish with bn_apply_bwd."""
     N, H, W, C = dx.shape
@@ -274,8 +286,9 @@ def conv2d_dgrad_bn(ctx, dy, wt, dx, stride, pad, bn_x, bn_mean, bn_invstd, part
     assert C == C2
     Ho, Wo = conv_out_hw(H, W, R, S, stride, pad)
     assert tuple(dy.shape) == (N, Ho, Wo, K) and dy.dtype == wt.dtype == dx.dtype
-    for t in (add, mask, bn_mask, bn_x):
+    for t in (mask, bn_mask, bn_x):
         assert t is None or (t.shape == dx.shape and t.dtype == dx.dtype)
+    _check_addend(add, dx, add_stride)
     assert bn_x is not None and bn_mean.numel() == C and bn_invstd.numel() == C
     rb = conv2d_dgrad_stat_rows(dx, K, R, S, stride, pad, tile_cfg)
     assert partial.dtype == torch.float32 and partial.numel() >= rb * C * 2
@@ -283,7 +296,7 @@ def conv2d_dgrad_bn(ctx, dy, wt, dx, stride, pad, bn_x, bn_mean, bn_invstd, part
     check(lib().tch_conv2d_dgrad_bn(ctx.handle, dtype_code(dy), _p(dy), _p(wt), _p(dx), _p(add), _p(mask),
                                     N, H, W, C, K, R, S, stride, pad, tile_cfg, c_logical, _p(bn_mask), _p(bn_x),
                                     _p(bn_mean), _p(bn_invstd), _p(partial), _p(counters), _p(gamma), _p(dgamma),
-                                    _p(dbeta), int(accumulate), _p(coef)), "tch_conv2d_dgrad_bn")
+                                    _p(dbeta), int(accumulate), _p(coef), add_stride), "tch_conv2d_dgrad_bn")
 
 
 def bn_apply_fwd(ctx, x, y, coef, residual=None, relu=True):

@@ -75,6 +75,8 @@ class ResNetEngine(EngineBase):
         # fuse_eval_bn: the forward-only (inference) plan runs convolution + BatchNorm (+ residual) (+ ReLU) as one
         # launch each instead of two
         self.fuse_eval_bn = True
+        # compact_downsample_dgrad: the data gradient of a stride-2 downsample convolution stays on the small grid
+        self.compact_downsample_dgrad = True
         self.group_wgrad = group_wgrad and overlap_wgrad
         self.wgrad_group_wgs, self.wgrad_group_blocks = wgrad_group_wgs, wgrad_group_blocks
         self.wgrad_group_max_wgs = wgrad_group_max_wgs
@@ -630,10 +632,17 @@ class ResNetEngine(EngineBase):
                     dzd = galloc(zd.shape)
                     bn_bwd(pre + ".downsample.1", g_out, zd, dzd, out_gate)
                     conv_wgrad(blk.cd, xin, dzd, grouped=True)
-                    gx_id = galloc(xin.shape)
-                    conv_dgrad(blk.cd, dzd, gx_id)
+                    if blk.cd.stride == 2 and self.compact_downsample_dgrad:
+                        # a stride-2 1x1 convolution sends gradient to the even pixels of its input only: computed
+                        # as the stride-1 data gradient on dzd's own grid and added from there
+                        gx_id = galloc((B, Ho, Wo, xin.shape[3]))
+                        ops.conv2d_dgrad(ctx, dzd, self._wt(blk.cd.name + ".weight"), gx_id, 1, 0)
+                        add_kw = dict(add=gx_id, add_stride=2)
+                    else:
+                        gx_id = galloc(xin.shape)
+                        conv_dgrad(blk.cd, dzd, gx_id)
+                        add_kw = dict(add=gx_id)
                     gfree(dzd, True)
-                    add_kw = dict(add=gx_id)
                 else:
                     gx_id = None
                     add_kw = dict(add=g_out, mask=out_gate)

@@ -194,6 +194,56 @@ def test_huge_tile_equals_the_128_tile(ctx, shape):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("hw", [(14, 14), (7, 9), (5, 5)])
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 2, 6])
+def test_conv_dgrad_with_a_compact_addend(ctx, dtype, hw, tile_cfg):
+    """The data gradient of a stride-2 1x1 convolution is non-zero at the even pixels only: kept on the small grid
+    (odd sizes: ceil(H/2) x ceil(W/2)) and added from there by the data gradient it joins -- same result as adding
+    the full-size tensor, bit for bit; also with the BatchNorm-backward sums in the epilogue."""
+    from sirius_amd import ops
+    H, W = hw
+    N, C, K, Kd = 3, 64, 64, 128
+    g = _gen(31)
+    dy = rnd((N, H, W, K), dtype, g, K ** -0.5)
+    w = rnd((K, 1, 1, C), dtype, g)
+    Hs, Ws = (H + 1) // 2, (W + 1) // 2
+    dyd = rnd((N, Hs, Ws, Kd), dtype, g, Kd ** -0.5)         # gradient of the downsample branch's output
+    wd = rnd((Kd, 1, 1, C), dtype, g)
+    wt, wdt = ops.filter_transpose(ctx, w.cuda()), ops.filter_transpose(ctx, wd.cuda())
+    # full-size route: stride-2 data gradient blown up to the input grid, then added
+    full = torch.empty((N, H, W, C), dtype=dtype, device="cuda")
+    ops.conv2d_dgrad(ctx, dyd.cuda(), wdt, full, 2, 0)
+    ref_full = O.conv2d_dgrad(dyd, wd, (N, H, W, C), 2, 0)
+    torch.cuda.synchronize()
+    close(full, ref_full, dtype, "stride-2 data gradient")
+    assert float(full[:, 1::2].float().abs().max()) == 0.0 and float(full[:, :, 1::2].float().abs().max()) == 0.0
+    dx_a = torch.empty((N, H, W, C), dtype=dtype, device="cuda")
+    ops.conv2d_dgrad(ctx, dy.cuda(), wt, dx_a, 1, 0, add=full, tile_cfg=tile_cfg)
+    # compact route
+    small = torch.empty((N, Hs, Ws, C), dtype=dtype, device="cuda")
+    ops.conv2d_dgrad(ctx, dyd.cuda(), wdt, small, 1, 0)
+    dx_b = torch.empty((N, H, W, C), dtype=dtype, device="cuda")
+    ops.conv2d_dgrad(ctx, dy.cuda(), wt, dx_b, 1, 0, add=small, add_stride=2, tile_cfg=tile_cfg)
+    torch.cuda.synchronize()
+    assert torch.equal(small, full[:, ::2, ::2])
+    assert torch.equal(dx_a, dx_b)
+    close(dx_b, O.conv2d_dgrad(dy, w, (N, H, W, C), 1, 0) + ref_full, dtype, "data gradient + compact addend")
+    # the same with the BatchNorm-backward sums and the ReLU gate in the epilogue
+    bn_x, relu_out = rnd((N, H, W, C), dtype, g), rnd((N, H, W, C), dtype, g)
+    mean, invstd = torch.randn(C, generator=g), torch.rand(C, generator=g) + 0.5
+    outs = []
+    for add, stride in ((full, 1), (small, 2)):
+        dx = torch.empty((N, H, W, C), dtype=dtype, device="cuda")
+        rb = ops.conv2d_dgrad_stat_rows(dx, K, 1, 1, 1, 0, tile_cfg)
+        partial = torch.zeros(rb * C * 2, dtype=torch.float32, device="cuda")
+        ops.conv2d_dgrad_bnsums(ctx, dy.cuda(), wt, dx, 1, 0, bn_x.cuda(), mean.cuda(), invstd.cuda(), partial,
+                                bn_mask=relu_out.cuda(), add=add, add_stride=stride, tile_cfg=tile_cfg)
+        torch.cuda.synchronize()
+        outs.append((dx, partial))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", CONV_CASES)
 @pytest.mark.parametrize("splits", [1, 0, 3])
 def test_conv_wgrad(ctx, dtype, case, splits):

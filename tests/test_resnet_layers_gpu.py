@@ -151,8 +151,18 @@ def _layer_local(batch, depths=(3, 8, 36, 3), width=64, classes=1000, image=224,
         if blk.cd is not None:
             bn_bwd(pre + ".downsample.1", G, t["zd"], t["dzd"])
             conv_wgrad(blk.cd, t["x"], t["dzd"])
-            chk("conv_dgrad", blk.cd.name, t["gx_id"], conv_dgrad(blk.cd, t["dzd"], t["x"]))
-            shortcut = _f(t["gx_id"])
+            ref_id = conv_dgrad(blk.cd, t["dzd"], t["x"])
+            got_id = _f(t["gx_id"])
+            if got_id.shape != ref_id.shape:
+                # the engine keeps the gradient of a stride-2 downsample convolution on the small grid: the even
+                # pixels of the oracle's tensor, whose other pixels are exactly zero
+                assert float(ref_id[:, 1::2].abs().max()) == 0.0 and float(ref_id[:, :, 1::2].abs().max()) == 0.0
+                chk("conv_dgrad", blk.cd.name, t["gx_id"], ref_id[:, ::2, ::2])
+                shortcut = torch.zeros_like(ref_id)
+                shortcut[:, ::2, ::2] = got_id
+            else:
+                chk("conv_dgrad", blk.cd.name, t["gx_id"], ref_id)
+                shortcut = got_id
         else:
             shortcut = G
         gx_ref = conv_dgrad(blk.c1, t["dz1"], t["x"]) + shortcut
