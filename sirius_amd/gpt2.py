@@ -179,6 +179,7 @@ class GPT2Engine(EngineBase):
             self.momentum_buf.zero_()
 
     def refresh_shadow(self):
+        self.ctx.synchronize()      # nothing of an earlier step (either lane) still reads or writes the copies
         if self.shadow is not None:
             ops.cast_from_f32(self.ctx, self.params, self.shadow)
         self._refresh_transposed()
@@ -318,6 +319,8 @@ class GPT2Engine(EngineBase):
             mark("fwd", "loss")
 
             # ================= backward =================
+            if self.overlap_wgrad:
+                ctx.join()      # the second lane may still be writing the transposed filters of the last optimizer step
             g_c = [act(R, C) for _ in range(4)]       # gradients of [R, C] tensors, handed round
             g_f1, g_f2, g_qkv = act(R, 4 * C), act(R, 4 * C), act(R, 3 * C)
             dP = act(B * H, T, dtype=torch.float32) if fused else act(B, H, T, T)   # fused: the delta scratch
@@ -394,4 +397,10 @@ class GPT2Engine(EngineBase):
         else:
             ops.sgd_momentum_step(self.ctx, self.params, grads, self.momentum_buf, self.lr, self.momentum,
                                   self.weight_decay, shadow=self.shadow)
-        self._refresh_transposed()
+        # the transposed copies are read by the data gradients only: made on the second lane, beside the next
+        # step's forward pass; the backward program joins the lanes before its first data gradient
+        if self.overlap_wgrad:
+            with self.ctx.side_lane(wait_main=True):
+                self._refresh_transposed()
+        else:
+            self._refresh_transposed()

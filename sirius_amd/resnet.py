@@ -237,6 +237,7 @@ class ResNetEngine(EngineBase):
         torch.cuda.synchronize()
 
     def refresh_shadow(self):
+        self.ctx.synchronize()      # nothing of an earlier step (either lane) still reads or writes the copies
         if self.shadow is not None:
             ops.cast_from_f32(self.ctx, self.params, self.shadow)
         self._refresh_transposed()
@@ -572,6 +573,8 @@ class ResNetEngine(EngineBase):
             mark("fwd", "loss")
 
             # ================= backward =================
+            if self.overlap_wgrad:
+                ctx.join()      # the second lane may still be writing the transposed filters of the last optimizer step
             fc_conv = _Conv("fc", self.feat, self.num_classes, 1, 1, 0)
             conv_wgrad(fc_conv, pooled.view(B, 1, 1, self.feat), dlogits.view(B, 1, 1, self.num_classes))
             ops.bias_grad(ctx, dlogits, self._view(self.grads, "fc.bias"))
@@ -791,4 +794,10 @@ class ResNetEngine(EngineBase):
     def _record_optimizer(self, grads):
         ops.sgd_momentum_step(self.ctx, self.params, grads, self.momentum_buf, self.lr, self.momentum,
                               self.weight_decay, shadow=self.shadow)
-        self._refresh_transposed()
+        # the transposed copies are read by the data gradients only: made on the second lane, beside the next
+        # step's forward pass; the backward program joins the lanes before its first data gradient
+        if self.overlap_wgrad:
+            with self.ctx.side_lane(wait_main=True):
+                self._refresh_transposed()
+        else:
+            self._refresh_transposed()

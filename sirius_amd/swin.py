@@ -208,6 +208,7 @@ class SwinEngine(EngineBase):
         torch.cuda.synchronize()
 
     def refresh_shadow(self):
+        self.ctx.synchronize()      # nothing of an earlier step (either lane) still reads or writes the copies
         if self.shadow is not None:
             ops.cast_from_f32(self.ctx, self.params, self.shadow)
         self._refresh_transposed()
@@ -459,6 +460,8 @@ class SwinEngine(EngineBase):
             mark("fwd", "loss")
 
             # ================= backward =================
+            if self.overlap_wgrad:
+                ctx.join()      # the second lane may still be writing the transposed filters of the last optimizer step
             g_pooled = v2(g_bufs[0], B, CL)
             lin_bwd("head", pooled, dlogits, g_pooled)
             g_hf = v2(g_bufs[1], rowsL, CL)
@@ -586,4 +589,10 @@ class SwinEngine(EngineBase):
         ops.adamw_step(self.ctx, self.params, grads, self.exp_avg, self.exp_avg_sq, self.step_dev, self.adam_scalars,
                        lr=self.lr, beta1=self.betas[0], beta2=self.betas[1], eps=self.eps,
                        weight_decay=self.weight_decay, shadow=self.shadow)
-        self._refresh_transposed()
+        # the transposed copies are read by the data gradients only: made on the second lane, beside the next
+        # step's forward pass; the backward program joins the lanes before its first data gradient
+        if self.overlap_wgrad:
+            with self.ctx.side_lane(wait_main=True):
+                self._refresh_transposed()
+        else:
+            self._refresh_transposed()
