@@ -918,7 +918,9 @@ __global__ __launch_bounds__(WM* WN * 64) void wgrad_group_kernel(WgradGroupArgs
 //     operand read touches every bank once;
 //   * a step never straddles a filter tap (channels % 64 == 0), so the tap walk is scalar:
 //     a lane keeps one byte offset and one validity bit per tap for each row it loads;
-//   * NBUF tiles in flight, one barrier per step.
+//   * NBUF tiles in flight, one barrier per step;
+//   * KS = 32 halves the step (64-byte rows, sixteen rows per direct load): half the LDS per tile in flight, so
+//     more workgroups share a CU and a small grid is resident in one round.
 constexpr int kStep2 = 64;                  // reduction elements per step
 constexpr int kRowBytes2 = kStep2 * 2;      // 128
 
@@ -931,17 +933,25 @@ __device__ inline void load_to_lds(__amdgpu_buffer_rsrc_t rsrc, unsigned char* d
   __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)dst, 16, voff, soff, 0, 0);
 }
 
-template <int MODE, int WM, int WN, int TM, int TN, int NBUF, int ROT = 0>
+template <int MODE, int WM, int WN, int TM, int TN, int NBUF, int ROT = 0, int KS = kStep2>
 __global__ __launch_bounds__(WM* WN * 64) void igemm2_kernel(IgemmArgs p) {
   using T = bf16;
   constexpr int E = 8;
   constexpr int BM = WM * TM * 32;
   constexpr int BN = WN * TN * 32;
   constexpr int NW = WM * WN;
-  constexpr int A_LD = BM / 8 / NW;  // direct loads per wave and step for the activation tile (8 rows each)
-  constexpr int B_LD = BN / 8 / NW;
-  static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile/loader mismatch");
-  constexpr int A_BYTES = BM * kRowBytes2, B_BYTES = BN * kRowBytes2;
+  static_assert(KS == 64 || KS == 32, "reduction elements per step");
+  constexpr int RB = KS * 2;             // bytes of one LDS row
+  constexpr int SLOTS = RB / 16;         // 16-byte slots per row: 8 or 4
+  constexpr int SLOT_SH = KS == 64 ? 3 : 2;
+  constexpr int LD_ROWS = 1024 / RB;     // rows one direct load of a wave fills: 8 or 16
+  constexpr int A_LD = BM / LD_ROWS / NW;  // direct loads per wave and step for the activation tile
+  constexpr int B_LD = BN / LD_ROWS / NW;
+  static_assert(BM % (LD_ROWS * NW) == 0 && BN % (LD_ROWS * NW) == 0, "tile/loader mismatch");
+  constexpr int A_BYTES = BM * RB, B_BYTES = BN * RB;
+  // slot = chunk ^ swizzle(row): with 128-byte rows two rows span the 64 banks and (row >> 1) & 7 spreads sixteen
+  // rows of one chunk over all of them; with 64-byte rows four rows span them and (row >> 2) & 3 does the same
+  auto swizzle = [](int row) { return KS == 64 ? (row >> 1) & 7 : (row >> 2) & 3; };
   constexpr int BUF_BYTES = A_BYTES + B_BYTES;
   constexpr int STAGE_BYTES = WM * 32 * (BN + kStagePad) * 4;
   constexpr int LDS_BYTES = NBUF * BUF_BYTES > STAGE_BYTES ? NBUF * BUF_BYTES : STAGE_BYTES;
@@ -973,18 +983,18 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm2_kernel(IgemmArgs p) {
   const int in_h = (MODE == kFwd) ? p.H : p.Ho;
   const int in_w = (MODE == kFwd) ? p.W : p.Wo;
   const int in_c = (MODE == kFwd) ? p.C : p.K;
-  const int cblocks = in_c / kStep2;
+  const int cblocks = in_c / KS;
   const int nk = p.R * p.S * cblocks;
   const int sl = p.stride_log2, sm = p.stride - 1;
 
   // ---- per lane: the rows it feeds, their byte offset at tap (0,0) and which taps exist ----
-  const int sub_row = lane >> 3, slot = lane & 7;
+  const int sub_row = lane >> SLOT_SH, slot = lane & (SLOTS - 1);
   int a_off[A_LD];
   uint32_t a_taps[A_LD];
 #pragma unroll
   for (int j = 0; j < A_LD; ++j) {
-    const int trow = (wave * A_LD + j) * 8 + sub_row;
-    const int chunk = slot ^ ((trow >> 1) & 7);
+    const int trow = (wave * A_LD + j) * LD_ROWS + sub_row;
+    const int chunk = slot ^ swizzle(trow);
     const int row = m0 + trow;
     uint32_t img = 0, pix = 0, oh = 0, ow = 0, taps = 0;
     int base = 0;
@@ -1016,8 +1026,8 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm2_kernel(IgemmArgs p) {
   int b_off[B_LD];
 #pragma unroll
   for (int j = 0; j < B_LD; ++j) {
-    const int trow = (wave * B_LD + j) * 8 + sub_row;
-    const int chunk = slot ^ ((trow >> 1) & 7);
+    const int trow = (wave * B_LD + j) * LD_ROWS + sub_row;
+    const int chunk = slot ^ swizzle(trow);
     const int row = n0 + trow;
     b_off[j] = row < p.gemm_n ? (row * p.gemm_k + chunk * E) * 2 : static_cast<int>(kOutOfRange);
   }
@@ -1030,8 +1040,8 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm2_kernel(IgemmArgs p) {
   auto issue_loads = [&](int buf) {
     // element offset of this tap relative to tap (0,0), then bytes
     const int tap_elems = (MODE == kFwd) ? (ld_r * in_w + ld_s) * in_c : -((ld_r >> sl) * in_w + (ld_s >> sl)) * in_c;
-    const int a_step = (tap_elems + ld_cb * kStep2) * 2;
-    const int b_step = ld_kt * kRowBytes2;
+    const int a_step = (tap_elems + ld_cb * KS) * 2;
+    const int b_step = ld_kt * RB;
     unsigned char* dst_a = lds + buf * BUF_BYTES + wave * A_LD * 1024;
     unsigned char* dst_b = lds + buf * BUF_BYTES + A_BYTES + wave * B_LD * 1024;
 #pragma unroll
@@ -1062,13 +1072,13 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm2_kernel(IgemmArgs p) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  // operand reads: row = tile row of the lane, slot = chunk ^ ((row >> 1) & 7); the tile bases are
+  // operand reads: row = tile row of the lane, slot = chunk ^ swizzle(row); the tile bases are
   // multiples of 32 rows, so the swizzle term depends on the lane only
   const int frag_row = lane & 31, frag_half = lane >> 5;
-  const int swz = (frag_row >> 1) & 7;
+  const int swz = swizzle(frag_row);
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds));
-  const uint32_t a_rd = lds_base + (wm * TM * 32 + frag_row) * kRowBytes2 + swz * 16;
-  const uint32_t b_rd = lds_base + A_BYTES + (wn * TN * 32 + frag_row) * kRowBytes2 + swz * 16;
+  const uint32_t a_rd = lds_base + (wm * TM * 32 + frag_row) * RB + swz * 16;
+  const uint32_t b_rd = lds_base + A_BYTES + (wn * TN * 32 + frag_row) * RB + swz * 16;
   // The operand reads are written as asm: the compiler orders every LDS read it can see behind
   // ALL outstanding direct-to-LDS loads (vmcnt(0)), which would serialise the prefetch of the
   // next tiles with the multiply of this one.  Which loads must have landed is known here (the
@@ -1078,10 +1088,10 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm2_kernel(IgemmArgs p) {
     const uint32_t pa = (a_rd ^ cx) + buf * BUF_BYTES, pb = (b_rd ^ cx) + buf * BUF_BYTES;
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm)
-      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fa[tm]) : "v"(pa), "n"(tm * 32 * kRowBytes2));
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fa[tm]) : "v"(pa), "n"(tm * 32 * RB));
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn)
-      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fb[tn]) : "v"(pb), "n"(tn * 32 * kRowBytes2));
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(fb[tn]) : "v"(pb), "n"(tn * 32 * RB));
   };
   auto multiply = [&](uint4_t* fa, uint4_t* fb) {
     // ties the registers to the wait that precedes this call in program order
@@ -1102,6 +1112,11 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm2_kernel(IgemmArgs p) {
     read_frags(buf, 1, fa1, fb1);
     asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(TM + TN));
     multiply(fa0, fb0);
+    if constexpr (KS == 32) {   // a 32-element step holds two 16-element slices
+      asm volatile("s_waitcnt lgkmcnt(0)");
+      multiply(fa1, fb1);
+      return;
+    }
     read_frags(buf, 2, fa0, fb0);
     asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(TM + TN));
     multiply(fa1, fb1);
@@ -1141,7 +1156,7 @@ __global__ __launch_bounds__(WM* WN * 64) void igemm2_kernel(IgemmArgs p) {
     // barrier, the reads' latency and the issue of the next tile's loads pass.  Every wait stands behind a
     // quarter's multiplies that were issued after the reads it waits for, and nothing is in flight at the loop
     // edge.  Order of additions per accumulator: as in the plain loop (same results bit for bit).
-    static_assert(NBUF == 2, "the rotated loop keeps two tiles in LDS");
+    static_assert(NBUF == 2 && KS == 64, "the rotated loop keeps two 64-element tiles in LDS");
     uint4_t fa0[TM], fb0[TN], fa1[TM], fb1[TN];
     issue_loads(0);
     asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
@@ -1507,12 +1522,12 @@ int launch_cfg(Context* ctx, IgemmArgs& a, double flops) {
                   flops, 0, conv_bytes<MODE>(a, sizeof(T)));
 }
 
-template <int MODE, int WM, int WN, int TM, int TN, int NBUF, int ROT = 0>
+template <int MODE, int WM, int WN, int TM, int TN, int NBUF, int ROT = 0, int KS = kStep2>
 int launch_cfg2(Context* ctx, IgemmArgs& a, double flops) {
   constexpr int BM = WM * TM * 32, BN = WN * TN * 32;
   static const std::string name = std::string("igemm2_kernel<bf16,") + (MODE == kFwd ? "fwd," : "dgrad,") +
                                   std::to_string(BM) + "x" + std::to_string(BN) + "," + std::to_string(NBUF) + "buf" +
-                                  (WM * WN == 8 ? ",8w" : "") + (ROT ? ",rot>" : ">");
+                                  (WM * WN == 8 ? ",8w" : "") + (KS == 32 ? ",k32" : "") + (ROT ? ",rot>" : ">");
   a.tiles_m = (a.gemm_m + BM - 1) / BM;
   a.tiles_n = (a.gemm_n + BN - 1) / BN;
   static const int group_env = [] {
@@ -1525,7 +1540,7 @@ int launch_cfg2(Context* ctx, IgemmArgs& a, double flops) {
     set_error("igemm: grid out of range");
     return -22;
   }
-  return launch(ctx, igemm2_kernel<MODE, WM, WN, TM, TN, NBUF, ROT>, dim3(static_cast<unsigned>(wgs)), dim3(WM * WN * 64), a,
+  return launch(ctx, igemm2_kernel<MODE, WM, WN, TM, TN, NBUF, ROT, KS>, dim3(static_cast<unsigned>(wgs)), dim3(WM * WN * 64), a,
                 name.c_str(), flops, 0, conv_bytes<MODE>(a, 2));
 }
 
@@ -1592,6 +1607,17 @@ int launch_mode(Context* ctx, IgemmArgs& a, int tile_cfg, double flops) {
         return tile_cfg == 9 ? launch_cfg2<MODE, 2, 4, 4, 2, 2>(ctx, a, flops) : launch_cfg2<MODE, 2, 4, 4, 2, 2, 1>(ctx, a, flops);
       tile_cfg = 0;
     }
+    // 11 - 14: 32-element reduction steps.  11 / 12: 128 x 128 with three / two LDS tiles in flight (48 / 34 KB:
+    // three / four workgroups per CU), 13: 128 x 64 and 14: 64 x 64 with three (36 / 24 KB)
+    if (tile_cfg >= 11 && tile_cfg <= 14) {
+      if (setting != 0 && in_c % kStep2 == 0 && a.R * a.S <= 32) {
+        if (tile_cfg == 11) return launch_cfg2<MODE, 2, 2, 2, 2, 3, 0, 32>(ctx, a, flops);
+        if (tile_cfg == 12) return launch_cfg2<MODE, 2, 2, 2, 2, 2, 0, 32>(ctx, a, flops);
+        if (tile_cfg == 13) return launch_cfg2<MODE, 2, 2, 2, 1, 3, 0, 32>(ctx, a, flops);
+        return launch_cfg2<MODE, 2, 2, 1, 1, 3, 0, 32>(ctx, a, flops);
+      }
+      tile_cfg = tile_cfg <= 12 ? 0 : tile_cfg - 12;
+    }
     // 6 / 7: tilings 1 / 2 with two LDS tiles in flight instead of three (48 / 32 KB of LDS: three or four
     // workgroups per CU, which the memory-bound data gradients of the large feature maps prefer)
     if (tile_cfg == 6 || tile_cfg == 7) {
@@ -1610,6 +1636,7 @@ int launch_mode(Context* ctx, IgemmArgs& a, int tile_cfg, double flops) {
   if (tile_cfg == 5) tile_cfg = 1;
   if (tile_cfg == 6 || tile_cfg == 7) tile_cfg -= 5;
   if (tile_cfg == 9 || tile_cfg == 10) tile_cfg = 0;
+  if (tile_cfg >= 11 && tile_cfg <= 14) tile_cfg = tile_cfg <= 12 ? 0 : tile_cfg - 12;
   switch (tile_cfg) {
     case 0:
       return launch_cfg<T, MODE, 2, 2, 2, 2>(ctx, a, flops);  // 128 x 128
@@ -1630,6 +1657,7 @@ double conv_flops(const ConvShape& s, int Ho, int Wo) {
 // rows of the workgroup tile of a tiling number (5 = the 3x3 patch kernel, or tiling 1 where it does not fit)
 int tile_rows(int tile_cfg) {
   if (tile_cfg == 9 || tile_cfg == 10) return 256;
+  if (tile_cfg >= 11 && tile_cfg <= 14) return tile_cfg == 14 ? 64 : 128;
   return (tile_cfg == 5 || tile_cfg == 6) ? 128 : tile_cfg >= 2 ? 64 : 128;
 }
 

@@ -316,10 +316,12 @@ class ResNetEngine(EngineBase):
         # 5 = the 3x3 patch kernel (stride-1 3x3 layers; elsewhere the library runs tiling 1 for it)
         patch = (5,) if (c.k == 3 and c.stride == 1 and c.pad == 1) else ()
         # 6 / 7 = tilings 1 / 2 with two LDS tiles in flight (more workgroups per CU)
-        cfgs = ((0, 1, 2, 3, 6, 7) if c.cout > 64 else (1, 2, 3, 6, 7)) + patch
+        # 11 - 14 = 128 x 128 (three / two LDS tiles), 128 x 64, 64 x 64 with 32-element reduction steps: half the LDS
+        # per workgroup, which the wide, shallow products of the first two stages prefer
+        cfgs = ((0, 1, 2, 3, 6, 7, 11, 12, 13, 14) if c.cout > 64 else (1, 2, 3, 6, 7, 13, 14)) + patch
         t_f = {cfg: self._time_program(fwd(cfg)) / reps for cfg in cfgs}
         tf = min(t_f, key=t_f.get)
-        cfgs_d = ((0, 1, 2, 3, 6, 7) if c.cin_store > 64 else (1, 2, 3, 6, 7)) + patch
+        cfgs_d = ((0, 1, 2, 3, 6, 7, 11, 12, 13, 14) if c.cin_store > 64 else (1, 2, 3, 6, 7, 13, 14)) + patch
         t_d = {cfg: self._time_program(dgrad(cfg)) / reps for cfg in cfgs_d} if c.cin_store >= 64 else {-1: 0.0}
         td = min(t_d, key=t_d.get)
         self._tile_cache[key] = (tf, td)

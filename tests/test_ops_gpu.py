@@ -60,7 +60,7 @@ CONV_CASES = [
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", CONV_CASES)
-@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3, 5, 6, 7, 9, 10])
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3, 5, 6, 7, 9, 10, 11, 12, 13, 14])
 def test_conv_fwd(ctx, dtype, case, tile_cfg):
     from sirius_amd import ops
     N, H, W, C, K, R, S, st, pad = case
@@ -94,7 +94,7 @@ def test_conv_fwd_epilogue(ctx, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", CONV_CASES)
-@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3, 5, 6, 7, 9, 10])
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3, 5, 6, 7, 9, 10, 11, 12, 13, 14])
 def test_conv_dgrad(ctx, dtype, case, tile_cfg):
     from sirius_amd import ops
     N, H, W, C, K, R, S, st, pad = case
@@ -163,9 +163,10 @@ def test_conv_fwd_with_inference_batchnorm_in_the_epilogue(ctx, dtype, case, til
 
 @pytest.mark.parametrize("shape", [(1000, 128, 520), (2048, 192, 1024), (300, 64, 72), (1100, 64, 1200), (2900, 64, 2320)])
 def test_huge_tile_equals_the_128_tile(ctx, shape):
-    """The 256 x 256 tilings (plain and rotated loop, eight wavefronts) on products with several such tiles and
-    ragged edges: within the bf16 bound of the oracle and bit-equal to the 128 x 128 tiling (same order of
-    additions per output), forward and data gradient, with the grouped tile order on and off (wide and narrow N)."""
+    """The 256 x 256 tilings (plain and rotated loop, eight wavefronts) and the tilings with 32-element reduction
+    steps (11 - 14) on products with several such tiles and ragged edges: within the bf16 bound of the oracle and
+    bit-equal to the 128 x 128 tiling (same order of additions per output), forward and data gradient, with the
+    grouped tile order on and off (wide and narrow N)."""
     from sirius_amd import ops
     M, C, K = shape
     g = _gen(17)
@@ -173,24 +174,24 @@ def test_huge_tile_equals_the_128_tile(ctx, shape):
     w = rnd((K, 1, 1, C), torch.bfloat16, g, C ** -0.5)
     ref = O.conv2d_fwd(x, w, 1, 0)
     outs = {}
-    for cfg in (0, 9, 10):
+    for cfg in (0, 9, 10, 11, 12, 13, 14):
         y = torch.full((1, 1, M, K), 3.0, dtype=torch.bfloat16, device="cuda")
         ops.conv2d_fwd(ctx, x.cuda(), w.cuda(), y, 1, 0, tile_cfg=cfg)
         torch.cuda.synchronize()
         close(y, ref, torch.bfloat16, f"forward tiling {cfg}")
         outs[cfg] = y
-    assert torch.equal(outs[9], outs[0]) and torch.equal(outs[10], outs[0])
+    assert all(torch.equal(outs[c], outs[0]) for c in outs), [c for c in outs if not torch.equal(outs[c], outs[0])]
     dy = rnd((1, 1, M, K), torch.bfloat16, g)
     ref_dx = O.conv2d_dgrad(dy, w, (1, 1, M, C), 1, 0)
     wt = ops.filter_transpose(ctx, w.cuda())
     outs = {}
-    for cfg in (0, 9, 10):
+    for cfg in (0, 9, 10, 11, 12, 13, 14):
         dx = torch.full((1, 1, M, C), 3.0, dtype=torch.bfloat16, device="cuda")
         ops.conv2d_dgrad(ctx, dy.cuda(), wt, dx, 1, 0, tile_cfg=cfg)
         torch.cuda.synchronize()
         close(dx, ref_dx, torch.bfloat16, f"data gradient tiling {cfg}")
         outs[cfg] = dx
-    assert torch.equal(outs[9], outs[0]) and torch.equal(outs[10], outs[0])
+    assert all(torch.equal(outs[c], outs[0]) for c in outs), [c for c in outs if not torch.equal(outs[c], outs[0])]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -366,7 +367,7 @@ def test_bn_fwd(ctx, dtype, rows, C, fuse):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", [CONV_CASES[0], CONV_CASES[2], CONV_CASES[3], CONV_CASES[5], CONV_CASES[6], CONV_CASES[10], CONV_CASES[13]])
-@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3, 5, 6, 7, 9, 10])
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3, 5, 6, 7, 9, 10, 11, 12, 13, 14])
 def test_conv_with_bn_statistics(ctx, dtype, case, tile_cfg):
     """The convolution leaves per-tile sums of its stored output; BatchNorm starts from them.
     Checked against the oracle's conv -> BatchNorm(train) on the same inputs; the statistics must be
@@ -528,7 +529,7 @@ def test_bn_bwd(ctx, dtype, rows, C, masked):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", [CONV_CASES[0], CONV_CASES[1], CONV_CASES[3], CONV_CASES[4], CONV_CASES[6], CONV_CASES[10], CONV_CASES[13]])
-@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3, 5, 6, 7, 9, 10])
+@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 3, 5, 6, 7, 9, 10, 11, 12, 13, 14])
 @pytest.mark.parametrize("with_add", [False, True])
 def test_conv_dgrad_with_bn_backward_sums(ctx, dtype, case, tile_cfg, with_add):
     """The data-gradient convolution gates its output by the ReLU of the BatchNorm it flows into and
