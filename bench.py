@@ -186,7 +186,7 @@ def through_plugin(batch, batches=30, skip=8):
     tmp = tempfile.mkdtemp(prefix="tch_bench_")
     os.environ.update({"COLTRAIN_MODE": "colocate-l1", "COLTRAIN_HOOK_MODE": "xsched-sync", "COLTRAIN_USE_XSCHED": "1",
                        "COLTRAIN_HAS_INFER_SERVER": "0", "COLTRAIN_USE_SHARED_TENSOR": "1",
-                       "COLTRAIN_SHARED_TENSOR_POOL_GB": "48", "COLTRAIN_POOL_PAGE_MB": "32",
+                       "COLTRAIN_SHARED_TENSOR_POOL_GB": "48", "COLTRAIN_POOL_PAGE_MB": "32", "COLTRAIN_AUTOTUNE": "1",
                        "COLTRAIN_PROFILE_LOG_PATH": os.path.join(tmp, "train-profile.csv"),
                        "SIRIUS_PORT": str(19000 + os.getpid() % 1000)})
     with contextlib.redirect_stdout(sys.stderr):
@@ -211,7 +211,7 @@ def gpt2_step(batch=8, seq_len=1024, warmup=2, steps=5):
     weights, token ids uniform in [0, 50257) of shape [8, 1024], AdamW.  Reported beside the headline figure."""
     import torch
     from sirius_amd.gpt2 import GPT2Engine
-    eng = GPT2Engine(seq_len=seq_len, dtype=torch.bfloat16, optimizer="adamw")
+    eng = GPT2Engine(seq_len=seq_len, dtype=torch.bfloat16, optimizer="adamw", autotune=True)
     eng.init_normal(0)
     g = torch.Generator(device="cuda")
     g.manual_seed(2)
@@ -261,7 +261,7 @@ def interleaving(batch=8, seq_len=1024, rate_per_s=50.0, train_s=3.0):
     xsched.register_stream(train_stream, False)
     server = None
     try:
-        eng = GPT2Engine(seq_len=seq_len, dtype=torch.bfloat16, optimizer="adamw", stream=train_stream)
+        eng = GPT2Engine(seq_len=seq_len, dtype=torch.bfloat16, optimizer="adamw", stream=train_stream, autotune=True)
         eng.init_normal(0)
         g = torch.Generator(device="cuda")
         g.manual_seed(2)
@@ -326,7 +326,7 @@ def swin_b_step(batch=32, warmup=2, steps=5):
     [32, 3, 224, 224] N(0,1), AdamW(lr 1e-3, wd 0.05), stochastic depth 0.  Reported beside the headline figure."""
     import torch
     from sirius_amd.swin import SwinEngine
-    eng = SwinEngine(dtype=torch.bfloat16)
+    eng = SwinEngine(dtype=torch.bfloat16, autotune=True)
     eng.init_normal(0)
     g = torch.Generator(device="cuda")
     g.manual_seed(3)

@@ -265,19 +265,6 @@ class ResNetEngine(EngineBase):
         return {p.name: self._from_store(p, flat) for p in self._specs}
 
     # ------------------------------------------------------------------ tiling choice
-    def _time_program(self, fn, reps=3):
-        prog = self._flat_prog(fn)
-        self.ctx.run(prog)
-        best = float("inf")
-        for _ in range(reps):
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(self.ctx.stream)
-            self.ctx.run(prog)
-            e1.record(self.ctx.stream)
-            e1.synchronize()
-            best = min(best, e0.elapsed_time(e1))
-        return best
-
     def _tune_conv(self, c, n, h, w):
         """(forward tiling, data-gradient tiling) for one convolution at one input shape."""
         key = (c.cin_store, c.cout, c.k, c.stride, c.pad, n, h, w)
@@ -286,11 +273,12 @@ class ResNetEngine(EngineBase):
             return hit
         T, ctx = self.dtype, self.ctx
         ho, wo = ops.conv_out_hw(h, w, c.k, c.k, c.stride, c.pad)
-        x = torch.zeros((n, h, w, c.cin_store), dtype=T, device=self.dev)
-        z = torch.zeros((n, ho, wo, c.cout), dtype=T, device=self.dev)
+        # scratch operands from the engine's allocator (the shared pool when there is one), dropped on return
+        x = self._scratch((n, h, w, c.cin_store), T)
+        z = self._scratch((n, ho, wo, c.cout), T)
         wgt, wt = self._w(c.name + ".weight"), self._wt(c.name + ".weight")
-        part = torch.empty(ops.conv2d_fwd_stat_rows(x, c.cout, c.k, c.k, c.stride, c.pad, 2) * c.cout * 2,
-                           dtype=torch.float32, device=self.dev)
+        part = self._scratch((ops.conv2d_fwd_stat_rows(x, c.cout, c.k, c.k, c.stride, c.pad, 2) * c.cout * 2,),
+                             torch.float32)
         reps = 4
 
         def fwd(cfg):
@@ -299,10 +287,12 @@ class ResNetEngine(EngineBase):
                     ops.conv2d_fwd_bnstats(ctx, x, wgt, z, c.stride, c.pad, part, tile_cfg=cfg, c_logical=c.cin)
             return rec
 
-        mean, invstd = torch.zeros(c.cin_store, device=self.dev), torch.ones(c.cin_store, device=self.dev)
-        x2 = torch.ones_like(x)
-        dpart = torch.empty(ops.conv2d_dgrad_stat_rows(x, c.cout, c.k, c.k, c.stride, c.pad, 2) * c.cin_store * 2,
-                            dtype=torch.float32, device=self.dev)
+        mean = self._scratch((c.cin_store,), torch.float32)
+        invstd = self._scratch((c.cin_store,), torch.float32, 1.0)
+        x2 = self._scratch(tuple(x.shape), T, 1.0)
+        dpart = self._scratch((ops.conv2d_dgrad_stat_rows(x, c.cout, c.k, c.k, c.stride, c.pad, 2) * c.cin_store * 2,),
+                              torch.float32)
+        torch.cuda.synchronize()
 
         def dgrad(cfg):
             def rec():

@@ -72,6 +72,14 @@ class PeerScript:
             raise RuntimeError(f"PeerScript.stop: {len(alive)} command thread(s) still running after 5 s")
 
 
+def autotune_requested():
+    """COLTRAIN_AUTOTUNE=1: the engine times every tiling of each distinct layer shape whenever it builds the plan
+    of a new batch size and keeps the fastest (a few tenths of a second per plan, scratch tensors from the same
+    allocator as the activations).  Off by default: a colocated run rebuilds plans while the inference side waits
+    for memory."""
+    return os.environ.get("COLTRAIN_AUTOTUNE", "0") == "1"
+
+
 def attach_cu_partition(model):
     """With COLTRAIN_DYNAMIC_SM_PARTITION the engine asks the shared board before every launch segment how
     many compute units training may use (csrc/init.cc:43-71 + common/sm_partition.cc:96-112)."""

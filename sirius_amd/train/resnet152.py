@@ -19,7 +19,7 @@ import torch
 from .. import torch_col
 from ..resnet import ResNetEngine
 from ..torch_col import MemoryPool, dynamic_batch
-from .common import PeerScript, attach_cu_partition, cleanup, run_epochs, setup  # noqa: F401  (PeerScript is part of this module's interface)
+from .common import PeerScript, attach_cu_partition, autotune_requested, cleanup, run_epochs, setup  # noqa: F401  (PeerScript is part of this module's interface)
 
 
 def train(num_epoch: int, batch_size: int, global_batch_size: Optional[int] = None, dataset_size: int = 1000,
@@ -34,7 +34,8 @@ def train(num_epoch: int, batch_size: int, global_batch_size: Optional[int] = No
         torch_col.tag_model_start()
     allocator = torch_col.pool_empty if torch_col.is_enable_shared_tensor() else None
     model = ResNetEngine(depths=depths, width=width, num_classes=num_classes, dtype=dtype, image_size=image_size,
-                         lr=0.1, momentum=0.9, weight_decay=1e-4, stream=stream, allocator=allocator)
+                         lr=0.1, momentum=0.9, weight_decay=1e-4, stream=stream, allocator=allocator,
+                         autotune=autotune_requested())
     model.init_kaiming(seed)
     print(f"Train params memory usage: {MemoryPool.get_memory_usage() * 1024:.2f}M")
 
