@@ -124,11 +124,15 @@ class EngineBase:
         """Best-of-`reps` milliseconds of the launches `fn` records, replayed alone on this engine's stream."""
         prog = self._flat_prog(fn)
         self.ctx.run(prog)
+        self.ctx.synchronize()
         best = float("inf")
         for _ in range(reps):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record(self.ctx.stream)
             self.ctx.run(prog)
+            # behind a launch queue the launches reach the stream from the queue's own thread: the closing event
+            # must not overtake them
+            self.ctx.flush()
             e1.record(self.ctx.stream)
             e1.synchronize()
             best = min(best, e0.elapsed_time(e1))
