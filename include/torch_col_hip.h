@@ -48,11 +48,15 @@ uint64_t tch_context_take_rejected(tch_context* ctx);
 /* While recording: launches are stamped with `lane` (0 = the context's stream, 1 = may run beside
  * lane 0 on a second stream of the same priority); with wait_main the next lane-1 launch first
  * waits for everything lane 0 was given before it.  tch_context_join records the point where
- * lane 0 waits for lane 1.  A program stays a valid serial order: behind a registered
- * (preemptible) stream and under tch_program_profile it runs on one stream, in order.
+ * lane 0 waits for lane 1; tch_context_join_behind a point where lane 0 waits for what lane 1 had
+ * been given at the PREVIOUS such point (for a caller that rotates three sets of buffers: lane 1
+ * may trail by one set).  A program stays a valid serial order (tch_program_profile runs it on
+ * one stream, in order); behind a registered (preemptible) stream the lanes stay two streams and
+ * their meeting points are queued in order with the launches.
  * No counterpart in the reference (its backward runs on one stream). */
 int tch_context_set_lane(tch_context* ctx, int lane, int wait_main);
 int tch_context_join(tch_context* ctx);
+int tch_context_join_behind(tch_context* ctx);
 int tch_context_synchronize(tch_context* ctx); /* both streams of the context */
 
 /* ---- programs: record once, replay every step ---------------------------------- */

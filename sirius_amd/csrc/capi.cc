@@ -64,6 +64,14 @@ int tch_context_join(tch_context* ctx) {
   return ctx->ctx.record_join();
 }
 
+int tch_context_join_behind(tch_context* ctx) {
+  if (!ctx) {
+    set_error("tch_context_join_behind: null context");
+    return -22;
+  }
+  return ctx->ctx.record_join(true);
+}
+
 int tch_context_synchronize(tch_context* ctx) {
   if (!ctx) {
     set_error("tch_context_synchronize: null context");

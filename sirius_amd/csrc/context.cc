@@ -296,6 +296,10 @@ Context::~Context() {
     (void)hipStreamSynchronize(side);
     (void)hipStreamDestroy(side);
   }
+  if (relay) {
+    (void)hipStreamSynchronize(relay);
+    (void)hipStreamDestroy(relay);
+  }
   for (hipEvent_t e : events_) (void)hipEventDestroy(e);
 }
 
@@ -310,12 +314,12 @@ hipEvent_t Context::next_event() {
   return events_[event_next_++ % kRing];
 }
 
-int Context::record_join() {
+int Context::record_join(bool behind) {
   if (!recording) return 0;
   LaunchRecord rec{};
   rec.fn = nullptr;
-  rec.name = "join";
-  rec.op = kOpJoin;
+  rec.name = behind ? "join_behind" : "join";
+  rec.op = behind ? kOpJoinBehind : kOpJoin;
   recording->launches.push_back(rec);
   return 0;
 }
@@ -350,6 +354,7 @@ int Context::set_cu_limit(int n_cus) {
   if (side_dirty && old_side) {
     if (int rc = depend(old_side, new_main)) return rc;
     side_dirty = false;
+    relay_dirty = false;
   }
   cu_limit = n_cus;
   masked_main = n_cus > 0 ? new_main : nullptr;
@@ -375,6 +380,7 @@ int Context::synchronize() {
     return -5;
   }
   side_dirty = false;
+  relay_dirty = false;
   return 0;
 }
 
@@ -384,6 +390,22 @@ int Context::dispatch(const LaunchRecord& rec) {
     return 0;
   }
   hipStream_t main = main_stream();
+  if (rec.op == kOpJoinBehind) {
+    // depend() makes the event calls here, or queues them in order with the launches behind a launch queue
+    if (relay_dirty) {
+      if (int rc = depend(relay, main)) return rc;
+      relay_dirty = false;
+    }
+    if (side_dirty) {
+      if (!relay && hipStreamCreateWithFlags(&relay, hipStreamNonBlocking) != hipSuccess) {
+        set_error("hipStreamCreateWithFlags failed");
+        return -5;
+      }
+      if (int rc = depend(cu_limit > 0 ? masked_side : side, relay)) return rc;
+      relay_dirty = true;   // side_dirty stays up: lane 0 has not waited for this work yet
+    }
+    return 0;
+  }
   if (queue) {
     // behind the preemptible queue the two lanes stay two streams: what would be event calls here are
     // dependencies queued in order with the launches, and the worker makes them when their turn comes
@@ -392,6 +414,7 @@ int Context::dispatch(const LaunchRecord& rec) {
         queue->submit_dependency(cu_limit > 0 ? masked_side : side, main);
         side_dirty = false;
       }
+      relay_dirty = false;   // what the relay waits for is older than what lane 0 waits for now
       return 0;
     }
     if (!rec.fn) return 0;
@@ -419,6 +442,7 @@ int Context::dispatch(const LaunchRecord& rec) {
       }
       side_dirty = false;
     }
+    relay_dirty = false;
     return 0;
   }
   if (rec.lane == 1) {

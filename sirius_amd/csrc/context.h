@@ -134,11 +134,15 @@ class Context {
   // everything given to `to` afterwards waits for what `from` holds now (direct or through the queue)
   int depend(hipStream_t from, hipStream_t to);
   bool side_dirty = false;  // lane 1 was given work since the last join
+  // A join one point behind (kOpJoinBehind) goes through a stream of its own that carries nothing but waits:
+  // at such a point it is made to wait for lane 1, and lane 0 waits for it at the next one.
+  hipStream_t relay = nullptr;
+  bool relay_dirty = false;  // the relay waits for lane-1 work that lane 0 has not waited for
   // recording state: the lane new launches are stamped with, and whether the next lane-1 launch
   // has to wait for lane 0
   int lane = 0;
   bool wait_main = false;
-  int record_join();
+  int record_join(bool behind = false);
   int synchronize();  // both streams
   // set while the stream is registered for preemption; owned by the registry
   std::shared_ptr<LaunchQueue> queue;

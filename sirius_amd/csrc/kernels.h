@@ -196,11 +196,13 @@ struct LaunchRecord {
   //   kOpLaunch       plain launch on its lane
   //   kOpLaunchAfter  lane-1 launch that must see everything lane 0 was given before it
   //   kOpJoin         no kernel: lane 0 waits for everything lane 1 was given so far
+  //   kOpJoinBehind   no kernel: lane 0 waits for what lane 1 had been given at the PREVIOUS point of this kind
+  //                   (nothing at the first one), and lane 1's work up to here is what the next one waits for
   int lane;
   int op;
   alignas(16) unsigned char args[360];
 };
-enum LaunchOp : int { kOpLaunch = 0, kOpLaunchAfter = 1, kOpJoin = 2 };
+enum LaunchOp : int { kOpLaunch = 0, kOpLaunchAfter = 1, kOpJoin = 2, kOpJoinBehind = 3 };
 
 class Context;  // defined in context.h
 

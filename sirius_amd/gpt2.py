@@ -44,7 +44,8 @@ class _Plan:
 class GPT2Engine(EngineBase):
     def __init__(self, vocab=50257, n_pos=1024, n_embd=768, n_layer=12, n_head=12, seq_len=1024, dtype=torch.bfloat16,
                  optimizer="adamw", lr=1e-3, weight_decay=0.01, betas=(0.9, 0.999), eps=1e-8, momentum=0.9,
-                 stream=None, allocator=None, overlap_wgrad=True, fused_attention=True, autotune=False):
+                 stream=None, allocator=None, overlap_wgrad=True, fused_attention=True, autotune=False,
+                 trailing_wgrad=True):
         self._init_engine(dtype, stream, allocator)
         # autotune: when a plan is built, time each distinct projection shape with every tiling and keep the fastest
         self.autotune = autotune
@@ -52,6 +53,9 @@ class GPT2Engine(EngineBase):
         # the layer is done: recorded on a second lane, they run beside the data-gradient chain; the lanes
         # meet at the end of every layer, before its gradient buffers are handed round again
         self.overlap_wgrad = overlap_wgrad
+        # trailing_wgrad: three sets of gradient buffers taken in turn, so that the second lane may trail the first
+        # by a layer instead of meeting it at the end of every layer
+        self.trailing_wgrad = trailing_wgrad and overlap_wgrad
         self.fused_attention = fused_attention
         assert n_embd % n_head == 0 and n_embd % 8 == 0 and seq_len <= n_pos
         assert optimizer in ("adamw", "sgd")
@@ -332,8 +336,15 @@ class GPT2Engine(EngineBase):
             # ================= backward =================
             if self.overlap_wgrad:
                 ctx.join()      # the second lane may still be writing the transposed filters of the last optimizer step
-            g_c = [act(R, C) for _ in range(4)]       # gradients of [R, C] tensors, handed round
-            g_f1, g_f2, g_qkv = act(R, 4 * C), act(R, 4 * C), act(R, 3 * C)
+            # Gradient buffers, handed round.  The second lane reads a layer's incoming gradient and three of the
+            # layer's own (the right-hand sides of its four weight gradients).  With one set the lanes would have
+            # to meet at the end of every layer; with three sets taken in turn the second lane may trail the first
+            # by a layer: what layer j reads lies in the sets of layers j-1 and j, layer j+1 writes a third set,
+            # and before layer j+2 takes the first set again the main lane has waited for layer j's weight gradients.
+            n_sets = 3 if self.trailing_wgrad else 1
+            g_sets = [([act(R, C) for _ in range(4 if k == 0 else 3)], act(R, 4 * C), act(R, 3 * C)) for k in range(n_sets)]
+            g_c = g_sets[0][0]
+            g_f2 = act(R, 4 * C)                      # main lane only
             dP = act(B * H, T, dtype=torch.float32) if fused else act(B, H, T, T)   # fused: the delta scratch
             d_hf, g = g_c[0], g_c[1]
             with side():
@@ -345,8 +356,9 @@ class GPT2Engine(EngineBase):
             for i in range(L - 1, -1, -1):
                 pre = f"transformer.h.{i}."
                 h_in, a, qkv, P, o, h1, m, f1, f2 = saved[i]
+                own_c, g_f1, g_qkv = g_sets[(L - i) % n_sets]
                 flat, gflat = qkv.view(-1), g_qkv.view(-1)
-                spare = [t for t in g_c if t is not g]
+                spare = [t for t in own_c if t is not g]
                 d_m, g1, d_o = spare[0], spare[1], spare[2]
                 # MLP
                 lin_bwd(pre + "mlp.c_proj", f2, g, g_f2)
@@ -375,8 +387,10 @@ class GPT2Engine(EngineBase):
                 ln_bwd(pre + "ln_1", 2 * i, d_a, h_in, g_next, residual=g1)
                 g = g_next
                 if self.overlap_wgrad:
-                    ctx.join()
+                    ctx.join(behind=self.trailing_wgrad)
                 mark("bwd", f"h.{i}")
+            if self.overlap_wgrad:
+                ctx.join()
             # tied weights: the scattered embedding gradient lands on top of the head's weight gradient
             ops.embedding_bwd(ctx, plan.ids, g.view(B, T, C), self._view(self.grads, "transformer.wte.weight").view(Vp, C),
                               self._view(self.grads, "transformer.wpe.weight"), chain=act(2 * B * T, dtype=torch.int32))

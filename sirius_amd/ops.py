@@ -118,8 +118,14 @@ class Context:
         finally:
             check(lib().tch_context_set_lane(self.handle, 0, 0), "tch_context_set_lane")
 
-    def join(self):
-        check(lib().tch_context_join(self.handle), "tch_context_join")
+    def join(self, behind=False):
+        """While recording: the main lane waits for everything the second lane was given so far.  With `behind`
+        it waits for what the second lane had been given at the previous join(behind=True) only, so the second
+        lane may trail by one such section (whose buffers must then stay untouched for one section more)."""
+        if behind:
+            check(lib().tch_context_join_behind(self.handle), "tch_context_join_behind")
+        else:
+            check(lib().tch_context_join(self.handle), "tch_context_join")
 
     def set_cu_limit(self, n_cus):
         """From the next launch on, run on at most n_cus compute units (0 lifts the limit); needs

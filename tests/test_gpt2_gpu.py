@@ -186,6 +186,36 @@ def test_measured_tilings_change_no_bit():
         assert torch.equal(v, out[1][1][k]), k
 
 
+def test_trailing_weight_gradient_lane_changes_no_bit():
+    """trailing_wgrad rotates three sets of gradient buffers so that the weight-gradient lane may run a layer
+    behind the data-gradient chain (join one point behind) instead of meeting it after every layer.  Launch order
+    on each lane and every kernel's inputs are the same: three steps at GPT-2 small's widths, four layers deep
+    (so that every set is taken twice), give the same loss, gradients and weights bit for bit."""
+    from sirius_amd.gpt2 import GPT2Engine
+    cfg = dict(vocab=50257, n_pos=256, n_embd=768, n_layer=4, n_head=12)
+    sd = G.make_state_dict(cfg["vocab"], cfg["n_pos"], cfg["n_embd"], cfg["n_layer"], seed=6)
+    g = torch.Generator()
+    g.manual_seed(14)
+    ids = torch.randint(0, cfg["vocab"], (4, 256), generator=g).cuda()
+    out = []
+    for trailing in (False, True):
+        eng = GPT2Engine(seq_len=256, dtype=torch.bfloat16, trailing_wgrad=trailing, **cfg)
+        eng.load_state_dict(sd)
+        seen = []
+        for _ in range(3):
+            p, cut = eng.forward_backward(ids)
+            assert not cut
+            seen.append((eng.last_loss(), {k: v.clone() for k, v in eng.grads_dict().items()}))
+            eng.optimizer_step()
+        out.append((seen, eng.state_dict()))
+    for (la, ga), (lb, gb) in zip(out[0][0], out[1][0]):
+        assert la == lb
+        for k in ga:
+            assert torch.equal(ga[k], gb[k]), k
+    for k, v in out[0][1].items():
+        assert torch.equal(v, out[1][1][k]), k
+
+
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-3), (torch.bfloat16, 2e-2)])
 def test_gpt2_small_full_depth_1024_tokens(dtype, tol):
     """BASELINE configs[4]'s model as it is benchmarked -- 12 layers, 768 channels, 12 heads, vocabulary 50 257, a
