@@ -34,16 +34,19 @@ HANDOVER_PAGE_MB = 128
 # is what this file can measure itself, the in-step figure is what the trace shows.
 PROFILE_FILE = "profiles/resnet152_bf16_bs64_step_kernel_stats_and_traffic.txt"
 MEASURED_IN_STEP_US = {
-    "wgrad_kernel<bf16,128x128>": 35.52,
-    "igemm2_kernel<bf16,dgrad,128x64,2buf>": 51.56,
+    "wgrad_kernel<bf16,128x128>": 35.14,
+    "igemm2_kernel<bf16,dgrad,128x64,3buf,k32>": 47.66,
+    "igemm2_kernel<bf16,dgrad,128x64,3buf>": 37.41,
 }
 MEASURED_TRAFFIC_MIB = {
     "wgrad_kernel<bf16,128x128>": 31.79 + 13.77,
-    "igemm2_kernel<bf16,dgrad,128x128,2buf>": 67.94 + 32.72,
-    "igemm2_kernel<bf16,dgrad,128x64,3buf>": 63.10 + 31.49,
-    "igemm2_kernel<bf16,fwd,128x128,2buf>": 30.03 + 22.89,
-    "igemm2_kernel<bf16,fwd,128x64,3buf>": 35.10 + 18.06,
-    "igemm3_kernel<bf16,dgrad,128x64,3buf,patch160>": 29.72 + 5.90,
+    "igemm2_kernel<bf16,dgrad,128x64,3buf,k32>": 71.00 + 31.63,
+    "igemm2_kernel<bf16,dgrad,128x128,2buf>": 67.43 + 31.64,
+    "igemm2_kernel<bf16,dgrad,128x64,3buf>": 69.51 + 25.92,
+    "igemm2_kernel<bf16,fwd,128x128,2buf>": 29.62 + 22.39,
+    "igemm2_kernel<bf16,fwd,128x128,2buf,k32>": 35.75 + 29.29,
+    "igemm2_kernel<bf16,fwd,128x64,3buf>": 37.94 + 18.21,
+    "igemm3_kernel<bf16,dgrad,128x64,3buf,patch160>": 28.96 + 5.90,
     "bn_apply_kernel<bf16,bwd>": 72.04 + 34.61,
     "bn_apply_kernel<bf16,fwd>": 54.69 + 36.09,
 }
