@@ -33,6 +33,8 @@ class EngineBase:
         self._acc_prog = None
         self._opt_global_prog = None
         self.global_grads = None
+        self._linear_cache = {}    # (rows, in, out) -> (forward tiling, data-gradient tiling), see _tune_linear
+        self.linear_timings = {}   # what _tune_linear measured, per shape
 
     def plan(self, batch, loss_scale=1.0):
         key = (int(batch), float(loss_scale))
@@ -150,8 +152,6 @@ class EngineBase:
         """(forward tiling, data-gradient tiling) of a [rows, cin] -> [rows, cout] projection: every tiling timed
         once per distinct shape when a plan is built (the library's heuristic knows the tile count only, not how
         the shape sits on the chip).  Results per shape in ``linear_timings``."""
-        if not hasattr(self, "_linear_cache"):
-            self._linear_cache, self.linear_timings = {}, {}
         key = (int(rows), int(cin), int(cout))
         hit = self._linear_cache.get(key)
         if hit is not None:
