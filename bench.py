@@ -214,7 +214,7 @@ def gpt2_step(batch=8, seq_len=1024, warmup=2, steps=5):
     weights, token ids uniform in [0, 50257) of shape [8, 1024], AdamW.  Reported beside the headline figure."""
     import torch
     from sirius_amd.gpt2 import GPT2Engine
-    eng = GPT2Engine(seq_len=seq_len, dtype=torch.bfloat16, optimizer="adamw", autotune=True)
+    eng = GPT2Engine(seq_len=seq_len, dtype=torch.bfloat16, optimizer="adamw")
     eng.init_normal(0)
     g = torch.Generator(device="cuda")
     g.manual_seed(2)
@@ -264,7 +264,7 @@ def interleaving(batch=8, seq_len=1024, rate_per_s=50.0, train_s=3.0):
     xsched.register_stream(train_stream, False)
     server = None
     try:
-        eng = GPT2Engine(seq_len=seq_len, dtype=torch.bfloat16, optimizer="adamw", stream=train_stream, autotune=True)
+        eng = GPT2Engine(seq_len=seq_len, dtype=torch.bfloat16, optimizer="adamw", stream=train_stream)
         eng.init_normal(0)
         g = torch.Generator(device="cuda")
         g.manual_seed(2)
@@ -329,7 +329,7 @@ def swin_b_step(batch=32, warmup=2, steps=5):
     [32, 3, 224, 224] N(0,1), AdamW(lr 1e-3, wd 0.05), stochastic depth 0.  Reported beside the headline figure."""
     import torch
     from sirius_amd.swin import SwinEngine
-    eng = SwinEngine(dtype=torch.bfloat16, autotune=True)
+    eng = SwinEngine(dtype=torch.bfloat16)
     eng.init_normal(0)
     g = torch.Generator(device="cuda")
     g.manual_seed(3)

@@ -33,8 +33,6 @@ class EngineBase:
         self._acc_prog = None
         self._opt_global_prog = None
         self.global_grads = None
-        self._linear_cache = {}    # (rows, in, out) -> (forward tiling, data-gradient tiling), see _tune_linear
-        self.linear_timings = {}   # what _tune_linear measured, per shape
 
     def plan(self, batch, loss_scale=1.0):
         key = (int(batch), float(loss_scale))
@@ -143,45 +141,6 @@ class EngineBase:
     def _scratch(self, shape, dtype, fill=0.0):
         """A filled tensor from this engine's allocator, for measurements made while a plan is built."""
         return self._alloc(tuple(shape), dtype).fill_(fill)
-
-    # tilings offered to a projection: 0 / 1 / 2 = 128x128 / 128x64 / 64x64, 6 / 7 = 1 / 2 with two LDS tiles,
-    # 11 - 14 = the same shapes with 32-element reduction steps
-    _LINEAR_TILINGS = (0, 1, 2, 6, 7, 11, 12, 13, 14)
-
-    def _tune_linear(self, rows, cin, cout):
-        """(forward tiling, data-gradient tiling) of a [rows, cin] -> [rows, cout] projection: every tiling timed
-        once per distinct shape when a plan is built (the library's heuristic knows the tile count only, not how
-        the shape sits on the chip).  Results per shape in ``linear_timings``."""
-        key = (int(rows), int(cin), int(cout))
-        hit = self._linear_cache.get(key)
-        if hit is not None:
-            return hit
-        if self.dtype != torch.bfloat16 or cin % 64 or cout % 64:
-            self._linear_cache[key] = (-1, -1)   # the tilings differ for the direct-to-LDS kernel only
-            return -1, -1
-        ctx, T = self.ctx, self.dtype
-        x, y = self._scratch((rows, 1, 1, cin), T), self._scratch((rows, 1, 1, cout), T)
-        w, wt = self._scratch((cout, 1, 1, cin), T), self._scratch((cin, 1, 1, cout), T)
-        torch.cuda.synchronize()
-        reps = 4
-
-        def fwd(cfg):
-            def rec():
-                for _ in range(reps):
-                    ops.conv2d_fwd(ctx, x, w, y, 1, 0, tile_cfg=cfg)
-            return rec
-
-        def dgrad(cfg):
-            def rec():
-                for _ in range(reps):
-                    ops.conv2d_dgrad(ctx, y, wt, x, 1, 0, tile_cfg=cfg)
-            return rec
-        t_f = {cfg: self._time_program(fwd(cfg)) / reps for cfg in self._LINEAR_TILINGS if cfg not in (0, 11, 12) or cout > 64}
-        t_d = {cfg: self._time_program(dgrad(cfg)) / reps for cfg in self._LINEAR_TILINGS if cfg not in (0, 11, 12) or cin > 64}
-        best = (min(t_f, key=t_f.get), min(t_d, key=t_d.get))
-        self._linear_cache[key] = best
-        self.linear_timings[key] = {"fwd_ms": t_f, "dgrad_ms": t_d}
-        return best
 
     def ensure_global_grads(self):
         if self.global_grads is None:

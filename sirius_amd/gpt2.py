@@ -44,11 +44,8 @@ class _Plan:
 class GPT2Engine(EngineBase):
     def __init__(self, vocab=50257, n_pos=1024, n_embd=768, n_layer=12, n_head=12, seq_len=1024, dtype=torch.bfloat16,
                  optimizer="adamw", lr=1e-3, weight_decay=0.01, betas=(0.9, 0.999), eps=1e-8, momentum=0.9,
-                 stream=None, allocator=None, overlap_wgrad=True, fused_attention=True, autotune=False,
-                 trailing_wgrad=True):
+                 stream=None, allocator=None, overlap_wgrad=True, fused_attention=True, trailing_wgrad=True):
         self._init_engine(dtype, stream, allocator)
-        # autotune: when a plan is built, time each distinct projection shape with every tiling and keep the fastest
-        self.autotune = autotune
         # weight and bias gradients depend only on a saved activation and on a gradient that stays put until
         # the layer is done: recorded on a second lane, they run beside the data-gradient chain; the lanes
         # meet at the end of every layer, before its gradient buffers are handed round again
@@ -233,13 +230,6 @@ class GPT2Engine(EngineBase):
                 sp = int(ops.lib().tch_conv2d_wgrad_pick_splits(code, R, 1, 1, Cin, K, 1, 1, 1, 0))
                 ws_bytes = max(ws_bytes, ops.conv2d_wgrad_workspace_bytes(code, K, 1, 1, Cin, sp))
         wg_ws = act(ws_bytes // 4, dtype=torch.float32)
-        # (forward, data-gradient) tiling per projection shape, measured before the recording starts
-        tiles = {}
-        if self.autotune:
-            for p in self._specs:
-                if p.kind == "linear":
-                    K, _, _, Cin = p.store_shape
-                    tiles[(Cin, K)] = self._tune_linear(R, Cin, K)
 
         def ln_stats(i):
             return ln_mean[i * R:(i + 1) * R], ln_rstd[i * R:(i + 1) * R]
@@ -260,8 +250,7 @@ class GPT2Engine(EngineBase):
 
         def lin_fwd(name, x, y, add=None):
             ops.conv2d_fwd(ctx, as4(x), self._w(name + ".weight"), as4(y), 1, 0,
-                           bias=self._view(self.params, name + ".bias"), add=None if add is None else as4(add),
-                           tile_cfg=tiles.get((x.shape[1], y.shape[1]), (-1, -1))[0])
+                           bias=self._view(self.params, name + ".bias"), add=None if add is None else as4(add))
 
         def side():
             return ctx.side_lane(wait_main=True) if self.overlap_wgrad else contextlib.nullcontext()
@@ -271,8 +260,7 @@ class GPT2Engine(EngineBase):
             with side():
                 ops.conv2d_wgrad(ctx, as4(x), as4(dy), self._view(self.grads, name + ".weight"), 1, 0, workspace=wg_ws,
                                  dbias=self._view(self.grads, name + ".bias"))
-            ops.conv2d_dgrad(ctx, as4(dy), self._wt(name + ".weight"), as4(dx), 1, 0,
-                             tile_cfg=tiles.get((dx.shape[1], dy.shape[1]), (-1, -1))[1])
+            ops.conv2d_dgrad(ctx, as4(dy), self._wt(name + ".weight"), as4(dx), 1, 0)
 
         # strides / batch offsets of head h of sample b inside the packed projection and the score tensor
         qkv_row, qkv_b = 3 * C, (T * 3 * C, D)

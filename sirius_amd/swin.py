@@ -70,10 +70,8 @@ def shifted_window_mask(H, W, ws, shift):
 class SwinEngine(EngineBase):
     def __init__(self, embed=128, depths=(2, 2, 18, 2), heads=(4, 8, 16, 32), window=7, patch=4, image_size=224,
                  num_classes=1000, dtype=torch.bfloat16, lr=1e-3, weight_decay=0.05, betas=(0.9, 0.999), eps=1e-8,
-                 stream=None, allocator=None, overlap_wgrad=True, fused_attention=True, autotune=False):
+                 stream=None, allocator=None, overlap_wgrad=True, fused_attention=True):
         self._init_engine(dtype, stream, allocator)
-        # autotune: when a plan is built, time each distinct projection shape with every tiling and keep the fastest
-        self.autotune = autotune
         # weight / bias / bias-table gradients on a second lane beside the data-gradient chain; the lanes meet
         # at the end of every block, before its gradient buffers are handed round again
         self.overlap_wgrad = overlap_wgrad
@@ -274,11 +272,6 @@ class SwinEngine(EngineBase):
             sp = int(ops.lib().tch_conv2d_wgrad_pick_splits(code, n_, h_, w_, cin, k_, r_, s_, stride, 0))
             ws_bytes = max(ws_bytes, ops.conv2d_wgrad_workspace_bytes(code, k_, r_, s_, cin, sp))
         wg_ws = act(ws_bytes // 4, dtype=torch.float32)
-        # (forward, data-gradient) tiling per projection shape, measured before the recording starts
-        tiles = {}
-        if self.autotune:
-            for n_, h_, w_, cin, k_, r_, s_, stride in calls[2:]:
-                tiles[(n_, cin, k_)] = self._tune_linear(n_, cin, k_)
         bias_ws = act(64 * 4 * self.feat, dtype=torch.float32)
 
         def ln_fwd(name, x, y, stats):
@@ -296,8 +289,7 @@ class SwinEngine(EngineBase):
         def lin_fwd(name, x, y, add=None, bias=True):
             ops.conv2d_fwd(ctx, as4(x), self._w(name + ".weight"), as4(y), 1, 0,
                            bias=self._view(self.params, name + ".bias") if bias else None,
-                           add=None if add is None else as4(add),
-                           tile_cfg=tiles.get((x.shape[0], x.shape[1], y.shape[1]), (-1, -1))[0])
+                           add=None if add is None else as4(add))
 
         def side():
             return ctx.side_lane(wait_main=True) if self.overlap_wgrad else contextlib.nullcontext()
@@ -307,8 +299,7 @@ class SwinEngine(EngineBase):
                 ops.conv2d_wgrad(ctx, as4(x), as4(dy), self._view(self.grads, name + ".weight"), 1, 0, workspace=wg_ws,
                                  dbias=self._view(self.grads, name + ".bias") if bias else None)
             if dx is not None:
-                ops.conv2d_dgrad(ctx, as4(dy), self._wt(name + ".weight"), as4(dx), 1, 0,
-                                 tile_cfg=tiles.get((dx.shape[0], dx.shape[1], dy.shape[1]), (-1, -1))[1])
+                ops.conv2d_dgrad(ctx, as4(dy), self._wt(name + ".weight"), as4(dx), 1, 0)
 
         # scratch the blocks share (program order is the only hazard: one lane)
         def flat(n):
@@ -499,8 +490,7 @@ class SwinEngine(EngineBase):
                     with side():
                         ops.conv2d_wgrad(ctx, as4(nm), as4(g), self._view(self.grads, pre + "reduction.weight"), 1, 0,
                                          workspace=wg_ws)
-                    ops.conv2d_dgrad(ctx, as4(g), self._wt(pre + "reduction.weight"), as4(d_nm), 1, 0,
-                                     tile_cfg=tiles.get((rows // 4, 4 * C, 2 * C), (-1, -1))[1])
+                    ops.conv2d_dgrad(ctx, as4(g), self._wt(pre + "reduction.weight"), as4(d_nm), 1, 0)
                     d_xm = v2(g_4c_b, rows // 4, 4 * C)
                     ln_bwd(pre + "norm", d_nm, xm, d_xm, mstats)
                     gi = spare[0]

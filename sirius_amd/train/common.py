@@ -73,7 +73,7 @@ class PeerScript:
 
 
 def autotune_requested():
-    """COLTRAIN_AUTOTUNE=1: the engine times every tiling of each distinct layer shape whenever it builds the plan
+    """COLTRAIN_AUTOTUNE=1 (train/resnet152.py): the engine times every tiling of each distinct layer shape whenever it builds the plan
     of a new batch size and keeps the fastest (a few tenths of a second per plan, scratch tensors from the same
     allocator as the activations).  Off by default: a colocated run rebuilds plans while the inference side waits
     for memory."""

@@ -17,7 +17,7 @@ import torch
 from .. import torch_col
 from ..gpt2 import GPT2Engine
 from ..torch_col import MemoryPool, dynamic_batch
-from .common import PeerScript, attach_cu_partition, autotune_requested, run_epochs, setup
+from .common import PeerScript, attach_cu_partition, run_epochs, setup
 
 
 def train(num_epoch: int, batch_size: int, global_batch_size: Optional[int] = None, dataset_size: int = 500,
@@ -33,7 +33,7 @@ def train(num_epoch: int, batch_size: int, global_batch_size: Optional[int] = No
     allocator = torch_col.pool_empty if torch_col.is_enable_shared_tensor() else None
     hp = dict(lr=0.1, momentum=0.9, weight_decay=1e-4) if optimizer == "sgd" else dict(lr=1e-3, weight_decay=0.01)
     model = GPT2Engine(seq_len=seq_len, dtype=dtype, optimizer=optimizer, stream=stream, allocator=allocator, **hp,
-                       autotune=autotune_requested(), **model_config)
+                       **model_config)
     model.init_normal(seed)
     print(f"Train params memory usage: {MemoryPool.get_memory_usage() * 1024:.2f}M")
 

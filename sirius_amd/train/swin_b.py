@@ -15,7 +15,7 @@ import torch
 from .. import torch_col
 from ..swin import SwinEngine
 from ..torch_col import MemoryPool, dynamic_batch
-from .common import PeerScript, attach_cu_partition, autotune_requested, run_epochs, setup
+from .common import PeerScript, attach_cu_partition, run_epochs, setup
 
 
 def train(num_epoch: int, batch_size: int, global_batch_size: Optional[int] = None, dataset_size: int = 1000,
@@ -29,7 +29,7 @@ def train(num_epoch: int, batch_size: int, global_batch_size: Optional[int] = No
     if torch_col.is_enable_shared_tensor():
         torch_col.tag_model_start()
     allocator = torch_col.pool_empty if torch_col.is_enable_shared_tensor() else None
-    model = SwinEngine(dtype=dtype, stream=stream, allocator=allocator, autotune=autotune_requested(), **model_config)
+    model = SwinEngine(dtype=dtype, stream=stream, allocator=allocator, **model_config)
     model.init_normal(seed)
     print(f"Train params memory usage: {MemoryPool.get_memory_usage() * 1024:.2f}M")
 

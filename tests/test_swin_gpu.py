@@ -292,28 +292,6 @@ def test_fused_attention_step():
     assert abs(losses[0] - losses[1]) <= 5e-3 * abs(losses[1])
 
 
-def test_measured_tilings_change_no_bit():
-    """SwinEngine(autotune=True) runs every projection with the tiling that was fastest when the plan was built:
-    same bits as with the library's own choice (every tiling adds up an output's products in the same order)."""
-    cfg = S.config(**CFGS["window7"])
-    sd = S.make_state_dict(cfg, seed=3)
-    g = _gen(12)
-    x = torch.randn(2, 3, cfg["image"], cfg["image"], generator=g).cuda()
-    y = torch.randint(0, cfg["classes"], (2,), generator=g).cuda()
-    out = []
-    for tune in (False, True):
-        eng = _engine(cfg, torch.bfloat16, autotune=tune)
-        eng.load_state_dict(sd)
-        p, cut = eng.forward_backward(x, y)
-        assert not cut
-        out.append((eng.last_loss(), {k: v.clone() for k, v in eng.grads_dict().items()}))
-        if tune:
-            assert len(eng.linear_timings) >= 8, eng.linear_timings.keys()
-    assert out[0][0] == out[1][0]
-    for k, v in out[0][1].items():
-        assert torch.equal(v, out[1][1][k]), k
-
-
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-3), (torch.bfloat16, 2e-2)])
 def test_swin_b_real_config_loss_and_every_gradient(dtype, tol):
     """BASELINE configs[3]'s model at its real configuration (embed 128, depths 2/2/18/2, heads 4/8/16/32, window
