@@ -141,7 +141,8 @@ int tch_program_run(tch_context* ctx, const tch_program* prog, int64_t first, in
   if (limited)
     if (int rc = ctx->ctx.depend(ctx->ctx.stream, ctx->ctx.main_stream())) return rc;
   for (int64_t i = first; i < last; ++i) {
-    int rc = ctx->ctx.dispatch(prog->prog.launches[static_cast<size_t>(i)]);
+    const auto& launches = prog->prog.launches;
+    int rc = ctx->ctx.dispatch(launches[static_cast<size_t>(i)], i + 1 < last ? &launches[static_cast<size_t>(i + 1)] : nullptr);
     if (rc) return rc;
   }
   if (limited)

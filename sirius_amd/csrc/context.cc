@@ -1,5 +1,7 @@
 #include "context.h"
 
+#include <hip/hip_ext.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <map>
@@ -17,14 +19,24 @@ int g_queue_length = 16;
 // is worth 1.2 ms per ResNet-152 step here; one per launch costs more in event records than it saves.
 int g_sync_interval = 4;
 
-int launch_now(hipStream_t stream, const LaunchRecord& rec) {
+int launch_now(hipStream_t stream, const LaunchRecord& rec, hipEvent_t stop_event = nullptr) {
   void* args[1] = {const_cast<unsigned char*>(rec.args)};
-  hipError_t e = hipLaunchKernel(rec.fn, rec.grid, rec.block, args, 0, stream);
+  hipError_t e = stop_event ? hipExtLaunchKernel(rec.fn, rec.grid, rec.block, args, 0, stream, nullptr, stop_event, 0)
+                           : hipLaunchKernel(rec.fn, rec.grid, rec.block, args, 0, stream);
   if (e != hipSuccess) {
     set_error(std::string("hipLaunchKernel failed: ") + hipGetErrorString(e));
     return -5;
   }
   return 0;
+}
+
+// TCH_FORK_STOP_EVENT=0: every fork to the second lane records an event of its own behind the lane-0 kernel
+bool fork_by_stop_event() {
+  static const bool on = [] {
+    const char* e = getenv("TCH_FORK_STOP_EVENT");
+    return !(e && atoi(e) == 0);
+  }();
+  return on;
 }
 }  // namespace
 
@@ -212,15 +224,21 @@ void LaunchQueue::drain_log_until(size_t keep) {
   in_flight_.store(log_.size());
 }
 
-void LaunchQueue::launch_one(const LaunchRecord& rec, hipStream_t on) {
+void LaunchQueue::launch_one(const LaunchRecord& rec, hipStream_t on, bool fork_follows) {
   if (log_.size() >= queue_length_) drain_log_until(queue_length_ - 1);
   hipStream_t target = on ? on : stream_;
   void* args[1] = {const_cast<unsigned char*>(rec.args)};
-  hipError_t e = hipLaunchKernel(rec.fn, rec.grid, rec.block, args, 0, target);
+  // a launch that a dependency on its stream follows carries that dependency's event as its stop event
+  hipEvent_t stop = fork_follows ? take_event() : nullptr;
+  hipError_t e = stop ? hipExtLaunchKernel(rec.fn, rec.grid, rec.block, args, 0, target, nullptr, stop, 0)
+                      : hipLaunchKernel(rec.fn, rec.grid, rec.block, args, 0, target);
   if (e != hipSuccess) {
+    if (stop) free_events_.push_back(stop);
     error_.store(static_cast<int>(e));
     return;
   }
+  fork_event_ = stop;
+  fork_from_ = target;
   const uint64_t idx = ++next_idx_;
   StreamState& st = state_of(target);
   hipEvent_t ev = nullptr;
@@ -242,6 +260,7 @@ void LaunchQueue::worker_loop() {
   (void)hipSetDevice(device_);
   for (;;) {
     Item item;
+    bool fork_follows = false;
     {
       std::unique_lock<std::mutex> lock(mu_);
       cv_work_.wait(lock, [&] { return stop_ || (suspended_ ? !parked_ : !wait_.empty()); });
@@ -263,10 +282,24 @@ void LaunchQueue::worker_loop() {
       }
       item = wait_.front();
       wait_.pop_front();
+      fork_follows = !item.is_dependency && !item.is_sync && fork_by_stop_event() && !wait_.empty() &&
+                     wait_.front().is_dependency && wait_.front().on == (item.on ? item.on : stream_);
     }
     if (item.is_dependency) {
-      chain(item.on, item.to);
+      if (fork_event_ && fork_from_ == item.on && item.to != item.on) {
+        // the launch before this entry signals fork_event_ when it ends; as in chain(), the event may be used
+        // again once the wait is enqueued
+        if (hipStreamWaitEvent(item.to, fork_event_, 0) != hipSuccess) error_.store(static_cast<int>(hipErrorUnknown));
+        free_events_.push_back(fork_event_);
+        fork_event_ = nullptr;
+      } else {
+        chain(item.on, item.to);
+      }
       continue;
+    }
+    if (fork_event_) {   // nobody asked for it after all
+      free_events_.push_back(fork_event_);
+      fork_event_ = nullptr;
     }
     if (item.is_sync) {
       sync_everything();
@@ -276,7 +309,7 @@ void LaunchQueue::worker_loop() {
       }
       cv_done_.notify_all();
     } else {
-      launch_one(item.rec, item.on);
+      launch_one(item.rec, item.on, fork_follows);
     }
   }
   // release waiters that raced with shutdown
@@ -384,9 +417,10 @@ int Context::synchronize() {
   return 0;
 }
 
-int Context::dispatch(const LaunchRecord& rec) {
+int Context::dispatch(const LaunchRecord& rec, const LaunchRecord* next) {
   if (g_reject.load(std::memory_order_acquire)) {
     if (rec.fn) rejected.fetch_add(1);
+    fork_event_ = nullptr;
     return 0;
   }
   hipStream_t main = main_stream();
@@ -452,14 +486,28 @@ int Context::dispatch(const LaunchRecord& rec) {
     }
     hipStream_t s = cu_limit > 0 ? masked_side : side;
     if (rec.op == kOpLaunchAfter) {
-      hipEvent_t e = next_event();
-      if (!e || hipEventRecord(e, main) != hipSuccess || hipStreamWaitEvent(s, e, 0) != hipSuccess) {
-        set_error("fork to the side stream failed");
-        return -5;
+      hipEvent_t e = fork_event_;
+      fork_event_ = nullptr;
+      if (e) {   // the lane-0 kernel before this record signals e when it ends
+        if (hipStreamWaitEvent(s, e, 0) != hipSuccess) {
+          set_error("fork to the side stream failed");
+          return -5;
+        }
+      } else {
+        e = next_event();
+        if (!e || hipEventRecord(e, main) != hipSuccess || hipStreamWaitEvent(s, e, 0) != hipSuccess) {
+          set_error("fork to the side stream failed");
+          return -5;
+        }
       }
     }
     side_dirty = true;
     return launch_now(s, rec);
+  }
+  fork_event_ = nullptr;
+  if (next && next->fn && next->lane == 1 && next->op == kOpLaunchAfter && fork_by_stop_event()) {
+    fork_event_ = next_event();
+    return launch_now(main, rec, fork_event_);
   }
   return launch_now(main, rec);
 }

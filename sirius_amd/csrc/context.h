@@ -78,7 +78,7 @@ class LaunchQueue {
     uint64_t since_event;  // launches on the stream since its last sync point
   };
   void worker_loop();
-  void launch_one(const LaunchRecord& rec, hipStream_t on);
+  void launch_one(const LaunchRecord& rec, hipStream_t on, bool fork_follows);
   void chain(hipStream_t from, hipStream_t to);
   void drain_log_until(size_t keep);
   void sync_everything();
@@ -103,6 +103,8 @@ class LaunchQueue {
   // worker-private
   std::deque<Logged> log_;
   std::vector<hipEvent_t> free_events_;
+  hipEvent_t fork_event_ = nullptr;   // stop event of the launch just made, for a dependency entry right behind it
+  hipStream_t fork_from_ = nullptr;
   std::vector<StreamState> streams_;  // every stream a launch went to since the last full synchronisation
   uint64_t next_idx_ = 0;
 
@@ -150,10 +152,15 @@ class Context {
   // launches skipped because the reject flag was up since the last reset
   std::atomic<uint64_t> rejected{0};
 
-  int dispatch(const LaunchRecord& rec);
+  // `next`: the record that follows in the program being replayed (nullptr: none or unknown).  A lane-0 launch
+  // that is followed by a lane-1 launch which has to wait for it carries the event of that wait as its own stop
+  // event (the kernel's completion signal), so that no separate event record stands between it and the next
+  // lane-0 kernel in the queue.
+  int dispatch(const LaunchRecord& rec, const LaunchRecord* next = nullptr);
 
  private:
   hipEvent_t next_event();
+  hipEvent_t fork_event_ = nullptr;  // stop event of the last lane-0 launch, not yet waited for by lane 1
   std::vector<hipEvent_t> events_;
   size_t event_next_ = 0;
 };
