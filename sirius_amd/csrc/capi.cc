@@ -135,6 +135,7 @@ int tch_program_run(tch_context* ctx, const tch_program* prog, int64_t first, in
   // the stream may have been registered after the context was made
   ctx->ctx.queue = queue_for_stream(reinterpret_cast<uint64_t>(ctx->ctx.stream));
   const uint64_t before = ctx->ctx.rejected.load();
+  ctx->ctx.note_foreign_work();   // the caller may have given the stream work of its own since the last run
   // with a compute-unit limit the launches go to another stream than the caller's: order them behind
   // what the caller's stream holds, and what the caller does next behind them
   const bool limited = ctx->ctx.cu_limit > 0 && first < last;

@@ -390,6 +390,7 @@ int Context::set_cu_limit(int n_cus) {
     relay_dirty = false;
   }
   cu_limit = n_cus;
+  main_since_fork_ = true;   // another pair of streams
   masked_main = n_cus > 0 ? new_main : nullptr;
   masked_side = n_cus > 0 ? new_side : nullptr;
   return 0;
@@ -458,11 +459,15 @@ int Context::dispatch(const LaunchRecord& rec, const LaunchRecord* next) {
         return -5;
       }
       hipStream_t s = cu_limit > 0 ? masked_side : side;
-      if (rec.op == kOpLaunchAfter) queue->submit_dependency(main, s);
+      if (rec.op == kOpLaunchAfter && main_since_fork_) {
+        queue->submit_dependency(main, s);
+        main_since_fork_ = false;
+      }
       side_dirty = true;
       queue->submit(rec, s);
       return 0;
     }
+    main_since_fork_ = true;
     queue->submit(rec, main);
     return 0;
   }
@@ -485,7 +490,8 @@ int Context::dispatch(const LaunchRecord& rec, const LaunchRecord* next) {
       return -5;
     }
     hipStream_t s = cu_limit > 0 ? masked_side : side;
-    if (rec.op == kOpLaunchAfter) {
+    if (rec.op == kOpLaunchAfter && main_since_fork_) {
+      main_since_fork_ = false;
       hipEvent_t e = fork_event_;
       fork_event_ = nullptr;
       if (e) {   // the lane-0 kernel before this record signals e when it ends
@@ -505,6 +511,7 @@ int Context::dispatch(const LaunchRecord& rec, const LaunchRecord* next) {
     return launch_now(s, rec);
   }
   fork_event_ = nullptr;
+  main_since_fork_ = true;
   if (next && next->fn && next->lane == 1 && next->op == kOpLaunchAfter && fork_by_stop_event()) {
     fork_event_ = next_event();
     return launch_now(main, rec, fork_event_);

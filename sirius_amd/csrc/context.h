@@ -145,6 +145,8 @@ class Context {
   int lane = 0;
   bool wait_main = false;
   int record_join(bool behind = false);
+  // work reached lane 0's stream from outside this context: the next fork has to wait for it
+  void note_foreign_work() { main_since_fork_ = true; }
   int synchronize();  // both streams
   // set while the stream is registered for preemption; owned by the registry
   std::shared_ptr<LaunchQueue> queue;
@@ -161,6 +163,8 @@ class Context {
  private:
   hipEvent_t next_event();
   hipEvent_t fork_event_ = nullptr;  // stop event of the last lane-0 launch, not yet waited for by lane 1
+  // lane 0 was given a launch since lane 1 last waited for it (a fork with nothing new to wait for is skipped)
+  bool main_since_fork_ = true;
   std::vector<hipEvent_t> events_;
   size_t event_next_ = 0;
 };
