@@ -313,6 +313,19 @@ int tch_layernorm_bwd(tch_context* ctx, int dtype, const void* dy, const void* x
                       const float* gamma,
                       const float* mean, const float* rstd, float* dgamma, float* dbeta, int accumulate, int64_t rows,
                       int C, float* partial);
+/* LayerNorm next to a window partition (Swin: train/swin_b_tiny.py:8-19, 116-131 roll + window_partition /
+ * window_reverse around the attention of a block).  rows = B * H * W pixels in row order; x, mean and rstd stay in
+ * that order.  Forward: y is written as window tokens (cyclic shift by -shift, then window x window windows), i.e.
+ * LayerNorm and partition in one pass.  Backward: windowed_tensors flags which of dx (1), dy (2) and the residual (4)
+ * are laid out as window tokens; the others are pixel rows.  Same values as the plain call followed / preceded
+ * by tch_window_partition. */
+int tch_layernorm_fwd_windowed(tch_context* ctx, int dtype, const void* x, void* y, const float* gamma, const float* beta,
+                               float* mean, float* rstd, int64_t rows, int C, float eps, int H, int W, int window,
+                               int shift);
+int tch_layernorm_bwd_windowed(tch_context* ctx, int dtype, const void* dy, const void* x, void* dx, const void* residual,
+                               const float* gamma, const float* mean, const float* rstd, float* dgamma, float* dbeta,
+                               int accumulate, int64_t rows, int C, float* partial, int H, int W, int window, int shift,
+                               int windowed_tensors);
 /* tanh_form 0: 0.5 x (1 + erf(x / sqrt 2)) (nn.GELU); 1: GPT-2's gelu_new.  n is a multiple of a 16-byte chunk. */
 int tch_gelu_fwd(tch_context* ctx, int dtype, const void* x, void* y, int64_t n, int tanh_form);
 int tch_gelu_bwd(tch_context* ctx, int dtype, const void* dy, const void* x, void* dx, int64_t n, int tanh_form);

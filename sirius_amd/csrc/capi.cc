@@ -261,6 +261,22 @@ int tch_layernorm_fwd(tch_context* ctx, int dtype, const void* x, void* y, const
   return layernorm_fwd(C(ctx), dtype, x, y, gamma, beta, mean, rstd, rows, Cc, eps);
 }
 
+int tch_layernorm_fwd_windowed(tch_context* ctx, int dtype, const void* x, void* y, const float* gamma, const float* beta,
+                               float* mean, float* rstd, int64_t rows, int Cc, float eps, int H, int W, int window,
+                               int shift) {
+  LnWindow win{H, W, window, shift, 1};
+  return layernorm_fwd(C(ctx), dtype, x, y, gamma, beta, mean, rstd, rows, Cc, eps, &win);
+}
+
+int tch_layernorm_bwd_windowed(tch_context* ctx, int dtype, const void* dy, const void* x, void* dx, const void* residual,
+                               const float* gamma, const float* mean, const float* rstd, float* dgamma, float* dbeta,
+                               int accumulate, int64_t rows, int Cc, float* partial, int H, int W, int window, int shift,
+                               int windowed_tensors) {
+  LnWindow win{H, W, window, shift, windowed_tensors};
+  return layernorm_bwd(C(ctx), dtype, dy, x, dx, residual, gamma, mean, rstd, dgamma, dbeta, accumulate, rows, Cc,
+                       partial, &win);
+}
+
 int tch_layernorm_bwd_partial_rows(int64_t rows) { return layernorm_bwd_partial_rows(rows); }
 
 int tch_layernorm_bwd(tch_context* ctx, int dtype, const void* dy, const void* x, void* dx, const void* residual,

@@ -118,12 +118,17 @@ int bn_bwd_partials(Context* ctx, int dtype, const void* g, const void* x, void*
                     float* dbeta, int accumulate, const float* partial, int row_blocks, float* scratch);
 
 // seq_ops.hip
+// Window order (Swin): rows = B * H * W pixels; a tensor flagged in `tensors` (1 = output, 2 = dy, 4 = the addend) is
+// laid out as window tokens (cyclic shift by -shift, then ws x ws windows) instead of pixel rows.  ws == 0: none.
+struct LnWindow {
+  int H = 0, W = 0, ws = 0, shift = 0, tensors = 0;
+};
 int layernorm_fwd(Context* ctx, int dtype, const void* x, void* y, const float* gamma, const float* beta, float* mean,
-                  float* rstd, int64_t rows, int C, float eps);
+                  float* rstd, int64_t rows, int C, float eps, const LnWindow* win = nullptr);
 int layernorm_bwd_partial_rows(int64_t rows);  // rows of [C][2] fp32 scratch layernorm_bwd needs
 int layernorm_bwd(Context* ctx, int dtype, const void* dy, const void* x, void* dx, const void* residual, const float* gamma,
                   const float* mean, const float* rstd, float* dgamma, float* dbeta, int accumulate, int64_t rows,
-                  int C, float* partial);
+                  int C, float* partial, const LnWindow* win = nullptr);
 int gelu_fwd(Context* ctx, int dtype, const void* x, void* y, int64_t n, int tanh_form);
 int gelu_bwd(Context* ctx, int dtype, const void* dy, const void* x, void* dx, int64_t n, int tanh_form);
 int attn_softmax_fwd(Context* ctx, int dtype, const void* scores, void* probs, int64_t batch, int heads, int Lq, int Lk,

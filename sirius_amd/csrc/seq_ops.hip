@@ -41,7 +41,27 @@ struct LnArgs {
   int C, cc;
   int rows_per_wg;
   float eps;
+  // Optional window order (Swin): rows are the pixels of [B, win_h, win_w] images; a tensor flagged below is laid
+  // out as window tokens instead (cyclic shift by -win_shift, then win_ws x win_ws windows) and is reached through
+  // window_row().  win_ws == 0: every tensor is in row order.
+  int win_h, win_w, win_ws, win_shift;
+  int win_out;   // forward: y   backward: dx
+  int win_dy;    // backward: dy
+  int win_add;   // backward: the addend
 };
+
+// pixel row (b, h, w) -> its window token (b, wh, ww, i, j): h - shift = wh * ws + i, w - shift = ww * ws + j (mod H, W)
+__device__ inline int64_t window_row(const LnArgs& p, int64_t row) {
+  const int w = static_cast<int>(row % p.win_w);
+  int64_t t = row / p.win_w;
+  const int h = static_cast<int>(t % p.win_h);
+  t /= p.win_h;
+  int hs = h - p.win_shift, wsft = w - p.win_shift;
+  if (hs < 0) hs += p.win_h;
+  if (wsft < 0) wsft += p.win_w;
+  const int wh = hs / p.win_ws, i = hs - wh * p.win_ws, ww = wsft / p.win_ws, j = wsft - ww * p.win_ws;
+  return (((t * (p.win_h / p.win_ws) + wh) * (p.win_w / p.win_ws) + ww) * p.win_ws + i) * p.win_ws + j;
+}
 
 // L lanes per row (L = 64: one wavefront per row, NCH 16-byte chunks per lane; L = 16 or 32: short rows, 64 / L
 // rows per wavefront, one chunk per lane); the row stays in registers between the passes
@@ -105,7 +125,7 @@ __global__ __launch_bounds__(256) void ln_fwd_kernel(LnArgs p) {
     p.mean[row] = mean;
     p.rstd[row] = rstd;
   }
-  uint4* dst = static_cast<uint4*>(p.out) + row * p.cc;
+  uint4* dst = static_cast<uint4*>(p.out) + (p.win_ws && p.win_out ? window_row(p, row) : row) * p.cc;
 #pragma unroll
   for (int j = 0; j < NCH; ++j) {
     const int c = sub + j * L;
@@ -149,6 +169,7 @@ __global__ __launch_bounds__(256) void ln_bwd_kernel(LnArgs p) {
   constexpr int R = 2;
   for (int64_t base = r0; base < r1; base += R * GROUPS) {
     bool live[R];
+    int64_t wrows[R];
     float mean[R], rstd[R];
     Chunk cx[R][NCH], cg[R][NCH], cr[R][NCH];
 #pragma unroll
@@ -156,18 +177,21 @@ __global__ __launch_bounds__(256) void ln_bwd_kernel(LnArgs p) {
       const int64_t row = base + q * GROUPS + group;
       live[q] = row < r1;
       mean[q] = rstd[q] = 0.f;
+      int64_t wrow = row;
       if (live[q]) {
         mean[q] = p.mean[row];
         rstd[q] = p.rstd[row];
+        if (p.win_ws) wrow = window_row(p, row);
       }
+      wrows[q] = wrow;
 #pragma unroll
       for (int j = 0; j < NCH; ++j) {
         const int c = sub + j * L;
         cx[q][j] = cg[q][j] = cr[q][j] = zero_chunk();
         if (live[q] && c < p.cc) {
           cx[q][j].u = (static_cast<const uint4*>(p.x) + row * p.cc)[c];
-          cg[q][j].u = (static_cast<const uint4*>(p.dy) + row * p.cc)[c];
-          if (p.add) cr[q][j].u = (static_cast<const uint4*>(p.add) + row * p.cc)[c];
+          cg[q][j].u = (static_cast<const uint4*>(p.dy) + (p.win_dy ? wrow : row) * p.cc)[c];
+          if (p.add) cr[q][j].u = (static_cast<const uint4*>(p.add) + (p.win_add ? wrow : row) * p.cc)[c];
         }
       }
     }
@@ -196,7 +220,7 @@ __global__ __launch_bounds__(256) void ln_bwd_kernel(LnArgs p) {
       a = row_sum<L>(a) * inv_c;
       b = row_sum<L>(b) * inv_c;
       if (!live[q]) continue;
-      uint4* dst = static_cast<uint4*>(p.out) + row * p.cc;
+      uint4* dst = static_cast<uint4*>(p.out) + (p.win_out ? wrows[q] : row) * p.cc;
 #pragma unroll
       for (int j = 0; j < NCH; ++j) {
         const int c = sub + j * L;
@@ -646,13 +670,32 @@ int layernorm_bwd_partial_rows(int64_t rows) {
   return static_cast<int>((rows + r - 1) / r);
 }
 
+int bind_window(LnArgs& a, const LnWindow* win, int64_t rows, int allowed) {
+  if (!win || win->ws == 0) return 0;
+  TCH_CHECK_ARG(win->H > 0 && win->W > 0 && win->ws > 0 && win->H % win->ws == 0 && win->W % win->ws == 0,
+                "layernorm: the window must tile the image");
+  TCH_CHECK_ARG(win->shift >= 0 && win->shift < win->ws, "layernorm: shift must be in [0, window)");
+  TCH_CHECK_ARG(rows % (static_cast<int64_t>(win->H) * win->W) == 0, "layernorm: rows must be whole images");
+  TCH_CHECK_ARG((win->tensors & ~allowed) == 0, "layernorm: a tensor flagged as window-ordered does not exist in this direction");
+  a.win_h = win->H;
+  a.win_w = win->W;
+  a.win_ws = win->ws;
+  a.win_shift = win->shift;
+  a.win_out = win->tensors & 1;
+  a.win_dy = (win->tensors >> 1) & 1;
+  a.win_add = (win->tensors >> 2) & 1;
+  return 0;
+}
+
 int layernorm_fwd(Context* ctx, int dtype, const void* x, void* y, const float* gamma, const float* beta, float* mean,
-                  float* rstd, int64_t rows, int C, float eps) {
+                  float* rstd, int64_t rows, int C, float eps, const LnWindow* win) {
   if (int rc = check_rows("layernorm_fwd", dtype, rows, C)) return rc;
   const int E = dtype == kBF16 ? 8 : 4;
   TCH_CHECK_ARG(C <= kLnMaxC, "layernorm: rows longer than 2048 elements are not supported");
   TCH_CHECK_ARG(x && y && gamma && beta && mean && rstd, "layernorm_fwd: null tensor");
   LnArgs a{x, nullptr, nullptr, y, gamma, beta, mean, rstd, nullptr, rows, C, C / E, 0, eps};
+  if (int rc = bind_window(a, win, rows, 1)) return rc;
+  TCH_CHECK_ARG(!(a.win_out && x == y), "layernorm_fwd: a window-ordered output cannot overwrite the input");
   const double bytes = static_cast<double>(rows) * C * (dtype == kBF16 ? 4.0 : 8.0);
   const LnShape sh = ln_shape(a.cc);
   const dim3 grid(static_cast<unsigned>((rows + 4 * (64 / sh.lanes) - 1) / (4 * (64 / sh.lanes))));
@@ -662,7 +705,7 @@ int layernorm_fwd(Context* ctx, int dtype, const void* x, void* y, const float* 
 
 int layernorm_bwd(Context* ctx, int dtype, const void* dy, const void* x, void* dx, const void* residual, const float* gamma,
                   const float* mean, const float* rstd, float* dgamma, float* dbeta, int accumulate, int64_t rows,
-                  int C, float* partial) {
+                  int C, float* partial, const LnWindow* win) {
   if (int rc = check_rows("layernorm_bwd", dtype, rows, C)) return rc;
   const int E = dtype == kBF16 ? 8 : 4;
   TCH_CHECK_ARG(C <= kLnMaxC, "layernorm: rows longer than 2048 elements are not supported");
@@ -671,6 +714,10 @@ int layernorm_bwd(Context* ctx, int dtype, const void* dy, const void* x, void* 
   const int blocks = static_cast<int>((rows + rpw - 1) / rpw);
   LnArgs a{x,    dy,   residual, dx, gamma, nullptr, const_cast<float*>(mean), const_cast<float*>(rstd), partial,
            rows, C,    C / E,    rpw, 0.f};
+  if (int rc = bind_window(a, win, rows, residual ? 7 : 3)) return rc;
+  // a workgroup reads and writes rows of its own only while source and destination are in the same order
+  TCH_CHECK_ARG(!(dx == dy && a.win_out != a.win_dy) && !(dx == residual && a.win_out != a.win_add),
+                "layernorm_bwd: dx may overwrite an operand only where both are in the same order");
   const double bytes = static_cast<double>(rows) * C * (dtype == kBF16 ? 6.0 : 12.0);
   const LnShape sh = ln_shape(a.cc);
   int rc = dtype == kBF16 ? launch(ctx, ln_kernel_for<bf16, true>(sh), dim3(blocks), dim3(256), a, "ln_bwd_kernel<bf16>", bytes, 1)

@@ -629,12 +629,19 @@ def cast_to_f32(ctx, src, dst):
 # transformer operators (Swin-B / GPT-2 steps)
 # ---------------------------------------------------------------------------
 
-def layernorm_fwd(ctx, x, y, gamma, beta, mean, rstd, eps=1e-5):
+def layernorm_fwd(ctx, x, y, gamma, beta, mean, rstd, eps=1e-5, window=None):
+    """window = (H, W, window size, shift): x is [B*H*W, C] in pixel order and y is written as window tokens (the
+    LayerNorm and the window partition that follows it in a Swin block in one pass)."""
     C = x.shape[-1]
     rows = x.numel() // C
     assert y.shape == x.shape and y.dtype == x.dtype and x.is_contiguous() and y.is_contiguous()
     assert gamma.numel() == C and beta.numel() == C and gamma.dtype == beta.dtype == torch.float32
     assert mean.numel() == rows and rstd.numel() == rows and mean.dtype == rstd.dtype == torch.float32
+    if window is not None:
+        H, W, ws, shift = window
+        check(lib().tch_layernorm_fwd_windowed(ctx.handle, dtype_code(x), _p(x), _p(y), _p(gamma), _p(beta), _p(mean),
+                                               _p(rstd), rows, C, eps, H, W, ws, shift), "tch_layernorm_fwd_windowed")
+        return
     check(lib().tch_layernorm_fwd(ctx.handle, dtype_code(x), _p(x), _p(y), _p(gamma), _p(beta), _p(mean), _p(rstd),
                                   rows, C, eps), "tch_layernorm_fwd")
 
@@ -643,12 +650,22 @@ def layernorm_bwd_partial_rows(rows):
     return int(lib().tch_layernorm_bwd_partial_rows(rows))
 
 
-def layernorm_bwd(ctx, dy, x, dx, gamma, mean, rstd, dgamma, dbeta, partial, accumulate=False, residual=None):
+def layernorm_bwd(ctx, dy, x, dx, gamma, mean, rstd, dgamma, dbeta, partial, accumulate=False, residual=None,
+                  window=None, windowed=()):
+    """window = (H, W, window size, shift) and windowed, a subset of ("dx", "dy", "residual"): those tensors are laid
+    out as window tokens, everything else ([B*H*W, C] x, the statistics) in pixel order."""
     C = x.shape[-1]
     rows = x.numel() // C
     assert dy.shape == x.shape == dx.shape and dy.dtype == x.dtype == dx.dtype
     assert partial.dtype == torch.float32 and partial.numel() >= layernorm_bwd_partial_rows(rows) * C * 2
     assert residual is None or (residual.shape == x.shape and residual.dtype == x.dtype)
+    if window is not None:
+        H, W, ws, shift = window
+        flags = sum({"dx": 1, "dy": 2, "residual": 4}[t] for t in windowed)
+        check(lib().tch_layernorm_bwd_windowed(ctx.handle, dtype_code(x), _p(dy), _p(x), _p(dx), _p(residual), _p(gamma),
+                                               _p(mean), _p(rstd), _p(dgamma), _p(dbeta), int(accumulate), rows, C,
+                                               _p(partial), H, W, ws, shift, flags), "tch_layernorm_bwd_windowed")
+        return
     check(lib().tch_layernorm_bwd(ctx.handle, dtype_code(x), _p(dy), _p(x), _p(dx), _p(residual), _p(gamma), _p(mean), _p(rstd),
                                   _p(dgamma), _p(dbeta), int(accumulate), rows, C, _p(partial)), "tch_layernorm_bwd")
 

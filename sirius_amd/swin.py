@@ -70,11 +70,13 @@ def shifted_window_mask(H, W, ws, shift):
 class SwinEngine(EngineBase):
     def __init__(self, embed=128, depths=(2, 2, 18, 2), heads=(4, 8, 16, 32), window=7, patch=4, image_size=224,
                  num_classes=1000, dtype=torch.bfloat16, lr=1e-3, weight_decay=0.05, betas=(0.9, 0.999), eps=1e-8,
-                 stream=None, allocator=None, overlap_wgrad=True, fused_attention=True):
+                 stream=None, allocator=None, overlap_wgrad=True, fused_attention=True, fuse_window_ln=True):
         self._init_engine(dtype, stream, allocator)
         # weight / bias / bias-table gradients on a second lane beside the data-gradient chain; the lanes meet
         # at the end of every block, before its gradient buffers are handed round again
         self.overlap_wgrad = overlap_wgrad
+        # fuse_window_ln: the LayerNorms next to a window partition read / write window order themselves
+        self.fuse_window_ln = fuse_window_ln
         self.fused_attention = fused_attention
         assert len(depths) == len(heads) and image_size % patch == 0 and num_classes % 8 == 0 and embed % 8 == 0
         self.embed, self.depths, self.heads = embed, tuple(depths), tuple(heads)
@@ -274,14 +276,14 @@ class SwinEngine(EngineBase):
         wg_ws = act(ws_bytes // 4, dtype=torch.float32)
         bias_ws = act(64 * 4 * self.feat, dtype=torch.float32)
 
-        def ln_fwd(name, x, y, stats):
+        def ln_fwd(name, x, y, stats, window=None):
             ops.layernorm_fwd(ctx, x, y, self._view(self.params, name + ".weight"), self._view(self.params, name + ".bias"),
-                              stats[0], stats[1])
+                              stats[0], stats[1], window=window)
 
-        def ln_bwd(name, dy, x, dx, stats, residual=None):
+        def ln_bwd(name, dy, x, dx, stats, residual=None, window=None, windowed=()):
             ops.layernorm_bwd(ctx, dy, x, dx, self._view(self.params, name + ".weight"), stats[0], stats[1],
                               self._view(self.grads, name + ".weight"), self._view(self.grads, name + ".bias"), ln_partial,
-                              residual=residual)
+                              residual=residual, window=window, windowed=windowed)
 
         def as4(t):
             return t.view(t.shape[0], 1, 1, t.shape[1])
@@ -397,6 +399,9 @@ class SwinEngine(EngineBase):
                     if whole:
                         xw = act(rows, C)
                         ln_fwd(pre + "norm1", x, xw, stats1)
+                    elif self.fuse_window_ln:
+                        xw = act(rows, C)   # LayerNorm and window partition in one pass
+                        ln_fwd(pre + "norm1", x, xw, stats1, window=(R, R, ws, shift))
                     else:
                         n1, xw = v2(s_n1, rows, C), act(rows, C)
                         ln_fwd(pre + "norm1", x, n1, stats1)
@@ -513,11 +518,19 @@ class SwinEngine(EngineBase):
                     ops.gelu_bwd(ctx, d_f2, f1, d_f1, tanh_form=False)
                     lin_bwd(pre + "mlp.0", n2, d_f1, t_a)
                     g1 = t_b
-                    ln_bwd(pre + "norm2", t_a, x1, g1, stats2, residual=g)
+                    fuse_w = self.fuse_window_ln and not whole
+                    win = (R, R, ws, shift)
                     # attention
-                    if whole:
+                    if fuse_w:
+                        # the gradient behind norm2 is written as window tokens right away: the projection's gradients
+                        # want it in that order, and norm1's backward reads its residual through the same map
+                        ln_bwd(pre + "norm2", t_a, x1, g1, stats2, residual=g, window=win, windowed=("dx",))
+                        d_pr = g1
+                    elif whole:
+                        ln_bwd(pre + "norm2", t_a, x1, g1, stats2, residual=g)
                         d_pr = g1
                     else:
+                        ln_bwd(pre + "norm2", t_a, x1, g1, stats2, residual=g)
                         d_pr = t_a
                         ops.window_partition(ctx, g1, d_pr, ws, shift, image_shape=(B, R, R, C))
                     d_o = t_c
@@ -547,15 +560,19 @@ class SwinEngine(EngineBase):
                                          qkv_b, alpha=scale)
                     d_xw = t_d
                     lin_bwd(pre + "attn.qkv", xw, d_qkv, d_xw)
-                    if whole:
-                        d_n1 = d_xw
-                    else:
-                        d_n1 = t_c
-                        ops.window_partition(ctx, d_xw, d_n1, ws, shift, reverse=True, image_shape=(B, R, R, C))
                     # the new running gradient goes into a buffer of its own: the old one may still be read by
                     # this block's first weight gradient on the second lane
                     g_next = t_e
-                    ln_bwd(pre + "norm1", d_n1, x_in, g_next, stats1, residual=g1)
+                    if fuse_w:
+                        ln_bwd(pre + "norm1", d_xw, x_in, g_next, stats1, residual=g1, window=win,
+                               windowed=("dy", "residual"))
+                    else:
+                        if whole:
+                            d_n1 = d_xw
+                        else:
+                            d_n1 = t_c
+                            ops.window_partition(ctx, d_xw, d_n1, ws, shift, reverse=True, image_shape=(B, R, R, C))
+                        ln_bwd(pre + "norm1", d_n1, x_in, g_next, stats1, residual=g1)
                     g, gi = g_next, spare[4]
                     if self.overlap_wgrad:
                         ctx.join()

@@ -44,6 +44,82 @@ def test_window_partition_is_a_bit_exact_permutation(ctx, dtype, B, H, W, C, ws,
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,H,W,C,ws,shift", [(2, 8, 8, 128, 4, 0), (2, 8, 12, 256, 4, 2), (1, 14, 14, 512, 7, 3), (3, 28, 28, 64, 7, 3),
+                                              (2, 14, 14, 1024, 7, 0)])
+def test_layernorm_in_window_order_equals_layernorm_and_partition(ctx, dtype, B, H, W, C, ws, shift):
+    """The LayerNorm that writes window tokens (forward) and the ones that read / write them (backward) give the
+    bits of the plain LayerNorm calls with tch_window_partition between them: outputs, statistics, dgamma, dbeta."""
+    from sirius_amd import ops
+    g = _gen(52)
+    rows = B * H * W
+    img = (B, H, W, C)
+    x = torch.randn(rows, C, generator=g).to(dtype).cuda()
+    gamma, beta = (torch.rand(C, generator=g) + 0.5).cuda(), torch.randn(C, generator=g).cuda()
+    new = lambda: torch.empty(rows, C, dtype=dtype, device="cuda")
+    stat = lambda: (torch.empty(rows, device="cuda"), torch.empty(rows, device="cuda"))
+    # forward
+    y_rows, y_win, y_fused = new(), new(), new()
+    st, st_f = stat(), stat()
+    ops.layernorm_fwd(ctx, x, y_rows, gamma, beta, *st)
+    ops.window_partition(ctx, y_rows, y_win, ws, shift, image_shape=img)
+    ops.layernorm_fwd(ctx, x, y_fused, gamma, beta, *st_f, window=(H, W, ws, shift))
+    torch.cuda.synchronize()
+    assert torch.equal(y_fused, y_win) and torch.equal(st[0], st_f[0]) and torch.equal(st[1], st_f[1])
+    # backward: every combination of window-ordered dx, dy and residual against explicit permutations
+    dy_rows = torch.randn(rows, C, generator=g).to(dtype).cuda()
+    res_rows = torch.randn(rows, C, generator=g).to(dtype).cuda()
+    dy_win, res_win = new(), new()
+    ops.window_partition(ctx, dy_rows, dy_win, ws, shift, image_shape=img)
+    ops.window_partition(ctx, res_rows, res_win, ws, shift, image_shape=img)
+    partial = torch.empty(ops.layernorm_bwd_partial_rows(rows) * C * 2, device="cuda")
+    dx_ref, dg_ref, db_ref = new(), torch.zeros(C, device="cuda"), torch.zeros(C, device="cuda")
+    ops.layernorm_bwd(ctx, dy_rows, x, dx_ref, gamma, st[0], st[1], dg_ref, db_ref, partial, residual=res_rows)
+    dx_ref_win = new()
+    ops.window_partition(ctx, dx_ref, dx_ref_win, ws, shift, image_shape=img)
+    for windowed in [(), ("dx",), ("dy",), ("residual",), ("dy", "residual"), ("dx", "dy", "residual")]:
+        dx, dg, db = new(), torch.zeros(C, device="cuda"), torch.zeros(C, device="cuda")
+        ops.layernorm_bwd(ctx, dy_win if "dy" in windowed else dy_rows, x, dx, gamma, st[0], st[1], dg, db, partial,
+                          residual=res_win if "residual" in windowed else res_rows, window=(H, W, ws, shift),
+                          windowed=windowed)
+        torch.cuda.synchronize()
+        assert torch.equal(dx, dx_ref_win if "dx" in windowed else dx_ref), windowed
+        assert torch.equal(dg, dg_ref) and torch.equal(db, db_ref), windowed
+    with pytest.raises(Exception):   # in place across two orders
+        ops.layernorm_bwd(ctx, dy_rows, x, dy_rows, gamma, st[0], st[1], dg, db, partial, window=(H, W, ws, shift),
+                          windowed=("dx",))
+
+
+@pytest.mark.parametrize("name,dtype", [("window7", torch.bfloat16), ("shifted", torch.float32)])
+def test_window_order_layernorms_change_no_bit(name, dtype):
+    """SwinEngine(fuse_window_ln=True) drops three window-partition launches per block: same loss, gradients and
+    weights after three steps as with the separate launches."""
+    cfg = S.config(**CFGS[name])
+    sd = S.make_state_dict(cfg, seed=4)
+    g = _gen(13)
+    x = torch.randn(3, 3, cfg["image"], cfg["image"], generator=g).cuda()
+    y = torch.randint(0, cfg["classes"], (3,), generator=g).cuda()
+    out = []
+    for fuse in (False, True):
+        eng = _engine(cfg, dtype, fuse_window_ln=fuse)
+        eng.load_state_dict(sd)
+        seen = []
+        for _ in range(3):
+            p, cut = eng.forward_backward(x, y)
+            assert not cut
+            seen.append((eng.last_loss(), {k: v.clone() for k, v in eng.grads_dict().items()}))
+            eng.optimizer_step()
+        names = [r["name"] for r in eng.ctx.profile(p.prog, 1)]
+        assert any("window_kernel" in n for n in names) == (not fuse) or name == "shifted", names
+        out.append((seen, eng.state_dict()))
+    for (la, ga), (lb, gb) in zip(out[0][0], out[1][0]):
+        assert la == lb
+        for k in ga:
+            assert torch.equal(ga[k], gb[k]), k
+    for k, v in out[0][1].items():
+        assert torch.equal(v, out[1][1][k]), k
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("B,H,W,C", [(2, 8, 8, 16), (1, 14, 6, 32), (3, 2, 2, 8)])
 def test_patch_merge_gather_is_a_bit_exact_permutation(ctx, dtype, B, H, W, C):
     from sirius_amd import ops
