@@ -315,13 +315,15 @@ int tch_layernorm_bwd(tch_context* ctx, int dtype, const void* dy, const void* x
                       int C, float* partial);
 /* LayerNorm next to a window partition (Swin: train/swin_b_tiny.py:8-19, 116-131 roll + window_partition /
  * window_reverse around the attention of a block).  rows = B * H * W pixels in row order; x, mean and rstd stay in
- * that order.  Forward: y is written as window tokens (cyclic shift by -shift, then window x window windows), i.e.
- * LayerNorm and partition in one pass.  Backward: windowed_tensors flags which of dx (1), dy (2) and the residual (4)
- * are laid out as window tokens; the others are pixel rows.  Same values as the plain call followed / preceded
- * by tch_window_partition. */
+ * that order.  windowed_tensors flags the tensors that are laid out as window tokens (cyclic shift by -shift, then
+ * window x window windows) instead: forward y (1) and the addend (4); backward dx (1), dy (2), the residual (4).
+ * Forward with an addend (add, sum_out both non-NULL; sum_out in pixel order): sum_out = x + add rounded to the
+ * tensors' type, y = LayerNorm(sum_out): the residual sum behind the attention of a block (window_reverse + add)
+ * and the LayerNorm in front of its MLP in one pass.  Same values as the plain calls with tch_window_partition
+ * between them. */
 int tch_layernorm_fwd_windowed(tch_context* ctx, int dtype, const void* x, void* y, const float* gamma, const float* beta,
                                float* mean, float* rstd, int64_t rows, int C, float eps, int H, int W, int window,
-                               int shift);
+                               int shift, int windowed_tensors, const void* add, void* sum_out);
 int tch_layernorm_bwd_windowed(tch_context* ctx, int dtype, const void* dy, const void* x, void* dx, const void* residual,
                                const float* gamma, const float* mean, const float* rstd, float* dgamma, float* dbeta,
                                int accumulate, int64_t rows, int C, float* partial, int H, int W, int window, int shift,

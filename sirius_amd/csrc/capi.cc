@@ -263,9 +263,9 @@ int tch_layernorm_fwd(tch_context* ctx, int dtype, const void* x, void* y, const
 
 int tch_layernorm_fwd_windowed(tch_context* ctx, int dtype, const void* x, void* y, const float* gamma, const float* beta,
                                float* mean, float* rstd, int64_t rows, int Cc, float eps, int H, int W, int window,
-                               int shift) {
-  LnWindow win{H, W, window, shift, 1};
-  return layernorm_fwd(C(ctx), dtype, x, y, gamma, beta, mean, rstd, rows, Cc, eps, &win);
+                               int shift, int windowed_tensors, const void* add, void* sum_out) {
+  LnWindow win{H, W, window, shift, windowed_tensors};
+  return layernorm_fwd(C(ctx), dtype, x, y, gamma, beta, mean, rstd, rows, Cc, eps, &win, add, sum_out);
 }
 
 int tch_layernorm_bwd_windowed(tch_context* ctx, int dtype, const void* dy, const void* x, void* dx, const void* residual,

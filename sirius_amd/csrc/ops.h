@@ -124,7 +124,8 @@ struct LnWindow {
   int H = 0, W = 0, ws = 0, shift = 0, tensors = 0;
 };
 int layernorm_fwd(Context* ctx, int dtype, const void* x, void* y, const float* gamma, const float* beta, float* mean,
-                  float* rstd, int64_t rows, int C, float eps, const LnWindow* win = nullptr);
+                  float* rstd, int64_t rows, int C, float eps, const LnWindow* win = nullptr,
+                  const void* add = nullptr, void* sum_out = nullptr);  // with add: sum_out = x + add, y = LN(sum_out)
 int layernorm_bwd_partial_rows(int64_t rows);  // rows of [C][2] fp32 scratch layernorm_bwd needs
 int layernorm_bwd(Context* ctx, int dtype, const void* dy, const void* x, void* dx, const void* residual, const float* gamma,
                   const float* mean, const float* rstd, float* dgamma, float* dbeta, int accumulate, int64_t rows,

@@ -31,6 +31,8 @@ struct LnArgs {
   const void* x;
   const void* dy;  // backward
   const void* add; // backward, optional: added to dx (the residual branch's gradient)
+                   // forward, optional: added to x before anything else; the sum, rounded to T, goes to sum_out
+  void* sum_out;   // forward with add: x + add in row order
   void* out;       // forward: y   backward: dx
   const float* gamma;
   const float* beta;
@@ -94,6 +96,7 @@ __global__ __launch_bounds__(256) void ln_fwd_kernel(LnArgs p) {
   const int64_t row = (static_cast<int64_t>(blockIdx.x) * 4 + wave) * RPW + lane / L;
   const bool live = row < p.rows;
   const uint4* src = static_cast<const uint4*>(p.x) + row * p.cc;
+  const int64_t wrow = (live && p.win_ws) ? window_row(p, row) : row;
   float v[NCH][E];
   float s = 0.f;
 #pragma unroll
@@ -103,6 +106,18 @@ __global__ __launch_bounds__(256) void ln_fwd_kernel(LnArgs p) {
       Chunk ch;
       ch.u = src[c];
       chunk_to_float<T>(ch, v[j]);
+      if (p.add) {
+        // the residual sum of a block: rounded to T as the separate addition would leave it, kept for later
+        Chunk ca;
+        ca.u = (static_cast<const uint4*>(p.add) + (p.win_add ? wrow : row) * p.cc)[c];
+        float a[E];
+        chunk_to_float<T>(ca, a);
+#pragma unroll
+        for (int e = 0; e < E; ++e) v[j][e] += a[e];
+        ch = float_to_chunk<T>(v[j]);
+        chunk_to_float<T>(ch, v[j]);
+        (static_cast<uint4*>(p.sum_out) + row * p.cc)[c] = ch.u;
+      }
 #pragma unroll
       for (int e = 0; e < E; ++e) s += v[j][e];
     }
@@ -125,7 +140,7 @@ __global__ __launch_bounds__(256) void ln_fwd_kernel(LnArgs p) {
     p.mean[row] = mean;
     p.rstd[row] = rstd;
   }
-  uint4* dst = static_cast<uint4*>(p.out) + (p.win_ws && p.win_out ? window_row(p, row) : row) * p.cc;
+  uint4* dst = static_cast<uint4*>(p.out) + (p.win_out ? wrow : row) * p.cc;
 #pragma unroll
   for (int j = 0; j < NCH; ++j) {
     const int c = sub + j * L;
@@ -688,15 +703,17 @@ int bind_window(LnArgs& a, const LnWindow* win, int64_t rows, int allowed) {
 }
 
 int layernorm_fwd(Context* ctx, int dtype, const void* x, void* y, const float* gamma, const float* beta, float* mean,
-                  float* rstd, int64_t rows, int C, float eps, const LnWindow* win) {
+                  float* rstd, int64_t rows, int C, float eps, const LnWindow* win, const void* add, void* sum_out) {
   if (int rc = check_rows("layernorm_fwd", dtype, rows, C)) return rc;
   const int E = dtype == kBF16 ? 8 : 4;
   TCH_CHECK_ARG(C <= kLnMaxC, "layernorm: rows longer than 2048 elements are not supported");
   TCH_CHECK_ARG(x && y && gamma && beta && mean && rstd, "layernorm_fwd: null tensor");
-  LnArgs a{x, nullptr, nullptr, y, gamma, beta, mean, rstd, nullptr, rows, C, C / E, 0, eps};
-  if (int rc = bind_window(a, win, rows, 1)) return rc;
-  TCH_CHECK_ARG(!(a.win_out && x == y), "layernorm_fwd: a window-ordered output cannot overwrite the input");
-  const double bytes = static_cast<double>(rows) * C * (dtype == kBF16 ? 4.0 : 8.0);
+  TCH_CHECK_ARG((add == nullptr) == (sum_out == nullptr), "layernorm_fwd: an addend goes with a place for the sum");
+  LnArgs a{x, nullptr, add, sum_out, y, gamma, beta, mean, rstd, nullptr, rows, C, C / E, 0, eps};
+  if (int rc = bind_window(a, win, rows, add ? 5 : 1)) return rc;
+  TCH_CHECK_ARG(!(a.win_out && (x == y || sum_out == y)), "layernorm_fwd: a window-ordered output cannot overwrite a row-ordered tensor");
+  TCH_CHECK_ARG(!(a.win_add && (sum_out == add || y == add)), "layernorm_fwd: a window-ordered addend cannot be overwritten in row order");
+  const double bytes = static_cast<double>(rows) * C * (dtype == kBF16 ? 4.0 : 8.0) * (add ? 2.0 : 1.0);
   const LnShape sh = ln_shape(a.cc);
   const dim3 grid(static_cast<unsigned>((rows + 4 * (64 / sh.lanes) - 1) / (4 * (64 / sh.lanes))));
   return dtype == kBF16 ? launch(ctx, ln_kernel_for<bf16, false>(sh), grid, dim3(256), a, "ln_fwd_kernel<bf16>", bytes, 1)
@@ -712,8 +729,8 @@ int layernorm_bwd(Context* ctx, int dtype, const void* dy, const void* x, void* 
   TCH_CHECK_ARG(dy && x && dx && gamma && mean && rstd && dgamma && dbeta && partial, "layernorm_bwd: null tensor");
   const int rpw = ln_rows_per_wg(rows);
   const int blocks = static_cast<int>((rows + rpw - 1) / rpw);
-  LnArgs a{x,    dy,   residual, dx, gamma, nullptr, const_cast<float*>(mean), const_cast<float*>(rstd), partial,
-           rows, C,    C / E,    rpw, 0.f};
+  LnArgs a{x,    dy,   residual, nullptr, dx,  gamma, nullptr, const_cast<float*>(mean), const_cast<float*>(rstd),
+           partial, rows, C, C / E, rpw, 0.f};
   if (int rc = bind_window(a, win, rows, residual ? 7 : 3)) return rc;
   // a workgroup reads and writes rows of its own only while source and destination are in the same order
   TCH_CHECK_ARG(!(dx == dy && a.win_out != a.win_dy) && !(dx == residual && a.win_out != a.win_add),

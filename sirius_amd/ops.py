@@ -629,9 +629,10 @@ def cast_to_f32(ctx, src, dst):
 # transformer operators (Swin-B / GPT-2 steps)
 # ---------------------------------------------------------------------------
 
-def layernorm_fwd(ctx, x, y, gamma, beta, mean, rstd, eps=1e-5, window=None):
-    """window = (H, W, window size, shift): x is [B*H*W, C] in pixel order and y is written as window tokens (the
-    LayerNorm and the window partition that follows it in a Swin block in one pass)."""
+def layernorm_fwd(ctx, x, y, gamma, beta, mean, rstd, eps=1e-5, window=None, windowed=("y",), add=None, sum_out=None):
+    """window = (H, W, window size, shift): x is [B*H*W, C] in pixel order; the tensors named in `windowed` ("y",
+    "add") are laid out as window tokens (the LayerNorm and the window partition next to it in a Swin block in one
+    pass).  add / sum_out: sum_out = x + add (pixel order, rounded to the tensors' type), y = LayerNorm(sum_out)."""
     C = x.shape[-1]
     rows = x.numel() // C
     assert y.shape == x.shape and y.dtype == x.dtype and x.is_contiguous() and y.is_contiguous()
@@ -639,9 +640,14 @@ def layernorm_fwd(ctx, x, y, gamma, beta, mean, rstd, eps=1e-5, window=None):
     assert mean.numel() == rows and rstd.numel() == rows and mean.dtype == rstd.dtype == torch.float32
     if window is not None:
         H, W, ws, shift = window
+        assert (add is None) == (sum_out is None)
+        assert add is None or (add.numel() == x.numel() == sum_out.numel() and add.dtype == sum_out.dtype == x.dtype)
+        flags = sum({"y": 1, "add": 4}[t] for t in windowed)
         check(lib().tch_layernorm_fwd_windowed(ctx.handle, dtype_code(x), _p(x), _p(y), _p(gamma), _p(beta), _p(mean),
-                                               _p(rstd), rows, C, eps, H, W, ws, shift), "tch_layernorm_fwd_windowed")
+                                               _p(rstd), rows, C, eps, H, W, ws, shift, flags, _p(add), _p(sum_out)),
+              "tch_layernorm_fwd_windowed")
         return
+    assert add is None and sum_out is None, "the residual sum comes with the windowed form"
     check(lib().tch_layernorm_fwd(ctx.handle, dtype_code(x), _p(x), _p(y), _p(gamma), _p(beta), _p(mean), _p(rstd),
                                   rows, C, eps), "tch_layernorm_fwd")
 

@@ -276,9 +276,9 @@ class SwinEngine(EngineBase):
         wg_ws = act(ws_bytes // 4, dtype=torch.float32)
         bias_ws = act(64 * 4 * self.feat, dtype=torch.float32)
 
-        def ln_fwd(name, x, y, stats, window=None):
+        def ln_fwd(name, x, y, stats, window=None, **kw):
             ops.layernorm_fwd(ctx, x, y, self._view(self.params, name + ".weight"), self._view(self.params, name + ".bias"),
-                              stats[0], stats[1], window=window)
+                              stats[0], stats[1], window=window, **kw)
 
         def ln_bwd(name, dy, x, dx, stats, residual=None, window=None, windowed=()):
             ops.layernorm_bwd(ctx, dy, x, dx, self._view(self.params, name + ".weight"), stats[0], stats[1],
@@ -426,14 +426,20 @@ class SwinEngine(EngineBase):
                         ops.attn_softmax_fwd(ctx, Pm, Pm, 1.0, bias=bias, mask=st["mask_dev"] if shift else None)
                         ops.batched_gemm(ctx, Pm, fq[2 * C:], o, N, D, N, (N, 1), (1, qkv_row), C, (B_, Hh), s_b, qkv_b, o_b)
                     x1 = act(rows, C)
+                    n2, f1, f2, x2 = act(rows, C), act(rows, 4 * C), act(rows, 4 * C), act(rows, C)
                     if whole:
                         lin_fwd(pre + "attn.proj", o, x1, add=x)
+                        ln_fwd(pre + "norm2", x1, n2, stats2)
+                    elif self.fuse_window_ln:
+                        # x1 = x + window_reverse(projection) and n2 = LayerNorm(x1) in one pass
+                        pr = v2(s_n1, rows, C)
+                        lin_fwd(pre + "attn.proj", o, pr)
+                        ln_fwd(pre + "norm2", x, n2, stats2, window=(R, R, ws, shift), windowed=("add",), add=pr, sum_out=x1)
                     else:
                         pr = v2(s_n1, rows, C)
                         lin_fwd(pre + "attn.proj", o, pr)
                         ops.window_partition(ctx, pr, x1, ws, shift, reverse=True, add=x, image_shape=(B, R, R, C))
-                    n2, f1, f2, x2 = act(rows, C), act(rows, 4 * C), act(rows, 4 * C), act(rows, C)
-                    ln_fwd(pre + "norm2", x1, n2, stats2)
+                        ln_fwd(pre + "norm2", x1, n2, stats2)
                     lin_fwd(pre + "mlp.0", n2, f1)
                     ops.gelu_fwd(ctx, f1, f2, tanh_form=False)
                     lin_fwd(pre + "mlp.3", f2, x2, add=x1)

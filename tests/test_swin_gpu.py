@@ -65,6 +65,15 @@ def test_layernorm_in_window_order_equals_layernorm_and_partition(ctx, dtype, B,
     ops.layernorm_fwd(ctx, x, y_fused, gamma, beta, *st_f, window=(H, W, ws, shift))
     torch.cuda.synchronize()
     assert torch.equal(y_fused, y_win) and torch.equal(st[0], st_f[0]) and torch.equal(st[1], st_f[1])
+    # forward with the residual sum: window_reverse(pr) + x, then LayerNorm, against the three separate launches
+    pr_win = torch.randn(rows, C, generator=g).to(dtype).cuda()
+    x1_ref, n2_ref, x1, n2 = new(), new(), new(), new()
+    st2, st2_f = stat(), stat()
+    ops.window_partition(ctx, pr_win, x1_ref, ws, shift, reverse=True, add=x, image_shape=img)
+    ops.layernorm_fwd(ctx, x1_ref, n2_ref, gamma, beta, *st2)
+    ops.layernorm_fwd(ctx, x, n2, gamma, beta, *st2_f, window=(H, W, ws, shift), windowed=("add",), add=pr_win, sum_out=x1)
+    torch.cuda.synchronize()
+    assert torch.equal(x1, x1_ref) and torch.equal(n2, n2_ref) and torch.equal(st2[0], st2_f[0]) and torch.equal(st2[1], st2_f[1])
     # backward: every combination of window-ordered dx, dy and residual against explicit permutations
     dy_rows = torch.randn(rows, C, generator=g).to(dtype).cuda()
     res_rows = torch.randn(rows, C, generator=g).to(dtype).cuda()
@@ -91,7 +100,7 @@ def test_layernorm_in_window_order_equals_layernorm_and_partition(ctx, dtype, B,
 
 @pytest.mark.parametrize("name,dtype", [("window7", torch.bfloat16), ("shifted", torch.float32)])
 def test_window_order_layernorms_change_no_bit(name, dtype):
-    """SwinEngine(fuse_window_ln=True) drops three window-partition launches per block: same loss, gradients and
+    """SwinEngine(fuse_window_ln=True) drops four window-partition launches per block: same loss, gradients and
     weights after three steps as with the separate launches."""
     cfg = S.config(**CFGS[name])
     sd = S.make_state_dict(cfg, seed=4)
@@ -109,7 +118,7 @@ def test_window_order_layernorms_change_no_bit(name, dtype):
             seen.append((eng.last_loss(), {k: v.clone() for k, v in eng.grads_dict().items()}))
             eng.optimizer_step()
         names = [r["name"] for r in eng.ctx.profile(p.prog, 1)]
-        assert any("window_kernel" in n for n in names) == (not fuse) or name == "shifted", names
+        assert any("window_kernel" in n or "window_reverse" in n for n in names) == (not fuse) or name == "shifted", names
         out.append((seen, eng.state_dict()))
     for (la, ga), (lb, gb) in zip(out[0][0], out[1][0]):
         assert la == lb
