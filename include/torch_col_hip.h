@@ -395,6 +395,13 @@ int tch_relpos_bias_gather_pairs(tch_context* ctx, const float* table, const int
                                  int pairs, int entries);
 int tch_relpos_bias_scatter_pairs(tch_context* ctx, const float* dbias, const int32_t* index, float* dtable, int heads,
                                   int pairs, int entries, int accumulate);
+/* tch_relpos_bias_gather_pairs for the `count` bias tables of a whole model at once (one launch per eight tables):
+ * tables / indices / biases / heads are HOST arrays of `count` device pointers / head counts; table k is
+ * [entries][heads[k]], bias k [heads[k]][pairs].  The tables are parameters, so the gathers of every block can run
+ * before the first block of the forward pass (torchvision's shifted_window_attention gathers per block;
+ * train/swin_b_tiny.py:95-99 likewise). */
+int tch_relpos_bias_gather_batch(tch_context* ctx, const float* const* tables, const int32_t* const* indices,
+                                 float* const* biases, const int* heads, int count, int pairs, int entries);
 
 /* The scatter through the inverse of the index, built once by the caller: table entry e receives the pairs
  * list[ptr[e]] .. list[ptr[e + 1] - 1] (pair numbers below `pairs`, ptr non-decreasing, both on the device),

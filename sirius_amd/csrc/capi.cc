@@ -345,6 +345,11 @@ int tch_relpos_bias_gather_pairs(tch_context* ctx, const float* table, const int
   return relpos_bias_gather_pairs(C(ctx), table, index, bias, heads, pairs, entries);
 }
 
+int tch_relpos_bias_gather_batch(tch_context* ctx, const float* const* tables, const int32_t* const* indices,
+                                 float* const* biases, const int* heads, int count, int pairs, int entries) {
+  return relpos_bias_gather_batch(C(ctx), tables, indices, biases, heads, count, pairs, entries);
+}
+
 int tch_relpos_bias_scatter_pairs(tch_context* ctx, const float* dbias, const int32_t* index, float* dtable, int heads,
                                   int pairs, int entries, int accumulate) {
   return relpos_bias_scatter_pairs(C(ctx), dbias, index, dtable, heads, pairs, entries, accumulate);

@@ -158,6 +158,9 @@ int relpos_bias_gather_pairs(Context* ctx, const float* table, const int32_t* in
                              int entries);
 int relpos_bias_scatter_pairs(Context* ctx, const float* dbias, const int32_t* index, float* dtable, int heads, int pairs,
                               int entries, int accumulate);
+// relpos_bias_gather_pairs for `count` tables (host arrays of device pointers) in count / 8 launches
+int relpos_bias_gather_batch(Context* ctx, const float* const* tables, const int32_t* const* indices, float* const* biases,
+                             const int* heads, int count, int pairs, int entries);
 // scatter through the inverse of the index (ptr [entries + 1], list of pair numbers per entry; the caller
 // vouches that every listed pair is below `pairs` and ptr is non-decreasing)
 int relpos_bias_scatter_csr(Context* ctx, const float* dbias, const int32_t* ptr, const int32_t* list, float* dtable,

@@ -142,6 +142,26 @@ __global__ __launch_bounds__(256) void relpos_gather_kernel(RelPosArgs p) {
   p.bias[e] = idx < 0 ? -INFINITY : p.table[idx * p.heads + h];   // a negative index marks padding: masked out
 }
 
+// the same for up to kRelPosBatch bias tables in one launch: blockIdx.y names the table
+constexpr int kRelPosBatch = 8;
+struct RelPosBatchArgs {
+  const float* table[kRelPosBatch];    // [entries][heads[k]]
+  const int32_t* index[kRelPosBatch];  // [nn]
+  float* bias[kRelPosBatch];           // [heads[k]][nn]
+  int heads[kRelPosBatch];
+  int nn;
+};
+
+__global__ __launch_bounds__(256) void relpos_gather_batch_kernel(RelPosBatchArgs p) {
+  const int k = blockIdx.y;
+  const int heads = p.heads[k];
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= heads * p.nn) return;
+  const int h = e / p.nn, ij = e - h * p.nn;
+  const int idx = p.index[k][ij];
+  p.bias[k][e] = idx < 0 ? -INFINITY : p.table[k][idx * heads + h];
+}
+
 // one wavefront per (table entry, head): the (i, j) pairs that point at the entry are summed in index order
 __global__ __launch_bounds__(64) void relpos_scatter_kernel(RelPosArgs p) {
   const int entry = blockIdx.x / p.heads, h = blockIdx.x - entry * p.heads;
@@ -258,6 +278,32 @@ int relpos_bias_gather_pairs(Context* ctx, const float* table, const int32_t* in
   RelPosArgs a{table, index, bias, nullptr, nullptr, heads, pairs, entries, 0};
   return launch(ctx, relpos_gather_kernel, dim3((heads * a.nn + 255) / 256), dim3(256), a, "relpos_gather_kernel",
                 8.0 * heads * a.nn, 1);
+}
+
+int relpos_bias_gather_batch(Context* ctx, const float* const* tables, const int32_t* const* indices, float* const* biases,
+                             const int* heads, int count, int pairs, int entries) {
+  TCH_CHECK_ARG(tables && indices && biases && heads && count > 0 && pairs > 0 && entries > 0,
+                "relpos_bias_gather_batch: bad arguments");
+  for (int k = 0; k < count; ++k)
+    TCH_CHECK_ARG(tables[k] && indices[k] && biases[k] && heads[k] > 0, "relpos_bias_gather_batch: bad table in the batch");
+  for (int first = 0; first < count; first += kRelPosBatch) {
+    const int n = count - first < kRelPosBatch ? count - first : kRelPosBatch;
+    RelPosBatchArgs a{};
+    int most = 0, total = 0;
+    for (int k = 0; k < n; ++k) {
+      a.table[k] = tables[first + k];
+      a.index[k] = indices[first + k];
+      a.bias[k] = biases[first + k];
+      a.heads[k] = heads[first + k];
+      most = a.heads[k] > most ? a.heads[k] : most;
+      total += a.heads[k];
+    }
+    a.nn = pairs;
+    const int rc = launch(ctx, relpos_gather_batch_kernel, dim3((most * pairs + 255) / 256, n), dim3(256), a,
+                          "relpos_gather_batch_kernel", 8.0 * total * pairs, 1);
+    if (rc != 0) return rc;
+  }
+  return 0;
 }
 
 int relpos_bias_scatter_pairs(Context* ctx, const float* dbias, const int32_t* index, float* dtable, int heads, int pairs,

@@ -840,6 +840,23 @@ def relpos_bias_gather_pairs(ctx, table, index, bias):
           "tch_relpos_bias_gather_pairs")
 
 
+def relpos_bias_gather_batch(ctx, tables, indices, biases):
+    """relpos_bias_gather_pairs for lists of tables / indices / bias tensors, eight tables per launch."""
+    count = len(tables)
+    assert count > 0 and len(indices) == len(biases) == count
+    entries, pairs = tables[0].shape[0], indices[0].numel()
+    for t, ix, b in zip(tables, indices, biases):
+        assert t.shape[0] == entries and ix.numel() == pairs and ix.dtype == torch.int32
+        assert t.dtype == b.dtype == torch.float32 and b.numel() == t.shape[1] * pairs
+        assert t.is_contiguous() and ix.is_contiguous() and b.is_contiguous()
+    ptrs = ctypes.c_void_p * count
+    heads = (ctypes.c_int * count)(*[t.shape[1] for t in tables])
+    check(lib().tch_relpos_bias_gather_batch(ctx.handle, ptrs(*[t.data_ptr() for t in tables]),
+                                             ptrs(*[ix.data_ptr() for ix in indices]),
+                                             ptrs(*[b.data_ptr() for b in biases]), heads, count, pairs, entries),
+          "tch_relpos_bias_gather_batch")
+
+
 def relpos_bias_scatter_pairs(ctx, dbias, index, dtable, accumulate=False):
     """dtable[entry, h] (+)= sum of dbias[h, pair] over the pairs with index[pair] == entry."""
     entries, heads = dtable.shape

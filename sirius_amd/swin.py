@@ -70,13 +70,17 @@ def shifted_window_mask(H, W, ws, shift):
 class SwinEngine(EngineBase):
     def __init__(self, embed=128, depths=(2, 2, 18, 2), heads=(4, 8, 16, 32), window=7, patch=4, image_size=224,
                  num_classes=1000, dtype=torch.bfloat16, lr=1e-3, weight_decay=0.05, betas=(0.9, 0.999), eps=1e-8,
-                 stream=None, allocator=None, overlap_wgrad=True, fused_attention=True, fuse_window_ln=True):
+                 stream=None, allocator=None, overlap_wgrad=True, fused_attention=True, fuse_window_ln=True,
+                 batch_bias_gather=True):
         self._init_engine(dtype, stream, allocator)
         # weight / bias / bias-table gradients on a second lane beside the data-gradient chain; the lanes meet
         # at the end of every block, before its gradient buffers are handed round again
         self.overlap_wgrad = overlap_wgrad
         # fuse_window_ln: the LayerNorms next to a window partition read / write window order themselves
         self.fuse_window_ln = fuse_window_ln
+        # batch_bias_gather: the dense bias of every block is gathered from its table at the start of the forward
+        # pass, eight tables per launch, instead of one launch per block in front of its attention
+        self.batch_bias_gather = batch_bias_gather
         self.fused_attention = fused_attention
         assert len(depths) == len(heads) and image_size % patch == 0 and num_classes % 8 == 0 and embed % 8 == 0
         self.embed, self.depths, self.heads = embed, tuple(depths), tuple(heads)
@@ -384,6 +388,15 @@ class SwinEngine(EngineBase):
             ln_fwd("features.0.2", e0, x, embed_stats)
             mark("fwd", "features.0")
             saved_blocks, saved_merges = [], []
+            block_bias = {}
+            if self.batch_bias_gather:
+                fused = [(f"features.{st['f']}.{i}.", st) for st in self.stages if st["fused"] for i in range(st["depth"])]
+                for pre, st in fused:
+                    block_bias[pre] = act(st["heads"] * 64 * 64, dtype=torch.float32)
+                if fused:
+                    ops.relpos_bias_gather_batch(
+                        ctx, [self._view(self.params, pre + "attn.relative_position_bias_table") for pre, _ in fused],
+                        [st["pairs_dev"] for _, st in fused], [block_bias[pre] for pre, _ in fused])
             for si, st in enumerate(self.stages):
                 C, R, ws, Hh = st["C"], st["R"], st["ws"], st["heads"]
                 rows, N, D = B * R * R, ws * ws, C // Hh
@@ -412,9 +425,11 @@ class SwinEngine(EngineBase):
                     o = act(rows, C)
                     if st["fused"]:
                         Pm = act(B_ * Hh, N, 64)
-                        bias = bias_buf[:Hh * 64 * 64]
-                        ops.relpos_bias_gather_pairs(ctx, self._view(self.params, pre + "attn.relative_position_bias_table"),
-                                                     st["pairs_dev"], bias)
+                        bias = block_bias.get(pre)
+                        if bias is None:
+                            bias = bias_buf[:Hh * 64 * 64]
+                            ops.relpos_bias_gather_pairs(ctx, self._view(self.params, pre + "attn.relative_position_bias_table"),
+                                                         st["pairs_dev"], bias)
                         ops.window_attn_fwd(ctx, qkv, o, Pm, bias, st["mask_dev"] if shift else None, B_, Hh, N, scale)
                     else:
                         Pm = act(B_, Hh, N, N)

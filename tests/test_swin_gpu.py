@@ -128,6 +128,65 @@ def test_window_order_layernorms_change_no_bit(name, dtype):
         assert torch.equal(v, out[1][1][k]), k
 
 
+@pytest.mark.parametrize("count", [1, 8, 11])
+def test_batched_bias_gather_equals_one_gather_per_table(ctx, count):
+    """relpos_bias_gather_batch (eight tables per launch, head counts mixed) writes what relpos_bias_gather_pairs
+    writes for each table, and that is the table indexed by hand."""
+    from sirius_amd import ops
+    from sirius_amd.swin import relative_position_index
+    g = _gen(61 + count)
+    N, entries = 49, 169
+    index = relative_position_index(7)
+    pairs = _padded_pairs(index, N).cuda()
+    other = pairs.clone()   # a second index array: the batch takes one per table
+    heads = [(4, 8, 16, 32, 2)[k % 5] for k in range(count)]
+    tables = [torch.randn(entries, h, generator=g).cuda() for h in heads]
+    indices = [pairs if k % 2 == 0 else other for k in range(count)]
+    got = [torch.full((h * 64 * 64,), 7.0, device="cuda") for h in heads]
+    ops.relpos_bias_gather_batch(ctx, tables, indices, got)
+    for t, h, b in zip(tables, heads, got):
+        one = torch.zeros(h * 64 * 64, device="cuda")
+        ops.relpos_bias_gather_pairs(ctx, t, pairs, one)
+        ctx.synchronize()
+        assert torch.equal(b, one)
+        dense = b.view(h, 64, 64).cpu()
+        assert torch.equal(dense[:, :N, :N], t.cpu()[index.reshape(-1)].view(N, N, h).permute(2, 0, 1))
+        assert torch.all(dense[:, :, N:] == float("-inf")) and torch.all(dense[:, N:, :] == float("-inf"))
+    with pytest.raises(Exception):
+        ops.relpos_bias_gather_batch(ctx, tables, indices[:-1] + [pairs[:-1]], got)
+
+
+@pytest.mark.parametrize("name,dtype", [("window7", torch.bfloat16)])
+def test_batched_bias_gather_changes_no_bit(name, dtype):
+    """SwinEngine(batch_bias_gather=True) gathers every block's bias before the first block: same loss, gradients
+    and weights after three steps (the tables change between the steps) as one gather per block."""
+    cfg = S.config(**CFGS[name])
+    sd = S.make_state_dict(cfg, seed=5)
+    g = _gen(14)
+    x = torch.randn(3, 3, cfg["image"], cfg["image"], generator=g).cuda()
+    y = torch.randint(0, cfg["classes"], (3,), generator=g).cuda()
+    out = []
+    for batch in (False, True):
+        eng = _engine(cfg, dtype, batch_bias_gather=batch)
+        eng.load_state_dict(sd)
+        seen = []
+        for _ in range(3):
+            p, cut = eng.forward_backward(x, y)
+            assert not cut
+            seen.append((eng.last_loss(), {k: v.clone() for k, v in eng.grads_dict().items()}))
+            eng.optimizer_step()
+        launches = {r["name"]: r["launches"] for r in eng.ctx.profile(p.prog, 1)}
+        assert launches.get("relpos_gather_batch_kernel", 0) == (1 if batch else 0), launches
+        assert launches.get("relpos_gather_kernel", 0) == (0 if batch else sum(cfg["depths"])), launches
+        out.append((seen, eng.state_dict()))
+    for (la, ga), (lb, gb) in zip(out[0][0], out[1][0]):
+        assert la == lb
+        for k in ga:
+            assert torch.equal(ga[k], gb[k]), k
+    for k, v in out[0][1].items():
+        assert torch.equal(v, out[1][1][k]), k
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("B,H,W,C", [(2, 8, 8, 16), (1, 14, 6, 32), (3, 2, 2, 8)])
 def test_patch_merge_gather_is_a_bit_exact_permutation(ctx, dtype, B, H, W, C):
