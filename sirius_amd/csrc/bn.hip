@@ -238,6 +238,9 @@ struct ApplyArgs {
   int64_t chunks;
   FastDiv div_cc;
   int relu;
+  int64_t rows;        // bn_apply_cols_kernel: rows of the tensor and rows per workgroup slab
+  int rows_per_slab;
+  int nt;
 };
 
 template <typename T, int BWD>
@@ -290,6 +293,89 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(ApplyArgs p) {
       }
     }
     static_cast<uint4*>(p.out)[i] = float_to_chunk<T>(vo).u;
+  }
+}
+
+// The same with the coefficients resident: a thread keeps one 16-byte chunk column (its 4 or 8 channels'
+// coefficients in registers, loaded once) and walks down the rows of its workgroup's slab, four rows per trip,
+// all of them requested before any is used.  bn_apply_kernel fetches 64-96 bytes of coefficients from the cache
+// per 16-byte chunk of data; this one none.  CPR chunk columns per workgroup (CPR * 16 contiguous bytes per row).
+typedef unsigned int stream_u4 __attribute__((ext_vector_type(4)));
+// a 16-byte load that does not ask the caches to keep the line (tensors read once per pass)
+__device__ inline uint4 load_streaming(const void* base, int64_t i) {
+  const stream_u4 v = __builtin_nontemporal_load(static_cast<const stream_u4*>(base) + i);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+template <typename T, int BWD, int CPR>
+__global__ __launch_bounds__(256) void bn_apply_cols_kernel(ApplyArgs p) {
+  constexpr int E = Elem<T>::kPerChunk;
+  constexpr int RPP = 256 / CPR;   // rows per pass of the workgroup
+  constexpr int U = 4;
+  const int tx = threadIdx.x % CPR, ty = threadIdx.x / CPR;
+  const int64_t cc = p.div_cc.d;
+  const int64_t col_chunk = static_cast<int64_t>(blockIdx.x) * CPR + tx;
+  const int ch = static_cast<int>(col_chunk) * E;
+  float k0[E], k1[E], k2[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    k0[e] = p.c0[ch + e];
+    k1[e] = p.c1[ch + e];
+    k2[e] = BWD ? p.c2[ch + e] : 0.f;
+  }
+  const int64_t r0 = static_cast<int64_t>(blockIdx.y) * p.rows_per_slab;
+  int64_t r1 = r0 + p.rows_per_slab;
+  if (r1 > p.rows) r1 = p.rows;
+  for (int64_t r = r0 + ty; r < r1; r += U * RPP) {
+    Chunk ca[U], cb[U], cx[U];
+#pragma unroll
+    for (int q = 0; q < U; ++q) {
+      const int64_t row = r + q * RPP;
+      ca[q] = cb[q] = cx[q] = zero_chunk();
+      if (row < r1) {
+        const int64_t i = row * cc + col_chunk;
+        if (p.nt) {
+          ca[q].u = load_streaming(p.a, i);
+          if (BWD) cx[q].u = load_streaming(p.x, i);
+          if (p.b) cb[q].u = load_streaming(p.b, i);
+        } else {
+          ca[q].u = static_cast<const uint4*>(p.a)[i];
+          if (BWD) cx[q].u = static_cast<const uint4*>(p.x)[i];
+          if (p.b) cb[q].u = static_cast<const uint4*>(p.b)[i];
+        }
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < U; ++q) {
+      const int64_t row = r + q * RPP;
+      if (row >= r1) continue;
+      float va[E], vb[E], vo[E];
+      chunk_to_float<T>(ca[q], va);
+      chunk_to_float<T>(cb[q], vb);
+      if (BWD) {
+        float vx[E];
+        chunk_to_float<T>(cx[q], vx);
+        if (p.b) {
+#pragma unroll
+          for (int e = 0; e < E; ++e)
+            if (!(vb[e] > 0.f)) va[e] = 0.f;
+        }
+#pragma unroll
+        for (int e = 0; e < E; ++e) vo[e] = k0[e] * va[e] + k1[e] * vx[e] + k2[e];
+      } else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) vo[e] = va[e] * k0[e] + k1[e];
+        if (p.b) {
+#pragma unroll
+          for (int e = 0; e < E; ++e) vo[e] += vb[e];
+        }
+        if (p.relu) {
+#pragma unroll
+          for (int e = 0; e < E; ++e) vo[e] = vo[e] > 0.f ? vo[e] : 0.f;
+        }
+      }
+      static_cast<uint4*>(p.out)[row * cc + col_chunk] = float_to_chunk<T>(vo).u;
+    }
   }
 }
 
@@ -518,6 +604,54 @@ unsigned apply_blocks(int64_t chunks) {
   return static_cast<unsigned>(b);
 }
 
+template <typename T, int BWD, int CPR>
+int launch_apply_cols(Context* ctx, ApplyArgs& a, const char* name, double bytes) {
+  static const int target = [] {
+    const char* e = getenv("TCH_BN_APPLY_WGS");
+    return e && atoi(e) > 0 ? atoi(e) : 8192;
+  }();
+  constexpr int trip = 4 * (256 / CPR);   // rows a workgroup takes per trip
+  const int64_t col_blocks = a.div_cc.d / CPR;
+  int64_t slabs = target / col_blocks;
+  if (slabs < 1) slabs = 1;
+  int64_t rps = (a.rows + slabs - 1) / slabs;
+  rps = (rps + trip - 1) / trip * trip;
+  a.rows_per_slab = static_cast<int>(rps);
+  static const int nt = [] {
+    const char* e = getenv("TCH_BN_APPLY_NT");
+    return e ? atoi(e) : 1;
+  }();
+  a.nt = nt;
+  const dim3 grid(static_cast<unsigned>(col_blocks), static_cast<unsigned>((a.rows + rps - 1) / rps));
+  return launch(ctx, bn_apply_cols_kernel<T, BWD, CPR>, grid, dim3(256), a, name, bytes, 1);
+}
+
+// normalise / input gradient from per-channel coefficients: the column-resident kernel where the chunk columns
+// split into groups of 8, 16 or 32 (TCH_BN_APPLY_COLS=0: always the flat kernel)
+template <typename T, int BWD>
+int launch_apply_t(Context* ctx, ApplyArgs& a, const char* name, double bytes) {
+  static const bool cols = [] {
+    const char* e = getenv("TCH_BN_APPLY_COLS");
+    return !(e && atoi(e) == 0);
+  }();
+  const int64_t cc = a.div_cc.d;
+  a.rows = a.chunks / cc;
+  if (cols && cc % 8 == 0 && a.rows >= 1024) {
+    if (cc % 32 == 0) return launch_apply_cols<T, BWD, 32>(ctx, a, name, bytes);
+    if (cc % 16 == 0) return launch_apply_cols<T, BWD, 16>(ctx, a, name, bytes);
+    return launch_apply_cols<T, BWD, 8>(ctx, a, name, bytes);
+  }
+  return launch(ctx, bn_apply_kernel<T, BWD>, dim3(apply_blocks(a.chunks)), dim3(256), a, name, bytes, 1);
+}
+
+int launch_apply(Context* ctx, int dtype, bool bwd, ApplyArgs& a, double bytes) {
+  if (dtype == kBF16)
+    return bwd ? launch_apply_t<bf16, 1>(ctx, a, "bn_apply_kernel<bf16,bwd>", bytes)
+               : launch_apply_t<bf16, 0>(ctx, a, "bn_apply_kernel<bf16,fwd>", bytes);
+  return bwd ? launch_apply_t<float, 1>(ctx, a, "bn_apply_kernel<f32,bwd>", bytes)
+             : launch_apply_t<float, 0>(ctx, a, "bn_apply_kernel<f32,fwd>", bytes);
+}
+
 // Inference-mode BatchNorm as one scale and one shift per channel, from the running statistics:
 // y = (x - running_mean) / sqrt(running_var + eps) * gamma + beta = x * scale + shift.
 struct EvalCoefArgs {
@@ -578,10 +712,7 @@ int bn_fwd_train(Context* ctx, int dtype, const void* x, void* y, const void* re
   if (rc) return rc;
   ApplyArgs a{x, residual, nullptr, y, scale, shift, nullptr, rows * g.cc, FastDiv(g.cc), relu};
   const double apply_bytes = tensor_bytes * (residual ? 3.0 : 2.0);
-  return dtype == kBF16 ? launch(ctx, bn_apply_kernel<bf16, 0>, dim3(apply_blocks(a.chunks)), dim3(256), a,
-                                 "bn_apply_kernel<bf16,fwd>", apply_bytes, 1)
-                        : launch(ctx, bn_apply_kernel<float, 0>, dim3(apply_blocks(a.chunks)), dim3(256), a,
-                                 "bn_apply_kernel<f32,fwd>", apply_bytes, 1);
+  return launch_apply(ctx, dtype, false, a, apply_bytes);
 }
 
 int bn_fwd_finalize(Context* ctx, const float* partial, int row_blocks, int C, int64_t rows, const float* gamma,
@@ -615,10 +746,7 @@ int bn_apply_fwd(Context* ctx, int dtype, const void* x, void* y, const void* re
   const double tensor_bytes = static_cast<double>(rows) * C * (dtype == kBF16 ? 2.0 : 4.0);
   ApplyArgs a{x, residual, nullptr, y, coef, coef + C, nullptr, rows * g.cc, FastDiv(g.cc), relu};
   const double apply_bytes = tensor_bytes * (residual ? 3.0 : 2.0);
-  return dtype == kBF16 ? launch(ctx, bn_apply_kernel<bf16, 0>, dim3(apply_blocks(a.chunks)), dim3(256), a,
-                                 "bn_apply_kernel<bf16,fwd>", apply_bytes, 1)
-                        : launch(ctx, bn_apply_kernel<float, 0>, dim3(apply_blocks(a.chunks)), dim3(256), a,
-                                 "bn_apply_kernel<f32,fwd>", apply_bytes, 1);
+  return launch_apply(ctx, dtype, false, a, apply_bytes);
 }
 
 int bn_eval_coef(Context* ctx, const float* gamma, const float* beta, const float* running_mean,
@@ -635,10 +763,7 @@ int bn_apply_bwd(Context* ctx, int dtype, const void* g, const void* x, void* dx
   Geometry geo = geometry(rows, C, dtype);
   const double tensor_bytes = static_cast<double>(rows) * C * (dtype == kBF16 ? 2.0 : 4.0);
   ApplyArgs a{g, nullptr, x, dx, coef, coef + C, coef + 2 * C, rows * geo.cc, FastDiv(geo.cc), 0};
-  return dtype == kBF16 ? launch(ctx, bn_apply_kernel<bf16, 1>, dim3(apply_blocks(a.chunks)), dim3(256), a,
-                                 "bn_apply_kernel<bf16,bwd>", tensor_bytes * 3.0, 1)
-                        : launch(ctx, bn_apply_kernel<float, 1>, dim3(apply_blocks(a.chunks)), dim3(256), a,
-                                 "bn_apply_kernel<f32,bwd>", tensor_bytes * 3.0, 1);
+  return launch_apply(ctx, dtype, true, a, tensor_bytes * 3.0);
 }
 
 int bn_fwd_train_partials(Context* ctx, int dtype, const void* x, void* y, const void* residual, int relu,
@@ -672,10 +797,7 @@ int bn_fwd_train_partials(Context* ctx, int dtype, const void* x, void* y, const
   const double tensor_bytes = static_cast<double>(rows) * C * eb;
   ApplyArgs a{x, residual, nullptr, y, scale, shift, nullptr, rows * g.cc, FastDiv(g.cc), relu};
   const double apply_bytes = tensor_bytes * (residual ? 3.0 : 2.0);
-  return dtype == kBF16 ? launch(ctx, bn_apply_kernel<bf16, 0>, dim3(apply_blocks(a.chunks)), dim3(256), a,
-                                 "bn_apply_kernel<bf16,fwd>", apply_bytes, 1)
-                        : launch(ctx, bn_apply_kernel<float, 0>, dim3(apply_blocks(a.chunks)), dim3(256), a,
-                                 "bn_apply_kernel<f32,fwd>", apply_bytes, 1);
+  return launch_apply(ctx, dtype, false, a, apply_bytes);
 }
 
 int bn_bwd(Context* ctx, int dtype, const void* dy, const void* relu_mask, const void* x, void* dx, int64_t rows,
@@ -702,10 +824,7 @@ int bn_bwd(Context* ctx, int dtype, const void* dy, const void* relu_mask, const
               8.0 * g.row_blocks * C, 1);
   if (rc) return rc;
   ApplyArgs a{dy, relu_mask, x, dx, coef, coef + C, coef + 2 * C, rows * g.cc, FastDiv(g.cc), 0};
-  return dtype == kBF16 ? launch(ctx, bn_apply_kernel<bf16, 1>, dim3(apply_blocks(a.chunks)), dim3(256), a,
-                                 "bn_apply_kernel<bf16,bwd>", tensor_bytes * (in_tensors + 1.0), 1)
-                        : launch(ctx, bn_apply_kernel<float, 1>, dim3(apply_blocks(a.chunks)), dim3(256), a,
-                                 "bn_apply_kernel<f32,bwd>", tensor_bytes * (in_tensors + 1.0), 1);
+  return launch_apply(ctx, dtype, true, a, tensor_bytes * (in_tensors + 1.0));
 }
 
 int bn_bwd_partials(Context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int C,
@@ -733,10 +852,7 @@ int bn_bwd_partials(Context* ctx, int dtype, const void* g, const void* x, void*
   const double eb = dtype == kBF16 ? 2.0 : 4.0;
   const double tensor_bytes = static_cast<double>(rows) * C * eb;
   ApplyArgs a{g, nullptr, x, dx, coef, coef + C, coef + 2 * C, rows * geo.cc, FastDiv(geo.cc), 0};
-  return dtype == kBF16 ? launch(ctx, bn_apply_kernel<bf16, 1>, dim3(apply_blocks(a.chunks)), dim3(256), a,
-                                 "bn_apply_kernel<bf16,bwd>", tensor_bytes * 3.0, 1)
-                        : launch(ctx, bn_apply_kernel<float, 1>, dim3(apply_blocks(a.chunks)), dim3(256), a,
-                                 "bn_apply_kernel<f32,bwd>", tensor_bytes * 3.0, 1);
+  return launch_apply(ctx, dtype, true, a, tensor_bytes * 3.0);
 }
 
 }  // namespace tch

@@ -145,6 +145,22 @@ struct FastDiv {
   }
 };
 
+// 16-byte fp32 accesses that do not ask the caches to keep the line: optimizer state and master weights are touched
+// once per step and are larger than every cache
+typedef float stream_f4 __attribute__((ext_vector_type(4)));
+__device__ inline float4 load_streaming_f4(const float* p) {
+  const stream_f4 v = __builtin_nontemporal_load(reinterpret_cast<const stream_f4*>(p));
+  return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ inline void store_streaming_f4(float* p, const float4& v) {
+  stream_f4 s;
+  s.x = v.x;
+  s.y = v.y;
+  s.z = v.z;
+  s.w = v.w;
+  __builtin_nontemporal_store(s, reinterpret_cast<stream_f4*>(p));
+}
+
 // ---------------------------------------------------------------------------
 // wavefront reductions (64 lanes)
 // ---------------------------------------------------------------------------

@@ -205,15 +205,16 @@ struct SgdArgs {
   uint16_t* shadow;
   int64_t n;
   float lr, momentum, wd;
+  int aligned;   // every buffer starts on a 16-byte boundary (the shadow on 8): 16-byte accesses are in order
 };
 
 __global__ __launch_bounds__(256) void sgd_kernel(SgdArgs p) {
   const int64_t stride = static_cast<int64_t>(gridDim.x) * 256 * 4;
   for (int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4; i < p.n; i += stride) {
-    if (i + 4 <= p.n) {
-      float4 w = *reinterpret_cast<float4*>(p.param + i);
-      float4 g = *reinterpret_cast<const float4*>(p.grad + i);
-      float4 b = *reinterpret_cast<float4*>(p.buf + i);
+    if (p.aligned && i + 4 <= p.n) {
+      float4 w = load_streaming_f4(p.param + i);
+      float4 g = load_streaming_f4(p.grad + i);
+      float4 b = load_streaming_f4(p.buf + i);
       b.x = p.momentum * b.x + (g.x + p.wd * w.x);
       b.y = p.momentum * b.y + (g.y + p.wd * w.y);
       b.z = p.momentum * b.z + (g.z + p.wd * w.z);
@@ -222,8 +223,8 @@ __global__ __launch_bounds__(256) void sgd_kernel(SgdArgs p) {
       w.y -= p.lr * b.y;
       w.z -= p.lr * b.z;
       w.w -= p.lr * b.w;
-      *reinterpret_cast<float4*>(p.param + i) = w;
-      *reinterpret_cast<float4*>(p.buf + i) = b;
+      store_streaming_f4(p.param + i, w);
+      store_streaming_f4(p.buf + i, b);
       if (p.shadow) {
         uint2 s;
         s.x = float_to_bf16_bits(w.x) | (static_cast<uint32_t>(float_to_bf16_bits(w.y)) << 16);
@@ -231,7 +232,7 @@ __global__ __launch_bounds__(256) void sgd_kernel(SgdArgs p) {
         *reinterpret_cast<uint2*>(p.shadow + i) = s;
       }
     } else {
-      for (int64_t j = i; j < p.n; ++j) {
+      for (int64_t j = i; j < p.n && j < i + 4; ++j) {
         float w = p.param[j];
         float b = p.momentum * p.buf[j] + (p.grad[j] + p.wd * w);
         w -= p.lr * b;
@@ -356,7 +357,7 @@ __global__ __launch_bounds__(256) void slab_sum_kernel(SlabSumArgs p) {
 
 unsigned flat_blocks(int64_t n_vec) {
   int64_t b = (n_vec + 255) / 256;
-  if (b > 4096) b = 4096;
+  if (b > (1 << 20)) b = 1 << 20;
   if (b < 1) b = 1;
   return static_cast<unsigned>(b);
 }
@@ -411,7 +412,9 @@ int softmax_ce_lm(Context* ctx, int dtype, const float* logits, int ld_logits, c
 int sgd_momentum_step(Context* ctx, float* param, const float* grad, float* momentum_buf, void* shadow_bf16,
                       int64_t n, float lr, float momentum, float weight_decay) {
   TCH_CHECK_ARG(param && grad && momentum_buf && n > 0, "sgd_momentum_step: null tensor or empty");
-  SgdArgs a{param, grad, momentum_buf, static_cast<uint16_t*>(shadow_bf16), n, lr, momentum, weight_decay};
+  SgdArgs a{param, grad, momentum_buf, static_cast<uint16_t*>(shadow_bf16), n, lr, momentum, weight_decay, 0};
+  a.aligned = ((reinterpret_cast<uintptr_t>(param) | reinterpret_cast<uintptr_t>(grad) | reinterpret_cast<uintptr_t>(momentum_buf)) & 15) == 0 &&
+              (reinterpret_cast<uintptr_t>(shadow_bf16) & 7) == 0;
   return launch(ctx, sgd_kernel, dim3(flat_blocks((n + 3) / 4)), dim3(256), a, "sgd_kernel",
                 static_cast<double>(n) * (shadow_bf16 ? 22.0 : 20.0), 1);
 }

@@ -15,7 +15,7 @@
 namespace tch {
 namespace {
 
-unsigned flat_blocks(int64_t items, int64_t cap = 8192) {
+unsigned flat_blocks(int64_t items, int64_t cap = 1 << 20) {
   int64_t b = (items + 255) / 256;
   if (b > cap) b = cap;
   if (b < 1) b = 1;
@@ -460,25 +460,52 @@ struct AdamArgs {
   // every constant is rounded to fp32 once, from the double the caller gave (1 - beta as well:
   // 1 - 0.999f is off by 1e-5 relative)
   float lr, beta2, one_minus_beta1, one_minus_beta2, eps, decay;
+  int aligned;   // every buffer starts on a 16-byte boundary (the shadow on 8): 16-byte accesses are in order
 };
 
+__device__ inline void adamw_element(const AdamArgs& p, float step_size, float bc2_sqrt, float g, float& w, float& m,
+                                     float& v) {
+  w *= p.decay;
+  m = m + (g - m) * p.one_minus_beta1;
+  v = v * p.beta2 + p.one_minus_beta2 * g * g;
+  const float denom = sqrtf(v) / bc2_sqrt + p.eps;
+  w -= step_size * (m / denom);
+}
+
+// four elements per thread and trip, 16-byte streaming accesses; the last n % 4 elements one by one
 __global__ __launch_bounds__(256) void adamw_kernel(AdamArgs p) {
   const float bc1 = p.scalars[0], bc2_sqrt = p.scalars[1];
   const float step_size = p.lr / bc1;
-  const float decay = p.decay;
-  const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
-  for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < p.n; i += stride) {
-    const float g = p.grad[i];
-    float w = p.param[i] * decay;
-    float m = p.m[i];
-    m = m + (g - m) * p.one_minus_beta1;
-    const float v = p.v[i] * p.beta2 + p.one_minus_beta2 * g * g;
-    const float denom = sqrtf(v) / bc2_sqrt + p.eps;
-    w -= step_size * (m / denom);
-    p.param[i] = w;
-    p.m[i] = m;
-    p.v[i] = v;
-    if (p.shadow) p.shadow[i] = float_to_bf16_bits(w);
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * 256 * 4;
+  for (int64_t i = (static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x) * 4; i < p.n; i += stride) {
+    if (p.aligned && i + 4 <= p.n) {
+      const float4 g = load_streaming_f4(p.grad + i);
+      float4 w = load_streaming_f4(p.param + i);
+      float4 m = load_streaming_f4(p.m + i);
+      float4 v = load_streaming_f4(p.v + i);
+      adamw_element(p, step_size, bc2_sqrt, g.x, w.x, m.x, v.x);
+      adamw_element(p, step_size, bc2_sqrt, g.y, w.y, m.y, v.y);
+      adamw_element(p, step_size, bc2_sqrt, g.z, w.z, m.z, v.z);
+      adamw_element(p, step_size, bc2_sqrt, g.w, w.w, m.w, v.w);
+      store_streaming_f4(p.param + i, w);
+      store_streaming_f4(p.m + i, m);
+      store_streaming_f4(p.v + i, v);
+      if (p.shadow) {
+        uint2 sh;
+        sh.x = float_to_bf16_bits(w.x) | (static_cast<uint32_t>(float_to_bf16_bits(w.y)) << 16);
+        sh.y = float_to_bf16_bits(w.z) | (static_cast<uint32_t>(float_to_bf16_bits(w.w)) << 16);
+        *reinterpret_cast<uint2*>(p.shadow + i) = sh;
+      }
+    } else {
+      for (int64_t j = i; j < p.n && j < i + 4; ++j) {
+        float w = p.param[j], m = p.m[j], v = p.v[j];
+        adamw_element(p, step_size, bc2_sqrt, p.grad[j], w, m, v);
+        p.param[j] = w;
+        p.m[j] = m;
+        p.v[j] = v;
+        if (p.shadow) p.shadow[j] = float_to_bf16_bits(w);
+      }
+    }
   }
 }
 
@@ -809,8 +836,12 @@ int adamw_step(Context* ctx, float* param, const float* grad, float* exp_avg, fl
              static_cast<float>(1.0 - beta1),
              static_cast<float>(1.0 - beta2),
              static_cast<float>(eps),
-             static_cast<float>(1.0 - lr * weight_decay)};
-  return launch(ctx, adamw_kernel, dim3(flat_blocks(n)), dim3(256), a, "adamw_kernel",
+             static_cast<float>(1.0 - lr * weight_decay),
+             0};
+  a.aligned = ((reinterpret_cast<uintptr_t>(param) | reinterpret_cast<uintptr_t>(grad) | reinterpret_cast<uintptr_t>(exp_avg) |
+                reinterpret_cast<uintptr_t>(exp_avg_sq)) & 15) == 0 &&
+              (reinterpret_cast<uintptr_t>(shadow_bf16) & 7) == 0;
+  return launch(ctx, adamw_kernel, dim3(flat_blocks((n + 3) / 4)), dim3(256), a, "adamw_kernel",
                 static_cast<double>(n) * (shadow_bf16 ? 30.0 : 28.0), 1);
 }
 

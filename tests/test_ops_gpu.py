@@ -656,13 +656,19 @@ def test_softmax_ce(ctx, dtype, rows, classes, scale):
 
 
 @pytest.mark.parametrize("n", [1024, 1000003])
-def test_sgd_and_accumulate(ctx, n):
+@pytest.mark.parametrize("offset", [0, 1])   # 1: the buffers start 4 bytes past a 16-byte boundary (scalar accesses)
+def test_sgd_and_accumulate(ctx, n, offset):
     from sirius_amd import ops
     g = _gen(11)
     p, gr, buf = torch.randn(n, generator=g), torch.randn(n, generator=g), torch.zeros(n)
     p_ref, buf_ref = O.sgd_momentum(p, gr, buf, 0.1, 0.9, 1e-4, steps=2)
-    p_d, g_d, b_d = p.cuda(), gr.cuda(), buf.cuda()
-    shadow = torch.empty(n, dtype=torch.bfloat16, device="cuda")
+
+    def dev(t):
+        d = torch.zeros(n + offset, device="cuda")[offset:]
+        d.copy_(t)
+        return d
+    p_d, g_d, b_d = dev(p), dev(gr), dev(buf)
+    shadow = torch.empty(n + offset, dtype=torch.bfloat16, device="cuda")[offset:]
     for _ in range(2):
         ops.sgd_momentum_step(ctx, p_d, g_d, b_d, 0.1, 0.9, 1e-4, shadow=shadow)
     torch.cuda.synchronize()
@@ -670,10 +676,10 @@ def test_sgd_and_accumulate(ctx, n):
     close(b_d, buf_ref, torch.float32, "sgd momentum", rtol=1e-6)
     assert torch.equal(shadow.cpu(), p_d.cpu().to(torch.bfloat16)), "bf16 shadow must be the RNE rounding of the master"
     acc = torch.randn(n, generator=g)
-    acc_d = acc.cuda()
-    ops.grad_accumulate(ctx, acc_d, g_d)
+    acc_d, g_al = acc.cuda(), gr.cuda()
+    ops.grad_accumulate(ctx, acc_d, g_al)
     torch.cuda.synchronize()
-    assert torch.equal(acc_d.cpu(), acc + gr) and (g_d == 0).all()
+    assert torch.equal(acc_d.cpu(), acc + gr) and (g_al == 0).all()
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

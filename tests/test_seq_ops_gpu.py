@@ -150,16 +150,19 @@ def test_attn_softmax(ctx, dtype, case):
 
 @pytest.mark.parametrize("n", [5, 1000, (1 << 20) + 3])
 @pytest.mark.parametrize("with_shadow", [False, True])
-def test_adamw(ctx, n, with_shadow):
+@pytest.mark.parametrize("offset", [0, 1])   # 1: the buffers start 4 bytes past a 16-byte boundary (scalar accesses)
+def test_adamw(ctx, n, with_shadow, offset):
     from sirius_amd import ops
     g = _gen(34)
     p0 = torch.randn(n, generator=g)
     grads = [torch.randn(n, generator=g) * (0.1 + i) for i in range(3)]
     hp = dict(lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, weight_decay=0.05)
     p_ref, m_ref, v_ref = S.adamw(p0, grads, hp["lr"], hp["beta1"], hp["beta2"], hp["eps"], hp["weight_decay"])
-    p, m, v = p0.cuda(), torch.zeros(n, device="cuda"), torch.zeros(n, device="cuda")
+    p = torch.zeros(n + offset, device="cuda")[offset:]
+    p.copy_(p0)
+    m, v = torch.zeros(n + offset, device="cuda")[offset:], torch.zeros(n + offset, device="cuda")[offset:]
     step, scal = torch.zeros(1, dtype=torch.int32, device="cuda"), torch.zeros(2, device="cuda")
-    shadow = torch.empty(n, dtype=torch.bfloat16, device="cuda") if with_shadow else None
+    shadow = torch.empty(n + offset, dtype=torch.bfloat16, device="cuda")[offset:] if with_shadow else None
     for gi in grads:
         ops.adamw_step(ctx, p, gi.cuda(), m, v, step, scal, shadow=shadow, **hp)
         torch.cuda.synchronize()
