@@ -300,13 +300,6 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(ApplyArgs p) {
 // coefficients in registers, loaded once) and walks down the rows of its workgroup's slab, four rows per trip,
 // all of them requested before any is used.  bn_apply_kernel fetches 64-96 bytes of coefficients from the cache
 // per 16-byte chunk of data; this one none.  CPR chunk columns per workgroup (CPR * 16 contiguous bytes per row).
-typedef unsigned int stream_u4 __attribute__((ext_vector_type(4)));
-// a 16-byte load that does not ask the caches to keep the line (tensors read once per pass)
-__device__ inline uint4 load_streaming(const void* base, int64_t i) {
-  const stream_u4 v = __builtin_nontemporal_load(static_cast<const stream_u4*>(base) + i);
-  return make_uint4(v.x, v.y, v.z, v.w);
-}
-
 template <typename T, int BWD, int CPR>
 __global__ __launch_bounds__(256) void bn_apply_cols_kernel(ApplyArgs p) {
   constexpr int E = Elem<T>::kPerChunk;
@@ -335,9 +328,9 @@ __global__ __launch_bounds__(256) void bn_apply_cols_kernel(ApplyArgs p) {
       if (row < r1) {
         const int64_t i = row * cc + col_chunk;
         if (p.nt) {
-          ca[q].u = load_streaming(p.a, i);
-          if (BWD) cx[q].u = load_streaming(p.x, i);
-          if (p.b) cb[q].u = load_streaming(p.b, i);
+          ca[q].u = load_streaming_u4(p.a, i);
+          if (BWD) cx[q].u = load_streaming_u4(p.x, i);
+          if (p.b) cb[q].u = load_streaming_u4(p.b, i);
         } else {
           ca[q].u = static_cast<const uint4*>(p.a)[i];
           if (BWD) cx[q].u = static_cast<const uint4*>(p.x)[i];

@@ -145,6 +145,13 @@ struct FastDiv {
   }
 };
 
+typedef unsigned int stream_u4 __attribute__((ext_vector_type(4)));
+// 16 bytes of a tensor that is read once per pass: the caches are not asked to keep the line
+__device__ inline uint4 load_streaming_u4(const void* base, int64_t i) {
+  const stream_u4 v = __builtin_nontemporal_load(static_cast<const stream_u4*>(base) + i);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 // 16-byte fp32 accesses that do not ask the caches to keep the line: optimizer state and master weights are touched
 // once per step and are larger than every cache
 typedef float stream_f4 __attribute__((ext_vector_type(4)));

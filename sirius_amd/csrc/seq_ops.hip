@@ -356,12 +356,12 @@ __global__ __launch_bounds__(256) void gelu_kernel(GeluArgs p) {
   const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
   for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < p.chunks; i += stride) {
     Chunk cx;
-    cx.u = static_cast<const uint4*>(p.x)[i];
+    cx.u = load_streaming_u4(p.x, i);
     float x[E], o[E];
     chunk_to_float<T>(cx, x);
     if (BWD) {
       Chunk cg;
-      cg.u = static_cast<const uint4*>(p.dy)[i];
+      cg.u = load_streaming_u4(p.dy, i);
       float g[E];
       chunk_to_float<T>(cg, g);
 #pragma unroll
