@@ -191,11 +191,21 @@ struct MeanArgs {
   float divisor;
 };
 
-__global__ __launch_bounds__(64) void mean_kernel(MeanArgs p) {
+// one workgroup of 1024 threads: thread t adds rows t, t + 1024, ...; the wavefronts' sums meet in LDS in wavefront
+// order (a fixed order: the mean does not change from run to run)
+__global__ __launch_bounds__(1024) void mean_kernel(MeanArgs p) {
+  __shared__ float part[16];
   float s = 0.f;
-  for (int i = threadIdx.x; i < p.n; i += 64) s += p.in[i];
+  for (int i = threadIdx.x; i < p.n; i += 1024) s += p.in[i];
   s = wave_sum(s);
-  if (threadIdx.x == 0) *p.out = s / p.divisor;
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float t = 0.f;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) t += part[w];
+    *p.out = t / p.divisor;
+  }
 }
 
 struct SgdArgs {
@@ -375,7 +385,7 @@ int softmax_ce_fwd_bwd(Context* ctx, int dtype, const float* logits, const int64
                           : launch(ctx, softmax_ce_kernel<float>, dim3(rows), dim3(64), a, "softmax_ce_kernel<f32>", bytes, 1);
   if (rc) return rc;
   MeanArgs m{loss_rows, loss_mean, rows, static_cast<float>(rows)};
-  return launch(ctx, mean_kernel, dim3(1), dim3(64), m, "mean_kernel", 4.0 * rows, 1);
+  return launch(ctx, mean_kernel, dim3(1), dim3(1024), m, "mean_kernel", 4.0 * rows, 1);
 }
 
 int softmax_ce_lm(Context* ctx, int dtype, const float* logits, int ld_logits, const int64_t* labels, float* loss_rows,
@@ -406,7 +416,7 @@ int softmax_ce_lm(Context* ctx, int dtype, const float* logits, int ld_logits, c
   }
   if (rc) return rc;
   MeanArgs m{loss_rows, loss_mean, rows, static_cast<float>(valid_rows)};
-  return launch(ctx, mean_kernel, dim3(1), dim3(64), m, "mean_kernel", 4.0 * rows, 1);
+  return launch(ctx, mean_kernel, dim3(1), dim3(1024), m, "mean_kernel", 4.0 * rows, 1);
 }
 
 int sgd_momentum_step(Context* ctx, float* param, const float* grad, float* momentum_buf, void* shadow_bf16,
