@@ -334,7 +334,7 @@ def test_conv_wgrad_group(ctx, dtype, target_wgs, tile_cfg, max_wgs):
             close(db, 2 * db_ref, torch.float32, f"grouped bias gradient accumulate {case}", rtol=1e-4)
 
 
-BN_CASES = [(2 * 14 * 14, 64), (4 * 28 * 28, 128), (3 * 7 * 7, 2048), (37, 8), (100000, 64)]
+BN_CASES = [(2 * 14 * 14, 64), (4 * 28 * 28, 128), (3 * 7 * 7, 2048), (37, 8), (100000, 64), (1024 + 37, 256)]
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
