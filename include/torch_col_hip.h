@@ -84,6 +84,18 @@ typedef struct tch_kernel_stat {
  * with a HIP event between any two launches; one row per kernel name. */
 int tch_program_profile(tch_context* ctx, const tch_program* prog, int reps, tch_kernel_stat* out, int max_out,
                         int* n_out);
+typedef struct tch_launch_stat {
+  char name[96];      /* kernel name; empty for a program entry that launches nothing (a join of the lanes) */
+  double ms;          /* mean HIP-event time of this launch over the repetitions */
+  double flops;       /* ALGORITHMIC flops of the launch (0 where it is annotated with bytes only) */
+  double bytes;       /* ALGORITHMIC bytes of the launch */
+  int lane;           /* 0 = main lane, 1 = the lane that may run beside it */
+  int64_t workgroups;
+} tch_launch_stat;
+/* The same replay, one row per program position (out[i] is launch i): what each launch of a step costs alone
+ * on the chip, next to the work it states -- the input of a per-layer roofline table. */
+int tch_program_profile_launches(tch_context* ctx, const tch_program* prog, int reps, tch_launch_stat* out,
+                                 int64_t max_out, int64_t* n_out);
 
 /* ---- preemptible launch queues (replaces common/xsched_ctrl.h:12-40) ------------ */
 uint64_t tch_RegisterStream(uint64_t hip_stream);   /* xsched_ctrl.cc:27-46; 0 on failure */
@@ -173,6 +185,19 @@ int tch_conv2d_dgrad_bnsums(tch_context* ctx, int dtype, const void* dy, const v
                             const float* bn_invstd, float* bn_partial, int add_stride);
 int tch_conv2d_dgrad_stat_rows(int dtype, int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
                                int tile_cfg);
+/* The same two with the sums ADDED to one pair of exact accumulators per channel instead of left per row tile:
+ * bn_acc[c * 4 + {0,1}] collects the first sum, [c * 4 + {2,3}] the second, each as a pair of 64-bit integers
+ * (units of 2^-24 and of 2^-66: integer additions, so the totals do not depend on the order the workgroups finish
+ * in and a step stays bit-identical from run to run).  bn_acc must be zero before the call (tch_fill_zero); feed it
+ * to tch_bn_fwd_train_acc / tch_bn_bwd_acc, which need no finalize launch and no pass over per-tile partials.
+ * What torch's conv2d -> batch_norm pairs (train/resnet152.py:22) need of each other, as two launches. */
+int tch_conv2d_fwd_bnacc(tch_context* ctx, int dtype, const void* x, const void* w, void* y, int N, int H, int W,
+                         int C, int K, int R, int S, int stride, int pad, int tile_cfg, int c_logical,
+                         int64_t* bn_acc);
+int tch_conv2d_dgrad_bnacc(tch_context* ctx, int dtype, const void* dy, const void* wt, void* dx, const void* add,
+                           const void* mask, int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
+                           int tile_cfg, int c_logical, const void* bn_mask, const void* bn_x, const float* bn_mean,
+                           const float* bn_invstd, int64_t* bn_acc, int add_stride);
 /* Convolution + the whole front half of the BatchNorm next to it, in one call: the sums as above, and the
  * per-channel coefficients from them (by the workgroup that finishes a column tile last, or by a finalize launch
  * when there are more than 256 row tiles).  counters: >= ceil(channels / 64) ints, zero before the call, zero
@@ -262,6 +287,17 @@ int tch_bn_bwd(tch_context* ctx, int dtype, const void* dy, const void* relu_mas
 int tch_bn_bwd_partials(tch_context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int C,
                         const float* gamma, const float* save_mean, const float* save_invstd, float* dgamma,
                         float* dbeta, int accumulate, const float* partial, int row_blocks, float* scratch);
+
+/* tch_bn_fwd_train_partials / tch_bn_bwd_partials from the accumulators of tch_conv2d_fwd_bnacc /
+ * tch_conv2d_dgrad_bnacc (acc[C * 4] 64-bit words): coefficients and apply in ONE launch whatever the number of
+ * rows.  C must be a multiple of eight 16-byte chunks (64 for bf16, 32 for fp32). */
+int tch_bn_fwd_train_acc(tch_context* ctx, int dtype, const void* x, void* y, const void* residual, int relu,
+                         int64_t rows, int C, const float* gamma, const float* beta, float* running_mean,
+                         float* running_var, float* save_mean, float* save_invstd, float momentum, float eps,
+                         const int64_t* acc);
+int tch_bn_bwd_acc(tch_context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int C,
+                   const float* gamma, const float* save_mean, const float* save_invstd, float* dgamma, float* dbeta,
+                   int accumulate, const int64_t* acc);
 
 /* ---- pooling -------------------------------------------------------------------- */
 /* index[N,Ho,Wo,C] (int32) = h*W + w of the FIRST maximum in row-major window order (NaN wins). */

@@ -90,6 +90,11 @@ void tch_pool_counters(int device, uint64_t* out6);
  * how many it removed. */
 uint64_t tch_pool_trim(int device, uint64_t max_pages);
 uint64_t tch_pool_unmap_calls(int device); /* driver calls behind the unmaps (a run of neighbouring slots is one) */
+/* The page table as training sees it: owner_out[i] = 0 free / 1 training / 2 inference, slot_out[i] = the slot
+ * (offset / page size) of training's range that physical page i is mapped at, live or stale, or -1.  Returns the
+ * number of pages written (at most max_pages).  What the pages pool of the reference keeps per page
+ * (common/cuda_allocator.h:48-58), exposed so that a model of the placement can be compared page for page. */
+int tch_pool_page_table(int device, uint8_t* owner_out, int64_t* slot_out, int max_pages);
 /* The pool from ANOTHER process (the inference side; the TVM-side allocator over the same PagesPool,
  * common/cuda_allocator.cc:86-99): attach to the page table, claim FREE pages (lowest index first; returns how
  * many, indices in pages_out), map a claimed page (its device address in this process; the descriptor comes from

@@ -138,3 +138,195 @@ def infer_require_mem_target(cur_target_bs, required_mem_mb, slope, min_train_bs
     if num_gpus > 1:
         t = max(t, min_train_bs)
     return t
+
+
+class PoolModel:
+    """Independent model of where the training allocator places blocks and which physical pages back them.
+
+    Configuration as the reference gives it to the allocator it delegates to (common/cuda_allocator.cc:61-85):
+    32 MB pages (`PageNbytes`, cuda_allocator.h:81-87), small-block threshold = page / 16 = 2 MB, 1024-byte
+    alignment, virtual range 8x the pool; zero-byte requests are null (cuda_allocator.cc:129-132);
+    `FreeTrainLocals` = empty the cache (cuda_allocator.cc:304-307); page states train-local-free -> free <->
+    infer, free -> train (cuda_allocator.h:48-58).  The allocator itself (third_party/mpool) is not in the
+    reference tree, so the policy inside those constants is THIS BUILD'S and is stated here in full -- parity with
+    mpool's own tie-breaking is unpinned; what this model pins is that the C++ pool (CPU backend and HIP
+    virtual-memory backend alike) follows the stated policy offset for offset and page for page:
+
+    * two segments of the range: [0, range/8 rounded up to a page) for requests < 2 MB after rounding to 1024,
+      the rest for the others; each grows at its end, in whole pages;
+    * a request takes the smallest free block that fits (lowest offset among equals); if none fits the segment
+      grows, extending a trailing free block rather than leaving it behind; the block is split when at least
+      one alignment unit remains;
+    * a freed block merges with free neighbours and keeps its pages; empty_cache() returns every page that
+      lies wholly inside free blocks;
+    * a block is backed page by page: a slot that still carries the (stale, lazy mode) mapping of a page
+      nobody took gets that page back; otherwise the lowest-numbered free page that carries no stale mapping,
+      and only then the lowest-numbered one that does;
+    * a request that finds too few free pages empties the cache first and fails (leaving the block free and
+      merged) if that is not enough.
+
+    Written with plain lists and linear scans on purpose (the C++ uses ordered maps and a size index): a shared
+    data-structure mistake cannot hide in both.
+    """
+    ALIGN = 1024
+    FREE, TRAIN, INFER = 0, 1, 2
+
+    def __init__(self, pool_bytes, page_bytes=32 << 20, lazy_unmap=False):
+        self.page = page_bytes
+        self.small_limit_bytes = 2 << 20      # the reference's page / 16 at ITS page size; kept when the page size is a parameter
+        self.n_pages = pool_bytes // page_bytes
+        va = self.n_pages * page_bytes * 8
+        small = -(-(va // 8) // page_bytes) * page_bytes
+        # segment: [begin, limit), frontier, blocks = list of [offset, size, allocated] in address order
+        self.segs = [dict(begin=0, limit=small, frontier=0, blocks=[]),
+                     dict(begin=small, limit=va, frontier=small, blocks=[])]
+        self.owner = [self.FREE] * self.n_pages
+        self.slot_page = {}      # slot -> page mapped there (live or stale)
+        self.slot_live = set()   # slots whose page training owns
+        self.lazy = lazy_unmap
+        self.train_usage = 0
+        self.maps = self.unmaps = self.revives = 0
+
+    # -- pages ---------------------------------------------------------------------------------------
+    def free_pages(self):
+        return sum(1 for o in self.owner if o == self.FREE)
+
+    def train_pages(self):
+        return sum(1 for o in self.owner if o == self.TRAIN)
+
+    def _stale_pages(self):
+        return {p for s, p in self.slot_page.items() if s not in self.slot_live}
+
+    def _take_free_page(self):
+        stale = self._stale_pages()
+        free = [i for i, o in enumerate(self.owner) if o == self.FREE]
+        clean = [i for i in free if i not in stale]
+        if clean:
+            return clean[0]
+        if not free:
+            return None
+        page = free[0]
+        slot = next(s for s, p in self.slot_page.items() if p == page)
+        del self.slot_page[slot]
+        self.unmaps += 1
+        return page
+
+    def _back(self, off, size):
+        slots = range(off // self.page, (off + size - 1) // self.page + 1)
+        if all(s in self.slot_live for s in slots):
+            return True
+        for s in slots:     # a stale mapping whose page is still free comes back as it is
+            if s in self.slot_page and s not in self.slot_live and self.owner[self.slot_page[s]] == self.FREE:
+                self.owner[self.slot_page[s]] = self.TRAIN
+                self.slot_live.add(s)
+                self.revives += 1
+        missing = [s for s in slots if s not in self.slot_live]
+        if not missing:
+            return True
+        if self.free_pages() < len(missing):
+            self.empty_cache()
+            missing = [s for s in slots if s not in self.slot_live]
+            if self.free_pages() < len(missing):
+                return False
+        for s in missing:
+            if s in self.slot_page:          # stale mapping of a page that went elsewhere
+                del self.slot_page[s]
+                self.unmaps += 1
+            page = self._take_free_page()
+            self.owner[page] = self.TRAIN
+            self.slot_page[s] = page
+            self.slot_live.add(s)
+            self.maps += 1
+        return True
+
+    # -- blocks --------------------------------------------------------------------------------------
+    def _seg_of(self, off):
+        return self.segs[0] if off < self.segs[0]["limit"] else self.segs[1]
+
+    def _merge_free(self, seg, i):
+        b = seg["blocks"]
+        if i + 1 < len(b) and not b[i + 1][2]:
+            b[i][1] += b[i + 1][1]
+            del b[i + 1]
+        if i > 0 and not b[i - 1][2]:
+            b[i - 1][1] += b[i][1]
+            del b[i]
+
+    def alloc(self, nbytes):
+        """Offset of the block, or None (zero bytes, out of range, out of pages)."""
+        if nbytes == 0:
+            return None
+        n = -(-nbytes // self.ALIGN) * self.ALIGN
+        seg = self.segs[0] if n < self.small_limit_bytes else self.segs[1]
+        b = seg["blocks"]
+        fits = [(blk[1], blk[0], i) for i, blk in enumerate(b) if not blk[2] and blk[1] >= n]
+        if fits:
+            i = min(fits)[2]
+        else:
+            start = seg["frontier"]
+            if b and not b[-1][2]:
+                start = b[-1][0]
+            frontier = -(-(start + n) // self.page) * self.page
+            if frontier > seg["limit"]:
+                return None
+            if b and not b[-1][2]:
+                b.pop()
+            b.append([start, frontier - start, False])
+            seg["frontier"] = frontier
+            i = len(b) - 1
+        if b[i][1] - n >= self.ALIGN:
+            b.insert(i + 1, [b[i][0] + n, b[i][1] - n, False])
+            b[i][1] = n
+        if not self._back(b[i][0], b[i][1]):
+            # empty_cache inside _back may have changed nothing about the blocks; the block stays free, merged
+            self._merge_free(seg, i)
+            return None
+        b[i][2] = True
+        self.train_usage += n
+        return b[i][0]
+
+    def free(self, off):
+        seg = self._seg_of(off)
+        i = next(k for k, blk in enumerate(seg["blocks"]) if blk[0] == off and blk[2])
+        seg["blocks"][i][2] = False
+        self.train_usage -= seg["blocks"][i][1]
+        self._merge_free(seg, i)
+
+    def empty_cache(self):
+        """Bytes of pages handed back."""
+        slots = []
+        for seg in self.segs:
+            for off, size, allocated in seg["blocks"]:
+                if allocated:
+                    continue
+                lo = -(-off // self.page)
+                hi = (off + size) // self.page
+                slots += [s for s in range(lo, hi) if s in self.slot_live]
+        for s in slots:
+            self.owner[self.slot_page[s]] = self.FREE
+            self.slot_live.discard(s)
+            if not self.lazy:
+                del self.slot_page[s]
+                self.unmaps += 1
+        return len(slots) * self.page
+
+    # -- the other tenant ----------------------------------------------------------------------------
+    def infer_claim(self, n):
+        moved = 0
+        for i in range(self.n_pages):
+            if moved == n:
+                break
+            if self.owner[i] == self.FREE:
+                self.owner[i] = self.INFER
+                moved += 1
+        return moved
+
+    def infer_release(self, n):
+        moved = 0
+        for i in range(self.n_pages - 1, -1, -1):
+            if moved == n:
+                break
+            if self.owner[i] == self.INFER:
+                self.owner[i] = self.FREE
+                moved += 1
+        return moved

@@ -26,6 +26,12 @@ class KernelStat(ctypes.Structure):
                 ("launches", ctypes.c_int64), ("work_is_bytes", ctypes.c_int), ("bytes", ctypes.c_double)]
 
 
+class LaunchStat(ctypes.Structure):
+    """Mirror of tch_launch_stat (include/torch_col_hip.h)."""
+    _fields_ = [("name", ctypes.c_char * 96), ("ms", ctypes.c_double), ("flops", ctypes.c_double),
+                ("bytes", ctypes.c_double), ("lane", ctypes.c_int), ("workgroups", ctypes.c_int64)]
+
+
 class CtrlMsg(ctypes.Structure):
     """Mirror of tch_ctrl_msg (include/torch_col_host.h)."""
     _fields_ = [("id", ctypes.c_uint64), ("event", ctypes.c_int), ("value", ctypes.c_int)]

@@ -542,6 +542,182 @@ __global__ __launch_bounds__(256) void bn_fin_apply_kernel(FinApplyArgs p) {
   }
 }
 
+// Coefficients from exact accumulators AND apply in one launch, for any number of rows: the convolution next to
+// the BatchNorm added its per-tile sums to one pair of accumulators per channel (acc_add), so there are no
+// per-tile partials to add up and no finalize launch.  A workgroup owns CPR chunk columns (CPR * E channels, at
+// most 256: one thread per channel turns the two totals into the channel's coefficients, through LDS) and a slab
+// of rows, which it walks like bn_apply_cols_kernel: a thread keeps one chunk column, four rows per trip.  The
+// workgroups of slab 0 also write the per-channel outputs (saved statistics, running statistics / dgamma, dbeta).
+struct AccApplyArgs {
+  const long long* acc;   // [C][2][kAccWords]: forward sum x, sum x^2; backward sum g, sum g * xhat
+  int C;
+  int64_t rows;
+  const float* gamma;
+  const float* beta;      // forward
+  float* running_mean;    // forward (may be null)
+  float* running_var;
+  float* save_mean;       // forward: written   backward: read
+  float* save_invstd;
+  float* dgamma;          // backward
+  float* dbeta;
+  float momentum, eps;
+  int accumulate;
+  const void* a;          // forward: x         backward: g
+  const void* b;          // forward: residual (may be null)   backward: x
+  void* out;
+  int relu;
+  int rows_per_slab;
+  int nt;                 // stream the inputs past the caches
+};
+
+template <typename T, int BWD, int CPR>
+__global__ __launch_bounds__(256) void bn_acc_apply_kernel(AccApplyArgs p) {
+  constexpr int E = Elem<T>::kPerChunk;
+  constexpr int COLS = CPR * E;
+  static_assert(COLS <= 256, "one thread per channel of the workgroup");
+  constexpr int RPP = 256 / CPR;   // rows per pass of the workgroup
+  constexpr int U = 4;
+  __shared__ float coef[3][COLS];
+  const int tid = threadIdx.x;
+  const int c0 = blockIdx.x * COLS;
+  if (tid < COLS) {
+    const int c = c0 + tid;
+    const double s = acc_total(p.acc + static_cast<int64_t>(c) * 2 * kAccWords);
+    const double q = acc_total(p.acc + static_cast<int64_t>(c) * 2 * kAccWords + kAccWords);
+    const double n = static_cast<double>(p.rows);
+    const bool writer = blockIdx.y == 0;
+    if (!BWD) {
+      const double mean = s / n;
+      double var = q / n - mean * mean;
+      if (var < 0.0) var = 0.0;
+      const float invstd = 1.0f / sqrtf(static_cast<float>(var) + p.eps);
+      const float sc = p.gamma[c] * invstd;
+      coef[0][tid] = sc;
+      coef[1][tid] = p.beta[c] - static_cast<float>(mean) * sc;
+      if (writer) {
+        p.save_mean[c] = static_cast<float>(mean);
+        p.save_invstd[c] = invstd;
+        if (p.running_mean) {
+          const double unbiased = p.rows > 1 ? var * n / (n - 1.0) : var;
+          p.running_mean[c] = (1.f - p.momentum) * p.running_mean[c] + p.momentum * static_cast<float>(mean);
+          p.running_var[c] = (1.f - p.momentum) * p.running_var[c] + p.momentum * static_cast<float>(unbiased);
+        }
+      }
+    } else {
+      const double invstd = p.save_invstd[c];
+      const double scale = static_cast<double>(p.gamma[c]) * invstd;
+      const double cb = -scale * invstd * (q / n);
+      const double cz = -scale * (s / n) - cb * p.save_mean[c];
+      coef[0][tid] = static_cast<float>(scale);
+      coef[1][tid] = static_cast<float>(cb);
+      coef[2][tid] = static_cast<float>(cz);
+      if (writer) {
+        const float db = static_cast<float>(s), dg = static_cast<float>(q);
+        p.dbeta[c] = p.accumulate ? p.dbeta[c] + db : db;
+        p.dgamma[c] = p.accumulate ? p.dgamma[c] + dg : dg;
+      }
+    }
+  }
+  __syncthreads();
+
+  const int tx = tid % CPR, ty = tid / CPR;
+  float k0[E], k1[E], k2[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    k0[e] = coef[0][tx * E + e];
+    k1[e] = coef[1][tx * E + e];
+    k2[e] = BWD ? coef[2][tx * E + e] : 0.f;
+  }
+  const int64_t cc = p.C / E;
+  const int64_t col_chunk = static_cast<int64_t>(blockIdx.x) * CPR + tx;
+  const int64_t r0 = static_cast<int64_t>(blockIdx.y) * p.rows_per_slab;
+  int64_t r1 = r0 + p.rows_per_slab;
+  if (r1 > p.rows) r1 = p.rows;
+  const bool has_b = BWD || p.b != nullptr;
+  for (int64_t r = r0 + ty; r < r1; r += U * RPP) {
+    Chunk ca[U], cb[U];
+#pragma unroll
+    for (int q = 0; q < U; ++q) {
+      const int64_t row = r + q * RPP;
+      ca[q] = cb[q] = zero_chunk();
+      if (row < r1) {
+        const int64_t i = row * cc + col_chunk;
+        if (p.nt) {
+          ca[q].u = load_streaming_u4(p.a, i);
+          if (has_b) cb[q].u = load_streaming_u4(p.b, i);
+        } else {
+          ca[q].u = static_cast<const uint4*>(p.a)[i];
+          if (has_b) cb[q].u = static_cast<const uint4*>(p.b)[i];
+        }
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < U; ++q) {
+      const int64_t row = r + q * RPP;
+      if (row >= r1) continue;
+      float va[E], vb[E], vo[E];
+      chunk_to_float<T>(ca[q], va);
+      chunk_to_float<T>(cb[q], vb);
+      if (BWD) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) vo[e] = k0[e] * va[e] + k1[e] * vb[e] + k2[e];
+      } else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) vo[e] = va[e] * k0[e] + k1[e];
+        if (p.b) {
+#pragma unroll
+          for (int e = 0; e < E; ++e) vo[e] += vb[e];
+        }
+        if (p.relu) {
+#pragma unroll
+          for (int e = 0; e < E; ++e) vo[e] = vo[e] > 0.f ? vo[e] : 0.f;
+        }
+      }
+      static_cast<uint4*>(p.out)[row * cc + col_chunk] = float_to_chunk<T>(vo).u;
+    }
+  }
+}
+
+// Workgroups to aim for: a small tensor (the 14x14 and 7x7 stages) wants few, since every workgroup repeats the
+// coefficient prologue; a large one wants many short ones (TCH_BN_ACC_WGS / TCH_BN_ACC_WGS_LARGE).
+template <typename T, int BWD, int CPR>
+int launch_acc_apply(Context* ctx, AccApplyArgs& a, const char* name, double bytes) {
+  static const int target_small = [] {
+    const char* e = getenv("TCH_BN_ACC_WGS");
+    return e && atoi(e) > 0 ? atoi(e) : 512;
+  }();
+  static const int target_large = [] {
+    const char* e = getenv("TCH_BN_ACC_WGS_LARGE");
+    return e && atoi(e) > 0 ? atoi(e) : 4096;
+  }();
+  constexpr int E = Elem<T>::kPerChunk;
+  constexpr int trip = 4 * (256 / CPR);
+  const int64_t col_blocks = a.C / (CPR * E);
+  const double tensor_mb = static_cast<double>(a.rows) * a.C * sizeof(T) / 1e6;
+  const int target = tensor_mb > 40.0 ? target_large : target_small;
+  int64_t slabs = target / col_blocks;
+  if (slabs < 1) slabs = 1;
+  int64_t rps = (a.rows + slabs - 1) / slabs;
+  rps = (rps + trip - 1) / trip * trip;
+  a.rows_per_slab = static_cast<int>(rps);
+  static const int nt = [] {
+    const char* e = getenv("TCH_BN_APPLY_NT");
+    return e ? atoi(e) : 1;
+  }();
+  a.nt = (nt && tensor_mb > 40.0) ? 1 : 0;   // small tensors were just written and sit in the caches
+  const dim3 grid(static_cast<unsigned>(col_blocks), static_cast<unsigned>((a.rows + rps - 1) / rps));
+  return launch(ctx, bn_acc_apply_kernel<T, BWD, CPR>, grid, dim3(256), a, name, bytes, 1);
+}
+
+template <typename T, int BWD>
+int launch_acc_apply_t(Context* ctx, AccApplyArgs& a, const char* name, double bytes) {
+  constexpr int E = Elem<T>::kPerChunk;
+  const int cc = a.C / E;
+  if (cc % 32 == 0) return launch_acc_apply<T, BWD, 32>(ctx, a, name, bytes);
+  if (cc % 16 == 0) return launch_acc_apply<T, BWD, 16>(ctx, a, name, bytes);
+  return launch_acc_apply<T, BWD, 8>(ctx, a, name, bytes);
+}
+
 // rows per slab so that the grid has about 512 workgroups (TCH_BN_FUSED_WGS), at least 32 rows each: alone the
 // kernel takes the same time with 512 to 1024, in the step 512 is 0.1 ms faster (every workgroup repeats the
 // sum over the partials, and the weight gradients on the other stream want the room)
@@ -846,6 +1022,33 @@ int bn_bwd_partials(Context* ctx, int dtype, const void* g, const void* x, void*
   const double tensor_bytes = static_cast<double>(rows) * C * eb;
   ApplyArgs a{g, nullptr, x, dx, coef, coef + C, coef + 2 * C, rows * geo.cc, FastDiv(geo.cc), 0};
   return launch_apply(ctx, dtype, true, a, tensor_bytes * 3.0);
+}
+
+int bn_fwd_train_acc(Context* ctx, int dtype, const void* x, void* y, const void* residual, int relu, int64_t rows,
+                     int C, const float* gamma, const float* beta, float* running_mean, float* running_var,
+                     float* save_mean, float* save_invstd, float momentum, float eps, const long long* acc) {
+  if (int rc = check_common(rows, C, dtype)) return rc;
+  TCH_CHECK_ARG(x && y && gamma && beta && save_mean && save_invstd && acc, "bn_fwd_train_acc: null tensor");
+  TCH_CHECK_ARG((running_mean == nullptr) == (running_var == nullptr), "bn_fwd_train_acc: running stats come in pairs");
+  TCH_CHECK_ARG(C % (dtype == kBF16 ? 64 : 32) == 0, "bn_fwd_train_acc: channels must come in groups of eight 16-byte chunks");
+  AccApplyArgs a{acc, C, rows, gamma, beta, running_mean, running_var, save_mean, save_invstd, nullptr, nullptr,
+                 momentum, eps, 0, x, residual, y, relu, 0, 0};
+  const double bytes = static_cast<double>(rows) * C * (dtype == kBF16 ? 2.0 : 4.0) * (residual ? 3.0 : 2.0);
+  return dtype == kBF16 ? launch_acc_apply_t<bf16, 0>(ctx, a, "bn_acc_apply_kernel<bf16,fwd>", bytes)
+                        : launch_acc_apply_t<float, 0>(ctx, a, "bn_acc_apply_kernel<f32,fwd>", bytes);
+}
+
+int bn_bwd_acc(Context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int C,
+               const float* gamma, const float* save_mean, const float* save_invstd, float* dgamma, float* dbeta,
+               int accumulate, const long long* acc) {
+  if (int rc = check_common(rows, C, dtype)) return rc;
+  TCH_CHECK_ARG(g && x && dx && gamma && save_mean && save_invstd && dgamma && dbeta && acc, "bn_bwd_acc: null tensor");
+  TCH_CHECK_ARG(C % (dtype == kBF16 ? 64 : 32) == 0, "bn_bwd_acc: channels must come in groups of eight 16-byte chunks");
+  AccApplyArgs a{acc, C, rows, gamma, nullptr, nullptr, nullptr, const_cast<float*>(save_mean),
+                 const_cast<float*>(save_invstd), dgamma, dbeta, 0.f, 0.f, accumulate, g, x, dx, 0, 0, 0};
+  const double bytes = static_cast<double>(rows) * C * (dtype == kBF16 ? 2.0 : 4.0) * 3.0;
+  return dtype == kBF16 ? launch_acc_apply_t<bf16, 1>(ctx, a, "bn_acc_apply_kernel<bf16,bwd>", bytes)
+                        : launch_acc_apply_t<float, 1>(ctx, a, "bn_acc_apply_kernel<f32,bwd>", bytes);
 }
 
 }  // namespace tch

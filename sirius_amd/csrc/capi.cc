@@ -256,6 +256,41 @@ int tch_bn_bwd_partials(tch_context* ctx, int dtype, const void* g, const void* 
                          partial, row_blocks, scratch);
 }
 
+int tch_conv2d_fwd_bnacc(tch_context* ctx, int dtype, const void* x, const void* w, void* y, int N, int H, int W,
+                         int Cc, int K, int R, int S, int stride, int pad, int tile_cfg, int c_logical,
+                         int64_t* bn_acc) {
+  if (!bn_acc) {
+    set_error("tch_conv2d_fwd_bnacc: null accumulator buffer");
+    return -22;
+  }
+  return conv2d_fwd(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad, c_logical), x, w, y, nullptr, nullptr, nullptr,
+                    0, tile_cfg, nullptr, nullptr, nullptr, 0, reinterpret_cast<long long*>(bn_acc));
+}
+
+int tch_conv2d_dgrad_bnacc(tch_context* ctx, int dtype, const void* dy, const void* w, void* dx, const void* add,
+                           const void* mask, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad,
+                           int tile_cfg, int c_logical, const void* bn_mask, const void* bn_x, const float* bn_mean,
+                           const float* bn_invstd, int64_t* bn_acc, int add_stride) {
+  BnBwdSums bn{bn_mask, bn_x, bn_mean, bn_invstd, nullptr, nullptr, reinterpret_cast<long long*>(bn_acc)};
+  return conv2d_dgrad(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad, c_logical), dy, w, dx, add, mask, tile_cfg,
+                      &bn, add_stride);
+}
+
+int tch_bn_fwd_train_acc(tch_context* ctx, int dtype, const void* x, void* y, const void* residual, int relu,
+                         int64_t rows, int Cc, const float* gamma, const float* beta, float* running_mean,
+                         float* running_var, float* save_mean, float* save_invstd, float momentum, float eps,
+                         const int64_t* acc) {
+  return bn_fwd_train_acc(C(ctx), dtype, x, y, residual, relu, rows, Cc, gamma, beta, running_mean, running_var, save_mean,
+                          save_invstd, momentum, eps, reinterpret_cast<const long long*>(acc));
+}
+
+int tch_bn_bwd_acc(tch_context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int Cc,
+                   const float* gamma, const float* save_mean, const float* save_invstd, float* dgamma, float* dbeta,
+                   int accumulate, const int64_t* acc) {
+  return bn_bwd_acc(C(ctx), dtype, g, x, dx, rows, Cc, gamma, save_mean, save_invstd, dgamma, dbeta, accumulate,
+                    reinterpret_cast<const long long*>(acc));
+}
+
 int tch_layernorm_fwd(tch_context* ctx, int dtype, const void* x, void* y, const float* gamma, const float* beta,
                       float* mean, float* rstd, int64_t rows, int Cc, float eps) {
   return layernorm_fwd(C(ctx), dtype, x, y, gamma, beta, mean, rstd, rows, Cc, eps);
@@ -612,6 +647,30 @@ extern "C" int tch_program_profile(tch_context* ctx, const tch_program* prog, in
     o.launches = s.launches;
     o.work_is_bytes = s.work_is_bytes;
     o.bytes = s.bytes;
+  }
+  *n_out = n;
+  return 0;
+}
+
+extern "C" int tch_program_profile_launches(tch_context* ctx, const tch_program* prog, int reps, tch_launch_stat* out,
+                                            int64_t max_out, int64_t* n_out) {
+  if (!ctx || !prog || !out || !n_out || max_out < 1) {
+    set_error("tch_program_profile_launches: bad arguments");
+    return -22;
+  }
+  std::vector<LaunchStat> stats;
+  int rc = profile_program(&ctx->ctx, prog->prog, reps, nullptr, &stats);
+  if (rc) return rc;
+  int64_t n = 0;
+  for (auto& s : stats) {
+    if (n >= max_out) break;
+    tch_launch_stat& o = out[n++];
+    snprintf(o.name, sizeof(o.name), "%s", s.name.c_str());
+    o.ms = s.ms;
+    o.flops = s.flops;
+    o.bytes = s.bytes;
+    o.lane = s.lane;
+    o.workgroups = s.grid;
   }
   *n_out = n;
   return 0;

@@ -626,9 +626,11 @@ int submit(Context* ctx, const void* fn, dim3 grid, dim3 block, const void* args
 // per-kernel timing of a recorded program
 // ---------------------------------------------------------------------------
 
-int profile_program(Context* ctx, const Program& prog, int reps, std::vector<KernelStat>* out) {
+int profile_program(Context* ctx, const Program& prog, int reps, std::vector<KernelStat>* out,
+                    std::vector<LaunchStat>* per_launch) {
   const size_t n = prog.launches.size();
   if (n == 0 || reps < 1) return 0;
+  if (per_launch) per_launch->assign(n, LaunchStat());
   std::vector<hipEvent_t> ev(n + 1, nullptr);
   for (auto& e : ev) {
     if (hipEventCreate(&e) != hipSuccess) {
@@ -664,10 +666,19 @@ int profile_program(Context* ctx, const Program& prog, int reps, std::vector<Ker
       k.launches += 1;
       k.work_is_bytes = l.work_is_bytes;
       k.bytes += l.bytes;
+      if (per_launch) {
+        LaunchStat& p = (*per_launch)[i];
+        p.name = k.name;
+        p.ms += ms / reps;
+        p.flops = l.work_is_bytes ? 0.0 : l.work;
+        p.bytes = l.bytes;
+        p.lane = l.lane;
+        p.grid = static_cast<int64_t>(l.grid.x) * l.grid.y * l.grid.z;
+      }
     }
   }
   for (auto e : ev) (void)hipEventDestroy(e);
-  if (rc == 0)
+  if (rc == 0 && out)
     for (auto& kv : agg) out->push_back(kv.second);
   return rc;
 }

@@ -178,9 +178,21 @@ struct KernelStat {
   double bytes = 0.0;  // sum of the algorithmic bytes of the launches (0 where a flops-annotated launch gave none)
 };
 
+// One launch of a program as the profiler saw it (entries that are not kernel launches keep an empty name).
+struct LaunchStat {
+  std::string name;
+  double ms = 0.0;     // mean HIP-event time over the repetitions
+  double flops = 0.0;  // algorithmic flops (0 for a launch annotated with bytes only)
+  double bytes = 0.0;  // algorithmic bytes
+  int lane = 0;
+  int64_t grid = 0;    // workgroups
+};
+
 // Replays prog `reps` times directly on the context's stream with a HIP event between any
-// two launches and sums the elapsed time per kernel name.
-int profile_program(Context* ctx, const Program& prog, int reps, std::vector<KernelStat>* out);
+// two launches and sums the elapsed time per kernel name (`out`) and / or per launch (`per_launch`,
+// one entry per program position).
+int profile_program(Context* ctx, const Program& prog, int reps, std::vector<KernelStat>* out,
+                    std::vector<LaunchStat>* per_launch = nullptr);
 
 // ---- process-wide registry of preemptible streams (xsched_ctrl equivalent) ----
 uint64_t register_stream(uint64_t stream);  // returns a handle, 0 on failure

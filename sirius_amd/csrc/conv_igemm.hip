@@ -61,6 +61,7 @@ struct IgemmArgs {
   int relu_out;       // FWD: the stored output is max(0, .) of everything above
   float* dbias;       // WGRAD, optional: column sums of dy (the gradient of that bias), [splits][K] partials or final
   float* stats;       // optional: per (row tile, column) pair of sums over the stored output (see finish_tile)
+  long long* stat_acc;  // optional, instead of stats: the same pair added to exact accumulators, [column][2][kAccWords]
   const void* bn_mask;      // DGRAD with stats, optional: the stored output is zeroed where bn_mask <= 0
   const void* bn_x;         // DGRAD with stats: input of the BatchNorm this gradient flows into, laid out like out
   const float* bn_mean;     // DGRAD with stats: that BatchNorm's saved batch mean / inverse std per column
@@ -324,7 +325,7 @@ __device__ inline void finish_tile(const IgemmArgs& p, f32x16_t (&acc)[TM][TN], 
   constexpr int CH = BN / E;   // column chunks of the tile; a thread always gets chunk tid % CH
   constexpr int ROWS = NT / CH;
   static_assert(NT % CH == 0, "stats mapping");
-  const bool want_stats = p.stats != nullptr;
+  const bool want_stats = p.stats != nullptr || p.stat_acc != nullptr;
   float st_sum[E], st_sq[E];
 #pragma unroll
   for (int e = 0; e < E; ++e) st_sum[e] = st_sq[e] = 0.f;
@@ -457,7 +458,11 @@ __device__ inline void finish_tile(const IgemmArgs& p, f32x16_t (&acc)[TM][TN], 
         b += red[((r * CH + cc) * 2 * E) + E + e];
       }
       const int col = n0 + tid;
-      if (col < p.gemm_n) {
+      if (col < p.gemm_n && p.stat_acc) {
+        // every row tile adds to the same pair of accumulators: no per-tile partials, nothing to sum up later
+        acc_add(p.stat_acc + static_cast<int64_t>(col) * 2 * kAccWords, a);
+        acc_add(p.stat_acc + static_cast<int64_t>(col) * 2 * kAccWords + kAccWords, b);
+      } else if (col < p.gemm_n) {
         float2* dst = reinterpret_cast<float2*>(p.stats + (static_cast<int64_t>(tile_m) * p.gemm_n + col) * 2);
         if (p.fin_counters) {
           // published for the workgroup that finishes this column tile (see finalize_column_tile)
@@ -1773,10 +1778,13 @@ void bind_finalize(IgemmArgs& a, const BnFinalize* f) {
 
 int conv2d_fwd(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* w, void* y, const void* add,
                const void* mask, const float* bias, int out_f32, int tile_cfg, float* bn_partial,
-               const BnFinalize* finalize, const float* scale, int relu_out) {
+               const BnFinalize* finalize, const float* scale, int relu_out, long long* bn_acc) {
   IgemmArgs a{};
   if (int rc = fill_common(a, s, dtype)) return rc;
-  TCH_CHECK_ARG(!((scale || relu_out) && bn_partial), "conv2d_fwd: statistics are taken of the plain convolution output");
+  TCH_CHECK_ARG(!((scale || relu_out) && (bn_partial || bn_acc)), "conv2d_fwd: statistics are taken of the plain convolution output");
+  TCH_CHECK_ARG(!(bn_acc && (bn_partial || finalize || out_f32)),
+                "conv2d_fwd: accumulated statistics replace the per-tile ones and are taken of outputs stored in the compute type");
+  a.stat_acc = bn_acc;
   a.scale = scale;
   a.relu_out = relu_out ? 1 : 0;
   TCH_CHECK_ARG(x && w && y, "conv2d_fwd: null tensor");
@@ -1802,7 +1810,7 @@ int conv2d_fwd(Context* ctx, int dtype, const ConvShape& s, const void* x, const
   if (tile_cfg < 0) {
     tile_cfg = shallow_tile(pick_tile(a.gemm_m, a.gemm_n, 1), dtype, s.C, s.R * s.S);
     // statistics are sized by the caller for the heuristic's row tiles: leave those launches alone
-    if (!bn_partial && wants_huge_tile(dtype, a.gemm_m, a.gemm_n, s.C, s.R * s.S)) tile_cfg = 10;
+    if (!bn_partial && !bn_acc && wants_huge_tile(dtype, a.gemm_m, a.gemm_n, s.C, s.R * s.S)) tile_cfg = 10;
   }
   tile_cfg = effective_tile(tile_cfg, dtype, s.C, s.R * s.S);
   const int row_tiles = (a.gemm_m + tile_rows(tile_cfg) - 1) / tile_rows(tile_cfg);
@@ -1842,9 +1850,12 @@ int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, co
   TCH_CHECK_ARG(add_stride == 1 || add_stride == 2, "conv2d_dgrad: the addend's grid is the output's or every second pixel of it");
   a.add_sub = (add && add_stride == 2) ? 1 : 0;
   if (bn) {
-    TCH_CHECK_ARG(bn->x && bn->mean && bn->invstd && bn->partial, "conv2d_dgrad: incomplete BatchNorm operands");
-    TCH_CHECK_ARG(!bn->finalize || check_finalize(bn->finalize, false), "conv2d_dgrad: incomplete BatchNorm finalize operands");
+    TCH_CHECK_ARG(bn->x && bn->mean && bn->invstd && ((bn->partial != nullptr) != (bn->acc != nullptr)),
+                  "conv2d_dgrad: incomplete BatchNorm operands");
+    TCH_CHECK_ARG(!bn->finalize || (bn->partial && check_finalize(bn->finalize, false)),
+                  "conv2d_dgrad: incomplete BatchNorm finalize operands");
     a.stats = bn->partial;
+    a.stat_acc = bn->acc;
     a.bn_mask = bn->mask;
     a.bn_x = bn->x;
     a.bn_mean = bn->mean;

@@ -185,6 +185,10 @@ void tch_pool_counters(int device, uint64_t* out6) {
   out6[4] = s.num_revives;
   out6[5] = s.stale_pages;
 }
+int tch_pool_page_table(int device, uint8_t* owner_out, int64_t* slot_out, int max_pages) {
+  auto p = pool(device);
+  return p ? p->page_table(owner_out, slot_out, max_pages) : 0;
+}
 uint64_t tch_pool_unmap_calls(int device) { auto p = pool(device); return p ? p->stats().num_unmap_calls : 0; }
 uint64_t tch_pool_trim(int device, uint64_t max_pages) { auto p = pool(device); return p ? p->trim(max_pages) : 0; }
 int tch_pool_infer_claim_pages(int d, int n) { auto p = pool(d); return p ? p->infer_claim_pages(n) : 0; }

@@ -573,6 +573,17 @@ int64_t HbmPool::offset_of(const void* ptr) const {
   return static_cast<int64_t>(a - base_);
 }
 
+int HbmPool::page_table(uint8_t* owner_out, int64_t* slot_out, int max_pages) {
+  std::lock_guard<std::mutex> lock(mu_);
+  ShmLock table_lock(&table_->mu);
+  const int n = std::min(max_pages, num_pages_);
+  for (int i = 0; i < n; ++i) {
+    if (owner_out) owner_out[i] = table_->owner[i];
+    if (slot_out) slot_out[i] = page_slot_[i];
+  }
+  return n;
+}
+
 int HbmPool::infer_claim_pages(int n) {
   std::lock_guard<std::mutex> lock(mu_);
   ShmLock table_lock(&table_->mu);

@@ -156,6 +156,8 @@ class HbmPool {
   size_t page_bytes() const { return page_bytes_; }
   PoolBackend* backend() { return backend_.get(); }
   int64_t offset_of(const void* ptr) const;
+  // owner of every physical page and the slot it is mapped at (live or stale, -1: none); returns pages written
+  int page_table(uint8_t* owner_out, int64_t* slot_out, int max_pages);
 
   // the inference side inside this process (a stand-in peer on a thread): label FREE pages as
   // inference-owned / give them back.  Returns the number of pages actually moved.

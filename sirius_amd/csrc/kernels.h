@@ -182,6 +182,32 @@ __device__ inline float wave_max(float v) {
   return v;
 }
 
+// ---------------------------------------------------------------------------
+// exact accumulators for per-channel sums that many workgroups contribute to
+// ---------------------------------------------------------------------------
+// A sum over workgroups by floating-point atomics depends on the order the workgroups finish in; a sum of
+// integers does not.  An accumulator is a pair of 64-bit integers: a contribution v (fp32) is split exactly
+// into hi = trunc(v * 2^24) (units of 2^-24) and lo = round((v - hi * 2^-24) * 2^66) (units of 2^-66),
+// each added with an integer atomic that returns nothing (no wave waits for it).  Only what lies below
+// 2^-66 (1.4e-20) of a contribution is dropped, |v| < 2^38 and up to 2^20 contributions fit; the total
+// hi * 2^-24 + lo * 2^-66 is the same whatever order the additions happened in, so the kernels that read it
+// are bit-identical from run to run.
+constexpr int kAccWords = 2;   // 64-bit words per accumulator
+__device__ inline void acc_add(long long* acc, float v) {
+  const double d = static_cast<double>(v);
+  const long long hi = static_cast<long long>(d * 16777216.0);
+  const double rest = d - static_cast<double>(hi) * (1.0 / 16777216.0);
+  const long long lo = __double2ll_rn(rest * 73786976294838206464.0);   // 2^66
+  atomicAdd(reinterpret_cast<unsigned long long*>(acc), static_cast<unsigned long long>(hi));
+  atomicAdd(reinterpret_cast<unsigned long long*>(acc) + 1, static_cast<unsigned long long>(lo));
+}
+// read by a LATER launch than the ones that added (device-scope loads: they do not trust a cached copy)
+__device__ inline double acc_total(const long long* acc) {
+  const long long hi = __hip_atomic_load(acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const long long lo = __hip_atomic_load(acc + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return static_cast<double>(hi) * (1.0 / 16777216.0) + static_cast<double>(lo) * (1.0 / 73786976294838206464.0);
+}
+
 // Workgroups are dealt round-robin to the 8 XCDs (each with a private L2).
 // Remap the hardware workgroup id so that CONSECUTIVE logical ids land on the
 // same XCD: neighbouring tiles then share operand rows through one L2.

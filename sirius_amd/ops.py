@@ -148,6 +148,18 @@ class Context:
         return [dict(name=buf[i].name.decode(), total_ms=buf[i].total_ms, launches=int(buf[i].launches),
                      work=buf[i].work, work_is_bytes=bool(buf[i].work_is_bytes), bytes=buf[i].bytes) for i in range(n.value)]
 
+    def profile_launches(self, program, reps=1):
+        """The same replay, one dict per program position: name ('' for an entry that launches nothing), ms
+        (mean over the repetitions, the launch alone on the chip), flops, bytes (algorithmic), lane, workgroups."""
+        from ._lib import LaunchStat
+        cap = len(program)
+        buf = (LaunchStat * cap)()
+        n = ctypes.c_int64(0)
+        check(lib().tch_program_profile_launches(self.handle, program.handle, reps, buf, cap, ctypes.byref(n)),
+              "tch_program_profile_launches")
+        return [dict(name=buf[i].name.decode(), ms=buf[i].ms, flops=buf[i].flops, bytes=buf[i].bytes,
+                     lane=int(buf[i].lane), workgroups=int(buf[i].workgroups)) for i in range(n.value)]
+
 
 # ---------------------------------------------------------------------------
 # convolution
@@ -209,6 +221,23 @@ def conv2d_fwd_bnstats(ctx, x, w, y, stride, pad, partial, tile_cfg=-1, c_logica
     return rb
 
 
+def _check_acc(acc, C):
+    assert acc.dtype == torch.int64 and acc.numel() == 4 * C and acc.is_contiguous(), "accumulators: [C, 2, 2] int64"
+
+
+def conv2d_fwd_bnacc(ctx, x, w, y, stride, pad, acc, tile_cfg=-1, c_logical=0):
+    """conv2d_fwd that also ADDS the BatchNorm sums of y (sum, sum of squares per output channel) to the exact
+    accumulators `acc` ([K, 2, 2] int64, zero before the call): no per-tile partials, see bn_fwd_train_acc."""
+    N, H, W, C = x.shape
+    K, R, S, C2 = w.shape
+    assert C == C2 and w.dtype == x.dtype == y.dtype
+    Ho, Wo = conv_out_hw(H, W, R, S, stride, pad)
+    assert tuple(y.shape) == (N, Ho, Wo, K)
+    _check_acc(acc, K)
+    check(lib().tch_conv2d_fwd_bnacc(ctx.handle, dtype_code(x), _p(x), _p(w), _p(y), N, H, W, C, K, R, S, stride, pad,
+                                     tile_cfg, c_logical, _p(acc)), "tch_conv2d_fwd_bnacc")
+
+
 def _check_addend(add, dx, add_stride):
     """add is laid out like dx, or (add_stride 2) holds the even (h, w) of dx's grid only."""
     assert add_stride in (1, 2)
@@ -262,6 +291,27 @@ def conv2d_dgrad_bnsums(ctx, dy, wt, dx, stride, pad, bn_x, bn_mean, bn_invstd, 
                                         N, H, W, C, K, R, S, stride, pad, tile_cfg, c_logical, _p(bn_mask), _p(bn_x),
                                         _p(bn_mean), _p(bn_invstd), _p(partial), add_stride), "tch_conv2d_dgrad_bnsums")
     return rb
+
+
+def conv2d_dgrad_bnacc(ctx, dy, wt, dx, stride, pad, bn_x, bn_mean, bn_invstd, acc, bn_mask=None, add=None,
+                       mask=None, tile_cfg=-1, c_logical=0, add_stride=1):
+    """conv2d_dgrad_bnsums with the two reductions ADDED to the exact accumulators `acc` ([C, 2, 2] int64, zero before
+    the call) instead of left per row tile; see bn_bwd_acc."""
+    N, H, W, C = dx.shape
+    C2, R, S, K = wt.shape
+    assert C == C2
+    Ho, Wo = conv_out_hw(H, W, R, S, stride, pad)
+    assert tuple(dy.shape) == (N, Ho, Wo, K)
+    assert dy.dtype == wt.dtype == dx.dtype
+    for t in (mask, bn_mask, bn_x):
+        assert t is None or (t.shape == dx.shape and t.dtype == dx.dtype)
+    _check_addend(add, dx, add_stride)
+    assert bn_x is not None and bn_mean.numel() == C and bn_invstd.numel() == C
+    assert bn_mean.dtype == bn_invstd.dtype == torch.float32
+    _check_acc(acc, C)
+    check(lib().tch_conv2d_dgrad_bnacc(ctx.handle, dtype_code(dy), _p(dy), _p(wt), _p(dx), _p(add), _p(mask),
+                                       N, H, W, C, K, R, S, stride, pad, tile_cfg, c_logical, _p(bn_mask), _p(bn_x),
+                                       _p(bn_mean), _p(bn_invstd), _p(acc), add_stride), "tch_conv2d_dgrad_bnacc")
 
 
 def conv2d_fwd_bn(ctx, x, w, y, stride, pad, partial, counters, gamma, beta, running_mean, running_var, save_mean,
@@ -463,6 +513,31 @@ def bn_fwd_train_partials(ctx, x, y, gamma, beta, running_mean, running_var, sav
                                           _p(gamma), _p(beta), _p(running_mean), _p(running_var), _p(save_mean),
                                           _p(save_invstd), momentum, eps, _p(partial), int(row_blocks), _p(scratch)),
           "tch_bn_fwd_train_partials")
+
+
+def bn_fwd_train_acc(ctx, x, y, gamma, beta, running_mean, running_var, save_mean, save_invstd, acc, residual=None,
+                     relu=False, momentum=0.1, eps=1e-5):
+    """bn_fwd_train from the accumulators conv2d_fwd_bnacc added the statistics of x to: one launch."""
+    C = x.shape[-1]
+    rows = x.numel() // C
+    assert y.shape == x.shape and y.dtype == x.dtype
+    assert residual is None or (residual.shape == x.shape and residual.dtype == x.dtype)
+    for t in (gamma, beta, save_mean, save_invstd):
+        assert t.dtype == torch.float32 and t.numel() == C
+    _check_acc(acc, C)
+    check(lib().tch_bn_fwd_train_acc(ctx.handle, dtype_code(x), _p(x), _p(y), _p(residual), int(relu), rows, C,
+                                     _p(gamma), _p(beta), _p(running_mean), _p(running_var), _p(save_mean),
+                                     _p(save_invstd), momentum, eps, _p(acc)), "tch_bn_fwd_train_acc")
+
+
+def bn_bwd_acc(ctx, g, x, dx, gamma, save_mean, save_invstd, dgamma, dbeta, acc, accumulate=False):
+    """bn_bwd from the accumulators conv2d_dgrad_bnacc added the two sums to; g is already gated by the ReLU."""
+    C = x.shape[-1]
+    rows = x.numel() // C
+    assert g.shape == x.shape == dx.shape and g.dtype == x.dtype == dx.dtype
+    _check_acc(acc, C)
+    check(lib().tch_bn_bwd_acc(ctx.handle, dtype_code(x), _p(g), _p(x), _p(dx), rows, C, _p(gamma), _p(save_mean),
+                               _p(save_invstd), _p(dgamma), _p(dbeta), int(accumulate), _p(acc)), "tch_bn_bwd_acc")
 
 
 def bn_bwd(ctx, dy, x, dx, gamma, save_mean, save_invstd, dgamma, dbeta, workspace, relu_mask=None,

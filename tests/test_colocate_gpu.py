@@ -100,6 +100,19 @@ def test_pool_on_hip_vmm_matches_cpu_model(clean_runtime):
         L.tch_pool_shutdown(0)
 
 
+@pytest.mark.parametrize("page_mb,lazy", [(32, 0), (32, 1), (128, 0)])
+def test_pool_on_hip_vmm_follows_the_independent_model(clean_runtime, page_mb, lazy):
+    """The HIP virtual-memory pool against oracle.host.PoolModel (not against the pool's own CPU backend): offsets,
+    refusals, the owner of every physical page and the slot it is mapped at, after every operation of the walk."""
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    from pool_walk import walk_against_model
+    torch.cuda.init()
+    print("pool walk against the model, page", page_mb, "MB, lazy", lazy, flush=True)
+    ok, refused = walk_against_model(lib(), 7, 1024, page_mb, lazy, use_gpu=True, steps=300)
+    assert ok > 80 and refused > 0
+
+
 class _RawBytes:
     """A span of device memory for torch to wrap without copying (CUDA array interface)."""
 

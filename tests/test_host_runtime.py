@@ -691,6 +691,53 @@ def test_pool_no_overlap_and_best_fit(fresh):
         L.tch_pool_shutdown(0)
 
 
+@pytest.mark.parametrize("pool_mb,page_mb,lazy", [(1024, 32, 0), (1024, 32, 1), (512, 64, 0), (2048, 128, 1)])
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_pool_placement_follows_the_independent_model(fresh, seed, pool_mb, page_mb, lazy):
+    """oracle.host.PoolModel states the placement policy with lists and linear scans; the C++ pool (ordered maps,
+    a size index, a shared page table) must agree with it after EVERY operation of a random walk: the offset of
+    each block, which requests are refused, the bytes empty_cache returns, the owner of every physical page and
+    the slot it is mapped at -- in eager and lazy unmapping, at three page sizes, with the other tenant taking
+    and returning pages in between.  (The reference's own allocator, mpool, is not in its tree: what is pinned is
+    that the pool follows the policy this build states, not mpool's tie-breaking.)"""
+    from pool_walk import walk_against_model
+    ok, refused = walk_against_model(fresh, seed, pool_mb, page_mb, lazy, use_gpu=False)
+    assert ok > 150, "the walk must allocate"
+    if pool_mb <= 1024:
+        assert refused > 0, "and must run out of pages now and then (the refusal path is part of the policy)"
+
+
+def test_pool_model_by_hand():
+    """The model itself, on cases small enough to follow on paper (so that the two sides cannot agree on nonsense)."""
+    from oracle.host import PoolModel
+    m = PoolModel(512 * MB)                          # 16 pages of 32 MB, range 4 GB, small segment 512 MB
+    assert m.alloc(0) is None
+    a = m.alloc(1000)                                # rounded to 1024, small segment, page 0 at slot 0
+    assert a == 0 and m.train_usage == 1024 and m.owner[0] == m.TRAIN and m.slot_page == {0: 0}
+    b = m.alloc(2 * MB)                              # the threshold itself goes to the large segment
+    assert b == 512 * MB and m.slot_page[16] == 1    # slot = 512 MB / 32 MB, next free page
+    c = m.alloc(2 * MB - 1024)                       # just below: small segment, right behind a
+    assert c == 1024
+    m.free(a)
+    d = m.alloc(512)                                 # best fit: the 1024-byte hole, not the tail of the page
+    assert d == 0
+    m.free(c)
+    m.free(d)                                        # a + c + the rest of the page merge into one free block
+    assert m.segs[0]["blocks"] == [[0, 32 * MB, False]]
+    assert m.empty_cache() == 32 * MB and m.owner[0] == m.FREE and 0 not in m.slot_page
+    assert m.empty_cache() == 0                      # b is live: its page stays
+    assert m.infer_claim(100) == 15 and m.alloc(64 * MB) is None and m.segs[1]["blocks"][-1][2] is False
+    assert m.infer_release(2) == 2 and m.owner[14:] == [m.FREE, m.FREE]
+    e = m.alloc(40 * MB)                             # grows over the refused request's free tail block: 514 .. 554 MB
+    assert e == b + 2 * MB and m.slot_page == {16: 1, 17: 14}   # slot 16 is live already, slot 17 takes the lowest free page
+    # lazy mode: the mapping stays, and the same range gets the same pages back without a map
+    z = PoolModel(128 * MB, lazy_unmap=True)
+    p = z.alloc(64 * MB)
+    z.free(p)
+    assert z.empty_cache() == 64 * MB and z.maps == 2 and z.unmaps == 0 and len(z.slot_page) == 2
+    assert z.alloc(64 * MB) == p and z.maps == 2 and z.revives == 2
+
+
 def _counters(L):
     c = (ctypes.c_uint64 * 6)()
     L.tch_pool_counters(0, c)

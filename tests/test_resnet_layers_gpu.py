@@ -175,7 +175,10 @@ def _layer_local(batch, depths=(3, 8, 36, 3), width=64, classes=1000, image=224,
 
     names = [r["name"] for r in eng.ctx.profile(plan.prog, 1)]
     kinds = {n.split("<")[0] for n in names}
-    for must in ("igemm2_kernel", "igemm3_kernel", "wgrad_kernel", "bn_fin_apply_kernel", "splitk_reduce_kernel"):
+    # the plan under test is the fused one: convolutions on the direct-to-LDS kernels, BatchNorm sums in their
+    # epilogues, the BatchNorm itself as one launch from the accumulators (or from per-tile sums, bn_acc off)
+    bn_kind = "bn_acc_apply_kernel" if eng.bn_acc else "bn_fin_apply_kernel"
+    for must in ("igemm2_kernel", "igemm3_kernel", "wgrad_kernel", bn_kind, "splitk_reduce_kernel"):
         assert must in kinds, (must, sorted(kinds))
     print(f"batch {batch}: {chk.count} tensors checked; worst per kind:", flush=True)
     for kind, (e, name) in sorted(chk.worst.items()):
