@@ -185,19 +185,21 @@ int tch_conv2d_dgrad_bnsums(tch_context* ctx, int dtype, const void* dy, const v
                             const float* bn_invstd, float* bn_partial, int add_stride);
 int tch_conv2d_dgrad_stat_rows(int dtype, int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
                                int tile_cfg);
-/* The same two with the sums ADDED to one pair of exact accumulators per channel instead of left per row tile:
- * bn_acc[c * 4 + {0,1}] collects the first sum, [c * 4 + {2,3}] the second, each as a pair of 64-bit integers
- * (units of 2^-24 and of 2^-66: integer additions, so the totals do not depend on the order the workgroups finish
- * in and a step stays bit-identical from run to run).  bn_acc must be zero before the call (tch_fill_zero); feed it
- * to tch_bn_fwd_train_acc / tch_bn_bwd_acc, which need no finalize launch and no pass over per-tile partials.
+/* The same two with the sums ADDED to exact accumulators instead of left per row tile.  bn_acc is
+ * [acc_copies][4][channels] 64-bit integers: planes 0 / 1 collect the first sum in units of 2^-24 / 2^-66, planes
+ * 2 / 3 the second (integer additions, so the totals do not depend on the order the workgroups finish in and a step
+ * stays bit-identical from run to run); row tile t adds to copy t % acc_copies (a power of two: additions to one
+ * address queue up behind each other, about 20 ns each, so layers with many row tiles want several copies).
+ * bn_acc must be zero before the call (tch_fill_zero); feed it, with the same acc_copies, to tch_bn_fwd_train_acc /
+ * tch_bn_bwd_acc, which need no finalize launch and no pass over per-tile partials.
  * What torch's conv2d -> batch_norm pairs (train/resnet152.py:22) need of each other, as two launches. */
 int tch_conv2d_fwd_bnacc(tch_context* ctx, int dtype, const void* x, const void* w, void* y, int N, int H, int W,
                          int C, int K, int R, int S, int stride, int pad, int tile_cfg, int c_logical,
-                         int64_t* bn_acc);
+                         int64_t* bn_acc, int acc_copies);
 int tch_conv2d_dgrad_bnacc(tch_context* ctx, int dtype, const void* dy, const void* wt, void* dx, const void* add,
                            const void* mask, int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
                            int tile_cfg, int c_logical, const void* bn_mask, const void* bn_x, const float* bn_mean,
-                           const float* bn_invstd, int64_t* bn_acc, int add_stride);
+                           const float* bn_invstd, int64_t* bn_acc, int acc_copies, int add_stride);
 /* Convolution + the whole front half of the BatchNorm next to it, in one call: the sums as above, and the
  * per-channel coefficients from them (by the workgroup that finishes a column tile last, or by a finalize launch
  * when there are more than 256 row tiles).  counters: >= ceil(channels / 64) ints, zero before the call, zero
@@ -254,7 +256,11 @@ int tch_conv2d_wgrad_group(tch_context* ctx, int dtype, int n, const int* shapes
  * part of the library's code object on every GPU it runs on.  The call allocates and frees nothing.  splits <= 0:
  * the library's choice, lowered to what the buffer holds; an explicit split count whose partials
  * (splits * (K*R*S*C + K) * 4 bytes) exceed the buffer is rejected with an error.  All calls on one GPU share the
- * buffer: calls that overlap on one GPU (two streams, two threads) race. */
+ * buffer.  Calls whose launches go to a stream at once are kept apart by the library: a call on another stream
+ * than the buffer's last user first waits (on the device, hipStreamWaitEvent) for that user's reduction.  Calls
+ * that are recorded into a program, held in a preemptible launch queue or captured into a HIP graph run later, in
+ * an order the library does not see: ONE such program / queue / graph may use the buffer at a time, and two that
+ * overlap on one GPU race. */
 int64_t tch_conv2d_wgrad_static_capacity_bytes(void);
 int tch_conv2d_wgrad_static(tch_context* ctx, int dtype, const void* x, const void* dy, float* dw, int splits,
                             int accumulate, int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
@@ -289,15 +295,15 @@ int tch_bn_bwd_partials(tch_context* ctx, int dtype, const void* g, const void* 
                         float* dbeta, int accumulate, const float* partial, int row_blocks, float* scratch);
 
 /* tch_bn_fwd_train_partials / tch_bn_bwd_partials from the accumulators of tch_conv2d_fwd_bnacc /
- * tch_conv2d_dgrad_bnacc (acc[C * 4] 64-bit words): coefficients and apply in ONE launch whatever the number of
- * rows.  C must be a multiple of eight 16-byte chunks (64 for bf16, 32 for fp32). */
+ * tch_conv2d_dgrad_bnacc (acc[acc_copies * 4 * C] 64-bit words): coefficients and apply in ONE launch whatever the
+ * number of rows.  C must be a multiple of eight 16-byte chunks (64 for bf16, 32 for fp32). */
 int tch_bn_fwd_train_acc(tch_context* ctx, int dtype, const void* x, void* y, const void* residual, int relu,
                          int64_t rows, int C, const float* gamma, const float* beta, float* running_mean,
                          float* running_var, float* save_mean, float* save_invstd, float momentum, float eps,
-                         const int64_t* acc);
+                         const int64_t* acc, int acc_copies);
 int tch_bn_bwd_acc(tch_context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int C,
                    const float* gamma, const float* save_mean, const float* save_invstd, float* dgamma, float* dbeta,
-                   int accumulate, const int64_t* acc);
+                   int accumulate, const int64_t* acc, int acc_copies);
 
 /* ---- pooling -------------------------------------------------------------------- */
 /* index[N,Ho,Wo,C] (int32) = h*W + w of the FIRST maximum in row-major window order (NaN wins). */

@@ -118,8 +118,18 @@ void tch_tag_model_end(int device);         /* main.pyx tag_model_end */
 int tch_tag_interm_memory(int device, void* ptr);      /* TagIntermMemory :322-341 */
 uint64_t tch_release_interm_memory(int device);        /* ReleaseIntermMemory :343-369 */
 void tch_untag_interm_memory(int device);              /* UntagIntermMemory */
+/* fn(arg) is called by FreeTrainLocals before the pool takes any lock and before it waits for the device: where a
+ * runtime that holds launches in queues of its own hands them over and waits for them, so that nothing submitted
+ * earlier can touch a page after it has changed hands.  (The launch queues of this library are drained by the
+ * pool itself.)  fn may call back into the pool.  NULL removes the hook.  Same role as the synchronisation the
+ * reference does before FreeTrainLocals (pytorch/torch_col/csrc/torch_allocator_plugin.cc:383-412). */
+void tch_pool_set_quiesce_hook(int device, void (*fn)(void*), void* arg);
 /* CPU model only: let the first n recorded events count as finished */
 void tch_pool_null_backend_complete_events(int device, uint64_t upto);
+/* CPU model only: the nth mapping from now is refused by the "driver" (0: none) */
+void tch_pool_null_backend_fail_map_in(int device, int nth);
+/* CPU model only: 0 = mapped slots that never got access rights, 1 = quiesce calls, 2 = access-right calls */
+int64_t tch_pool_null_backend_probe(int device, int what);
 
 /* ---- inference <-> training communicator (cython/main.pyx:346-528) ---- */
 typedef struct tch_ctrl_msg {

@@ -549,7 +549,8 @@ __global__ __launch_bounds__(256) void bn_fin_apply_kernel(FinApplyArgs p) {
 // of rows, which it walks like bn_apply_cols_kernel: a thread keeps one chunk column, four rows per trip.  The
 // workgroups of slab 0 also write the per-channel outputs (saved statistics, running statistics / dgamma, dbeta).
 struct AccApplyArgs {
-  const long long* acc;   // [C][2][kAccWords]: forward sum x, sum x^2; backward sum g, sum g * xhat
+  const long long* acc;   // [copies][4][C]: forward sum x, sum x^2; backward sum g, sum g * xhat
+  int acc_copies;
   int C;
   int64_t rows;
   const float* gamma;
@@ -582,8 +583,8 @@ __global__ __launch_bounds__(256) void bn_acc_apply_kernel(AccApplyArgs p) {
   const int c0 = blockIdx.x * COLS;
   if (tid < COLS) {
     const int c = c0 + tid;
-    const double s = acc_total(p.acc + static_cast<int64_t>(c) * 2 * kAccWords);
-    const double q = acc_total(p.acc + static_cast<int64_t>(c) * 2 * kAccWords + kAccWords);
+    double s, q;
+    acc_totals(p.acc, p.C, p.acc_copies, c, &s, &q);
     const double n = static_cast<double>(p.rows);
     const bool writer = blockIdx.y == 0;
     if (!BWD) {
@@ -1026,12 +1027,14 @@ int bn_bwd_partials(Context* ctx, int dtype, const void* g, const void* x, void*
 
 int bn_fwd_train_acc(Context* ctx, int dtype, const void* x, void* y, const void* residual, int relu, int64_t rows,
                      int C, const float* gamma, const float* beta, float* running_mean, float* running_var,
-                     float* save_mean, float* save_invstd, float momentum, float eps, const long long* acc) {
+                     float* save_mean, float* save_invstd, float momentum, float eps, const long long* acc,
+                     int acc_copies) {
   if (int rc = check_common(rows, C, dtype)) return rc;
   TCH_CHECK_ARG(x && y && gamma && beta && save_mean && save_invstd && acc, "bn_fwd_train_acc: null tensor");
   TCH_CHECK_ARG((running_mean == nullptr) == (running_var == nullptr), "bn_fwd_train_acc: running stats come in pairs");
   TCH_CHECK_ARG(C % (dtype == kBF16 ? 64 : 32) == 0, "bn_fwd_train_acc: channels must come in groups of eight 16-byte chunks");
-  AccApplyArgs a{acc, C, rows, gamma, beta, running_mean, running_var, save_mean, save_invstd, nullptr, nullptr,
+  TCH_CHECK_ARG(acc_copies >= 1 && (acc_copies & (acc_copies - 1)) == 0, "bn_fwd_train_acc: copies must be a power of two");
+  AccApplyArgs a{acc, acc_copies, C, rows, gamma, beta, running_mean, running_var, save_mean, save_invstd, nullptr, nullptr,
                  momentum, eps, 0, x, residual, y, relu, 0, 0};
   const double bytes = static_cast<double>(rows) * C * (dtype == kBF16 ? 2.0 : 4.0) * (residual ? 3.0 : 2.0);
   return dtype == kBF16 ? launch_acc_apply_t<bf16, 0>(ctx, a, "bn_acc_apply_kernel<bf16,fwd>", bytes)
@@ -1040,11 +1043,12 @@ int bn_fwd_train_acc(Context* ctx, int dtype, const void* x, void* y, const void
 
 int bn_bwd_acc(Context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int C,
                const float* gamma, const float* save_mean, const float* save_invstd, float* dgamma, float* dbeta,
-               int accumulate, const long long* acc) {
+               int accumulate, const long long* acc, int acc_copies) {
   if (int rc = check_common(rows, C, dtype)) return rc;
   TCH_CHECK_ARG(g && x && dx && gamma && save_mean && save_invstd && dgamma && dbeta && acc, "bn_bwd_acc: null tensor");
   TCH_CHECK_ARG(C % (dtype == kBF16 ? 64 : 32) == 0, "bn_bwd_acc: channels must come in groups of eight 16-byte chunks");
-  AccApplyArgs a{acc, C, rows, gamma, nullptr, nullptr, nullptr, const_cast<float*>(save_mean),
+  TCH_CHECK_ARG(acc_copies >= 1 && (acc_copies & (acc_copies - 1)) == 0, "bn_bwd_acc: copies must be a power of two");
+  AccApplyArgs a{acc, acc_copies, C, rows, gamma, nullptr, nullptr, nullptr, const_cast<float*>(save_mean),
                  const_cast<float*>(save_invstd), dgamma, dbeta, 0.f, 0.f, accumulate, g, x, dx, 0, 0, 0};
   const double bytes = static_cast<double>(rows) * C * (dtype == kBF16 ? 2.0 : 4.0) * 3.0;
   return dtype == kBF16 ? launch_acc_apply_t<bf16, 1>(ctx, a, "bn_acc_apply_kernel<bf16,bwd>", bytes)

@@ -258,20 +258,20 @@ int tch_bn_bwd_partials(tch_context* ctx, int dtype, const void* g, const void* 
 
 int tch_conv2d_fwd_bnacc(tch_context* ctx, int dtype, const void* x, const void* w, void* y, int N, int H, int W,
                          int Cc, int K, int R, int S, int stride, int pad, int tile_cfg, int c_logical,
-                         int64_t* bn_acc) {
+                         int64_t* bn_acc, int acc_copies) {
   if (!bn_acc) {
     set_error("tch_conv2d_fwd_bnacc: null accumulator buffer");
     return -22;
   }
   return conv2d_fwd(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad, c_logical), x, w, y, nullptr, nullptr, nullptr,
-                    0, tile_cfg, nullptr, nullptr, nullptr, 0, reinterpret_cast<long long*>(bn_acc));
+                    0, tile_cfg, nullptr, nullptr, nullptr, 0, reinterpret_cast<long long*>(bn_acc), acc_copies);
 }
 
 int tch_conv2d_dgrad_bnacc(tch_context* ctx, int dtype, const void* dy, const void* w, void* dx, const void* add,
                            const void* mask, int N, int H, int W, int Cc, int K, int R, int S, int stride, int pad,
                            int tile_cfg, int c_logical, const void* bn_mask, const void* bn_x, const float* bn_mean,
-                           const float* bn_invstd, int64_t* bn_acc, int add_stride) {
-  BnBwdSums bn{bn_mask, bn_x, bn_mean, bn_invstd, nullptr, nullptr, reinterpret_cast<long long*>(bn_acc)};
+                           const float* bn_invstd, int64_t* bn_acc, int acc_copies, int add_stride) {
+  BnBwdSums bn{bn_mask, bn_x, bn_mean, bn_invstd, nullptr, nullptr, reinterpret_cast<long long*>(bn_acc), acc_copies};
   return conv2d_dgrad(C(ctx), dtype, shape(N, H, W, Cc, K, R, S, stride, pad, c_logical), dy, w, dx, add, mask, tile_cfg,
                       &bn, add_stride);
 }
@@ -279,16 +279,16 @@ int tch_conv2d_dgrad_bnacc(tch_context* ctx, int dtype, const void* dy, const vo
 int tch_bn_fwd_train_acc(tch_context* ctx, int dtype, const void* x, void* y, const void* residual, int relu,
                          int64_t rows, int Cc, const float* gamma, const float* beta, float* running_mean,
                          float* running_var, float* save_mean, float* save_invstd, float momentum, float eps,
-                         const int64_t* acc) {
+                         const int64_t* acc, int acc_copies) {
   return bn_fwd_train_acc(C(ctx), dtype, x, y, residual, relu, rows, Cc, gamma, beta, running_mean, running_var, save_mean,
-                          save_invstd, momentum, eps, reinterpret_cast<const long long*>(acc));
+                          save_invstd, momentum, eps, reinterpret_cast<const long long*>(acc), acc_copies);
 }
 
 int tch_bn_bwd_acc(tch_context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int Cc,
                    const float* gamma, const float* save_mean, const float* save_invstd, float* dgamma, float* dbeta,
-                   int accumulate, const int64_t* acc) {
+                   int accumulate, const int64_t* acc, int acc_copies) {
   return bn_bwd_acc(C(ctx), dtype, g, x, dx, rows, Cc, gamma, save_mean, save_invstd, dgamma, dbeta, accumulate,
-                    reinterpret_cast<const long long*>(acc));
+                    reinterpret_cast<const long long*>(acc), acc_copies);
 }
 
 int tch_layernorm_fwd(tch_context* ctx, int dtype, const void* x, void* y, const float* gamma, const float* beta,

@@ -34,6 +34,7 @@
 #include <algorithm>
 #include <vector>
 
+#include "context.h"
 #include "ops.h"
 
 #include <mutex>
@@ -61,7 +62,8 @@ struct IgemmArgs {
   int relu_out;       // FWD: the stored output is max(0, .) of everything above
   float* dbias;       // WGRAD, optional: column sums of dy (the gradient of that bias), [splits][K] partials or final
   float* stats;       // optional: per (row tile, column) pair of sums over the stored output (see finish_tile)
-  long long* stat_acc;  // optional, instead of stats: the same pair added to exact accumulators, [column][2][kAccWords]
+  long long* stat_acc;  // optional, instead of stats: the same pair added to exact accumulators, [copies][4][columns]
+  int stat_acc_copies;  // power of two
   const void* bn_mask;      // DGRAD with stats, optional: the stored output is zeroed where bn_mask <= 0
   const void* bn_x;         // DGRAD with stats: input of the BatchNorm this gradient flows into, laid out like out
   const float* bn_mean;     // DGRAD with stats: that BatchNorm's saved batch mean / inverse std per column
@@ -460,8 +462,7 @@ __device__ inline void finish_tile(const IgemmArgs& p, f32x16_t (&acc)[TM][TN], 
       const int col = n0 + tid;
       if (col < p.gemm_n && p.stat_acc) {
         // every row tile adds to the same pair of accumulators: no per-tile partials, nothing to sum up later
-        acc_add(p.stat_acc + static_cast<int64_t>(col) * 2 * kAccWords, a);
-        acc_add(p.stat_acc + static_cast<int64_t>(col) * 2 * kAccWords + kAccWords, b);
+        acc_add2(p.stat_acc, p.gemm_n, p.stat_acc_copies, tile_m, col, a, b);
       } else if (col < p.gemm_n) {
         float2* dst = reinterpret_cast<float2*>(p.stats + (static_cast<int64_t>(tile_m) * p.gemm_n + col) * 2);
         if (p.fin_counters) {
@@ -1778,13 +1779,16 @@ void bind_finalize(IgemmArgs& a, const BnFinalize* f) {
 
 int conv2d_fwd(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* w, void* y, const void* add,
                const void* mask, const float* bias, int out_f32, int tile_cfg, float* bn_partial,
-               const BnFinalize* finalize, const float* scale, int relu_out, long long* bn_acc) {
+               const BnFinalize* finalize, const float* scale, int relu_out, long long* bn_acc, int bn_acc_copies) {
   IgemmArgs a{};
   if (int rc = fill_common(a, s, dtype)) return rc;
   TCH_CHECK_ARG(!((scale || relu_out) && (bn_partial || bn_acc)), "conv2d_fwd: statistics are taken of the plain convolution output");
   TCH_CHECK_ARG(!(bn_acc && (bn_partial || finalize || out_f32)),
                 "conv2d_fwd: accumulated statistics replace the per-tile ones and are taken of outputs stored in the compute type");
+  TCH_CHECK_ARG(!bn_acc || (bn_acc_copies >= 1 && (bn_acc_copies & (bn_acc_copies - 1)) == 0),
+                "conv2d_fwd: the number of accumulator copies must be a power of two");
   a.stat_acc = bn_acc;
+  a.stat_acc_copies = bn_acc_copies;
   a.scale = scale;
   a.relu_out = relu_out ? 1 : 0;
   TCH_CHECK_ARG(x && w && y, "conv2d_fwd: null tensor");
@@ -1854,8 +1858,11 @@ int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, co
                   "conv2d_dgrad: incomplete BatchNorm operands");
     TCH_CHECK_ARG(!bn->finalize || (bn->partial && check_finalize(bn->finalize, false)),
                   "conv2d_dgrad: incomplete BatchNorm finalize operands");
+    TCH_CHECK_ARG(!bn->acc || (bn->acc_copies >= 1 && (bn->acc_copies & (bn->acc_copies - 1)) == 0),
+                  "conv2d_dgrad: the number of accumulator copies must be a power of two");
     a.stats = bn->partial;
     a.stat_acc = bn->acc;
+    a.stat_acc_copies = bn->acc_copies;
     a.bn_mask = bn->mask;
     a.bn_x = bn->x;
     a.bn_mean = bn->mean;
@@ -2205,6 +2212,10 @@ namespace {
 constexpr int kScratchDevices = 16;
 std::mutex g_scratch_mu;
 float* g_scratch_ptr[kScratchDevices] = {};
+// who used the buffer last on each device: a call on another stream waits for that call's reduction first
+hipEvent_t g_scratch_done[kScratchDevices] = {};
+hipStream_t g_scratch_stream[kScratchDevices] = {};
+bool g_scratch_used[kScratchDevices] = {};
 
 // The device address of `scratch` on the current device (every GPU holds its own copy at its own address).
 int static_scratch(float** out) {
@@ -2218,9 +2229,23 @@ int static_scratch(float** out) {
     e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
     TCH_CHECK_ARG(e == hipSuccess && ptr, std::string("conv2d_wgrad_static: hipGetSymbolAddress: ") + hipGetErrorString(e));
     g_scratch_ptr[dev] = static_cast<float*>(ptr);
+    // set-up, once per device: the event that orders two streams' use of the buffer
+    e = hipEventCreateWithFlags(&g_scratch_done[dev], hipEventDisableTiming);
+    TCH_CHECK_ARG(e == hipSuccess, std::string("conv2d_wgrad_static: hipEventCreate: ") + hipGetErrorString(e));
   }
   *out = g_scratch_ptr[dev];
   return 0;
+}
+
+// Launches that go to a stream right now (not recorded into a program, not held in a launch queue, not captured
+// into a graph) are ordered here: the buffer's previous user on ANOTHER stream must have finished its reduction
+// before this call's partials overwrite it.  In the other three cases the launches run later, in an order only
+// the caller knows: there the caller keeps two users of the buffer apart.
+bool orders_itself(Context* ctx, hipStream_t stream) {
+  if (ctx->recording || ctx->queue) return false;
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &st) != hipSuccess || st != hipStreamCaptureStatusNone) return false;
+  return true;
 }
 }  // namespace
 
@@ -2246,7 +2271,20 @@ int conv2d_wgrad_static(Context* ctx, int dtype, const ConvShape& s, const void*
     if (int rc = static_scratch(&ptr)) return rc;
   // Every partial element the reduction reads is written by the split kernels of the same call first, so
   // what an earlier call left in the buffer never shows; two calls that overlap on one GPU would race on it.
-  return conv2d_wgrad(ctx, dtype, s, x, dy, dw, ptr, splits, accumulate, tile_cfg);
+  if (splits <= 1) return conv2d_wgrad(ctx, dtype, s, x, dy, dw, ptr, splits, accumulate, tile_cfg);
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  const hipStream_t stream = ctx->main_stream();
+  const bool ordered = orders_itself(ctx, stream);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);   // two host threads do not interleave their launches either
+  if (ordered && g_scratch_used[dev] && g_scratch_stream[dev] != stream)
+    (void)hipStreamWaitEvent(stream, g_scratch_done[dev], 0);
+  const int rc = conv2d_wgrad(ctx, dtype, s, x, dy, dw, ptr, splits, accumulate, tile_cfg);
+  if (ordered && rc == 0 && hipEventRecord(g_scratch_done[dev], stream) == hipSuccess) {
+    g_scratch_stream[dev] = stream;
+    g_scratch_used[dev] = true;
+  }
+  return rc;
 }
 
 }  // namespace tch

@@ -198,6 +198,31 @@ void tch_tag_model_end(int d) { if (auto p = pool(d)) p->tag_model_end(); }
 int tch_tag_interm_memory(int d, void* ptr) { auto p = pool(d); return p && p->tag_interm_memory(ptr) ? 1 : 0; }
 uint64_t tch_release_interm_memory(int d) { auto p = pool(d); return p ? p->release_interm_memory() : 0; }
 void tch_untag_interm_memory(int d) { if (auto p = pool(d)) p->untag_interm_memory(); }
+void tch_pool_set_quiesce_hook(int d, void (*fn)(void*), void* arg) {
+  auto p = pool(d);
+  if (!p) return;
+  if (fn)
+    p->set_quiesce_hook([fn, arg] { fn(arg); });
+  else
+    p->set_quiesce_hook(nullptr);
+}
+void tch_pool_null_backend_fail_map_in(int d, int nth) {
+  auto p = pool(d);
+  if (!p) return;
+  if (auto* nb = dynamic_cast<NullBackend*>(p->backend())) nb->fail_map_in = nth;
+}
+int64_t tch_pool_null_backend_probe(int d, int what) {
+  auto p = pool(d);
+  if (!p) return -1;
+  auto* nb = dynamic_cast<NullBackend*>(p->backend());
+  if (!nb) return -1;
+  switch (what) {
+    case 0: return static_cast<int64_t>(nb->no_access.size());
+    case 1: return nb->quiesces;
+    case 2: return nb->access_calls;
+    default: return -1;
+  }
+}
 void tch_pool_null_backend_complete_events(int d, uint64_t upto) {
   auto p = pool(d);
   if (!p) return;

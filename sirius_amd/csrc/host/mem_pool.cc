@@ -2,6 +2,7 @@
 
 #include <errno.h>
 #include <poll.h>
+#include <signal.h>
 #include <string.h>
 #include <sys/socket.h>
 #include <sys/un.h>
@@ -232,7 +233,7 @@ bool HbmPool::ensure_mapped(uint64_t off, size_t n, std::string* err) {
       ++n_revive_;
     }
   }
-  // count what is missing before touching anything, so a failure leaves no half-mapped block
+  // count what is missing before touching anything: running out of pages is found before the first driver call
   auto count_missing = [&] {
     int m = 0;
     for (uint64_t s = first; s <= last; ++s) m += slot_live_[s] ? 0 : 1;
@@ -245,6 +246,8 @@ bool HbmPool::ensure_mapped(uint64_t off, size_t n, std::string* err) {
   };
   int missing = count_missing();
   if (missing == 0) return true;
+  // a peer that died without detaching still owns its pages in the table: they come back first
+  if (count_free() < missing) sweep_dead_owners_table_locked();
   if (count_free() < missing) {
     // pages cached under free blocks elsewhere may cover the shortfall
     empty_cache_table_locked();
@@ -264,6 +267,15 @@ bool HbmPool::ensure_mapped(uint64_t off, size_t n, std::string* err) {
     run_len = 0;
     return ok;
   };
+  // A driver call that fails in the middle leaves the slots mapped so far live and owned by training (the caller
+  // frees the block, and the next request over them takes the fast path above): they must not be left without
+  // access rights, so the open run is closed before the failure is reported.
+  auto fail = [&]() -> bool {
+    std::string ignored;
+    if (run_len) (void)backend_->set_access(base_ + run_first * page_bytes_, run_len * page_bytes_, &ignored);
+    run_len = 0;
+    return false;
+  };
   for (uint64_t s = first; s <= last; ++s) {
     if (slot_live_[s]) {
       if (!close_run()) return false;
@@ -272,15 +284,15 @@ bool HbmPool::ensure_mapped(uint64_t off, size_t n, std::string* err) {
     if (slot_page_[s] >= 0) {
       // the page this slot used to hold now belongs to someone else: drop the stale mapping
       const int old = slot_page_[s];
-      if (!backend_->unmap(base_ + s * page_bytes_, 1, err)) return false;
+      if (!backend_->unmap(base_ + s * page_bytes_, 1, err)) return fail();
       ++n_unmap_;
       ++n_unmap_calls_;
       page_slot_[old] = -1;
       slot_page_[s] = -1;
     }
     const int page = take_free_page(err);
-    if (page < 0) return false;
-    if (!backend_->map(base_ + s * page_bytes_, page, err)) return false;
+    if (page < 0) return fail();
+    if (!backend_->map(base_ + s * page_bytes_, page, err)) return fail();
     set_owner(page, kOwnerTrain);
     slot_page_[s] = page;
     page_slot_[page] = static_cast<int64_t>(s);
@@ -533,8 +545,44 @@ size_t HbmPool::trim(size_t max_pages) {
 
 size_t HbmPool::empty_cache() {
   process_events();
+  // Before any lock: a launch that still waits in a software launch queue is on no stream yet, so the device
+  // synchronisation inside the locked part would not see it, and it may refer to a block freed since (frees are
+  // stream ordered).  Draining here also keeps the wait out of the cross-process table lock: the quiesce that
+  // follows under the locks finds an idle device.
+  std::function<void()> hook;
+  {
+    std::lock_guard<std::mutex> lock(mu_);
+    hook = quiesce_hook_;
+  }
+  if (hook) hook();
+  backend_->quiesce();
   std::lock_guard<std::mutex> lock(mu_);
   return empty_cache_locked();
+}
+
+void HbmPool::set_quiesce_hook(std::function<void()> fn) {
+  std::lock_guard<std::mutex> lock(mu_);
+  quiesce_hook_ = std::move(fn);
+}
+
+int HbmPool::sweep_dead_owners_table_locked() {
+  // The robust mutex covers a process that dies holding the table's lock; this covers one that dies holding
+  // PAGES (killed, crashed, or gone without detaching): its mappings went with it, the labels stay.  kill(pid, 0)
+  // says ESRCH for a pid that names no process.
+  const int32_t me = static_cast<int32_t>(getpid());
+  int freed = 0;
+  for (int i = 0; i < num_pages_; ++i) {
+    if (table_->owner[i] != kOwnerInfer) continue;
+    const int32_t pid = table_->owner_pid[i];
+    if (pid == me || pid <= 0) continue;
+    if (kill(static_cast<pid_t>(pid), 0) != 0 && errno == ESRCH) {
+      table_->owner[i] = kOwnerFree;
+      table_->owner_pid[i] = 0;
+      table_->changes++;
+      ++freed;
+    }
+  }
+  return freed;
 }
 
 PoolStats HbmPool::stats() {
@@ -547,6 +595,7 @@ PoolStats HbmPool::stats() {
   size_t train_pages = 0, infer_pages = 0, free_pages = 0;
   {
     ShmLock table_lock(&table_->mu);
+    sweep_dead_owners_table_locked();
     for (int i = 0; i < num_pages_; ++i) {
       const uint8_t o = table_->owner[i];
       train_pages += o == kOwnerTrain;

@@ -90,7 +90,10 @@ class PoolBackend {
   virtual bool set_access(uint64_t va, size_t bytes, std::string* err) = 0;    // read/write for the device
   virtual bool unmap(uint64_t va, int n_pages, std::string* err) = 0;          // a run of neighbouring slots
   virtual int export_fd(int page, std::string* err) = 0;                       // dma-buf descriptor, or -1
-  virtual void quiesce() {}  // wait until the device is idle (called once before a round of unmaps)
+  // Nothing that was submitted so far may still run or wait to run when pages change hands: drains the software
+  // launch queues (what waits there is on no stream yet, a device synchronisation alone does not see it), then
+  // waits until the device is idle.
+  virtual void quiesce() {}
   // event support for frees that must wait for other streams
   virtual uint64_t record_event(uint64_t stream) = 0;
   virtual bool event_done(uint64_t event) = 0;  // also destroys a finished event
@@ -100,14 +103,34 @@ class PoolBackend {
 // CPU model: no device, fake base address, events finish when the test says so.
 class NullBackend : public PoolBackend {
  public:
-  bool reserve(size_t, size_t, uint64_t* base, std::string*) override {
+  bool reserve(size_t, size_t page_bytes, uint64_t* base, std::string*) override {
     *base = 0x100000000000ull;
+    page_ = page_bytes;
     return true;
   }
   bool create_pages(int, std::string*) override { return true; }
-  bool map(uint64_t, int, std::string*) override { ++maps; return true; }
-  bool set_access(uint64_t, size_t, std::string*) override { ++access_calls; return true; }
-  bool unmap(uint64_t, int n, std::string*) override { unmaps += n; ++unmap_calls; return true; }
+  bool map(uint64_t va, int, std::string* err) override {
+    if (fail_map_in > 0 && --fail_map_in == 0) {
+      if (err) *err = "the CPU model of the pool was told to refuse this mapping";
+      return false;
+    }
+    ++maps;
+    no_access.insert(va);
+    return true;
+  }
+  bool set_access(uint64_t va, size_t bytes, std::string*) override {
+    ++access_calls;
+    for (auto it = no_access.lower_bound(va); it != no_access.end() && *it < va + bytes;) it = no_access.erase(it);
+    return true;
+  }
+  bool unmap(uint64_t va, int n, std::string*) override {
+    unmaps += n;
+    ++unmap_calls;
+    for (auto it = no_access.lower_bound(va); it != no_access.end() && *it < va + static_cast<uint64_t>(n) * page_;)
+      it = no_access.erase(it);
+    return true;
+  }
+  void quiesce() override { ++quiesces; }
   int export_fd(int, std::string* err) override {
     if (err) *err = "the CPU model of the pool has no device memory to export";
     return -1;
@@ -116,7 +139,10 @@ class NullBackend : public PoolBackend {
   bool event_done(uint64_t e) override { return e <= completed_upto; }
   bool has_device() const override { return false; }
   uint64_t next_event = 0, completed_upto = 0;
-  int64_t maps = 0, unmaps = 0, unmap_calls = 0, access_calls = 0;
+  int64_t maps = 0, unmaps = 0, unmap_calls = 0, access_calls = 0, quiesces = 0;
+  int fail_map_in = 0;            // test knob: the n-th map from now is refused (0: none)
+  std::set<uint64_t> no_access;   // mapped addresses that were never given access rights
+  uint64_t page_ = 0;
 };
 
 PoolBackend* make_hip_vmm_backend(int device);  // mem_pool_hip.cc
@@ -172,6 +198,9 @@ class HbmPool {
   size_t release_interm_memory();  // frees every tagged block still alive; returns bytes
   void untag_interm_memory();
   void register_oom_handler(std::function<void()> fn);
+  // Called by empty_cache() before it takes any lock, ahead of the backend's own quiesce: where a runtime that
+  // queues launches of its own drains them.  The hook may call back into the pool.
+  void set_quiesce_hook(std::function<void()> fn);
 
  private:
   struct Block {
@@ -222,6 +251,8 @@ class HbmPool {
   std::unordered_map<uint64_t, std::unordered_set<uint64_t>> stream_sets_;
   std::vector<Deferred> deferred_;
   std::vector<std::function<void()>> oom_handlers_;
+  std::function<void()> quiesce_hook_;
+  int sweep_dead_owners_table_locked();   // pages of processes that no longer exist go back to FREE; returns how many
   int listen_fd_ = -1;
   std::atomic<bool> serving_{false};
   std::unique_ptr<std::thread> server_;

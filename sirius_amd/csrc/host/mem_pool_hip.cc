@@ -13,6 +13,10 @@
 #include "mem_pool.h"
 
 namespace tch {
+int sync_all_streams();   // context.cc: every registered launch queue drained and finished on the device
+}
+
+namespace tch {
 namespace host {
 
 namespace {
@@ -92,6 +96,8 @@ class HipVmmBackend : public PoolBackend {
   }
 
   void quiesce() override {
+    // what still waits in a preemptible launch queue is on no stream yet: hand it over and wait for it first
+    (void)tch::sync_all_streams();
     (void)hipSetDevice(device_);
     (void)hipDeviceSynchronize();
   }

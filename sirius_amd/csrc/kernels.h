@@ -192,20 +192,37 @@ __device__ inline float wave_max(float v) {
 // 2^-66 (1.4e-20) of a contribution is dropped, |v| < 2^38 and up to 2^20 contributions fit; the total
 // hi * 2^-24 + lo * 2^-66 is the same whatever order the additions happened in, so the kernels that read it
 // are bit-identical from run to run.
-constexpr int kAccWords = 2;   // 64-bit words per accumulator
-__device__ inline void acc_add(long long* acc, float v) {
-  const double d = static_cast<double>(v);
-  const long long hi = static_cast<long long>(d * 16777216.0);
-  const double rest = d - static_cast<double>(hi) * (1.0 / 16777216.0);
-  const long long lo = __double2ll_rn(rest * 73786976294838206464.0);   // 2^66
-  atomicAdd(reinterpret_cast<unsigned long long*>(acc), static_cast<unsigned long long>(hi));
-  atomicAdd(reinterpret_cast<unsigned long long*>(acc) + 1, static_cast<unsigned long long>(lo));
+//
+// Layout of a set of accumulators for C channels and two sums per channel: copies x [4][C] 64-bit words -- the
+// planes hi(sum 0), lo(sum 0), hi(sum 1), lo(sum 1), so that the 64 lanes of one atomic instruction touch 512
+// contiguous bytes.  A device-scope add costs about 20 ns per earlier add to the SAME address that is still in
+// flight (measured: 1568 workgroups adding to one word take 20-35 us), so contributors are spread over `copies`
+// (a power of two) by their row-tile number and the reader adds the copies up -- integers again, any order.
+constexpr int kAccPlanes = 4;
+__device__ inline void acc_add2(long long* acc, int C, int copies, int contributor, int c, float v0, float v1) {
+  long long* base = acc + static_cast<int64_t>(contributor & (copies - 1)) * kAccPlanes * C + c;
+  const float v[2] = {v0, v1};
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const double d = static_cast<double>(v[j]);
+    const long long hi = static_cast<long long>(d * 16777216.0);
+    const double rest = d - static_cast<double>(hi) * (1.0 / 16777216.0);
+    const long long lo = __double2ll_rn(rest * 73786976294838206464.0);   // 2^66
+    atomicAdd(reinterpret_cast<unsigned long long*>(base + (2 * j) * C), static_cast<unsigned long long>(hi));
+    atomicAdd(reinterpret_cast<unsigned long long*>(base + (2 * j + 1) * C), static_cast<unsigned long long>(lo));
+  }
 }
 // read by a LATER launch than the ones that added (device-scope loads: they do not trust a cached copy)
-__device__ inline double acc_total(const long long* acc) {
-  const long long hi = __hip_atomic_load(acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  const long long lo = __hip_atomic_load(acc + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  return static_cast<double>(hi) * (1.0 / 16777216.0) + static_cast<double>(lo) * (1.0 / 73786976294838206464.0);
+__device__ inline void acc_totals(const long long* acc, int C, int copies, int c, double* t0, double* t1) {
+  long long w[kAccPlanes] = {0, 0, 0, 0};
+  for (int k = 0; k < copies; ++k) {
+#pragma unroll
+    for (int j = 0; j < kAccPlanes; ++j)
+      w[j] += __hip_atomic_load(acc + (static_cast<int64_t>(k) * kAccPlanes + j) * C + c, __ATOMIC_RELAXED,
+                                __HIP_MEMORY_SCOPE_AGENT);
+  }
+  *t0 = static_cast<double>(w[0]) * (1.0 / 16777216.0) + static_cast<double>(w[1]) * (1.0 / 73786976294838206464.0);
+  *t1 = static_cast<double>(w[2]) * (1.0 / 16777216.0) + static_cast<double>(w[3]) * (1.0 / 73786976294838206464.0);
 }
 
 // Workgroups are dealt round-robin to the 8 XCDs (each with a private L2).

@@ -41,7 +41,7 @@ struct BnFinalize {
 int conv2d_fwd(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* w, void* y, const void* add,
                const void* mask, const float* bias, int out_f32, int tile_cfg, float* bn_partial = nullptr,
                const BnFinalize* finalize = nullptr, const float* scale = nullptr, int relu_out = 0,
-               long long* bn_acc = nullptr);
+               long long* bn_acc = nullptr, int bn_acc_copies = 1);
 // rows of partial statistics conv2d_fwd writes for this shape and tiling (one per row tile)
 int conv2d_fwd_stat_rows(const ConvShape& s, int dtype, int tile_cfg);
 // The two reductions of a BatchNorm backward, taken in the epilogue of the data-gradient
@@ -53,7 +53,8 @@ struct BnBwdSums {
   const float* invstd;
   float* partial;       // [conv2d_dgrad_stat_rows][C][2]
   const BnFinalize* finalize;  // optional
-  long long* acc = nullptr;    // instead of partial: exact accumulators [C][2][2] the sums are added to
+  long long* acc = nullptr;    // instead of partial: exact accumulators [copies][4][C] the sums are added to
+  int acc_copies = 1;          // power of two: row tile t adds to copy t % copies
 };
 int conv2d_dgrad(Context* ctx, int dtype, const ConvShape& s, const void* dy, const void* w, void* dx,
                  const void* add, const void* mask, int tile_cfg, const BnBwdSums* bn = nullptr, int add_stride = 1);
@@ -120,13 +121,14 @@ int bn_bwd_partials(Context* ctx, int dtype, const void* g, const void* x, void*
                     float* dbeta, int accumulate, const float* partial, int row_blocks, float* scratch);
 // The same two, where the convolution next to the BatchNorm ADDED its sums to exact per-channel accumulators
 // (conv2d_fwd's bn_acc / BnBwdSums::acc) instead of leaving per-tile partials: one launch for any number of rows,
-// no finalize.  acc: [C][2][2] 64-bit words, zero before the convolution ran; C in groups of eight chunks.
+// no finalize.  acc: [copies][4][C] 64-bit words, zero before the convolution ran; C in groups of eight chunks.
 int bn_fwd_train_acc(Context* ctx, int dtype, const void* x, void* y, const void* residual, int relu, int64_t rows,
                      int C, const float* gamma, const float* beta, float* running_mean, float* running_var,
-                     float* save_mean, float* save_invstd, float momentum, float eps, const long long* acc);
+                     float* save_mean, float* save_invstd, float momentum, float eps, const long long* acc,
+                     int acc_copies);
 int bn_bwd_acc(Context* ctx, int dtype, const void* g, const void* x, void* dx, int64_t rows, int C,
                const float* gamma, const float* save_mean, const float* save_invstd, float* dgamma, float* dbeta,
-               int accumulate, const long long* acc);
+               int accumulate, const long long* acc, int acc_copies);
 
 // seq_ops.hip
 // Window order (Swin): rows = B * H * W pixels; a tensor flagged in `tensors` (1 = output, 2 = dy, 4 = the addend) is

@@ -222,20 +222,24 @@ def conv2d_fwd_bnstats(ctx, x, w, y, stride, pad, partial, tile_cfg=-1, c_logica
 
 
 def _check_acc(acc, C):
-    assert acc.dtype == torch.int64 and acc.numel() == 4 * C and acc.is_contiguous(), "accumulators: [C, 2, 2] int64"
+    """copies of an accumulator set [copies, 4, C] int64 (copies a power of two)."""
+    assert acc.dtype == torch.int64 and acc.is_contiguous() and acc.numel() % (4 * C) == 0, "accumulators: [copies, 4, C] int64"
+    copies = acc.numel() // (4 * C)
+    assert copies >= 1 and copies & (copies - 1) == 0, "accumulator copies: a power of two"
+    return copies
 
 
 def conv2d_fwd_bnacc(ctx, x, w, y, stride, pad, acc, tile_cfg=-1, c_logical=0):
     """conv2d_fwd that also ADDS the BatchNorm sums of y (sum, sum of squares per output channel) to the exact
-    accumulators `acc` ([K, 2, 2] int64, zero before the call): no per-tile partials, see bn_fwd_train_acc."""
+    accumulators `acc` ([copies, 4, K] int64, zero before the call): no per-tile partials, see bn_fwd_train_acc."""
     N, H, W, C = x.shape
     K, R, S, C2 = w.shape
     assert C == C2 and w.dtype == x.dtype == y.dtype
     Ho, Wo = conv_out_hw(H, W, R, S, stride, pad)
     assert tuple(y.shape) == (N, Ho, Wo, K)
-    _check_acc(acc, K)
+    copies = _check_acc(acc, K)
     check(lib().tch_conv2d_fwd_bnacc(ctx.handle, dtype_code(x), _p(x), _p(w), _p(y), N, H, W, C, K, R, S, stride, pad,
-                                     tile_cfg, c_logical, _p(acc)), "tch_conv2d_fwd_bnacc")
+                                     tile_cfg, c_logical, _p(acc), copies), "tch_conv2d_fwd_bnacc")
 
 
 def _check_addend(add, dx, add_stride):
@@ -295,7 +299,7 @@ def conv2d_dgrad_bnsums(ctx, dy, wt, dx, stride, pad, bn_x, bn_mean, bn_invstd, 
 
 def conv2d_dgrad_bnacc(ctx, dy, wt, dx, stride, pad, bn_x, bn_mean, bn_invstd, acc, bn_mask=None, add=None,
                        mask=None, tile_cfg=-1, c_logical=0, add_stride=1):
-    """conv2d_dgrad_bnsums with the two reductions ADDED to the exact accumulators `acc` ([C, 2, 2] int64, zero before
+    """conv2d_dgrad_bnsums with the two reductions ADDED to the exact accumulators `acc` ([copies, 4, C] int64, zero before
     the call) instead of left per row tile; see bn_bwd_acc."""
     N, H, W, C = dx.shape
     C2, R, S, K = wt.shape
@@ -308,10 +312,10 @@ def conv2d_dgrad_bnacc(ctx, dy, wt, dx, stride, pad, bn_x, bn_mean, bn_invstd, a
     _check_addend(add, dx, add_stride)
     assert bn_x is not None and bn_mean.numel() == C and bn_invstd.numel() == C
     assert bn_mean.dtype == bn_invstd.dtype == torch.float32
-    _check_acc(acc, C)
+    copies = _check_acc(acc, C)
     check(lib().tch_conv2d_dgrad_bnacc(ctx.handle, dtype_code(dy), _p(dy), _p(wt), _p(dx), _p(add), _p(mask),
                                        N, H, W, C, K, R, S, stride, pad, tile_cfg, c_logical, _p(bn_mask), _p(bn_x),
-                                       _p(bn_mean), _p(bn_invstd), _p(acc), add_stride), "tch_conv2d_dgrad_bnacc")
+                                       _p(bn_mean), _p(bn_invstd), _p(acc), copies, add_stride), "tch_conv2d_dgrad_bnacc")
 
 
 def conv2d_fwd_bn(ctx, x, w, y, stride, pad, partial, counters, gamma, beta, running_mean, running_var, save_mean,
@@ -524,10 +528,10 @@ def bn_fwd_train_acc(ctx, x, y, gamma, beta, running_mean, running_var, save_mea
     assert residual is None or (residual.shape == x.shape and residual.dtype == x.dtype)
     for t in (gamma, beta, save_mean, save_invstd):
         assert t.dtype == torch.float32 and t.numel() == C
-    _check_acc(acc, C)
+    copies = _check_acc(acc, C)
     check(lib().tch_bn_fwd_train_acc(ctx.handle, dtype_code(x), _p(x), _p(y), _p(residual), int(relu), rows, C,
                                      _p(gamma), _p(beta), _p(running_mean), _p(running_var), _p(save_mean),
-                                     _p(save_invstd), momentum, eps, _p(acc)), "tch_bn_fwd_train_acc")
+                                     _p(save_invstd), momentum, eps, _p(acc), copies), "tch_bn_fwd_train_acc")
 
 
 def bn_bwd_acc(ctx, g, x, dx, gamma, save_mean, save_invstd, dgamma, dbeta, acc, accumulate=False):
@@ -535,9 +539,9 @@ def bn_bwd_acc(ctx, g, x, dx, gamma, save_mean, save_invstd, dgamma, dbeta, acc,
     C = x.shape[-1]
     rows = x.numel() // C
     assert g.shape == x.shape == dx.shape and g.dtype == x.dtype == dx.dtype
-    _check_acc(acc, C)
+    copies = _check_acc(acc, C)
     check(lib().tch_bn_bwd_acc(ctx.handle, dtype_code(x), _p(g), _p(x), _p(dx), rows, C, _p(gamma), _p(save_mean),
-                               _p(save_invstd), _p(dgamma), _p(dbeta), int(accumulate), _p(acc)), "tch_bn_bwd_acc")
+                               _p(save_invstd), _p(dgamma), _p(dbeta), int(accumulate), _p(acc), copies), "tch_bn_bwd_acc")
 
 
 def bn_bwd(ctx, dy, x, dx, gamma, save_mean, save_invstd, dgamma, dbeta, workspace, relu_mask=None,

@@ -102,9 +102,14 @@ class ResNetEngine(EngineBase):
         # finalize launches go, but every convolution that adds to the accumulators gets 6-8 us LONGER: the
         # integer atomics of all row tiles of a channel meet at one address, a device-scope read-modify-write on
         # one address takes about 70 ns, and the kernel is not done before the last of them is (98 row tiles x 70 ns
-        # = 7 us at 14x14, 1568 tiles at 56x56).  Same bits in the loss as the per-tile form either way.
+        # = 7 us at 14x14, 1568 tiles at 56x56) -- that with one pair of words per channel, interleaved.  With the
+        # words laid out in planes (512 contiguous bytes per atomic instruction) and the row tiles spread over 4 / 8
+        # copies per channel the 14x14 and 7x7 stages alone cost 15.61 / 15.79 ms against 15.52 ms: still no gain,
+        # what the shorter BatchNorm launch wins the tail of the convolution loses.  Same bits in the loss as the
+        # per-tile form in every variant.
         self.bn_acc = (os.environ.get("TCH_BN_ACC", "0") != "0") if bn_acc is None else bool(bn_acc)
         self.bn_acc_max_rows = int(os.environ.get("TCH_BN_ACC_MAX_ROWS", "0"))
+        self.bn_acc_copies = int(os.environ.get("TCH_BN_ACC_COPIES", "4"))   # row tile t adds to copy t % copies
         # autotune: when a plan is built, time each distinct convolution shape with every tiling and
         # keep the fastest (forward and data gradient separately); off = the library's heuristic
         self.autotune = autotune
@@ -464,16 +469,17 @@ class ResNetEngine(EngineBase):
 
         # exact accumulators: [forward | backward][BatchNorm channel][2 sums][2 words]
         use_acc = self.bn_acc and self.fuse_bn_stats and not self.fuse_bn_finalize
-        acc_all = act(2 * nbn * 4, dtype=torch.int64) if use_acc else None
+        copies = self.bn_acc_copies
+        acc_all = act(2 * nbn * 4 * copies, dtype=torch.int64) if use_acc else None
         plan.bn_acc = acc_all
 
         def acc_of(name, backward, rows):
-            """The accumulators of one BatchNorm, or None where the layer keeps the per-tile form."""
+            """The accumulators of one BatchNorm ([copies, 4, channels]), or None where the layer keeps the per-tile form."""
             o, ch = self._bn_off[name]
             if not use_acc or ch % 64 or (self.bn_acc_max_rows and rows > self.bn_acc_max_rows):
                 return None
-            base = (nbn if backward else 0) + o
-            return acc_all[4 * base:4 * (base + ch)]
+            base = ((nbn if backward else 0) + o) * 4 * copies
+            return acc_all[base:base + 4 * copies * ch]
 
         def conv_bn_fwd(c, name, x, z, y, residual=None, relu=True):
             if not self.fuse_bn_stats:

@@ -97,6 +97,16 @@ class Batch(dict):
 
 
 # ----------------------------------------------------------------------------------------------------------------
+def _hand_over_queued_launches(stream):
+    """Wait until the preemptible launch queue of `stream` (if it has one) holds nothing that has not reached the
+    stream yet.  Does not wait for the GPU."""
+    import time
+    from .._lib import lib
+    handle = stream.cuda_stream
+    while lib().tch_GetXQueueSize(handle):
+        time.sleep(0)
+
+
 class _HostSamples:
     """`resident` rows per input tensor in pinned host memory; sample i of the dataset is row i % resident
     (the reference's ring repeat, dynamic_batch.py:449-454), so a small resident set stands for a dataset of
@@ -114,26 +124,37 @@ class _HostSamples:
         return torch.cat([torch.arange(lo, hi) for lo, hi in range_vec]) % self.resident if range_vec \
             else torch.empty(0, dtype=torch.long)
 
-    def _copy_run(self, first: int, n: int, device) -> dict:
+    def _copy_run(self, first: int, n: int, device, copy_stream=None) -> dict:
+        """Rows [first, first + n) on the device.  The tensors are always allocated on the CURRENT (training) stream,
+        which is the stream that will read them: the allocator then orders their reuse against that stream.  With a
+        copy stream the copy alone is issued there, and the copy stream is recorded as a second user."""
         out = {}
         for key, src in self.tensors.items():
             dst = torch.empty((n, *src.shape[1:]), dtype=src.dtype, device=device)
-            dst.copy_(src[first:first + n], non_blocking=True)
+            if copy_stream is None:
+                dst.copy_(src[first:first + n], non_blocking=True)
+            else:
+                with torch.cuda.stream(copy_stream):
+                    dst.copy_(src[first:first + n], non_blocking=True)
+                dst.record_stream(copy_stream)
             out[key] = dst
         return out
 
     def _prefetch(self, first: int, n: int, device):
         """Start copying rows [first, first + n) on the copy stream: the guess for the next micro-batch (the run
-        that follows this one, same size).  The copy stream first waits for the training stream, which is idle
-        here (a micro-batch ends with a synchronisation), so memory the allocator hands out again is not still in
-        use; the copy then runs beside the micro-batch that is launched next."""
+        that follows this one, same size).  The destination is allocated on the training stream; the copy stream
+        first waits for everything the training stream has been given -- including launches that still sit in the
+        stream's preemptible launch queue, which are handed over first (a stream wait only covers what is ON the
+        stream) -- so memory the allocator hands out again is not still in use by a cut or killed batch; the copy
+        then runs beside the micro-batch that is launched next."""
         if self._copy_stream is None:
             self._copy_stream = torch.cuda.Stream(device=device)
-        self._copy_stream.wait_stream(torch.cuda.current_stream(device))
-        with torch.cuda.stream(self._copy_stream):
-            tensors = self._copy_run(first, n, device)
-            done = torch.cuda.Event()
-            done.record(self._copy_stream)
+        train_stream = torch.cuda.current_stream(device)
+        _hand_over_queued_launches(train_stream)
+        self._copy_stream.wait_stream(train_stream)
+        tensors = self._copy_run(first, n, device, copy_stream=self._copy_stream)
+        done = torch.cuda.Event()
+        done.record(self._copy_stream)
         self._ahead = (first, n, tensors, done)
 
     def drop_prefetched(self):

@@ -12,10 +12,15 @@ from . import _C
 # (base MB, slope MB / sample), shared-tensor mode (train_adjuster.cc:647-698)
 MODEL_MEM_PARAM = {"resnet152": (1150, 85), "swin_b": (1700, 145), "swin_b_ddp": (2560, 140),
                    "gpt2": (2700, 490), "qwen": (9000, 600)}
-# this engine, bf16: flat fp32 params + grads + momentum + accumulated grads + bf16 shadow +
-# transposed bf16 filters = 60.2 M x 20 B = 1.15 GB base; activations and gradient scratch of a
-# batch-64 plan measure 6.50 GB = 97 MB per sample
-MODEL_MEM_PARAM_MI355X = {"resnet152": (1210, 97)}
+# This engine on MI355X, bf16 compute with fp32 master state, from pool readings (bytes held by torch before any
+# plan exists, and the bytes of the plans at three batch sizes; the plan grows linearly, its intercept is < 30 MB):
+#   resnet152  state 920 MB (+ 241 MB of accumulated gradients in colocate mode), plans 1109 / 2190 / 8673 MB at
+#              batch 8 / 16 / 64
+#   swin_b     state 1675 MB (+ 351 MB), plans 544 / 1083 / 4200 MB at batch 4 / 8 / 32
+#   gpt2       state 2375 MB (+ 498 MB); 256-token rows as train/gpt2.py:45 builds them: plans 1306 / 2585 / 10258 MB
+#              at batch 8 / 16 / 64 (1024-token rows: 640 MB per row)
+# base = state + accumulated gradients + the plan's intercept, slope = plan bytes per sample.
+MODEL_MEM_PARAM_MI355X = {"resnet152": (1190, 136), "swin_b": (2050, 131), "gpt2": (2900, 160)}
 
 
 class TrainAdjuster:

@@ -6,7 +6,6 @@ import glob
 import inspect
 import io
 import os
-from dataclasses import dataclass
 from typing import Optional
 
 from . import _C, dist
@@ -99,13 +98,24 @@ class MemoryPool:
         return _C.pool_trim(_C.get_train_rank())
 
 
-@dataclass
 class Event:
-    timestamp: int
-    name: str
-    loc: str
-    duration: float
-    tag: str
+    """One row of the training profile: a name, when it began (microseconds since the epoch), how long it took
+    (milliseconds, filled in when the span closes), where it was recorded and a free-form tag.  The field names are
+    the columns of the reference's train-profile.csv (pytorch/torch_col/util.py:100-110)."""
+    __slots__ = ("timestamp", "name", "loc", "duration", "tag")
+
+    def __init__(self, timestamp: int, name: str, loc: str = 'none', duration: float = 0, tag: str = ''):
+        self.timestamp, self.name, self.loc, self.duration, self.tag = timestamp, name, loc, duration, tag
+
+    def close(self, now_us: int):
+        """The span ends now: duration in milliseconds from the two microsecond stamps."""
+        self.duration = (now_us - self.timestamp) / 1000
+
+    def __eq__(self, other):
+        return isinstance(other, Event) and all(getattr(self, f) == getattr(other, f) for f in self.__slots__)
+
+    def __repr__(self) -> str:
+        return f'Event({self.timestamp}, {self.name!r}, {self.loc!r}, {self.duration}, {self.tag!r})'
 
     def __str__(self) -> str:
         return f'{self.timestamp} {self.loc} {self.name} {self.duration} {self.tag}'
@@ -114,10 +124,19 @@ class Event:
 _CSV_FIELDS = ("timestamp", "name", "loc", "duration", "tag", "rank")
 
 
+def _call_site(depth: int) -> str:
+    """file:line of the frame `depth` levels above the caller of this function."""
+    frame = inspect.currentframe()
+    for _ in range(depth + 1):
+        frame = frame.f_back
+    return f'{frame.f_code.co_filename}:{frame.f_lineno}'
+
+
 class EventManager:
-    """util.py:113-179.  Timestamps are kept in microseconds; the dump writes milliseconds with
-    two decimals, columns timestamp,name,loc,duration,tag,rank -- the schema of the reference's
-    train-profile.csv."""
+    """The training profile (pytorch/torch_col/util.py:113-179): a list of spans in the order they began.
+    Timestamps are kept in microseconds so that two events do not collide; durations are milliseconds; the dump
+    writes milliseconds with two decimals, columns timestamp,name,loc,duration,tag,rank -- the schema of the
+    reference's train-profile.csv."""
     _event_list: list = []
     _default_event_log_path = 'train-profile.csv'
 
@@ -130,28 +149,30 @@ class EventManager:
         cls._event_list = []
 
     @classmethod
+    def _open(cls, name: str, now_us: int, loc: str = 'none') -> Event:
+        span = Event(now_us, name, loc)
+        cls._event_list.append(span)
+        return span
+
+    @classmethod
     def record_event(cls, name: str, prev_event: Optional[Event] = None, record_loc: bool = False):
-        timestamp = _C.get_unix_timestamp_us()
-        if record_loc:
-            caller = inspect.getframeinfo(inspect.stack()[1][0])
-            loc = f'{caller.filename}:{caller.lineno}'
-        else:
-            loc = 'none'
+        """Close `prev_event` (if any) and open a span called `name` at the same instant; an empty name only closes.
+        Returns the new span, or None."""
+        now = _C.get_unix_timestamp_us()
         if prev_event is not None:
-            prev_event.duration = (timestamp - prev_event.timestamp) / 1000
-        if len(name) > 0:
-            event = Event(timestamp, name, loc, 0, '')
-            cls._event_list.append(event)
-            return event
+            prev_event.close(now)
+        if not name:
+            return None
+        return cls._open(name, now, _call_site(1) if record_loc else 'none')
 
     @classmethod
     @contextlib.contextmanager
     def record_duration_event(cls, name: str):
-        timestamp = _C.get_unix_timestamp_us()
-        event = Event(timestamp, name, 'none', 0, '')
-        cls._event_list.append(event)
-        yield event
-        event.duration = (_C.get_unix_timestamp_us() - timestamp) / 1000
+        """A span around the body of a `with` block.  A body that raises (a micro-batch that is cut short) leaves
+        its span open, duration 0, as in the reference."""
+        span = cls._open(name, _C.get_unix_timestamp_us())
+        yield span
+        span.close(_C.get_unix_timestamp_us())
 
     @classmethod
     def _to_csv(cls, header: bool) -> str:

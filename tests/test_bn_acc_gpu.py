@@ -2,7 +2,7 @@
 tch_conv2d_dgrad_bnacc -> tch_bn_fwd_train_acc / tch_bn_bwd_acc), through the C ABI.
 
 What is checked:
-* the accumulators hold the SUM OF THE PER-TILE PARTIALS the per-tile form of the same convolution leaves
+* the accumulators (their copies added up) hold the SUM OF THE PER-TILE PARTIALS the per-tile form of the same convolution leaves
   (same tiling, same fp32 partials), to the last bit the split keeps: compared with math.fsum of those
   partials (exact summation on the host), a bound of 2^-60 relative -- not with a second floating-point sum;
 * they are integers: two runs give the same words bit for bit, although the order the workgroups add in is
@@ -55,9 +55,10 @@ def close(got, ref, rtol, what):
 
 
 def decode(acc, C):
-    """[C, 2] python floats from the [C, 2, 2] int64 words: hi * 2^-24 + lo * 2^-66 (both exact in binary)."""
-    a = acc.cpu().reshape(C, 2, 2).tolist()
-    return [[hi * 2.0 ** -24 + lo * 2.0 ** -66 for hi, lo in ch] for ch in a]
+    """[C][2] python floats from the [copies, 4, C] int64 words: the copies are added up as integers, then
+    hi * 2^-24 + lo * 2^-66 (both exact in binary)."""
+    w = acc.cpu().reshape(-1, 4, C).sum(0).tolist()
+    return [[w[0][c] * 2.0 ** -24 + w[1][c] * 2.0 ** -66, w[2][c] * 2.0 ** -24 + w[3][c] * 2.0 ** -66] for c in range(C)]
 
 
 def exact_sums(partial, rb, C):
@@ -76,11 +77,11 @@ def assert_totals(acc, partial, rb, C, what):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", CASES)
-@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 5, 11, 13])
-def test_forward_statistics_through_accumulators(ctx, dtype, case, tile_cfg):
+@pytest.mark.parametrize("tile_cfg,copies", [(-1, 1), (0, 4), (1, 2), (2, 8), (5, 1), (11, 4), (13, 16)])
+def test_forward_statistics_through_accumulators(ctx, dtype, case, tile_cfg, copies):
     from sirius_amd import ops
     N, H, W, C, K, R, S, st, pad = case
-    print("case", case, dtype, tile_cfg, flush=True)
+    print("case", case, dtype, tile_cfg, copies, flush=True)
     g = _gen(31)
     x = rnd((N, H, W, C), dtype, g)
     w = rnd((K, R, S, C), dtype, g, (R * S * C) ** -0.5)
@@ -103,7 +104,7 @@ def test_forward_statistics_through_accumulators(ctx, dtype, case, tile_cfg):
     # accumulator form, twice
     accs = []
     for _ in range(2):
-        acc = torch.zeros(K * 4, dtype=torch.int64, device="cuda")
+        acc = torch.zeros(copies * 4 * K, dtype=torch.int64, device="cuda")
         z = torch.empty_like(z0)
         ops.conv2d_fwd_bnacc(ctx, xd, wd, z, st, pad, acc, tile_cfg=tile_cfg)
         y = torch.empty_like(z)
@@ -131,11 +132,11 @@ def test_forward_statistics_through_accumulators(ctx, dtype, case, tile_cfg):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("case", CASES)
-@pytest.mark.parametrize("tile_cfg", [-1, 0, 1, 2, 5, 11, 13])
-def test_backward_sums_through_accumulators(ctx, dtype, case, tile_cfg):
+@pytest.mark.parametrize("tile_cfg,copies", [(-1, 4), (0, 1), (1, 8), (2, 2), (5, 4), (11, 1), (13, 2)])
+def test_backward_sums_through_accumulators(ctx, dtype, case, tile_cfg, copies):
     from sirius_amd import ops
     N, H, W, C, K, R, S, st, pad = case
-    print("case", case, dtype, tile_cfg, flush=True)
+    print("case", case, dtype, tile_cfg, copies, flush=True)
     g = _gen(32)
     Ho, Wo = ops.conv_out_hw(H, W, R, S, st, pad)
     dy = rnd((N, Ho, Wo, K), dtype, g, 1e-3)     # gradients are small: the split must keep them
@@ -162,7 +163,7 @@ def test_backward_sums_through_accumulators(ctx, dtype, case, tile_cfg):
                         torch.empty(3 * C, device="cuda"))
     accs = []
     for _ in range(2):
-        acc = torch.zeros(C * 4, dtype=torch.int64, device="cuda")
+        acc = torch.zeros(copies * 4 * C, dtype=torch.int64, device="cuda")
         gx = torch.empty_like(gx0)
         ops.conv2d_dgrad_bnacc(ctx, dy.cuda(), wt, gx, st, pad, zd, mean.cuda(), invstd.cuda(), acc,
                                bn_mask=relu_out.cuda(), add=add.cuda(), tile_cfg=tile_cfg)
@@ -200,7 +201,7 @@ def test_many_row_tiles_and_large_values(ctx, dtype):
     gamma, beta = torch.rand(K, generator=g) + 0.5, torch.randn(K, generator=g) * 0.1
     xd, wd = x.cuda(), w.cuda()
     z = torch.empty((N, H, W, K), dtype=dtype, device="cuda")
-    acc = torch.zeros(K * 4, dtype=torch.int64, device="cuda")
+    acc = torch.zeros(8 * 4 * K, dtype=torch.int64, device="cuda")     # eight copies
     ops.conv2d_fwd_bnacc(ctx, xd, wd, z, 1, 0, acc, tile_cfg=2)
     y = torch.empty_like(z)
     rm, rv = torch.zeros(K, device="cuda"), torch.ones(K, device="cuda")
@@ -233,3 +234,5 @@ def test_accumulator_arguments_are_checked(ctx):
         ops.bn_fwd_train_acc(ctx, z, z.clone(), f, f, None, None, f.clone(), f.clone(), acc)
     with pytest.raises(AssertionError):
         ops.conv2d_fwd_bnacc(ctx, x, w, z, 1, 0, acc[:-1])
+    with pytest.raises(AssertionError):      # three copies: not a power of two
+        ops.conv2d_fwd_bnacc(ctx, x, w, z, 1, 0, torch.zeros(3 * 48 * 4, dtype=torch.int64, device="cuda"))

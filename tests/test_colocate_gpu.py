@@ -109,8 +109,8 @@ def test_pool_on_hip_vmm_follows_the_independent_model(clean_runtime, page_mb, l
     from pool_walk import walk_against_model
     torch.cuda.init()
     print("pool walk against the model, page", page_mb, "MB, lazy", lazy, flush=True)
-    ok, refused = walk_against_model(lib(), 7, 1024, page_mb, lazy, use_gpu=True, steps=300)
-    assert ok > 80 and refused > 0
+    ok, refused = walk_against_model(lib(), 7, 512, page_mb, lazy, use_gpu=True, steps=300)
+    assert ok > 60 and refused > 0, (ok, refused)
 
 
 class _RawBytes:

@@ -884,9 +884,11 @@ def test_pool_page_table_is_shared_with_another_process(fresh, tmp_path):
         child.stdin.write("\n")
         child.stdin.flush()
         child.wait(timeout=20)
-        # the in-process stand-in only ever gives back its own pages, not the dead peer's
+        # the in-process stand-in only ever gives back its own pages, not the dead peer's ...
         assert L.tch_pool_infer_release_pages(0, 8) == 0
-        assert L.tch_cuda_memory_pool_infer_usage(0) == 3 * 32 * MB
+        # ... but a process that no longer exists owns nothing: its three pages come back on the next look
+        assert L.tch_cuda_memory_pool_infer_usage(0) == 0
+        assert L.tch_cuda_memory_pool_num_free_pages(0) == 4
         L.tch_pool_free(a, 0, 0, None)
         L.tch_pool_free(b, 0, 0, None)
     finally:
@@ -896,6 +898,91 @@ def test_pool_page_table_is_shared_with_another_process(fresh, tmp_path):
     # a second pool of the same name can be made once the first is gone; a live one is not taken over
     assert L.tch_pool_init(0, 64 * MB, 0) == 0
     L.tch_pool_shutdown(0)
+
+
+_HOLDER_CHILD = r"""
+import ctypes, sys, time
+sys.path.insert(0, sys.argv[1])
+from sirius_amd._lib import lib
+L = lib()
+assert L.tch_pool_peer_attach(0) == 0, L.tch_host_last_error()
+got = (ctypes.c_int * 8)()
+print(L.tch_pool_peer_claim(0, 6, got), flush=True)
+time.sleep(600)                           # killed by the parent while it holds the pages
+"""
+
+
+def test_pool_takes_back_the_pages_of_a_killed_peer(fresh):
+    """An inference process that is killed (SIGKILL: no destructor, no detach) while it owns pages must not keep
+    them for good: training's next request that finds too few free pages looks for owners that no longer exist."""
+    L = fresh
+    assert L.tch_pool_init(0, 256 * MB, 0) == 0              # 8 pages
+    child = subprocess.Popen([sys.executable, "-c", _HOLDER_CHILD, ROOT], stdout=subprocess.PIPE, env=dict(os.environ),
+                             text=True)
+    try:
+        assert int(child.stdout.readline()) == 6
+        assert L.tch_cuda_memory_pool_num_free_pages(0) == 2
+        assert L.tch_pool_malloc(4 * 32 * MB, 0, None) is None          # the peer is alive: its pages are its own
+        assert b"out of pool memory" in L.tch_host_last_error()
+        child.kill()
+        child.wait(timeout=20)
+        a = L.tch_pool_malloc(4 * 32 * MB, 0, None)                     # the request itself takes them back
+        assert a, L.tch_host_last_error()
+        assert L.tch_cuda_memory_pool_infer_usage(0) == 0 and L.tch_cuda_memory_pool_num_free_pages(0) == 4
+        L.tch_pool_free(a, 0, 0, None)
+    finally:
+        if child.poll() is None:
+            child.kill()
+        L.tch_pool_shutdown(0)
+
+
+def test_pool_quiesces_before_pages_change_hands_and_outside_its_locks(fresh):
+    """FreeTrainLocals first lets a runtime drain what it has queued (the hook), then waits for the device, and only
+    then takes its locks: the hook below calls back into the pool (it would deadlock under the locks) and sees the
+    pages still in training's hands."""
+    L = fresh
+    assert L.tch_pool_init(0, 256 * MB, 0) == 0
+    seen = []
+    HOOK = ctypes.CFUNCTYPE(None, ctypes.c_void_p)
+
+    def hook(_):
+        seen.append((L.tch_cuda_memory_pool_train_all_usage(0), L.tch_pool_null_backend_probe(0, 1)))
+    cb = HOOK(hook)
+    try:
+        a = L.tch_pool_malloc(64 * MB, 0, None)
+        L.tch_pool_free(a, 0, 0, None)
+        L.tch_pool_set_quiesce_hook(0, ctypes.cast(cb, ctypes.c_void_p), None)
+        assert L.tch_cuda_memory_pool_free_train_local(0) == 64 * MB
+        assert seen == [(64 * MB, 0)], seen            # called once, before the backend's quiesce, pages still mapped
+        assert L.tch_pool_null_backend_probe(0, 1) >= 1
+        L.tch_pool_set_quiesce_hook(0, None, None)
+        b = L.tch_pool_malloc(32 * MB, 0, None)
+        L.tch_pool_free(b, 0, 0, None)
+        L.tch_cuda_memory_pool_free_train_local(0)
+        assert len(seen) == 1
+    finally:
+        L.tch_pool_shutdown(0)
+
+
+def test_pool_mapping_failure_leaves_no_slot_without_access(fresh):
+    """The driver refuses the second of three mappings: the request fails, the slot mapped before the failure
+    keeps its page AND has access rights, and the next request over it works."""
+    L = fresh
+    assert L.tch_pool_init(0, 256 * MB, 0) == 0
+    try:
+        L.tch_pool_null_backend_fail_map_in(0, 2)
+        assert L.tch_pool_malloc(96 * MB, 0, None) is None
+        assert b"refuse" in L.tch_host_last_error()
+        assert L.tch_pool_null_backend_probe(0, 0) == 0, "a mapped slot was left without access rights"
+        assert L.tch_cuda_memory_pool_train_usage(0) == 0
+        assert L.tch_cuda_memory_pool_train_all_usage(0) == 32 * MB     # the first slot stays mapped under a free block
+        a = L.tch_pool_malloc(96 * MB, 0, None)
+        assert a and L.tch_pool_null_backend_probe(0, 0) == 0
+        assert L.tch_cuda_memory_pool_train_all_usage(0) == 96 * MB
+        L.tch_pool_free(a, 0, 0, None)
+        assert L.tch_cuda_memory_pool_free_train_local(0) == 96 * MB
+    finally:
+        L.tch_pool_shutdown(0)
 
 
 def test_pool_cross_stream_free_is_deferred(fresh):

@@ -148,7 +148,10 @@ def test_suspended_queue_holds_launches_back_and_keeps_their_order():
         xsched.unregister_stream(stream)
 
 
-def test_training_interleaved_with_preempting_requests_is_bit_identical():
+def _interleave(gpt_cfg, batch, seq, steps, rate_per_s, min_served, lr=1e-3):
+    """`steps` GPT-2 training steps alone, then the same steps beside batch-1 ResNet-152 requests that arrive as a
+    seeded Poisson process and preempt between training's launches: same weights, same loss, same logits."""
+    from sirius_amd.gpt2 import GPT2Engine
     from sirius_amd.resnet import ResNetEngine
     from sirius_amd.serve import ColocatedInference, poisson_arrivals
     from sirius_amd.torch_col import xsched
@@ -156,10 +159,12 @@ def test_training_interleaved_with_preempting_requests_is_bit_identical():
     xsched.register_stream(train_stream, False)
     server = None
     try:
-        sd = G.make_state_dict(GPT_CFG["vocab"], GPT_CFG["n_pos"], GPT_CFG["n_embd"], GPT_CFG["n_layer"], seed=1)
+        sd = G.make_state_dict(gpt_cfg["vocab"], gpt_cfg["n_pos"], gpt_cfg["n_embd"], gpt_cfg["n_layer"], seed=1)
         g = torch.Generator().manual_seed(5)
-        batches = [torch.randint(0, GPT_CFG["vocab"], (4, 256), generator=g).cuda() for _ in range(40)]
-        eng = _gpt2(train_stream, sd)
+        distinct = [torch.randint(0, gpt_cfg["vocab"], (batch, seq), generator=g).cuda() for _ in range(min(steps, 8))]
+        batches = [distinct[i % len(distinct)] for i in range(steps)]
+        eng = GPT2Engine(seq_len=seq, dtype=torch.bfloat16, lr=lr, weight_decay=0.01, stream=train_stream, **gpt_cfg)
+        eng.load_state_dict(sd)
         _train(eng, batches[:2])                     # plans built, kernels loaded
         eng.load_state_dict(sd)
         t0 = time.perf_counter()
@@ -168,8 +173,9 @@ def test_training_interleaved_with_preempting_requests_is_bit_identical():
 
         infer = ResNetEngine(dtype=torch.bfloat16, stream=infer_stream)
         infer.init_kaiming(seed=9)
-        # requests every 2.5 ms on average: several per training step, for the whole run and beyond
-        server = ColocatedInference(infer, poisson_arrivals(400.0, 4000, seed=7), batch=1, preempt=True)
+        # arrivals for the whole run and beyond
+        server = ColocatedInference(infer, poisson_arrivals(rate_per_s, int(rate_per_s * (4 * alone_s + 2)) + 50, seed=7),
+                                    batch=1, preempt=True)
         server.warm_up()
         idle_logits = server.engine.eval_plan(1).logits.clone()   # what the warm-up requests left: the same image
 
@@ -182,10 +188,10 @@ def test_training_interleaved_with_preempting_requests_is_bit_identical():
         served_during = len(server.latencies_ms)
         server.stop()
         s = server.summary()
-        print(f"{len(batches)} GPT-2 steps alone {alone_s * 1e3:.1f} ms, with {served_during} preempting ResNet-152 "
-              f"requests {mixed_s * 1e3:.1f} ms; request latency p50 {s['p50_ms']:.2f} ms p99 {s['p99_ms']:.2f} ms",
-              flush=True)
-        assert served_during >= 20, "requests were served while training ran"
+        print(f"{steps} GPT-2 steps ({batch} x {seq}) alone {alone_s * 1e3:.1f} ms, with {served_during} preempting "
+              f"ResNet-152 requests at {rate_per_s:g}/s {mixed_s * 1e3:.1f} ms; request latency p50 {s['p50_ms']:.2f} ms "
+              f"p99 {s['p99_ms']:.2f} ms", flush=True)
+        assert served_during >= min_served, "requests were served while training ran"
         assert torch.equal(mixed_params, alone_params), "training's weights do not depend on the interleaving"
         assert mixed_loss == alone_loss
         assert torch.equal(server.last_logits, idle_logits), "a request's logits do not depend on the interleaving"
@@ -197,3 +203,16 @@ def test_training_interleaved_with_preempting_requests_is_bit_identical():
         xsched.resume_all_streams()
         torch.cuda.synchronize()
         xsched.unregister_stream(train_stream)
+
+
+def test_training_interleaved_with_preempting_requests_is_bit_identical():
+    """A small GPT-2 (4 x 256 tokens) under heavy preemption: a request every 2.5 ms on average, several per step."""
+    _interleave(GPT_CFG, 4, 256, 40, 400.0, 20)
+
+
+def test_baseline_config5_gpt2_small_8x1024_beside_50_requests_per_second():
+    """BASELINE configs[4] as stated: GPT-2 small (12 layers, 768 channels, 12 heads, vocabulary 50 257), 8 x 1024
+    tokens, AdamW, beside batch-1 ResNet-152 forward requests arriving Poisson at 50 per second that preempt between
+    training kernels; 80 steps (about a second of training, about fifty requests)."""
+    cfg = dict(vocab=50257, n_pos=1024, n_embd=768, n_layer=12, n_head=12)
+    _interleave(cfg, 8, 1024, 80, 50.0, 20, lr=1e-4)

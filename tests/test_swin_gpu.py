@@ -476,3 +476,88 @@ def test_swin_b_real_config_loss_and_every_gradient(dtype, tol):
     for e, k in errs:
         assert torch.isfinite(grads[k]).all(), k
         assert e <= (table_tol if k.endswith("relative_position_bias_table") else tol), (k, e)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-3), (torch.bfloat16, 2e-2)])
+def test_swin_b_real_config_three_adamw_steps(dtype, tol):
+    """BASELINE configs[3]: Swin-B at its real configuration, AdamW lr 1e-3 wd 0.05, THREE steps at batch 3 on three
+    different batches, against oracle/swin.py: loss and every gradient of every step (oracle at the engine's weights),
+    the optimizer's update of every step (torch.optim.AdamW on the engine's gradients), the free-running loss of
+    every step.  Why in three parts: tests/adamw_steps.py."""
+    import os
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    from adamw_steps import bf16_matrix_view, run_adamw_steps
+    cfg = S.config()
+    sd = S.make_state_dict(cfg, seed=7)
+    gsd = _gen(70)
+    for k, v in sd.items():
+        if v.dim() == 1 or k.endswith("relative_position_bias_table"):
+            v.add_(torch.randn(v.shape, generator=gsd) * 0.05)
+    if dtype == torch.bfloat16:
+        sd = {k: (v.to(torch.bfloat16).float() if v.is_floating_point() else v) for k, v in sd.items()}
+    g = _gen(9)
+    batches = [(torch.randn(3, 3, 224, 224, generator=g), torch.randint(0, 1000, (3,), generator=g)) for _ in range(3)]
+    free_losses, _ = S.train_steps(sd, batches, cfg, lr=1e-3, weight_decay=0.05)
+    eng = _engine(cfg, dtype, lr=1e-3, weight_decay=0.05)
+    eng.load_state_dict(sd)
+
+    def fb(batch):
+        _, cut = eng.forward_backward(batch[0].cuda(), batch[1].cuda())
+        assert not cut
+
+    table_tols = {}
+
+    def grad_tol(name, w, batch, grads_ref):
+        if dtype != torch.bfloat16 or not name.endswith("relative_position_bias_table"):
+            return tol
+        key = id(batch)
+        if key not in table_tols:     # what PyTorch's own CPU bf16-autocast step makes of the bias tables, once per step
+            table_tols[key] = max(tol, _cpu_bf16_table_error(w, batch[0], batch[1], cfg, grads_ref))
+        return table_tols[key]
+
+    run_adamw_steps(eng, batches, fb, lambda w, b: S.loss_and_grads(w, b[0], b[1], cfg), free_losses, lr=1e-3,
+                    weight_decay=0.05, tol=tol, grad_tol=grad_tol, tag=f"Swin-B {dtype}",
+                    oracle_view=bf16_matrix_view(("relative_position_bias_table",)) if dtype == torch.bfloat16 else None)
+
+
+def test_swin_b_batch32_properties():
+    """BASELINE configs[3] at its own batch size (32 images, bf16): too large for the CPU oracle, so the step is held
+    to what does not depend on size.  Swin has no batch statistics: the logits of an image do not depend on the other
+    images of the batch, so images 0-2 must give, inside the batch of 32, the logits they give in the batch of 3 that
+    the oracle covers (bit for bit: same kernels, same rows -- asserted at 1e-3 of the largest logit to allow for a
+    different tiling of a larger product); everything is finite; two runs from the same state are bit-identical in
+    loss, every gradient and every updated weight."""
+    cfg = S.config()
+    sd = S.make_state_dict(cfg, seed=7)
+    sd = {k: (v.to(torch.bfloat16).float() if v.is_floating_point() else v) for k, v in sd.items()}
+    g = _gen(8)
+    x = torch.randn(32, 3, 224, 224, generator=g)
+    y = torch.randint(0, 1000, (32,), generator=g)
+    runs = []
+    for _ in range(2):
+        eng = _engine(cfg, torch.bfloat16, lr=1e-3, weight_decay=0.05)
+        eng.load_state_dict(sd)
+        p, cut = eng.forward_backward(x.cuda(), y.cuda())
+        assert not cut
+        logits = p.logits.float().cpu().clone()
+        loss, grads = eng.last_loss(), {k: v.clone() for k, v in eng.grads_dict().items()}
+        eng.optimizer_step()
+        runs.append((loss, logits, grads, eng.state_dict()))
+    (l0, lg0, g0, w0), (l1, lg1, g1, w1) = runs
+    assert l0 == l1 and torch.equal(lg0, lg1)
+    for k in g0:
+        assert torch.isfinite(g0[k]).all(), k
+        assert torch.equal(g0[k], g1[k]), k
+    for k in w0:
+        assert torch.equal(w0[k], w1[k]), k
+    assert torch.isfinite(lg0).all() and l0 == l0 and abs(l0) < 50
+    # images 0-2 alone (the batch the oracle test covers)
+    small = _engine(cfg, torch.bfloat16)
+    small.load_state_dict(sd)
+    p3, cut = small.forward_backward(x[:3].cuda(), y[:3].cuda())
+    assert not cut
+    lg3 = p3.logits.float().cpu()
+    assert _rel(lg0[:3], lg3) <= 1e-3, _rel(lg0[:3], lg3)
+    assert _rel(lg3, S.forward(sd, x[:3], cfg)) <= 2e-2
+    print("Swin-B batch 32: loss", l0, "logits of images 0-2 vs batch of 3:", _rel(lg0[:3], lg3), flush=True)

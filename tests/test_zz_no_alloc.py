@@ -76,3 +76,40 @@ def test_static_scratch_weight_gradient_equals_the_workspace_one(ctx, dtype):
     ops.conv2d_wgrad_static(ctx, xb, dyb, dwb, 1, 1)
     ctx.synchronize()
     assert float(dwb.abs().max()) == 0.0
+
+
+def test_two_streams_share_the_static_buffer_in_order():
+    """Calls that launch at once on two different streams of one GPU: the library makes the second wait for the first
+    one's reduction (on the device, no host synchronisation in between), so both results equal the workspace form bit
+    for bit although the two problems overwrite each other's partials."""
+    from sirius_amd import ops
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    c1, c2 = ops.Context(s1), ops.Context(s2)
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(5)
+    xa = torch.randn(16, 28, 28, 128, generator=g).to(dtype).cuda()
+    dya = torch.randn(16, 28, 28, 128, generator=g).to(dtype).cuda()
+    xb = torch.randn(8, 14, 14, 256, generator=g).to(dtype).cuda()
+    dyb = torch.randn(8, 14, 14, 512, generator=g).to(dtype).cuda()
+    main = ops.Context(torch.cuda.current_stream())
+    code = ops.dtype_code(xa)
+    wsa = torch.empty(ops.conv2d_wgrad_workspace_bytes(code, 128, 3, 3, 128, 12) // 4, device="cuda")
+    wsb = torch.empty(ops.conv2d_wgrad_workspace_bytes(code, 512, 1, 1, 256, 6) // 4, device="cuda")
+    refa = torch.zeros(128, 3, 3, 128, device="cuda")
+    refb = torch.zeros(512, 1, 1, 256, device="cuda")
+    ops.conv2d_wgrad(main, xa, dya, refa, 1, 1, workspace=wsa, splits=12)
+    ops.conv2d_wgrad(main, xb, dyb, refb, 1, 0, workspace=wsb, splits=6)
+    main.synchronize()
+    torch.cuda.synchronize()
+    gota = [torch.empty_like(refa) for _ in range(6)]
+    gotb = [torch.empty_like(refb) for _ in range(6)]
+    print("two streams, 6 rounds", flush=True)
+    for i in range(6):          # no host synchronisation inside the loop
+        ops.conv2d_wgrad_static(c1, xa, dya, gota[i], 1, 1, splits=12)
+        ops.conv2d_wgrad_static(c2, xb, dyb, gotb[i], 1, 0, splits=6)
+    c1.synchronize()
+    c2.synchronize()
+    torch.cuda.synchronize()
+    for i in range(6):
+        assert torch.equal(gota[i], refa), f"round {i}: the 3x3 problem on stream 1"
+        assert torch.equal(gotb[i], refb), f"round {i}: the 1x1 problem on stream 2"
