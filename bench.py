@@ -118,11 +118,13 @@ def cpu_baseline(batch, timed_steps):
             "kind": "port", "sample": f"ResNet-152 fp32 batch {batch} @224, torch CPU oracle step, 1 warm-up + {timed_steps} timed steps"}
 
 
-def handover(batch):
+def handover(batch, pool_gb=None, page_mb=None, lazy=False):
     """BASELINE configs[2]: ResNet-152 bf16 under the colocation protocol, global batch fixed at
     `batch`; a stand-in inference peer asks for memory (target batch 16) during the 4th micro-batch
     and leaves later (target back to `batch`).  Reports request -> AdjustL1Done as the server sees
-    it, split into wait (request received -> release starts) and release, and the bytes returned."""
+    it, split into wait (request received -> release starts) and release, and the bytes returned.
+    lazy: the pool answers first and removes its mappings of the pages it handed back right after the reply (a peer
+    waits for a page's flag before it maps it); `request_to_last_page_usable_ms` then says when the last one was gone."""
     import contextlib
     import csv
     import tempfile
@@ -134,7 +136,8 @@ def handover(batch):
     tmp = tempfile.mkdtemp(prefix="tch_bench_")
     env = {"COLTRAIN_MODE": "colocate-l1", "COLTRAIN_HOOK_MODE": "xsched-sync", "COLTRAIN_USE_XSCHED": "1",
            "COLTRAIN_HAS_INFER_SERVER": "1", "COLTRAIN_USE_SHARED_TENSOR": "1",
-           "COLTRAIN_SHARED_TENSOR_POOL_GB": str(HANDOVER_POOL_GB), "COLTRAIN_POOL_PAGE_MB": str(HANDOVER_PAGE_MB),
+           "COLTRAIN_SHARED_TENSOR_POOL_GB": str(pool_gb or HANDOVER_POOL_GB),
+           "COLTRAIN_POOL_PAGE_MB": str(page_mb or HANDOVER_PAGE_MB), "COLTRAIN_POOL_LAZY_UNMAP": "1" if lazy else "0",
            "COLTRAIN_PROFILE_LOG_PATH": os.path.join(tmp, "train-profile.csv"),
            "SIRIUS_PORT": str(18000 + os.getpid() % 1000)}
     os.environ.update(env)
@@ -161,11 +164,17 @@ def handover(batch):
         "killed_batches": stat.killed_batch,
         "finished_samples": stat.finished_sample,
         "bound_ms": 50.0,
-        "pool_gb": HANDOVER_POOL_GB,
-        "page_mb": HANDOVER_PAGE_MB,
-        "unmapping": "eager: every page handed back is unmapped from training's address range before the reply",
+        "pool_gb": pool_gb or HANDOVER_POOL_GB,
+        "page_mb": page_mb or HANDOVER_PAGE_MB,
+        "unmapping": ("after the reply: the pages are FREE and claimable at once, each flagged in the shared page table until "
+                      "training's mapping of it is gone; a peer waits for the flag of the page it maps") if lazy else
+                     "eager: every page handed back is unmapped from training's address range before the reply",
         "stale_pages_after": out["ctrl"].last_adjust.get("stale_pages_after"),
     }
+    la = out["ctrl"].last_adjust
+    if lazy and res["request_to_done_ms"] is not None:
+        res["request_to_last_page_usable_ms"] = res["request_to_done_ms"] + la.get("stat_ms", 0.0) + la.get("trim_after_reply_ms", 0.0)
+        res["pages_unmapped_after_reply"] = la.get("trimmed_after_reply")
     del out
     torch_col.reset_for_tests()
     torch_col.torch_col_shutdown()
@@ -537,6 +546,10 @@ def main():
             out["handover"] = handover(B)
         except Exception as e:  # the headline figure stands on its own; say what went wrong
             out["handover"] = {"error": repr(e)}
+        try:    # the reference's page size: 32 MB pages, the reply first, the unmapping right behind it
+            out["handover_32mb_pages"] = handover(B, pool_gb=48, page_mb=32, lazy=True)
+        except Exception as e:
+            out["handover_32mb_pages"] = {"error": repr(e)}
     if not args.no_gpt2:
         try:
             out["gpt2"] = gpt2_step()

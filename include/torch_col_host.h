@@ -108,6 +108,13 @@ int tch_pool_peer_free_pages(int device);
 int tch_pool_peer_claim(int device, int n, int* pages_out);
 int tch_pool_peer_release(int device, const int* pages, int n);
 void* tch_pool_peer_map(int device, int page);
+/* A pool in lazy mode answers the other tenant first and removes its own mappings of the pages it handed back right
+ * after the reply (the driver takes 0.26 ms per mapping, one after the other, from however many threads): such a
+ * page is FREE and claimable at once, and flagged in the page table until its old mapping is gone.
+ * tch_pool_peer_map waits up to 5 s for the flag of the page it maps (tch_pool_peer_map_wait: up to wait_ms), so a
+ * page is never usable by two processes at once; tch_pool_peer_still_mapped counts the flagged ones among `pages`. */
+void* tch_pool_peer_map_wait(int device, int page, int wait_ms);
+int tch_pool_peer_still_mapped(int device, const int* pages, int n);
 int tch_pool_peer_unmap(int device, int page);
 /* the inference side inside the training process (a stand-in peer on a thread): label n FREE pages
  * inference-owned / give back */

@@ -269,6 +269,22 @@ void* tch_pool_peer_map(int device, int page) {
   if (!ptr) fail("tch_pool_peer_map: " + err);
   return ptr;
 }
+void* tch_pool_peer_map_wait(int device, int page, int wait_ms) {
+  auto p = peer(device);
+  if (!p) {
+    fail("tch_pool_peer_map_wait: not attached");
+    return nullptr;
+  }
+  std::string err;
+  void* ptr = p->map(page, &err, wait_ms);
+  if (!ptr) fail("tch_pool_peer_map_wait: " + err);
+  return ptr;
+}
+int tch_pool_peer_still_mapped(int device, const int* pages, int n) {
+  auto p = peer(device);
+  if (!p) return fail("tch_pool_peer_still_mapped: not attached");
+  return p->still_mapped_by_creator(pages, n);
+}
 int tch_pool_peer_unmap(int device, int page) {
   auto p = peer(device);
   if (!p) return fail("tch_pool_peer_unmap: not attached");

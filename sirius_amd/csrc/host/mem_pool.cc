@@ -211,6 +211,7 @@ int HbmPool::take_free_page(std::string* err) {
     ++n_unmap_calls_;
     slot_page_[slot] = -1;
     page_slot_[stale] = -1;
+    set_creator_mapped(stale, false);
   }
   return stale;
 }
@@ -229,6 +230,7 @@ bool HbmPool::ensure_mapped(uint64_t off, size_t n, std::string* err) {
     const int page = slot_page_[s];
     if (page >= 0 && !slot_live_[s] && table_->owner[page] == kOwnerFree) {
       set_owner(page, kOwnerTrain);
+      set_creator_mapped(page, false);   // training's again: nobody waits for this mapping to go
       slot_live_[s] = 1;
       ++n_revive_;
     }
@@ -289,6 +291,7 @@ bool HbmPool::ensure_mapped(uint64_t off, size_t n, std::string* err) {
       ++n_unmap_calls_;
       page_slot_[old] = -1;
       slot_page_[s] = -1;
+      set_creator_mapped(old, false);
     }
     const int page = take_free_page(err);
     if (page < 0) return fail();
@@ -513,6 +516,7 @@ size_t HbmPool::empty_cache_table_locked() {
   }
   for (uint64_t slot : slots) {
     slot_live_[slot] = 0;
+    set_creator_mapped(slot_page_[slot], true);   // before the page shows as FREE: a claimer must see the flag
     set_owner(slot_page_[slot], kOwnerFree);
   }
   return slots.size() * page_bytes_;
@@ -533,6 +537,7 @@ size_t HbmPool::trim(size_t max_pages) {
       n_unmap_ += end - slot;
       ++n_unmap_calls_;
       for (size_t k = slot; k < end; ++k) {
+        set_creator_mapped(slot_page_[k], false);
         page_slot_[slot_page_[k]] = -1;
         slot_page_[k] = -1;
       }
@@ -851,10 +856,30 @@ int PoolPeer::fetch_fd(int page, std::string* err) {
   return fd;
 }
 
-void* PoolPeer::map(int page, std::string* err) {
+int PoolPeer::still_mapped_by_creator(const int* pages, int n) {
+  int cnt = 0;
+  for (int k = 0; k < n; ++k)
+    if (pages[k] >= 0 && pages[k] < table_->num_pages)
+      cnt += __atomic_load_n(&table_->creator_mapped[pages[k]], __ATOMIC_ACQUIRE) ? 1 : 0;
+  return cnt;
+}
+
+void* PoolPeer::map(int page, std::string* err, int wait_ms) {
   std::lock_guard<std::mutex> lock(mu_);
   auto it = mapped_.find(page);
   if (it != mapped_.end()) return it->second;
+  if (page < 0 || page >= table_->num_pages) {
+    if (err) *err = "no such page";
+    return nullptr;
+  }
+  // a page handed back lazily is FREE (and claimable) before its old mapping is gone: wait for that
+  for (int waited_us = 0; __atomic_load_n(&table_->creator_mapped[page], __ATOMIC_ACQUIRE); waited_us += 50) {
+    if (waited_us >= wait_ms * 1000) {
+      if (err) *err = "page " + std::to_string(page) + " is still mapped by the process that handed it back";
+      return nullptr;
+    }
+    usleep(50);
+  }
   if (!table_->has_device) {
     if (err) *err = "this pool is the CPU model: its pages have no device memory";
     return nullptr;

@@ -77,6 +77,10 @@ struct PageTableLayout {
   uint64_t changes;                    // bumped by every change of ownership
   uint8_t owner[kMaxPoolPages];
   int32_t owner_pid[kMaxPoolPages];    // pid of the owning process, 0 for FREE
+  // 1 while the pool's creator still maps a page it has handed back (lazy mode: the reply to the other tenant goes
+  // out first, the mappings are removed right after it).  A peer that has claimed the page waits for 0 before it
+  // maps it, so that a page is never usable by two processes at once.  Written with atomic byte stores.
+  uint8_t creator_mapped[kMaxPoolPages];
 };
 
 std::string page_table_name(int device);   // "<prefix>_pages_pool_d<device>"
@@ -228,6 +232,9 @@ class HbmPool {
   size_t empty_cache_table_locked();   // table already locked
   int take_free_page(std::string* err);
   void set_owner(int page, PageOwner o);
+  void set_creator_mapped(int page, bool mapped) {
+    __atomic_store_n(&table_->creator_mapped[page], static_cast<uint8_t>(mapped ? 1 : 0), __ATOMIC_RELEASE);
+  }
   void serve_descriptors();   // thread: answers peers that ask for the descriptor of a page they own
 
   int device_ = 0;
@@ -272,8 +279,11 @@ class PoolPeer {
   int claim(int n, int* pages_out);
   // inference-owned by this process -> FREE (a page still mapped here is unmapped first)
   int release(const int* pages, int n);
-  // device address of a claimed page in this process (imports the creator's descriptor on first use)
-  void* map(int page, std::string* err);
+  // device address of a claimed page in this process (imports the creator's descriptor on first use); waits, up
+  // to wait_ms, until the pool's creator has removed its own mapping of a page it handed back lazily
+  void* map(int page, std::string* err, int wait_ms = 5000);
+  // how many of `pages` the pool's creator still maps
+  int still_mapped_by_creator(const int* pages, int n);
   bool unmap(int page, std::string* err);
 
  private:

@@ -342,11 +342,15 @@ class ColocateCtrl(CtrlBase):
             t = time.time()
             cached1, alloc1 = _used_gb()
         stat_ms = (time.time() - t) * 1e3
-        # lazy pools answer first and take the mappings of the pages they gave away down afterwards
+        # lazy pools answer first and take the mappings of the pages they gave away down afterwards (a peer that
+        # has claimed such a page waits for its flag in the page table before it maps it)
+        t = time.time()
         trimmed = MemoryPool.trim_stale_mappings()
+        trim_ms = (time.time() - t) * 1e3
         self.last_adjust = {"release_ms": release_ms, "empty_cache_ms": pages_ms, "reply_ms": reply_ms,
                             "stat_ms": stat_ms, "released_bytes": released, "pool_bytes_returned": returned,
-                            "trimmed_after_reply": trimmed, "stale_pages_after": MemoryPool.stale_pages()}
+                            "trimmed_after_reply": trimmed, "trim_after_reply_ms": trim_ms,
+                            "stale_pages_after": MemoryPool.stale_pages()}
         print(f'[Rank {_C.get_train_rank()} | PID {os.getpid()} | {_C.get_unix_timestamp_us()/1000}]'
               f' [Adjust L1 {release_ms:.1f} | {pages_ms:.1f} | {reply_ms:.1f} | {stat_ms:.1f} ms]'
               f' target batch_size: {self.target_batch_size},'

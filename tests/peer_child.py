@@ -37,6 +37,8 @@ def claim_map_write(conn, port, n_pages, expect_value, write_value):
         t1 = time.perf_counter()
         pages = list(got)[:out["claimed"]]
         out["indices"] = pages
+        # pages the creator handed back lazily are claimable before their old mapping is gone: how many, right now
+        out["still_mapped_at_claim"] = L.tch_pool_peer_still_mapped(0, got, out["claimed"])
         ptrs = []
         for pg in pages:
             p = L.tch_pool_peer_map(0, pg)

@@ -192,20 +192,23 @@ def _peer(port, n_pages, expect_word, write_word):
     return proc, here
 
 
-@pytest.mark.parametrize("page_mb", [32, 128])
-def test_returned_pages_are_claimed_mapped_and_written_by_another_process(clean_runtime, page_mb):
+@pytest.mark.parametrize("page_mb,lazy", [(32, 0), (128, 0), (32, 1)])
+def test_returned_pages_are_claimed_mapped_and_written_by_another_process(clean_runtime, page_mb, lazy):
     """The handover gives memory to somebody: the trainer fills a block in pool memory, frees it and hands the
     pages back (unmapped here: nothing stale); a SEPARATE process attaches to the page table, claims those pages,
     maps them from the creator's dma-buf descriptors, finds the trainer's bytes in them (same physical memory),
     overwrites them and gives them back; the trainer maps the pages again and finds the other process's bytes.
     The creator hands a descriptor only to the page's owner; while the peer holds the pages the trainer cannot
-    grow over them."""
+    grow over them.
+    lazy: the pages are handed back still mapped in the trainer (the reply to the other tenant goes out first); the
+    peer claims them at once, sees them flagged, and its map calls wait until the trainer -- 0.3 s later here -- has
+    removed its mappings: the peer's map time says so."""
     tc = clean_runtime
     L = lib()
     port = int(os.environ["SIRIUS_PORT"])
     page = page_mb * MB
     n = 8
-    assert L.tch_pool_init_ex(0, 16 * page, 1, page, 0) == 0, L.tch_host_last_error()
+    assert L.tch_pool_init_ex(0, 16 * page, 1, page, lazy) == 0, L.tch_host_last_error()
     proc = None
     try:
         t = tc.pool_empty((n * page // 4,), torch.float32, device=0)
@@ -216,12 +219,27 @@ def test_returned_pages_are_claimed_mapped_and_written_by_another_process(clean_
         assert L.tch_cuda_memory_pool_free_train_local(0) == n * page
         c = (ctypes.c_uint64 * 6)()
         L.tch_pool_counters(0, c)
-        assert int(c[3]) == n and int(c[5]) == 0, "handed-back pages are unmapped, none is left stale"
-        assert L.tch_pool_unmap_calls(0) == 1, "one driver call for the run"
+        if lazy:
+            assert int(c[3]) == 0 and int(c[5]) == n, "lazy: relabelled, every mapping still in place"
+        else:
+            assert int(c[3]) == n and int(c[5]) == 0, "handed-back pages are unmapped, none is left stale"
+            assert L.tch_pool_unmap_calls(0) == 1, "one driver call for the run"
         proc, conn = _peer(port, n, 1234.5, 4321.25)
+        if lazy:
+            # let the peer claim and block in its first map, then take the mappings down
+            deadline = time.time() + 120
+            while L.tch_cuda_memory_pool_infer_usage(0) != n * page and time.time() < deadline:
+                time.sleep(0.01)
+            assert L.tch_cuda_memory_pool_infer_usage(0) == n * page, "the peer did not claim"
+            time.sleep(0.3)
+            assert not conn.poll(0), "the peer must still be waiting for the trainer's mappings to go"
+            assert L.tch_pool_trim(0, 1 << 30) == n
         assert conn.poll(120), "the peer process did not answer"
         first = conn.recv()
         assert "error" not in first, first
+        assert first["still_mapped_at_claim"] == (n if lazy else 0)
+        if lazy:
+            assert first["map_ms"] >= 250.0, first["map_ms"]
         print(f"peer pid {first['pid']} (this process {os.getpid()}): attach+claim {first['attach_claim_ms']:.2f} ms, "
               f"map {n} pages of {page_mb} MB {first['map_ms']:.2f} ms, read+fill {first['rw_ms']:.2f} ms", flush=True)
         assert first["pid"] != os.getpid()
@@ -490,7 +508,10 @@ def test_dynamic_compute_unit_partition_under_the_colocation_protocol(clean_runt
     assert tc.GetXQueueSizeAllStreams() == 0
 
 
-@pytest.mark.parametrize("page_mb,pool_gb,lazy,bound_ms", [(128, 256, 0, 50.0), (32, 48, 0, None), (32, 48, 1, 50.0)])
+# the driver takes 0.26 ms per mapping it removes, one after the other from however many host threads (measured:
+# 256 mappings of 32 MB take 66.5 ms from 1, 2, 4 or 8 threads): "driver" = that cost for the pages handed back,
+# with 25 % and 12 ms of slack, the only bound real unmapping of that many mappings can be held to
+@pytest.mark.parametrize("page_mb,pool_gb,lazy,bound_ms", [(128, 256, 0, 50.0), (32, 48, 0, "driver"), (32, 48, 1, 50.0)])
 def test_handover_64_16_64_on_the_real_resnet152(clean_runtime, monkeypatch, tmp_path, page_mb, pool_gb, lazy, bound_ms):
     """BASELINE configs[2] at its real size: ResNet-152 (depths 3/8/36/3, 224 x 224, 1000 classes) in bf16 from the
     shared pool, micro-batches of 64; the peer asks for memory at micro-batch 10 (target 16) and leaves at
@@ -499,10 +520,12 @@ def test_handover_64_16_64_on_the_real_resnet152(clean_runtime, monkeypatch, tmp
     the handover does inside it: killing the batch, waiting for the launches in flight, freeing the plan, and
     (eager mode) removing the mapping of every page that is handed back.
 
-    The driver takes 0.26 ms per mapping it removes, whatever the mapping's size.  With 128 MB pages in a pool of
-    256 GB (the part has 288) the bound of 50 ms holds with the unmapping included.  With the reference's 32 MB
-    pages it does not at this size (284 mappings: about 70 ms; the test prints the figure and asserts the
-    rest); it holds again when the mappings are left in place and removed after the reply (lazy mode)."""
+    The driver takes 0.26 ms per mapping it removes, whatever the mapping's size and however many threads ask.  With
+    128 MB pages in a pool of 256 GB (the part has 288) the bound of 50 ms holds with the unmapping included.  With the
+    reference's 32 MB pages and the unmapping inside the reply it cannot at this size (284 mappings: about 74 ms):
+    that row is held to the driver's own cost.  With the reply first and the unmapping right behind it (lazy mode:
+    the pages are claimable at once, a peer waits for a page's flag before it maps it) request -> done is held to
+    50 ms again, and request -> last page usable to the driver's cost."""
     tc = clean_runtime
     from sirius_amd.train import resnet152 as script
     env = {"COLTRAIN_MODE": "colocate-l1", "COLTRAIN_HOOK_MODE": "xsched-sync", "COLTRAIN_USE_XSCHED": "1",
@@ -526,8 +549,15 @@ def test_handover_64_16_64_on_the_real_resnet152(clean_runtime, monkeypatch, tmp
     print(f"ResNet-152 64->16, {page_mb} MB pages, pool {pool_gb} GB, {'lazy' if lazy else 'eager'} unmapping: "
           f"request -> done {latency_ms:.2f} ms, {ctrl.last_adjust}", flush=True)
     assert latency_ms >= 0
-    if bound_ms is not None:
-        assert latency_ms < bound_ms
+    pages = ctrl.last_adjust["pool_bytes_returned"] // (page_mb * MB)
+    driver_ms = 1.25 * 0.26 * pages + 12.0
+    assert latency_ms < (driver_ms if bound_ms == "driver" else bound_ms), (latency_ms, bound_ms, driver_ms)
+    if lazy:
+        usable_ms = latency_ms + ctrl.last_adjust["stat_ms"] + ctrl.last_adjust["trim_after_reply_ms"]
+        print(f"  request -> last page usable by the peer {usable_ms:.2f} ms ({ctrl.last_adjust['trimmed_after_reply']} "
+              f"mappings removed after the reply in {ctrl.last_adjust['trim_after_reply_ms']:.2f} ms)", flush=True)
+        assert ctrl.last_adjust["trimmed_after_reply"] == pages and ctrl.last_adjust["stale_pages_after"] == 0
+        assert usable_ms < driver_ms
     assert ctrl.last_adjust["released_bytes"] > 4 << 30, "a batch-64 plan holds more than 6 GB of activations"
     assert ctrl.last_adjust["pool_bytes_returned"] > 4 << 30
     if not lazy:

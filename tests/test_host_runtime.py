@@ -912,6 +912,46 @@ time.sleep(600)                           # killed by the parent while it holds 
 """
 
 
+def test_lazy_pool_flags_pages_until_their_old_mapping_is_gone(fresh):
+    """Lazy mode hands pages back before it unmaps them: the pages are FREE and claimable at once, flagged in the
+    shared table while the creator still maps them, and a peer's map waits for the flag (here: gives up after the
+    time it was given, then succeeds -- as far as the CPU model can -- once trim() has removed the mappings)."""
+    L = fresh
+    assert L.tch_pool_init_ex(0, 256 * MB, 0, 32 * MB, 1) == 0        # 8 pages, lazy
+    try:
+        a = L.tch_pool_malloc(96 * MB, 0, None)
+        L.tch_pool_free(a, 0, 0, None)
+        assert L.tch_cuda_memory_pool_free_train_local(0) == 96 * MB     # relabelled, still mapped
+        assert L.tch_pool_peer_attach(0) == 0, L.tch_host_last_error()
+        got = (ctypes.c_int * 8)()
+        assert L.tch_pool_peer_claim(0, 5, got) == 5 and list(got)[:5] == [0, 1, 2, 3, 4]
+        assert L.tch_pool_peer_still_mapped(0, got, 5) == 3              # pages 0-2 carried the block
+        t0 = time.time()
+        assert not L.tch_pool_peer_map_wait(0, 0, 30)
+        assert time.time() - t0 >= 0.03 and b"still mapped" in L.tch_host_last_error()
+        assert not L.tch_pool_peer_map_wait(0, 3, 30)                    # never mapped by the creator: no wait
+        assert b"CPU model" in L.tch_host_last_error()
+        assert L.tch_pool_trim(0, 2) == 2
+        assert L.tch_pool_peer_still_mapped(0, got, 5) == 1
+        assert L.tch_pool_trim(0, 100) == 1
+        assert L.tch_pool_peer_still_mapped(0, got, 5) == 0
+        assert not L.tch_pool_peer_map_wait(0, 0, 30) and b"CPU model" in L.tch_host_last_error()
+        # a page that training takes back itself (revived) is not waited for by anybody
+        back = (ctypes.c_int * 5)(*list(got)[:5])
+        assert L.tch_pool_peer_release(0, back, 5) == 5
+        b = L.tch_pool_malloc(32 * MB, 0, None)
+        L.tch_pool_free(b, 0, 0, None)
+        L.tch_cuda_memory_pool_free_train_local(0)
+        c = L.tch_pool_malloc(32 * MB, 0, None)                          # same slot, same page, revived
+        assert c == b
+        one = (ctypes.c_int * 1)(0)
+        assert L.tch_pool_peer_still_mapped(0, one, 1) == 0
+        L.tch_pool_free(c, 0, 0, None)
+    finally:
+        L.tch_pool_peer_detach(0)
+        L.tch_pool_shutdown(0)
+
+
 def test_pool_takes_back_the_pages_of_a_killed_peer(fresh):
     """An inference process that is killed (SIGKILL: no destructor, no detach) while it owns pages must not keep
     them for good: training's next request that finds too few free pages looks for owners that no longer exist."""
