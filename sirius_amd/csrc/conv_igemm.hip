@@ -444,20 +444,25 @@ __device__ inline void finish_tile(const IgemmArgs& p, f32x16_t (&acc)[TM][TN], 
   if (want_stats) {
     // threads tid, tid + CH, tid + 2 CH, ... hold partial sums of the same E columns
     __syncthreads();
-    float* red = stage;  // [ROWS][CH][2E]
+    // [2][E] planes of one float per thread, plane stride NT + 8 floats: the 64 lanes of a store hit 64 consecutive
+    // banks, and the 64 lanes of a load below (8 values of e x 8 values of cc) land 8 banks apart per plane: neither
+    // has a bank conflict (a [thread][2E] layout made every store a 16-way one)
+    constexpr int PS = NT + 8;
+    static_assert(2 * E * PS * 4 <= WM * 32 * (BN + kStagePad) * 4, "the sums fit the staging tile");
+    float* red = stage;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-      red[(tid * 2 * E) + e] = st_sum[e];
-      red[(tid * 2 * E) + E + e] = st_sq[e];
+      red[e * PS + tid] = st_sum[e];
+      red[(E + e) * PS + tid] = st_sq[e];
     }
     __syncthreads();
     if (tid < BN) {
       const int cc = tid / E, e = tid - cc * E;
       float a = 0.f, b = 0.f;
 #pragma unroll 4
-      for (int r = 0; r < ROWS; ++r) {
-        a += red[((r * CH + cc) * 2 * E) + e];
-        b += red[((r * CH + cc) * 2 * E) + E + e];
+      for (int r = 0; r < ROWS; ++r) {   // thread r * CH + cc holds row group r of chunk column cc
+        a += red[e * PS + r * CH + cc];
+        b += red[(E + e) * PS + r * CH + cc];
       }
       const int col = n0 + tid;
       if (col < p.gemm_n && p.stat_acc) {
