@@ -231,6 +231,18 @@ int64_t tch_conv2d_wgrad_workspace_bytes(int dtype, int K, int R, int S, int C, 
 int tch_conv2d_wgrad(tch_context* ctx, int dtype, const void* x, const void* dy, float* dw, float* workspace,
                      int splits, int accumulate, int N, int H, int W, int C, int K, int R, int S, int stride,
                      int pad, int tile_cfg, int c_logical);
+/* tch_conv2d_wgrad_bias (dbias may be NULL) for a RUN of weight gradients on one context, without a launch per
+ * split reduction: the reduction of a call's partials is not launched with it but rides the NEXT call of this kind
+ * on the same context as extra workgroups of that launch (the partials are complete by stream order, and the
+ * reduction then runs beside the next gradient's multiplications instead of behind its own), in the same fixed
+ * order of the splits: same bits as tch_conv2d_wgrad.  Consecutive calls must alternate between two workspaces
+ * (a call's workspace is read by the call after it); dw / dbias of a call are complete once the next call, or
+ * tch_conv2d_wgrad_flush, has run: flush before anything reads the last gradient.  What autograd's per-layer
+ * weight-gradient calls (train/resnet152.py:84-91) become on a stream of their own. */
+int tch_conv2d_wgrad_trailing(tch_context* ctx, int dtype, const void* x, const void* dy, float* dw, float* dbias,
+                              float* workspace, int splits, int accumulate, int N, int H, int W, int C, int K, int R,
+                              int S, int stride, int pad, int tile_cfg, int c_logical);
+int tch_conv2d_wgrad_flush(tch_context* ctx);
 /* The weight gradients (and optional bias gradients) of n convolutions as ONE launch over a table in device
  * memory, plus one launch for the split reductions that remain: what a training step does once a stage's
  * data-gradient chain has passed and every dy of the stage is at hand (the reference gets one cuDNN call per

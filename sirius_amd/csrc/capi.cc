@@ -486,6 +486,16 @@ int tch_conv2d_wgrad(tch_context* ctx, int dtype, const void* x, const void* dy,
   return conv2d_wgrad(C(ctx), dtype, s, x, dy, dw, workspace, splits, accumulate, tile_cfg);
 }
 
+int tch_conv2d_wgrad_trailing(tch_context* ctx, int dtype, const void* x, const void* dy, float* dw, float* dbias,
+                              float* workspace, int splits, int accumulate, int N, int H, int W, int Cc, int K, int R,
+                              int S, int stride, int pad, int tile_cfg, int c_logical) {
+  ConvShape s = shape(N, H, W, Cc, K, R, S, stride, pad, c_logical);
+  if (splits <= 0) splits = workspace ? conv2d_wgrad_pick_splits(s, dtype) : 1;
+  return conv2d_wgrad(C(ctx), dtype, s, x, dy, dw, workspace, splits, accumulate, tile_cfg, dbias, 1);
+}
+
+int tch_conv2d_wgrad_flush(tch_context* ctx) { return conv2d_wgrad_flush(C(ctx)); }
+
 int tch_conv2d_wgrad_group_plan(int dtype, int n, const int* shapes, int target_wgs, int tile_cfg, int* splits,
                                 int64_t* table_bytes, int64_t* workspace_bytes) {
   if (n <= 0 || !shapes || !splits) {

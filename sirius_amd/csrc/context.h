@@ -153,6 +153,14 @@ class Context {
   Program* recording = nullptr;
   // launches skipped because the reject flag was up since the last reset
   std::atomic<uint64_t> rejected{0};
+  // A split reduction that was not launched with its weight gradient: it rides the next weight-gradient launch of
+  // this context as extra workgroups (conv2d_wgrad with trailing = 1), or goes out with conv2d_wgrad_flush.
+  struct {
+    bool valid = false;
+    ReduceArgs args{};
+    unsigned blocks = 0;
+    double bytes = 0.0;
+  } trailing_reduce;
 
   // `next`: the record that follows in the program being replayed (nullptr: none or unknown).  A lane-0 launch
   // that is followed by a lane-1 launch which has to wait for it carries the event of that wait as its own stop

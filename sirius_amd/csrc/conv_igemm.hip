@@ -90,6 +90,7 @@ struct IgemmArgs {
   int k_per_split;  // multiple of BK
   int out_f32;      // FWD/DGRAD: store fp32 instead of T
   int accumulate;   // WGRAD with splits == 1: out += result
+  int take_pending; // WGRAD, read by the launcher only: the context's pending split reduction rides this launch
   int pointwise;    // 1x1, stride 1, pad 0
   uint32_t a_bytes, b_bytes;  // extents of a_src / b_src for the bounds-checked buffer loads
   FastDiv div_plane;  // pixels per image on the gather side
@@ -891,9 +892,24 @@ __device__ __forceinline__ void wgrad_body(const IgemmArgs& p, uint32_t id) {
   }
 }
 
+__device__ __forceinline__ void splitk_reduce_body(const ReduceArgs& p, uint32_t block);
+
+// One weight gradient, and optionally -- as the workgroups from gemm_wgs on -- the split reduction of the weight
+// gradient launched BEFORE it on the same stream: its partials are complete by stream order, so the reduction needs no
+// launch of its own and runs beside this gradient's multiplications instead of behind them.
+struct WgradArgs {
+  IgemmArgs a;
+  ReduceArgs red;      // red.n == 0: nothing rides along
+  uint32_t gemm_wgs;
+};
+
 template <typename T, int WM, int WN, int TM, int TN>
-__global__ __launch_bounds__(WM* WN * 64) void wgrad_kernel(IgemmArgs p) {
-  wgrad_body<T, WM, WN, TM, TN>(p, xcd_remap(blockIdx.x, gridDim.x));
+__global__ __launch_bounds__(WM* WN * 64) void wgrad_kernel(WgradArgs w) {
+  if (blockIdx.x >= w.gemm_wgs) {
+    splitk_reduce_body(w.red, blockIdx.x - w.gemm_wgs);
+    return;
+  }
+  wgrad_body<T, WM, WN, TM, TN>(w.a, xcd_remap(blockIdx.x, w.gemm_wgs));
 }
 
 // The weight gradients of several convolutions in one launch.  `table` holds one argument block per convolution,
@@ -1408,19 +1424,6 @@ __global__ __launch_bounds__(256) void igemm3_kernel(IgemmArgs p) {
   finish_tile<T, MODE, WM, WN, TM, TN>(p, acc, reinterpret_cast<float*>(lds), tid, m0, n0, tile_m);
 }
 
-struct ReduceArgs {
-  const float* partial;
-  float* out;
-  int64_t n;
-  int splits;
-  int accumulate;
-  // optional second, short vector reduced by the workgroups from first_blocks on (the bias gradient)
-  const float* partial2;
-  float* out2;
-  int n2;
-  unsigned first_blocks;
-};
-
 __device__ __forceinline__ void splitk_reduce_body(const ReduceArgs& p, uint32_t block) {
   if (block >= p.first_blocks) {
     const int i = (block - p.first_blocks) * 256 + threadIdx.x;
@@ -1525,10 +1528,23 @@ int launch_cfg(Context* ctx, IgemmArgs& a, double flops) {
     return -22;
   }
   const dim3 grid(static_cast<unsigned>(wgs)), block(WM * WN * 64);
-  if constexpr (MODE == kWgrad)
-    return launch(ctx, wgrad_kernel<T, WM, WN, TM, TN>, grid, block, a, igemm_name<T, MODE, WM, WN, TM, TN>(), flops, 0,
-                  conv_bytes<MODE>(a, sizeof(T)));
-  else
+  if constexpr (MODE == kWgrad) {
+    static_assert(WM * WN * 64 == 256, "the split reduction that may ride along is written for 256 threads");
+    WgradArgs w{};
+    w.a = a;
+    w.gemm_wgs = static_cast<uint32_t>(wgs);
+    double bytes = conv_bytes<MODE>(a, sizeof(T));
+    auto& tr = ctx->trailing_reduce;
+    unsigned blocks = grid.x;
+    if (a.take_pending && tr.valid) {
+      w.red = tr.args;
+      blocks += tr.blocks;
+      bytes += tr.bytes;
+      tr.valid = false;
+    }
+    return launch(ctx, wgrad_kernel<T, WM, WN, TM, TN>, dim3(blocks), block, w, igemm_name<T, MODE, WM, WN, TM, TN>(), flops, 0,
+                  bytes);
+  } else
     return launch(ctx, igemm_kernel<T, MODE, WM, WN, TM, TN>, grid, block, a, igemm_name<T, MODE, WM, WN, TM, TN>(),
                   flops, 0, conv_bytes<MODE>(a, sizeof(T)));
 }
@@ -1936,8 +1952,15 @@ int conv2d_wgrad_pick_splits(const ConvShape& s, int dtype) {
   return static_cast<int>(want);
 }
 
+int conv2d_wgrad_flush(Context* ctx) {
+  auto& tr = ctx->trailing_reduce;
+  if (!tr.valid) return 0;
+  tr.valid = false;
+  return launch(ctx, splitk_reduce_kernel, dim3(tr.blocks), dim3(256), tr.args, "splitk_reduce_kernel", tr.bytes, 1);
+}
+
 int conv2d_wgrad(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* dy, float* dw, float* workspace,
-                 int splits, int accumulate, int tile_cfg, float* dbias) {
+                 int splits, int accumulate, int tile_cfg, float* dbias, int trailing) {
   IgemmArgs a{};
   if (int rc = fill_common(a, s, dtype)) return rc;
   TCH_CHECK_ARG(x && dy && dw, "conv2d_wgrad: null tensor");
@@ -1958,6 +1981,7 @@ int conv2d_wgrad(Context* ctx, int dtype, const ConvShape& s, const void* x, con
   a.splits = splits;
   a.k_per_split = per;
   a.accumulate = accumulate;
+  a.take_pending = trailing ? 1 : 0;
   a.out = splits > 1 ? static_cast<void*>(workspace) : static_cast<void*>(dw);
   float* dbias_partial = workspace ? workspace + static_cast<int64_t>(splits) * a.gemm_m * a.gemm_n : nullptr;
   a.dbias = !dbias ? nullptr : splits > 1 ? dbias_partial : dbias;
@@ -1979,8 +2003,18 @@ int conv2d_wgrad(Context* ctx, int dtype, const ConvShape& s, const void* x, con
     TCH_CHECK_ARG(r.n % 4 == 0, "conv2d_wgrad: filter size must be a multiple of 4");
     r.first_blocks = static_cast<unsigned>((r.n / 4 + 255) / 256);
     const unsigned blocks = r.first_blocks + static_cast<unsigned>((r.n2 + 255) / 256);
-    return launch(ctx, splitk_reduce_kernel, dim3(blocks), dim3(256), r, "splitk_reduce_kernel",
-                  4.0 * r.n * (splits + 1 + (accumulate ? 1 : 0)), 1);
+    const double red_bytes = 4.0 * r.n * (splits + 1 + (accumulate ? 1 : 0));
+    if (trailing) {
+      // not launched now: rides the next weight gradient of this context (which must use ANOTHER workspace), or
+      // conv2d_wgrad_flush.  An earlier pending reduction was taken along by the launch above.
+      auto& tr = ctx->trailing_reduce;
+      tr.valid = true;
+      tr.args = r;
+      tr.blocks = blocks;
+      tr.bytes = red_bytes;
+      return 0;
+    }
+    return launch(ctx, splitk_reduce_kernel, dim3(blocks), dim3(256), r, "splitk_reduce_kernel", red_bytes, 1);
   }
   return 0;
 }

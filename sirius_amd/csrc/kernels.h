@@ -266,9 +266,23 @@ struct LaunchRecord {
   //                   (nothing at the first one), and lane 1's work up to here is what the next one waits for
   int lane;
   int op;
-  alignas(16) unsigned char args[360];
+  alignas(16) unsigned char args[448];
 };
 enum LaunchOp : int { kOpLaunch = 0, kOpLaunchAfter = 1, kOpJoin = 2, kOpJoinBehind = 3 };
+
+// The reduction of the partial results a split weight gradient left: out (+)= sum over the splits of partial, in the
+// order of the splits; optionally a second, short vector (the bias gradient) by the workgroups from first_blocks on.
+struct ReduceArgs {
+  const float* partial;
+  float* out;
+  int64_t n;
+  int splits;
+  int accumulate;
+  const float* partial2;
+  float* out2;
+  int n2;
+  unsigned first_blocks;
+};
 
 class Context;  // defined in context.h
 

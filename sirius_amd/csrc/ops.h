@@ -62,8 +62,13 @@ int conv2d_dgrad_stat_rows(const ConvShape& s, int dtype, int tile_cfg);
 int conv2d_wgrad_pick_splits(const ConvShape& s, int dtype);
 int64_t conv2d_wgrad_workspace_bytes(const ConvShape& s, int dtype, int splits);
 // dbias (optional, [K] fp32): also the column sums of dy, i.e. the gradient of a bias added to the output
+// trailing != 0: the split reduction of THIS call is not launched with it; it rides the next conv2d_wgrad call of the
+// context with trailing != 0 (as extra workgroups of that launch: its partials are complete by stream order), or goes
+// out with conv2d_wgrad_flush.  The workspace must stay untouched until then: consecutive calls alternate between
+// two workspaces.  dw is complete once the launch that carries its reduction has run.
 int conv2d_wgrad(Context* ctx, int dtype, const ConvShape& s, const void* x, const void* dy, float* dw,
-                 float* workspace, int splits, int accumulate, int tile_cfg, float* dbias = nullptr);
+                 float* workspace, int splits, int accumulate, int tile_cfg, float* dbias = nullptr, int trailing = 0);
+int conv2d_wgrad_flush(Context* ctx);
 // Several weight gradients as one launch (+ one for the split reductions that remain).  _plan picks a split
 // count per convolution so that the group yields about target_wgs workgroups of equal length (one split each if
 // the group is large enough without), says how large the device table and the workspace must be, and returns

@@ -21,17 +21,16 @@ PEAK_BYTES = 8.0e12
 def family(name):
     """Kernel family of a launch: what the kernel does, without its tiling."""
     if name.startswith(("igemm2_kernel", "igemm3_kernel", "igemm_kernel")):
-        m = re.search(r"<(?:bf16, |float, )?(\d)", name)
-        mode = m.group(1) if m else "?"
-        return "conv fwd" if mode == "0" else "conv dgrad"
+        return "conv data gradient" if ",dgrad" in name else "conv forward"
     if name.startswith("wgrad"):
-        return "conv wgrad"
+        return "conv weight gradient"
     if name.startswith("splitk"):
-        return "wgrad split reduce"
-    if name.startswith("bn_fin_apply"):
-        return "bn finalize+apply " + ("bwd" if name.rstrip(">").endswith("1") else "fwd")
+        return "split reduction"
+    direction = "bwd" if ",bwd" in name else "fwd"
+    if name.startswith(("bn_fin_apply", "bn_acc_apply")):
+        return f"bn coefficients+apply {direction}"
     if name.startswith("bn_apply"):
-        return "bn apply " + ("bwd" if ", 1," in name else "fwd")
+        return f"bn apply {direction}"
     if "finalize" in name:
         return "bn finalize"
     return name.split("<")[0]

@@ -22,6 +22,7 @@ torch supplies device memory and streams only.  Dropout is off (probabilities 0)
 """
 import contextlib
 import math
+import os
 
 import torch
 
@@ -44,8 +45,13 @@ class _Plan:
 class GPT2Engine(EngineBase):
     def __init__(self, vocab=50257, n_pos=1024, n_embd=768, n_layer=12, n_head=12, seq_len=1024, dtype=torch.bfloat16,
                  optimizer="adamw", lr=1e-3, weight_decay=0.01, betas=(0.9, 0.999), eps=1e-8, momentum=0.9,
-                 stream=None, allocator=None, overlap_wgrad=True, fused_attention=True, trailing_wgrad=True):
+                 stream=None, allocator=None, overlap_wgrad=True, fused_attention=True, trailing_wgrad=True,
+                 trailing_reduce=None):
         self._init_engine(dtype, stream, allocator)
+        # trailing_reduce: the split reduction of a weight gradient rides the next weight-gradient launch as extra
+        # workgroups instead of being a launch of its own (same bits)
+        self.trailing_reduce = (os.environ.get("TCH_TRAILING_REDUCE", "1") != "0") if trailing_reduce is None \
+            else bool(trailing_reduce)
         # weight and bias gradients depend only on a saved activation and on a gradient that stays put until
         # the layer is done: recorded on a second lane, they run beside the data-gradient chain; the lanes
         # meet at the end of every layer, before its gradient buffers are handed round again
@@ -229,7 +235,15 @@ class GPT2Engine(EngineBase):
                 K, _, _, Cin = p.store_shape
                 sp = int(ops.lib().tch_conv2d_wgrad_pick_splits(code, R, 1, 1, Cin, K, 1, 1, 1, 0))
                 ws_bytes = max(ws_bytes, ops.conv2d_wgrad_workspace_bytes(code, K, 1, 1, Cin, sp))
-        wg_ws = act(ws_bytes // 4, dtype=torch.float32)
+        # two workspaces taken in turn: the split reduction of a weight gradient rides the launch of the next one
+        wg_half = (ws_bytes // 4 + 63) // 64 * 64
+        wg_ws = act(2 * wg_half, dtype=torch.float32)
+        trail = ops.TrailingWgrad(ctx, wg_ws, wg_half) if self.trailing_reduce else None
+
+        def wgrad(x4, dy4, dw, dbias=None):
+            if trail is not None:
+                return trail.wgrad(x4, dy4, dw, 1, 0, dbias=dbias)
+            ops.conv2d_wgrad(ctx, x4, dy4, dw, 1, 0, workspace=wg_ws, dbias=dbias)
 
         def ln_stats(i):
             return ln_mean[i * R:(i + 1) * R], ln_rstd[i * R:(i + 1) * R]
@@ -258,8 +272,7 @@ class GPT2Engine(EngineBase):
         def lin_bwd(name, x, dy, dx):
             """dW, db from (x, dy); dx = dy W"""
             with side():
-                ops.conv2d_wgrad(ctx, as4(x), as4(dy), self._view(self.grads, name + ".weight"), 1, 0, workspace=wg_ws,
-                                 dbias=self._view(self.grads, name + ".bias"))
+                wgrad(as4(x), as4(dy), self._view(self.grads, name + ".weight"), self._view(self.grads, name + ".bias"))
             ops.conv2d_dgrad(ctx, as4(dy), self._wt(name + ".weight"), as4(dx), 1, 0)
 
         # strides / batch offsets of head h of sample b inside the packed projection and the score tensor
@@ -336,8 +349,7 @@ class GPT2Engine(EngineBase):
             dP = act(B * H, T, dtype=torch.float32) if fused else act(B, H, T, T)   # fused: the delta scratch
             d_hf, g = g_c[0], g_c[1]
             with side():
-                ops.conv2d_wgrad(ctx, as4(hf), as4(dlogits), self._view(self.grads, "transformer.wte.weight"), 1, 0,
-                                 workspace=wg_ws)
+                wgrad(as4(hf), as4(dlogits), self._view(self.grads, "transformer.wte.weight"))
             ops.conv2d_dgrad(ctx, as4(dlogits), self._wt("transformer.wte.weight"), as4(d_hf), 1, 0)
             ln_bwd("transformer.ln_f", 2 * L, d_hf, h, g)
             mark("bwd", "ln_f")
@@ -377,6 +389,9 @@ class GPT2Engine(EngineBase):
                 if self.overlap_wgrad:
                     ctx.join(behind=self.trailing_wgrad)
                 mark("bwd", f"h.{i}")
+            if trail is not None:
+                with side():
+                    trail.flush()     # the last weight gradient's own reduction
             if self.overlap_wgrad:
                 ctx.join()
             # tied weights: the scattered embedding gradient lands on top of the head's weight gradient

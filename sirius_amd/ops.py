@@ -415,6 +415,35 @@ def conv2d_wgrad(ctx, x, dy, dw, stride, pad, workspace=None, splits=0, accumula
           "tch_conv2d_wgrad")
 
 
+class TrailingWgrad:
+    """A run of weight gradients on one context whose split reductions ride the launches behind them
+    (tch_conv2d_wgrad_trailing): `workspace` holds TWO workspaces of `half` floats each, taken in turn (the partials
+    of a call are read by the call after it).  flush() launches the last reduction; until then the last dw is
+    incomplete."""
+
+    def __init__(self, ctx, workspace, half):
+        assert workspace.dtype == torch.float32 and workspace.numel() >= 2 * half
+        self.ctx, self.ws, self.half, self.turn = ctx, workspace, half, 0
+
+    def wgrad(self, x, dy, dw, stride, pad, accumulate=False, tile_cfg=-1, c_logical=0, dbias=None):
+        N, H, W, C = x.shape
+        K, R, S, C2 = dw.shape
+        assert C == C2 and dw.dtype == torch.float32
+        Ho, Wo = conv_out_hw(H, W, R, S, stride, pad)
+        assert tuple(dy.shape) == (N, Ho, Wo, K) and dy.dtype == x.dtype
+        assert dbias is None or (dbias.dtype == torch.float32 and dbias.numel() == K)
+        splits = conv2d_wgrad_splits(x, K, R, S, stride, pad)
+        assert self.half * 4 >= conv2d_wgrad_workspace_bytes(dtype_code(x), K, R, S, C, splits), "wgrad workspace too small"
+        ws = self.ws[self.turn * self.half:(self.turn + 1) * self.half]
+        self.turn ^= 1
+        check(lib().tch_conv2d_wgrad_trailing(self.ctx.handle, dtype_code(x), _p(x), _p(dy), _p(dw), _p(dbias), _p(ws),
+                                              splits, int(accumulate), N, H, W, C, K, R, S, stride, pad, tile_cfg,
+                                              c_logical), "tch_conv2d_wgrad_trailing")
+
+    def flush(self):
+        check(lib().tch_conv2d_wgrad_flush(self.ctx.handle), "tch_conv2d_wgrad_flush")
+
+
 def _wgrad_group_shapes(items):
     import ctypes
     flat = []

@@ -52,7 +52,7 @@ class ResNetEngine(EngineBase):
                  lr=0.1, momentum=0.9, weight_decay=1e-4, bn_momentum=0.1, bn_eps=1e-5, stream=None, allocator=None,
                  overlap_wgrad=True, fuse_bn_stats=True, fuse_bn_bwd=True, fuse_bn_finalize=False, autotune=False,
                  retain_gradients=False, group_wgrad=False, wgrad_group_wgs=256, wgrad_group_blocks=2,
-                 wgrad_group_max_wgs=0, bn_acc=None):
+                 wgrad_group_max_wgs=0, bn_acc=None, trailing_reduce=None):
         self._init_engine(dtype, stream, allocator)
         assert num_classes % 8 == 0, "class count must be a multiple of one 16-byte chunk"
         self.image_size, self.num_classes = image_size, num_classes
@@ -82,6 +82,10 @@ class ResNetEngine(EngineBase):
         self.wgrad_group_wgs, self.wgrad_group_blocks = wgrad_group_wgs, wgrad_group_blocks
         self.wgrad_group_max_wgs = wgrad_group_max_wgs
         self.fuse_bn_stats = fuse_bn_stats
+        # trailing_reduce: the split reduction of a weight gradient is not a launch of its own but rides the next
+        # weight-gradient launch of the step as extra workgroups (two workspaces taken in turn); same bits
+        self.trailing_reduce = (os.environ.get("TCH_TRAILING_REDUCE", "1") != "0") if trailing_reduce is None \
+            else bool(trailing_reduce)
         # fuse_bn_bwd: a data-gradient convolution whose output flows into a BatchNorm(+ReLU) backward applies
         # the ReLU gate and takes that BatchNorm's two reductions in its epilogue (no reduction pass)
         self.fuse_bn_bwd = fuse_bn_bwd
@@ -434,7 +438,9 @@ class ResNetEngine(EngineBase):
         fc = _Conv("fc", self.feat, self.num_classes, 1, 1, 0)
         wg_need(fc, B, 1, 1)
         bn_ws = act(bn_ws_bytes[0] // 4, dtype=torch.float32)
-        wg_ws = act(wg_ws_bytes[0] // 4, dtype=torch.float32)
+        wg_half = (wg_ws_bytes[0] // 4 + 63) // 64 * 64
+        wg_ws = act(2 * wg_half, dtype=torch.float32)
+        trail = ops.TrailingWgrad(ctx, wg_ws, wg_half) if self.trailing_reduce else None
 
         def bn_fwd(name, x, y, residual=None, relu=True):
             o, c = self._bn_off[name]
@@ -530,13 +536,16 @@ class ResNetEngine(EngineBase):
             if grouped and self.group_wgrad:
                 pending.append((c, x, dy))
                 return
-            if self.overlap_wgrad:
-                with ctx.side_lane(wait_main=True):
-                    ops.conv2d_wgrad(ctx, x, dy, self._view(self.grads, c.name + ".weight"), c.stride, c.pad,
-                                     workspace=wg_ws, c_logical=c.cin)
-            else:
+            def one():
+                if trail is not None:
+                    return trail.wgrad(x, dy, self._view(self.grads, c.name + ".weight"), c.stride, c.pad, c_logical=c.cin)
                 ops.conv2d_wgrad(ctx, x, dy, self._view(self.grads, c.name + ".weight"), c.stride, c.pad,
                                  workspace=wg_ws, c_logical=c.cin)
+            if self.overlap_wgrad:
+                with ctx.side_lane(wait_main=True):
+                    one()
+            else:
+                one()
 
         def conv_dgrad(c, dy, dx, **kw):
             ops.conv2d_dgrad(ctx, dy, self._wt(c.name + ".weight"), dx, c.stride, c.pad, c_logical=c.cin,
@@ -734,6 +743,12 @@ class ResNetEngine(EngineBase):
             bn_bwd("bn1", g_a0, z0, dz0, a0)
             gfree(g_a0)
             conv_wgrad(self.stem, x0, dz0)
+            if trail is not None:      # the stem's own reduction: nothing behind it to ride on
+                if self.overlap_wgrad:
+                    with ctx.side_lane(wait_main=False):
+                        trail.flush()
+                else:
+                    trail.flush()
             named["head"].update(g_p0=g_out, g_a0=g_a0, dz0=dz0)
             gfree(dz0, True)
             ctx.join()

@@ -21,6 +21,7 @@ torch supplies device memory and streams only.  Stochastic depth and dropout are
 """
 import contextlib
 import math
+import os
 
 import torch
 
@@ -71,8 +72,12 @@ class SwinEngine(EngineBase):
     def __init__(self, embed=128, depths=(2, 2, 18, 2), heads=(4, 8, 16, 32), window=7, patch=4, image_size=224,
                  num_classes=1000, dtype=torch.bfloat16, lr=1e-3, weight_decay=0.05, betas=(0.9, 0.999), eps=1e-8,
                  stream=None, allocator=None, overlap_wgrad=True, fused_attention=True, fuse_window_ln=True,
-                 batch_bias_gather=True):
+                 batch_bias_gather=True, trailing_reduce=None):
         self._init_engine(dtype, stream, allocator)
+        # trailing_reduce: the split reduction of a weight gradient rides the next weight-gradient launch as extra
+        # workgroups instead of being a launch of its own (same bits)
+        self.trailing_reduce = (os.environ.get("TCH_TRAILING_REDUCE", "1") != "0") if trailing_reduce is None \
+            else bool(trailing_reduce)
         # weight / bias / bias-table gradients on a second lane beside the data-gradient chain; the lanes meet
         # at the end of every block, before its gradient buffers are handed round again
         self.overlap_wgrad = overlap_wgrad
@@ -277,7 +282,14 @@ class SwinEngine(EngineBase):
         for n_, h_, w_, cin, k_, r_, s_, stride in calls:
             sp = int(ops.lib().tch_conv2d_wgrad_pick_splits(code, n_, h_, w_, cin, k_, r_, s_, stride, 0))
             ws_bytes = max(ws_bytes, ops.conv2d_wgrad_workspace_bytes(code, k_, r_, s_, cin, sp))
-        wg_ws = act(ws_bytes // 4, dtype=torch.float32)
+        wg_half = (ws_bytes // 4 + 63) // 64 * 64
+        wg_ws = act(2 * wg_half, dtype=torch.float32)     # two workspaces taken in turn (trailing reductions)
+        trail = ops.TrailingWgrad(ctx, wg_ws, wg_half) if self.trailing_reduce else None
+
+        def wgrad(x4, dy4, dw, stride=1, dbias=None, c_logical=0):
+            if trail is not None:
+                return trail.wgrad(x4, dy4, dw, stride, 0, dbias=dbias, c_logical=c_logical)
+            ops.conv2d_wgrad(ctx, x4, dy4, dw, stride, 0, workspace=wg_ws, dbias=dbias, c_logical=c_logical)
         bias_ws = act(64 * 4 * self.feat, dtype=torch.float32)
 
         def ln_fwd(name, x, y, stats, window=None, **kw):
@@ -302,8 +314,8 @@ class SwinEngine(EngineBase):
 
         def lin_bwd(name, x, dy, dx, bias=True):
             with side():
-                ops.conv2d_wgrad(ctx, as4(x), as4(dy), self._view(self.grads, name + ".weight"), 1, 0, workspace=wg_ws,
-                                 dbias=self._view(self.grads, name + ".bias") if bias else None)
+                wgrad(as4(x), as4(dy), self._view(self.grads, name + ".weight"),
+                      dbias=self._view(self.grads, name + ".bias") if bias else None)
             if dx is not None:
                 ops.conv2d_dgrad(ctx, as4(dy), self._wt(name + ".weight"), as4(dx), 1, 0)
 
@@ -514,8 +526,7 @@ class SwinEngine(EngineBase):
                     spare = [k for k in range(len(g_bufs)) if k != gi]
                     d_nm = v2(g_4c_a, rows // 4, 4 * C)
                     with side():
-                        ops.conv2d_wgrad(ctx, as4(nm), as4(g), self._view(self.grads, pre + "reduction.weight"), 1, 0,
-                                         workspace=wg_ws)
+                        wgrad(as4(nm), as4(g), self._view(self.grads, pre + "reduction.weight"))
                     ops.conv2d_dgrad(ctx, as4(g), self._wt(pre + "reduction.weight"), as4(d_nm), 1, 0)
                     d_xm = v2(g_4c_b, rows // 4, 4 * C)
                     ln_bwd(pre + "norm", d_nm, xm, d_xm, mstats)
@@ -602,8 +613,11 @@ class SwinEngine(EngineBase):
             spare = [k for k in range(len(g_bufs)) if k != gi]
             d_e0 = v2(g_bufs[spare[0]], rows0, C0)
             ln_bwd("features.0.2", g, e0, d_e0, embed_stats)
-            ops.conv2d_wgrad(ctx, x0, d_e0.view(B, R0, R0, C0), self._view(self.grads, "features.0.0.weight"), P, 0,
-                             workspace=wg_ws, c_logical=3)
+            # on the main lane, behind the join that ended the last block: the second lane's last weight gradient has
+            # finished, so its pending reduction may ride this launch; this one's own reduction follows at once
+            wgrad(x0, d_e0.view(B, R0, R0, C0), self._view(self.grads, "features.0.0.weight"), stride=P, c_logical=3)
+            if trail is not None:
+                trail.flush()
             ops.bias_grad(ctx, d_e0, self._view(self.grads, "features.0.0.bias"), workspace=bias_ws)
             if self.overlap_wgrad:
                 ctx.join()

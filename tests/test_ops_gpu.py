@@ -330,6 +330,68 @@ def test_conv_wgrad(ctx, dtype, case, splits):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_conv_wgrad_with_trailing_reductions(ctx, dtype):
+    """A run of weight gradients whose split reductions ride the launches behind them (tch_conv2d_wgrad_trailing):
+    every dw / dbias equals the one-call-per-layer result BIT FOR BIT (same splits, same order of additions), with
+    and without bias gradients, accumulating and not, a layer without splits in the middle of the run, twice in a row
+    on the same workspaces; and no reduction launch is left in the run except the flush."""
+    from sirius_amd import ops
+    g = _gen(61)
+    layers = [  # N, H, W, C, K, R, stride, pad, with bias
+        (4, 14, 14, 256, 64, 1, 1, 0, False),
+        (4, 14, 14, 64, 64, 3, 1, 1, True),
+        (1, 4, 4, 64, 256, 1, 1, 0, False),       # few pixels: one split, nothing to reduce
+        (4, 14, 14, 64, 256, 1, 1, 0, True),
+        (2, 16, 16, 64, 128, 3, 2, 1, False),
+    ]
+    data = []
+    for N, H, W, C, K, R, st, pad, bias in layers:
+        Ho, Wo = ops.conv_out_hw(H, W, R, R, st, pad)
+        data.append((rnd((N, H, W, C), dtype, g).cuda(), rnd((N, Ho, Wo, K), dtype, g).cuda()))
+    code = ops.dtype_code(data[0][0])
+    half = 0
+    for (x, dy), (N, H, W, C, K, R, st, pad, bias) in zip(data, layers):
+        sp = ops.conv2d_wgrad_splits(x, K, R, R, st, pad)
+        half = max(half, ops.conv2d_wgrad_workspace_bytes(code, K, R, R, C, sp) // 4)
+    half = (half + 63) // 64 * 64
+    ws_ref = torch.empty(half, device="cuda")
+    ws = torch.full((2 * half,), float("nan"), device="cuda")
+    for accumulate in (False, True):
+        ref, got = [], []
+        for (x, dy), (N, H, W, C, K, R, st, pad, bias) in zip(data, layers):
+            dw = torch.full((K, R, R, C), 0.5, device="cuda")
+            db = torch.full((K,), 0.25, device="cuda") if bias else None
+            ops.conv2d_wgrad(ctx, x, dy, dw, st, pad, workspace=ws_ref, accumulate=accumulate, dbias=db)
+            ref.append((dw, db))
+        prog = ops.Program()
+        ctx.begin_record(prog)
+        try:
+            trail = ops.TrailingWgrad(ctx, ws, half)
+            for (x, dy), (N, H, W, C, K, R, st, pad, bias) in zip(data, layers):
+                dw = torch.full((K, R, R, C), 0.5, device="cuda")
+                db = torch.full((K,), 0.25, device="cuda") if bias else None
+                trail.wgrad(x, dy, dw, st, pad, accumulate=accumulate, dbias=db)
+                got.append((dw, db))
+            trail.flush()
+        finally:
+            ctx.end_record()
+        names = [r["name"] for r in ctx.profile(prog, 1)]
+        # at most the flush: nothing is left for it when the last layer of the run has a single split
+        assert sum(r["launches"] for r in ctx.profile(prog, 1) if r["name"].startswith("splitk_reduce")) <= 1, names
+        for t, _ in got:        # the profile replays ran the program: start again from the initial values
+            t.fill_(0.5)
+        for _, b in got:
+            if b is not None:
+                b.fill_(0.25)
+        ctx.run(prog)
+        ctx.synchronize()
+        torch.cuda.synchronize()
+        for i, ((dw, db), (rw, rb)) in enumerate(zip(got, ref)):
+            assert torch.equal(dw, rw), f"layer {i}, accumulate {accumulate}: dw"
+            assert (db is None) or torch.equal(db, rb), f"layer {i}, accumulate {accumulate}: dbias"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("target_wgs,tile_cfg,max_wgs", [(0, -1, 0), (40, -1, 0), (300, 0, 0), (64, 2, 0), (0, -1, 37), (300, 0, 8)])
 def test_conv_wgrad_group(ctx, dtype, target_wgs, tile_cfg, max_wgs):
     """Several weight gradients in one launch over a table: each layer's result equals the oracle's, and equals
