@@ -96,6 +96,13 @@ typedef struct tch_launch_stat {
  * on the chip, next to the work it states -- the input of a per-layer roofline table. */
 int tch_program_profile_launches(tch_context* ctx, const tch_program* prog, int reps, tch_launch_stat* out,
                                  int64_t max_out, int64_t* n_out);
+/* One kernel family INSIDE the program as it runs: `reps` plain replays (both lanes, nothing added between the
+ * launches; not for a context behind a launch queue), every launch of the kernel called `kernel_name` carrying
+ * a start and a stop event of its own.  mean_us: mean duration of those launches while the rest of the program
+ * shares the chip with them -- the figure a rocprofv3 kernel trace of the same run shows, and what a roofline
+ * fraction of a kernel that runs beside others should be quoted on. */
+int tch_program_time_kernel(tch_context* ctx, const tch_program* prog, const char* kernel_name, int reps,
+                            double* mean_us, int64_t* launches_per_replay);
 
 /* ---- preemptible launch queues (replaces common/xsched_ctrl.h:12-40) ------------ */
 uint64_t tch_RegisterStream(uint64_t hip_stream);   /* xsched_ctrl.cc:27-46; 0 on failure */

@@ -662,6 +662,16 @@ extern "C" int tch_program_profile(tch_context* ctx, const tch_program* prog, in
   return 0;
 }
 
+extern "C" int tch_program_time_kernel(tch_context* ctx, const tch_program* prog, const char* kernel_name, int reps,
+                                       double* mean_us, int64_t* launches_per_replay) {
+  if (!ctx || !prog) {
+    set_error("tch_program_time_kernel: null argument");
+    return -22;
+  }
+  // the name must outlive the call only: launches are compared by content
+  return time_kernel_in_program(&ctx->ctx, prog->prog, kernel_name, reps, mean_us, launches_per_replay);
+}
+
 extern "C" int tch_program_profile_launches(tch_context* ctx, const tch_program* prog, int reps, tch_launch_stat* out,
                                             int64_t max_out, int64_t* n_out) {
   if (!ctx || !prog || !out || !n_out || max_out < 1) {

@@ -418,6 +418,23 @@ int Context::synchronize() {
   return 0;
 }
 
+int Context::launch_direct(hipStream_t s, const LaunchRecord& rec, hipEvent_t stop) {
+  if (!timed_name || !rec.name || strcmp(rec.name, timed_name) != 0) return launch_now(s, rec, stop);
+  hipEvent_t begin = nullptr, end = stop;
+  if (hipEventCreate(&begin) != hipSuccess || (!end && hipEventCreate(&end) != hipSuccess)) {
+    if (begin) (void)hipEventDestroy(begin);
+    set_error("timed launch: hipEventCreate failed");
+    return -12;
+  }
+  timed_events.emplace_back(begin, end);
+  void* args[1] = {const_cast<unsigned char*>(rec.args)};
+  if (hipExtLaunchKernel(rec.fn, rec.grid, rec.block, args, 0, s, begin, end, 0) != hipSuccess) {
+    set_error("timed launch: hipExtLaunchKernel failed");
+    return -5;
+  }
+  return 0;
+}
+
 int Context::dispatch(const LaunchRecord& rec, const LaunchRecord* next) {
   if (g_reject.load(std::memory_order_acquire)) {
     if (rec.fn) rejected.fetch_add(1);
@@ -508,15 +525,24 @@ int Context::dispatch(const LaunchRecord& rec, const LaunchRecord* next) {
       }
     }
     side_dirty = true;
-    return launch_now(s, rec);
+    return launch_direct(s, rec, nullptr);
   }
   fork_event_ = nullptr;
   main_since_fork_ = true;
   if (next && next->fn && next->lane == 1 && next->op == kOpLaunchAfter && fork_by_stop_event()) {
-    fork_event_ = next_event();
-    return launch_now(main, rec, fork_event_);
+    const bool timed = timed_name && rec.name && strcmp(rec.name, timed_name) == 0;
+    if (timed) {   // the fork event doubles as the end of the measurement: it must keep its timestamps
+      if (hipEventCreate(&fork_event_) != hipSuccess) {
+        fork_event_ = nullptr;
+        set_error("timed launch: hipEventCreate failed");
+        return -12;
+      }
+    } else {
+      fork_event_ = next_event();
+    }
+    return launch_direct(main, rec, fork_event_);
   }
-  return launch_now(main, rec);
+  return launch_direct(main, rec, nullptr);
 }
 
 // ---------------------------------------------------------------------------
@@ -681,6 +707,40 @@ int profile_program(Context* ctx, const Program& prog, int reps, std::vector<Ker
   if (rc == 0 && out)
     for (auto& kv : agg) out->push_back(kv.second);
   return rc;
+}
+
+int time_kernel_in_program(Context* ctx, const Program& prog, const char* name, int reps, double* mean_us,
+                           int64_t* launches_per_replay) {
+  if (!name || reps < 1 || ctx->recording || ctx->queue) {
+    set_error("time_kernel_in_program: needs a kernel name, reps >= 1 and a context that is neither recording nor "
+              "behind a launch queue");
+    return -22;
+  }
+  const size_t n = prog.launches.size();
+  double sum_ms = 0.0;
+  int64_t count = 0;
+  int rc = 0;
+  for (int r = 0; r < reps && rc == 0; ++r) {
+    ctx->timed_name = name;
+    ctx->note_foreign_work();
+    for (size_t i = 0; i < n && rc == 0; ++i) rc = ctx->dispatch(prog.launches[i], i + 1 < n ? &prog.launches[i + 1] : nullptr);
+    ctx->timed_name = nullptr;
+    if (ctx->synchronize() != 0 && rc == 0) rc = -5;
+    for (auto& be : ctx->timed_events) {
+      float ms = 0.f;
+      if (rc == 0 && hipEventElapsedTime(&ms, be.first, be.second) == hipSuccess) {
+        sum_ms += ms;
+        ++count;
+      }
+      (void)hipEventDestroy(be.first);
+      (void)hipEventDestroy(be.second);
+    }
+    ctx->timed_events.clear();
+  }
+  if (rc) return rc;
+  if (mean_us) *mean_us = count ? sum_ms / static_cast<double>(count) * 1e3 : 0.0;
+  if (launches_per_replay) *launches_per_replay = count / reps;
+  return 0;
 }
 
 // ---------------------------------------------------------------------------

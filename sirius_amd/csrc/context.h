@@ -168,7 +168,14 @@ class Context {
   // lane-0 kernel in the queue.
   int dispatch(const LaunchRecord& rec, const LaunchRecord* next = nullptr);
 
+  // Timing of one kernel family INSIDE a plain replay (both lanes, nothing added between launches): while
+  // timed_name is set, every direct launch of a kernel of that name carries a start and a stop event of its
+  // own (the launch's own begin / end timestamps), collected in timed_events.
+  const char* timed_name = nullptr;
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> timed_events;
+
  private:
+  int launch_direct(hipStream_t s, const LaunchRecord& rec, hipEvent_t stop);
   hipEvent_t next_event();
   hipEvent_t fork_event_ = nullptr;  // stop event of the last lane-0 launch, not yet waited for by lane 1
   // lane 0 was given a launch since lane 1 last waited for it (a fork with nothing new to wait for is skipped)
@@ -201,6 +208,12 @@ struct LaunchStat {
 // one entry per program position).
 int profile_program(Context* ctx, const Program& prog, int reps, std::vector<KernelStat>* out,
                     std::vector<LaunchStat>* per_launch = nullptr);
+
+// Replays prog `reps` times as it runs (tch_program_run: two lanes, no launch queue) and measures the launches
+// of the kernel called `name` with the begin / end timestamps of each launch itself: their mean duration in
+// microseconds while the rest of the program shares the chip with them, and how many there are per replay.
+int time_kernel_in_program(Context* ctx, const Program& prog, const char* name, int reps, double* mean_us,
+                           int64_t* launches_per_replay);
 
 // ---- process-wide registry of preemptible streams (xsched_ctrl equivalent) ----
 uint64_t register_stream(uint64_t stream);  // returns a handle, 0 on failure

@@ -1537,9 +1537,10 @@ int launch_cfg(Context* ctx, IgemmArgs& a, double flops) {
     auto& tr = ctx->trailing_reduce;
     unsigned blocks = grid.x;
     if (a.take_pending && tr.valid) {
+      // the launch keeps its own algorithmic bytes (operands once, the filter gradient once): the partial filters
+      // the extra workgroups read are traffic, not work
       w.red = tr.args;
       blocks += tr.blocks;
-      bytes += tr.bytes;
       tr.valid = false;
     }
     return launch(ctx, wgrad_kernel<T, WM, WN, TM, TN>, dim3(blocks), block, w, igemm_name<T, MODE, WM, WN, TM, TN>(), flops, 0,

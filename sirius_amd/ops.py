@@ -148,6 +148,14 @@ class Context:
         return [dict(name=buf[i].name.decode(), total_ms=buf[i].total_ms, launches=int(buf[i].launches),
                      work=buf[i].work, work_is_bytes=bool(buf[i].work_is_bytes), bytes=buf[i].bytes) for i in range(n.value)]
 
+    def time_kernel(self, program, kernel_name, reps=1):
+        """Mean duration (microseconds) of the launches of one kernel inside plain replays of the program, both
+        lanes running, measured with each launch's own begin / end timestamps; and their number per replay."""
+        us, n = ctypes.c_double(0.0), ctypes.c_int64(0)
+        check(lib().tch_program_time_kernel(self.handle, program.handle, kernel_name.encode(), int(reps),
+                                            ctypes.byref(us), ctypes.byref(n)), "tch_program_time_kernel")
+        return us.value, int(n.value)
+
     def profile_launches(self, program, reps=1):
         """The same replay, one dict per program position: name ('' for an entry that launches nothing), ms
         (mean over the repetitions, the launch alone on the chip), flops, bytes (algorithmic), lane, workgroups."""

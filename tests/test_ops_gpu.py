@@ -855,3 +855,46 @@ def test_program_record_replay(ctx):
         assert ctx.run(prog) is False
         torch.cuda.synchronize()
         assert torch.equal(y_prog, y_eager)
+
+
+def test_kernel_timed_inside_a_two_lane_program(ctx):
+    """tch_program_time_kernel: the launches of one kernel timed by their own begin / end timestamps while the
+    program runs on its two lanes -- every launch of that name is counted, the duration is a kernel's (more than
+    nothing, far less than the replay's wall time), the results stay those of a plain replay, and a name no
+    launch carries counts nothing."""
+    import time
+    from sirius_amd import ops
+    g = _gen(15)
+    x = rnd((8, 28, 28, 64), torch.bfloat16, g).cuda()
+    w = rnd((64, 3, 3, 64), torch.bfloat16, g, 0.04).cuda()
+    ys = [torch.zeros((8, 28, 28, 64), dtype=torch.bfloat16, device="cuda") for _ in range(6)]
+    dws = [torch.zeros((64, 3, 3, 64), device="cuda") for _ in range(6)]
+    ws = torch.empty(ops.conv2d_wgrad_workspace_bytes(ops.dtype_code(x), 64, 3, 3, 64, ops.conv2d_wgrad_splits(x, 64, 3, 3, 1, 1)) // 4 + 64,
+                     device="cuda")
+    prog = ops.Program()
+    ctx.begin_record(prog)
+    try:
+        for y, dw in zip(ys, dws):
+            ops.conv2d_fwd(ctx, x, w, y, 1, 1)
+            with ctx.side_lane(wait_main=True):     # reads what the main-lane launch before it wrote
+                ops.conv2d_wgrad(ctx, x, y, dw, 1, 1, workspace=ws)
+        ctx.join()
+    finally:
+        ctx.end_record()
+    ctx.run(prog)
+    ctx.synchronize()
+    torch.cuda.synchronize()
+    want_y, want_dw = [y.clone() for y in ys], [d.clone() for d in dws]
+    names = {r["name"]: r["launches"] for r in ctx.profile(prog, 1)}
+    fwd = next(n for n in names if "fwd" in n)
+    wg = next(n for n in names if n.startswith("wgrad_kernel"))
+    t0 = time.perf_counter()
+    us_fwd, n_fwd = ctx.time_kernel(prog, fwd, 2)        # main-lane kernel whose stop event is also the fork
+    wall_us = (time.perf_counter() - t0) * 1e6
+    us_wg, n_wg = ctx.time_kernel(prog, wg, 2)           # second-lane kernel
+    assert n_fwd == names[fwd] == 6 and n_wg == names[wg] == 6
+    assert 1.0 < us_fwd < wall_us / 2 and 1.0 < us_wg < 5000.0, (us_fwd, us_wg, wall_us)
+    assert ctx.time_kernel(prog, "no_such_kernel", 1) == (0.0, 0)
+    torch.cuda.synchronize()
+    for y, d, wy, wd in zip(ys, dws, want_y, want_dw):
+        assert torch.equal(y, wy) and torch.equal(d, wd)
