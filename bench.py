@@ -33,16 +33,19 @@ HANDOVER_PAGE_MB = 128
 # FETCH_SIZE / WRITE_SIZE counter runs the traffic figures below are taken from.
 PROFILE_FILE = "profiles/resnet152_bf16_bs64_step_kernel_stats_and_traffic.txt"
 MEASURED_TRAFFIC_MIB = {
-    "wgrad_kernel<bf16,128x128>": 31.79 + 13.77,
-    "igemm2_kernel<bf16,dgrad,128x64,3buf,k32>": 71.49 + 31.23,
-    "igemm2_kernel<bf16,dgrad,128x128,2buf>": 59.16 + 36.01,
-    "igemm2_kernel<bf16,dgrad,128x64,3buf>": 70.56 + 33.85,
-    "igemm2_kernel<bf16,fwd,128x128,2buf>": 30.63 + 21.92,
-    "igemm2_kernel<bf16,fwd,128x128,2buf,k32>": 27.89 + 26.94,
-    "igemm2_kernel<bf16,fwd,128x64,3buf>": 37.95 + 22.92,
-    "igemm3_kernel<bf16,dgrad,128x64,3buf,patch160>": 29.74 + 5.90,
-    "bn_apply_kernel<bf16,bwd>": 72.05 + 34.61,
-    "bn_apply_kernel<bf16,fwd>": 54.70 + 36.09,
+    "wgrad_kernel<bf16,128x128>": 44.18 + 15.41,
+    "wgrad_kernel<bf16,64x64>": 93.22 + 6.32,
+    "igemm2_kernel<bf16,dgrad,128x64,3buf,k32>": 73.34 + 33.50,
+    "igemm2_kernel<bf16,dgrad,128x128,2buf>": 63.51 + 30.53,
+    "igemm2_kernel<bf16,dgrad,128x128,3buf,k32>": 66.89 + 35.55,
+    "igemm2_kernel<bf16,dgrad,128x128,2buf,k32>": 89.75 + 34.04,
+    "igemm2_kernel<bf16,dgrad,128x64,3buf>": 70.39 + 31.94,
+    "igemm2_kernel<bf16,fwd,128x128,2buf>": 28.05 + 15.45,
+    "igemm2_kernel<bf16,fwd,128x128,2buf,k32>": 32.77 + 29.51,
+    "igemm2_kernel<bf16,fwd,128x64,3buf>": 37.96 + 16.22,
+    "igemm3_kernel<bf16,dgrad,128x64,3buf,patch160>": 29.50 + 5.99,
+    "bn_fin_apply_kernel<bf16,bwd>": 24.39 + 11.91,
+    "bn_fin_apply_kernel<bf16,fwd>": 20.39 + 12.03,
 }
 
 
