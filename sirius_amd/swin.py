@@ -98,7 +98,8 @@ class SwinEngine(EngineBase):
         for s, (depth, nh) in enumerate(zip(self.depths, self.heads)):
             assert C % nh == 0 and (C // nh) % 8 == 0, "head dimension must be a multiple of one 16-byte chunk"
             ws = min(window, R)
-            assert R % ws == 0, "the window must tile the feature map (padding is not built)"
+            assert R % ws == 0, ("the window must tile the feature map of every stage: the reference trains at 224 x 224 only "
+                                 "(train/swin_b.py:59), padded windows are not built")
             self.stages.append(dict(f=1 + 2 * s, depth=depth, heads=nh, C=C, R=R, ws=ws))
             if s + 1 < len(self.depths):
                 assert R % 2 == 0
