@@ -381,7 +381,11 @@ int tch_layernorm_bwd(tch_context* ctx, int dtype, const void* dy, const void* x
  * Forward with an addend (add, sum_out both non-NULL; sum_out in pixel order): sum_out = x + add rounded to the
  * tensors' type, y = LayerNorm(sum_out): the residual sum behind the attention of a block (window_reverse + add)
  * and the LayerNorm in front of its MLP in one pass.  Same values as the plain calls with tch_window_partition
- * between them. */
+ * between them.  Where the window does not tile the image (H or W not a multiple of window) the window tokens live in
+ * the frame padded at the bottom and the right to whole windows, as torchvision's shifted_window_attention pads its
+ * input: a window-ordered tensor then has B * Hp * Wp rows (Hp, Wp = H, W rounded up), these calls read and write the
+ * rows that belong to pixels only, and the caller keeps the others zero where they are read (tch_fill_zero before a
+ * forward y / a backward dx is written). */
 int tch_layernorm_fwd_windowed(tch_context* ctx, int dtype, const void* x, void* y, const float* gamma, const float* beta,
                                float* mean, float* rstd, int64_t rows, int C, float eps, int H, int W, int window,
                                int shift, int windowed_tensors, const void* add, void* sum_out);
@@ -477,8 +481,9 @@ int tch_relpos_bias_scatter_csr(tch_context* ctx, const float* dbias, const int3
  * also the gradient of the other. */
 int tch_window_partition(tch_context* ctx, int dtype, const void* src, void* dst, const void* add, int B, int H, int W,
                          int C, int window, int shift, int reverse);
-/* reverse == 0: dst[B,H/2,W/2,4C] = concat(src[0::2,0::2], src[1::2,0::2], src[0::2,1::2], src[1::2,1::2]);
- * reverse != 0: the inverse permutation (its gradient). */
+/* reverse == 0: dst[B,H2,W2,4C] = concat(src[0::2,0::2], src[1::2,0::2], src[0::2,1::2], src[1::2,1::2]) with
+ * H2 = (H + 1) / 2, W2 = (W + 1) / 2: an odd side is padded with a zero row / column first;
+ * reverse != 0: the inverse permutation (its gradient; what fell on the padding is dropped). */
 int tch_patch_merge_gather(tch_context* ctx, int dtype, const void* src, void* dst, int B, int H, int W, int C,
                            int reverse);
 /* bias[h, i, j] = table[index[i, j], h] (index int32 [tokens * tokens]); scatter: dtable[e, h] (+)= sum of

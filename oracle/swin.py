@@ -105,10 +105,21 @@ def block(sd, p, x, heads, ws, shift, use_mask=True):
     """One SwinTransformerBlock on x [B, H, W, C] (train/swin_b_tiny.py:104-137; with use_mask the attention mask
     of shifted windows that the full model adds and the toy leaves out)."""
     B, H, W, C = x.shape
-    if ws >= H:             # window covers the image: no shift (train/swin_b_tiny.py:99-101)
-        ws, shift = H, 0
     D = C // heads
     h = F.layer_norm(x, (C,), sd[p + "norm1.weight"], sd[p + "norm1.bias"], 1e-5)
+    # A feature map the window does not tile, or one smaller than the window: the reference's toy asserts the sizes and
+    # shrinks the window (train/swin_b_tiny.py:99-105); the model its train script builds (torchvision's swin_b,
+    # train/swin_b.py:38-45) keeps the window (its bias table has (2 * window - 1)^2 rows whatever the feature map),
+    # pads the normalised map with zeros at the bottom and the right to whole windows, attends over the padded frame
+    # (the padding takes part as keys, with qkv = bias), crops, and does not shift when one window covers the frame.
+    # Restated from torchvision's documented shifted_window_attention; parity unpinned by the reference (it trains at
+    # 224 x 224 only, where nothing is padded and both rules agree); pinned by brute force in the tests.
+    pad_b, pad_r = (-H) % ws, (-W) % ws
+    if pad_b or pad_r:
+        h = F.pad(h, (0, 0, 0, pad_r, 0, pad_b))
+    Hp, Wp = H + pad_b, W + pad_r
+    if ws >= Hp and ws >= Wp:
+        shift = 0
     if shift:
         h = torch.roll(h, shifts=(-shift, -shift), dims=(1, 2))
     win = window_partition(h, ws)                                                   # [B_, N, C]
@@ -120,23 +131,26 @@ def block(sd, p, x, heads, ws, shift, use_mask=True):
     bias = sd[p + "attn.relative_position_bias_table"][idx].view(N, N, heads).permute(2, 0, 1)
     attn = attn + bias.unsqueeze(0)
     if shift and use_mask:
-        m = shift_mask(H, W, ws, shift)
+        m = shift_mask(Hp, Wp, ws, shift)
         nW = m.shape[0]
         attn = (attn.view(B_ // nW, nW, heads, N, N) + m.unsqueeze(1).unsqueeze(0)).view(B_, heads, N, N)
     attn = torch.softmax(attn, dim=-1)
     o = (attn @ v).transpose(1, 2).reshape(B_, N, C)
     o = F.linear(o, sd[p + "attn.proj.weight"], sd[p + "attn.proj.bias"])
-    o = window_reverse(o, ws, B, H, W)
+    o = window_reverse(o, ws, B, Hp, Wp)
     if shift:
         o = torch.roll(o, shifts=(shift, shift), dims=(1, 2))
-    x = x + o
+    x = x + o[:, :H, :W]
     m = F.layer_norm(x, (C,), sd[p + "norm2.weight"], sd[p + "norm2.bias"], 1e-5)
     m = F.gelu(F.linear(m, sd[p + "mlp.0.weight"], sd[p + "mlp.0.bias"]))
     return x + F.linear(m, sd[p + "mlp.3.weight"], sd[p + "mlp.3.bias"])
 
 
 def patch_merging(sd, p, x):
+    """An odd side gets a zero row / column first (torchvision's PatchMerging pads to even sizes)."""
     C = x.shape[-1]
+    if x.shape[1] % 2 or x.shape[2] % 2:
+        x = F.pad(x, (0, 0, 0, x.shape[2] % 2, 0, x.shape[1] % 2))
     x = torch.cat([x[:, 0::2, 0::2], x[:, 1::2, 0::2], x[:, 0::2, 1::2], x[:, 1::2, 1::2]], dim=-1)
     x = F.layer_norm(x, (4 * C,), sd[p + "norm.weight"], sd[p + "norm.bias"], 1e-5)
     return F.linear(x, sd[p + "reduction.weight"])

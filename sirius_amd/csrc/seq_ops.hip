@@ -45,24 +45,28 @@ struct LnArgs {
   float eps;
   // Optional window order (Swin): rows are the pixels of [B, win_h, win_w] images; a tensor flagged below is laid
   // out as window tokens instead (cyclic shift by -win_shift, then win_ws x win_ws windows) and is reached through
-  // window_row().  win_ws == 0: every tensor is in row order.
+  // window_row().  win_ws == 0: every tensor is in row order.  Where the window does not tile the image the window
+  // tokens live in the frame padded at the bottom and the right to win_hp x win_wp (whole windows): a window-ordered
+  // tensor then has B * win_hp * win_wp rows, of which these kernels touch the ones that belong to pixels.
   int win_h, win_w, win_ws, win_shift;
+  int win_hp, win_wp;
   int win_out;   // forward: y   backward: dx
   int win_dy;    // backward: dy
   int win_add;   // backward: the addend
 };
 
-// pixel row (b, h, w) -> its window token (b, wh, ww, i, j): h - shift = wh * ws + i, w - shift = ww * ws + j (mod H, W)
+// pixel row (b, h, w) -> its window token (b, wh, ww, i, j): h - shift = wh * ws + i, w - shift = ww * ws + j, modulo
+// the (padded) frame
 __device__ inline int64_t window_row(const LnArgs& p, int64_t row) {
   const int w = static_cast<int>(row % p.win_w);
   int64_t t = row / p.win_w;
   const int h = static_cast<int>(t % p.win_h);
   t /= p.win_h;
   int hs = h - p.win_shift, wsft = w - p.win_shift;
-  if (hs < 0) hs += p.win_h;
-  if (wsft < 0) wsft += p.win_w;
+  if (hs < 0) hs += p.win_hp;
+  if (wsft < 0) wsft += p.win_wp;
   const int wh = hs / p.win_ws, i = hs - wh * p.win_ws, ww = wsft / p.win_ws, j = wsft - ww * p.win_ws;
-  return (((t * (p.win_h / p.win_ws) + wh) * (p.win_w / p.win_ws) + ww) * p.win_ws + i) * p.win_ws + j;
+  return (((t * (p.win_hp / p.win_ws) + wh) * (p.win_wp / p.win_ws) + ww) * p.win_ws + i) * p.win_ws + j;
 }
 
 // L lanes per row (L = 64: one wavefront per row, NCH 16-byte chunks per lane; L = 16 or 32: short rows, 64 / L
@@ -714,8 +718,7 @@ int layernorm_bwd_partial_rows(int64_t rows) {
 
 int bind_window(LnArgs& a, const LnWindow* win, int64_t rows, int allowed) {
   if (!win || win->ws == 0) return 0;
-  TCH_CHECK_ARG(win->H > 0 && win->W > 0 && win->ws > 0 && win->H % win->ws == 0 && win->W % win->ws == 0,
-                "layernorm: the window must tile the image");
+  TCH_CHECK_ARG(win->H > 0 && win->W > 0 && win->ws > 0, "layernorm: window geometry must be positive");
   TCH_CHECK_ARG(win->shift >= 0 && win->shift < win->ws, "layernorm: shift must be in [0, window)");
   TCH_CHECK_ARG(rows % (static_cast<int64_t>(win->H) * win->W) == 0, "layernorm: rows must be whole images");
   TCH_CHECK_ARG((win->tensors & ~allowed) == 0, "layernorm: a tensor flagged as window-ordered does not exist in this direction");
@@ -723,6 +726,8 @@ int bind_window(LnArgs& a, const LnWindow* win, int64_t rows, int allowed) {
   a.win_w = win->W;
   a.win_ws = win->ws;
   a.win_shift = win->shift;
+  a.win_hp = (win->H + win->ws - 1) / win->ws * win->ws;
+  a.win_wp = (win->W + win->ws - 1) / win->ws * win->ws;
   a.win_out = win->tensors & 1;
   a.win_dy = (win->tensors >> 1) & 1;
   a.win_add = (win->tensors >> 2) & 1;

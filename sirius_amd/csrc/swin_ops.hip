@@ -103,16 +103,20 @@ struct MergeArgs {
 // x0 = (even row, even col), x1 = (odd, even), x2 = (even, odd), x3 = (odd, odd)
 __global__ __launch_bounds__(256) void patch_merge_kernel(MergeArgs p) {
   const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
-  const int H2 = p.H / 2, W2 = p.W / 2;
+  // odd sizes: the image is padded with a zero row / column (the merged map is (H + 1) / 2 x (W + 1) / 2)
+  const int H2 = (p.H + 1) / 2, W2 = (p.W + 1) / 2;
   for (int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; e < p.chunks; e += stride) {
     int64_t src;
+    bool real = true;
     if (!p.reverse) {
       const int c = static_cast<int>(e % p.cc);
       int64_t t = e / p.cc;
       const int q = static_cast<int>(t % 4); t /= 4;
       const int w2 = static_cast<int>(t % W2); t /= W2;
       const int h2 = static_cast<int>(t % H2); t /= H2;
-      src = (((t * p.H + 2 * h2 + (q & 1)) * p.W + 2 * w2 + (q >> 1)) * p.cc) + c;
+      const int h = 2 * h2 + (q & 1), w = 2 * w2 + (q >> 1);
+      real = h < p.H && w < p.W;
+      src = (((t * p.H + h) * p.W + w) * p.cc) + c;
     } else {
       const int c = static_cast<int>(e % p.cc);
       int64_t t = e / p.cc;
@@ -121,7 +125,7 @@ __global__ __launch_bounds__(256) void patch_merge_kernel(MergeArgs p) {
       const int q = (h & 1) + 2 * (w & 1);
       src = ((((t * H2 + (h >> 1)) * W2 + (w >> 1)) * 4 + q) * p.cc) + c;
     }
-    static_cast<uint4*>(p.dst)[e] = static_cast<const uint4*>(p.src)[src];
+    static_cast<uint4*>(p.dst)[e] = real ? static_cast<const uint4*>(p.src)[src] : make_uint4(0u, 0u, 0u, 0u);
   }
 }
 
@@ -249,9 +253,11 @@ int window_partition(Context* ctx, int dtype, const void* src, void* dst, const 
 int patch_merge_gather(Context* ctx, int dtype, const void* src, void* dst, int B, int H, int W, int C, int reverse) {
   TCH_CHECK_ARG(dtype == kBF16 || dtype == kF32, "patch_merge_gather: dtype must be f32(0) or bf16(1)");
   const int E = dtype == kBF16 ? 8 : 4;
-  TCH_CHECK_ARG(src && dst && B > 0 && C > 0 && C % E == 0 && H % 2 == 0 && W % 2 == 0 && H > 0 && W > 0,
-                "patch_merge_gather: bad arguments (even image sides, C a multiple of a 16-byte chunk)");
-  MergeArgs a{src, dst, B, H, W, C / E, reverse, static_cast<int64_t>(B) * H * W * (C / E)};
+  TCH_CHECK_ARG(src && dst && B > 0 && C > 0 && C % E == 0 && H > 0 && W > 0,
+                "patch_merge_gather: bad arguments (C a multiple of a 16-byte chunk)");
+  // one thread per 16-byte chunk of the destination: the merged map (padded to even sides) forward, the image backward
+  const int64_t dst_pixels = reverse ? static_cast<int64_t>(H) * W : static_cast<int64_t>((H + 1) / 2) * ((W + 1) / 2) * 4;
+  MergeArgs a{src, dst, B, H, W, C / E, reverse, B * dst_pixels * (C / E)};
   return launch(ctx, patch_merge_kernel, dim3(flat_blocks(a.chunks)), dim3(256), a,
                 reverse ? "patch_merge_kernel<reverse>" : "patch_merge_kernel<gather>", static_cast<double>(a.chunks) * 32.0, 1);
 }

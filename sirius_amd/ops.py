@@ -745,25 +745,36 @@ def cast_to_f32(ctx, src, dst):
 # transformer operators (Swin-B / GPT-2 steps)
 # ---------------------------------------------------------------------------
 
+def window_token_rows(rows, H, W, ws):
+    """Rows of a window-ordered tensor that belongs to `rows` = B * H * W pixels: the frame is padded at the bottom and
+    the right to whole ws x ws windows."""
+    assert rows % (H * W) == 0
+    return rows // (H * W) * (-(-H // ws) * ws) * (-(-W // ws) * ws)
+
+
 def layernorm_fwd(ctx, x, y, gamma, beta, mean, rstd, eps=1e-5, window=None, windowed=("y",), add=None, sum_out=None):
     """window = (H, W, window size, shift): x is [B*H*W, C] in pixel order; the tensors named in `windowed` ("y",
     "add") are laid out as window tokens (the LayerNorm and the window partition next to it in a Swin block in one
     pass).  add / sum_out: sum_out = x + add (pixel order, rounded to the tensors' type), y = LayerNorm(sum_out)."""
     C = x.shape[-1]
     rows = x.numel() // C
-    assert y.shape == x.shape and y.dtype == x.dtype and x.is_contiguous() and y.is_contiguous()
+    assert y.dtype == x.dtype and x.is_contiguous() and y.is_contiguous()
     assert gamma.numel() == C and beta.numel() == C and gamma.dtype == beta.dtype == torch.float32
     assert mean.numel() == rows and rstd.numel() == rows and mean.dtype == rstd.dtype == torch.float32
     if window is not None:
         H, W, ws, shift = window
+        wrows = window_token_rows(rows, H, W, ws)      # rows of a window-ordered tensor (more than rows when padded)
         assert (add is None) == (sum_out is None)
-        assert add is None or (add.numel() == x.numel() == sum_out.numel() and add.dtype == sum_out.dtype == x.dtype)
+        assert y.numel() == (wrows if "y" in windowed else rows) * C
+        assert add is None or (add.numel() == (wrows if "add" in windowed else rows) * C and sum_out.numel() == x.numel()
+                               and add.dtype == sum_out.dtype == x.dtype)
         flags = sum({"y": 1, "add": 4}[t] for t in windowed)
         check(lib().tch_layernorm_fwd_windowed(ctx.handle, dtype_code(x), _p(x), _p(y), _p(gamma), _p(beta), _p(mean),
                                                _p(rstd), rows, C, eps, H, W, ws, shift, flags, _p(add), _p(sum_out)),
               "tch_layernorm_fwd_windowed")
         return
     assert add is None and sum_out is None, "the residual sum comes with the windowed form"
+    assert y.shape == x.shape
     check(lib().tch_layernorm_fwd(ctx.handle, dtype_code(x), _p(x), _p(y), _p(gamma), _p(beta), _p(mean), _p(rstd),
                                   rows, C, eps), "tch_layernorm_fwd")
 
@@ -778,16 +789,19 @@ def layernorm_bwd(ctx, dy, x, dx, gamma, mean, rstd, dgamma, dbeta, partial, acc
     out as window tokens, everything else ([B*H*W, C] x, the statistics) in pixel order."""
     C = x.shape[-1]
     rows = x.numel() // C
-    assert dy.shape == x.shape == dx.shape and dy.dtype == x.dtype == dx.dtype
+    assert dy.dtype == x.dtype == dx.dtype and (residual is None or residual.dtype == x.dtype)
     assert partial.dtype == torch.float32 and partial.numel() >= layernorm_bwd_partial_rows(rows) * C * 2
-    assert residual is None or (residual.shape == x.shape and residual.dtype == x.dtype)
     if window is not None:
         H, W, ws, shift = window
+        wrows = window_token_rows(rows, H, W, ws)      # rows of a window-ordered tensor (more than rows when padded)
+        for name, t in (("dx", dx), ("dy", dy), ("residual", residual)):
+            assert t is None or t.numel() == (wrows if name in windowed else rows) * C, name
         flags = sum({"dx": 1, "dy": 2, "residual": 4}[t] for t in windowed)
         check(lib().tch_layernorm_bwd_windowed(ctx.handle, dtype_code(x), _p(dy), _p(x), _p(dx), _p(residual), _p(gamma),
                                                _p(mean), _p(rstd), _p(dgamma), _p(dbeta), int(accumulate), rows, C,
                                                _p(partial), H, W, ws, shift, flags), "tch_layernorm_bwd_windowed")
         return
+    assert dy.shape == x.shape == dx.shape and (residual is None or residual.shape == x.shape)
     check(lib().tch_layernorm_bwd(ctx.handle, dtype_code(x), _p(dy), _p(x), _p(dx), _p(residual), _p(gamma), _p(mean), _p(rstd),
                                   _p(dgamma), _p(dbeta), int(accumulate), rows, C, _p(partial)), "tch_layernorm_bwd")
 
@@ -921,9 +935,12 @@ def window_partition(ctx, src, dst, window, shift, reverse=False, add=None, imag
 
 
 def patch_merge_gather(ctx, src, dst, image_shape, reverse=False):
-    """image_shape = (B, H, W, C) of the unmerged side; the merged side is [B, H/2, W/2, 4C]."""
+    """image_shape = (B, H, W, C) of the unmerged side; the merged side is [B, (H+1)//2, (W+1)//2, 4C] (an odd side
+    is padded with zeros)."""
     B, H, W, C = image_shape
-    assert src.numel() == dst.numel() == B * H * W * C and src.dtype == dst.dtype
+    merged = B * ((H + 1) // 2) * ((W + 1) // 2) * 4 * C
+    a, b = (merged, B * H * W * C) if reverse else (B * H * W * C, merged)
+    assert src.numel() == a and dst.numel() == b and src.dtype == dst.dtype
     check(lib().tch_patch_merge_gather(ctx.handle, dtype_code(src), _p(src), _p(dst), B, H, W, C, int(reverse)),
           "tch_patch_merge_gather")
 

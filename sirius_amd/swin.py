@@ -97,13 +97,16 @@ class SwinEngine(EngineBase):
         C, R = embed, image_size // patch
         for s, (depth, nh) in enumerate(zip(self.depths, self.heads)):
             assert C % nh == 0 and (C // nh) % 8 == 0, "head dimension must be a multiple of one 16-byte chunk"
-            ws = min(window, R)
-            assert R % ws == 0, ("the window must tile the feature map of every stage: the reference trains at 224 x 224 only "
-                                 "(train/swin_b.py:59), padded windows are not built")
-            self.stages.append(dict(f=1 + 2 * s, depth=depth, heads=nh, C=C, R=R, ws=ws))
+            # A feature map the window does not tile (or one smaller than the window) is padded at the bottom and the
+            # right to whole windows (Rp), the way torchvision's shifted_window_attention pads its input; the window,
+            # and with it the bias table, stays what it is.  Not needed at the reference's 224 x 224
+            # (train/swin_b.py:59), where the stages are 56, 28, 14 and 7 wide under a 7 x 7 window.
+            ws = window
+            Rp = -(-R // ws) * ws
+            assert Rp == R or fuse_window_ln, "padded windows are built into the LayerNorms next to the partitions only"
+            self.stages.append(dict(f=1 + 2 * s, depth=depth, heads=nh, C=C, R=R, ws=ws, Rp=Rp))
             if s + 1 < len(self.depths):
-                assert R % 2 == 0
-                C, R = 2 * C, R // 2
+                C, R = 2 * C, (R + 1) // 2      # an odd side is padded with a zero row / column by the merge
         self.feat = C
 
         # ---- parameter table (torchvision naming) ----
@@ -259,7 +262,7 @@ class SwinEngine(EngineBase):
 
         st0 = self.stages[0]
         rows0 = B * st0["R"] ** 2
-        max_rc = max(B * st["R"] ** 2 * st["C"] for st in self.stages)          # elements of the largest [rows, C]
+        max_rc = max(B * st["Rp"] ** 2 * st["C"] for st in self.stages)         # elements of the largest [rows, C]
         n_ln = 2 + sum(2 * st["depth"] for st in self.stages) + (len(self.stages) - 1)
         ln_mean, ln_rstd = act(n_ln * rows0, dtype=torch.float32), act(n_ln * rows0, dtype=torch.float32)
         ln_partial = act(max(ops.layernorm_bwd_partial_rows(B * st["R"] ** 2) * 4 * st["C"] * 2 for st in self.stages),
@@ -274,11 +277,11 @@ class SwinEngine(EngineBase):
         # weight-gradient workspace: the largest need over every projection call of the plan
         calls = [(B, S, S, PATCH_CIN_PAD, self.embed, P, P, P), (B, 1, 1, self.feat, self.num_classes, 1, 1, 1)]
         for si, st in enumerate(self.stages):
-            rows, C = B * st["R"] ** 2, st["C"]
+            rows, C = B * st["Rp"] ** 2, st["C"]    # window-ordered operands have the padded frame's rows
             calls += [(rows, 1, 1, C, 3 * C, 1, 1, 1), (rows, 1, 1, C, C, 1, 1, 1), (rows, 1, 1, C, 4 * C, 1, 1, 1),
                       (rows, 1, 1, 4 * C, C, 1, 1, 1)]
             if si + 1 < len(self.stages):
-                calls.append((rows // 4, 1, 1, 4 * C, 2 * C, 1, 1, 1))
+                calls.append((B * ((st["R"] + 1) // 2) ** 2, 1, 1, 4 * C, 2 * C, 1, 1, 1))
         ws_bytes = 4
         for n_, h_, w_, cin, k_, r_, s_, stride in calls:
             sp = int(ops.lib().tch_conv2d_wgrad_pick_splits(code, n_, h_, w_, cin, k_, r_, s_, stride, 0))
@@ -335,12 +338,12 @@ class SwinEngine(EngineBase):
                            st["heads"] % 2 == 0 and st["ws"] ** 2 <= 64)
             st["keys_ld"] = 64 if st["fused"] else st["ws"] ** 2      # leading dimension of a score row
             st["bias_elems"] = st["heads"] * (64 * 64 if st["fused"] else st["ws"] ** 4)
-        max_scores = max(B * (st["R"] // st["ws"]) ** 2 * st["heads"] * st["ws"] ** 2 * st["keys_ld"] for st in self.stages)
+        max_scores = max(B * (st["Rp"] // st["ws"]) ** 2 * st["heads"] * st["ws"] ** 2 * st["keys_ld"] for st in self.stages)
         d_scores = flat(max_scores)
         max_bias = max(st["bias_elems"] for st in self.stages)
         bias_buf = act(max_bias, dtype=torch.float32)
         dbias_buf = act(max_bias, dtype=torch.float32)
-        colsum_ws = act(max(ops.column_sum_workspace_floats(B * (st["R"] // st["ws"]) ** 2,
+        colsum_ws = act(max(ops.column_sum_workspace_floats(B * (st["Rp"] // st["ws"]) ** 2,
                                                             st["heads"] * st["ws"] ** 2 * st["keys_ld"])
                             for st in self.stages), dtype=torch.float32)
 
@@ -350,20 +353,12 @@ class SwinEngine(EngineBase):
         # constants per stage: index of the bias table, mask of the shifted windows
         for st in self.stages:
             ws = st["ws"]
-            st["index"] = relative_position_index(self.window)[:ws * ws, :ws * ws] if ws == self.window else None
-            if st["index"] is None:
-                # a window smaller than the table's: the offsets of a ws-window inside the (2*window-1)^2 table
-                coords = torch.stack(torch.meshgrid([torch.arange(ws), torch.arange(ws)], indexing="ij")).flatten(1)
-                rel = (coords[:, :, None] - coords[:, None, :]).permute(1, 2, 0).contiguous()
-                rel[:, :, 0] += self.window - 1
-                rel[:, :, 1] += self.window - 1
-                rel[:, :, 0] *= 2 * self.window - 1
-                st["index"] = rel.sum(-1)
+            st["index"] = relative_position_index(ws)
             st["index_dev"] = st["index"].to(torch.int32).contiguous().to(dev)
             keep.append(st["index_dev"])
-            shift = ws // 2 if ws < st["R"] else 0
+            shift = ws // 2 if ws < st["Rp"] else 0
             st["shift"] = shift
-            mask = shifted_window_mask(st["R"], st["R"], ws, shift) if shift else None
+            mask = shifted_window_mask(st["Rp"], st["Rp"], ws, shift) if shift else None     # over the padded frame
             if st["fused"]:
                 # (query, key) pairs in rows of 64 keys: -1 = padding (gathers -inf, which masks the padded keys)
                 pairs = torch.full((64, 64), -1, dtype=torch.int32)
@@ -413,7 +408,9 @@ class SwinEngine(EngineBase):
             for si, st in enumerate(self.stages):
                 C, R, ws, Hh = st["C"], st["R"], st["ws"], st["heads"]
                 rows, N, D = B * R * R, ws * ws, C // Hh
-                B_ = rows // N
+                wrows = B * st["Rp"] ** 2       # rows of a window-ordered tensor: the frame padded to whole windows
+                padded = wrows != rows
+                B_ = wrows // N
                 whole = ws == R                 # one window covers the image: window order == image order
                 qkv_row, qkv_b = 3 * C, (N * 3 * C, D)
                 s_b, o_b = (Hh * N * N, N * N), (N * C, D)
@@ -426,16 +423,18 @@ class SwinEngine(EngineBase):
                         xw = act(rows, C)
                         ln_fwd(pre + "norm1", x, xw, stats1)
                     elif self.fuse_window_ln:
-                        xw = act(rows, C)   # LayerNorm and window partition in one pass
+                        xw = act(wrows, C)   # LayerNorm and window partition in one pass
+                        if padded:
+                            ops.fill_zero(ctx, xw)      # the tokens of the padding are zeros behind norm1
                         ln_fwd(pre + "norm1", x, xw, stats1, window=(R, R, ws, shift))
                     else:
                         n1, xw = v2(s_n1, rows, C), act(rows, C)
                         ln_fwd(pre + "norm1", x, n1, stats1)
                         ops.window_partition(ctx, n1, xw, ws, shift, image_shape=(B, R, R, C))
-                    qkv = act(rows, 3 * C)
+                    qkv = act(wrows, 3 * C)
                     lin_fwd(pre + "attn.qkv", xw, qkv)
                     fq = qkv.view(-1)
-                    o = act(rows, C)
+                    o = act(wrows, C)
                     if st["fused"]:
                         Pm = act(B_ * Hh, N, 64)
                         bias = block_bias.get(pre)
@@ -459,8 +458,9 @@ class SwinEngine(EngineBase):
                         lin_fwd(pre + "attn.proj", o, x1, add=x)
                         ln_fwd(pre + "norm2", x1, n2, stats2)
                     elif self.fuse_window_ln:
-                        # x1 = x + window_reverse(projection) and n2 = LayerNorm(x1) in one pass
-                        pr = v2(s_n1, rows, C)
+                        # x1 = x + window_reverse(projection) and n2 = LayerNorm(x1) in one pass (what the projection
+                        # left on the tokens of the padding is never read: the crop)
+                        pr = v2(s_n1, wrows, C)
                         lin_fwd(pre + "attn.proj", o, pr)
                         ln_fwd(pre + "norm2", x, n2, stats2, window=(R, R, ws, shift), windowed=("add",), add=pr, sum_out=x1)
                     else:
@@ -476,8 +476,9 @@ class SwinEngine(EngineBase):
                     mark("fwd", pre[:-1])
                 if si + 1 < len(self.stages):
                     pre = f"features.{st['f'] + 1}."
-                    xm, nm, y = act(rows // 4, 4 * C), act(rows // 4, 4 * C), act(rows // 4, 2 * C)
-                    mstats = new_ln(rows // 4)
+                    mrows = B * ((R + 1) // 2) ** 2
+                    xm, nm, y = act(mrows, 4 * C), act(mrows, 4 * C), act(mrows, 2 * C)
+                    mstats = new_ln(mrows)
                     ops.patch_merge_gather(ctx, x, xm, (B, R, R, C))
                     ln_fwd(pre + "norm", xm, nm, mstats)
                     lin_fwd(pre + "reduction", nm, y, bias=False)
@@ -515,7 +516,10 @@ class SwinEngine(EngineBase):
                 st = self.stages[si]
                 C, R, ws, Hh = st["C"], st["R"], st["ws"], st["heads"]
                 rows, N, D = B * R * R, ws * ws, C // Hh
-                B_ = rows // N
+                wrows = B * st["Rp"] ** 2
+                padded = wrows != rows
+                mrows = B * ((R + 1) // 2) ** 2
+                B_ = wrows // N
                 whole = ws == R
                 qkv_row, qkv_b = 3 * C, (N * 3 * C, D)
                 s_b, o_b = (Hh * N * N, N * N), (N * C, D)
@@ -525,11 +529,11 @@ class SwinEngine(EngineBase):
                     xm, nm, mstats = merges[si]
                     pre = f"features.{st['f'] + 1}."
                     spare = [k for k in range(len(g_bufs)) if k != gi]
-                    d_nm = v2(g_4c_a, rows // 4, 4 * C)
+                    d_nm = v2(g_4c_a, mrows, 4 * C)
                     with side():
                         wgrad(as4(nm), as4(g), self._view(self.grads, pre + "reduction.weight"))
                     ops.conv2d_dgrad(ctx, as4(g), self._wt(pre + "reduction.weight"), as4(d_nm), 1, 0)
-                    d_xm = v2(g_4c_b, rows // 4, 4 * C)
+                    d_xm = v2(g_4c_b, mrows, 4 * C)
                     ln_bwd(pre + "norm", d_nm, xm, d_xm, mstats)
                     gi = spare[0]
                     g = v2(g_bufs[gi], rows, C)
@@ -542,8 +546,10 @@ class SwinEngine(EngineBase):
                     _, _, shift, x_in, xw, qkv, Pm, o, x1, n2, f1, f2, stats1, stats2 = saved_blocks[bi]
                     pre = f"features.{st['f']}.{i}."
                     spare = [k for k in range(len(g_bufs)) if k != gi]
-                    t_a, t_b, t_c, t_d, t_e = (v2(g_bufs[k], rows, C) for k in spare)
-                    d_f2, d_f1, d_qkv = v2(g_4c_a, rows, 4 * C), v2(g_4c_b, rows, 4 * C), v2(g_3c, rows, 3 * C)
+                    # t_b, t_c, t_d carry window-ordered gradients (the padded frame's rows) wherever the block has windows
+                    t_a, t_e = v2(g_bufs[spare[0]], rows, C), v2(g_bufs[spare[4]], rows, C)
+                    t_b, t_c, t_d = (v2(g_bufs[k], wrows, C) for k in spare[1:4])
+                    d_f2, d_f1, d_qkv = v2(g_4c_a, rows, 4 * C), v2(g_4c_b, rows, 4 * C), v2(g_3c, wrows, 3 * C)
                     fq, fg = qkv.view(-1), d_qkv.view(-1)
                     dP = d_scores[:B_ * Hh * N * st["keys_ld"]].view(B_, Hh, N, st["keys_ld"])
                     # MLP
@@ -557,6 +563,8 @@ class SwinEngine(EngineBase):
                     if fuse_w:
                         # the gradient behind norm2 is written as window tokens right away: the projection's gradients
                         # want it in that order, and norm1's backward reads its residual through the same map
+                        if padded:
+                            ops.fill_zero(ctx, g1)      # no gradient reaches the projection's output on the padding
                         ln_bwd(pre + "norm2", t_a, x1, g1, stats2, residual=g, window=win, windowed=("dx",))
                         d_pr = g1
                     elif whole:

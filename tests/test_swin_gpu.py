@@ -98,6 +98,88 @@ def test_layernorm_in_window_order_equals_layernorm_and_partition(ctx, dtype, B,
                           windowed=("dx",))
 
 
+def _to_window_frame(t, B, H, W, ws, shift):
+    """[B*H*W, C] in pixel order -> [B*Hp*Wp, C] window tokens of the frame padded with zeros to whole windows."""
+    C = t.shape[-1]
+    pad_b, pad_r = (-H) % ws, (-W) % ws
+    f = torch.nn.functional.pad(t.view(B, H, W, C), (0, 0, 0, pad_r, 0, pad_b))
+    if shift:
+        f = torch.roll(f, shifts=(-shift, -shift), dims=(1, 2))
+    Hp, Wp = H + pad_b, W + pad_r
+    return f.view(B, Hp // ws, ws, Wp // ws, ws, C).permute(0, 1, 3, 2, 4, 5).reshape(-1, C)
+
+
+def _from_window_frame(t, B, H, W, ws, shift):
+    C = t.shape[-1]
+    Hp, Wp = -(-H // ws) * ws, -(-W // ws) * ws
+    f = t.view(B, Hp // ws, Wp // ws, ws, ws, C).permute(0, 1, 3, 2, 4, 5).reshape(B, Hp, Wp, C)
+    if shift:
+        f = torch.roll(f, shifts=(shift, shift), dims=(1, 2))
+    return f[:, :H, :W].reshape(-1, C)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,H,W,C,ws,shift", [(2, 10, 10, 64, 4, 0), (2, 10, 6, 128, 4, 2), (1, 16, 16, 256, 7, 3), (3, 5, 9, 32, 4, 2)])
+def test_layernorm_in_window_order_on_a_padded_frame(ctx, dtype, B, H, W, C, ws, shift):
+    """A feature map the window does not tile: the window-ordered tensors live in the frame padded to whole windows
+    (more rows than the image).  Forward y and the addend, backward dx, dy and the residual go through that frame
+    with the bits of the plain LayerNorm calls and an explicit pad / roll / partition on the host; rows of the
+    padding are neither read nor written (they keep what the caller put there)."""
+    from sirius_amd import ops
+    g = _gen(53)
+    rows = B * H * W
+    wrows = ops.window_token_rows(rows, H, W, ws)
+    assert wrows > rows
+    win = (H, W, ws, shift)
+    x = torch.randn(rows, C, generator=g).to(dtype).cuda()
+    gamma, beta = (torch.rand(C, generator=g) + 0.5).cuda(), torch.randn(C, generator=g).cuda()
+    new = lambda n=rows: torch.empty(n, C, dtype=dtype, device="cuda")
+    stat = lambda: (torch.empty(rows, device="cuda"), torch.empty(rows, device="cuda"))
+    y_rows, st, st_f = new(), stat(), stat()
+    ops.layernorm_fwd(ctx, x, y_rows, gamma, beta, *st)
+    y_win = torch.full((wrows, C), 7.0, dtype=dtype, device="cuda")          # a marker where the padding is
+    ops.layernorm_fwd(ctx, x, y_win, gamma, beta, *st_f, window=win)
+    torch.cuda.synchronize()
+    marker = _to_window_frame(torch.zeros(rows, 1), B, H, W, ws, shift).squeeze(1)      # 0 at pixels ...
+    is_pad = _to_window_frame(torch.ones(rows, 1), B, H, W, ws, shift).squeeze(1) == 0     # ... True on the padding
+    assert is_pad.sum().item() == wrows - rows and marker.abs().sum() == 0
+    want = _to_window_frame(y_rows.cpu(), B, H, W, ws, shift)
+    got = y_win.cpu()
+    assert torch.equal(got[~is_pad], want[~is_pad]) and torch.all(got[is_pad] == 7.0)
+    assert torch.equal(st[0], st_f[0]) and torch.equal(st[1], st_f[1])
+    # forward with a window-ordered addend: x1 = x + crop(window_reverse(pr)), n2 = LayerNorm(x1)
+    pr_win = torch.randn(wrows, C, generator=g).to(dtype)
+    x1_ref = (x.cpu().float() + _from_window_frame(pr_win, B, H, W, ws, shift).float()).to(dtype).cuda()
+    n2_ref, x1, n2, st2, st2_f = new(), new(), new(), stat(), stat()
+    ops.layernorm_fwd(ctx, x1_ref, n2_ref, gamma, beta, *st2)
+    ops.layernorm_fwd(ctx, x, n2, gamma, beta, *st2_f, window=win, windowed=("add",), add=pr_win.cuda(), sum_out=x1)
+    torch.cuda.synchronize()
+    assert torch.equal(x1, x1_ref) and torch.equal(n2, n2_ref) and torch.equal(st2[0], st2_f[0])
+    # backward, every combination
+    dy_rows = torch.randn(rows, C, generator=g).to(dtype)
+    res_rows = torch.randn(rows, C, generator=g).to(dtype)
+    noise = torch.randn(wrows, C, generator=g).to(dtype)      # what sits on the padding must not matter
+    dy_win = torch.where(is_pad[:, None], noise, _to_window_frame(dy_rows, B, H, W, ws, shift)).cuda()
+    res_win = torch.where(is_pad[:, None], noise, _to_window_frame(res_rows, B, H, W, ws, shift)).cuda()
+    dy_rows, res_rows = dy_rows.cuda(), res_rows.cuda()
+    partial = torch.empty(ops.layernorm_bwd_partial_rows(rows) * C * 2, device="cuda")
+    dx_ref, dg_ref, db_ref = new(), torch.zeros(C, device="cuda"), torch.zeros(C, device="cuda")
+    ops.layernorm_bwd(ctx, dy_rows, x, dx_ref, gamma, st[0], st[1], dg_ref, db_ref, partial, residual=res_rows)
+    torch.cuda.synchronize()
+    dx_ref_win = _to_window_frame(dx_ref.cpu(), B, H, W, ws, shift)
+    for windowed in [("dx",), ("dy",), ("residual",), ("dy", "residual"), ("dx", "dy", "residual")]:
+        dx = torch.full((wrows if "dx" in windowed else rows, C), 7.0, dtype=dtype, device="cuda")
+        dg, db = torch.zeros(C, device="cuda"), torch.zeros(C, device="cuda")
+        ops.layernorm_bwd(ctx, dy_win if "dy" in windowed else dy_rows, x, dx, gamma, st[0], st[1], dg, db, partial,
+                          residual=res_win if "residual" in windowed else res_rows, window=win, windowed=windowed)
+        torch.cuda.synchronize()
+        if "dx" in windowed:
+            assert torch.equal(dx.cpu()[~is_pad], dx_ref_win[~is_pad]) and torch.all(dx.cpu()[is_pad] == 7.0), windowed
+        else:
+            assert torch.equal(dx, dx_ref), windowed
+        assert torch.equal(dg, dg_ref) and torch.equal(db, db_ref), windowed
+
+
 @pytest.mark.parametrize("name,dtype", [("window7", torch.bfloat16), ("shifted", torch.float32)])
 def test_window_order_layernorms_change_no_bit(name, dtype):
     """SwinEngine(fuse_window_ln=True) drops four window-partition launches per block: same loss, gradients and
@@ -188,11 +270,13 @@ def test_batched_bias_gather_changes_no_bit(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("B,H,W,C", [(2, 8, 8, 16), (1, 14, 6, 32), (3, 2, 2, 8)])
+@pytest.mark.parametrize("B,H,W,C", [(2, 8, 8, 16), (1, 14, 6, 32), (3, 2, 2, 8), (2, 5, 5, 16), (1, 7, 4, 8), (2, 1, 3, 32)])
 def test_patch_merge_gather_is_a_bit_exact_permutation(ctx, dtype, B, H, W, C):
+    """Odd sides: a zero row / column is appended first; the way back drops what fell on it."""
     from sirius_amd import ops
     x = torch.randn(B, H, W, C, generator=_gen(42)).to(dtype)
-    ref = torch.cat([x[:, 0::2, 0::2], x[:, 1::2, 0::2], x[:, 0::2, 1::2], x[:, 1::2, 1::2]], dim=-1)
+    xp = torch.nn.functional.pad(x, (0, 0, 0, W % 2, 0, H % 2))
+    ref = torch.cat([xp[:, 0::2, 0::2], xp[:, 1::2, 0::2], xp[:, 0::2, 1::2], xp[:, 1::2, 1::2]], dim=-1)
     merged = torch.empty(ref.shape, dtype=dtype, device="cuda")
     ops.patch_merge_gather(ctx, x.cuda(), merged, (B, H, W, C))
     back = torch.empty((B, H, W, C), dtype=dtype, device="cuda")
@@ -240,6 +324,9 @@ CFGS = {
     "shifted": dict(embed=32, depths=(2, 2), heads=(2, 4), window=4, patch=2, image=16, classes=16),
     # window 7 on 14x14 and 7x7 feature maps (the geometry of Swin-B's last two stages), head dimension 32
     "window7": dict(embed=64, depths=(2, 1), heads=(2, 4), window=7, patch=4, image=56, classes=8),
+    # feature maps the window does not tile: 10 x 10 under 4 x 4 windows (a 12 x 12 frame), merged to 5 x 5 (odd: the
+    # merge pads; an 8 x 8 frame), merged to 3 x 3 (smaller than the window); one head (unfused attention) and more
+    "padded": dict(embed=32, depths=(2, 2, 2), heads=(1, 2, 4), window=4, patch=4, image=40, classes=16),
 }
 
 
