@@ -10,7 +10,9 @@ adds: the attention mask of shifted windows, patch merging, patch embedding.
   shift and partition in one pass), runs every projection as a 1x1 convolution on the MFMA kernels, the
   attention products as batched strided GEMMs on the packed [B_, N, 3, heads, D] projection, and scatters
   the result back with the residual add fused; where one window covers the image (the last stage at 224) the
-  gathers vanish;
+  gathers vanish; a feature map the window does not tile is padded with zero tokens at the bottom and the right to
+  whole windows (torchvision's rule; window-ordered tensors then have the padded frame's rows), an odd side is
+  padded by the merge;
 * the relative-position bias is gathered from its table into a dense [heads, N, N] fp32 tensor per block
   (read by the softmax kernel); its gradient is the column sum of the logit gradients over the windows,
   scattered back through the index;
