@@ -184,8 +184,10 @@ __global__ __launch_bounds__(256) void ln_bwd_kernel(LnArgs p) {
   const float inv_c = 1.0f / static_cast<float>(p.C);
   // rows_per_wg is a multiple of GROUPS, so the groups of a wavefront stay in step (the row sums below are
   // taken by all lanes); a group beyond the last row works on nothing.  A group takes R rows per trip and
-  // requests the chunks of all of them before it uses any: a trip costs one round trip to memory, not R.
-  constexpr int R = 2;
+  // requests the chunks of all of them before it uses any.  R = 1: two rows per trip cost 36 registers more
+  // (161 against 125 for rows of 768), and beside the weight gradients of the second lane, which leave room for
+  // one such wave per SIMD, the kernel was slower for it (GPT-2: 40.7 against 36.5 us per launch in the step).
+  constexpr int R = 1;
   for (int64_t base = r0; base < r1; base += R * GROUPS) {
     bool live[R];
     int64_t wrows[R];
