@@ -6,7 +6,7 @@ the time it takes alone on the chip (HIP events around it in a one-at-a-time rep
 phase (forward / backward), per stage of the network and per kernel family, next to the wall time of the step
 as it runs (two lanes): where the step's time goes.
 
-    python -m sirius_amd.floor_table [--batch 64] [--reps 3] [--out gpurun_out/floor_table.txt]
+    python -m sirius_amd.floor_table [--batch 64] [--reps 3] [--out floor_table.txt]
 """
 import argparse
 import collections

@@ -93,7 +93,7 @@ def test_cross_entropy_and_sgd_closed_forms():
     np.testing.assert_allclose(rows_o.numpy(), rows, rtol=1e-5)
     np.testing.assert_allclose(mean_o.item(), mean, rtol=1e-5)
     np.testing.assert_allclose(grad_o.numpy(), 0.25 * grad, rtol=1e-4, atol=1e-7)
-    # the survey's probe: p=1, g=1, lr .1, mu .9, wd 1e-4 -> 0.89999 then 0.70997
+    # a hand-computed probe: p=1, g=1, lr .1, mu .9, wd 1e-4 -> 0.89999 then 0.70997
     p1, _ = B.sgd_scalar(1.0, 1.0, 0.1, 0.9, 1e-4, 1)
     p2, _ = B.sgd_scalar(1.0, 1.0, 0.1, 0.9, 1e-4, 2)
     assert abs(p1 - 0.89999) < 1e-6 and abs(p2 - 0.70997) < 2e-5
